@@ -1,0 +1,245 @@
+"""ctypes binding of the CPU oracle (libtqmoe_oracle.so) and, where it was built, of the reference's own host objects
+(oracle/_ref/libtqref.so). TEST INFRASTRUCTURE ONLY: imported by tests/, __graft_entry__.smoke() and the cpu_baseline
+leg of bench.py, never by the tqllm_amd package.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libtqmoe_oracle.so")
+REF_PATH = os.path.join(HERE, "_ref", "libtqref.so")
+
+F32, F16, Q4_K, IQ4_NL, IQ3_S, IQ4_XS, BF16, NVFP4G = 0, 1, 12, 20, 21, 23, 30, 323
+GATE_SOFTMAX, GATE_SIGMOID = 1, 2
+BLOCK = {Q4_K: (256, 144), IQ4_NL: (32, 18), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76)}
+
+
+def build(ref=True):
+    """Compile the oracle (and the reference objects when the reference tree is present)."""
+    targets = ["all"] + (["ref"] if ref and os.path.isdir("/root/reference/src") else [])
+    subprocess.run(["make", "-s", "-C", HERE] + targets, check=True)
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        build(ref=False)
+    return C.CDLL(LIB_PATH)
+
+
+_lib = _load()
+_p = C.c_void_p
+_lib.tqo_half_to_float.restype = C.c_float
+_lib.tqo_half_to_float.argtypes = [C.c_uint16]
+_lib.tqo_float_to_half.restype = C.c_uint16
+_lib.tqo_float_to_half.argtypes = [C.c_float]
+_lib.tqo_bf16_to_float.restype = C.c_float
+_lib.tqo_bf16_to_float.argtypes = [C.c_uint16]
+_lib.tqo_float_to_bf16.restype = C.c_uint16
+_lib.tqo_float_to_bf16.argtypes = [C.c_float]
+_lib.tqo_e4m3_to_float.restype = C.c_float
+_lib.tqo_e4m3_to_float.argtypes = [C.c_uint8]
+_lib.tqo_float_to_e4m3.restype = C.c_uint8
+_lib.tqo_float_to_e4m3.argtypes = [C.c_float]
+_lib.tqo_dequantize.argtypes = [C.c_uint32, _p, _p, C.c_int64]
+_lib.tqo_quantize.argtypes = [C.c_uint32, _p, _p, C.c_int64, C.c_int64]
+_lib.tqo_route.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _p, _p, _p, _p]
+_lib.tqo_route_min_gap_ulps.restype = C.c_double
+_lib.tqo_route_min_gap_ulps.argtypes = [C.c_int, C.c_int, _p]
+_lib.tqo_shared_weight.restype = C.c_float
+_lib.tqo_shared_weight.argtypes = [C.c_float]
+_lib.tqo_dispatch.argtypes = [_p, C.c_int, C.c_int, _p, _p, _p]
+_lib.tqo_expert_ffn.restype = None
+_lib.tqo_expert_ffn.argtypes = [_p, C.c_int, _p, _p, _p, C.c_int, C.c_float, C.c_int, _p]
+_lib.tqo_combine.restype = None
+_lib.tqo_combine.argtypes = [C.c_int, _p, _p, C.c_int, _p]
+_lib.tqo_router_logits.argtypes = [_p, C.c_uint32, _p, _p, C.c_uint32, C.c_int, C.c_int, C.c_int, _p]
+_lib.tqo_quant_act_row_i8.restype = None
+_lib.tqo_quant_act_row_i8.argtypes = [_p, C.c_int, _p, _p]
+_lib.tqo_quant_act_row_e4m3.restype = None
+_lib.tqo_quant_act_row_e4m3.argtypes = [_p, C.c_int, _p, _p]
+_lib.tqo_widen_i8_256.restype = None
+_lib.tqo_widen_i8_256.argtypes = [_p, _p, _p]
+_lib.tqo_cpu_expert_bench.restype = C.c_double
+_lib.tqo_cpu_expert_bench.argtypes = [C.c_uint32, _p, _p, _p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _p]
+_lib.tqo_hardware_threads.restype = C.c_int
+
+
+class _Layer(C.Structure):
+    _fields_ = [("hidden", C.c_int), ("ff", C.c_int), ("n_expert", C.c_int), ("k", C.c_int), ("has_shared", C.c_int),
+                ("shared_ff", C.c_int), ("wtype", C.c_uint32), ("gate", _p), ("up", _p), ("down", _p),
+                ("act_mode", C.c_int), ("threads", C.c_int)]
+
+
+_lib.tqo_layer_forward.argtypes = [C.POINTER(_Layer), _p, _p, C.c_int, _p, _p, _p]
+
+
+def _ptr(a):
+    return a.ctypes.data_as(_p) if a is not None else None
+
+
+def _c(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def half_to_float(h):
+    return _lib.tqo_half_to_float(int(h))
+
+
+def float_to_half(f):
+    return _lib.tqo_float_to_half(float(f))
+
+
+def e4m3_to_float(b):
+    return _lib.tqo_e4m3_to_float(int(b))
+
+
+def float_to_e4m3(f):
+    return _lib.tqo_float_to_e4m3(float(f))
+
+
+def to_bf16(a):
+    """fp32 array -> (uint16 bf16 bits, fp32 values after rounding), round to nearest even."""
+    a = _c(a, np.float32)
+    u = a.view(np.uint32)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    return r, (r.astype(np.uint32) << 16).view(np.float32).reshape(a.shape)
+
+
+def dequantize(wtype, raw, n):
+    raw = _c(raw, np.uint8)
+    out = np.empty(int(n), np.float32)
+    if _lib.tqo_dequantize(wtype, _ptr(raw), _ptr(out), int(n)):
+        raise ValueError("tqo_dequantize: bad type or size")
+    return out
+
+
+def quantize(wtype, w, row=None):
+    w = _c(w, np.float32)
+    elems, nbytes = BLOCK[wtype]
+    out = np.zeros(w.size // elems * nbytes, np.uint8)
+    if _lib.tqo_quantize(wtype, _ptr(w), _ptr(out), w.size, int(row if row is not None else w.shape[-1])):
+        raise ValueError("tqo_quantize: bad type or size")
+    return out
+
+
+def route(logits, k, gating=GATE_SOFTMAX, norm=True, scale=1.0, bias=None):
+    """logits [n][E] (or [E]) -> ids [n][k] int32, weights [n][k] fp32."""
+    lg = np.atleast_2d(_c(logits, np.float32))
+    n, e = lg.shape
+    ids = np.empty((n, k), np.int32)
+    w = np.empty((n, k), np.float32)
+    b = _c(bias, np.float32) if bias is not None else None
+    for t in range(n):
+        if _lib.tqo_route(gating, e, k, int(norm), float(scale), _ptr(lg[t]), _ptr(b), _ptr(ids[t]), _ptr(w[t])):
+            raise ValueError("tqo_route: bad shape")
+    return ids, w
+
+
+def route_min_gap_ulps(logits, k):
+    lg = np.atleast_2d(_c(logits, np.float32))
+    return np.array([_lib.tqo_route_min_gap_ulps(lg.shape[1], k, _ptr(lg[t])) for t in range(lg.shape[0])])
+
+
+def shared_weight(logit):
+    return _lib.tqo_shared_weight(float(logit))
+
+
+def dispatch(ids, n_expert):
+    ids = _c(ids, np.int32).reshape(-1)
+    counts = np.empty(n_expert, np.int32)
+    offsets = np.empty(n_expert + 1, np.int32)
+    perm = np.full(ids.size, -1, np.int32)
+    if _lib.tqo_dispatch(_ptr(ids), ids.size, n_expert, _ptr(counts), _ptr(offsets), _ptr(perm)):
+        raise ValueError("tqo_dispatch: id out of range")
+    return counts, offsets, perm
+
+
+def expert_ffn(x, w_gate, w_up, w_down, clamp=0.0, clamp_gate=False):
+    x, w_gate, w_up, w_down = (_c(a, np.float32) for a in (x, w_gate, w_up, w_down))
+    ff, hidden = w_gate.shape
+    out = np.empty(hidden, np.float32)
+    _lib.tqo_expert_ffn(_ptr(x), hidden, _ptr(w_gate), _ptr(w_up), _ptr(w_down), ff, float(clamp), int(clamp_gate), _ptr(out))
+    return out
+
+
+def combine(weights, expert_outs, out=None):
+    weights, expert_outs = _c(weights, np.float32), _c(expert_outs, np.float32)
+    k, hidden = expert_outs.shape
+    out = np.zeros(hidden, np.float32) if out is None else out
+    _lib.tqo_combine(k, _ptr(weights), _ptr(expert_outs), hidden, _ptr(out))
+    return out
+
+
+def router_logits(w, wtype, shared_gate, x, xtype, hidden, n_expert, n):
+    out = np.empty((n, n_expert + 1), np.float32)
+    if _lib.tqo_router_logits(_ptr(w), wtype, _ptr(shared_gate), _ptr(x), xtype, hidden, n_expert, n, _ptr(out)):
+        raise ValueError("tqo_router_logits: bad shape or type")
+    return out
+
+
+def quant_act_row_i8(x):
+    x = _c(x, np.float32)
+    q = np.empty(x.size, np.int8)
+    s = np.empty(1, np.float32)
+    _lib.tqo_quant_act_row_i8(_ptr(x), x.size, _ptr(q), _ptr(s))
+    return q, float(s[0])
+
+
+def quant_act_row_e4m3(x):
+    x = _c(x, np.float32)
+    q = np.empty(x.size, np.uint8)
+    s = np.empty(1, np.float32)
+    _lib.tqo_quant_act_row_e4m3(_ptr(x), x.size, _ptr(q), _ptr(s))
+    return q, float(s[0])
+
+
+def layer_forward(x, logits, gate, up, down, wtype, hidden, ff, n_expert, k, shared_ff=0, act_mode=0, threads=8):
+    """Whole layer on the host; returns (out [n][H] fp32, ids [n][k], weights [n][k])."""
+    x, logits = _c(x, np.float32), _c(logits, np.float32)
+    gate, up, down = (_c(a, np.uint8) for a in (gate, up, down))
+    n = x.shape[0]
+    L = _Layer(hidden, ff, n_expert, k, int(shared_ff > 0), shared_ff, wtype, _ptr(gate), _ptr(up), _ptr(down), act_mode, threads)
+    out = np.empty((n, hidden), np.float32)
+    ids = np.empty((n, k), np.int32)
+    w = np.empty((n, k), np.float32)
+    if _lib.tqo_layer_forward(C.byref(L), _ptr(x), _ptr(logits), n, _ptr(out), _ptr(ids), _ptr(w)):
+        raise ValueError("tqo_layer_forward: bad configuration")
+    return out, ids, w
+
+
+def cpu_expert_bench(wtype, gate, up, down, hidden, ff, n_expert, threads, int8_act, reps=3):
+    gate, up, down = (_c(a, np.uint8) for a in (gate, up, down))
+    chk = np.zeros(1, np.float32)
+    t = _lib.tqo_cpu_expert_bench(wtype, _ptr(gate), _ptr(up), _ptr(down), hidden, ff, n_expert, threads, int(int8_act), reps, _ptr(chk))
+    if t < 0:
+        raise ValueError("tqo_cpu_expert_bench: bad configuration")
+    return t, float(chk[0])
+
+
+def hardware_threads():
+    return _lib.tqo_hardware_threads()
+
+
+def ref_lib():
+    """The reference's own host objects, or None where they were not built (no reference tree)."""
+    if not os.path.exists(REF_PATH):
+        return None
+    r = C.CDLL(REF_PATH)
+    r.ref_half_to_float.restype = C.c_float
+    r.ref_half_to_float.argtypes = [C.c_uint16]
+    r.ref_float_to_half.restype = C.c_uint16
+    r.ref_float_to_half.argtypes = [C.c_float]
+    r.ref_e4m3_to_float.restype = C.c_float
+    r.ref_e4m3_to_float.argtypes = [C.c_uint8]
+    r.ref_dequantize.argtypes = [C.c_uint32, _p, _p, C.c_int64]
+    r.ref_route.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _p, _p, _p, _p]
+    r.ref_expert_ffn.restype = None
+    r.ref_expert_ffn.argtypes = [_p, C.c_int, _p, _p, _p, C.c_int, C.c_float, C.c_int, _p]
+    r.ref_combine.restype = None
+    r.ref_combine.argtypes = [C.c_int, _p, _p, C.c_int, _p]
+    r.ref_iq4nl_matvec.restype = None
+    r.ref_iq4nl_matvec.argtypes = [C.c_int, _p, C.c_int, C.c_int, _p, C.c_int, _p]
+    return r

@@ -1,0 +1,848 @@
+// CPU oracle for the mixture-of-experts layer: TEST INFRASTRUCTURE ONLY (see tqmoe_oracle.h for what each function
+// follows in the reference and how it is pinned). Nothing in the product library links or loads this file.
+#include "tqmoe_oracle.h"
+#include "iq3s_lattice.h"
+
+#include <algorithm>
+#include <atomic>
+#include <chrono>
+#include <cmath>
+#include <cstring>
+#include <limits>
+#include <mutex>
+#include <numeric>
+#include <thread>
+#include <vector>
+
+namespace {
+
+const int8_t kIq4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+const float kE2M1[16] = {0.f, 0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f, -0.f, -0.5f, -1.f, -1.5f, -2.f, -3.f, -4.f, -6.f};
+
+inline uint32_t f2u(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
+inline float u2f(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+inline uint16_t rd16(const uint8_t * p) { uint16_t v; std::memcpy(&v, p, 2); return v; }
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------- conversions
+// src/formats/weight/dequant.cpp:32-54: IEEE binary16 -> binary32, subnormals, inf and NaN payload kept.
+float tqo_half_to_float(uint16_t h) {
+    const uint32_t sign = uint32_t(h >> 15) << 31;
+    const int e = (h >> 10) & 31;
+    uint32_t m = h & 1023u;
+    if (e == 31) return u2f(sign | 0x7F800000u | (m << 13));
+    if (e) return u2f(sign | uint32_t(e + 112) << 23 | (m << 13));
+    if (!m) return u2f(sign);
+    int shift = 0;  // normalise the subnormal: value = m * 2^-24
+    while (!(m & 1024u)) { m <<= 1; ++shift; }
+    return u2f(sign | uint32_t(113 - shift) << 23 | ((m & 1023u) << 13));
+}
+
+// src/formats/weight/dequant.cpp:12-30: binary32 -> binary16, round to nearest even, overflow to inf.
+uint16_t tqo_float_to_half(float f) {
+    const uint32_t x = f2u(f), a = x & 0x7FFFFFFFu;
+    const uint16_t sign = uint16_t((x >> 16) & 0x8000u);
+    if (a > 0x7F800000u) return uint16_t(sign | 0x7E00u);
+    if (a == 0x7F800000u) return uint16_t(sign | 0x7C00u);
+    // work on the exact value: a = mant * 2^(e - 150)
+    const int e = int(a >> 23);
+    if (e < 102) return sign;  // below half the smallest subnormal (2^-25): zero; e == 102 may round up
+    uint32_t mant = (a & 0x7FFFFFu) | (e ? 0x800000u : 0u);
+    // target unit: 2^-24 for subnormal halves (e <= 112), else 2^(e - 127 - 10)
+    const int drop = e <= 112 ? 126 - e : 13;  // bits of mant below the target unit
+    uint32_t q = drop >= 32 ? 0 : mant >> drop;
+    const uint32_t rest = mant & ((1u << drop) - 1u), half = 1u << (drop - 1);
+    if (rest > half || (rest == half && (q & 1u))) ++q;
+    if (e <= 112) return uint16_t(sign | q);  // q == 1024 lands on the smallest normal by construction
+    // q in [1024, 2048]; exponent field e - 112
+    uint32_t bits = (uint32_t(e - 112) << 10) + (q - 1024u);
+    if (bits >= 0x7C00u) bits = 0x7C00u;
+    return uint16_t(sign | bits);
+}
+
+float tqo_bf16_to_float(uint16_t h) { return u2f(uint32_t(h) << 16); }
+uint16_t tqo_float_to_bf16(float f) {
+    const uint32_t x = f2u(f);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return uint16_t((x >> 16) | 0x40u);
+    return uint16_t((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
+}
+
+// src/formats/weight/dequant.cpp:387-391
+float tqo_e4m3_to_float(uint8_t b) {
+    const int e = (b >> 3) & 15, m = b & 7;
+    float v;
+    if (e == 15 && m == 7) v = std::numeric_limits<float>::quiet_NaN();
+    else if (e == 0) v = std::ldexp(float(m), -9);
+    else v = std::ldexp(float(8 + m), e - 10);
+    return (b & 0x80) ? -v : v;
+}
+
+uint8_t tqo_float_to_e4m3(float f) {
+    const uint8_t sign = (f2u(f) >> 31) ? 0x80 : 0;
+    const float a = std::fabs(f);
+    if (a != a) return uint8_t(sign | 0x7F);
+    if (a >= 448.f) return uint8_t(sign | 0x7E);
+    if (a < 0.015625f) {  // below 2^-6: subnormal step 2^-9
+        const int m = int(std::nearbyint(std::ldexp(a, 9)));
+        return uint8_t(sign | m);  // m == 8 is the code of 2^-6
+    }
+    int ex;
+    const float fr = std::frexp(a, &ex);            // a = fr * 2^ex, fr in [0.5, 1)
+    int m = int(std::nearbyint(std::ldexp(fr, 4)));  // 8..16 in units of 2^(ex - 4)
+    int e = ex - 1 + 7;
+    if (m == 16) { m = 8; ++e; }
+    int code = (e << 3) | (m - 8);
+    if (code > 0x7E) code = 0x7E;
+    return uint8_t(sign | code);
+}
+
+// ------------------------------------------------------------------------------------------------- decoding
+int tqo_block_layout(uint32_t type, int * elems, int * bytes) {
+    int e = 0, b = 0;
+    switch (type) {  // src/core/gguf.cpp:136-152
+        case TQO_Q4_K: e = 256; b = 144; break;
+        case TQO_IQ4_NL: e = 32; b = 18; break;
+        case TQO_IQ3_S: e = 256; b = 110; break;
+        case TQO_IQ4_XS: e = 256; b = 136; break;
+        case TQO_NVFP4G: e = 128; b = 76; break;
+        default: return 0;
+    }
+    if (elems) *elems = e;
+    if (bytes) *bytes = b;
+    return 1;
+}
+
+namespace {
+
+// 6-bit (scale, min) pair j of a Q4_K block's 12-byte field, src/formats/weight/dequant.cpp:56-64
+inline void q4k_scale_min(const uint8_t * q, int j, int & sc, int & mn) {
+    if (j < 4) { sc = q[j] & 63; mn = q[j + 4] & 63; }
+    else { sc = (q[j + 4] & 15) | ((q[j - 4] >> 6) << 4); mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4); }
+}
+
+void decode_q4k(const uint8_t * b, float * y) {
+    const float d = tqo_half_to_float(rd16(b)), dmin = tqo_half_to_float(rd16(b + 2));
+    for (int c = 0; c < 4; ++c) {
+        int s1, m1, s2, m2;
+        q4k_scale_min(b + 4, 2 * c, s1, m1);
+        q4k_scale_min(b + 4, 2 * c + 1, s2, m2);
+        // evaluation order of the reference: (d * sc) * code - (dmin * m)
+        const float d1 = d * float(s1), o1 = dmin * float(m1), d2 = d * float(s2), o2 = dmin * float(m2);
+        const uint8_t * q = b + 16 + 32 * c;
+        for (int l = 0; l < 32; ++l) {
+            y[64 * c + l] = d1 * float(q[l] & 15) - o1;
+            y[64 * c + 32 + l] = d2 * float(q[l] >> 4) - o2;
+        }
+    }
+}
+
+inline int iq4xs_subscale(const uint8_t * b, int ib) {  // 6-bit scale of sub-block ib, before the -32 offset
+    const uint16_t sh = rd16(b + 2);
+    return ((b[4 + ib / 2] >> (4 * (ib & 1))) & 15) | (((sh >> (2 * ib)) & 3) << 4);
+}
+
+void decode_iq4xs(const uint8_t * b, float * y) {
+    const float d = tqo_half_to_float(rd16(b));
+    for (int ib = 0; ib < 8; ++ib) {
+        const float dl = d * float(iq4xs_subscale(b, ib) - 32);
+        const uint8_t * q = b + 8 + 16 * ib;
+        for (int j = 0; j < 16; ++j) {
+            y[32 * ib + j] = dl * float(kIq4Values[q[j] & 15]);
+            y[32 * ib + 16 + j] = dl * float(kIq4Values[q[j] >> 4]);
+        }
+    }
+}
+
+void decode_iq4nl(const uint8_t * b, float * y) {
+    const float d = tqo_half_to_float(rd16(b));
+    for (int j = 0; j < 16; ++j) {
+        y[j] = d * float(kIq4Values[b[2 + j] & 15]);
+        y[16 + j] = d * float(kIq4Values[b[2 + j] >> 4]);
+    }
+}
+
+void decode_iq3s(const uint8_t * b, float * y) {
+    const float d = tqo_half_to_float(rd16(b));
+    const uint8_t * qs = b + 2, * qh = b + 66, * signs = b + 74, * sc = b + 106;
+    for (int ib = 0; ib < 8; ++ib) {
+        const float db = d * float(1 + 2 * ((sc[ib / 2] >> (4 * (ib & 1))) & 15));
+        for (int w = 0; w < 8; ++w) {
+            const uint32_t g = tq_iq3s_point(qs[8 * ib + w] | (((qh[ib] >> w) & 1) << 8));
+            const int sg = signs[4 * ib + w / 2] >> (4 * (w & 1));
+            for (int j = 0; j < 4; ++j) {
+                const float mag = db * float((g >> (8 * j)) & 255u);
+                y[32 * ib + 4 * w + j] = ((sg >> j) & 1) ? mag * -1.f : mag * 1.f;
+            }
+        }
+    }
+}
+
+void decode_nvfp4g(const uint8_t * b, float * y) {
+    float g;
+    std::memcpy(&g, b, 4);
+    for (int grp = 0; grp < 8; ++grp) {
+        const float d = tqo_e4m3_to_float(b[4 + grp]) * g;
+        for (int i = 0; i < 8; ++i) {
+            const uint8_t q = b[12 + 8 * grp + i];
+            y[16 * grp + 2 * i] = kE2M1[q & 15] * d;
+            y[16 * grp + 2 * i + 1] = kE2M1[q >> 4] * d;
+        }
+    }
+}
+
+}  // namespace
+
+int tqo_dequantize(uint32_t type, const void * src, float * dst, int64_t n) {
+    int elems, bytes;
+    if (!tqo_block_layout(type, &elems, &bytes) || n < 0 || n % elems) return -1;
+    const uint8_t * s = static_cast<const uint8_t *>(src);
+    for (int64_t b = 0; b < n / elems; ++b, s += bytes, dst += elems) switch (type) {
+        case TQO_Q4_K: decode_q4k(s, dst); break;
+        case TQO_IQ4_XS: decode_iq4xs(s, dst); break;
+        case TQO_IQ4_NL: decode_iq4nl(s, dst); break;
+        case TQO_IQ3_S: decode_iq3s(s, dst); break;
+        case TQO_NVFP4G: decode_nvfp4g(s, dst); break;
+    }
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------ encoders (own; unpinned)
+namespace {
+
+inline int nearest_iq4(float v) {  // index of the table value nearest to v, lower index on a tie
+    int best = 0;
+    float bd = std::fabs(v - float(kIq4Values[0]));
+    for (int i = 1; i < 16; ++i) {
+        const float dd = std::fabs(v - float(kIq4Values[i]));
+        if (dd < bd) { bd = dd; best = i; }
+    }
+    return best;
+}
+
+// sub-block scale that puts the largest-magnitude value on table entry 0 (-127)
+inline float iq4_block_scale(const float * x) {
+    float amax = 0.f, vmax = 0.f;
+    for (int i = 0; i < 32; ++i) if (std::fabs(x[i]) > amax) { amax = std::fabs(x[i]); vmax = x[i]; }
+    return vmax / -127.f;
+}
+
+void encode_iq4nl(const float * x, uint8_t * b) {
+    const uint16_t hd = tqo_float_to_half(iq4_block_scale(x));
+    const float d = tqo_half_to_float(hd), inv = d != 0.f ? 1.f / d : 0.f;
+    std::memcpy(b, &hd, 2);
+    for (int j = 0; j < 16; ++j)
+        b[2 + j] = uint8_t(nearest_iq4(x[j] * inv) | (nearest_iq4(x[16 + j] * inv) << 4));
+}
+
+void encode_iq4xs(const float * x, uint8_t * b) {
+    float ds[8], big = 0.f;
+    for (int ib = 0; ib < 8; ++ib) { ds[ib] = iq4_block_scale(x + 32 * ib); if (std::fabs(ds[ib]) > std::fabs(big)) big = ds[ib]; }
+    const uint16_t hd = tqo_float_to_half(big / -32.f);  // the largest sub-scale sits on ls - 32 = -32
+    const float d = tqo_half_to_float(hd);
+    std::memset(b, 0, 136);
+    std::memcpy(b, &hd, 2);
+    uint16_t sh = 0;
+    for (int ib = 0; ib < 8; ++ib) {
+        int l = d != 0.f ? int(std::nearbyint(ds[ib] / d)) : 0;
+        l = std::max(-32, std::min(31, l));
+        const int ls = l + 32;
+        b[4 + ib / 2] |= uint8_t((ls & 15) << (4 * (ib & 1)));
+        sh |= uint16_t((ls >> 4) << (2 * ib));
+        const float dl = d * float(l), inv = dl != 0.f ? 1.f / dl : 0.f;
+        const float * v = x + 32 * ib;
+        for (int j = 0; j < 16; ++j)
+            b[8 + 16 * ib + j] = uint8_t(nearest_iq4(v[j] * inv) | (nearest_iq4(v[16 + j] * inv) << 4));
+    }
+    std::memcpy(b + 2, &sh, 2);
+}
+
+void encode_q4k(const float * x, uint8_t * b) {
+    float sc[8], mn[8], smax = 0.f, mmax = 0.f;
+    for (int i = 0; i < 8; ++i) {
+        float lo = 0.f, hi = 0.f;  // the code range always holds zero
+        for (int l = 0; l < 32; ++l) { lo = std::min(lo, x[32 * i + l]); hi = std::max(hi, x[32 * i + l]); }
+        sc[i] = (hi - lo) / 15.f;
+        mn[i] = -lo;
+        smax = std::max(smax, sc[i]);
+        mmax = std::max(mmax, mn[i]);
+    }
+    const uint16_t hd = tqo_float_to_half(smax / 63.f), hm = tqo_float_to_half(mmax / 63.f);
+    const float d = tqo_half_to_float(hd), dm = tqo_half_to_float(hm);
+    std::memset(b, 0, 144);
+    std::memcpy(b, &hd, 2);
+    std::memcpy(b + 2, &hm, 2);
+    int s6[8], m6[8];
+    for (int i = 0; i < 8; ++i) {
+        s6[i] = d > 0.f ? std::min(63, std::max(0, int(std::nearbyint(sc[i] / d)))) : 0;
+        m6[i] = dm > 0.f ? std::min(63, std::max(0, int(std::nearbyint(mn[i] / dm)))) : 0;
+    }
+    uint8_t * q = b + 4;
+    for (int j = 0; j < 4; ++j) {
+        q[j] = uint8_t(s6[j] | ((s6[j + 4] >> 4) << 6));
+        q[j + 4] = uint8_t(m6[j] | ((m6[j + 4] >> 4) << 6));
+        q[j + 8] = uint8_t((s6[j + 4] & 15) | ((m6[j + 4] & 15) << 4));
+    }
+    for (int c = 0; c < 4; ++c)
+        for (int l = 0; l < 32; ++l) {
+            int code[2];
+            for (int h = 0; h < 2; ++h) {
+                const int i = 2 * c + h;
+                const float step = d * float(s6[i]), off = dm * float(m6[i]);
+                const float v = x[64 * c + 32 * h + l];
+                code[h] = step > 0.f ? std::min(15, std::max(0, int(std::nearbyint((v + off) / step)))) : 0;
+            }
+            b[16 + 32 * c + l] = uint8_t(code[0] | (code[1] << 4));
+        }
+}
+
+// for every point of {0..7}^4 (12-bit code of magnitude levels) the nearest codebook point, lower index on a tie
+const uint16_t * iq3s_nearest_table() {
+    static std::vector<uint16_t> t;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        t.resize(4096);
+        for (int c = 0; c < 4096; ++c) {
+            int best = 0, bd = 1 << 30;
+            for (int i = 0; i < 512; ++i) {
+                const int g = tq_iq3s_lattice12[i];
+                int dd = 0;
+                for (int j = 0; j < 4; ++j) { const int df = ((c >> (3 * j)) & 7) - ((g >> (3 * j)) & 7); dd += df * df; }
+                if (dd < bd) { bd = dd; best = i; }
+            }
+            t[size_t(c)] = uint16_t(best);
+        }
+    });
+    return t.data();
+}
+
+// quantise 32 values with step db onto the codebook; returns the squared error, fills 8 point indices and 8 nibbles
+float iq3s_fit(const float * x, float db, int * idx, int * sg) {
+    const uint16_t * near = iq3s_nearest_table();
+    const float inv = db > 0.f ? 1.f / db : 0.f;
+    float err = 0.f;
+    for (int w = 0; w < 8; ++w) {
+        int code = 0, s = 0;
+        for (int j = 0; j < 4; ++j) {
+            const float v = x[4 * w + j];
+            if (v < 0.f) s |= 1 << j;
+            const int lev = std::min(7, std::max(0, int(std::nearbyint((std::fabs(v) * inv - 1.f) * 0.5f))));
+            code |= lev << (3 * j);
+        }
+        idx[w] = near[code];
+        sg[w] = s;
+        const int g = tq_iq3s_lattice12[idx[w]];
+        for (int j = 0; j < 4; ++j) {
+            const float mag = db * float(2 * ((g >> (3 * j)) & 7) + 1);
+            const float e = std::fabs(x[4 * w + j]) - mag;
+            err += e * e;
+        }
+    }
+    return err;
+}
+
+void encode_iq3s(const float * x, uint8_t * b) {
+    float db[8], dmax = 0.f;
+    int idx[8], sg[8];
+    for (int ib = 0; ib < 8; ++ib) {
+        float amax = 0.f;
+        for (int i = 0; i < 32; ++i) amax = std::max(amax, std::fabs(x[32 * ib + i]));
+        float best = 0.f, be = std::numeric_limits<float>::infinity();
+        for (int c = 7; c <= 17; c += 2) {  // where on the magnitude ladder the largest value should sit
+            const float cand = amax / float(c);
+            const float e = iq3s_fit(x + 32 * ib, cand, idx, sg);
+            if (e < be) { be = e; best = cand; }
+        }
+        db[ib] = best;
+        dmax = std::max(dmax, best);
+    }
+    const uint16_t hd = tqo_float_to_half(dmax / 31.f);
+    const float d = tqo_half_to_float(hd);
+    std::memset(b, 0, 110);
+    std::memcpy(b, &hd, 2);
+    for (int ib = 0; ib < 8; ++ib) {
+        int s = d > 0.f ? int(std::nearbyint((db[ib] / d - 1.f) * 0.5f)) : 0;
+        s = std::min(15, std::max(0, s));
+        b[106 + ib / 2] |= uint8_t(s << (4 * (ib & 1)));
+        iq3s_fit(x + 32 * ib, d * float(1 + 2 * s), idx, sg);
+        for (int w = 0; w < 8; ++w) {
+            b[2 + 8 * ib + w] = uint8_t(idx[w] & 255);
+            b[66 + ib] |= uint8_t((idx[w] >> 8) << w);
+            b[74 + 4 * ib + w / 2] |= uint8_t(sg[w] << (4 * (w & 1)));
+        }
+    }
+}
+
+inline int nearest_e2m1(float v) {
+    int best = 0;
+    float bd = std::fabs(v);
+    for (int i = 1; i < 16; ++i) {
+        if (i == 8) continue;  // -0 is never emitted
+        const float dd = std::fabs(v - kE2M1[i]);
+        if (dd < bd) { bd = dd; best = i; }
+    }
+    return best;
+}
+
+void encode_nvfp4g_row(const float * x, uint8_t * b, int64_t cols) {
+    float amax = 0.f;
+    for (int64_t i = 0; i < cols; ++i) amax = std::max(amax, std::fabs(x[i]));
+    const float g = amax > 0.f ? amax / (6.f * 448.f) : 1.f;  // the largest group scale lands on 448
+    for (int64_t blk = 0; blk < cols / 128; ++blk, b += 76, x += 128) {
+        std::memcpy(b, &g, 4);
+        for (int grp = 0; grp < 8; ++grp) {
+            float ga = 0.f;
+            for (int i = 0; i < 16; ++i) ga = std::max(ga, std::fabs(x[16 * grp + i]));
+            uint8_t sc = tqo_float_to_e4m3(ga / 6.f / g);
+            if (ga > 0.f && sc == 0) sc = 1;
+            b[4 + grp] = sc;
+            const float d = tqo_e4m3_to_float(sc) * g, inv = d > 0.f ? 1.f / d : 0.f;
+            for (int i = 0; i < 8; ++i)
+                b[12 + 8 * grp + i] = uint8_t(nearest_e2m1(x[16 * grp + 2 * i] * inv) | (nearest_e2m1(x[16 * grp + 2 * i + 1] * inv) << 4));
+        }
+    }
+}
+
+}  // namespace
+
+int tqo_quantize(uint32_t type, const float * src, void * dst, int64_t n, int64_t row) {
+    int elems, bytes;
+    if (!tqo_block_layout(type, &elems, &bytes) || n < 0 || n % elems) return -1;
+    uint8_t * o = static_cast<uint8_t *>(dst);
+    if (type == TQO_NVFP4G) {
+        if (row <= 0 || row % 128 || n % row) return -1;
+        for (int64_t r = 0; r < n / row; ++r) encode_nvfp4g_row(src + r * row, o + r * (row / 128) * 76, row);
+        return 0;
+    }
+    for (int64_t b = 0; b < n / elems; ++b, src += elems, o += bytes) switch (type) {
+        case TQO_Q4_K: encode_q4k(src, o); break;
+        case TQO_IQ4_XS: encode_iq4xs(src, o); break;
+        case TQO_IQ4_NL: encode_iq4nl(src, o); break;
+        case TQO_IQ3_S: encode_iq3s(src, o); break;
+    }
+    return 0;
+}
+
+// -------------------------------------------------------------------------------------------------- routing
+namespace {
+void gate_probs(int gating, int n, const float * logits, std::vector<float> & probs) {
+    probs.resize(size_t(n));
+    if (gating == TQO_GATE_SOFTMAX) {  // src/experts/moe.cpp:35-44: max, exp(l - max) summed in index order, divide
+        float mx = -INFINITY;
+        for (int i = 0; i < n; ++i) mx = std::max(mx, logits[i]);
+        float sum = 0.f;
+        for (int i = 0; i < n; ++i) { probs[size_t(i)] = std::exp(logits[i] - mx); sum += probs[size_t(i)]; }
+        for (int i = 0; i < n; ++i) probs[size_t(i)] /= sum;
+    } else {  // sigmoid, src/experts/moe.cpp:10-14
+        for (int i = 0; i < n; ++i) probs[size_t(i)] = 1.0f / (1.0f + std::exp(-logits[i]));
+    }
+}
+}  // namespace
+
+int tqo_route(int gating, int n_expert, int k, int norm_weights, float weight_scale, const float * logits,
+              const float * bias, int32_t * ids, float * weights) {
+    if (n_expert <= 0 || k <= 0 || k > n_expert) return -1;
+    if (gating != TQO_GATE_SOFTMAX && gating != TQO_GATE_SIGMOID) return -1;
+    std::vector<float> probs;
+    gate_probs(gating, n_expert, logits, probs);
+    std::vector<float> sel(probs);  // selection values: bias added for the choice only (moe.cpp:63-65)
+    if (bias) for (int i = 0; i < n_expert; ++i) sel[size_t(i)] += bias[i];
+    std::vector<int> order(static_cast<size_t>(n_expert));
+    std::iota(order.begin(), order.end(), 0);
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) {  // moe.cpp:73-78
+        if (sel[size_t(a)] != sel[size_t(b)]) return sel[size_t(a)] > sel[size_t(b)];
+        return a < b;
+    });
+    for (int s = 0; s < k; ++s) { ids[s] = order[size_t(s)]; weights[s] = probs[size_t(order[size_t(s)])]; }
+    if (norm_weights) {  // moe.cpp:101-106
+        float sum = 0.f;
+        for (int s = 0; s < k; ++s) sum += weights[s];
+        sum = std::max(sum, 6.103515625e-5f);
+        for (int s = 0; s < k; ++s) weights[s] /= sum;
+    }
+    if (weight_scale != 0.f && weight_scale != 1.f) for (int s = 0; s < k; ++s) weights[s] *= weight_scale;
+    return 0;
+}
+
+double tqo_route_min_gap_ulps(int n_expert, int k, const float * logits) {
+    std::vector<float> probs;
+    gate_probs(TQO_GATE_SOFTMAX, n_expert, logits, probs);
+    std::sort(probs.begin(), probs.end(), [](float a, float b) { return a > b; });
+    double best = INFINITY;
+    for (int s = 0; s < k && s + 1 < n_expert; ++s) {
+        const float hi = probs[size_t(s)], lo = probs[size_t(s) + 1];
+        if (hi == lo) continue;
+        const float ulp = std::nextafter(hi, INFINITY) - hi;
+        best = std::min(best, double(hi - lo) / double(ulp));
+    }
+    return best;
+}
+
+float tqo_shared_weight(float logit) { return 1.f / (1.f + std::exp(-logit)); }
+
+int tqo_dispatch(const int32_t * ids, int A, int E, int32_t * counts, int32_t * offsets, int32_t * perm) {
+    if (A < 0 || E <= 0) return -1;
+    for (int e = 0; e < E; ++e) counts[e] = 0;
+    for (int a = 0; a < A; ++a) {
+        if (ids[a] >= E) return -1;
+        if (ids[a] >= 0) ++counts[ids[a]];
+    }
+    offsets[0] = 0;
+    for (int e = 0; e < E; ++e) offsets[e + 1] = offsets[e] + counts[e];
+    std::vector<int32_t> fill(offsets, offsets + E);
+    for (int a = 0; a < A; ++a) if (ids[a] >= 0) perm[fill[size_t(ids[a])]++] = a;  // ascending a inside an expert
+    return 0;
+}
+
+// -------------------------------------------------------------------------------------------- FFN and combine
+void tqo_expert_ffn(const float * x, int hidden, const float * w_gate, const float * w_up, const float * w_down,
+                    int ff, float swiglu_clamp, int clamp_gate, float * out) {
+    std::vector<float> act(size_t(ff), 0.f);
+    for (int o = 0; o < ff; ++o) {  // moe.cpp:119-128: fp32 sums in column order
+        float g = 0.f, u = 0.f;
+        const float * wg = w_gate + size_t(o) * hidden, * wu = w_up + size_t(o) * hidden;
+        for (int i = 0; i < hidden; ++i) { g += wg[i] * x[i]; u += wu[i] * x[i]; }
+        if (swiglu_clamp > 1e-6f) {  // moe.cpp:133-143
+            u = std::min(std::max(u, -swiglu_clamp), swiglu_clamp);
+            if (clamp_gate) g = std::min(g, swiglu_clamp);
+            float s = g / (1.f + std::exp(-g));
+            if (!clamp_gate) s = std::min(s, swiglu_clamp);
+            act[size_t(o)] = s * u;
+        } else {
+            act[size_t(o)] = (g / (1.f + std::exp(-g))) * u;
+        }
+    }
+    for (int i = 0; i < hidden; ++i) {
+        float s = 0.f;
+        const float * wd = w_down + size_t(i) * ff;
+        for (int o = 0; o < ff; ++o) s += wd[o] * act[size_t(o)];
+        out[i] = s;
+    }
+}
+
+void tqo_combine(const int k, const float * weights, const float * expert_outs, int hidden, float * out) {
+    for (int s = 0; s < k; ++s)
+        for (int i = 0; i < hidden; ++i) out[i] += weights[s] * expert_outs[size_t(s) * hidden + i];
+}
+
+namespace {
+inline float load_as_float(const void * p, uint32_t type, size_t i) {
+    switch (type) {
+        case TQO_F32: return static_cast<const float *>(p)[i];
+        case TQO_BF16: return tqo_bf16_to_float(static_cast<const uint16_t *>(p)[i]);
+        default: return tqo_half_to_float(static_cast<const uint16_t *>(p)[i]);
+    }
+}
+}  // namespace
+
+int tqo_router_logits(const void * w, uint32_t wtype, const void * shared_gate, const void * x, uint32_t xtype,
+                      int hidden, int E, int n, float * logits) {
+    if (hidden <= 0 || E <= 0 || n <= 0) return -1;
+    for (uint32_t t : {wtype, xtype}) if (t != TQO_F32 && t != TQO_BF16 && t != TQO_F16) return -1;
+    for (int t = 0; t < n; ++t)
+        for (int r = 0; r <= E; ++r) {
+            float sum = 0.f;
+            if (r < E || shared_gate) {
+                const void * row = r < E ? w : shared_gate;
+                const size_t base = r < E ? size_t(r) * hidden : 0;
+                for (int j = 0; j < hidden; ++j)
+                    sum += load_as_float(row, wtype, base + j) * load_as_float(x, xtype, size_t(t) * hidden + j);
+            }
+            logits[size_t(t) * (E + 1) + r] = sum;
+        }
+    return 0;
+}
+
+// --------------------------------------------------------------------------------- declared operand quantisers
+void tqo_quant_act_row_i8(const float * x, int cols, int8_t * q, float * scale) {
+    float m = 0.f;
+    for (int i = 0; i < cols; ++i) m = std::max(m, std::fabs(x[i]));
+    *scale = m / 127.f;
+    const float mul = m > 0.f ? 127.f / m : 0.f;
+    for (int i = 0; i < cols; ++i) q[i] = int8_t(std::nearbyint(x[i] * mul));
+}
+
+void tqo_quant_act_row_e4m3(const float * x, int cols, uint8_t * q, float * scale) {
+    float m = 0.f;
+    for (int i = 0; i < cols; ++i) m = std::max(m, std::fabs(x[i]));
+    *scale = m / 448.f;
+    const float mul = m > 0.f ? 448.f / m : 0.f;
+    for (int i = 0; i < cols; ++i) q[i] = tqo_float_to_e4m3(x[i] * mul);
+}
+
+void tqo_widen_i8_256(const float * w, int8_t * q, float * scale) {
+    float m = 0.f;
+    for (int i = 0; i < 256; ++i) m = std::max(m, std::fabs(w[i]));
+    *scale = m / 127.f;
+    const float mul = m > 0.f ? 127.f / m : 0.f;
+    for (int i = 0; i < 256; ++i) q[i] = int8_t(std::nearbyint(w[i] * mul));
+}
+
+// ------------------------------------------------------------------------------------------------ whole layer
+namespace {
+
+void requant_row_i8(float * x, int cols) {  // x <- dequantised per-row int8 image of x
+    std::vector<int8_t> q(static_cast<size_t>(cols));
+    float s;
+    tqo_quant_act_row_i8(x, cols, q.data(), &s);
+    for (int i = 0; i < cols; ++i) x[i] = float(q[size_t(i)]) * s;
+}
+
+void widen_matrix_i8(float * w, int64_t n) {
+    int8_t q[256];
+    float s;
+    for (int64_t b = 0; b < n / 256; ++b) {
+        tqo_widen_i8_256(w + b * 256, q, &s);
+        for (int i = 0; i < 256; ++i) w[b * 256 + i] = float(q[i]) * s;
+    }
+}
+
+struct Decoded { std::vector<float> gate, up, down; };
+
+int decode_expert(const tqo_layer & L, int e, int ff, Decoded & d) {
+    int elems, bytes;
+    tqo_block_layout(L.wtype, &elems, &bytes);
+    const int64_t gu = int64_t(L.ff) * L.hidden;           // weights of one stacked expert matrix
+    const size_t stride = size_t(gu / elems) * bytes;      // bytes of one expert in a bank
+    d.gate.resize(size_t(ff) * L.hidden);
+    d.up.resize(size_t(ff) * L.hidden);
+    d.down.resize(size_t(L.hidden) * ff);
+    // gate / up: the first ff rows of expert e
+    if (tqo_dequantize(L.wtype, static_cast<const uint8_t *>(L.gate) + stride * e, d.gate.data(), int64_t(ff) * L.hidden)) return -1;
+    if (tqo_dequantize(L.wtype, static_cast<const uint8_t *>(L.up) + stride * e, d.up.data(), int64_t(ff) * L.hidden)) return -1;
+    // down: rows of L.ff columns, the first ff columns kept
+    std::vector<float> row(static_cast<size_t>(L.ff));
+    const size_t row_bytes = size_t(L.ff / elems) * bytes;
+    for (int r = 0; r < L.hidden; ++r) {
+        if (tqo_dequantize(L.wtype, static_cast<const uint8_t *>(L.down) + stride * e + row_bytes * r, row.data(), L.ff)) return -1;
+        std::copy(row.begin(), row.begin() + ff, d.down.begin() + size_t(r) * ff);
+    }
+    if (L.act_mode == 3) {
+        if (ff % 256 || L.hidden % 256) return -1;
+        widen_matrix_i8(d.gate.data(), int64_t(ff) * L.hidden);
+        widen_matrix_i8(d.up.data(), int64_t(ff) * L.hidden);
+        widen_matrix_i8(d.down.data(), int64_t(L.hidden) * ff);
+    }
+    return 0;
+}
+
+// FFN with the declared activation quantiser applied to both matvec inputs
+void ffn_mode(const tqo_layer & L, const float * x, const Decoded & d, int ff, float * out) {
+    if (L.act_mode == 0) { tqo_expert_ffn(x, L.hidden, d.gate.data(), d.up.data(), d.down.data(), ff, 0.f, 0, out); return; }
+    std::vector<float> act(static_cast<size_t>(ff));
+    for (int o = 0; o < ff; ++o) {
+        float g = 0.f, u = 0.f;
+        const float * wg = d.gate.data() + size_t(o) * L.hidden, * wu = d.up.data() + size_t(o) * L.hidden;
+        for (int i = 0; i < L.hidden; ++i) { g += wg[i] * x[i]; u += wu[i] * x[i]; }
+        act[size_t(o)] = (g / (1.f + std::exp(-g))) * u;
+    }
+    requant_row_i8(act.data(), ff);
+    for (int i = 0; i < L.hidden; ++i) {
+        float s = 0.f;
+        const float * wd = d.down.data() + size_t(i) * ff;
+        for (int o = 0; o < ff; ++o) s += wd[o] * act[size_t(o)];
+        out[i] = s;
+    }
+}
+
+}  // namespace
+
+int tqo_layer_forward(const tqo_layer * Lp, const float * x, const float * logits, int n, float * out,
+                      int32_t * ids_out, float * weights_out) {
+    const tqo_layer & L = *Lp;
+    int elems, bytes;
+    if (!tqo_block_layout(L.wtype, &elems, &bytes)) return -1;
+    if (L.hidden % elems || L.ff % elems || n <= 0 || L.k <= 0 || L.k > L.n_expert) return -1;
+    if (L.act_mode != 0 && L.act_mode != 1 && L.act_mode != 3) return -1;
+    if (L.has_shared && (L.shared_ff <= 0 || L.shared_ff > L.ff || L.shared_ff % elems)) return -1;
+    const int E = L.n_expert, K = L.k, A = n * K, H = L.hidden;
+    std::vector<int32_t> ids(static_cast<size_t>(A)), counts(static_cast<size_t>(E)), offsets(size_t(E) + 1), perm(static_cast<size_t>(A));
+    std::vector<float> weights(static_cast<size_t>(A));
+    for (int t = 0; t < n; ++t)
+        if (tqo_route(TQO_GATE_SOFTMAX, E, K, 1, 1.f, logits + size_t(t) * (E + 1), nullptr, ids.data() + size_t(t) * K,
+                      weights.data() + size_t(t) * K)) return -1;
+    tqo_dispatch(ids.data(), A, E, counts.data(), offsets.data(), perm.data());
+    if (ids_out) std::copy(ids.begin(), ids.end(), ids_out);
+    if (weights_out) std::copy(weights.begin(), weights.end(), weights_out);
+
+    std::vector<float> xin(x, x + size_t(n) * H);
+    if (L.act_mode) for (int t = 0; t < n; ++t) requant_row_i8(xin.data() + size_t(t) * H, H);
+
+    std::vector<float> routed(size_t(A) * H), shared(L.has_shared ? size_t(n) * H : 0);
+    std::atomic<int> next{0}, failed{0};
+    const int jobs = E + (L.has_shared ? 1 : 0);
+    auto worker = [&]() {
+        Decoded d;
+        for (;;) {
+            const int e = next.fetch_add(1);
+            if (e >= jobs) break;
+            if (e < E) {
+                if (!counts[size_t(e)]) continue;
+                if (decode_expert(L, e, L.ff, d)) { failed = 1; continue; }
+                for (int i = offsets[size_t(e)]; i < offsets[size_t(e) + 1]; ++i) {
+                    const int a = perm[size_t(i)];
+                    ffn_mode(L, xin.data() + size_t(a / K) * H, d, L.ff, routed.data() + size_t(a) * H);
+                }
+            } else {
+                if (decode_expert(L, E, L.shared_ff, d)) { failed = 1; continue; }
+                for (int t = 0; t < n; ++t) ffn_mode(L, xin.data() + size_t(t) * H, d, L.shared_ff, shared.data() + size_t(t) * H);
+            }
+        }
+    };
+    const int nt = std::max(1, L.threads);
+    std::vector<std::thread> pool;
+    for (int i = 1; i < nt; ++i) pool.emplace_back(worker);
+    worker();
+    for (auto & th : pool) th.join();
+    if (failed) return -1;
+
+    for (int t = 0; t < n; ++t) {  // src/experts/moe.cu:224-234: slots in order, then the shared row
+        float * o = out + size_t(t) * H;
+        std::fill(o, o + H, 0.f);
+        tqo_combine(K, weights.data() + size_t(t) * K, routed.data() + size_t(t) * K * H, H, o);
+        if (L.has_shared) {
+            const float sw = tqo_shared_weight(logits[size_t(t) * (E + 1) + E]);
+            for (int i = 0; i < H; ++i) o[i] += sw * shared[size_t(t) * H + i];
+        }
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------- CPU baseline
+// Scheme of the reference's tests/bench_cpu_expert_mt.cpp:69-116 (workers pull whole experts from an atomic counter,
+// gate -> up -> down per expert, one warm pass, `reps` timed passes), on this build's bank formats. The int8 variant
+// quantises the input per 32-block (scale amax/127) and takes integer dots with the block's integer codes, as
+// src/experts/cpu_expert_matvec.cpp:200-280 does for IQ4_NL; the fp32 variant decodes and multiplies in fp32.
+namespace {
+
+// integer image of one 32-weight block: w = scale * q + offset (offset only for Q4_K)
+struct BlockI8 { int8_t q[32]; float scale, offset; };
+
+inline void block_image(uint32_t type, const uint8_t * super, int ib, BlockI8 & o) {
+    o.offset = 0.f;
+    switch (type) {
+        case TQO_IQ4_XS: {
+            o.scale = tqo_half_to_float(rd16(super)) * float(iq4xs_subscale(super, ib) - 32);
+            const uint8_t * q = super + 8 + 16 * ib;
+            for (int j = 0; j < 16; ++j) { o.q[j] = kIq4Values[q[j] & 15]; o.q[16 + j] = kIq4Values[q[j] >> 4]; }
+            break;
+        }
+        case TQO_IQ4_NL: {
+            o.scale = tqo_half_to_float(rd16(super));
+            for (int j = 0; j < 16; ++j) { o.q[j] = kIq4Values[super[2 + j] & 15]; o.q[16 + j] = kIq4Values[super[2 + j] >> 4]; }
+            break;
+        }
+        case TQO_Q4_K: {
+            int sc, mn;
+            q4k_scale_min(super + 4, ib, sc, mn);
+            o.scale = tqo_half_to_float(rd16(super)) * float(sc);
+            o.offset = -(tqo_half_to_float(rd16(super + 2)) * float(mn));
+            const uint8_t * q = super + 16 + 32 * (ib / 2);
+            for (int l = 0; l < 32; ++l) o.q[l] = int8_t((ib & 1) ? q[l] >> 4 : q[l] & 15);
+            break;
+        }
+        case TQO_IQ3_S: {
+            o.scale = tqo_half_to_float(rd16(super)) * float(1 + 2 * ((super[106 + ib / 2] >> (4 * (ib & 1))) & 15));
+            for (int w = 0; w < 8; ++w) {
+                const uint32_t g = tq_iq3s_point(super[2 + 8 * ib + w] | (((super[66 + ib] >> w) & 1) << 8));
+                const int sg = super[74 + 4 * ib + w / 2] >> (4 * (w & 1));
+                for (int j = 0; j < 4; ++j) { const int m = (g >> (8 * j)) & 255; o.q[4 * w + j] = int8_t(((sg >> j) & 1) ? -m : m); }
+            }
+            break;
+        }
+        default: {  // NVFP4G: two 16-groups per 32 weights are handled by the caller through the fp32 path
+            o.scale = 0.f;
+            std::memset(o.q, 0, 32);
+        }
+    }
+}
+
+struct XQ { std::vector<int8_t> q; std::vector<float> scale; std::vector<int> sum; };
+
+void quant_x_blocks(const float * x, int cols, XQ & o) {
+    o.q.resize(static_cast<size_t>(cols));
+    o.scale.resize(size_t(cols / 32));
+    o.sum.resize(size_t(cols / 32));
+    for (int b = 0; b < cols / 32; ++b) {
+        float m = 0.f;
+        for (int i = 0; i < 32; ++i) m = std::max(m, std::fabs(x[32 * b + i]));
+        o.scale[size_t(b)] = m / 127.f;
+        const float mul = m > 0.f ? 127.f / m : 0.f;
+        int s = 0;
+        for (int i = 0; i < 32; ++i) { const int v = int(std::nearbyint(x[32 * b + i] * mul)); o.q[size_t(32 * b + i)] = int8_t(v); s += v; }
+        o.sum[size_t(b)] = s;
+    }
+}
+
+void matvec(uint32_t type, const uint8_t * W, int rows, int cols, const float * x, const XQ * xq, float * y) {
+    int elems, bytes;
+    tqo_block_layout(type, &elems, &bytes);
+    const size_t row_bytes = size_t(cols / elems) * bytes;
+    std::vector<float> dec(static_cast<size_t>(elems));
+    for (int r = 0; r < rows; ++r) {
+        const uint8_t * row = W + row_bytes * r;
+        float acc = 0.f;
+        if (xq && type != TQO_NVFP4G) {
+            BlockI8 bi;
+            for (int b = 0; b < cols / 32; ++b) {
+                const uint8_t * super = row + size_t((32 * b) / elems) * bytes;
+                block_image(type, super, (32 * b % elems) / 32, bi);
+                const int8_t * q = xq->q.data() + 32 * b;
+                int dot = 0;
+                for (int i = 0; i < 32; ++i) dot += int(bi.q[i]) * int(q[i]);
+                acc += xq->scale[size_t(b)] * (bi.scale * float(dot) + bi.offset * float(xq->sum[size_t(b)]));
+            }
+        } else {
+            for (int b = 0; b < cols / elems; ++b) {
+                tqo_dequantize(type, row + size_t(b) * bytes, dec.data(), elems);
+                float part = 0.f;
+                for (int i = 0; i < elems; ++i) part += dec[size_t(i)] * x[b * elems + i];
+                acc += part;
+            }
+        }
+        y[r] = acc;
+    }
+}
+
+}  // namespace
+
+int tqo_hardware_threads(void) { return int(std::thread::hardware_concurrency()); }
+
+double tqo_cpu_expert_bench(uint32_t wtype, const void * gate, const void * up, const void * down, int hidden, int ff,
+                            int n_expert, int threads, int int8_act, int reps, float * checksum) {
+    int elems, bytes;
+    if (!tqo_block_layout(wtype, &elems, &bytes) || hidden % elems || ff % elems || n_expert <= 0 || threads <= 0 || reps <= 0) return -1.0;
+    const size_t stride = size_t(int64_t(ff) * hidden / elems) * bytes;
+    std::vector<float> sums(static_cast<size_t>(n_expert), 0.f);
+    auto pass = [&]() {
+        std::atomic<int> next{0};
+        auto worker = [&]() {
+            std::vector<float> x(static_cast<size_t>(hidden), 0.5f), g(static_cast<size_t>(ff)), u(static_cast<size_t>(ff)), act(static_cast<size_t>(ff)), y(static_cast<size_t>(hidden));
+            XQ xq, aq;
+            for (;;) {
+                const int e = next.fetch_add(1);
+                if (e >= n_expert) break;
+                for (int i = 0; i < hidden; ++i) x[size_t(i)] = 0.5f + 0.001f * float((i + e) & 15);
+                if (int8_act) quant_x_blocks(x.data(), hidden, xq);
+                matvec(wtype, static_cast<const uint8_t *>(gate) + stride * e, ff, hidden, x.data(), int8_act ? &xq : nullptr, g.data());
+                matvec(wtype, static_cast<const uint8_t *>(up) + stride * e, ff, hidden, x.data(), int8_act ? &xq : nullptr, u.data());
+                for (int o = 0; o < ff; ++o) act[size_t(o)] = (g[size_t(o)] / (1.f + std::exp(-g[size_t(o)]))) * u[size_t(o)];
+                if (int8_act) quant_x_blocks(act.data(), ff, aq);
+                matvec(wtype, static_cast<const uint8_t *>(down) + stride * e, hidden, ff, act.data(), int8_act ? &aq : nullptr, y.data());
+                float s = 0.f;
+                for (int i = 0; i < hidden; ++i) s += y[size_t(i)];
+                sums[size_t(e)] = s;
+            }
+        };
+        std::vector<std::thread> pool;
+        for (int i = 1; i < threads; ++i) pool.emplace_back(worker);
+        worker();
+        for (auto & th : pool) th.join();
+    };
+    pass();
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int r = 0; r < reps; ++r) pass();
+    const auto t1 = std::chrono::steady_clock::now();
+    if (checksum) { float s = 0.f; for (float v : sums) s += v; *checksum = s; }
+    return std::chrono::duration<double>(t1 - t0).count() / reps;
+}

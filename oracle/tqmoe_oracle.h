@@ -1,0 +1,131 @@
+/* CPU oracle for the mixture-of-experts layer: TEST INFRASTRUCTURE ONLY.
+ *
+ * A plain, single-purpose restatement of the reference's host algorithms for this path. Only tests, the smoke check
+ * and the CPU-baseline leg of the benchmark may link or load it; the product library never does.
+ *
+ * What each function follows in the reference (paths relative to the reference tree):
+ *   tqo_half_to_float / tqo_float_to_half  src/formats/weight/dequant.cpp:12-54
+ *   tqo_e4m3_to_float                      src/formats/weight/dequant.cpp:387-391
+ *   tqo_dequantize  Q4_K                   src/formats/weight/dequant.cpp:56-64, 80-99
+ *                   IQ3_S                  src/formats/weight/dequant.cpp:133-150
+ *                   IQ4_XS                 src/formats/weight/dequant.cpp:176-192
+ *                   IQ4_NL                 src/formats/weight/dequant.cpp:351-360
+ *                   NVFP4G                 src/formats/weight/dequant.cpp:397-409
+ *   tqo_route                              src/experts/moe.cpp:22-113 (softmax / sigmoid gating, selection bias,
+ *                                          stable top-k, unbiased weights, clamp 6.103515625e-5, scale)
+ *   tqo_shared_weight                      src/experts/moe.cu:92 (sigmoid of logits column E)
+ *   tqo_dispatch                           src/models/qwen/qwen4exp/prefill_plan.hpp:63-74 (ascending assignment
+ *                                          order inside each expert), counts as src/experts/moe.cu:168-176
+ *   tqo_expert_ffn                         src/experts/moe.cpp:115-155
+ *   tqo_combine                            src/experts/moe.cpp:157-163 and src/experts/moe.cu:224-234 (shared row)
+ *   tqo_router_logits                      src/experts/moe.cu:17-33 (row E = shared gate), bf16 variant
+ *                                          src/models/qwen/qwen4exp/qwen4exp.cu:1629-1659
+ *   tqo_layer_forward                      tests/glm_expert_bank.cu:166-184 (dequantise, route, FFN per selected
+ *                                          expert, combine)
+ *   tqo_quant_act_row_i8                   src/formats/weight/quant_u4h.inc:790-820 (per-token mode: scale m/127)
+ *   tqo_quant_act_row_e4m3                 src/core/fp8_gemm.cuh:19-20 (per-row scale amax/448)
+ *
+ * Pinned by: tests/golden/kquant_golden.bin (gguf-py values, bit for bit) for Q4_K / IQ3_S / IQ4_XS / IQ4_NL; the
+ * 65,536 halves against hardware conversion; the 256 E4M3 codes against the closed form; NVFP4G against the closed
+ * form value = e2m1 * e4m3(scale) * global; routing against an independent max-scan selection, scipy softmax and
+ * the closed forms of the reference's tests/moe.cpp; dispatch against a brute-force stable sort; FFN / combine /
+ * layer against float64 numpy on the decoded weights; and, where it builds, against the reference's own objects in
+ * oracle/_ref.
+ *
+ * PARITY UNPINNED: tqo_quantize (all formats). The reference holds no quantiser (it calls an external libggml that
+ * is not in its tree); the encoders here are this build's own and are checked only through round trip and block
+ * validity. Layer parity is defined on decoded values, so the encoder changes the weight distribution, not the
+ * pass criterion.
+ */
+#ifndef TQMOE_ORACLE_H
+#define TQMOE_ORACLE_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GGUF tensor type ids (src/core/gguf.hpp) */
+enum { TQO_F32 = 0, TQO_F16 = 1, TQO_Q4_K = 12, TQO_IQ4_NL = 20, TQO_IQ3_S = 21, TQO_IQ4_XS = 23, TQO_BF16 = 30,
+       TQO_NVFP4G = 323 };
+/* gating (src/experts/moe.hpp:20-26) */
+enum { TQO_GATE_SOFTMAX = 1, TQO_GATE_SIGMOID = 2 };
+
+float    tqo_half_to_float(uint16_t h);
+uint16_t tqo_float_to_half(float f);
+float    tqo_bf16_to_float(uint16_t h);
+uint16_t tqo_float_to_bf16(float f);          /* round to nearest even */
+float    tqo_e4m3_to_float(uint8_t b);
+uint8_t  tqo_float_to_e4m3(float f);          /* round to nearest even, saturating at +-448 */
+
+/* block layout: weights per block and bytes per block; returns 0 when the type is not one of the five */
+int tqo_block_layout(uint32_t type, int * elems, int * bytes);
+/* n weights (a multiple of the block size) from GGUF blocks to fp32; returns 0 on success */
+int tqo_dequantize(uint32_t type, const void * src, float * dst, int64_t n);
+/* n fp32 weights to GGUF blocks (this build's own encoders: parity unpinned); for NVFP4G `row` = weights per
+ * matrix row (one global scale per row). Returns 0 on success. */
+int tqo_quantize(uint32_t type, const float * src, void * dst, int64_t n, int64_t row);
+
+/* routing of one token: logits[E] (+ optional selection bias[E]) -> ids[k] (descending selection value, ties to
+ * the lower index) and weights[k] */
+int tqo_route(int gating, int n_expert, int k, int norm_weights, float weight_scale, const float * logits,
+              const float * bias, int32_t * ids, float * weights);
+/* smallest gap, in units of the larger value's ulp, between neighbouring selection values among the k + 1 largest
+ * (softmax probabilities as tqo_route computes them); a token with a gap of a few ulp is a near tie, where an
+ * exp() that rounds differently may order the pair differently. Equal values (true ties) are skipped. */
+double tqo_route_min_gap_ulps(int n_expert, int k, const float * logits);
+float tqo_shared_weight(float logit);
+
+/* stable dispatch: counts[E], offsets[E + 1] (exclusive scan), perm[A] = assignment indices grouped by expert in
+ * ascending order inside each expert; ids < 0 are skipped (offsets[E] = number kept) */
+int tqo_dispatch(const int32_t * ids, int A, int E, int32_t * counts, int32_t * offsets, int32_t * perm);
+
+void tqo_expert_ffn(const float * x, int hidden, const float * w_gate, const float * w_up, const float * w_down,
+                    int ff, float swiglu_clamp, int clamp_gate, float * out);
+/* out[hidden] += sum_s weights[s] * expert_outs[s][hidden] */
+void tqo_combine(const int k, const float * weights, const float * expert_outs, int hidden, float * out);
+
+/* logits[n][E + 1] = W x, row E from `shared_gate` (may be null: column E = 0). wtype / xtype: TQO_F32, TQO_BF16 or
+ * TQO_F16 storage; products and sums in fp32, j ascending. */
+int tqo_router_logits(const void * w, uint32_t wtype, const void * shared_gate, const void * x, uint32_t xtype,
+                      int hidden, int E, int n, float * logits);
+
+/* Declared activation quantisers of the lossy operand paths. */
+void tqo_quant_act_row_i8(const float * x, int cols, int8_t * q, float * scale);     /* scale = amax/127 */
+void tqo_quant_act_row_e4m3(const float * x, int cols, uint8_t * q, float * scale);  /* scale = amax/448 */
+
+/* Whole layer on the host.
+ *   x fp32 [n][H] (already rounded to the activation type by the caller), logits [n][E + 1] given (so that the
+ *   routing of a device run can be replayed on the device's own logits), banks = GGUF blocks [E (+1)][rows][cols]
+ *   for gate, up ([F][H]) and down ([H][F]); shared expert = expert index E of the same banks when has_shared,
+ *   its FFN size shared_ff <= F (the first shared_ff rows / columns), weighted by sigmoid(logits[.][E]).
+ *   act_mode: 0 = fp32 activations (oracle A); 1 = gate/up inputs and down inputs per-row int8 (oracle B of the
+ *   int8 path); 2 = per-row E4M3 inputs and weights rounded to E4M3 after a power-of-two row scale (oracle B of the
+ *   fp8 path); 3 = mode 1 with the weights widened to int8 per (row, 256-weight super-block).
+ *   out fp32 [n][H]; ids_out [n][k], weights_out [n][k] may be null. threads: worker threads over tokens.
+ */
+typedef struct tqo_layer {
+    int hidden, ff, n_expert, k, has_shared, shared_ff;
+    uint32_t wtype;
+    const void * gate, * up, * down;
+    int act_mode;
+    int threads;
+} tqo_layer;
+int tqo_layer_forward(const tqo_layer * L, const float * x, const float * logits, int n, float * out,
+                      int32_t * ids_out, float * weights_out);
+
+/* int8 widening of one decoded weight row segment (256 weights): q = rint(w * 127 / amax), scale = amax / 127
+ * (scale 0 and q 0 for an all-zero segment). The declared weight operand of the int8 MFMA path. */
+void tqo_widen_i8_256(const float * w, int8_t * q, float * scale);
+
+/* CPU baseline (port of the reference's tests/bench_cpu_expert_mt.cpp scheme onto an arbitrary bank format):
+ * `threads` workers pull experts from an atomic counter; each expert = gate, up, down matvec of one token with
+ * per-32-block int8 activations (int8_act = 1) or fp32 activations (0). Returns seconds per pass over n_expert
+ * experts, averaged over `reps` passes after one warm pass. */
+double tqo_cpu_expert_bench(uint32_t wtype, const void * gate, const void * up, const void * down, int hidden, int ff,
+                            int n_expert, int threads, int int8_act, int reps, float * checksum);
+int tqo_hardware_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

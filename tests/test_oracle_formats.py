@@ -1,0 +1,188 @@
+"""Pins the oracle's conversions and block decoders: golden vectors of the reference's own tests
+(tests/data/kquant_golden.bin, gguf-py values), exhaustive conversions against hardware / closed forms, the NVFP4G
+closed form, and, where built, the reference's own objects. Encoders (this build's own: parity unpinned) are held
+to round-trip error and block validity only."""
+import ctypes as C
+import os
+import struct
+
+import numpy as np
+import pytest
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "kquant_golden.bin")
+
+
+def golden_records():
+    b = open(GOLDEN, "rb").read()
+    o = 0
+    while o < len(b):
+        t, nb, bb, el = struct.unpack_from("<4I", b, o)
+        o += 16
+        raw = np.frombuffer(b, np.uint8, nb * bb, o)
+        o += nb * bb
+        vals = np.frombuffer(b, np.float32, nb * el, o)
+        o += nb * el * 4
+        yield t, nb, bb, el, raw, vals
+
+
+def test_golden_file_holds_the_path_types():
+    types = [r[0] for r in golden_records()]
+    assert types == [10, 11, 12, 13, 21, 23, 20]
+
+
+@pytest.mark.parametrize("wtype", [12, 21, 23, 20])
+def test_decoders_match_golden_bit_for_bit(oracle, wtype):
+    for t, nb, bb, el, raw, vals in golden_records():
+        if t != wtype:
+            continue
+        assert oracle.BLOCK[t] == (el, bb)
+        got = oracle.dequantize(t, raw, nb * el)
+        assert np.array_equal(got.view(np.uint32), vals.view(np.uint32))
+        return
+    pytest.fail("type not in the golden file")
+
+
+def test_half_to_float_exhaustive(oracle):
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([oracle.half_to_float(int(v)) for v in h], np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    assert np.isnan(got[nan]).all()
+
+
+def test_float_to_half_against_hardware(oracle):
+    rng = np.random.default_rng(1)
+    cases = np.concatenate([
+        np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32),        # every half, exactly
+        rng.standard_normal(20000).astype(np.float32) * 10.0 ** rng.uniform(-9, 6, 20000).astype(np.float32),
+        np.array([65504.0, 65519.99, 65520.0, 1e9, 5.96e-8, 2.98e-8, 2.9802322e-8, 2.99e-8, 6.1e-5, 0.0, -0.0], np.float32),
+    ])
+    cases = cases[~np.isnan(cases)]
+    # halfway cases between neighbouring halves (ties to even)
+    hs = np.arange(0, 0x7BFF, dtype=np.uint16)
+    mid = (hs.view(np.float16).astype(np.float64) + (hs + 1).astype(np.uint16).view(np.float16).astype(np.float64)) / 2
+    cases = np.concatenate([cases, mid.astype(np.float32)])
+    with np.errstate(over="ignore"):
+        want = cases.astype(np.float16).view(np.uint16)
+    got = np.array([oracle.float_to_half(float(v)) for v in cases], np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_e4m3_closed_form(oracle):
+    for b in range(256):
+        e, m = (b >> 3) & 15, b & 7
+        v = oracle.e4m3_to_float(b)
+        if e == 15 and m == 7:
+            assert np.isnan(v)
+            continue
+        want = (m / 8 * 2.0 ** -6) if e == 0 else (1 + m / 8) * 2.0 ** (e - 7)
+        assert v == (-want if b & 0x80 else want)
+    assert oracle.e4m3_to_float(0x7E) == 448.0
+
+
+def test_float_to_e4m3_is_nearest_even(oracle):
+    codes = [b for b in range(127)]  # positive finite codes, ascending in value
+    vals = np.array([oracle.e4m3_to_float(b) for b in codes])
+    assert (np.diff(vals) > 0).all()
+    for b in codes:
+        assert oracle.float_to_e4m3(vals[b]) == b
+        assert oracle.float_to_e4m3(-vals[b]) == (b | 0x80)
+    rng = np.random.default_rng(2)
+    for v in np.concatenate([rng.uniform(0, 460, 4000), rng.uniform(0, 0.05, 2000), (vals[:-1] + vals[1:]) / 2]):
+        v = float(np.float32(v))
+        got = oracle.float_to_e4m3(v)
+        d = np.abs(vals - min(v, 448.0))
+        best = np.flatnonzero(d == d.min())
+        if len(best) == 2:  # exact tie: even mantissa code
+            want = best[0] if best[0] % 2 == 0 else best[1]
+        else:
+            want = best[0]
+        assert got == want, (v, got, want)
+
+
+def test_nvfp4g_closed_form(oracle):
+    rng = np.random.default_rng(3)
+    e2m1 = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6], np.float32)
+    nb = 12
+    raw = rng.integers(0, 256, (nb, 76), dtype=np.uint8)
+    raw[:, 4:12] &= 0x7E                      # finite, positive scales
+    g = rng.uniform(1e-3, 2e-2, nb).astype(np.float32)
+    raw[:, 0:4] = g.view(np.uint8).reshape(nb, 4)
+    got = oracle.dequantize(oracle.NVFP4G, raw, nb * 128).reshape(nb, 128)
+    for b in range(nb):
+        for grp in range(8):
+            d = np.float32(oracle.e4m3_to_float(raw[b, 4 + grp])) * g[b]
+            q = raw[b, 12 + 8 * grp:20 + 8 * grp]
+            want = np.empty(16, np.float32)
+            want[0::2] = e2m1[q & 15] * d     # low nibble = even weight
+            want[1::2] = e2m1[q >> 4] * d
+            assert np.array_equal(got[b, 16 * grp:16 * grp + 16], want)
+
+
+def test_iq4xs_independent_decode(oracle):
+    """Second, independently written IQ4_XS decode (vectorised numpy over the raw layout)."""
+    rng = np.random.default_rng(4)
+    kv = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)
+    nb = 40
+    raw = rng.integers(0, 256, (nb, 136), dtype=np.uint8)
+    raw[:, 0:2] = np.float16(rng.uniform(1e-3, 5e-2, nb)).view(np.uint8).reshape(nb, 2)
+    d = raw[:, 0:2].copy().view(np.float16).astype(np.float32)[:, 0]
+    sh = raw[:, 2:4].copy().view(np.uint16)[:, 0].astype(np.int32)
+    ib = np.arange(8)
+    lo = (raw[:, 4:8].astype(np.int32)[:, ib // 2] >> (4 * (ib % 2))) & 15
+    ls = lo | (((sh[:, None] >> (2 * ib)) & 3) << 4)
+    dl = d[:, None] * (ls - 32).astype(np.float32)
+    qs = raw[:, 8:].reshape(nb, 8, 16)
+    want = np.concatenate([dl[:, :, None] * kv[qs & 15], dl[:, :, None] * kv[qs >> 4]], axis=2).reshape(nb, 256)
+    got = oracle.dequantize(oracle.IQ4_XS, raw, nb * 256).reshape(nb, 256)
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+@pytest.mark.parametrize("wtype", [12, 20, 21, 23, 323])
+def test_decoders_match_reference_objects(oracle, ref, wtype):
+    rng = np.random.default_rng(wtype)
+    el, bb = oracle.BLOCK[wtype]
+    nb = 64
+    raw = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
+    halves = {12: [0, 2], 20: [0], 21: [0], 23: [0]}.get(wtype, [])
+    for off in halves:
+        raw[:, off:off + 2] = np.float16(rng.uniform(1e-3, 5e-2, nb) * rng.choice([-1, 1], nb)).view(np.uint8).reshape(nb, 2)
+    if wtype == 323:
+        raw[:, 0:4] = rng.uniform(1e-3, 2e-2, nb).astype(np.float32).view(np.uint8).reshape(nb, 4)
+    got = oracle.dequantize(wtype, raw, nb * el)
+    want = np.empty(nb * el, np.float32)
+    assert ref.ref_dequantize(wtype, raw.ctypes.data_as(C.c_void_p), want.ctypes.data_as(C.c_void_p), nb * el) == 0
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))  # NaNs (E4M3 0x7F scales) compare by bits
+
+
+def test_conversions_match_reference_objects(oracle, ref):
+    for h in range(0, 65536, 7):
+        a, b = oracle.half_to_float(h), ref.ref_half_to_float(h)
+        assert (np.isnan(a) and np.isnan(b)) or a == b
+    rng = np.random.default_rng(5)
+    for v in rng.standard_normal(5000).astype(np.float32) * 10.0 ** rng.uniform(-9, 6, 5000).astype(np.float32):
+        assert oracle.float_to_half(float(v)) == ref.ref_float_to_half(float(v))
+    for b in range(256):
+        a, r = oracle.e4m3_to_float(b), ref.ref_e4m3_to_float(b)
+        assert (np.isnan(a) and np.isnan(r)) or a == r
+
+
+# relative round-trip error (rms(decode(encode(w)) - w) / rms(w)) each encoder must stay under on N(0, 0.02) weights
+ROUND_TRIP = {12: 0.09, 20: 0.09, 23: 0.09, 21: 0.20, 323: 0.12}
+
+
+@pytest.mark.parametrize("wtype", sorted(ROUND_TRIP))
+def test_encoders_round_trip(oracle, wtype):
+    rng = np.random.default_rng(100 + wtype)
+    w = (rng.standard_normal((16, 1024)) * 0.02).astype(np.float32)
+    raw = oracle.quantize(wtype, w)
+    el, bb = oracle.BLOCK[wtype]
+    assert raw.size == w.size // el * bb
+    back = oracle.dequantize(wtype, raw, w.size).reshape(w.shape)
+    assert np.isfinite(back).all()
+    rel = np.sqrt(np.mean((back - w) ** 2) / np.mean(w ** 2))
+    assert rel < ROUND_TRIP[wtype], rel
+    # zeros encode to blocks that decode to zeros
+    z = oracle.dequantize(wtype, oracle.quantize(wtype, np.zeros((1, 1024), np.float32)), 1024)
+    assert not z.any()

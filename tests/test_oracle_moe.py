@@ -1,0 +1,276 @@
+"""Pins the oracle's routing, dispatch, FFN, combine and whole-layer functions against checks the mathematics fixes
+(independent max-scan selection, scipy softmax, closed forms and invariants of the reference's tests/moe.cpp, brute
+force sorts, float64 numpy) and, where built, the reference's own objects."""
+import ctypes as C
+
+import numpy as np
+import pytest
+from scipy.special import softmax
+
+
+def max_scan_route(logits, k, gating, norm, scale, bias):
+    """Independent reference: repeated strict-greater max scan with a taken mask (the scheme of the reference's
+    tests/moe.cpp:36-89), float32 arithmetic through numpy scalars."""
+    lg = logits.astype(np.float32)
+    if gating == 1:
+        mx = lg.max()
+        p = np.exp(lg - mx, dtype=np.float32)
+        s = np.float32(0)
+        for v in p:
+            s = np.float32(s + v)
+        p = (p / s).astype(np.float32)
+    else:
+        p = (np.float32(1) / (np.float32(1) + np.exp(-lg, dtype=np.float32))).astype(np.float32)
+    sel = p + bias.astype(np.float32) if bias is not None else p
+    taken = np.zeros(len(lg), bool)
+    ids, w = [], []
+    for _ in range(k):
+        best, bv = -1, -np.inf
+        for i, v in enumerate(sel):
+            if not taken[i] and v > bv:
+                best, bv = i, v
+        taken[best] = True
+        ids.append(best)
+        w.append(p[best])
+    w = np.array(w, np.float32)
+    if norm:
+        s = np.float32(0)
+        for v in w:
+            s = np.float32(s + v)
+        w = (w / max(s, np.float32(6.103515625e-5))).astype(np.float32)
+    if scale not in (0.0, 1.0):
+        w = (w * np.float32(scale)).astype(np.float32)
+    return np.array(ids, np.int32), w
+
+
+def test_route_matches_independent_max_scan(oracle):
+    rng = np.random.default_rng(11)
+    for gating in (1, 2):
+        for norm in (False, True):
+            for biased in (False, True):
+                for _ in range(60):
+                    e = int(rng.integers(2, 62))
+                    k = int(rng.integers(1, e + 1))
+                    scale = float(np.float32(rng.uniform(0.01, 4)))
+                    lg = rng.uniform(-8, 8, e).astype(np.float32)
+                    bias = rng.uniform(-1, 1, e).astype(np.float32) if biased else None
+                    ids, w = oracle.route(lg, k, gating, norm, scale, bias)
+                    wi, ww = max_scan_route(lg, k, gating, norm, scale, bias)
+                    assert np.array_equal(ids[0], wi)
+                    assert np.abs(w[0] - ww).max() <= 1e-6
+
+
+def test_route_softmax_against_scipy(oracle):
+    rng = np.random.default_rng(12)
+    for e, k in ((64, 8), (512, 10), (256, 8)):
+        lg = rng.standard_normal((20, e)).astype(np.float32)
+        ids, w = oracle.route(lg, k)
+        p = softmax(lg.astype(np.float64), axis=1)
+        for t in range(20):
+            order = np.lexsort((np.arange(e), -p[t]))[:k]
+            assert np.array_equal(ids[t], order)
+            want = p[t, order] / p[t, order].sum()
+            assert np.abs(w[t] - want).max() < 3e-7
+            assert abs(float(w[t].sum()) - 1) < 1e-6
+            assert (np.diff(w[t]) <= 0).all()          # descending probability order
+
+
+def test_route_closed_forms(oracle):
+    # all-equal logits: lowest indices win (tests/moe.cpp:183-194)
+    ids, w = oracle.route(np.full(8, 0.5, np.float32), 3, gating=2, norm=False)
+    assert ids[0].tolist() == [0, 1, 2]
+    ids, w = oracle.route(np.full(512, -3.25, np.float32), 10)
+    assert ids[0].tolist() == list(range(10)) and np.allclose(w[0], 0.1, atol=1e-7)
+    # underflow: every sigmoid exactly 0, weights stay finite (tests/moe.cpp:196-210)
+    ids, w = oracle.route(np.array([-200, -300, -400, -500], np.float32), 4, gating=2, norm=True)
+    assert np.isfinite(w).all() and not w.any()
+    # scale 0 and 1 both mean no scaling; 2.5 multiplies (tests/moe.cpp:212-236)
+    lg = np.array([3, 1, -1, -3], np.float32)
+    i0, w0 = oracle.route(lg, 2, gating=2, norm=True, scale=0.0)
+    i1, w1 = oracle.route(lg, 2, gating=2, norm=True, scale=1.0)
+    i2, w2 = oracle.route(lg, 2, gating=2, norm=True, scale=2.5)
+    assert np.array_equal(w0, w1) and abs(w1.sum() - 1) < 1e-6 and abs(w2.sum() - 2.5) < 1e-6
+    assert np.abs(w2 - 2.5 * w1).max() < 1e-6
+    # selection bias moves the choice, not the weight (tests/moe.cpp:149-176)
+    ids, w = oracle.route(np.array([2, 1, 0, -1], np.float32), 2, gating=2, norm=False, bias=np.array([0, 0, 0, 100], np.float32))
+    assert ids[0, 0] == 3 and abs(w[0, 0] - 1 / (1 + np.exp(1.0))) < 1e-6
+    # softmax with far-apart logits: exp underflows to exact zeros, ties among zeros go to the lower index
+    ids, w = oracle.route(np.array([0, -200, 50, -300, -250], np.float32), 3)
+    assert ids[0].tolist() == [2, 0, 1] and w[0, 0] == 1.0 and w[0, 2] == 0.0
+    assert oracle.shared_weight(0.0) == 0.5 and oracle.shared_weight(-1e30) == 0.0
+    assert abs(oracle.shared_weight(1.25) - 1 / (1 + np.exp(-1.25))) < 1e-7
+
+
+def test_route_matches_reference_objects(oracle, ref):
+    rng = np.random.default_rng(13)
+    for gating in (1, 2):
+        for _ in range(200):
+            e = int(rng.integers(2, 600))
+            k = int(rng.integers(1, min(e, 16) + 1))
+            lg = (rng.standard_normal(e) * rng.uniform(0.1, 6)).astype(np.float32)
+            bias = rng.uniform(-1, 1, e).astype(np.float32) if rng.random() < 0.5 else None
+            scale = float(np.float32(rng.choice([0.0, 1.0, 2.5])))
+            ids, w = oracle.route(lg, k, gating, True, scale, bias)
+            ri = np.empty(k, np.int32)
+            rw = np.empty(k, np.float32)
+            bp = bias.ctypes.data_as(C.c_void_p) if bias is not None else None
+            assert ref.ref_route(gating, e, k, 1, scale, lg.ctypes.data_as(C.c_void_p), bp, ri.ctypes.data_as(C.c_void_p),
+                                 rw.ctypes.data_as(C.c_void_p)) == 0
+            assert np.array_equal(ids[0], ri)
+            assert np.array_equal(w[0].view(np.uint32), rw.view(np.uint32))   # same libm, same order: bit for bit
+
+
+def test_min_gap_flags_near_ties(oracle):
+    lg = np.zeros(16, np.float32)
+    lg[:4] = [3.0, 2.0, np.nextafter(np.float32(2.0), np.float32(0)), 1.0]
+    assert oracle.route_min_gap_ulps(lg, 3)[0] < 4
+    assert oracle.route_min_gap_ulps(np.arange(16, dtype=np.float32), 3)[0] > 1e5
+
+
+def test_dispatch_brute_force(oracle):
+    rng = np.random.default_rng(14)
+    for e, a in ((4, 0), (4, 1), (64, 128), (512, 40960), (7, 1000)):
+        ids = rng.integers(-1 if a > 10 else 0, e, a).astype(np.int32)
+        counts, offsets, perm = oracle.dispatch(ids, e)
+        kept = np.flatnonzero(ids >= 0)
+        assert np.array_equal(counts, np.bincount(ids[kept], minlength=e))
+        assert offsets[0] == 0 and np.array_equal(np.diff(offsets), counts) and offsets[-1] == len(kept)
+        want = kept[np.argsort(ids[kept], kind="stable")]
+        assert np.array_equal(perm[:len(kept)], want)
+        assert (perm[len(kept):] == -1).all()
+        for x in range(e):  # ascending assignment order inside each expert (prefill_plan.hpp:69-73)
+            seg = perm[offsets[x]:offsets[x + 1]]
+            assert (np.diff(seg) > 0).all() and (ids[seg] == x).all()
+    with pytest.raises(ValueError):
+        oracle.dispatch(np.array([0, 9], np.int32), 4)
+
+
+def test_expert_ffn_against_float64(oracle, ref):
+    rng = np.random.default_rng(15)
+    h, f = 96, 40
+    x = rng.standard_normal(h).astype(np.float32)
+    wg, wu = (rng.standard_normal((f, h)).astype(np.float32) * 0.2 for _ in range(2))
+    wd = rng.standard_normal((h, f)).astype(np.float32) * 0.2
+    g, u = wg.astype(np.float64) @ x, wu.astype(np.float64) @ x
+    want = wd.astype(np.float64) @ (g / (1 + np.exp(-g)) * u)
+    got = oracle.expert_ffn(x, wg, wu, wd)
+    assert np.abs(got - want).max() < 1e-5
+    # clamp branches (moe.cpp:133-143): GLM clamps gate, generic clamps silu(gate); both clamp up
+    xc = x * 40
+    g, u = wg.astype(np.float64) @ xc, np.clip(wu.astype(np.float64) @ xc, -7, 7)
+    gl = np.minimum(g, 7)
+    want_glm = wd.astype(np.float64) @ (gl / (1 + np.exp(-gl)) * u)
+    want_gen = wd.astype(np.float64) @ (np.minimum(g / (1 + np.exp(-g)), 7) * u)
+    assert np.abs(oracle.expert_ffn(xc, wg, wu, wd, 7.0, True) - want_glm).max() < 1e-3
+    assert np.abs(oracle.expert_ffn(xc, wg, wu, wd, 7.0, False) - want_gen).max() < 1e-3
+    out = np.empty(h, np.float32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    for clamp, cg in ((0.0, 0), (7.0, 1), (7.0, 0)):
+        ref.ref_expert_ffn(p(xc), h, p(wg), p(wu), p(wd), f, clamp, cg, p(out))
+        assert np.array_equal(oracle.expert_ffn(xc, wg, wu, wd, clamp, bool(cg)), out)
+
+
+def test_combine_closed_form(oracle):
+    outs = np.stack([np.arange(1, 5), np.arange(10, 14)]).astype(np.float32)
+    got = oracle.combine(np.array([0.75, 0.25], np.float32), outs)
+    assert np.allclose(got, 0.75 * outs[0] + 0.25 * outs[1], atol=1e-6)
+
+
+def test_router_logits_against_float64(oracle):
+    rng = np.random.default_rng(16)
+    h, e, n = 256, 24, 3
+    w = rng.standard_normal((e, h)).astype(np.float32) * 0.02
+    sg = rng.standard_normal(h).astype(np.float32) * 0.02
+    x = rng.standard_normal((n, h)).astype(np.float32)
+    got = oracle.router_logits(w, oracle.F32, sg, x, oracle.F32, h, e, n)
+    want = x.astype(np.float64) @ np.vstack([w, sg]).astype(np.float64).T
+    assert np.abs(got - want).max() < 3e-6
+    wb, wbf = oracle.to_bf16(w)
+    sb, sbf = oracle.to_bf16(sg)
+    xb, xbf = oracle.to_bf16(x)
+    got = oracle.router_logits(wb, oracle.BF16, sb, xb, oracle.BF16, h, e, n)
+    want = xbf.astype(np.float64) @ np.vstack([wbf, sbf]).astype(np.float64).T
+    assert np.abs(got - want).max() < 3e-6
+    got = oracle.router_logits(w, oracle.F32, None, x, oracle.F32, h, e, n)
+    assert not got[:, e].any()
+
+
+def test_layer_forward_against_float64(oracle):
+    """Whole layer vs float64 numpy on the decoded weights, routing taken from the oracle (ids are pinned above)."""
+    rng = np.random.default_rng(17)
+    h, f, e, k, sf, n = 256, 256, 6, 2, 256, 5
+    for wtype in (oracle.IQ4_XS, oracle.Q4_K):
+        banks = [oracle.quantize(wtype, (rng.standard_normal(((e + 1) * r, c)) * 0.05).astype(np.float32))
+                 for r, c in ((f, h), (f, h), (h, f))]
+        dec = [oracle.dequantize(wtype, b, (e + 1) * f * h).astype(np.float64) for b in banks]
+        wg, wu = dec[0].reshape(e + 1, f, h), dec[1].reshape(e + 1, f, h)
+        wd = dec[2].reshape(e + 1, h, f)
+        x = rng.standard_normal((n, h)).astype(np.float32)
+        logits = rng.standard_normal((n, e + 1)).astype(np.float32)
+        out, ids, w = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=sf, threads=3)
+        ri, rw = oracle.route(logits[:, :e], k)
+        assert np.array_equal(ids, ri) and np.array_equal(w, rw)
+
+        def ffn(j, xv, ff):
+            g, u = wg[j, :ff] @ xv, wu[j, :ff] @ xv
+            return wd[j, :, :ff] @ (g / (1 + np.exp(-g)) * u)
+
+        for t in range(n):
+            want = sum(float(w[t, s]) * ffn(ids[t, s], x[t].astype(np.float64), f) for s in range(k))
+            want = want + 1 / (1 + np.exp(-float(logits[t, e]))) * ffn(e, x[t].astype(np.float64), sf)
+            assert np.abs(out[t] - want).max() < 2e-5 * max(1.0, np.abs(want).max())
+        # no shared expert: that term disappears; linearity in the routed weights
+        out2, _, _ = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=0, threads=1)
+        t = 0
+        want = sum(float(w[t, s]) * ffn(ids[t, s], x[t].astype(np.float64), f) for s in range(k))
+        assert np.abs(out2[t] - want).max() < 2e-5 * max(1.0, np.abs(want).max())
+
+
+def test_declared_quantisers(oracle):
+    rng = np.random.default_rng(18)
+    x = rng.standard_normal(512).astype(np.float32)
+    q, s = oracle.quant_act_row_i8(x)
+    m = np.abs(x).max()
+    assert s == np.float32(m / np.float32(127)) and np.abs(q).max() == 127
+    assert np.array_equal(q, np.rint(x * (np.float32(127) / m)).astype(np.int8))
+    q0, s0 = oracle.quant_act_row_i8(np.zeros(64, np.float32))
+    assert s0 == 0 and not q0.any()
+    q8, s8 = oracle.quant_act_row_e4m3(x)
+    back = np.array([oracle.e4m3_to_float(b) for b in q8]) * s8
+    assert np.abs(back - x).max() <= m / 448 * 16 + 1e-6      # half a step at the top binade (step 32 of 448)
+    assert max(oracle.e4m3_to_float(b & 0x7F) for b in q8) == 448.0
+
+
+def test_cpu_baseline_kernels_agree_with_decode(oracle, ref):
+    """The CPU-baseline matvecs: fp32 variant vs decode + float64 dot; int8 variant within 1e-2 rms-rel (the gates of
+    the reference's tests/test_cpu_expert_matvec.cpp:117-118); the reference's own IQ4_NL kernels agree likewise."""
+    rng = np.random.default_rng(19)
+    h, f, ne = 512, 256, 2
+    for wtype in (oracle.IQ4_XS, oracle.Q4_K, oracle.IQ3_S, oracle.IQ4_NL):
+        banks = [oracle.quantize(wtype, (rng.standard_normal((ne * r, c)) * 0.02).astype(np.float32))
+                 for r, c in ((f, h), (f, h), (h, f))]
+        t0, c0 = oracle.cpu_expert_bench(wtype, *banks, h, f, ne, 2, False, reps=1)
+        t1, c1 = oracle.cpu_expert_bench(wtype, *banks, h, f, ne, 2, True, reps=1)
+        dec = [oracle.dequantize(wtype, b, ne * f * h).astype(np.float64) for b in banks]
+        want = 0.0
+        for e in range(ne):
+            x = 0.5 + 0.001 * ((np.arange(h) + e) & 15)
+            g, u = dec[0].reshape(ne, f, h)[e] @ x, dec[1].reshape(ne, f, h)[e] @ x
+            want += (dec[2].reshape(ne, h, f)[e] @ (g / (1 + np.exp(-g)) * u)).sum()
+        assert abs(c0 - want) < 1e-4 * max(1.0, abs(want)), (wtype, c0, want)
+        assert abs(c1 - want) < 3e-2 * max(1.0, abs(want)), (wtype, c1, want)
+        assert t0 > 0 and t1 > 0
+    # the reference's IQ4_NL kernels on the same blocks
+    rows, cols = 64, 512
+    raw = oracle.quantize(oracle.IQ4_NL, (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32))
+    x = np.float16(rng.standard_normal(cols)).astype(np.float32)
+    wd = oracle.dequantize(oracle.IQ4_NL, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    want = wd @ x.astype(np.float64)
+    y = np.empty(rows, np.float32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    ref.ref_iq4nl_matvec(1, p(raw), rows, cols, p(x), 1, p(y))
+    assert np.array_equal(y, want.astype(np.float32))
+    ref.ref_iq4nl_matvec(0, p(raw), rows, cols, p(x), 1, p(y))
+    assert np.sqrt(np.mean((y - want) ** 2) / np.mean(want ** 2)) < 1e-5
+    ref.ref_iq4nl_matvec(2, p(raw), rows, cols, p(x), 1, p(y))
+    assert np.sqrt(np.mean((y - want) ** 2) / np.mean(want ** 2)) < 1e-2

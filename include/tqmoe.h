@@ -1,0 +1,167 @@
+/* tqmoe: the mixture-of-experts layer of tqLLM for one AMD Instinct MI355X (gfx950), as a C ABI.
+ *
+ * The library is what the reference's `src/experts` free functions (namespace tqllm_cuda, moe_kernels.cuh) and the
+ * expert entry points of `tqllm::WeightFormat` (src/formats/weight/weight_format.hpp) are to its CUDA engine, with
+ * the conventions of the reference's only C ABI (include/tqllm/plugin.h, ABI 2):
+ *   - every pointer named `*_dev` or documented "device" is HIP device memory owned by the caller; streams travel as
+ *     `void *` (a hipStream_t, NULL = the default stream), so this header needs no GPU include;
+ *   - every call only enqueues work on the given stream: no host synchronisation, no allocation, no state kept between
+ *     calls (the one-time constant tables live in the library's own device image);
+ *   - every call returns 0 on success; on failure a negative TQMOE_E_* code, with the reason in `err` when given
+ *     (`err` may be NULL; set err->struct_size = sizeof(tqmoe_error) before the call);
+ *   - assignments whose expert id is negative are skipped and their output rows left untouched
+ *     (src/formats/weight/quant_u4h.inc:443-447).
+ * There is no CPU fallback: without a usable HIP device every compute entry point fails with TQMOE_E_DEVICE.
+ */
+#ifndef TQMOE_H
+#define TQMOE_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TQMOE_ABI_VERSION 1u
+
+/* error record, shaped as plugin.h:9 `tq_error` */
+typedef struct tqmoe_error { uint32_t struct_size; int32_t code; char message[256]; } tqmoe_error;
+enum { TQMOE_OK = 0, TQMOE_E_ARG = -1, TQMOE_E_UNSUPPORTED = -2, TQMOE_E_DEVICE = -3, TQMOE_E_WORKSPACE = -4 };
+
+/* element types (GGUF type ids, src/core/gguf.hpp) */
+enum { TQMOE_F32 = 0, TQMOE_F16 = 1, TQMOE_BF16 = 30 };
+/* bank formats (GGUF type ids) */
+enum { TQMOE_Q4_K = 12, TQMOE_IQ3_S = 21, TQMOE_IQ4_XS = 23, TQMOE_NVFP4G = 323 };
+
+uint32_t tqmoe_abi_version(void);
+
+/* ------------------------------------------------------------------------------------------------ routing
+ * Router logits: logits[t][r] = sum_j W[r][j] * x[t][j] for r < experts, logits[t][experts] = shared_gate . x[t]
+ * (0 when shared_gate is NULL); row stride experts + 1; products and sums in fp32.
+ * Replaces tqllm_cuda::moe_router / moe_router_f32 (src/experts/moe_kernels.cuh:7-10, moe.cu:17-33, 237-247) and
+ * the bf16 segmented GEMV fn_gemv_bf16_segments (src/models/qwen/qwen4exp/qwen4exp.cu:1629-1659).
+ * router: device [experts][hidden] of wtype (F32 or BF16); shared_gate: device [hidden] of wtype or NULL;
+ * x: device [n][hidden] of xtype (F32, F16 or BF16); logits: device [n][experts + 1] fp32. */
+int32_t tqmoe_router(const void * router, uint32_t wtype, const void * shared_gate, const void * x, uint32_t xtype,
+                     float * logits, int32_t hidden, int32_t experts, int32_t n, void * stream, tqmoe_error * err);
+
+/* Softmax over the first `experts` columns, the `topk` largest probabilities (descending, ties to the lower index),
+ * weights = probability / max(sum of the selected, 6.103515625e-5) * (scale == 0 ? 1 : scale), and
+ * shared_weights[t] = sigmoid(logits[t][experts]) (shared_weights may be NULL).
+ * Replaces tqllm_cuda::moe_topk (moe_kernels.cuh:19-20, moe.cu:35-166, 248-260); host meaning: moe_route
+ * (src/experts/moe.cpp:22-113) with Softmax gating, norm_weights, weight_scale = scale. experts <= 4096. */
+int32_t tqmoe_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t experts,
+                   int32_t topk, int32_t n, float scale, void * stream, tqmoe_error * err);
+
+/* Token-to-expert dispatch of the A = n * topk assignments a = t * topk + s:
+ *   counts[e]   assignments of expert e (ids < 0 skipped),
+ *   offsets[e]  exclusive scan of counts, offsets[experts] = number kept,
+ *   perm[i]     assignment indices grouped by expert, ascending inside each expert (a stable counting sort),
+ *   groups      optional (NULL to skip) [experts][capacity] view of the same lists, as the reference's kernels read
+ *               them; capacity >= the largest count, else TQMOE_E_ARG is NOT detectable on the host and the lists
+ *               are truncated at capacity (counts stay exact).
+ * Replaces tqllm_cuda::moe_group (moe_kernels.cuh:29, moe.cu:168-176, 268-273; order there is atomic) and the host
+ * fill_pass_lists (src/models/qwen/qwen4exp/prefill_plan.hpp:63-74; ascending order). The result is deterministic.
+ * workspace: device scratch of tqmoe_dispatch_workspace_bytes(). */
+size_t  tqmoe_dispatch_workspace_bytes(int32_t experts, int32_t n, int32_t topk);
+int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets, int32_t * perm, int32_t * groups,
+                       int32_t capacity, int32_t experts, int32_t n, int32_t topk, void * workspace,
+                       size_t workspace_bytes, void * stream, tqmoe_error * err);
+
+/* -------------------------------------------------------------------------------------------------- banks
+ * A bank is one projection of every expert: `experts` matrices of rows x cols stacked row-wise, expert e at row
+ * e * rows (weight_format.hpp:61 "Stacked weights [experts * rows][cols]"); a non-owning view like tqllm::Mat
+ * (weight_format.hpp:22-28). The library reads its own device layout, made from the raw GGUF block stream by
+ * tqmoe_bank_load (the counterpart of WeightFormat::load, weight_format.hpp:41, and of the loaders in
+ * src/formats/weight/q4.cpp:295-326, 495-530, 577-606, 802-836). Per 32 weights of a row (a sub-block):
+ *   IQ4_XS  codes 16 B: byte j = weights j (low nibble) and j + 16 (high) of the sub-block (GGUF order);
+ *           aux 8 B per 256 weights: d (f16), scales_h (u16), scales_l[4].
+ *   Q4_K    codes 16 B in the same nibble order; aux 16 B per 256 weights: d, dmin (f16), scales[12] as in GGUF.
+ *   IQ3_S   codes 12 B: 8 lattice index bytes then 4 sign bytes; aux 16 B per 256 weights: d (f16), qh[8],
+ *           scales[4], 2 B padding.
+ *   NVFP4G  codes 16 B in the same nibble order (weights j and j + 16 of the sub-block); aux: one E4M3 scale per
+ *           16 weights, [rows_total][cols / 16] bytes, then at the next multiple of 16 bytes rows_total fp32 globals
+ *           (one per row; rows whose blocks disagree are rejected by the reference loader, q4.cpp:519-521, and by
+ *           tqmoe_bank_load through *status).
+ * cols must be a multiple of 256 (128 for NVFP4G). */
+typedef struct tqmoe_bank {
+    uint32_t struct_size;
+    uint32_t type;            /* TQMOE_Q4_K, TQMOE_IQ3_S, TQMOE_IQ4_XS or TQMOE_NVFP4G */
+    int32_t experts;          /* matrices in the bank */
+    int32_t rows, cols;       /* of one expert */
+    const void * codes;       /* device, tqmoe_bank_layout's code_bytes */
+    const void * aux;         /* device, tqmoe_bank_layout's aux_bytes */
+} tqmoe_bank;
+
+/* device bytes of the two planes for rows_total = experts * rows stacked rows */
+int32_t tqmoe_bank_layout(uint32_t type, int64_t rows_total, int32_t cols, size_t * code_bytes, size_t * aux_bytes,
+                          tqmoe_error * err);
+/* gguf_blocks: device copy of the GGUF block stream of [rows_total][cols] (row-major, blocks of a row contiguous).
+ * codes / aux: device outputs. status: optional device int32, set non-zero when a row's data is rejected. */
+int32_t tqmoe_bank_load(uint32_t type, const void * gguf_blocks, int64_t rows_total, int32_t cols, void * codes,
+                        void * aux, int32_t * status, void * stream, tqmoe_error * err);
+/* rows [row0, row0 + nrows) of the stacked matrix as fp32 [nrows][cols]: the bank's decoded values, bit for bit those
+ * of the reference's host decoder dequantize_host (src/formats/weight/dequant.cpp). Counterpart of
+ * WeightFormat::dequant_rows_h (weight_format.hpp:84-86). */
+int32_t tqmoe_bank_dequant(const tqmoe_bank * bank, int64_t row0, int64_t nrows, float * out, void * stream,
+                           tqmoe_error * err);
+
+/* ------------------------------------------------------------------------------------------ decode products
+ * Activation image the decode products read: per 32 values a scale s = amax / 16383 and q = rint(x / s) held as
+ * two int8 planes (q = 128 * hi + lo, 0 <= lo < 128), so that integer dot products with the integer weight codes
+ * reproduce the fp32 product to 2^-15 of the block maximum. One image row is cols * 2 bytes of planes, then
+ * (cols / 32) * 8 bytes of (scale, sum of q * s); tqmoe_act_image_bytes gives the size for n rows. */
+size_t  tqmoe_act_image_bytes(int32_t n, int32_t cols);
+int32_t tqmoe_quant_act(const void * x, uint32_t xtype, int32_t n, int32_t cols, void * image, void * stream,
+                        tqmoe_error * err);
+
+/* y[a][r] = sum_c W[ids[a] * rows + r][c] * x[row(a)][c], a < n * topk, row(a) = a (per_expert_input) or a / topk.
+ * image: activation image of the input rows; y: device [n * topk][rows] of ytype (F32 or BF16).
+ * Replaces WeightFormat::expert_matvec (weight_format.hpp:62-64, src/formats/weight/quant.cu:69-111). */
+int32_t tqmoe_expert_matvec(const tqmoe_bank * bank, const void * image, void * y, uint32_t ytype, const int32_t * ids,
+                            int32_t n, int32_t topk, int32_t per_expert_input, void * stream, tqmoe_error * err);
+/* gate and up over the same ids in one launch (WeightFormat::expert_matvec2, weight_format.hpp:70-73) */
+int32_t tqmoe_expert_matvec2(const tqmoe_bank * gate, const tqmoe_bank * up, const void * image, void * y_gate,
+                             void * y_up, uint32_t ytype, const int32_t * ids, int32_t n, int32_t topk, void * stream,
+                             tqmoe_error * err);
+
+/* act[i] = silu(gate[i]) * up[i], fp32 in and out (the reference's moe_swiglu, moe_kernels.cuh:71-72, rounds its
+ * bf16 inputs' product through bf16 to fp16; here nothing is rounded below fp32). */
+int32_t tqmoe_swiglu(const float * gate, const float * up, float * act, int64_t count, void * stream, tqmoe_error * err);
+
+/* out[t][j] = sum_s weights[t][s] * routed[t * topk + s][j] (s ascending) + shared_weights[t] * shared[t][j];
+ * routed / shared fp32, shared and shared_weights may be NULL together; out of otype (F32 or BF16).
+ * Replaces tqllm_cuda::moe_sum (moe_kernels.cuh:73-74, moe.cu:224-234) and fn_moe_combine (qwen4exp.cu:846-851);
+ * host meaning: moe_combine (src/experts/moe.cpp:157-163). No atomics: the sum order is fixed. */
+int32_t tqmoe_combine(const float * routed, const float * shared, const float * weights, const float * shared_weights,
+                      void * out, uint32_t otype, int32_t hidden, int32_t topk, int32_t n, void * stream,
+                      tqmoe_error * err);
+
+/* ---------------------------------------------------------------------------------------------- whole layer
+ * hidden states + router weights + expert banks in, combined hidden states out: the sequence of
+ * Qwen35Engine::ffn_block steps 2-9 (src/models/qwen/qwen35/qwen35_forward.cpp:1123-1248) and of the Flash-Next
+ * layer (src/models/qwen/qwen4exp/fn_layer_forward.cpp:311-336, 447-520) in one call.
+ * The shared expert, when has_shared, is expert index n_expert of the three banks (so banks hold n_expert + 1
+ * matrices), uses the first shared_ff rows of gate / up and the first shared_ff columns of down, and is weighted by
+ * sigmoid(router logit column n_expert). */
+typedef struct tqmoe_layer {
+    uint32_t struct_size;
+    int32_t hidden, ff, n_expert, topk;
+    int32_t has_shared, shared_ff;
+    float weight_scale;               /* 0 or 1: none */
+    const void * router;              /* device [n_expert][hidden] of router_type */
+    const void * shared_gate;         /* device [hidden] of router_type, or NULL */
+    uint32_t router_type;             /* TQMOE_F32 or TQMOE_BF16 */
+    tqmoe_bank gate, up, down;        /* gate / up: rows ff, cols hidden; down: rows hidden, cols ff */
+} tqmoe_layer;
+
+size_t  tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t n);
+/* x: device [n][hidden] of xtype; out: device [n][hidden] of otype (F32 or BF16); ids_out [n][topk], weights_out
+ * [n][topk], logits_out [n][n_expert + 1] optional device outputs (NULL to skip). */
+int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x, uint32_t xtype, int32_t n, void * out,
+                            uint32_t otype, int32_t * ids_out, float * weights_out, float * logits_out,
+                            void * workspace, size_t workspace_bytes, void * stream, tqmoe_error * err);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,84 @@
+"""Seeded synthetic MoE layers for the parity tests and the benchmark: weights N(0, sigma) quantised by the oracle's
+encoders into GGUF blocks, router weights and activations as BASELINE's configs describe them. numpy only."""
+import numpy as np
+
+import oracle
+
+CONFIGS = {
+    # name: hidden, ff, experts, topk, shared_ff, bank format, router / activation storage
+    "c1": dict(hidden=2048, ff=768, experts=64, topk=8, shared_ff=0, wtype=oracle.Q4_K, rtype="f32", xtype="f32"),
+    "c2": dict(hidden=2048, ff=512, experts=512, topk=10, shared_ff=512, wtype=oracle.IQ4_XS, rtype="bf16", xtype="bf16"),
+    "c4": dict(hidden=2048, ff=768, experts=256, topk=8, shared_ff=0, wtype=oracle.IQ3_S, rtype="bf16", xtype="bf16"),
+    "c5": dict(hidden=3072, ff=1536, experts=256, topk=8, shared_ff=1536, wtype=oracle.NVFP4G, rtype="bf16", xtype="bf16"),
+}
+
+
+def small(cfg, hidden, ff, experts, topk=None):
+    c = dict(cfg)
+    c.update(hidden=hidden, ff=ff, experts=experts, topk=min(topk or cfg["topk"], experts))
+    if c["shared_ff"]:
+        c["shared_ff"] = ff
+    return c
+
+
+def _scale_field(raw, wtype, per_expert_blocks, factors):
+    """Multiplies the block scale of every block of expert e by factors[e] so that tiled experts differ."""
+    elems, nbytes = oracle.BLOCK[wtype]
+    blocks = raw.reshape(len(factors), per_expert_blocks, nbytes)
+    if wtype == oracle.NVFP4G:
+        g = blocks[:, :, 0:4].copy().view(np.float32)
+        blocks[:, :, 0:4] = (g * factors[:, None, None].astype(np.float32)).view(np.uint8)
+    else:
+        d = blocks[:, :, 0:2].copy().view(np.float16).astype(np.float32)
+        blocks[:, :, 0:2] = (d * factors[:, None, None]).astype(np.float16).view(np.uint8)
+        if wtype == oracle.Q4_K:
+            m = blocks[:, :, 2:4].copy().view(np.float16).astype(np.float32)
+            blocks[:, :, 2:4] = (m * factors[:, None, None]).astype(np.float16).view(np.uint8)
+    return blocks.reshape(-1)
+
+
+def make_banks(cfg, seed, distinct=None, sigma=0.02):
+    """gate, up, down GGUF block streams (uint8) of experts (+1 shared) stacked matrices. `distinct` experts are really
+    quantised; the rest repeat them with an expert-specific factor on the block scales (cheap, still all different)."""
+    h, f, e = cfg["hidden"], cfg["ff"], cfg["experts"] + (1 if cfg["shared_ff"] else 0)
+    d = min(distinct or e, e)
+    rng = np.random.default_rng(seed)
+    banks = []
+    for rows, cols in ((f, h), (f, h), (h, f)):
+        w = (rng.standard_normal((d * rows, cols)) * sigma).astype(np.float32)
+        raw = oracle.quantize(cfg["wtype"], w)
+        per = raw.size // d
+        if d < e:
+            raw = np.tile(raw, (e + d - 1) // d)[: per * e].copy()
+            factors = 1.0 + (np.arange(e) // d) / 64.0
+            raw = _scale_field(raw, cfg["wtype"], per // oracle.BLOCK[cfg["wtype"]][1], factors)
+        banks.append(raw)
+    return banks
+
+
+def make_inputs(cfg, n, seed, zipf=None):
+    """router [E][H], shared gate [H], x [n][H] as (storage array, fp32 values). zipf: adds ln p_e of a Zipf(s) popularity
+    over a seeded permutation of the experts to the router logits by scaling nothing: returned as a bias vector."""
+    h, e = cfg["hidden"], cfg["experts"]
+    rng = np.random.default_rng(seed)
+    router = (rng.standard_normal((e, h)) * 0.02).astype(np.float32)
+    gate = (rng.standard_normal(h) * 0.02).astype(np.float32)
+    x = rng.standard_normal((n, h)).astype(np.float32)
+    out = {}
+    for name, a, kind in (("router", router, cfg["rtype"]), ("shared_gate", gate, cfg["rtype"]), ("x", x, cfg["xtype"])):
+        if kind == "bf16":
+            bits, vals = oracle.to_bf16(a)
+            out[name] = (bits, vals)
+        else:
+            out[name] = (a, a)
+    if zipf:
+        p = 1.0 / np.arange(1, e + 1) ** zipf
+        p /= p.sum()
+        out["bias"] = np.log(p[rng.permutation(e)]).astype(np.float32)
+    return out
+
+
+def errors(got, want):
+    """(max abs error, rms error / rms of the reference) over the whole output."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    return float(np.abs(got - want).max()), float(np.sqrt(np.mean((got - want) ** 2) / np.mean(want ** 2)))

@@ -1,0 +1,113 @@
+"""GPU parity, through the C ABI: router logits, softmax top-k and the dispatch permutation against the CPU oracle.
+Bars: logits within 3e-6 (the reference's own gate, tests/moe_device.cu:45-72); ids bit-exact and weights within 3e-6
+against the oracle's routing of the device's own logits; counts, offsets and permutation bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import synth
+from gpu_util import dev, oracle_type
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tq():
+    import tqllm_amd
+    return tqllm_amd
+
+
+@pytest.mark.parametrize("name,n", [("c1", 1), ("c1", 16), ("c2", 1), ("c2", 4), ("c2", 16), ("c4", 64), ("c5", 33)])
+def test_router_logits(tq, oracle, name, n):
+    cfg = synth.CONFIGS[name]
+    inp = synth.make_inputs(cfg, n, seed=1000 + n)
+    logits = tq.moe_router(dev(inp["router"]), dev(inp["shared_gate"]), dev(inp["x"])).cpu().numpy()
+    want = oracle.router_logits(inp["router"][0], oracle_type(cfg["rtype"]), inp["shared_gate"][0], inp["x"][0], oracle_type(cfg["xtype"]),
+                                cfg["hidden"], cfg["experts"], n)
+    assert logits.shape == (n, cfg["experts"] + 1)
+    assert np.abs(logits - want).max() < 3e-6
+
+
+def test_router_without_shared_gate_and_f16(tq, oracle):
+    rng = np.random.default_rng(5)
+    h, e, n = 512, 33, 7
+    w = (rng.standard_normal((e, h)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((n, h)).astype(np.float16)
+    logits = tq.moe_router(dev(w), None, dev(x)).cpu().numpy()
+    want = oracle.router_logits(w, oracle.F32, None, x.view(np.uint16), oracle.F16, h, e, n)
+    assert np.abs(logits - want).max() < 3e-6 and not logits[:, e].any()
+
+
+@pytest.mark.parametrize("e,k,n", [(64, 8, 16), (512, 10, 16), (512, 10, 4096), (256, 8, 512), (4096, 6, 3), (5, 5, 2), (1000, 1, 9)])
+def test_topk_matches_oracle_on_device_logits(tq, oracle, e, k, n):
+    rng = np.random.default_rng(e * 7 + k)
+    logits = rng.standard_normal((n, e + 1)).astype(np.float32)
+    ids, w, sw = (t.cpu().numpy() for t in tq.moe_topk(dev(logits), e, k))
+    want_ids, want_w = oracle.route(logits[:, :e], k)
+    gaps = oracle.route_min_gap_ulps(logits[:, :e], k)
+    clear = gaps > 8          # tokens whose k + 1 largest probabilities are further apart than exp() rounding
+    assert clear.mean() > 0.99
+    assert np.array_equal(ids[clear], want_ids[clear])
+    same = (ids == want_ids).all(axis=1)
+    assert np.abs(w[same] - want_w[same]).max() < 3e-6
+    assert np.abs(w.sum(axis=1) - 1).max() < 1e-5
+    want_sw = np.array([oracle.shared_weight(v) for v in logits[:, e]], np.float32)
+    assert np.abs(sw - want_sw).max() < 3e-6
+
+
+def test_topk_ties_extremes_and_scale(tq, oracle):
+    e, k = 96, 6
+    rows = [np.full(e, 0.5, np.float32),                                   # all equal: lowest indices
+            np.where(np.arange(e) % 7 == 0, 3.0, -2.0).astype(np.float32),  # many exact ties at the top
+            np.linspace(-300, 80, e).astype(np.float32),                    # exp underflow to exact zeros
+            np.full(e, -1e4, np.float32)]
+    rows[3][10] = 5.0
+    logits = np.concatenate([np.stack(rows), np.zeros((4, 1), np.float32)], axis=1)
+    for scale in (1.0, 0.0, 2.5):
+        ids, w, _ = (t.cpu().numpy() for t in tq.moe_topk(dev(logits), e, k, scale))
+        want_ids, want_w = oracle.route(logits[:, :e], k, scale=scale)
+        assert np.array_equal(ids, want_ids)
+        assert np.abs(w - want_w).max() < 3e-6 * max(1.0, scale)
+    assert ids[0].tolist() == list(range(k)) and ids[3][0] == 10
+
+
+@pytest.mark.parametrize("e,n,k", [(64, 1, 8), (512, 16, 10), (512, 4096, 10), (256, 8192, 9), (7, 300, 3), (4096, 700, 2), (512, 102, 10)])
+def test_dispatch_bit_exact(tq, oracle, e, n, k):
+    rng = np.random.default_rng(n + e)
+    if e == 512 and n == 4096:   # skewed load: Zipf(1.1) popularity, as the prefill config
+        p = 1.0 / np.arange(1, e + 1) ** 1.1
+        ids = rng.choice(e, size=(n, k), p=p / p.sum()).astype(np.int32)
+    else:
+        ids = rng.integers(0, e, (n, k)).astype(np.int32)
+    if n == 300:
+        ids[rng.random((n, k)) < 0.2] = -1          # skipped assignments
+    want_c, want_o, want_p = oracle.dispatch(ids, e)
+    cap = int(want_c.max()) if want_c.max() else 1
+    counts, offsets, perm, groups = (t.cpu().numpy() for t in tq.moe_dispatch(dev(ids), e, capacity=cap))
+    assert np.array_equal(counts, want_c) and np.array_equal(offsets, want_o) and np.array_equal(perm, want_p)
+    for x in range(e):
+        assert np.array_equal(groups[x, :counts[x]], want_p[want_o[x]:want_o[x + 1]])
+        assert (groups[x, counts[x]:] == -1).all()
+    assert counts.sum() == (ids >= 0).sum()
+
+
+def test_dispatch_is_deterministic_and_truncates_groups(tq, oracle):
+    rng = np.random.default_rng(9)
+    ids = rng.integers(0, 32, (2000, 4)).astype(np.int32)
+    a = [t.cpu().numpy() for t in tq.moe_dispatch(dev(ids), 32, capacity=16)]
+    b = [t.cpu().numpy() for t in tq.moe_dispatch(dev(ids), 32, capacity=16)]
+    for u, v in zip(a, b):
+        assert np.array_equal(u, v)
+    want_c, want_o, want_p = oracle.dispatch(ids, 32)
+    assert np.array_equal(a[0], want_c)
+    for x in range(32):
+        assert np.array_equal(a[3][x], want_p[want_o[x]:want_o[x] + 16])
+
+
+def test_errors_are_reported(tq):
+    with pytest.raises(tq.TqmoeError):
+        tq.moe_topk(torch.zeros((2, 9), device="cuda"), 8, 9)
+    with pytest.raises(tq.TqmoeError):
+        tq.moe_router(torch.zeros((4, 12), device="cuda"), None, torch.zeros((1, 12), device="cuda"))
+    with pytest.raises(tq.TqmoeError):
+        tq.moe_router(torch.zeros((4, 16)), None, torch.zeros((1, 16)))      # host tensors: no CPU path

@@ -1,0 +1,277 @@
+"""ctypes binding of libtqmoe.so and the host-side mirror of the reference's MoE operator interface.
+
+Names follow the reference: moe_router / moe_topk / moe_group (here moe_dispatch, the deterministic form) / moe_swiglu /
+moe_sum (here moe_combine) of src/experts/moe_kernels.cuh, and expert_matvec / expert_matvec2 of tqllm::WeightFormat
+(src/formats/weight/weight_format.hpp:62-73). Every function enqueues on torch's current stream of the tensors' device
+and raises TqmoeError with the library's message on failure. There is no fallback path: a missing library or a missing
+GPU is an error.
+"""
+import ctypes as C
+import os
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libtqmoe.so")
+
+F32, F16, BF16 = 0, 1, 30
+Q4_K, IQ3_S, IQ4_XS, NVFP4G = 12, 21, 23, 323
+BLOCK = {Q4_K: (256, 144), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76)}
+_TORCH_TYPE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+_OUT_TYPE = {F32: torch.float32, BF16: torch.bfloat16}
+
+
+class TqmoeError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("tqmoe error %d: %s" % (code, message))
+        self.code = code
+
+
+class _Error(C.Structure):
+    _fields_ = [("struct_size", C.c_uint32), ("code", C.c_int32), ("message", C.c_char * 256)]
+
+
+class _Bank(C.Structure):
+    _fields_ = [("struct_size", C.c_uint32), ("type", C.c_uint32), ("experts", C.c_int32), ("rows", C.c_int32),
+                ("cols", C.c_int32), ("codes", C.c_void_p), ("aux", C.c_void_p)]
+
+
+class _Layer(C.Structure):
+    _fields_ = [("struct_size", C.c_uint32), ("hidden", C.c_int32), ("ff", C.c_int32), ("n_expert", C.c_int32),
+                ("topk", C.c_int32), ("has_shared", C.c_int32), ("shared_ff", C.c_int32), ("weight_scale", C.c_float),
+                ("router", C.c_void_p), ("shared_gate", C.c_void_p), ("router_type", C.c_uint32),
+                ("gate", _Bank), ("up", _Bank), ("down", _Bank)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises when it has not been built (python -m tqllm_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise TqmoeError(-3, "libtqmoe.so is not built: run `python -m tqllm_amd.build` (there is no fallback path)")
+        l = C.CDLL(LIB_PATH)
+        p, i32, i64, u32, f32, sz = C.c_void_p, C.c_int32, C.c_int64, C.c_uint32, C.c_float, C.c_size_t
+        e = C.POINTER(_Error)
+        l.tqmoe_abi_version.restype = u32
+        l.tqmoe_router.argtypes = [p, u32, p, p, u32, p, i32, i32, i32, p, e]
+        l.tqmoe_topk.argtypes = [p, p, p, p, i32, i32, i32, f32, p, e]
+        l.tqmoe_dispatch_workspace_bytes.restype = sz
+        l.tqmoe_dispatch_workspace_bytes.argtypes = [i32, i32, i32]
+        l.tqmoe_dispatch.argtypes = [p, p, p, p, p, i32, i32, i32, i32, p, sz, p, e]
+        l.tqmoe_bank_layout.argtypes = [u32, i64, i32, C.POINTER(sz), C.POINTER(sz), e]
+        l.tqmoe_bank_load.argtypes = [u32, p, i64, i32, p, p, p, p, e]
+        l.tqmoe_bank_dequant.argtypes = [C.POINTER(_Bank), i64, i64, p, p, e]
+        l.tqmoe_act_image_bytes.restype = sz
+        l.tqmoe_act_image_bytes.argtypes = [i32, i32]
+        l.tqmoe_quant_act.argtypes = [p, u32, i32, i32, p, p, e]
+        l.tqmoe_expert_matvec.argtypes = [C.POINTER(_Bank), p, p, u32, p, i32, i32, i32, p, e]
+        l.tqmoe_expert_matvec2.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, u32, p, i32, i32, p, e]
+        l.tqmoe_swiglu.argtypes = [p, p, p, i64, p, e]
+        l.tqmoe_combine.argtypes = [p, p, p, p, p, u32, i32, i32, i32, p, e]
+        l.tqmoe_layer_workspace_bytes.restype = sz
+        l.tqmoe_layer_workspace_bytes.argtypes = [C.POINTER(_Layer), i32]
+        l.tqmoe_layer_forward.argtypes = [C.POINTER(_Layer), p, u32, i32, p, u32, p, p, p, p, sz, p, e]
+        for name in ("tqmoe_router", "tqmoe_topk", "tqmoe_dispatch", "tqmoe_bank_layout", "tqmoe_bank_load", "tqmoe_bank_dequant",
+                     "tqmoe_quant_act", "tqmoe_expert_matvec", "tqmoe_expert_matvec2", "tqmoe_swiglu", "tqmoe_combine",
+                     "tqmoe_layer_forward"):
+            getattr(l, name).restype = i32
+        _lib = l
+    return _lib
+
+
+def abi_version():
+    return lib().tqmoe_abi_version()
+
+
+def _err():
+    return _Error(C.sizeof(_Error), 0, b"")
+
+
+def _check(rc, err):
+    if rc:
+        raise TqmoeError(rc, err.message.decode("utf-8", "replace"))
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream(t):
+    if not t.is_cuda:
+        raise TqmoeError(-3, "tensors must live on the GPU (there is no CPU path)")
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ttype(t):
+    try:
+        return _TORCH_TYPE[t.dtype]
+    except KeyError:
+        raise TqmoeError(-2, "unsupported tensor dtype %s" % t.dtype)
+
+
+def moe_router(router, shared_gate, x, experts=None):
+    """logits [n][E + 1] fp32 = x @ [router; shared_gate]^T (moe_kernels.cuh:7-10)."""
+    n, hidden = x.shape
+    e = router.shape[0] if experts is None else experts
+    logits = torch.empty((n, e + 1), dtype=torch.float32, device=x.device)
+    err = _err()
+    _check(lib().tqmoe_router(_ptr(router), _ttype(router), _ptr(shared_gate), _ptr(x), _ttype(x), _ptr(logits), hidden, e, n,
+                              _stream(x), C.byref(err)), err)
+    return logits
+
+
+def moe_topk(logits, experts, topk, scale=1.0):
+    """ids [n][k] int32, weights [n][k] fp32, shared_weights [n] fp32 (moe_kernels.cuh:19-20)."""
+    n = logits.shape[0]
+    ids = torch.empty((n, topk), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((n, topk), dtype=torch.float32, device=logits.device)
+    shared = torch.empty((n,), dtype=torch.float32, device=logits.device)
+    err = _err()
+    _check(lib().tqmoe_topk(_ptr(logits), _ptr(ids), _ptr(weights), _ptr(shared), experts, topk, n, float(scale), _stream(logits),
+                            C.byref(err)), err)
+    return ids, weights, shared
+
+
+def moe_dispatch(ids, experts, capacity=0):
+    """counts [E], offsets [E + 1], perm [A] (entries past offsets[E] are -1) and, with capacity > 0, the reference's
+    groups [E][capacity] view (moe_kernels.cuh:29; deterministic, ascending inside each expert)."""
+    n, topk = ids.shape
+    dev = ids.device
+    counts = torch.empty(experts, dtype=torch.int32, device=dev)
+    offsets = torch.empty(experts + 1, dtype=torch.int32, device=dev)
+    perm = torch.full((n * topk,), -1, dtype=torch.int32, device=dev)
+    groups = torch.full((experts, capacity), -1, dtype=torch.int32, device=dev) if capacity > 0 else None
+    wsb = lib().tqmoe_dispatch_workspace_bytes(experts, n, topk)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+    err = _err()
+    _check(lib().tqmoe_dispatch(_ptr(ids), _ptr(counts), _ptr(offsets), _ptr(perm), _ptr(groups), capacity, experts, n, topk, _ptr(ws),
+                                wsb, _stream(ids), C.byref(err)), err)
+    return counts, offsets, perm, groups
+
+
+class ExpertBank:
+    """One projection of every expert in the library's device layout: the counterpart of tqllm::Mat for stacked experts
+    (weight_format.hpp:22-28, 61). Built from the raw GGUF block stream of [experts * rows][cols]."""
+
+    def __init__(self, wtype, gguf_blocks, experts, rows, cols, device="cuda"):
+        self.type, self.experts, self.rows, self.cols = wtype, experts, rows, cols
+        cb, ab = C.c_size_t(0), C.c_size_t(0)
+        err = _err()
+        _check(lib().tqmoe_bank_layout(wtype, experts * rows, cols, C.byref(cb), C.byref(ab), C.byref(err)), err)
+        raw = gguf_blocks if isinstance(gguf_blocks, torch.Tensor) else torch.from_numpy(gguf_blocks)
+        elems, nbytes = BLOCK[wtype]
+        if raw.numel() != experts * rows * (cols // elems) * nbytes:
+            raise TqmoeError(-1, "GGUF block stream has %d bytes, %d expected" % (raw.numel(), experts * rows * (cols // elems) * nbytes))
+        raw = raw.to(device=device, dtype=torch.uint8).contiguous()
+        self.codes = torch.empty(cb.value, dtype=torch.uint8, device=raw.device)
+        self.aux = torch.empty(ab.value, dtype=torch.uint8, device=raw.device)
+        status = torch.zeros(1, dtype=torch.int32, device=raw.device)
+        _check(lib().tqmoe_bank_load(wtype, _ptr(raw), experts * rows, cols, _ptr(self.codes), _ptr(self.aux), _ptr(status), _stream(raw),
+                                     C.byref(err)), err)
+        if int(status.item()):
+            raise TqmoeError(-1, "NVFP4G rows whose blocks carry different global scales are not loadable")
+
+    def view(self):
+        return _Bank(C.sizeof(_Bank), self.type, self.experts, self.rows, self.cols, self.codes.data_ptr(), self.aux.data_ptr())
+
+    def dequant(self, row0=0, nrows=None):
+        """fp32 [nrows][cols] decoded values (WeightFormat::dequant_rows_h, weight_format.hpp:84-86)."""
+        nrows = self.experts * self.rows - row0 if nrows is None else nrows
+        out = torch.empty((nrows, self.cols), dtype=torch.float32, device=self.codes.device)
+        err = _err()
+        b = self.view()
+        _check(lib().tqmoe_bank_dequant(C.byref(b), row0, nrows, _ptr(out), _stream(out), C.byref(err)), err)
+        return out
+
+
+def quant_act(x):
+    """Activation image of x [n][cols] (see include/tqmoe.h): uint8 tensor."""
+    n, cols = x.shape
+    image = torch.empty(lib().tqmoe_act_image_bytes(n, cols), dtype=torch.uint8, device=x.device)
+    err = _err()
+    _check(lib().tqmoe_quant_act(_ptr(x), _ttype(x), n, cols, _ptr(image), _stream(x), C.byref(err)), err)
+    return image
+
+
+def expert_matvec(bank, image, ids, per_expert_input=False, out_type=F32):
+    """y [n * topk][rows] (WeightFormat::expert_matvec, weight_format.hpp:62-64). Rows of assignments with id < 0 stay as
+    allocated (zero here)."""
+    n, topk = ids.shape
+    y = torch.zeros((n * topk, bank.rows), dtype=_OUT_TYPE[out_type], device=ids.device)
+    err = _err()
+    b = bank.view()
+    _check(lib().tqmoe_expert_matvec(C.byref(b), _ptr(image), _ptr(y), out_type, _ptr(ids), n, topk, int(per_expert_input), _stream(ids),
+                                     C.byref(err)), err)
+    return y
+
+
+def expert_matvec2(gate, up, image, ids, out_type=F32):
+    """gate and up over the same ids in one launch (WeightFormat::expert_matvec2, weight_format.hpp:70-73)."""
+    n, topk = ids.shape
+    yg = torch.zeros((n * topk, gate.rows), dtype=_OUT_TYPE[out_type], device=ids.device)
+    yu = torch.zeros_like(yg)
+    err = _err()
+    g, u = gate.view(), up.view()
+    _check(lib().tqmoe_expert_matvec2(C.byref(g), C.byref(u), _ptr(image), _ptr(yg), _ptr(yu), out_type, _ptr(ids), n, topk, _stream(ids),
+                                      C.byref(err)), err)
+    return yg, yu
+
+
+def moe_swiglu(gate, up):
+    act = torch.empty_like(gate)
+    err = _err()
+    _check(lib().tqmoe_swiglu(_ptr(gate), _ptr(up), _ptr(act), gate.numel(), _stream(gate), C.byref(err)), err)
+    return act
+
+
+def moe_combine(routed, shared, weights, shared_weights, out_type=F32):
+    """out [n][hidden] = sum_s weights[t][s] * routed[t * k + s] + shared_weights[t] * shared[t] (moe_kernels.cuh:73-74)."""
+    n, topk = weights.shape
+    hidden = routed.shape[1]
+    out = torch.empty((n, hidden), dtype=_OUT_TYPE[out_type], device=routed.device)
+    err = _err()
+    _check(lib().tqmoe_combine(_ptr(routed), _ptr(shared), _ptr(weights), _ptr(shared_weights), _ptr(out), out_type, hidden, topk, n,
+                               _stream(routed), C.byref(err)), err)
+    return out
+
+
+class MoeLayer:
+    """hidden states + router weights + expert banks in, combined hidden states out, in one library call."""
+
+    def __init__(self, router, shared_gate, gate, up, down, topk, shared_ff=0, weight_scale=1.0):
+        self.router, self.shared_gate, self.gate, self.up, self.down = router, shared_gate, gate, up, down
+        self.n_expert, self.hidden = router.shape
+        self.ff, self.topk, self.shared_ff, self.weight_scale = gate.rows, topk, shared_ff, weight_scale
+        self._ws = None
+
+    def desc(self):
+        return _Layer(C.sizeof(_Layer), self.hidden, self.ff, self.n_expert, self.topk, int(self.shared_ff > 0), self.shared_ff,
+                      float(self.weight_scale), self.router.data_ptr(), self.shared_gate.data_ptr() if self.shared_gate is not None else None,
+                      _ttype(self.router), self.gate.view(), self.up.view(), self.down.view())
+
+    def workspace(self, n):
+        d = self.desc()
+        need = lib().tqmoe_layer_workspace_bytes(C.byref(d), n)
+        if need == 0:
+            raise TqmoeError(-1, "layer descriptor rejected (shapes of the banks do not match the layer)")
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device=self.router.device)
+        return self._ws
+
+    def forward(self, x, out_type=F32, return_routing=False):
+        n = x.shape[0]
+        ws = self.workspace(n)
+        out = torch.empty((n, self.hidden), dtype=_OUT_TYPE[out_type], device=x.device)
+        ids = weights = logits = None
+        if return_routing:
+            ids = torch.empty((n, self.topk), dtype=torch.int32, device=x.device)
+            weights = torch.empty((n, self.topk), dtype=torch.float32, device=x.device)
+            logits = torch.empty((n, self.n_expert + 1), dtype=torch.float32, device=x.device)
+        d = self.desc()
+        err = _err()
+        _check(lib().tqmoe_layer_forward(C.byref(d), _ptr(x), _ttype(x), n, _ptr(out), out_type, _ptr(ids), _ptr(weights), _ptr(logits),
+                                         _ptr(ws), ws.numel(), _stream(x), C.byref(err)), err)
+        return (out, ids, weights, logits) if return_routing else out

@@ -1,0 +1,219 @@
+// Expert banks: GGUF block stream -> device layout (one thread per 32-weight sub-block), and the fp32 dequantiser
+// whose values are those of the host decoder bit for bit (no fused multiply-add, same evaluation order).
+#include "formats.cuh"
+
+namespace tqmoe {
+namespace {
+
+__device__ __forceinline__ uint32_t rd_u16(const uint8_t * p) { return uint32_t(p[0]) | uint32_t(p[1]) << 8; }
+__device__ __forceinline__ uint32_t rd_u32(const uint8_t * p) { return rd_u16(p) | rd_u16(p + 2) << 16; }
+
+// canonical nibble order of a sub-block: byte j = code of weight j | code of weight j + 16 << 4
+template <class F> __device__ __forceinline__ void pack_sub(uint8_t * dst, F code) {
+    uint32_t w[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        w[q] = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) { const int j = 4 * q + b; w[q] |= (uint32_t(code(j)) | uint32_t(code(j + 16)) << 4) << (8 * b); }
+    }
+    *reinterpret_cast<uint4 *>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__global__ __launch_bounds__(256) void load_k(uint32_t type, const uint8_t * __restrict__ src, int64_t rows_total, int cols,
+                                              uint8_t * __restrict__ codes, uint8_t * __restrict__ aux, int * __restrict__ status) {
+    const int S = cols / 32;
+    const int64_t idx = int64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= rows_total * S) return;
+    const int64_t row = idx / S;
+    const int s = int(idx % S);
+    uint8_t * cd = codes + idx * code_bytes_per_sub(type);
+    switch (type) {
+        case TQMOE_IQ4_XS: {  // 136 B per 256: d, scales_h, scales_l[4], qs[128]; nibble order already canonical
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 136;
+            const uint8_t * q = blk + 8 + 16 * (s & 7);
+            pack_sub(cd, [&](int j) { return j < 16 ? q[j] & 15 : q[j - 16] >> 4; });
+            if ((s & 7) == 0) {
+                uint8_t * a = aux + (row * (S / 8) + s / 8) * 8;
+                *reinterpret_cast<uint2 *>(a) = make_uint2(rd_u32(blk), rd_u32(blk + 4));
+            }
+            break;
+        }
+        case TQMOE_Q4_K: {  // 144 B per 256: d, dmin, scales[12], qs[128]; 64-weight chunk c: low nibbles then high
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 144;
+            const int ib = s & 7;
+            const uint8_t * q = blk + 16 + 32 * (ib >> 1);
+            pack_sub(cd, [&](int j) { return (ib & 1) ? q[j] >> 4 : q[j] & 15; });
+            if (ib == 0) {
+                uint8_t * a = aux + (row * (S / 8) + s / 8) * 16;
+                *reinterpret_cast<uint4 *>(a) = make_uint4(rd_u32(blk), rd_u32(blk + 4), rd_u32(blk + 8), rd_u32(blk + 12));
+            }
+            break;
+        }
+        case TQMOE_IQ3_S: {  // 110 B per 256: d, qs[64], qh[8], signs[32], scales[4]
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 110;
+            const int ib = s & 7;
+            uint32_t * o = reinterpret_cast<uint32_t *>(cd);
+            o[0] = rd_u32(blk + 2 + 8 * ib);
+            o[1] = rd_u32(blk + 2 + 8 * ib + 4);
+            o[2] = rd_u32(blk + 74 + 4 * ib);
+            if (ib == 0) {
+                uint8_t * a = aux + (row * (S / 8) + s / 8) * 16;
+                *reinterpret_cast<uint4 *>(a) = make_uint4(rd_u16(blk) | rd_u16(blk + 66) << 16, rd_u32(blk + 68),
+                                                           rd_u16(blk + 72) | rd_u16(blk + 106) << 16, rd_u16(blk + 108));
+            }
+            break;
+        }
+        case TQMOE_NVFP4G: {  // 76 B per 128: global f32, 8 E4M3 scales, 64 code bytes (byte i of a 16-group: weights 2i, 2i + 1)
+            const uint8_t * blk = src + (row * (S / 4) + s / 4) * 76;
+            const int q4 = s & 3;
+            const uint8_t * q = blk + 12 + 16 * q4;  // two 16-groups
+            pack_sub(cd, [&](int j) { const uint8_t b = q[8 * (j >> 4) + ((j & 15) >> 1)]; return (j & 1) ? b >> 4 : b & 15; });
+            uint8_t * a = aux + row * (cols / 16) + 2 * s;
+            a[0] = blk[4 + 2 * q4];
+            a[1] = blk[4 + 2 * q4 + 1];
+            const uint32_t g = rd_u32(blk), g0 = rd_u32(src + row * (S / 4) * 76);
+            if (g != g0 && status) atomicOr(status, 1);  // the row's blocks disagree on the global scale
+            if (s == 0) *reinterpret_cast<uint32_t *>(aux + nvfp4_global_offset(rows_total, cols) + row * 4) = g0;
+            break;
+        }
+    }
+}
+
+// fp32 values of one sub-block, written exactly as the host decoder computes them
+__global__ __launch_bounds__(256) void dequant_k(uint32_t type, const uint8_t * __restrict__ codes, const uint8_t * __restrict__ aux,
+                                                 int64_t rows_total, int cols, int64_t row0, int64_t nrows, float * __restrict__ out) {
+    const int S = cols / 32;
+    const int64_t idx = int64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= nrows * S) return;
+    const int64_t row = row0 + idx / S;
+    const int s = int(idx % S), ib = s & 7;
+    const uint8_t * cd = codes + (row * S + s) * code_bytes_per_sub(type);
+    float * y = out + idx * 32;
+    switch (type) {
+        case TQMOE_IQ4_XS: {
+            const uint2 rec = *reinterpret_cast<const uint2 *>(aux + (row * (S / 8) + s / 8) * 8);
+            const float dl = __fmul_rn(half_bits_to_float(uint16_t(rec.x & 0xFFFFu)), float(iq4xs_ls(rec, ib) - 32));
+            const uint4 c = *reinterpret_cast<const uint4 *>(cd);
+            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t lo, hi;
+                lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(w[q], lo, hi);
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    y[4 * q + b] = __fmul_rn(dl, float(int8_t(lo >> (8 * b))));
+                    y[16 + 4 * q + b] = __fmul_rn(dl, float(int8_t(hi >> (8 * b))));
+                }
+            }
+            break;
+        }
+        case TQMOE_Q4_K: {
+            const uint4 rec = *reinterpret_cast<const uint4 *>(aux + (row * (S / 8) + s / 8) * 16);
+            const uint32_t sc12[3] = {rec.y, rec.z, rec.w};
+            int sc, mn;
+            q4k_scale_min(sc12, ib, sc, mn);
+            const float d1 = __fmul_rn(half_bits_to_float(uint16_t(rec.x & 0xFFFFu)), float(sc));
+            const float m1 = __fmul_rn(half_bits_to_float(uint16_t(rec.x >> 16)), float(mn));
+            const uint4 c = *reinterpret_cast<const uint4 *>(cd);
+            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const uint32_t byte = (w[q] >> (8 * b)) & 0xFFu;
+                    y[4 * q + b] = __fsub_rn(__fmul_rn(d1, float(byte & 15u)), m1);
+                    y[16 + 4 * q + b] = __fsub_rn(__fmul_rn(d1, float(byte >> 4)), m1);
+                }
+            break;
+        }
+        case TQMOE_IQ3_S: {
+            const uint4 rec = *reinterpret_cast<const uint4 *>(aux + (row * (S / 8) + s / 8) * 16);
+            // rec: d | qh[0..1] << 16, qh[2..5], qh[6..7] | scales[0..1] << 16, scales[2..3]
+            const uint32_t qh = ib < 2 ? (rec.x >> (16 + 8 * ib)) & 0xFFu : ib < 6 ? (rec.y >> (8 * (ib - 2))) & 0xFFu : (rec.z >> (8 * (ib - 6))) & 0xFFu;
+            const uint32_t scb = (ib >> 1) < 2 ? (rec.z >> (16 + 8 * (ib >> 1))) & 0xFFu : (rec.w >> (8 * ((ib >> 1) - 2))) & 0xFFu;
+            const float db = __fmul_rn(half_bits_to_float(uint16_t(rec.x & 0xFFFFu)), float(1 + 2 * int((scb >> (4 * (ib & 1))) & 15u)));
+            const uint32_t * c = reinterpret_cast<const uint32_t *>(cd);
+            const uint32_t qs[2] = {c[0], c[1]}, sg = c[2];
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {
+                const uint32_t g = d_iq3s_grid.v[((qs[w >> 2] >> (8 * (w & 3))) & 0xFFu) | (((qh >> w) & 1u) << 8)];
+                const uint32_t sn = sg >> (4 * w);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float mag = __fmul_rn(db, float((g >> (8 * j)) & 0xFFu));
+                    y[4 * w + j] = ((sn >> j) & 1u) ? -mag : mag;
+                }
+            }
+            break;
+        }
+        case TQMOE_NVFP4G: {
+            const float g = *reinterpret_cast<const float *>(aux + nvfp4_global_offset(rows_total, cols) + row * 4);
+            const uint8_t * sc = aux + row * (cols / 16) + 2 * s;
+            const float d0 = __fmul_rn(e4m3_to_float(sc[0]), g), d1 = __fmul_rn(e4m3_to_float(sc[1]), g);
+            const uint4 c = *reinterpret_cast<const uint4 *>(cd);
+            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t lo, hi;
+                lookup16<kFp4T0, kFp4T1, kFp4T2, kFp4T3>(w[q], lo, hi);
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    // table holds twice the E2M1 value; halving is exact. -0 codes give -0 * d on the host: keep the sign
+                    const uint32_t nlo = (w[q] >> (8 * b)) & 15u, nhi = (w[q] >> (8 * b + 4)) & 15u;
+                    const float vlo = nlo == 8 ? -0.f : 0.5f * float(int8_t(lo >> (8 * b)));
+                    const float vhi = nhi == 8 ? -0.f : 0.5f * float(int8_t(hi >> (8 * b)));
+                    y[4 * q + b] = __fmul_rn(vlo, d0);
+                    y[16 + 4 * q + b] = __fmul_rn(vhi, d1);
+                }
+            }
+            break;
+        }
+    }
+}
+
+}  // namespace
+
+int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err) {
+    if (!b || b->struct_size < sizeof(tqmoe_bank)) return fail(err, TQMOE_E_ARG, "%s: bank descriptor missing or too small", what);
+    if (!is_bank_type(b->type)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: bank type %u is not supported", what, b->type);
+    if (!b->codes || !b->aux || b->experts <= 0 || b->rows <= 0 || b->cols <= 0) return fail(err, TQMOE_E_ARG, "%s: invalid bank shape or pointer", what);
+    if (b->cols % (b->type == TQMOE_NVFP4G ? 128 : 256)) return fail(err, TQMOE_E_ARG, "%s: cols %d is not a multiple of the block size", what, b->cols);
+    return 0;
+}
+
+}  // namespace tqmoe
+
+using namespace tqmoe;
+
+extern "C" int32_t tqmoe_bank_layout(uint32_t type, int64_t rows_total, int32_t cols, size_t * code_bytes, size_t * aux_bytes, tqmoe_error * err) {
+    if (!is_bank_type(type)) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_bank_layout: bank type %u is not supported", type);
+    if (rows_total <= 0 || cols <= 0 || cols % (type == TQMOE_NVFP4G ? 128 : 256)) return fail(err, TQMOE_E_ARG, "tqmoe_bank_layout: invalid shape");
+    if (code_bytes) *code_bytes = size_t(rows_total * code_row_bytes(type, cols));
+    if (aux_bytes) *aux_bytes = type == TQMOE_NVFP4G ? size_t(nvfp4_global_offset(rows_total, cols) + rows_total * 4) : size_t(rows_total * aux_row_bytes(type, cols));
+    return ok(err);
+}
+
+extern "C" int32_t tqmoe_bank_load(uint32_t type, const void * gguf_blocks, int64_t rows_total, int32_t cols, void * codes, void * aux,
+                                   int32_t * status, void * stream, tqmoe_error * err) {
+    if (int32_t rc = tqmoe_bank_layout(type, rows_total, cols, nullptr, nullptr, err)) return rc;
+    if (!gguf_blocks || !codes || !aux) return fail(err, TQMOE_E_ARG, "tqmoe_bank_load: null pointer");
+    if (int32_t rc = need_device(err, "tqmoe_bank_load")) return rc;
+    const int64_t subs = rows_total * (cols / 32);
+    if ((subs + 255) / 256 > 0x7FFFFFFF) return fail(err, TQMOE_E_ARG, "tqmoe_bank_load: bank too large for one call");
+    load_k<<<unsigned((subs + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(type, static_cast<const uint8_t *>(gguf_blocks), rows_total, cols,
+                                                                                      static_cast<uint8_t *>(codes), static_cast<uint8_t *>(aux), status);
+    return launched(err, "tqmoe_bank_load");
+}
+
+extern "C" int32_t tqmoe_bank_dequant(const tqmoe_bank * bank, int64_t row0, int64_t nrows, float * out, void * stream, tqmoe_error * err) {
+    if (int32_t rc = check_bank(bank, "tqmoe_bank_dequant", err)) return rc;
+    const int64_t rows_total = int64_t(bank->experts) * bank->rows;
+    if (!out || row0 < 0 || nrows <= 0 || row0 + nrows > rows_total) return fail(err, TQMOE_E_ARG, "tqmoe_bank_dequant: invalid row range");
+    if (int32_t rc = need_device(err, "tqmoe_bank_dequant")) return rc;
+    const int64_t subs = nrows * (bank->cols / 32);
+    if ((subs + 255) / 256 > 0x7FFFFFFF) return fail(err, TQMOE_E_ARG, "tqmoe_bank_dequant: range too large for one call");
+    dequant_k<<<unsigned((subs + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(bank->type, static_cast<const uint8_t *>(bank->codes),
+                                                                                         static_cast<const uint8_t *>(bank->aux), rows_total, bank->cols, row0, nrows, out);
+    return launched(err, "tqmoe_bank_dequant");
+}

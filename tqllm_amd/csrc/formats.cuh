@@ -1,0 +1,73 @@
+// Bank formats: device layout arithmetic and the per-sub-block decode shared by the loader, the fp32 dequantiser and
+// the product kernels. A sub-block is 32 consecutive weights of a row; S = cols / 32 sub-blocks per row.
+#pragma once
+#include "common.cuh"
+#include "iq3s_lattice.h"
+
+namespace tqmoe {
+
+// code bytes per sub-block
+__host__ __device__ constexpr int code_bytes_per_sub(uint32_t type) { return type == TQMOE_IQ3_S ? 12 : 16; }
+// aux record bytes per 256 weights (NVFP4G keeps bytes per 16 weights instead: see aux_row_bytes)
+__host__ __device__ constexpr int aux_record_bytes(uint32_t type) { return type == TQMOE_IQ4_XS ? 8 : 16; }
+__host__ __device__ constexpr int64_t code_row_bytes(uint32_t type, int cols) { return int64_t(cols / 32) * code_bytes_per_sub(type); }
+__host__ __device__ constexpr int64_t aux_row_bytes(uint32_t type, int cols) {
+    return type == TQMOE_NVFP4G ? int64_t(cols / 16) : int64_t(cols / 256) * aux_record_bytes(type);
+}
+// NVFP4G: offset of the per-row fp32 globals inside the aux plane
+__host__ __device__ constexpr int64_t nvfp4_global_offset(int64_t rows_total, int cols) { return (rows_total * (cols / 16) + 15) / 16 * 16; }
+
+// IQ4_NL / IQ4_XS value table {-127,-104,-83,-65,-49,-35,-22,-10,1,13,25,38,53,69,89,113} as four little-endian dwords
+constexpr uint32_t kIq4T0 = 0xBFAD9881u, kIq4T1 = 0xF6EADDCFu, kIq4T2 = 0x26190D01u, kIq4T3 = 0x71594535u;
+// 2 * E2M1 {0,.5,1,1.5,2,3,4,6, -0,-.5,-1,-1.5,-2,-3,-4,-6} = {0,1,2,3,4,6,8,12, 0,-1,-2,-3,-4,-6,-8,-12}
+constexpr uint32_t kFp4T0 = 0x03020100u, kFp4T1 = 0x0C080604u, kFp4T2 = 0xFDFEFF00u, kFp4T3 = 0xF4F8FAFCu;
+
+// 8 four-bit codes of one dword -> int8 table values: lo = the four low nibbles, hi = the four high nibbles
+template <uint32_t T0, uint32_t T1, uint32_t T2, uint32_t T3>
+__device__ __forceinline__ void lookup16(uint32_t c, uint32_t & lo, uint32_t & hi) {
+    // v_perm_b32 picks from an 8-byte pool, so: both halves of the table by the low three index bits, then a third
+    // pick between the two results by index bit 3 (selector byte = position + 4 * bit3)
+    const uint32_t i_lo = c & 0x07070707u, i_hi = (c >> 4) & 0x07070707u;
+    const uint32_t a_lo = __builtin_amdgcn_perm(T1, T0, i_lo), b_lo = __builtin_amdgcn_perm(T3, T2, i_lo);
+    const uint32_t a_hi = __builtin_amdgcn_perm(T1, T0, i_hi), b_hi = __builtin_amdgcn_perm(T3, T2, i_hi);
+    lo = __builtin_amdgcn_perm(b_lo, a_lo, ((c >> 1) & 0x04040404u) | 0x03020100u);
+    hi = __builtin_amdgcn_perm(b_hi, a_hi, ((c >> 5) & 0x04040404u) | 0x03020100u);
+}
+__device__ __forceinline__ void nibbles(uint32_t c, uint32_t & lo, uint32_t & hi) { lo = c & 0x0F0F0F0Fu; hi = (c >> 4) & 0x0F0F0F0Fu; }
+
+// IQ3_S lattice points in the classic form (byte j = magnitude of weight j)
+struct Iq3sGrid { uint32_t v[512]; };
+constexpr Iq3sGrid make_iq3s_grid() {
+    constexpr uint16_t codes[512] = {TQMOE_IQ3S_LATTICE12};
+    Iq3sGrid g{};
+    for (int i = 0; i < 512; ++i) {
+        const uint32_t c = codes[i];
+        g.v[i] = (2u * (c & 7u) + 1u) | ((2u * ((c >> 3) & 7u) + 1u) << 8) | ((2u * ((c >> 6) & 7u) + 1u) << 16) | ((2u * ((c >> 9) & 7u) + 1u) << 24);
+    }
+    return g;
+}
+__device__ const Iq3sGrid d_iq3s_grid = make_iq3s_grid();
+
+// E4M3 byte -> float: (1 + m/8) 2^(e-7), subnormal m/8 2^-6, 0x7F / 0xFF NaN
+__device__ __forceinline__ float e4m3_to_float(uint32_t b) {
+    const int e = (b >> 3) & 15, m = b & 7;
+    float v;
+    if (e == 15 && m == 7) v = __uint_as_float(0x7FC00000u);
+    else if (e == 0) v = float(m) * 0.001953125f;                          // m * 2^-9
+    else v = __uint_as_float(uint32_t(e + 120) << 23 | uint32_t(m) << 20);  // (1 + m/8) * 2^(e - 7)
+    return (b & 0x80u) ? -v : v;
+}
+
+// Q4_K: 6-bit (scale, min) of sub-block j from the 12-byte field held as three dwords
+__device__ __forceinline__ void q4k_scale_min(const uint32_t (&q)[3], int j, int & sc, int & mn) {
+    auto byte = [&](int i) { return (q[i >> 2] >> (8 * (i & 3))) & 0xFFu; };
+    if (j < 4) { sc = byte(j) & 63; mn = byte(j + 4) & 63; }
+    else { sc = (byte(j + 4) & 15) | ((byte(j - 4) >> 6) << 4); mn = (byte(j + 4) >> 4) | ((byte(j) >> 6) << 4); }
+}
+
+// IQ4_XS: 6-bit scale of sub-block ib of a 256-weight record (d | scales_h << 16, scales_l[4])
+__device__ __forceinline__ int iq4xs_ls(uint2 rec, int ib) {
+    return int(((rec.y >> (4 * ib)) & 15u) | (((rec.x >> (16 + 2 * ib)) & 3u) << 4));
+}
+
+}  // namespace tqmoe

@@ -124,6 +124,24 @@ int32_t tqmoe_expert_matvec2(const tqmoe_bank * gate, const tqmoe_bank * up, con
                              void * y_up, uint32_t ytype, const int32_t * ids, int32_t n, int32_t topk, void * stream,
                              tqmoe_error * err);
 
+/* Fused decode stages of the layer (tqmoe_layer_forward is router, top-k, tqmoe_quant_act and these two):
+ *
+ * tqmoe_expert_gateup: for every assignment a = t * slots + s (slots = topk + has_shared; s == topk is the shared
+ * expert, bank index n_expert, first shared_ff rows), act = silu(gate_e x[t]) * (up_e x[t]) written as an activation
+ * image of n * slots rows of gate->rows values (rows past shared_ff of a shared assignment are not written and not
+ * read back). Counterpart of WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59: gate and up in one launch
+ * with the SwiGLU epilogue) at decode sizes.
+ * tqmoe_expert_down_combine: out[t] = sum_s weights[t][s] * (down_e(s) act[t][s]) (s ascending, then the shared expert
+ * with shared_weights[t]), fixed order, no atomics: expert_matvec on the down bank followed by moe_sum
+ * (moe_kernels.cuh:73-74) in one launch. out of otype (F32 or BF16), [n][down->rows]. */
+int32_t tqmoe_expert_gateup(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x_image, void * act_image,
+                            const int32_t * ids, int32_t n, int32_t topk, int32_t has_shared, int32_t shared_ff,
+                            void * stream, tqmoe_error * err);
+int32_t tqmoe_expert_down_combine(const tqmoe_bank * down, const void * act_image, const int32_t * ids,
+                                  const float * weights, const float * shared_weights, void * out, uint32_t otype,
+                                  int32_t n, int32_t topk, int32_t has_shared, int32_t shared_ff, void * stream,
+                                  tqmoe_error * err);
+
 /* act[i] = silu(gate[i]) * up[i], fp32 in and out (the reference's moe_swiglu, moe_kernels.cuh:71-72, rounds its
  * bf16 inputs' product through bf16 to fp16; here nothing is rounded below fp32). */
 int32_t tqmoe_swiglu(const float * gate, const float * up, float * act, int64_t count, void * stream, tqmoe_error * err);

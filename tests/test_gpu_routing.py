@@ -25,7 +25,11 @@ def test_router_logits(tq, oracle, name, n):
     want = oracle.router_logits(inp["router"][0], oracle_type(cfg["rtype"]), inp["shared_gate"][0], inp["x"][0], oracle_type(cfg["xtype"]),
                                 cfg["hidden"], cfg["experts"], n)
     assert logits.shape == (n, cfg["experts"] + 1)
-    assert np.abs(logits - want).max() < 3e-6
+    # against the exact (float64) product of the stored values: the reference's 3e-6 gate; against the oracle's
+    # column-order fp32 sum the distance is that sum's own rounding (a few 1e-6 at 2048 terms)
+    exact = inp["x"][1].astype(np.float64) @ np.vstack([inp["router"][1], inp["shared_gate"][1]]).astype(np.float64).T
+    assert np.abs(logits - exact).max() < 3e-6
+    assert np.abs(logits - want).max() < 2e-5
 
 
 def test_router_without_shared_gate_and_f16(tq, oracle):

@@ -411,49 +411,70 @@ int32_t enqueue_quant_act(const void * x, uint32_t xtype, int n, int cols, void 
     return 0;
 }
 
-int32_t enqueue_gateup(const tqmoe_bank & gate, const tqmoe_bank & up, const void * ximage, void * aimage, const int * ids, int n, int topk,
-                       int slots, int n_expert, int shared_ff, hipStream_t s) {
-    const Split sp = split_for(gate.cols / 32);
-    if (sp.m > 4) return -1;
-    const dim3 grid(unsigned(gate.rows / 32), unsigned(n * slots));
-    const BankView bg = view(gate), bu = view(up);
-    const uint8_t * xi = static_cast<const uint8_t *>(ximage);
-    uint8_t * ai = static_cast<uint8_t *>(aimage);
-    switch (gate.type) {
+}  // namespace tqmoe
+
+using namespace tqmoe;
+
+extern "C" int32_t tqmoe_expert_gateup(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x_image, void * act_image, const int32_t * ids,
+                                       int32_t n, int32_t topk, int32_t has_shared, int32_t shared_ff, void * stream, tqmoe_error * err) {
+    const char * what = "tqmoe_expert_gateup";
+    if (int32_t rc = check_bank(gate, what, err)) return rc;
+    if (int32_t rc = check_bank(up, what, err)) return rc;
+    if (up->type != gate->type || up->rows != gate->rows || up->cols != gate->cols || up->experts != gate->experts)
+        return fail(err, TQMOE_E_ARG, "%s: the two banks differ in format or shape", what);
+    if (!x_image || !act_image || !ids || n <= 0 || topk <= 0 || gate->rows % 32) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    if (has_shared && (shared_ff <= 0 || shared_ff > gate->rows || shared_ff % 32)) return fail(err, TQMOE_E_ARG, "%s: invalid shared_ff", what);
+    const int slots = topk + (has_shared ? 1 : 0), n_expert = gate->experts - (has_shared ? 1 : 0);
+    if (n_expert <= 0 || int64_t(n) * slots > 65535) return fail(err, TQMOE_E_ARG, "%s: n * slots exceeds 65535 or the bank is too small", what);
+    const Split sp = split_for(gate->cols / 32);
+    if (sp.m > 4) return fail(err, TQMOE_E_UNSUPPORTED, "%s: cols %d is too wide for the decode kernels", what, gate->cols);
+    if (int32_t rc = need_device(err, what)) return rc;
+    const hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid(unsigned(gate->rows / 32), unsigned(n * slots));
+    const BankView bg = view(*gate), bu = view(*up);
+    const uint8_t * xi = static_cast<const uint8_t *>(x_image);
+    uint8_t * ai = static_cast<uint8_t *>(act_image);
+    switch (gate->type) {
         case TQMOE_IQ4_XS: launch_gateup<TQMOE_IQ4_XS>(sp.m, grid, s, bg, bu, xi, ai, ids, topk, slots, n_expert, shared_ff, sp.lpr); break;
         case TQMOE_Q4_K: launch_gateup<TQMOE_Q4_K>(sp.m, grid, s, bg, bu, xi, ai, ids, topk, slots, n_expert, shared_ff, sp.lpr); break;
         case TQMOE_IQ3_S: launch_gateup<TQMOE_IQ3_S>(sp.m, grid, s, bg, bu, xi, ai, ids, topk, slots, n_expert, shared_ff, sp.lpr); break;
         default: launch_gateup<TQMOE_NVFP4G>(sp.m, grid, s, bg, bu, xi, ai, ids, topk, slots, n_expert, shared_ff, sp.lpr); break;
     }
-    return 0;
+    return launched(err, what);
 }
 
-int32_t enqueue_down_combine(const tqmoe_bank & down, const void * aimage, const int * ids, const float * weights, const float * shared_w, void * out,
-                             uint32_t otype, int n, int topk, int slots, int n_expert, int shared_ff, hipStream_t s) {
-    const Split sp = split_for(down.cols / 32);
-    if (sp.m > 4) return -1;
+extern "C" int32_t tqmoe_expert_down_combine(const tqmoe_bank * down, const void * act_image, const int32_t * ids, const float * weights,
+                                             const float * shared_weights, void * out, uint32_t otype, int32_t n, int32_t topk, int32_t has_shared,
+                                             int32_t shared_ff, void * stream, tqmoe_error * err) {
+    const char * what = "tqmoe_expert_down_combine";
+    if (int32_t rc = check_bank(down, what, err)) return rc;
+    if (!act_image || !ids || !weights || !out || n <= 0 || topk <= 0 || (has_shared && !shared_weights)) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    if (has_shared && (shared_ff <= 0 || shared_ff > down->cols || shared_ff % 32)) return fail(err, TQMOE_E_ARG, "%s: invalid shared_ff", what);
+    if (otype != TQMOE_F32 && otype != TQMOE_BF16) return fail(err, TQMOE_E_UNSUPPORTED, "%s: output type must be F32 or BF16", what);
+    const int slots = topk + (has_shared ? 1 : 0), n_expert = down->experts - (has_shared ? 1 : 0);
+    if (n_expert <= 0 || n > 65535) return fail(err, TQMOE_E_ARG, "%s: too many tokens for one call or the bank is too small", what);
+    const Split sp = split_for(down->cols / 32);
+    if (sp.m > 4) return fail(err, TQMOE_E_UNSUPPORTED, "%s: cols %d is too wide for the decode kernels", what, down->cols);
+    if (int32_t rc = need_device(err, what)) return rc;
+    const hipStream_t s = static_cast<hipStream_t>(stream);
     const int rw = 64 / sp.lpr;
     // few tokens: one wave per block so that the grid still covers the chip
-    const int waves = n * ((down.rows + rw - 1) / rw) >= 4096 ? 4 : 1;
-    const dim3 grid(unsigned((down.rows + rw * waves - 1) / (rw * waves)), unsigned(n));
-    const BankView bd = view(down);
-    const uint8_t * ai = static_cast<const uint8_t *>(aimage);
-#define TQ_DOWN(F)                                                                                                                     \
-    if (otype == TQMOE_F32) launch_down<F, TQMOE_F32>(sp.m, grid, waves * 64, s, bd, ai, ids, weights, shared_w, out, topk, slots, n_expert, shared_ff, sp.lpr); \
-    else launch_down<F, TQMOE_BF16>(sp.m, grid, waves * 64, s, bd, ai, ids, weights, shared_w, out, topk, slots, n_expert, shared_ff, sp.lpr)
-    switch (down.type) {
+    const int waves = int64_t(n) * ((down->rows + rw - 1) / rw) >= 4096 ? 4 : 1;
+    const dim3 grid(unsigned((down->rows + rw * waves - 1) / (rw * waves)), unsigned(n));
+    const BankView bd = view(*down);
+    const uint8_t * ai = static_cast<const uint8_t *>(act_image);
+#define TQ_DOWN(F)                                                                                                                              \
+    if (otype == TQMOE_F32) launch_down<F, TQMOE_F32>(sp.m, grid, waves * 64, s, bd, ai, ids, weights, shared_weights, out, topk, slots, n_expert, shared_ff, sp.lpr); \
+    else launch_down<F, TQMOE_BF16>(sp.m, grid, waves * 64, s, bd, ai, ids, weights, shared_weights, out, topk, slots, n_expert, shared_ff, sp.lpr)
+    switch (down->type) {
         case TQMOE_IQ4_XS: TQ_DOWN(TQMOE_IQ4_XS); break;
         case TQMOE_Q4_K: TQ_DOWN(TQMOE_Q4_K); break;
         case TQMOE_IQ3_S: TQ_DOWN(TQMOE_IQ3_S); break;
         default: TQ_DOWN(TQMOE_NVFP4G); break;
     }
 #undef TQ_DOWN
-    return 0;
+    return launched(err, what);
 }
-
-}  // namespace tqmoe
-
-using namespace tqmoe;
 
 extern "C" size_t tqmoe_act_image_bytes(int32_t n, int32_t cols) {
     if (n <= 0 || cols <= 0 || cols % 32) return 0;

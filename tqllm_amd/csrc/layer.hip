@@ -3,11 +3,6 @@
 
 namespace tqmoe {
 int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);
-int32_t enqueue_quant_act(const void * x, uint32_t xtype, int n, int cols, void * image, hipStream_t s);
-int32_t enqueue_gateup(const tqmoe_bank & gate, const tqmoe_bank & up, const void * ximage, void * aimage, const int * ids, int n, int topk,
-                       int slots, int n_expert, int shared_ff, hipStream_t s);
-int32_t enqueue_down_combine(const tqmoe_bank & down, const void * aimage, const int * ids, const float * weights, const float * shared_w, void * out,
-                             uint32_t otype, int n, int topk, int slots, int n_expert, int shared_ff, hipStream_t s);
 
 namespace {
 
@@ -70,7 +65,6 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
     const Plan p = plan_for(L, n);
     if (!workspace || workspace_bytes < p.total) return fail(err, TQMOE_E_WORKSPACE, "tqmoe_layer_forward: workspace of %zu bytes needed", p.total);
     if (int32_t rc = need_device(err, "tqmoe_layer_forward")) return rc;
-    const hipStream_t s = static_cast<hipStream_t>(stream);
     uint8_t * ws = static_cast<uint8_t *>(workspace);
     float * logits = logits_out ? logits_out : reinterpret_cast<float *>(ws + p.logits);
     int32_t * ids = ids_out ? ids_out : reinterpret_cast<int32_t *>(ws + p.ids);
@@ -79,10 +73,7 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
 
     if (int32_t rc = tqmoe_router(L.router, L.router_type, L.shared_gate, x, xtype, logits, L.hidden, L.n_expert, n, stream, err)) return rc;
     if (int32_t rc = tqmoe_topk(logits, ids, weights, shared_w, L.n_expert, L.topk, n, L.weight_scale, stream, err)) return rc;
-    enqueue_quant_act(x, xtype, n, L.hidden, ws + p.ximage, s);
-    if (enqueue_gateup(L.gate, L.up, ws + p.ximage, ws + p.aimage, ids, n, L.topk, slots, L.n_expert, L.shared_ff, s))
-        return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_layer_forward: hidden %d is not supported by the decode kernels", L.hidden);
-    if (enqueue_down_combine(L.down, ws + p.aimage, ids, weights, shared_w, out, otype, n, L.topk, slots, L.n_expert, L.shared_ff, s))
-        return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_layer_forward: ff %d is not supported by the decode kernels", L.ff);
-    return launched(err, "tqmoe_layer_forward");
+    if (int32_t rc = tqmoe_quant_act(x, xtype, n, L.hidden, ws + p.ximage, stream, err)) return rc;
+    if (int32_t rc = tqmoe_expert_gateup(&L.gate, &L.up, ws + p.ximage, ws + p.aimage, ids, n, L.topk, L.has_shared, L.shared_ff, stream, err)) return rc;
+    return tqmoe_expert_down_combine(&L.down, ws + p.aimage, ids, weights, shared_w, out, otype, n, L.topk, L.has_shared, L.shared_ff, stream, err);
 }

@@ -164,19 +164,21 @@ def main():
         logits = tq.moe_router(l.router, l.shared_gate, x)
         ids, w, sw = tq.moe_topk(logits, CFG["experts"], CFG["topk"])
         img = tq.quant_act(x)
-        act = tq.expert_gateup(l.gate, l.up, img, ids, shared_ff=CFG["shared_ff"])
-        prep.append((l, ids, w, sw, img, act))
+        ext = tq.moe_extend_ids(ids, CFG["experts"])
+        act = tq.expert_gateup(l.gate, l.up, img, ext, CFG["topk"], shared_ff=CFG["shared_ff"])
+        y = tq.expert_down(l.down, act, ext, CFG["topk"], shared_ff=CFG["shared_ff"])
+        prep.append((l, ext, img, act, y))
 
     def gateup_round():
-        for l, ids, w, sw, img, act in prep:
-            tq.expert_gateup(l.gate, l.up, img, ids, shared_ff=CFG["shared_ff"], act_image=act)
+        for l, ext, img, act, y in prep:
+            tq.expert_gateup(l.gate, l.up, img, ext, CFG["topk"], shared_ff=CFG["shared_ff"], act_image=act)
 
     def down_round():
-        for (l, ids, w, sw, img, act), o in zip(prep, outs):
-            tq.expert_down_combine(l.down, act, ids, w, sw, shared_ff=CFG["shared_ff"], out=o)
+        for l, ext, img, act, y in prep:
+            tq.expert_down(l.down, act, ext, CFG["topk"], shared_ff=CFG["shared_ff"], y=y)
 
     kernels = {}
-    for name, fn in (("gateup", gateup_round), ("down_combine", down_round)):
+    for name, fn in (("gateup", gateup_round), ("down", down_round)):
         gk = torch.cuda.CUDAGraph()
         fn()
         torch.cuda.synchronize()
@@ -199,8 +201,7 @@ def main():
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4), "traffic": None,
                      "algorithmic_bytes_per_launch": int(gu_bytes), "us_per_launch": round(kernels["gateup"] * 1e3, 2)},
         "layer": {"algorithmic_bytes_per_step": int(layer_bytes), "hbm_frac": round(layer_bytes / (ms_step * 1e-3) / HBM_PEAK, 4),
-                  "down_combine_us": round(kernels["down_combine"] * 1e3, 2),
-                  "down_combine_hbm_frac": round(dn_bytes / (kernels["down_combine"] * 1e-3) / HBM_PEAK, 4)},
+                  "down_us": round(kernels["down"] * 1e3, 2), "down_hbm_frac": round(dn_bytes / (kernels["down"] * 1e-3) / HBM_PEAK, 4)},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()

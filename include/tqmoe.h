@@ -124,23 +124,26 @@ int32_t tqmoe_expert_matvec2(const tqmoe_bank * gate, const tqmoe_bank * up, con
                              void * y_up, uint32_t ytype, const int32_t * ids, int32_t n, int32_t topk, void * stream,
                              tqmoe_error * err);
 
-/* Fused decode stages of the layer (tqmoe_layer_forward is router, top-k, tqmoe_quant_act and these two):
+/* Decode stages of the layer (tqmoe_layer_forward is router, top-k, tqmoe_extend_ids, tqmoe_quant_act, these two and
+ * tqmoe_combine_strided). `ids` holds the expert of every (token, slot), [n][slots]: the routed ids and, when
+ * slots == topk + 1, the shared expert's bank index in the last slot (tqmoe_extend_ids makes it). One block serves every
+ * assignment of its expert, so a step reads each distinct expert's weights from HBM once.
  *
- * tqmoe_expert_gateup: for every assignment a = t * slots + s (slots = topk + has_shared; s == topk is the shared
- * expert, bank index n_expert, first shared_ff rows), act = silu(gate_e x[t]) * (up_e x[t]) written as an activation
- * image of n * slots rows of gate->rows values (rows past shared_ff of a shared assignment are not written and not
- * read back). Counterpart of WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59: gate and up in one launch
- * with the SwiGLU epilogue) at decode sizes.
- * tqmoe_expert_down_combine: out[t] = sum_s weights[t][s] * (down_e(s) act[t][s]) (s ascending, then the shared expert
- * with shared_weights[t]), fixed order, no atomics: expert_matvec on the down bank followed by moe_sum
- * (moe_kernels.cuh:73-74) in one launch. out of otype (F32 or BF16), [n][down->rows]. */
+ * tqmoe_extend_ids: out[t][s] = s < topk ? ids[t][s] : extra. tqllm_cuda::moe_extend_ids without slot maps
+ * (src/experts/moe_kernels.cuh:77-78, moe.cu:204-216).
+ * tqmoe_expert_gateup: act[a] = silu(gate_e x[t]) * (up_e x[t]) for a = t * slots + s, written as an activation image of
+ * n * slots rows of gate->rows values; a shared assignment (s >= topk) only has its first shared_ff values.
+ * Counterpart of WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59: gate and up in one launch with the SwiGLU
+ * epilogue) at decode sizes.
+ * tqmoe_expert_down: y[a] = down_e act[a], fp32 [n * slots][down->rows]; a shared assignment reads the first shared_ff
+ * columns. WeightFormat::expert_matvec with per_expert_input (weight_format.hpp:62-64). */
+int32_t tqmoe_extend_ids(const int32_t * ids, int32_t * out, int32_t topk, int32_t n, int32_t extra, void * stream,
+                         tqmoe_error * err);
 int32_t tqmoe_expert_gateup(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x_image, void * act_image,
-                            const int32_t * ids, int32_t n, int32_t topk, int32_t has_shared, int32_t shared_ff,
+                            const int32_t * ids, int32_t n, int32_t slots, int32_t topk, int32_t shared_ff,
                             void * stream, tqmoe_error * err);
-int32_t tqmoe_expert_down_combine(const tqmoe_bank * down, const void * act_image, const int32_t * ids,
-                                  const float * weights, const float * shared_weights, void * out, uint32_t otype,
-                                  int32_t n, int32_t topk, int32_t has_shared, int32_t shared_ff, void * stream,
-                                  tqmoe_error * err);
+int32_t tqmoe_expert_down(const tqmoe_bank * down, const void * act_image, float * y, const int32_t * ids, int32_t n,
+                          int32_t slots, int32_t topk, int32_t shared_ff, void * stream, tqmoe_error * err);
 
 /* act[i] = silu(gate[i]) * up[i], fp32 in and out (the reference's moe_swiglu, moe_kernels.cuh:71-72, rounds its
  * bf16 inputs' product through bf16 to fp16; here nothing is rounded below fp32). */
@@ -153,6 +156,11 @@ int32_t tqmoe_swiglu(const float * gate, const float * up, float * act, int64_t 
 int32_t tqmoe_combine(const float * routed, const float * shared, const float * weights, const float * shared_weights,
                       void * out, uint32_t otype, int32_t hidden, int32_t topk, int32_t n, void * stream,
                       tqmoe_error * err);
+/* the same with `slots` routed rows per token (the first topk weighted) and the shared rows shared_ld floats apart:
+ * tqllm_cuda::moe_sum_strided (moe_kernels.cuh:80-81, moe.cu:197-210). hidden and shared_ld multiples of 4. */
+int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float * shared, int64_t shared_ld,
+                              const float * weights, const float * shared_weights, void * out, uint32_t otype,
+                              int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err);
 
 /* ---------------------------------------------------------------------------------------------- whole layer
  * hidden states + router weights + expert banks in, combined hidden states out: the sequence of

@@ -69,15 +69,17 @@ def lib():
         l.tqmoe_quant_act.argtypes = [p, u32, i32, i32, p, p, e]
         l.tqmoe_expert_matvec.argtypes = [C.POINTER(_Bank), p, p, u32, p, i32, i32, i32, p, e]
         l.tqmoe_expert_matvec2.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, u32, p, i32, i32, p, e]
+        l.tqmoe_extend_ids.argtypes = [p, p, i32, i32, i32, p, e]
         l.tqmoe_expert_gateup.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, i32, i32, i32, i32, p, e]
-        l.tqmoe_expert_down_combine.argtypes = [C.POINTER(_Bank), p, p, p, p, p, u32, i32, i32, i32, i32, p, e]
+        l.tqmoe_expert_down.argtypes = [C.POINTER(_Bank), p, p, p, i32, i32, i32, i32, p, e]
+        l.tqmoe_combine_strided.argtypes = [p, i32, p, i64, p, p, p, u32, i32, i32, i32, p, e]
         l.tqmoe_swiglu.argtypes = [p, p, p, i64, p, e]
         l.tqmoe_combine.argtypes = [p, p, p, p, p, u32, i32, i32, i32, p, e]
         l.tqmoe_layer_workspace_bytes.restype = sz
         l.tqmoe_layer_workspace_bytes.argtypes = [C.POINTER(_Layer), i32]
         l.tqmoe_layer_forward.argtypes = [C.POINTER(_Layer), p, u32, i32, p, u32, p, p, p, p, sz, p, e]
         for name in ("tqmoe_router", "tqmoe_topk", "tqmoe_dispatch", "tqmoe_bank_layout", "tqmoe_bank_load", "tqmoe_bank_dequant",
-                     "tqmoe_quant_act", "tqmoe_expert_matvec", "tqmoe_expert_matvec2", "tqmoe_expert_gateup", "tqmoe_expert_down_combine", "tqmoe_swiglu", "tqmoe_combine",
+                     "tqmoe_quant_act", "tqmoe_expert_matvec", "tqmoe_expert_matvec2", "tqmoe_extend_ids", "tqmoe_expert_gateup", "tqmoe_expert_down", "tqmoe_combine_strided", "tqmoe_swiglu", "tqmoe_combine",
                      "tqmoe_layer_forward"):
             getattr(l, name).restype = i32
         _lib = l
@@ -222,29 +224,49 @@ def expert_matvec2(gate, up, image, ids, out_type=F32):
     return yg, yu
 
 
-def expert_gateup(gate, up, x_image, ids, shared_ff=0, act_image=None):
-    """Activation image of silu(gate x) * (up x) for every (token, slot); slot topk is the shared expert when shared_ff > 0
-    (WeightFormat::expert_gemm_gateup, weight_format.hpp:57-59, at decode sizes)."""
+def moe_extend_ids(ids, extra):
+    """[n][topk + 1]: the routed ids with the shared expert's bank index as the last slot (moe_kernels.cuh:77-78)."""
     n, topk = ids.shape
-    slots = topk + (1 if shared_ff else 0)
+    out = torch.empty((n, topk + 1), dtype=torch.int32, device=ids.device)
+    err = _err()
+    _check(lib().tqmoe_extend_ids(_ptr(ids), _ptr(out), topk, n, extra, _stream(ids), C.byref(err)), err)
+    return out
+
+
+def expert_gateup(gate, up, x_image, ids, topk, shared_ff=0, act_image=None):
+    """Activation image of silu(gate x) * (up x) for every (token, slot) of ids [n][slots]; slots past topk are the shared
+    expert (WeightFormat::expert_gemm_gateup, weight_format.hpp:57-59, at decode sizes)."""
+    n, slots = ids.shape
     if act_image is None:
         act_image = torch.zeros(lib().tqmoe_act_image_bytes(n * slots, gate.rows), dtype=torch.uint8, device=ids.device)
     err = _err()
     g, u = gate.view(), up.view()
-    _check(lib().tqmoe_expert_gateup(C.byref(g), C.byref(u), _ptr(x_image), _ptr(act_image), _ptr(ids), n, topk, int(shared_ff > 0), shared_ff,
-                                     _stream(ids), C.byref(err)), err)
+    _check(lib().tqmoe_expert_gateup(C.byref(g), C.byref(u), _ptr(x_image), _ptr(act_image), _ptr(ids), n, slots, topk, shared_ff, _stream(ids),
+                                     C.byref(err)), err)
     return act_image
 
 
-def expert_down_combine(down, act_image, ids, weights, shared_weights=None, shared_ff=0, out_type=F32, out=None):
-    """out [n][hidden]: the down product of every slot summed with its routing weight in slot order, shared expert last."""
-    n, topk = ids.shape
-    if out is None:
-        out = torch.empty((n, down.rows), dtype=_OUT_TYPE[out_type], device=ids.device)
+def expert_down(down, act_image, ids, topk, shared_ff=0, y=None):
+    """y [n * slots][hidden] fp32: the down product of every (token, slot) from its row of the activation image."""
+    n, slots = ids.shape
+    if y is None:
+        y = torch.zeros((n * slots, down.rows), dtype=torch.float32, device=ids.device)
     err = _err()
     d = down.view()
-    _check(lib().tqmoe_expert_down_combine(C.byref(d), _ptr(act_image), _ptr(ids), _ptr(weights), _ptr(shared_weights), _ptr(out), out_type, n, topk,
-                                           int(shared_ff > 0), shared_ff, _stream(ids), C.byref(err)), err)
+    _check(lib().tqmoe_expert_down(C.byref(d), _ptr(act_image), _ptr(y), _ptr(ids), n, slots, topk, shared_ff, _stream(ids), C.byref(err)), err)
+    return y
+
+
+def moe_combine_strided(y, slots, weights, shared_weights=None, out_type=F32, out=None):
+    """moe_sum_strided (moe_kernels.cuh:80-81): y [n][slots][hidden], the first topk slots weighted, slot topk the shared row."""
+    n, topk = weights.shape
+    hidden = y.shape[-1]
+    if out is None:
+        out = torch.empty((n, hidden), dtype=_OUT_TYPE[out_type], device=y.device)
+    shared = y.view(-1)[topk * hidden:] if shared_weights is not None else None
+    err = _err()
+    _check(lib().tqmoe_combine_strided(_ptr(y), slots, _ptr(shared), slots * hidden, _ptr(weights), _ptr(shared_weights), _ptr(out), out_type, hidden,
+                                       topk, n, _stream(y), C.byref(err)), err)
     return out
 
 

@@ -1,0 +1,47 @@
+// Types shared by the decode entry points (decode.hip) and the per-format kernel translation units.
+#pragma once
+#include "common.cuh"
+
+namespace tqmoe {
+
+struct BankView { const uint8_t * codes; const uint8_t * aux; int64_t rows_total; int rows, cols; };
+inline BankView view(const tqmoe_bank & b) {
+    return BankView{static_cast<const uint8_t *>(b.codes), static_cast<const uint8_t *>(b.aux), int64_t(b.experts) * b.rows, b.rows, b.cols};
+}
+
+// lanes per row (8, 16, 32 or 64) and sub-blocks per lane (1..4) for S sub-blocks per row; m == 0: not supported
+struct Split { int lpr, m; };
+inline Split split_for(int S) {
+    if (S % 64 == 0) return Split{64, S / 64 <= 4 ? S / 64 : 0};
+    for (int lpr = 32; lpr >= 8; lpr >>= 1)
+        if (S % lpr == 0 && S / lpr <= 4 && (S / lpr == 1 || S / lpr == 3)) return Split{lpr, S / lpr};
+    return Split{64, (S + 63) / 64 <= 4 ? (S + 63) / 64 : 0};  // ragged: lanes past the row's last sub-block idle
+}
+
+struct MatvecArgs {
+    BankView b0, b1;
+    const uint8_t * image;
+    void * y0, * y1;
+    uint32_t ytype;
+    const int * ids;
+    int A, xdiv, mode, slots, topk, shared_cols;
+};
+struct GateupArgs {
+    BankView bg, bu;
+    const uint8_t * ximage;
+    uint8_t * aimage;
+    const int * ids;
+    int A, slots, topk, shared_ff, mode;
+};
+
+// launch tables, one explicit instantiation per bank format (decode_<format>.hip)
+template <uint32_t FMT> struct DecodeLaunch {
+    static void matvec(Split sp, int nb, const MatvecArgs & k, hipStream_t s);
+    static void gateup(Split sp, const GateupArgs & k, hipStream_t s);
+};
+extern template struct DecodeLaunch<TQMOE_IQ4_XS>;
+extern template struct DecodeLaunch<TQMOE_Q4_K>;
+extern template struct DecodeLaunch<TQMOE_IQ3_S>;
+extern template struct DecodeLaunch<TQMOE_NVFP4G>;
+
+}  // namespace tqmoe

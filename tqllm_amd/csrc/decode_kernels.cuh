@@ -1,0 +1,396 @@
+// Decode-sized expert products: the kernels and their per-format launch tables (one translation unit per bank format
+// instantiates DecodeLaunch<FMT>; decode.hip holds the entry points).
+//
+// HBM-streaming matrix-vector kernels over the bank layout.
+//
+// Arithmetic. The input row is held as an "activation image": per 32 values a scale s = amax / 16383 and the integers
+// q = rint(x / s) split into two int8 planes, q = 128 * hi + lo with 0 <= lo < 128. A weight sub-block is turned into
+// int8 table values in registers (v_perm_b32 lookups for the 4-bit code books, LDS lattice reads for IQ3_S), and the
+// product of the two is taken with v_dot4_i32_i8: sum(w * q) = 128 * dot(w, hi) + dot(w, lo), exact in int32. One
+// fp32 multiply per sub-block applies weight scale * s. Against an fp32 product the only approximation is the 15-bit
+// rounding of x relative to its block maximum (2^-15 relative), three orders below the layer tolerance.
+//
+// Mapping. A lane owns sub-block(s) sl, sl + LPR, ... of every row it visits, so its slice of the activation image stays
+// in registers for the whole kernel and each row costs one 16-byte (12 for IQ3_S) code load per owned sub-block. LPR
+// consecutive lanes cover one row; a wave covers 64 / LPR rows per step and finishes each row with a DPP butterfly.
+#pragma once
+#include "act_image.cuh"
+#include "decode_api.cuh"
+#include "formats.cuh"
+
+namespace tqmoe {
+namespace {
+
+// ------------------------------------------------------------------------------------------ sub-block products
+// A weight sub-block is fetched (Raw: what one lane loads), decoded once into eight dwords of int8 values in the order
+// of the activation planes (Dec), and multiplied with any number of activation blocks.
+struct Dec {
+    uint32_t w[8];   // int8 x 4 each; w[q] pairs with activation dword q
+    float s0, s1;    // scale of dwords 0..3 and of dwords 4..7 (equal except for NVFP4G's two 16-weight groups)
+    float mn;        // coefficient of the block's activation sum (Q4_K minimum), else 0
+};
+
+__device__ __forceinline__ int dot4x(const uint32_t * w, const int * x) {
+    int acc = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_sdot4(int(w[q]), x[q], acc, false);
+    return acc;
+}
+template <bool SPLIT> __device__ __forceinline__ float dot_block(const Dec & d, const ActBlock & x) {
+    if constexpr (SPLIT) {
+        const int t0 = (dot4x(d.w, x.hi) << 7) + dot4x(d.w, x.lo);
+        const int t1 = (dot4x(d.w + 4, x.hi + 4) << 7) + dot4x(d.w + 4, x.lo + 4);
+        return (float(t0) * d.s0 + float(t1) * d.s1) * x.scale;
+    } else {
+        int hi = 0, lo = 0;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) { hi = __builtin_amdgcn_sdot4(int(d.w[q]), x.hi[q], hi, false); lo = __builtin_amdgcn_sdot4(int(d.w[q]), x.lo[q], lo, false); }
+        return float((hi << 7) + lo) * (d.s0 * x.scale) - d.mn * x.sum;
+    }
+}
+
+template <uint32_t FMT> struct Sub;
+
+template <> struct Sub<TQMOE_IQ4_XS> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint4 c; uint2 rec; };
+    static __device__ __forceinline__ Raw load(const uint8_t * __restrict__ codes, const uint8_t * __restrict__ aux, int64_t, int, int64_t row, int S, int s) {
+        Raw r;
+        r.c = *reinterpret_cast<const uint4 *>(codes + (row * S + s) * 16);
+        r.rec = *reinterpret_cast<const uint2 *>(aux + (row * (S >> 3) + (s >> 3)) * 8);
+        return r;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int s, const uint32_t *, Dec & d) {
+        const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(w[q], d.w[q], d.w[4 + q]);
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.rec.x & 0xFFFFu)) * float(iq4xs_ls(r.rec, s & 7) - 32);
+        d.mn = 0.f;
+    }
+};
+
+template <> struct Sub<TQMOE_Q4_K> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint4 c; uint4 rec; };
+    static __device__ __forceinline__ Raw load(const uint8_t * __restrict__ codes, const uint8_t * __restrict__ aux, int64_t, int, int64_t row, int S, int s) {
+        Raw r;
+        r.c = *reinterpret_cast<const uint4 *>(codes + (row * S + s) * 16);
+        r.rec = *reinterpret_cast<const uint4 *>(aux + (row * (S >> 3) + (s >> 3)) * 16);
+        return r;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int s, const uint32_t *, Dec & d) {
+        const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) nibbles(w[q], d.w[q], d.w[4 + q]);
+        const uint32_t sc12[3] = {r.rec.y, r.rec.z, r.rec.w};
+        int sc, mn;
+        q4k_scale_min(sc12, s & 7, sc, mn);
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.rec.x & 0xFFFFu)) * float(sc);
+        d.mn = half_bits_to_float(uint16_t(r.rec.x >> 16)) * float(mn);
+    }
+};
+
+template <> struct Sub<TQMOE_NVFP4G> {
+    static constexpr bool kSplit = true;
+    struct Raw { uint4 c; uint32_t sc; float g; };
+    static __device__ __forceinline__ Raw load(const uint8_t * __restrict__ codes, const uint8_t * __restrict__ aux, int64_t rows_total, int cols, int64_t row,
+                                               int S, int s) {
+        Raw r;
+        r.c = *reinterpret_cast<const uint4 *>(codes + (row * S + s) * 16);
+        r.sc = *reinterpret_cast<const uint16_t *>(aux + row * (cols / 16) + 2 * s);
+        r.g = *reinterpret_cast<const float *>(aux + nvfp4_global_offset(rows_total, cols) + row * 4);
+        return r;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t *, Dec & d) {
+        const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) lookup16<kFp4T0, kFp4T1, kFp4T2, kFp4T3>(w[q], d.w[q], d.w[4 + q]);
+        // low nibbles = the first 16-weight group, high nibbles = the second; table values are twice the E2M1 value
+        d.s0 = e4m3_to_float(r.sc & 0xFFu) * (0.5f * r.g);
+        d.s1 = e4m3_to_float(r.sc >> 8) * (0.5f * r.g);
+        d.mn = 0.f;
+    }
+};
+
+template <> struct Sub<TQMOE_IQ3_S> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint32_t c[3]; uint4 rec; };
+    static __device__ __forceinline__ Raw load(const uint8_t * __restrict__ codes, const uint8_t * __restrict__ aux, int64_t, int, int64_t row, int S, int s) {
+        Raw r;
+        const uint32_t * cp = reinterpret_cast<const uint32_t *>(codes + (row * S + s) * 12);
+        r.c[0] = cp[0]; r.c[1] = cp[1]; r.c[2] = cp[2];
+        r.rec = *reinterpret_cast<const uint4 *>(aux + (row * (S >> 3) + (s >> 3)) * 16);
+        return r;
+    }
+    // grid: the 512-entry lattice in LDS
+    static __device__ __forceinline__ void decode(const Raw & r, int s, const uint32_t * grid, Dec & d) {
+        const int ib = s & 7;
+        const uint4 rec = r.rec;
+        const uint32_t qh = ib < 2 ? (rec.x >> (16 + 8 * ib)) & 0xFFu : ib < 6 ? (rec.y >> (8 * (ib - 2))) & 0xFFu : (rec.z >> (8 * (ib - 6))) & 0xFFu;
+        const uint32_t scb = (ib >> 1) < 2 ? (rec.z >> (16 + 8 * (ib >> 1))) & 0xFFu : (rec.w >> (8 * ((ib >> 1) - 2))) & 0xFFu;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            const uint32_t g = grid[((r.c[w >> 2] >> (8 * (w & 3))) & 0xFFu) | (((qh >> w) & 1u) << 8)];
+            // four sign bits -> byte masks 0xFF; negate the selected bytes: (g ^ m) + (m & 0x01010101), no carry leaves a byte
+            const uint32_t bits = (((r.c[2] >> (4 * w)) & 15u) * 0x00204081u) & 0x01010101u;
+            const uint32_t m = (bits << 8) - bits;
+            d.w[w] = (g ^ m) + bits;
+        }
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(rec.x & 0xFFFFu)) * float(1 + 2 * int((scb >> (4 * (ib & 1))) & 15u));
+        d.mn = 0.f;
+    }
+};
+
+template <uint32_t FMT> __device__ __forceinline__ const uint32_t * stage_grid(uint32_t * lds) {
+    if constexpr (FMT == TQMOE_IQ3_S) {
+        for (int i = threadIdx.x; i < 512; i += blockDim.x) lds[i] = d_iq3s_grid.v[i];
+        __syncthreads();
+        return lds;
+    } else {
+        return nullptr;
+    }
+}
+
+// sum over the LPR consecutive lanes of a row; valid in the last lane of each group
+template <int LPR> __device__ __forceinline__ float row_total(float v) {
+    v += dpp_f<kDppXor1>(v);
+    v += dpp_f<kDppXor2>(v);
+    v += dpp_f<kDppHalfMirror>(v);
+    if constexpr (LPR >= 16) v += dpp_f<kDppMirror>(v);
+    if constexpr (LPR >= 32) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));  // row_bcast:15
+    if constexpr (LPR >= 64) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));  // row_bcast:31
+    return v;
+}
+
+// The assignments that share this block's expert. mode 0: the block's own assignment only; mode 1: every assignment of
+// ids[0..A) with the same expert, and only the block of the first of them goes on (the others leave).
+constexpr int kMaxList = 1024;
+__device__ __forceinline__ int gather_same_expert(const int * __restrict__ ids, int A, int a, int e, int mode, int * list, int * meta) {
+    if (mode == 0) {
+        if (threadIdx.x == 0) list[0] = a;
+        __syncthreads();
+        return 1;
+    }
+    if (threadIdx.x == 0) { meta[0] = 0; meta[1] = 0x7FFFFFFF; }
+    __syncthreads();
+    for (int i = threadIdx.x; i < A; i += blockDim.x)
+        if (ids[i] == e) { atomicMin(&meta[1], i); const int pos = atomicAdd(&meta[0], 1); if (pos < kMaxList) list[pos] = i; }
+    __syncthreads();
+    return meta[1] == a ? min(meta[0], kMaxList) : 0;
+}
+
+// Core of every decode product: one block, one expert, rows [row0, row0 + NJ * 4 * (64 / LPR)) of up to two banks
+// (NB), NT activation rows at a time. Lane (rl, sl) of wave w handles row (j * 4 + w) * RW + rl, sub-blocks sl + LPR * m.
+// emit(j, nb, nt, value) is called in the last lane of each row group with the finished dot product.
+template <uint32_t FMT, int LPR, int M, int NB, int NT, int NJ, class Emit>
+__device__ __forceinline__ void block_rows(const BankView & b0, const BankView & b1, int e, int row0, int s_end, const ActBlock (&x)[NT][M],
+                                           const uint32_t * grid, Emit emit) {
+    using F = Sub<FMT>;
+    constexpr int RW = 64 / LPR;
+    const int S = b0.cols / 32, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int rl = lane / LPR, sl = lane % LPR;
+    const int64_t base = int64_t(e) * b0.rows + row0;
+#pragma unroll
+    for (int j0 = 0; j0 < NJ; j0 += 2) {
+        constexpr int U = NJ >= 2 ? 2 : 1;
+        typename F::Raw raw[U][NB][M];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    const BankView & b = nb ? b1 : b0;
+                    const int r = min(((j0 + u) * 4 + wave) * RW + rl, b0.rows - 1 - row0);
+                    raw[u][nb][m] = F::load(b.codes, b.aux, b.rows_total, b.cols, base + r, S, min(sl + LPR * m, S - 1));
+                }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                float acc[NT];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[nt] = 0.f;
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    Dec d;
+                    const int s = sl + LPR * m;
+                    F::decode(raw[u][nb][m], min(s, S - 1), grid, d);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const float v = dot_block<F::kSplit>(d, x[nt][m]);
+                        acc[nt] += s < s_end ? v : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float tot = row_total<LPR>(acc[nt]);
+                    if (sl == LPR - 1) emit(j0 + u, nb, nt, ((j0 + u) * 4 + wave) * RW + rl, tot);
+                }
+            }
+    }
+}
+
+template <int M, int NT>
+__device__ __forceinline__ void load_x(const uint8_t * __restrict__ image, const int64_t (&xrow)[NT], int S, int s_end, int lpr, int sl, ActBlock (&x)[NT][M]) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const int s = sl + lpr * m;
+            if (s < s_end) load_act_block(image + xrow[nt] * S * kImageSubBytes, S, s, x[nt][m]); else zero_act_block(x[nt][m]);
+        }
+}
+
+// ------------------------------------------------------------------------------------------- grouped mat-vec
+// grid (row tiles, assignments). y[a][r] for the tile's rows; NB banks (gate and up) share ids and the input image.
+// One block reads the tile's weights once for every assignment of its expert (mode 1), two activation rows at a time.
+template <uint32_t FMT, int LPR, int M, int NB, int NJ>
+__global__ __launch_bounds__(256) void matvec_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * y0, void * y1, uint32_t ytype,
+                                                const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_cols) {
+    __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : 1];
+    __shared__ int list[kMaxList], meta[2];
+    const uint32_t * grid = stage_grid<FMT>(grid_lds);
+    const int a = blockIdx.y, e = ids[a];
+    if (e < 0 || int64_t(e) * b0.rows >= b0.rows_total) return;   // skipped assignment, or an id outside the bank
+    const int cnt = gather_same_expert(ids, A, a, e, mode, list, meta);
+    if (cnt == 0) return;
+    constexpr int RW = 64 / LPR, kTile = NJ * 4 * RW;
+    const int S = b0.cols / 32, sl = (threadIdx.x & 63) % LPR, row0 = blockIdx.x * kTile, rows = b0.rows;
+    const int s_end = (a % slots) < topk ? S : shared_cols / 32;   // the shared expert's input row may be narrower
+    auto store = [&](int a2, int nb, int r, float v) {
+        if (row0 + r >= rows) return;
+        const int64_t o = int64_t(a2) * rows + row0 + r;
+        void * y = nb ? y1 : y0;
+        if (ytype == TQMOE_F32) static_cast<float *>(y)[o] = v; else static_cast<uint16_t *>(y)[o] = float_to_bf16_bits(v);
+    };
+    int i = 0;
+    for (; i + 2 <= cnt; i += 2) {
+        const int a0 = list[i], a1 = list[i + 1];
+        const int64_t xrow[2] = {a0 / xdiv, a1 / xdiv};
+        ActBlock x[2][M];
+        load_x<M, 2>(image, xrow, S, s_end, LPR, sl, x);
+        block_rows<FMT, LPR, M, NB, 2, NJ>(b0, b1, e, row0, s_end, x, grid, [&](int, int nb, int nt, int r, float v) { store(nt ? a1 : a0, nb, r, v); });
+    }
+    if (i < cnt) {
+        const int a0 = list[i];
+        const int64_t xrow[1] = {a0 / xdiv};
+        ActBlock x[1][M];
+        load_x<M, 1>(image, xrow, S, s_end, LPR, sl, x);
+        block_rows<FMT, LPR, M, NB, 1, NJ>(b0, b1, e, row0, s_end, x, grid, [&](int, int nb, int, int r, float v) { store(a0, nb, r, v); });
+    }
+}
+
+// ------------------------------------------------------------------------- fused gate + up + SwiGLU (layer path)
+// grid (ff / 32, n * slots): one block makes one 32-value sub-block of act = silu(gate x) * (up x) for every assignment
+// of its expert and writes it straight into the activation image the down product reads. ids: [n][slots] expert of
+// every (token, slot), the shared expert (bank index n_expert, rows below shared_ff only) in slot topk when slots > topk.
+template <uint32_t FMT, int LPR, int M>
+__global__ __launch_bounds__(256) void gateup_k(BankView bg, BankView bu, const uint8_t * __restrict__ ximage, uint8_t * __restrict__ aimage,
+                                                const int * __restrict__ ids, int A, int slots, int topk, int shared_ff, int mode) {
+    constexpr int RW = 64 / LPR, NJ = 32 / (4 * RW);
+    static_assert(NJ >= 1, "a block makes 32 rows: at least 8 lanes per row");
+    __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : 1];
+    __shared__ int list[kMaxList], meta[2];
+    __shared__ float gl[2][32], ul[2][32];
+    __shared__ int ql[2][32];
+    const uint32_t * grid = stage_grid<FMT>(grid_lds);
+    const int a = blockIdx.y, e = ids[a], row0 = blockIdx.x * 32;
+    if (e < 0 || int64_t(e) * bg.rows >= bg.rows_total || row0 >= ((a % slots) < topk ? bg.rows : shared_ff)) return;
+    const int cnt = gather_same_expert(ids, A, a, e, mode, list, meta);
+    if (cnt == 0) return;
+    const int S = bg.cols / 32, SA = bg.rows / 32, sl = (threadIdx.x & 63) % LPR;
+    // silu(g) * u of 32 rows for `nt` assignments (in gl / ul) -> their activation image sub-blocks
+    auto finish = [&](int nt_count, int a0, int a1) {
+        __syncthreads();
+        const int tid = threadIdx.x, which = tid >> 5, i = tid & 31;   // 32 consecutive lanes per assignment
+        if (tid < 64) {                                                 // wave 0, whole: the DPP reductions need every lane
+            const bool live = which < nt_count;
+            const float g = live ? gl[which][i] : 0.f, u = live ? ul[which][i] : 0.f;
+            const float v = g / (1.f + expf(-g)) * u;
+            float amax = fabsf(v);
+            amax = fmaxf(amax, dpp_f<kDppXor1>(amax));
+            amax = fmaxf(amax, dpp_f<kDppXor2>(amax));
+            amax = fmaxf(amax, dpp_f<kDppHalfMirror>(amax));
+            amax = fmaxf(amax, dpp_f<kDppMirror>(amax));
+            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+            const float inv = amax > 0.f ? 16383.f / amax : 0.f;
+            const int q = __float2int_rn(v * inv);
+            ql[which][i] = q;
+            int qs = q;
+            qs += dpp_i<kDppXor1>(qs);
+            qs += dpp_i<kDppXor2>(qs);
+            qs += dpp_i<kDppHalfMirror>(qs);
+            qs += dpp_i<kDppMirror>(qs);
+            qs += __shfl_xor(qs, 16, 64);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // ql is read below by other lanes of this same wave
+            __builtin_amdgcn_wave_barrier();
+            if (live) {
+                uint8_t * base = aimage + int64_t(which ? a1 : a0) * SA * kImageSubBytes;
+                if (i < 16) {   // dwords 0..7: hi plane, 8..15: lo plane
+                    const int d = i & 7;
+                    uint32_t word = 0;
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        const int qq = ql[which][4 * d + b];
+                        word |= uint32_t(i < 8 ? (qq >> 7) & 0xFF : qq & 127) << (8 * b);
+                    }
+                    reinterpret_cast<uint32_t *>(base + int64_t(blockIdx.x) * 64)[i] = word;
+                } else if (i == 16) {
+                    const float scale = amax * (1.f / 16383.f);
+                    *reinterpret_cast<float2 *>(base + int64_t(SA) * 64 + int64_t(blockIdx.x) * 8) = make_float2(scale, float(qs) * scale);
+                }
+            }
+        }
+        __syncthreads();
+    };
+    int i = 0;
+    for (; i + 2 <= cnt; i += 2) {
+        const int a0 = list[i], a1 = list[i + 1];
+        const int64_t xrow[2] = {a0 / slots, a1 / slots};
+        ActBlock x[2][M];
+        load_x<M, 2>(ximage, xrow, S, S, LPR, sl, x);
+        block_rows<FMT, LPR, M, 2, 2, NJ>(bg, bu, e, row0, S, x, grid, [&](int, int nb, int nt, int r, float v) { (nb ? ul : gl)[nt][r] = v; });
+        finish(2, a0, a1);
+    }
+    if (i < cnt) {
+        const int a0 = list[i];
+        const int64_t xrow[1] = {a0 / slots};
+        ActBlock x[1][M];
+        load_x<M, 1>(ximage, xrow, S, S, LPR, sl, x);
+        block_rows<FMT, LPR, M, 2, 1, NJ>(bg, bu, e, row0, S, x, grid, [&](int, int nb, int, int r, float v) { (nb ? ul : gl)[0][r] = v; });
+        finish(1, a0, a0);
+    }
+}
+
+// --------------------------------------------------------------------------------------------------- launchers
+constexpr int kMatvecNJ = 4;   // row steps per block of the plain products: 16 * (64 / LPR) rows per block
+
+template <uint32_t FMT, int LPR, int M> void launch_one_matvec(int nb, const MatvecArgs & k, hipStream_t s) {
+    constexpr int kTile = kMatvecNJ * 4 * (64 / LPR);
+    const dim3 grid(unsigned((k.b0.rows + kTile - 1) / kTile), unsigned(k.A));
+    if (nb == 2) matvec_k<FMT, LPR, M, 2, kMatvecNJ><<<grid, 256, 0, s>>>(k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols);
+    else matvec_k<FMT, LPR, M, 1, kMatvecNJ><<<grid, 256, 0, s>>>(k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols);
+}
+template <uint32_t FMT, int LPR, int M> void launch_one_gateup(const GateupArgs & k, hipStream_t s) {
+    const dim3 grid(unsigned(k.bg.rows / 32), unsigned(k.A));
+    gateup_k<FMT, LPR, M><<<grid, 256, 0, s>>>(k.bg, k.bu, k.ximage, k.aimage, k.ids, k.A, k.slots, k.topk, k.shared_ff, k.mode);
+}
+
+// the (lanes per row, sub-blocks per lane) pairs split_for() can return
+#define TQMOE_FOR_SPLITS(X) X(64, 1) X(64, 2) X(64, 3) X(64, 4) X(32, 1) X(32, 3) X(16, 1) X(16, 3) X(8, 1) X(8, 3)
+
+}  // namespace
+
+template <uint32_t FMT> void DecodeLaunch<FMT>::matvec(Split sp, int nb, const MatvecArgs & k, hipStream_t s) {
+#define X(L, MM) if (sp.lpr == L && sp.m == MM) return launch_one_matvec<FMT, L, MM>(nb, k, s);
+    TQMOE_FOR_SPLITS(X)
+#undef X
+}
+template <uint32_t FMT> void DecodeLaunch<FMT>::gateup(Split sp, const GateupArgs & k, hipStream_t s) {
+#define X(L, MM) if (sp.lpr == L && sp.m == MM) return launch_one_gateup<FMT, L, MM>(k, s);
+    TQMOE_FOR_SPLITS(X)
+#undef X
+}
+
+}  // namespace tqmoe

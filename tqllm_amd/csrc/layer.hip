@@ -7,7 +7,7 @@ int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);
 namespace {
 
 struct Plan {  // byte offsets into the workspace
-    size_t logits, ids, weights, shared_w, ximage, aimage, total;
+    size_t logits, ids, weights, shared_w, ids_ext, ximage, aimage, y, total;
 };
 
 Plan plan_for(const tqmoe_layer & L, int n) {
@@ -19,8 +19,10 @@ Plan plan_for(const tqmoe_layer & L, int n) {
     p.ids = take(size_t(n) * L.topk * 4);
     p.weights = take(size_t(n) * L.topk * 4);
     p.shared_w = take(size_t(n) * 4);
+    p.ids_ext = take(size_t(n) * slots * 4);
     p.ximage = take(tqmoe_act_image_bytes(n, L.hidden));
     p.aimage = take(tqmoe_act_image_bytes(n * slots, L.ff));
+    p.y = take(size_t(n) * slots * L.hidden * 4);
     p.total = o;
     return p;
 }
@@ -73,7 +75,15 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
 
     if (int32_t rc = tqmoe_router(L.router, L.router_type, L.shared_gate, x, xtype, logits, L.hidden, L.n_expert, n, stream, err)) return rc;
     if (int32_t rc = tqmoe_topk(logits, ids, weights, shared_w, L.n_expert, L.topk, n, L.weight_scale, stream, err)) return rc;
+    const int32_t * ids_ext = ids;
+    if (L.has_shared) {
+        if (int32_t rc = tqmoe_extend_ids(ids, reinterpret_cast<int32_t *>(ws + p.ids_ext), L.topk, n, L.n_expert, stream, err)) return rc;
+        ids_ext = reinterpret_cast<const int32_t *>(ws + p.ids_ext);
+    }
+    float * y = reinterpret_cast<float *>(ws + p.y);
     if (int32_t rc = tqmoe_quant_act(x, xtype, n, L.hidden, ws + p.ximage, stream, err)) return rc;
-    if (int32_t rc = tqmoe_expert_gateup(&L.gate, &L.up, ws + p.ximage, ws + p.aimage, ids, n, L.topk, L.has_shared, L.shared_ff, stream, err)) return rc;
-    return tqmoe_expert_down_combine(&L.down, ws + p.aimage, ids, weights, shared_w, out, otype, n, L.topk, L.has_shared, L.shared_ff, stream, err);
+    if (int32_t rc = tqmoe_expert_gateup(&L.gate, &L.up, ws + p.ximage, ws + p.aimage, ids_ext, n, slots, L.topk, L.shared_ff, stream, err)) return rc;
+    if (int32_t rc = tqmoe_expert_down(&L.down, ws + p.aimage, y, ids_ext, n, slots, L.topk, L.shared_ff, stream, err)) return rc;
+    return tqmoe_combine_strided(y, slots, L.has_shared ? y + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, weights, shared_w, out, otype,
+                                 L.hidden, L.topk, n, stream, err);
 }

@@ -29,12 +29,12 @@ __global__ __launch_bounds__(256) void load_k(uint32_t type, const uint8_t * __r
     const int s = int(idx % S);
     uint8_t * cd = codes + idx * code_bytes_per_sub(type);
     switch (type) {
-        case TQMOE_IQ4_XS: {  // 136 B per 256: d, scales_h, scales_l[4], qs[128]; nibble order already canonical
+        case TQMOE_IQ4_XS: {  // 136 B per 256: d, scales_h, scales_l[4], qs[128]; nibble order already canonical; tile-major
             const uint8_t * blk = src + (row * (S / 8) + s / 8) * 136;
             const uint8_t * q = blk + 8 + 16 * (s & 7);
-            pack_sub(cd, [&](int j) { return j < 16 ? q[j] & 15 : q[j - 16] >> 4; });
+            pack_sub(codes + iq4xs_code_offset(row, S, s), [&](int j) { return j < 16 ? q[j] & 15 : q[j - 16] >> 4; });
             if ((s & 7) == 0) {
-                uint8_t * a = aux + (row * (S / 8) + s / 8) * 8;
+                uint8_t * a = aux + iq4xs_aux_offset(row, S, s / 8);
                 *reinterpret_cast<uint2 *>(a) = make_uint2(rd_u32(blk), rd_u32(blk + 4));
             }
             break;
@@ -92,9 +92,9 @@ __global__ __launch_bounds__(256) void dequant_k(uint32_t type, const uint8_t * 
     float * y = out + idx * 32;
     switch (type) {
         case TQMOE_IQ4_XS: {
-            const uint2 rec = *reinterpret_cast<const uint2 *>(aux + (row * (S / 8) + s / 8) * 8);
+            const uint2 rec = *reinterpret_cast<const uint2 *>(aux + iq4xs_aux_offset(row, S, s / 8));
             const float dl = __fmul_rn(half_bits_to_float(uint16_t(rec.x & 0xFFFFu)), float(iq4xs_ls(rec, ib) - 32));
-            const uint4 c = *reinterpret_cast<const uint4 *>(cd);
+            const uint4 c = *reinterpret_cast<const uint4 *>(codes + iq4xs_code_offset(row, S, s));
             const uint32_t w[4] = {c.x, c.y, c.z, c.w};
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -179,6 +179,7 @@ int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err) {
     if (!is_bank_type(b->type)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: bank type %u is not supported", what, b->type);
     if (!b->codes || !b->aux || b->experts <= 0 || b->rows <= 0 || b->cols <= 0) return fail(err, TQMOE_E_ARG, "%s: invalid bank shape or pointer", what);
     if (b->cols % (b->type == TQMOE_NVFP4G ? 128 : 256)) return fail(err, TQMOE_E_ARG, "%s: cols %d is not a multiple of the block size", what, b->cols);
+    if (b->type == TQMOE_IQ4_XS && b->rows % 32) return fail(err, TQMOE_E_ARG, "%s: IQ4_XS banks need rows that are a multiple of 32 (got %d)", what, b->rows);
     return 0;
 }
 
@@ -189,6 +190,7 @@ using namespace tqmoe;
 extern "C" int32_t tqmoe_bank_layout(uint32_t type, int64_t rows_total, int32_t cols, size_t * code_bytes, size_t * aux_bytes, tqmoe_error * err) {
     if (!is_bank_type(type)) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_bank_layout: bank type %u is not supported", type);
     if (rows_total <= 0 || cols <= 0 || cols % (type == TQMOE_NVFP4G ? 128 : 256)) return fail(err, TQMOE_E_ARG, "tqmoe_bank_layout: invalid shape");
+    if (type == TQMOE_IQ4_XS && rows_total % 32) return fail(err, TQMOE_E_ARG, "tqmoe_bank_layout: IQ4_XS banks need a multiple of 32 rows");
     if (code_bytes) *code_bytes = size_t(rows_total * code_row_bytes(type, cols));
     if (aux_bytes) *aux_bytes = type == TQMOE_NVFP4G ? size_t(nvfp4_global_offset(rows_total, cols) + rows_total * 4) : size_t(rows_total * aux_row_bytes(type, cols));
     return ok(err);

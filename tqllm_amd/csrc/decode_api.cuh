@@ -39,7 +39,8 @@ template <uint32_t FMT> struct DecodeLaunch {
     static void matvec(Split sp, int nb, const MatvecArgs & k, hipStream_t s);
     static void gateup(Split sp, const GateupArgs & k, hipStream_t s);
 };
-extern template struct DecodeLaunch<TQMOE_IQ4_XS>;
+template <> void DecodeLaunch<TQMOE_IQ4_XS>::matvec(Split sp, int nb, const MatvecArgs & k, hipStream_t s);   // its own kernels (decode_iq4xs.hip)
+template <> void DecodeLaunch<TQMOE_IQ4_XS>::gateup(Split sp, const GateupArgs & k, hipStream_t s);
 extern template struct DecodeLaunch<TQMOE_Q4_K>;
 extern template struct DecodeLaunch<TQMOE_IQ3_S>;
 extern template struct DecodeLaunch<TQMOE_NVFP4G>;

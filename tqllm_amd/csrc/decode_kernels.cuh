@@ -25,58 +25,55 @@ namespace {
 // A weight sub-block is fetched (Raw: what one lane loads), decoded once into eight dwords of int8 values in the order
 // of the activation planes (Dec), and multiplied with any number of activation blocks.
 struct Dec {
-    uint32_t w[8];   // int8 x 4 each; w[q] pairs with activation dword q
+    uint32_t w[8];   // int8 x 4 each; w[q] = values 4q .. 4q + 3 of the sub-block
     float s0, s1;    // scale of dwords 0..3 and of dwords 4..7 (equal except for NVFP4G's two 16-weight groups)
     float mn;        // coefficient of the block's activation sum (Q4_K minimum), else 0
 };
 
-__device__ __forceinline__ int dot4x(const uint32_t * w, const int * x) {
+// w: natural dwords d0 .. d0 + 3 of a sub-block's values; x: a plane indexed by plane position
+template <int D0> __device__ __forceinline__ int dot4x(const uint32_t * w, const int * x) {
     int acc = 0;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_sdot4(int(w[q]), x[q], acc, false);
+    for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_sdot4(int(w[q]), x[plane_pos(D0 + q)], acc, false);
     return acc;
 }
 template <bool SPLIT> __device__ __forceinline__ float dot_block(const Dec & d, const ActBlock & x) {
     if constexpr (SPLIT) {
-        const int t0 = (dot4x(d.w, x.hi) << 7) + dot4x(d.w, x.lo);
-        const int t1 = (dot4x(d.w + 4, x.hi + 4) << 7) + dot4x(d.w + 4, x.lo + 4);
+        const int t0 = (dot4x<0>(d.w, x.hi) << 7) + dot4x<0>(d.w, x.lo);
+        const int t1 = (dot4x<4>(d.w + 4, x.hi) << 7) + dot4x<4>(d.w + 4, x.lo);
         return (float(t0) * d.s0 + float(t1) * d.s1) * x.scale;
     } else {
         int hi = 0, lo = 0;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) { hi = __builtin_amdgcn_sdot4(int(d.w[q]), x.hi[q], hi, false); lo = __builtin_amdgcn_sdot4(int(d.w[q]), x.lo[q], lo, false); }
+        for (int q = 0; q < 8; ++q) {
+            hi = __builtin_amdgcn_sdot4(int(d.w[q]), x.hi[plane_pos(q)], hi, false);
+            lo = __builtin_amdgcn_sdot4(int(d.w[q]), x.lo[plane_pos(q)], lo, false);
+        }
         return float((hi << 7) + lo) * (d.s0 * x.scale) - d.mn * x.sum;
     }
 }
 
-template <uint32_t FMT> struct Sub;
+// Uniform base pointers of one bank for the rows [row0, ...) of expert e: lanes add 32-bit offsets to them.
+struct Tile { const uint8_t * codes; const uint8_t * aux; const uint8_t * aux2; };
+template <uint32_t FMT> __device__ __forceinline__ Tile tile_of(const BankView & b, int e, int row0) {
+    const int64_t row = int64_t(e) * b.rows + row0;
+    Tile t;
+    t.codes = b.codes + row * code_row_bytes(FMT, b.cols);
+    t.aux = b.aux + row * aux_row_bytes(FMT, b.cols);
+    t.aux2 = FMT == TQMOE_NVFP4G ? b.aux + nvfp4_global_offset(b.rows_total, b.cols) + row * 4 : nullptr;
+    return t;
+}
 
-template <> struct Sub<TQMOE_IQ4_XS> {
-    static constexpr bool kSplit = false;
-    struct Raw { uint4 c; uint2 rec; };
-    static __device__ __forceinline__ Raw load(const uint8_t * __restrict__ codes, const uint8_t * __restrict__ aux, int64_t, int, int64_t row, int S, int s) {
-        Raw r;
-        r.c = *reinterpret_cast<const uint4 *>(codes + (row * S + s) * 16);
-        r.rec = *reinterpret_cast<const uint2 *>(aux + (row * (S >> 3) + (s >> 3)) * 8);
-        return r;
-    }
-    static __device__ __forceinline__ void decode(const Raw & r, int s, const uint32_t *, Dec & d) {
-        const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(w[q], d.w[q], d.w[4 + q]);
-        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.rec.x & 0xFFFFu)) * float(iq4xs_ls(r.rec, s & 7) - 32);
-        d.mn = 0.f;
-    }
-};
+template <uint32_t FMT> struct Sub;
 
 template <> struct Sub<TQMOE_Q4_K> {
     static constexpr bool kSplit = false;
     struct Raw { uint4 c; uint4 rec; };
-    static __device__ __forceinline__ Raw load(const uint8_t * __restrict__ codes, const uint8_t * __restrict__ aux, int64_t, int, int64_t row, int S, int s) {
-        Raw r;
-        r.c = *reinterpret_cast<const uint4 *>(codes + (row * S + s) * 16);
-        r.rec = *reinterpret_cast<const uint4 *>(aux + (row * (S >> 3) + (s >> 3)) * 16);
-        return r;
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        v.c = *reinterpret_cast<const uint4 *>(t.codes + (r * S + s) * 16u);
+        v.rec = *reinterpret_cast<const uint4 *>(t.aux + (r * (S >> 3) + (s >> 3)) * 16u);
+        return v;
     }
     static __device__ __forceinline__ void decode(const Raw & r, int s, const uint32_t *, Dec & d) {
         const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
@@ -93,13 +90,12 @@ template <> struct Sub<TQMOE_Q4_K> {
 template <> struct Sub<TQMOE_NVFP4G> {
     static constexpr bool kSplit = true;
     struct Raw { uint4 c; uint32_t sc; float g; };
-    static __device__ __forceinline__ Raw load(const uint8_t * __restrict__ codes, const uint8_t * __restrict__ aux, int64_t rows_total, int cols, int64_t row,
-                                               int S, int s) {
-        Raw r;
-        r.c = *reinterpret_cast<const uint4 *>(codes + (row * S + s) * 16);
-        r.sc = *reinterpret_cast<const uint16_t *>(aux + row * (cols / 16) + 2 * s);
-        r.g = *reinterpret_cast<const float *>(aux + nvfp4_global_offset(rows_total, cols) + row * 4);
-        return r;
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        v.c = *reinterpret_cast<const uint4 *>(t.codes + (r * S + s) * 16u);
+        v.sc = *reinterpret_cast<const uint16_t *>(t.aux + (r * S + s) * 2u);
+        v.g = *reinterpret_cast<const float *>(t.aux2 + r * 4u);
+        return v;
     }
     static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t *, Dec & d) {
         const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
@@ -115,12 +111,12 @@ template <> struct Sub<TQMOE_NVFP4G> {
 template <> struct Sub<TQMOE_IQ3_S> {
     static constexpr bool kSplit = false;
     struct Raw { uint32_t c[3]; uint4 rec; };
-    static __device__ __forceinline__ Raw load(const uint8_t * __restrict__ codes, const uint8_t * __restrict__ aux, int64_t, int, int64_t row, int S, int s) {
-        Raw r;
-        const uint32_t * cp = reinterpret_cast<const uint32_t *>(codes + (row * S + s) * 12);
-        r.c[0] = cp[0]; r.c[1] = cp[1]; r.c[2] = cp[2];
-        r.rec = *reinterpret_cast<const uint4 *>(aux + (row * (S >> 3) + (s >> 3)) * 16);
-        return r;
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        const uint32_t * cp = reinterpret_cast<const uint32_t *>(t.codes + (r * S + s) * 12u);
+        v.c[0] = cp[0]; v.c[1] = cp[1]; v.c[2] = cp[2];
+        v.rec = *reinterpret_cast<const uint4 *>(t.aux + (r * (S >> 3) + (s >> 3)) * 16u);
+        return v;
     }
     // grid: the 512-entry lattice in LDS
     static __device__ __forceinline__ void decode(const Raw & r, int s, const uint32_t * grid, Dec & d) {
@@ -162,48 +158,49 @@ template <int LPR> __device__ __forceinline__ float row_total(float v) {
     return v;
 }
 
-// The assignments that share this block's expert. mode 0: the block's own assignment only; mode 1: every assignment of
-// ids[0..A) with the same expert, and only the block of the first of them goes on (the others leave).
-constexpr int kMaxList = 1024;
-__device__ __forceinline__ int gather_same_expert(const int * __restrict__ ids, int A, int a, int e, int mode, int * list, int * meta) {
-    if (mode == 0) {
-        if (threadIdx.x == 0) list[0] = a;
-        __syncthreads();
-        return 1;
-    }
+// Pairing of the assignments that share an expert, so that their blocks read the weights once for two input rows.
+// mode 0: every assignment alone. mode 1: among the assignments of ids[0..A) with this block's expert, in index order,
+// the 1st, 3rd, ... each take the next one along (returns 2 and sets partner) or go alone when they are the last
+// (returns 1); the 2nd, 4th, ... leave (returns 0). meta: two ints of LDS.
+__device__ __forceinline__ int pair_up(const int * __restrict__ ids, int A, int a, int e, int mode, int * meta, int & partner) {
+    partner = a;
+    if (mode == 0) return 1;
     if (threadIdx.x == 0) { meta[0] = 0; meta[1] = 0x7FFFFFFF; }
     __syncthreads();
     for (int i = threadIdx.x; i < A; i += blockDim.x)
-        if (ids[i] == e) { atomicMin(&meta[1], i); const int pos = atomicAdd(&meta[0], 1); if (pos < kMaxList) list[pos] = i; }
+        if (ids[i] == e) {
+            if (i < a) atomicAdd(&meta[0], 1);
+            if (i > a) atomicMin(&meta[1], i);
+        }
     __syncthreads();
-    return meta[1] == a ? min(meta[0], kMaxList) : 0;
+    if (meta[0] & 1) return 0;
+    if (meta[1] == 0x7FFFFFFF) return 1;
+    partner = meta[1];
+    return 2;
 }
 
-// Core of every decode product: one block, one expert, rows [row0, row0 + NJ * 4 * (64 / LPR)) of up to two banks
-// (NB), NT activation rows at a time. Lane (rl, sl) of wave w handles row (j * 4 + w) * RW + rl, sub-blocks sl + LPR * m.
-// emit(j, nb, nt, value) is called in the last lane of each row group with the finished dot product.
-template <uint32_t FMT, int LPR, int M, int NB, int NT, int NJ, class Emit>
-__device__ __forceinline__ void block_rows(const BankView & b0, const BankView & b1, int e, int row0, int s_end, const ActBlock (&x)[NT][M],
-                                           const uint32_t * grid, Emit emit) {
+// Core of every decode product: one block of NW waves, rows [0, NJ * NW * (64 / LPR)) of the tiles of NB banks (the
+// same rows of each), NT activation rows at a time. Lane (rl, sl) of wave w handles row (j * NW + w) * RW + rl and
+// sub-blocks sl + LPR * m of it. Rows past `rows_left` are computed on the last valid row (and dropped by emit's
+// caller). emit(nb, nt, row, value) runs in the last lane of each row group.
+template <uint32_t FMT, int LPR, int M, int NB, int NT, int NJ, int NW, class Emit>
+__device__ __forceinline__ void block_rows(const Tile (&tile)[NB], int S, int rows_left, const ActBlock (&x)[NT][M], const uint32_t * grid, Emit emit) {
     using F = Sub<FMT>;
-    constexpr int RW = 64 / LPR;
-    const int S = b0.cols / 32, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int RW = 64 / LPR, U = NJ >= 2 ? 2 : 1;
+    static_assert(NJ % U == 0, "row steps come in pairs");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rl = lane / LPR, sl = lane % LPR;
-    const int64_t base = int64_t(e) * b0.rows + row0;
+    const uint32_t last = uint32_t(rows_left - 1);
 #pragma unroll
-    for (int j0 = 0; j0 < NJ; j0 += 2) {
-        constexpr int U = NJ >= 2 ? 2 : 1;
+    for (int j0 = 0; j0 < NJ; j0 += U) {
         typename F::Raw raw[U][NB][M];
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-                for (int m = 0; m < M; ++m) {
-                    const BankView & b = nb ? b1 : b0;
-                    const int r = min(((j0 + u) * 4 + wave) * RW + rl, b0.rows - 1 - row0);
-                    raw[u][nb][m] = F::load(b.codes, b.aux, b.rows_total, b.cols, base + r, S, min(sl + LPR * m, S - 1));
-                }
+                for (int m = 0; m < M; ++m)
+                    raw[u][nb][m] = F::load(tile[nb], min(uint32_t(((j0 + u) * NW + wave) * RW + rl), last), uint32_t(S), min(uint32_t(sl + LPR * m), uint32_t(S - 1)));
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -214,167 +211,126 @@ __device__ __forceinline__ void block_rows(const BankView & b0, const BankView &
 #pragma unroll
                 for (int m = 0; m < M; ++m) {
                     Dec d;
-                    const int s = sl + LPR * m;
-                    F::decode(raw[u][nb][m], min(s, S - 1), grid, d);
+                    F::decode(raw[u][nb][m], min(sl + LPR * m, S - 1), grid, d);
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        const float v = dot_block<F::kSplit>(d, x[nt][m]);
-                        acc[nt] += s < s_end ? v : 0.f;
-                    }
+                    for (int nt = 0; nt < NT; ++nt) acc[nt] += dot_block<F::kSplit>(d, x[nt][m]);   // blocks past the row's end are zero
                 }
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     const float tot = row_total<LPR>(acc[nt]);
-                    if (sl == LPR - 1) emit(j0 + u, nb, nt, ((j0 + u) * 4 + wave) * RW + rl, tot);
+                    if (sl == LPR - 1) emit(nb, nt, ((j0 + u) * NW + wave) * RW + rl, tot);
                 }
             }
     }
 }
 
+// the lane's activation blocks of NT image rows; sub-blocks at or past s_end are zero
 template <int M, int NT>
-__device__ __forceinline__ void load_x(const uint8_t * __restrict__ image, const int64_t (&xrow)[NT], int S, int s_end, int lpr, int sl, ActBlock (&x)[NT][M]) {
+__device__ __forceinline__ void load_x(const uint8_t * __restrict__ image, const int (&xrow)[NT], int S, int s_end, int lpr, int sl, ActBlock (&x)[NT][M]) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             const int s = sl + lpr * m;
-            if (s < s_end) load_act_block(image + xrow[nt] * S * kImageSubBytes, S, s, x[nt][m]); else zero_act_block(x[nt][m]);
+            if (s < s_end) load_act_block(image + int64_t(xrow[nt]) * S * kImageSubBytes, S, s, x[nt][m]); else zero_act_block(x[nt][m]);
         }
 }
 
 // ------------------------------------------------------------------------------------------- grouped mat-vec
-// grid (row tiles, assignments). y[a][r] for the tile's rows; NB banks (gate and up) share ids and the input image.
-// One block reads the tile's weights once for every assignment of its expert (mode 1), two activation rows at a time.
-template <uint32_t FMT, int LPR, int M, int NB, int NJ>
-__global__ __launch_bounds__(256) void matvec_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * y0, void * y1, uint32_t ytype,
-                                                const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_cols) {
+// grid (row tiles, assignments), NW waves. y[a][r] for the tile's rows; NB banks (gate and up) share ids and the input.
+template <uint32_t FMT, int LPR, int M, int NB, int NJ, int NW>
+__global__ __launch_bounds__(NW * 64) void matvec_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * y0, void * y1, uint32_t ytype,
+                                                    const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_cols) {
     __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : 1];
-    __shared__ int list[kMaxList], meta[2];
+    __shared__ int meta[2];
     const uint32_t * grid = stage_grid<FMT>(grid_lds);
     const int a = blockIdx.y, e = ids[a];
     if (e < 0 || int64_t(e) * b0.rows >= b0.rows_total) return;   // skipped assignment, or an id outside the bank
-    const int cnt = gather_same_expert(ids, A, a, e, mode, list, meta);
+    int a1;
+    const int cnt = pair_up(ids, A, a, e, mode, meta, a1);
     if (cnt == 0) return;
-    constexpr int RW = 64 / LPR, kTile = NJ * 4 * RW;
+    constexpr int RW = 64 / LPR, kTile = NJ * NW * RW;
     const int S = b0.cols / 32, sl = (threadIdx.x & 63) % LPR, row0 = blockIdx.x * kTile, rows = b0.rows;
     const int s_end = (a % slots) < topk ? S : shared_cols / 32;   // the shared expert's input row may be narrower
+    Tile tile[NB];
+    tile[0] = tile_of<FMT>(b0, e, row0);
+    if constexpr (NB == 2) tile[1] = tile_of<FMT>(b1, e, row0);
     auto store = [&](int a2, int nb, int r, float v) {
         if (row0 + r >= rows) return;
         const int64_t o = int64_t(a2) * rows + row0 + r;
         void * y = nb ? y1 : y0;
         if (ytype == TQMOE_F32) static_cast<float *>(y)[o] = v; else static_cast<uint16_t *>(y)[o] = float_to_bf16_bits(v);
     };
-    int i = 0;
-    for (; i + 2 <= cnt; i += 2) {
-        const int a0 = list[i], a1 = list[i + 1];
-        const int64_t xrow[2] = {a0 / xdiv, a1 / xdiv};
+    if (cnt == 2) {
+        const int xrow[2] = {a / xdiv, a1 / xdiv};
         ActBlock x[2][M];
         load_x<M, 2>(image, xrow, S, s_end, LPR, sl, x);
-        block_rows<FMT, LPR, M, NB, 2, NJ>(b0, b1, e, row0, s_end, x, grid, [&](int, int nb, int nt, int r, float v) { store(nt ? a1 : a0, nb, r, v); });
-    }
-    if (i < cnt) {
-        const int a0 = list[i];
-        const int64_t xrow[1] = {a0 / xdiv};
+        block_rows<FMT, LPR, M, NB, 2, NJ, NW>(tile, S, rows - row0, x, grid, [&](int nb, int nt, int r, float v) { store(nt ? a1 : a, nb, r, v); });
+    } else {
+        const int xrow[1] = {a / xdiv};
         ActBlock x[1][M];
         load_x<M, 1>(image, xrow, S, s_end, LPR, sl, x);
-        block_rows<FMT, LPR, M, NB, 1, NJ>(b0, b1, e, row0, s_end, x, grid, [&](int, int nb, int, int r, float v) { store(a0, nb, r, v); });
+        block_rows<FMT, LPR, M, NB, 1, NJ, NW>(tile, S, rows - row0, x, grid, [&](int nb, int, int r, float v) { store(a, nb, r, v); });
     }
 }
 
 // ------------------------------------------------------------------------- fused gate + up + SwiGLU (layer path)
-// grid (ff / 32, n * slots): one block makes one 32-value sub-block of act = silu(gate x) * (up x) for every assignment
-// of its expert and writes it straight into the activation image the down product reads. ids: [n][slots] expert of
-// every (token, slot), the shared expert (bank index n_expert, rows below shared_ff only) in slot topk when slots > topk.
-template <uint32_t FMT, int LPR, int M>
-__global__ __launch_bounds__(256) void gateup_k(BankView bg, BankView bu, const uint8_t * __restrict__ ximage, uint8_t * __restrict__ aimage,
-                                                const int * __restrict__ ids, int A, int slots, int topk, int shared_ff, int mode) {
-    constexpr int RW = 64 / LPR, NJ = 32 / (4 * RW);
-    static_assert(NJ >= 1, "a block makes 32 rows: at least 8 lanes per row");
+// grid (ff / 32, n * slots), NW waves: one block makes one 32-value sub-block of act = silu(gate x) * (up x) for its
+// assignment (and the paired one) and writes it straight into the activation image the down product reads. ids:
+// [n][slots] expert of every (token, slot); slots past topk hold the shared expert, which only has shared_ff rows.
+template <uint32_t FMT, int LPR, int M, int NW>
+__global__ __launch_bounds__(NW * 64) void gateup_k(BankView bg, BankView bu, const uint8_t * __restrict__ ximage, uint8_t * __restrict__ aimage,
+                                                    const int * __restrict__ ids, int A, int slots, int topk, int shared_ff, int mode) {
+    constexpr int RW = 64 / LPR, NJ = 32 / (NW * RW);
+    static_assert(NJ >= 1 && NJ * NW * RW == 32, "a block makes exactly 32 rows");
     __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : 1];
-    __shared__ int list[kMaxList], meta[2];
+    __shared__ int meta[2];
     __shared__ float gl[2][32], ul[2][32];
     __shared__ int ql[2][32];
     const uint32_t * grid = stage_grid<FMT>(grid_lds);
     const int a = blockIdx.y, e = ids[a], row0 = blockIdx.x * 32;
     if (e < 0 || int64_t(e) * bg.rows >= bg.rows_total || row0 >= ((a % slots) < topk ? bg.rows : shared_ff)) return;
-    const int cnt = gather_same_expert(ids, A, a, e, mode, list, meta);
+    int a1;
+    const int cnt = pair_up(ids, A, a, e, mode, meta, a1);
     if (cnt == 0) return;
     const int S = bg.cols / 32, SA = bg.rows / 32, sl = (threadIdx.x & 63) % LPR;
-    // silu(g) * u of 32 rows for `nt` assignments (in gl / ul) -> their activation image sub-blocks
-    auto finish = [&](int nt_count, int a0, int a1) {
-        __syncthreads();
-        const int tid = threadIdx.x, which = tid >> 5, i = tid & 31;   // 32 consecutive lanes per assignment
-        if (tid < 64) {                                                 // wave 0, whole: the DPP reductions need every lane
-            const bool live = which < nt_count;
-            const float g = live ? gl[which][i] : 0.f, u = live ? ul[which][i] : 0.f;
-            const float v = g / (1.f + expf(-g)) * u;
-            float amax = fabsf(v);
-            amax = fmaxf(amax, dpp_f<kDppXor1>(amax));
-            amax = fmaxf(amax, dpp_f<kDppXor2>(amax));
-            amax = fmaxf(amax, dpp_f<kDppHalfMirror>(amax));
-            amax = fmaxf(amax, dpp_f<kDppMirror>(amax));
-            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-            const float inv = amax > 0.f ? 16383.f / amax : 0.f;
-            const int q = __float2int_rn(v * inv);
-            ql[which][i] = q;
-            int qs = q;
-            qs += dpp_i<kDppXor1>(qs);
-            qs += dpp_i<kDppXor2>(qs);
-            qs += dpp_i<kDppHalfMirror>(qs);
-            qs += dpp_i<kDppMirror>(qs);
-            qs += __shfl_xor(qs, 16, 64);
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // ql is read below by other lanes of this same wave
-            __builtin_amdgcn_wave_barrier();
-            if (live) {
-                uint8_t * base = aimage + int64_t(which ? a1 : a0) * SA * kImageSubBytes;
-                if (i < 16) {   // dwords 0..7: hi plane, 8..15: lo plane
-                    const int d = i & 7;
-                    uint32_t word = 0;
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        const int qq = ql[which][4 * d + b];
-                        word |= uint32_t(i < 8 ? (qq >> 7) & 0xFF : qq & 127) << (8 * b);
-                    }
-                    reinterpret_cast<uint32_t *>(base + int64_t(blockIdx.x) * 64)[i] = word;
-                } else if (i == 16) {
-                    const float scale = amax * (1.f / 16383.f);
-                    *reinterpret_cast<float2 *>(base + int64_t(SA) * 64 + int64_t(blockIdx.x) * 8) = make_float2(scale, float(qs) * scale);
-                }
-            }
-        }
-        __syncthreads();
-    };
-    int i = 0;
-    for (; i + 2 <= cnt; i += 2) {
-        const int a0 = list[i], a1 = list[i + 1];
-        const int64_t xrow[2] = {a0 / slots, a1 / slots};
+    const Tile tile[2] = {tile_of<FMT>(bg, e, row0), tile_of<FMT>(bu, e, row0)};
+    if (cnt == 2) {
+        const int xrow[2] = {a / slots, a1 / slots};
         ActBlock x[2][M];
         load_x<M, 2>(ximage, xrow, S, S, LPR, sl, x);
-        block_rows<FMT, LPR, M, 2, 2, NJ>(bg, bu, e, row0, S, x, grid, [&](int, int nb, int nt, int r, float v) { (nb ? ul : gl)[nt][r] = v; });
-        finish(2, a0, a1);
-    }
-    if (i < cnt) {
-        const int a0 = list[i];
-        const int64_t xrow[1] = {a0 / slots};
+        block_rows<FMT, LPR, M, 2, 2, NJ, NW>(tile, S, 32, x, grid, [&](int nb, int nt, int r, float v) { (nb ? ul : gl)[nt][r] = v; });
+    } else {
+        const int xrow[1] = {a / slots};
         ActBlock x[1][M];
         load_x<M, 1>(ximage, xrow, S, S, LPR, sl, x);
-        block_rows<FMT, LPR, M, 2, 1, NJ>(bg, bu, e, row0, S, x, grid, [&](int, int nb, int, int r, float v) { (nb ? ul : gl)[0][r] = v; });
-        finish(1, a0, a0);
+        block_rows<FMT, LPR, M, 2, 1, NJ, NW>(tile, S, 32, x, grid, [&](int nb, int, int r, float v) { (nb ? ul : gl)[0][r] = v; });
+    }
+    __syncthreads();
+    // silu(g) * u of the 32 rows -> the activation image sub-block of each assignment: 32 lanes per assignment in wave 0
+    const int tid = threadIdx.x, which = tid >> 5, i = tid & 31;
+    if (tid < 64) {                                                 // the whole wave: the lane exchanges need every lane
+        const bool live = which < cnt;
+        const float g = live ? gl[which][i] : 0.f, u = live ? ul[which][i] : 0.f;
+        quantise_block_lanes(g / (1.f + expf(-g)) * u, i, live, ql[which], aimage + int64_t(which ? a1 : a) * SA * kImageSubBytes, SA, blockIdx.x);
     }
 }
 
 // --------------------------------------------------------------------------------------------------- launchers
-constexpr int kMatvecNJ = 4;   // row steps per block of the plain products: 16 * (64 / LPR) rows per block
+constexpr int kMatvecNJ = 4, kMatvecNW = 4;   // plain products: 4 row steps of 4 waves, 16 * (64 / LPR) rows per block
+constexpr int kGateupNW = 8;                   // gate/up: 8 waves share the block's 32 + 32 rows
 
 template <uint32_t FMT, int LPR, int M> void launch_one_matvec(int nb, const MatvecArgs & k, hipStream_t s) {
-    constexpr int kTile = kMatvecNJ * 4 * (64 / LPR);
+    constexpr int kTile = kMatvecNJ * kMatvecNW * (64 / LPR);
     const dim3 grid(unsigned((k.b0.rows + kTile - 1) / kTile), unsigned(k.A));
-    if (nb == 2) matvec_k<FMT, LPR, M, 2, kMatvecNJ><<<grid, 256, 0, s>>>(k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols);
-    else matvec_k<FMT, LPR, M, 1, kMatvecNJ><<<grid, 256, 0, s>>>(k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols);
+    if (nb == 2) matvec_k<FMT, LPR, M, 2, kMatvecNJ, kMatvecNW><<<grid, kMatvecNW * 64, 0, s>>>(k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols);
+    else matvec_k<FMT, LPR, M, 1, kMatvecNJ, kMatvecNW><<<grid, kMatvecNW * 64, 0, s>>>(k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols);
 }
 template <uint32_t FMT, int LPR, int M> void launch_one_gateup(const GateupArgs & k, hipStream_t s) {
     const dim3 grid(unsigned(k.bg.rows / 32), unsigned(k.A));
-    gateup_k<FMT, LPR, M><<<grid, 256, 0, s>>>(k.bg, k.bu, k.ximage, k.aimage, k.ids, k.A, k.slots, k.topk, k.shared_ff, k.mode);
+    // as many waves as divide the block's 32 rows: 8 for 8 lanes or more per row
+    constexpr int NW = 32 / (64 / LPR) >= kGateupNW ? kGateupNW : 32 / (64 / LPR);
+    gateup_k<FMT, LPR, M, NW><<<grid, NW * 64, 0, s>>>(k.bg, k.bu, k.ximage, k.aimage, k.ids, k.A, k.slots, k.topk, k.shared_ff, k.mode);
 }
 
 // the (lanes per row, sub-blocks per lane) pairs split_for() can return

@@ -17,6 +17,12 @@ __host__ __device__ constexpr int64_t aux_row_bytes(uint32_t type, int cols) {
 // NVFP4G: offset of the per-row fp32 globals inside the aux plane
 __host__ __device__ constexpr int64_t nvfp4_global_offset(int64_t rows_total, int cols) { return (rows_total * (cols / 16) + 15) / 16 * 16; }
 
+// IQ4_XS banks are stored tile-major: 32 consecutive rows form a tile, and inside a tile the codes of sub-block s of
+// all 32 rows are contiguous (512 B), as are the 32 records of a super-block (256 B). A wave then reads whole tiles with
+// fully coalesced loads whichever lane owns which row. rows of an expert must be a multiple of 32.
+__host__ __device__ constexpr int64_t iq4xs_code_offset(int64_t row, int S, int s) { return (((row >> 5) * S + s) * 32 + (row & 31)) * 16; }
+__host__ __device__ constexpr int64_t iq4xs_aux_offset(int64_t row, int S, int sb) { return (((row >> 5) * (S >> 3) + sb) * 32 + (row & 31)) * 8; }
+
 // IQ4_NL / IQ4_XS value table {-127,-104,-83,-65,-49,-35,-22,-10,1,13,25,38,53,69,89,113} as four little-endian dwords
 constexpr uint32_t kIq4T0 = 0xBFAD9881u, kIq4T1 = 0xF6EADDCFu, kIq4T2 = 0x26190D01u, kIq4T3 = 0x71594535u;
 // 2 * E2M1 {0,.5,1,1.5,2,3,4,6, -0,-.5,-1,-1.5,-2,-3,-4,-6} = {0,1,2,3,4,6,8,12, 0,-1,-2,-3,-4,-6,-8,-12}

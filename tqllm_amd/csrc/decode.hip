@@ -152,6 +152,7 @@ extern "C" int32_t tqmoe_expert_down(const tqmoe_bank * down, const void * act_i
     const char * what = "tqmoe_expert_down";
     if (n <= 0 || topk <= 0 || slots < topk) return fail(err, TQMOE_E_ARG, "%s: invalid shape", what);
     if (slots > topk && (!down || shared_ff <= 0 || shared_ff > down->cols || shared_ff % 32)) return fail(err, TQMOE_E_ARG, "%s: invalid shared_ff", what);
+    if (slots > topk && down->type == TQMOE_IQ4_XS && shared_ff % 256) return fail(err, TQMOE_E_UNSUPPORTED, "%s: IQ4_XS needs shared_ff in whole 256-weight blocks", what);
     return matvec_common(down, nullptr, act_image, y, nullptr, TQMOE_F32, ids, int64_t(n) * slots, 1, slots, topk, shared_ff, stream, err, what);
 }
 

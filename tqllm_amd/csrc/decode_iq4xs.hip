@@ -13,6 +13,8 @@
 #include "decode_api.cuh"
 #include "formats.cuh"
 
+#include <cstdlib>
+
 namespace tqmoe {
 namespace {
 
@@ -55,20 +57,38 @@ __device__ __forceinline__ int chunk_up(const int * __restrict__ ids, int A, int
     return n;
 }
 
+// 16 four-bit codes (two dwords) -> operand B of the MFMA: the lookups of lookup16(). The selector of the third pick
+// is (bit 3 of the code at bit 2) | byte position, written as a bit-field insert so that it is one instruction.
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) { return (x & mask) | (bits & ~mask); }
+__device__ __forceinline__ v4i decode16(uint2 c, uint32_t pos) {
+    v4i w;
+    const uint32_t k7 = 0x07070707u, k4 = 0x04040404u;
+    const uint32_t x0 = c.x, x1 = c.y;
+    const uint32_t i0 = x0 & k7, j0 = (x0 >> 4) & k7, i1 = x1 & k7, j1 = (x1 >> 4) & k7;
+    w[0] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, i0), __builtin_amdgcn_perm(kIq4T1, kIq4T0, i0), and_or(x0 >> 1, k4, pos)));
+    w[1] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, j0), __builtin_amdgcn_perm(kIq4T1, kIq4T0, j0), and_or(x0 >> 5, k4, pos)));
+    w[2] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, i1), __builtin_amdgcn_perm(kIq4T1, kIq4T0, i1), and_or(x1 >> 1, k4, pos)));
+    w[3] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, j1), __builtin_amdgcn_perm(kIq4T1, kIq4T0, j1), and_or(x1 >> 5, k4, pos)));
+    return w;
+}
+
+constexpr int kStageBytes = 4096;   // codes of one (row tile, super-block) of one bank: 8 sub-blocks x 32 rows x 16 B
+
 // NB banks (gate and up, or one). gateup != 0: out0 is the activation image that receives silu(gate) * up; else out0 /
 // out1 receive the products as rows of `ytype`. wk waves share a row's super-blocks, tpw row tiles per block.
+// Dynamic LDS: waves * NB * kStageBytes of code staging (filled by direct-to-LDS loads, so a wave has all the bytes of
+// its share in flight at once without holding them in registers); the id list and the partial sums reuse that space.
 template <int NB>
 __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * out0, void * out1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_lim, int wk,
                                                     int tpw, int gateup) {
-    __shared__ int list[kMaxList];
+    extern __shared__ __attribute__((aligned(1024))) uint8_t stage[];
     __shared__ int meta[2], s_tok[kTP];
-    __shared__ float red[kMaxWaves][NB][kTP][32];
     __shared__ int ql[kMaxWaves * 2][32];
     const int a = blockIdx.y, e = ids[a];
     if (e < 0 || int64_t(e) * b0.rows >= b0.rows_total) return;   // skipped assignment, or an id outside the bank
     int tok[kTP];
-    const int n_tok = chunk_up(ids, A, a, e, mode, list, meta, tok);
+    const int n_tok = chunk_up(ids, A, a, e, mode, reinterpret_cast<int *>(stage), meta, tok);   // the list lives in the staging space
     if (n_tok == 0) return;
     if (threadIdx.x < kTP) s_tok[threadIdx.x] = tok[threadIdx.x];
     __syncthreads();
@@ -81,57 +101,65 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
     const int row_lim = gateup && shared_slot ? shared_lim : rows;
     const int s_end = !gateup && shared_slot ? shared_lim / 32 : S;
     const bool valid = tile < tiles && tile * 32 < row_lim;
+    uint8_t * my_stage = stage + wave * (NB * kStageBytes);
 
     float accf[NB][2];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) accf[nb][0] = accf[nb][1] = 0.f;
 
     if (valid) {
-        // this lane's part of operand A: plane row n of the MFMA = plane (n & 1) of input row n >> 1
+        // this lane's part of operand A: plane row n of the MFMA = plane (n & 1) of input row n >> 1 (zero past the rows served)
         const int a_tok = n < 2 * kTP ? s_tok[n >> 1] : -1;
-        const uint8_t * a_row = a_tok >= 0 ? image_row_ptr(image, a_tok / xdiv, S) + (n & 1) * 32 + g * 16 : nullptr;
+        const uint8_t * a_row = image_row_ptr(image, max(a_tok, 0) / xdiv, S) + (n & 1) * 32 + g * 16;
         // the two input rows whose sums land in this lane half's result registers
         const int t0 = s_tok[2 * g], t1 = s_tok[2 * g + 1];
-        const float * sc0 = t0 >= 0 ? image_scales(image_row_ptr(image, t0 / xdiv, S), S) : nullptr;
-        const float * sc1 = t1 >= 0 ? image_scales(image_row_ptr(image, t1 / xdiv, S), S) : nullptr;
+        const float * sc0 = image_scales(image_row_ptr(image, max(t0, 0) / xdiv, S), S);
+        const float * sc1 = image_scales(image_row_ptr(image, max(t1, 0) / xdiv, S), S);
         const int64_t tile_g = int64_t(e) * tiles + tile;
-        for (int sb = wk_i; sb < NSB; sb += wk) {
-            v4i areg[8];
-            float xs0[8], xs1[8];
-#pragma unroll
-            for (int ib = 0; ib < 8; ++ib) {
-                const int s = sb * 8 + ib;
-                const bool in = s < s_end;
-                areg[ib] = a_row && in ? *reinterpret_cast<const v4i *>(a_row + int64_t(s) * 64) : v4i{0, 0, 0, 0};
-                xs0[ib] = sc0 && in ? sc0[s] : 0.f;
-                xs1[ib] = sc1 && in ? sc1[s] : 0.f;
-            }
+        const uint32_t pos = 0x03020100u;
+        const int sb_end = s_end / 8;   // whole super-blocks only (the launcher checks)
+        for (int sb = wk_i; sb < sb_end; sb += wk) {
+            // all the code bytes of this wave's share go in flight at once, straight into LDS
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-                const BankView & b = nb ? b1 : b0;
-                const uint2 rec = *reinterpret_cast<const uint2 *>(b.aux + ((tile_g * NSB + sb) * 32 + n) * 8);
-                const float d = half_bits_to_float(uint16_t(rec.x & 0xFFFFu));
-                const uint8_t * cp = b.codes + ((tile_g * S + int64_t(sb) * 8) * 32 + n) * 16 + g * 8;
-                uint2 c[8];
+                const uint8_t * src = (nb ? b1 : b0).codes + (tile_g * S + int64_t(sb) * 8) * 512 + lane * 16;
 #pragma unroll
-                for (int ib = 0; ib < 8; ++ib) c[ib] = *reinterpret_cast<const uint2 *>(cp + ib * 512);
+                for (int c = 0; c < 4; ++c)
+                    __builtin_amdgcn_global_load_lds(src + c * 1024, my_stage + nb * kStageBytes + c * 1024, 16, 0, 0);
+            }
+            uint2 rec[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) rec[nb] = *reinterpret_cast<const uint2 *>((nb ? b1 : b0).aux + ((tile_g * NSB + sb) * 32 + n) * 8);
+            v4i areg[8];
+#pragma unroll
+            for (int ib = 0; ib < 8; ++ib) areg[ib] = a_tok >= 0 ? *reinterpret_cast<const v4i *>(a_row + (sb * 8 + ib) * 64) : v4i{0, 0, 0, 0};
+            // activation scales of the 8 sub-blocks (rows not served read row 0's: their operand A is zero anyway)
+            float xs0[8], xs1[8];
+            {
+                const float4 p0 = *reinterpret_cast<const float4 *>(sc0 + sb * 8), p1 = *reinterpret_cast<const float4 *>(sc0 + sb * 8 + 4);
+                const float4 q0 = *reinterpret_cast<const float4 *>(sc1 + sb * 8), q1 = *reinterpret_cast<const float4 *>(sc1 + sb * 8 + 4);
+                xs0[0] = p0.x; xs0[1] = p0.y; xs0[2] = p0.z; xs0[3] = p0.w; xs0[4] = p1.x; xs0[5] = p1.y; xs0[6] = p1.z; xs0[7] = p1.w;
+                xs1[0] = q0.x; xs1[1] = q0.y; xs1[2] = q0.z; xs1[3] = q0.w; xs1[4] = q1.x; xs1[5] = q1.y; xs1[6] = q1.z; xs1[7] = q1.w;
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const uint8_t * cl = my_stage + nb * kStageBytes + n * 16 + g * 8;
+                const float d = half_bits_to_float(uint16_t(rec[nb].x & 0xFFFFu));
+                const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
                 for (int ib = 0; ib < 8; ++ib) {
-                    v4i bw;
-                    uint32_t lo, hi;
-                    lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(c[ib].x, lo, hi);
-                    bw[0] = int(lo); bw[1] = int(hi);
-                    lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(c[ib].y, lo, hi);
-                    bw[2] = int(lo); bw[3] = int(hi);
-                    v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[ib], bw, acc, 0, 0, 0);
-                    const float ws = d * float(iq4xs_ls(rec, ib) - 32);
+                    const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[ib], decode16(*reinterpret_cast<const uint2 *>(cl + ib * 512), pos), zero, 0, 0, 0);
+                    const float ws = d * float(iq4xs_ls(rec[nb], ib) - 32);
                     accf[nb][0] += float((acc[0] << 7) + acc[1]) * (ws * xs0[ib]);
-                    accf[nb][1] += float((acc[2] << 7) + acc[3]) * (ws * xs1[ib]);
+                    accf[nb][1] += float((acc[2] << 7) + acc[3]) * (ws * xs1[ib]);   // zero when that input row is not served
                 }
             }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the staged bytes are consumed before the next share overwrites them
         }
     }
+    __syncthreads();                                       // staging space is free: it now holds the partial sums
+    float (*red)[NB][kTP][32] = reinterpret_cast<float (*)[NB][kTP][32]>(stage);
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) { red[wave][nb][2 * g][n] = accf[nb][0]; red[wave][nb][2 * g + 1][n] = accf[nb][1]; }
     __syncthreads();
@@ -160,14 +188,18 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
 void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0, void * out1, uint32_t ytype, const int * ids, int A, int xdiv, int mode,
             int slots, int topk, int shared_lim, int gateup, hipStream_t s) {
     const int NSB = b0.cols / 256, tiles = b0.rows / 32;
-    int wk = 1;
-    for (int w = 1; w <= kMaxWaves; ++w) if (NSB % w == 0) wk = w;      // waves that share a row's super-blocks
+    int wk = 1, cap = kMaxWaves;
+    if (const char * v = getenv("TQMOE_WK")) cap = atoi(v) > 0 ? atoi(v) : cap;   // tuning aid
+    for (int w = 1; w <= kMaxWaves && w <= cap; ++w) if (NSB % w == 0) wk = w;      // waves that share a row's super-blocks
     int tpw = kMaxWaves / wk;                                             // row tiles per block
     if (tpw > tiles) tpw = tiles;
     const dim3 grid(unsigned((tiles + tpw - 1) / tpw), unsigned(A));
     const unsigned threads = unsigned(wk * tpw * 64);
-    if (nb == 2) iq4xs_mfma_k<2><<<grid, threads, 0, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
-    else iq4xs_mfma_k<1><<<grid, threads, 0, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
+    // staging for the codes; the same space first holds the id list (kMaxList ints) and last the partial sums
+    size_t lds = size_t(wk * tpw) * nb * kStageBytes;
+    if (lds < size_t(kMaxList) * sizeof(int)) lds = size_t(kMaxList) * sizeof(int);
+    if (nb == 2) iq4xs_mfma_k<2><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
+    else iq4xs_mfma_k<1><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
 }
 
 }  // namespace

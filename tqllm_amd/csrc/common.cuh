@@ -113,6 +113,15 @@ constexpr int kDppXor2 = 0x4E;          // quad_perm [2,3,0,1]
 constexpr int kDppHalfMirror = 0x141;   // lane i <-> 7 - i inside 8
 constexpr int kDppMirror = 0x140;       // lane i <-> 15 - i inside 16
 
+// sum over each row of 16 lanes, in every lane of the row
+__device__ __forceinline__ float row_sum16(float v) {
+    v += dpp_f<kDppXor1>(v);
+    v += dpp_f<kDppXor2>(v);
+    v += dpp_f<kDppHalfMirror>(v);
+    v += dpp_f<kDppMirror>(v);
+    return v;
+}
+
 // all-reduce sum over groups of WIDTH consecutive lanes (WIDTH a power of two, 1..64); every lane gets the total
 template <int WIDTH> __device__ __forceinline__ float group_sum(float v) {
     if constexpr (WIDTH >= 2) v += dpp_f<kDppXor1>(v);

@@ -3,6 +3,8 @@
 
 namespace tqmoe {
 int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);
+int32_t enqueue_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t * ext_ids, int32_t extra, const void * x,
+                     uint32_t xtype, int32_t cols, void * image, int32_t experts, int32_t topk, int32_t n, float scale, hipStream_t s);
 
 namespace {
 
@@ -74,14 +76,13 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
     float * shared_w = reinterpret_cast<float *>(ws + p.shared_w);
 
     if (int32_t rc = tqmoe_router(L.router, L.router_type, L.shared_gate, x, xtype, logits, L.hidden, L.n_expert, n, stream, err)) return rc;
-    if (int32_t rc = tqmoe_topk(logits, ids, weights, shared_w, L.n_expert, L.topk, n, L.weight_scale, stream, err)) return rc;
-    const int32_t * ids_ext = ids;
-    if (L.has_shared) {
-        if (int32_t rc = tqmoe_extend_ids(ids, reinterpret_cast<int32_t *>(ws + p.ids_ext), L.topk, n, L.n_expert, stream, err)) return rc;
-        ids_ext = reinterpret_cast<const int32_t *>(ws + p.ids_ext);
-    }
+    // one launch: softmax top-k, the ids extended by the shared expert, and the input rows' activation image
+    int32_t * ext = L.has_shared ? reinterpret_cast<int32_t *>(ws + p.ids_ext) : nullptr;
+    enqueue_topk(logits, ids, weights, shared_w, ext, L.n_expert, x, xtype, L.hidden, ws + p.ximage, L.n_expert, L.topk, n, L.weight_scale,
+                 static_cast<hipStream_t>(stream));
+    if (int32_t rc = launched(err, "tqmoe_layer_forward (top-k)")) return rc;
+    const int32_t * ids_ext = ext ? ext : ids;
     float * y = reinterpret_cast<float *>(ws + p.y);
-    if (int32_t rc = tqmoe_quant_act(x, xtype, n, L.hidden, ws + p.ximage, stream, err)) return rc;
     if (int32_t rc = tqmoe_expert_gateup(&L.gate, &L.up, ws + p.ximage, ws + p.aimage, ids_ext, n, slots, L.topk, L.shared_ff, stream, err)) return rc;
     if (int32_t rc = tqmoe_expert_down(&L.down, ws + p.aimage, y, ids_ext, n, slots, L.topk, L.shared_ff, stream, err)) return rc;
     return tqmoe_combine_strided(y, slots, L.has_shared ? y + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, weights, shared_w, out, otype,

@@ -1,4 +1,5 @@
 // Router logits, softmax + top-k, and the stable token-to-expert dispatch.
+#include "act_image.cuh"
 #include "common.cuh"
 
 namespace tqmoe {
@@ -55,52 +56,148 @@ template <int WT> int32_t launch_router_x(uint32_t xtype, const void * w, const 
 }
 
 // ------------------------------------------------------------------------------------------------------ top-k
-// One wave per token. Probabilities live in LDS (experts floats); lane l owns entries l, l + 64, ...
-// Selection rule of the reference: larger probability first, equal probabilities to the lower index.
-struct Best { float v; int i; };
-__device__ __forceinline__ Best better(Best a, Best b) { return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a; }
-__device__ __forceinline__ Best wave_best(Best b) {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        Best o;
-        o.v = __shfl_xor(b.v, d, 64);
-        o.i = __shfl_xor(b.i, d, 64);
-        b = better(b, o);
-    }
-    return b;
+// One wave per token. Selection rule of the reference: larger probability first, equal probabilities to the lower
+// index. Up to 1024 experts the probabilities stay in registers (lane l owns entries l, l + 64, ...) and every
+// reduction is a DPP butterfly ending in a scalar broadcast; larger layers keep them in LDS.
+template <int CTRL, int ROWS> __device__ __forceinline__ float dpp_keep_f(float v) {   // lanes outside ROWS get their own value back
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, ROWS, 0xF, false));
+}
+template <int CTRL, int ROWS> __device__ __forceinline__ int dpp_keep_i(int v) { return __builtin_amdgcn_update_dpp(v, v, CTRL, ROWS, 0xF, false); }
+__device__ __forceinline__ float wave_max_all(float v) {   // the wave's maximum, the same in every lane
+    v = fmaxf(v, dpp_f<kDppXor1>(v));
+    v = fmaxf(v, dpp_f<kDppXor2>(v));
+    v = fmaxf(v, dpp_f<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_f<kDppMirror>(v));
+    v = fmaxf(v, dpp_keep_f<0x142, 0xA>(v));   // row_bcast:15 into rows 1 and 3
+    v = fmaxf(v, dpp_keep_f<0x143, 0xC>(v));   // row_bcast:31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+__device__ __forceinline__ int wave_min_all(int v) {
+    v = min(v, dpp_i<kDppXor1>(v));
+    v = min(v, dpp_i<kDppXor2>(v));
+    v = min(v, dpp_i<kDppHalfMirror>(v));
+    v = min(v, dpp_i<kDppMirror>(v));
+    v = min(v, dpp_keep_i<0x142, 0xA>(v));
+    v = min(v, dpp_keep_i<0x143, 0xC>(v));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ __forceinline__ float wave_sum_all(float v) {
+    v = row_sum16(v);
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
-__global__ __launch_bounds__(64) void topk_k(const float * __restrict__ logits, int * __restrict__ ids, float * __restrict__ weights,
-                                             float * __restrict__ shared_weights, int e, int k, float scale) {
+struct TopkOut {
+    int * ids; float * weights; float * shared_weights;
+    int * ext_ids; int extra;          // optional [n][k + 1] copy of the ids with `extra` in the last slot
+    const void * x; uint8_t * image;   // optional: the token's input row is written as an activation image row
+    int cols;
+};
+
+__device__ __forceinline__ void topk_finish(const TopkOut & o, const float * x_logits, int token, int lane, int e, int k, float scale, float selected) {
+    if (lane == 0) {
+        const float total = fmaxf(selected, 6.103515625e-5f);
+        for (int s = 0; s < k; ++s) {   // the host divides by the clamped sum, then multiplies by the scale
+            float v = o.weights[int64_t(token) * k + s] / total;
+            if (scale != 0.f && scale != 1.f) v *= scale;
+            o.weights[int64_t(token) * k + s] = v;
+        }
+        if (o.shared_weights) o.shared_weights[token] = 1.f / (1.f + expf(-x_logits[e]));
+        if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + k] = o.extra;
+    }
+}
+
+template <int XT> __device__ __forceinline__ void topk_quantise_row(const TopkOut & o, int token, int lane) {
+    const int S = o.cols / 32;
+    uint8_t * row = o.image + int64_t(token) * S * kImageSubBytes;
+    for (int s = lane; s < S; s += 64) {
+        float v[32];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float t[8];
+            load8<XT>(o.x, int64_t(token) * o.cols + 32 * s + 8 * c, t);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[8 * c + j] = t[j];
+        }
+        quantise_block(v, row, S, s);
+    }
+}
+
+template <int R, int XT>
+__global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logits, TopkOut o, int e, int k, float scale) {
+    const int token = blockIdx.x, lane = threadIdx.x;
+    const float * x = logits + int64_t(token) * (e + 1);
+    float p[R];
+    float m = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < R; ++r) { const int j = lane + 64 * r; p[r] = j < e ? x[j] : -INFINITY; m = fmaxf(m, p[r]); }
+    m = wave_max_all(m);
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) { const int j = lane + 64 * r; p[r] = j < e ? expf(p[r] - m) : 0.f; sum += p[r]; }
+    sum = wave_sum_all(sum);
+#pragma unroll
+    for (int r = 0; r < R; ++r) p[r] = lane + 64 * r < e ? p[r] / sum : -2.f;   // entries past the end never win
+    float selected = 0.f;
+    for (int s = 0; s < k; ++s) {
+        float bv = p[0];
+        int bi = lane;
+#pragma unroll
+        for (int r = 1; r < R; ++r) if (p[r] > bv) { bv = p[r]; bi = lane + 64 * r; }   // strict: the lowest index of equal values
+        const float top = wave_max_all(bv);
+        const int best = wave_min_all(bv == top ? bi : 0x7FFFFFFF);
+        if (lane == 0) {
+            o.ids[int64_t(token) * k + s] = best;
+            o.weights[int64_t(token) * k + s] = top;
+            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + s] = best;
+        }
+        selected += top;                       // slot order, as the host sums the selected weights
+#pragma unroll
+        for (int r = 0; r < R; ++r) if (lane + 64 * r == best) p[r] = -1.f;
+    }
+    topk_finish(o, x, token, lane, e, k, scale, selected);
+    if (o.image) topk_quantise_row<XT>(o, token, lane);
+}
+
+template <int XT>
+__global__ __launch_bounds__(64) void topk_lds_k(const float * __restrict__ logits, TopkOut o, int e, int k, float scale) {
     extern __shared__ float probs[];
     const int token = blockIdx.x, lane = threadIdx.x;
     const float * x = logits + int64_t(token) * (e + 1);
     float m = -INFINITY;
     for (int j = lane; j < e; j += 64) m = fmaxf(m, x[j]);
-    m = wave_max(m);
+    m = wave_max_all(m);
     float sum = 0.f;
     for (int j = lane; j < e; j += 64) { const float p = expf(x[j] - m); probs[j] = p; sum += p; }
-    sum = group_sum<64>(sum);
+    sum = wave_sum_all(sum);
     for (int j = lane; j < e; j += 64) probs[j] = probs[j] / sum;
-    __syncthreads();
     float selected = 0.f;
     for (int s = 0; s < k; ++s) {
-        Best b{-INFINITY, e};
-        for (int j = lane; j < e; j += 64) b = better(b, Best{probs[j], j});
-        b = wave_best(b);
-        if (lane == 0) { ids[int64_t(token) * k + s] = b.i; weights[int64_t(token) * k + s] = b.v; }
-        selected += b.v;                       // slot order, as the host sums the selected weights
-        if ((b.i & 63) == lane) probs[b.i] = -1.f;
-    }
-    if (lane == 0) {
-        const float total = fmaxf(selected, 6.103515625e-5f);
-        for (int s = 0; s < k; ++s) {
-            float v = weights[int64_t(token) * k + s] / total;
-            if (scale != 0.f && scale != 1.f) v *= scale;
-            weights[int64_t(token) * k + s] = v;
+        float bv = -INFINITY;
+        int bi = 0x7FFFFFFF;
+        for (int j = lane; j < e; j += 64) if (probs[j] > bv) { bv = probs[j]; bi = j; }
+        const float top = wave_max_all(bv);
+        const int best = wave_min_all(bv == top ? bi : 0x7FFFFFFF);
+        if (lane == 0) {
+            o.ids[int64_t(token) * k + s] = best;
+            o.weights[int64_t(token) * k + s] = top;
+            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + s] = best;
         }
-        if (shared_weights) shared_weights[token] = 1.f / (1.f + expf(-x[e]));
+        selected += top;
+        if ((best & 63) == lane) probs[best] = -1.f;
     }
+    topk_finish(o, x, token, lane, e, k, scale, selected);
+    if (o.image) topk_quantise_row<XT>(o, token, lane);
+}
+
+template <int XT> void launch_topk(const float * logits, const TopkOut & o, int e, int k, int n, float scale, hipStream_t s) {
+    if (e <= 64) topk_reg_k<1, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
+    else if (e <= 128) topk_reg_k<2, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
+    else if (e <= 256) topk_reg_k<4, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
+    else if (e <= 512) topk_reg_k<8, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
+    else if (e <= 1024) topk_reg_k<16, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
+    else topk_lds_k<XT><<<unsigned(n), 64, size_t(e) * sizeof(float), s>>>(logits, o, e, k, scale);
 }
 
 // --------------------------------------------------------------------------------------------------- dispatch
@@ -248,13 +345,26 @@ extern "C" int32_t tqmoe_router(const void * router, uint32_t wtype, const void 
     return launched(err, "tqmoe_router");
 }
 
+// top-k with the optional extras of the whole-layer path: extended ids and the input rows' activation image
+namespace tqmoe {
+int32_t enqueue_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t * ext_ids, int32_t extra, const void * x,
+                     uint32_t xtype, int32_t cols, void * image, int32_t experts, int32_t topk, int32_t n, float scale, hipStream_t s) {
+    const TopkOut o{ids, weights, shared_weights, ext_ids, extra, x, static_cast<uint8_t *>(image), cols};
+    switch (image ? xtype : uint32_t(TQMOE_F32)) {
+        case TQMOE_F32: launch_topk<TQMOE_F32>(logits, o, experts, topk, n, scale, s); break;
+        case TQMOE_F16: launch_topk<TQMOE_F16>(logits, o, experts, topk, n, scale, s); break;
+        default: launch_topk<TQMOE_BF16>(logits, o, experts, topk, n, scale, s); break;
+    }
+    return 0;
+}
+}  // namespace tqmoe
+
 extern "C" int32_t tqmoe_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t experts,
                               int32_t topk, int32_t n, float scale, void * stream, tqmoe_error * err) {
     if (!logits || !ids || !weights || experts <= 0 || experts > 4096 || topk <= 0 || topk > experts || n <= 0)
         return fail(err, TQMOE_E_ARG, "tqmoe_topk: invalid shape or pointer");
     if (int32_t rc = need_device(err, "tqmoe_topk")) return rc;
-    topk_k<<<unsigned(n), 64, size_t(experts) * sizeof(float), static_cast<hipStream_t>(stream)>>>(logits, ids, weights, shared_weights,
-                                                                                                  experts, topk, scale);
+    enqueue_topk(logits, ids, weights, shared_weights, nullptr, 0, nullptr, TQMOE_F32, 0, nullptr, experts, topk, n, scale, static_cast<hipStream_t>(stream));
     return launched(err, "tqmoe_topk");
 }
 

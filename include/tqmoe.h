@@ -162,6 +162,35 @@ int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float *
                               const float * weights, const float * shared_weights, void * out, uint32_t otype,
                               int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err);
 
+/* ------------------------------------------------------------------------------------------ prefill products
+ * Grouped int8 x int8 -> int32 products on the matrix cores over the dispatch lists (IQ4_XS banks).
+ *
+ * tqmoe_quant_rows_i8: per input row q = rint(x * 127 / amax), scale = amax / 127 (0 for a zero row): the per-token mode
+ * of the reference's activation quantiser k_quant_act_rows (src/formats/weight/quant_kernels.cuh:17-19, mode 2;
+ * quant_u4h.inc:790-820). q: device int8 [rows][cols] with every 32 values in the bank's byte order (private to the
+ * library: only tqmoe_expert_gemm_* read it); scale: device fp32 [rows]. cols a multiple of 32.
+ * tqmoe_expert_gemm_gateup_i8: act[a] = silu(gate_e x) * (up_e x) as fp16 [n * slots][gate->rows] for every assignment
+ * a = t * slots + s in the lists; input row of a is t. WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59) with
+ * the int8 operands of expert_gemm_i8 (weight_format.hpp:54-56).
+ * tqmoe_expert_gemm_i8: y[a] = W_e x[a] as fp16 [n * slots][bank->rows]; input row of a is a itself
+ * (per_expert_input). WeightFormat::expert_gemm_i8, mode 2 (per-token scales).
+ * counts / offsets / perm: tqmoe_dispatch's lists over ids [n][slots] with `experts` = bank->experts. Assignments of the
+ * bank's last expert use only shared_lim rows (gate / up) or columns (down) when slots > topk (the shared expert);
+ * shared_lim a multiple of 256. Rows of assignments that are in no list stay untouched. */
+int32_t tqmoe_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int32_t cols, int8_t * q, float * scale,
+                            void * stream, tqmoe_error * err);
+int32_t tqmoe_expert_gemm_gateup_i8(const tqmoe_bank * gate, const tqmoe_bank * up, const int8_t * xq, const float * xs,
+                                    const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t n,
+                                    int32_t slots, int32_t topk, int32_t shared_lim, void * act_f16, void * stream,
+                                    tqmoe_error * err);
+int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const int32_t * counts,
+                             const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk,
+                             int32_t shared_lim, void * y_f16, void * stream, tqmoe_error * err);
+/* tqmoe_combine_strided with fp16 rows (the prefill products' output) */
+int32_t tqmoe_combine_strided_f16(const void * routed, int32_t slots, const void * shared, int64_t shared_ld,
+                                  const float * weights, const float * shared_weights, void * out, uint32_t otype,
+                                  int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err);
+
 /* ---------------------------------------------------------------------------------------------- whole layer
  * hidden states + router weights + expert banks in, combined hidden states out: the sequence of
  * Qwen35Engine::ffn_block steps 2-9 (src/models/qwen/qwen35/qwen35_forward.cpp:1123-1248) and of the Flash-Next

@@ -636,12 +636,14 @@ void ffn_mode(const tqo_layer & L, const float * x, const Decoded & d, int ff, f
         for (int i = 0; i < L.hidden; ++i) { g += wg[i] * x[i]; u += wu[i] * x[i]; }
         act[size_t(o)] = (g / (1.f + std::exp(-g))) * u;
     }
+    const bool f16 = L.act_mode == 5;   // the grouped products keep act and y as fp16 rows
+    if (f16) for (float & v : act) v = tqo_half_to_float(tqo_float_to_half(v));
     requant_row_i8(act.data(), ff);
     for (int i = 0; i < L.hidden; ++i) {
         float s = 0.f;
         const float * wd = d.down.data() + size_t(i) * ff;
         for (int o = 0; o < ff; ++o) s += wd[o] * act[size_t(o)];
-        out[i] = s;
+        out[i] = f16 ? tqo_half_to_float(tqo_float_to_half(s)) : s;
     }
 }
 
@@ -653,7 +655,7 @@ int tqo_layer_forward(const tqo_layer * Lp, const float * x, const float * logit
     int elems, bytes;
     if (!tqo_block_layout(L.wtype, &elems, &bytes)) return -1;
     if (L.hidden % elems || L.ff % elems || n <= 0 || L.k <= 0 || L.k > L.n_expert) return -1;
-    if (L.act_mode != 0 && L.act_mode != 1 && L.act_mode != 3) return -1;
+    if (L.act_mode != 0 && L.act_mode != 1 && L.act_mode != 3 && L.act_mode != 5) return -1;
     if (L.has_shared && (L.shared_ff <= 0 || L.shared_ff > L.ff || L.shared_ff % elems)) return -1;
     const int E = L.n_expert, K = L.k, A = n * K, H = L.hidden;
     std::vector<int32_t> ids(static_cast<size_t>(A)), counts(static_cast<size_t>(E)), offsets(size_t(E) + 1), perm(static_cast<size_t>(A));

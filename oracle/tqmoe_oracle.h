@@ -100,7 +100,8 @@ void tqo_quant_act_row_e4m3(const float * x, int cols, uint8_t * q, float * scal
  *   its FFN size shared_ff <= F (the first shared_ff rows / columns), weighted by sigmoid(logits[.][E]).
  *   act_mode: 0 = fp32 activations (oracle A); 1 = gate/up inputs and down inputs per-row int8 (oracle B of the
  *   int8 path); 2 = per-row E4M3 inputs and weights rounded to E4M3 after a power-of-two row scale (oracle B of the
- *   fp8 path); 3 = mode 1 with the weights widened to int8 per (row, 256-weight super-block).
+ *   fp8 path; not implemented); 3 = mode 1 with the weights widened to int8 per (row, 256-weight super-block);
+ *   5 = mode 1 with silu(gate) * up and the down product each rounded to fp16 (what the grouped int8 products store).
  *   out fp32 [n][H]; ids_out [n][k], weights_out [n][k] may be null. threads: worker threads over tokens.
  */
 typedef struct tqo_layer {

@@ -57,13 +57,20 @@ def make_banks(cfg, seed, distinct=None, sigma=0.02):
 
 
 def make_inputs(cfg, n, seed, zipf=None):
-    """router [E][H], shared gate [H], x [n][H] as (storage array, fp32 values). zipf: adds ln p_e of a Zipf(s) popularity
-    over a seeded permutation of the experts to the router logits by scaling nothing: returned as a bias vector."""
+    """router [E][H], shared gate [H], x [n][H] as (storage array, fp32 values).
+    zipf: router logits become N(0, 1) plus a per-expert bias ln p_e of a Zipf(s = zipf) popularity over a seeded
+    permutation of the experts (skewed expert load): router rows are N(0, 1 / H), their last column holds the bias and
+    the last activation of every token is 1."""
     h, e = cfg["hidden"], cfg["experts"]
     rng = np.random.default_rng(seed)
-    router = (rng.standard_normal((e, h)) * 0.02).astype(np.float32)
+    router = (rng.standard_normal((e, h)) * (0.02 if not zipf else h ** -0.5)).astype(np.float32)
     gate = (rng.standard_normal(h) * 0.02).astype(np.float32)
     x = rng.standard_normal((n, h)).astype(np.float32)
+    if zipf:
+        p = 1.0 / np.arange(1, e + 1) ** zipf
+        p /= p.sum()
+        router[:, -1] = np.log(p[rng.permutation(e)])
+        x[:, -1] = 1.0
     out = {}
     for name, a, kind in (("router", router, cfg["rtype"]), ("shared_gate", gate, cfg["rtype"]), ("x", x, cfg["xtype"])):
         if kind == "bf16":
@@ -71,10 +78,6 @@ def make_inputs(cfg, n, seed, zipf=None):
             out[name] = (bits, vals)
         else:
             out[name] = (a, a)
-    if zipf:
-        p = 1.0 / np.arange(1, e + 1) ** zipf
-        p /= p.sum()
-        out["bias"] = np.log(p[rng.permutation(e)]).astype(np.float32)
     return out
 
 

@@ -73,6 +73,10 @@ def lib():
         l.tqmoe_expert_gateup.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, i32, i32, i32, i32, p, e]
         l.tqmoe_expert_down.argtypes = [C.POINTER(_Bank), p, p, p, i32, i32, i32, i32, p, e]
         l.tqmoe_combine_strided.argtypes = [p, i32, p, i64, p, p, p, u32, i32, i32, i32, p, e]
+        l.tqmoe_combine_strided_f16.argtypes = [p, i32, p, i64, p, p, p, u32, i32, i32, i32, p, e]
+        l.tqmoe_quant_rows_i8.argtypes = [p, u32, i64, i32, p, p, p, e]
+        l.tqmoe_expert_gemm_gateup_i8.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
+        l.tqmoe_expert_gemm_i8.argtypes = [C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_swiglu.argtypes = [p, p, p, i64, p, e]
         l.tqmoe_combine.argtypes = [p, p, p, p, p, u32, i32, i32, i32, p, e]
         l.tqmoe_layer_workspace_bytes.restype = sz
@@ -265,9 +269,45 @@ def moe_combine_strided(y, slots, weights, shared_weights=None, out_type=F32, ou
         out = torch.empty((n, hidden), dtype=_OUT_TYPE[out_type], device=y.device)
     shared = y.view(-1)[topk * hidden:] if shared_weights is not None else None
     err = _err()
-    _check(lib().tqmoe_combine_strided(_ptr(y), slots, _ptr(shared), slots * hidden, _ptr(weights), _ptr(shared_weights), _ptr(out), out_type, hidden,
-                                       topk, n, _stream(y), C.byref(err)), err)
+    fn = lib().tqmoe_combine_strided_f16 if y.dtype == torch.float16 else lib().tqmoe_combine_strided
+    _check(fn(_ptr(y), slots, _ptr(shared), slots * hidden, _ptr(weights), _ptr(shared_weights), _ptr(out), out_type, hidden, topk, n, _stream(y),
+              C.byref(err)), err)
     return out
+
+
+def quant_rows_i8(x):
+    """Per-row int8 activations (k_quant_act_rows mode 2, quant_kernels.cuh:17-19): (q int8 [rows][cols] in the library's
+    byte order, scale fp32 [rows])."""
+    rows, cols = x.shape
+    q = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
+    scale = torch.empty(rows, dtype=torch.float32, device=x.device)
+    err = _err()
+    _check(lib().tqmoe_quant_rows_i8(_ptr(x), _ttype(x), rows, cols, _ptr(q), _ptr(scale), _stream(x), C.byref(err)), err)
+    return q, scale
+
+
+def expert_gemm_gateup(gate, up, xq, xs, lists, n, slots, topk, shared_ff=0):
+    """WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59) on int8 rows: fp16 act [n * slots][ff]; rows of
+    assignments that are in no list are zero here (the library leaves them untouched)."""
+    counts, offsets, perm = lists
+    act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=xq.device)
+    err = _err()
+    g, u = gate.view(), up.view()
+    _check(lib().tqmoe_expert_gemm_gateup_i8(C.byref(g), C.byref(u), _ptr(xq), _ptr(xs), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk,
+                                             shared_ff, _ptr(act), _stream(xq), C.byref(err)), err)
+    return act
+
+
+def expert_gemm_i8(bank, xq, xs, lists, n, slots, topk, shared_ff=0):
+    """WeightFormat::expert_gemm_i8 (weight_format.hpp:54-56), per-token scales, one input row per assignment: fp16
+    y [n * slots][rows]."""
+    counts, offsets, perm = lists
+    y = torch.zeros((n * slots, bank.rows), dtype=torch.float16, device=xq.device)
+    err = _err()
+    b = bank.view()
+    _check(lib().tqmoe_expert_gemm_i8(C.byref(b), _ptr(xq), _ptr(xs), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff, _ptr(y),
+                                      _stream(xq), C.byref(err)), err)
+    return y
 
 
 def moe_swiglu(gate, up):

@@ -4,6 +4,11 @@
 
 namespace tqmoe {
 int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);  // bank.hip
+// prefill_iq4xs.hip
+int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, hipStream_t s);
+int32_t enqueue_iq4xs_gemm(int nb, const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
+                           const int * perm, int experts, int64_t assignments, int xdiv, void * out_f16, int gateup, int shared_expert, int shared_lim,
+                           hipStream_t s);
 
 namespace {
 
@@ -13,8 +18,14 @@ __global__ __launch_bounds__(256) void swiglu_k(const float * __restrict__ g, co
 }
 
 // out[t][j] = sum_s weights[t][s] * routed[t][s][j] (s < topk ascending, rows `slots` per token) + shared_w[t] * shared[t][j]
-template <int OT>
-__global__ __launch_bounds__(256) void combine_k(const float * __restrict__ routed, int slots, const float * __restrict__ shared, int64_t shared_ld,
+__device__ __forceinline__ float4 load4(const float * p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ float4 load4(const uint16_t * p) {   // four fp16 values
+    const uint2 v = *reinterpret_cast<const uint2 *>(p);
+    return make_float4(half_bits_to_float(uint16_t(v.x & 0xFFFFu)), half_bits_to_float(uint16_t(v.x >> 16)), half_bits_to_float(uint16_t(v.y & 0xFFFFu)),
+                       half_bits_to_float(uint16_t(v.y >> 16)));
+}
+template <int OT, class RT>
+__global__ __launch_bounds__(256) void combine_k(const RT * __restrict__ routed, int slots, const RT * __restrict__ shared, int64_t shared_ld,
                                                  const float * __restrict__ weights, const float * __restrict__ shared_w, void * __restrict__ out, int h, int k,
                                                  int64_t count) {
     const int64_t i = (int64_t(blockIdx.x) * 256 + threadIdx.x) * 4;   // h is a multiple of 4
@@ -24,12 +35,12 @@ __global__ __launch_bounds__(256) void combine_k(const float * __restrict__ rout
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s = 0; s < k; ++s) {
         const float w = weights[t * k + s];
-        const float4 v = *reinterpret_cast<const float4 *>(routed + (t * slots + s) * h + j);
+        const float4 v = load4(routed + (t * slots + s) * h + j);
         sum.x += w * v.x; sum.y += w * v.y; sum.z += w * v.z; sum.w += w * v.w;
     }
     if (shared) {
         const float w = shared_w[t];
-        const float4 v = *reinterpret_cast<const float4 *>(shared + t * shared_ld + j);
+        const float4 v = load4(shared + t * shared_ld + j);
         sum.x += w * v.x; sum.y += w * v.y; sum.z += w * v.z; sum.w += w * v.w;
     }
     store_out<OT>(out, i, sum.x); store_out<OT>(out, i + 1, sum.y); store_out<OT>(out, i + 2, sum.z); store_out<OT>(out, i + 3, sum.w);
@@ -163,9 +174,9 @@ extern "C" int32_t tqmoe_swiglu(const float * gate, const float * up, float * ac
     return launched(err, "tqmoe_swiglu");
 }
 
-extern "C" int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float * shared, int64_t shared_ld, const float * weights,
-                                         const float * shared_weights, void * out, uint32_t otype, int32_t hidden, int32_t topk, int32_t n, void * stream,
-                                         tqmoe_error * err) {
+template <class RT>
+static int32_t combine_common(const RT * routed, int32_t slots, const RT * shared, int64_t shared_ld, const float * weights, const float * shared_weights,
+                              void * out, uint32_t otype, int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err) {
     if (!routed || !weights || !out || hidden <= 0 || hidden % 4 || topk <= 0 || slots < topk || n <= 0 || (shared && (!shared_weights || shared_ld % 4)))
         return fail(err, TQMOE_E_ARG, "tqmoe_combine: invalid shape or pointer (hidden must be a multiple of 4)");
     if (otype != TQMOE_F32 && otype != TQMOE_BF16) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_combine: output type must be F32 or BF16");
@@ -173,12 +184,68 @@ extern "C" int32_t tqmoe_combine_strided(const float * routed, int32_t slots, co
     const int64_t count = int64_t(n) * hidden;
     const unsigned blocks = unsigned((count / 4 + 255) / 256);
     const hipStream_t s = static_cast<hipStream_t>(stream);
-    if (otype == TQMOE_F32) combine_k<TQMOE_F32><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count);
-    else combine_k<TQMOE_BF16><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count);
+    if (otype == TQMOE_F32) combine_k<TQMOE_F32, RT><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count);
+    else combine_k<TQMOE_BF16, RT><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count);
     return launched(err, "tqmoe_combine");
+}
+
+extern "C" int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float * shared, int64_t shared_ld, const float * weights,
+                                         const float * shared_weights, void * out, uint32_t otype, int32_t hidden, int32_t topk, int32_t n, void * stream,
+                                         tqmoe_error * err) {
+    return combine_common<float>(routed, slots, shared, shared_ld, weights, shared_weights, out, otype, hidden, topk, n, stream, err);
+}
+
+extern "C" int32_t tqmoe_combine_strided_f16(const void * routed, int32_t slots, const void * shared, int64_t shared_ld, const float * weights,
+                                             const float * shared_weights, void * out, uint32_t otype, int32_t hidden, int32_t topk, int32_t n,
+                                             void * stream, tqmoe_error * err) {
+    return combine_common<uint16_t>(static_cast<const uint16_t *>(routed), slots, static_cast<const uint16_t *>(shared), shared_ld, weights, shared_weights, out,
+                                    otype, hidden, topk, n, stream, err);
 }
 
 extern "C" int32_t tqmoe_combine(const float * routed, const float * shared, const float * weights, const float * shared_weights, void * out,
                                  uint32_t otype, int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err) {
     return tqmoe_combine_strided(routed, topk, shared, hidden, weights, shared_weights, out, otype, hidden, topk, n, stream, err);
+}
+
+extern "C" int32_t tqmoe_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int32_t cols, int8_t * q, float * scale, void * stream, tqmoe_error * err) {
+    if (!x || !q || !scale || rows <= 0 || cols <= 0 || cols % 32 || (rows + 3) / 4 > 0x7FFFFFFF) return fail(err, TQMOE_E_ARG, "tqmoe_quant_rows_i8: invalid shape or pointer");
+    if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_quant_rows_i8: unsupported element type");
+    if (int32_t rc = need_device(err, "tqmoe_quant_rows_i8")) return rc;
+    enqueue_quant_rows_i8(x, xtype, rows, cols, q, scale, static_cast<hipStream_t>(stream));
+    return launched(err, "tqmoe_quant_rows_i8");
+}
+
+static int32_t gemm_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
+                           const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
+                           tqmoe_error * err, const char * what) {
+    if (int32_t rc = check_bank(b0, what, err)) return rc;
+    if (b1) {
+        if (int32_t rc = check_bank(b1, what, err)) return rc;
+        if (b1->type != b0->type || b1->rows != b0->rows || b1->cols != b0->cols || b1->experts != b0->experts)
+            return fail(err, TQMOE_E_ARG, "%s: the two banks differ in format or shape", what);
+    }
+    if (b0->type != TQMOE_IQ4_XS) return fail(err, TQMOE_E_UNSUPPORTED, "%s: no int8 grouped product for bank type %u (false in the reference's terms: use the decode products)", what, b0->type);
+    if (!xq || !xs || !counts || !offsets || !perm || !out || n <= 0 || topk <= 0 || slots < topk) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    const int lim_max = gateup ? b0->rows : b0->cols;
+    if (slots > topk && (shared_lim <= 0 || shared_lim > lim_max || shared_lim % 256)) return fail(err, TQMOE_E_ARG, "%s: shared_lim must be a multiple of 256 within the bank", what);
+    if (b0->experts > 4096) return fail(err, TQMOE_E_ARG, "%s: more than 4096 experts", what);
+    if (int32_t rc = need_device(err, what)) return rc;
+    const int shared_expert = slots > topk ? b0->experts - 1 : -1;
+    if (enqueue_iq4xs_gemm(b1 ? 2 : 1, *b0, b1, xq, xs, counts, offsets, perm, b0->experts, int64_t(n) * slots, gateup ? slots : 1, out, gateup, shared_expert,
+                           shared_lim, static_cast<hipStream_t>(stream)))
+        return fail(err, TQMOE_E_ARG, "%s: too many assignments for one call", what);
+    return launched(err, what);
+}
+
+extern "C" int32_t tqmoe_expert_gemm_gateup_i8(const tqmoe_bank * gate, const tqmoe_bank * up, const int8_t * xq, const float * xs, const int32_t * counts,
+                                               const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim,
+                                               void * act_f16, void * stream, tqmoe_error * err) {
+    if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_gemm_gateup_i8: second bank missing");
+    return gemm_common(gate, up, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err, "tqmoe_expert_gemm_gateup_i8");
+}
+
+extern "C" int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
+                                        const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * y_f16, void * stream,
+                                        tqmoe_error * err) {
+    return gemm_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8");
 }

@@ -1,4 +1,6 @@
 // The whole layer behind one entry point: router -> top-k -> activation image -> gate/up + SwiGLU -> down + combine.
+#include <algorithm>
+
 #include "formats.cuh"
 
 namespace tqmoe {
@@ -8,13 +10,29 @@ int32_t enqueue_topk(const float * logits, int32_t * ids, float * weights, float
 
 namespace {
 
+// Token counts from kGroupedMin up take the grouped int8 products (IQ4_XS banks), fewer the decode kernels.
+constexpr int kGroupedMin = 64;
+constexpr int kDecodeAssignments = 65535;   // per decode launch
+
 struct Plan {  // byte offsets into the workspace
-    size_t logits, ids, weights, shared_w, ids_ext, ximage, aimage, y, total;
+    bool grouped;
+    int chunk;   // tokens per pass of the expert stages
+    size_t logits, ids, weights, shared_w, ids_ext, total;
+    size_t ximage, aimage, y;                                                // decode path
+    size_t xq, xs, counts, offsets, perm, dispatch_ws, act16, aq, as, y16;   // grouped path
 };
+
+bool grouped_ok(const tqmoe_layer & L, int n) {
+    return L.gate.type == TQMOE_IQ4_XS && n >= kGroupedMin && (!L.has_shared || L.shared_ff % 256 == 0);
+}
 
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
-    const int slots = L.topk + (L.has_shared ? 1 : 0);
+    const int slots = L.topk + (L.has_shared ? 1 : 0), banks = L.n_expert + (L.has_shared ? 1 : 0);
+    p.grouped = grouped_ok(L, n);
+    // the grouped products take 65535 chunks of 128 assignments a launch, the decode kernels 65535 assignments
+    const int64_t per_pass = p.grouped ? int64_t(65535 - banks) * 128 : kDecodeAssignments;
+    p.chunk = int(std::min<int64_t>(n, std::max<int64_t>(1, per_pass / slots)));
     size_t o = 0;
     auto take = [&](size_t bytes) { const size_t at = o; o = align_up(o + bytes, 256); return at; };
     p.logits = take(size_t(n) * (L.n_expert + 1) * 4);
@@ -22,9 +40,23 @@ Plan plan_for(const tqmoe_layer & L, int n) {
     p.weights = take(size_t(n) * L.topk * 4);
     p.shared_w = take(size_t(n) * 4);
     p.ids_ext = take(size_t(n) * slots * 4);
-    p.ximage = take(tqmoe_act_image_bytes(n, L.hidden));
-    p.aimage = take(tqmoe_act_image_bytes(n * slots, L.ff));
-    p.y = take(size_t(n) * slots * L.hidden * 4);
+    const size_t c = size_t(p.chunk), a = c * slots;
+    if (p.grouped) {
+        p.xq = take(c * L.hidden);
+        p.xs = take(c * 4);
+        p.counts = take(size_t(banks) * 4);
+        p.offsets = take(size_t(banks + 1) * 4);
+        p.perm = take(a * 4);
+        p.dispatch_ws = take(tqmoe_dispatch_workspace_bytes(banks, p.chunk, slots));
+        p.act16 = take(a * L.ff * 2);
+        p.aq = take(a * L.ff);
+        p.as = take(a * 4);
+        p.y16 = take(a * L.hidden * 2);
+    } else {
+        p.ximage = take(tqmoe_act_image_bytes(n, L.hidden));
+        p.aimage = take(tqmoe_act_image_bytes(int32_t(a), L.ff));
+        p.y = take(a * L.hidden * 4);
+    }
     p.total = o;
     return p;
 }
@@ -64,8 +96,7 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
     const tqmoe_layer & L = *layer;
     if (!x || !out || n <= 0) return fail(err, TQMOE_E_ARG, "tqmoe_layer_forward: invalid shape or pointer");
     if (!is_act_type(xtype) || (otype != TQMOE_F32 && otype != TQMOE_BF16)) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_layer_forward: unsupported element type");
-    const int slots = L.topk + (L.has_shared ? 1 : 0);
-    if (int64_t(n) * slots > 65535) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_layer_forward: n * (topk + shared) exceeds 65535 on the decode path");
+    const int slots = L.topk + (L.has_shared ? 1 : 0), banks = L.n_expert + (L.has_shared ? 1 : 0);
     const Plan p = plan_for(L, n);
     if (!workspace || workspace_bytes < p.total) return fail(err, TQMOE_E_WORKSPACE, "tqmoe_layer_forward: workspace of %zu bytes needed", p.total);
     if (int32_t rc = need_device(err, "tqmoe_layer_forward")) return rc;
@@ -74,17 +105,45 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
     int32_t * ids = ids_out ? ids_out : reinterpret_cast<int32_t *>(ws + p.ids);
     float * weights = weights_out ? weights_out : reinterpret_cast<float *>(ws + p.weights);
     float * shared_w = reinterpret_cast<float *>(ws + p.shared_w);
+    const size_t xbytes = elem_bytes(xtype), obytes = elem_bytes(otype);
+    const uint8_t * xb = static_cast<const uint8_t *>(x);
+    uint8_t * ob = static_cast<uint8_t *>(out);
 
     if (int32_t rc = tqmoe_router(L.router, L.router_type, L.shared_gate, x, xtype, logits, L.hidden, L.n_expert, n, stream, err)) return rc;
-    // one launch: softmax top-k, the ids extended by the shared expert, and the input rows' activation image
+    // one launch: softmax top-k, the ids extended by the shared expert, and (decode path) the input rows' activation image
     int32_t * ext = L.has_shared ? reinterpret_cast<int32_t *>(ws + p.ids_ext) : nullptr;
-    enqueue_topk(logits, ids, weights, shared_w, ext, L.n_expert, x, xtype, L.hidden, ws + p.ximage, L.n_expert, L.topk, n, L.weight_scale,
-                 static_cast<hipStream_t>(stream));
+    enqueue_topk(logits, ids, weights, shared_w, ext, L.n_expert, x, xtype, L.hidden, p.grouped ? nullptr : ws + p.ximage, L.n_expert, L.topk, n,
+                 L.weight_scale, static_cast<hipStream_t>(stream));
     if (int32_t rc = launched(err, "tqmoe_layer_forward (top-k)")) return rc;
     const int32_t * ids_ext = ext ? ext : ids;
-    float * y = reinterpret_cast<float *>(ws + p.y);
-    if (int32_t rc = tqmoe_expert_gateup(&L.gate, &L.up, ws + p.ximage, ws + p.aimage, ids_ext, n, slots, L.topk, L.shared_ff, stream, err)) return rc;
-    if (int32_t rc = tqmoe_expert_down(&L.down, ws + p.aimage, y, ids_ext, n, slots, L.topk, L.shared_ff, stream, err)) return rc;
-    return tqmoe_combine_strided(y, slots, L.has_shared ? y + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, weights, shared_w, out, otype,
-                                 L.hidden, L.topk, n, stream, err);
+
+    for (int t0 = 0; t0 < n; t0 += p.chunk) {
+        const int c = std::min(p.chunk, n - t0);
+        const int32_t * cid = ids_ext + size_t(t0) * slots;
+        const float * cw = weights + size_t(t0) * L.topk, * csw = shared_w + t0;
+        void * cout = ob + size_t(t0) * L.hidden * obytes;
+        if (p.grouped) {
+            int8_t * xq = reinterpret_cast<int8_t *>(ws + p.xq), * aq = reinterpret_cast<int8_t *>(ws + p.aq);
+            float * xs = reinterpret_cast<float *>(ws + p.xs), * as = reinterpret_cast<float *>(ws + p.as);
+            int32_t * counts = reinterpret_cast<int32_t *>(ws + p.counts), * offsets = reinterpret_cast<int32_t *>(ws + p.offsets),
+                    * perm = reinterpret_cast<int32_t *>(ws + p.perm);
+            uint16_t * act16 = reinterpret_cast<uint16_t *>(ws + p.act16), * y16 = reinterpret_cast<uint16_t *>(ws + p.y16);
+            if (int32_t rc = tqmoe_quant_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, xq, xs, stream, err)) return rc;
+            if (int32_t rc = tqmoe_dispatch(cid, counts, offsets, perm, nullptr, 0, banks, c, slots, ws + p.dispatch_ws,
+                                            tqmoe_dispatch_workspace_bytes(banks, c, slots), stream, err)) return rc;
+            if (int32_t rc = tqmoe_expert_gemm_gateup_i8(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
+            if (int32_t rc = tqmoe_quant_rows_i8(act16, TQMOE_F16, int64_t(c) * slots, L.ff, aq, as, stream, err)) return rc;
+            if (int32_t rc = tqmoe_expert_gemm_i8(&L.down, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
+            if (int32_t rc = tqmoe_combine_strided_f16(y16, slots, L.has_shared ? y16 + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, cw, csw,
+                                                       cout, otype, L.hidden, L.topk, c, stream, err)) return rc;
+        } else {
+            const uint8_t * ximage = ws + p.ximage + tqmoe_act_image_bytes(1, L.hidden) * size_t(t0);
+            float * y = reinterpret_cast<float *>(ws + p.y);
+            if (int32_t rc = tqmoe_expert_gateup(&L.gate, &L.up, ximage, ws + p.aimage, cid, c, slots, L.topk, L.shared_ff, stream, err)) return rc;
+            if (int32_t rc = tqmoe_expert_down(&L.down, ws + p.aimage, y, cid, c, slots, L.topk, L.shared_ff, stream, err)) return rc;
+            if (int32_t rc = tqmoe_combine_strided(y, slots, L.has_shared ? y + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, cw, csw, cout,
+                                                   otype, L.hidden, L.topk, c, stream, err)) return rc;
+        }
+    }
+    return ok(err);
 }

@@ -74,7 +74,10 @@ int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets,
  * tqmoe_bank_load (the counterpart of WeightFormat::load, weight_format.hpp:41, and of the loaders in
  * src/formats/weight/q4.cpp:295-326, 495-530, 577-606, 802-836). Per 32 weights of a row (a sub-block):
  *   IQ4_XS  codes 16 B: byte j = weights j (low nibble) and j + 16 (high) of the sub-block (GGUF order);
- *           aux 8 B per 256 weights: d (f16), scales_h (u16), scales_l[4].
+ *           aux 8 B per 256 weights: d (f16), scales_h (u16), scales_l[4]. Rows are stored in tiles of 32: the 16 B
+ *           of sub-block s of the 32 rows of a tile are contiguous (512 B), tiles of a row group follow each other by
+ *           sub-block, and the 8 B records likewise (256 B per tile and super-block); rows must be a multiple of 32.
+ *           The other formats are row-major (codes of a row contiguous, then its records).
  *   Q4_K    codes 16 B in the same nibble order; aux 16 B per 256 weights: d, dmin (f16), scales[12] as in GGUF.
  *   IQ3_S   codes 12 B: 8 lattice index bytes then 4 sign bytes; aux 16 B per 256 weights: d (f16), qh[8],
  *           scales[4], 2 B padding.
@@ -108,8 +111,10 @@ int32_t tqmoe_bank_dequant(const tqmoe_bank * bank, int64_t row0, int64_t nrows,
 /* ------------------------------------------------------------------------------------------ decode products
  * Activation image the decode products read: per 32 values a scale s = amax / 16383 and q = rint(x / s) held as
  * two int8 planes (q = 128 * hi + lo, 0 <= lo < 128), so that integer dot products with the integer weight codes
- * reproduce the fp32 product to 2^-15 of the block maximum. One image row is cols * 2 bytes of planes, then
- * (cols / 32) * 8 bytes of (scale, sum of q * s); tqmoe_act_image_bytes gives the size for n rows. */
+ * reproduce the fp32 product to 2^-15 of the block maximum. One image row is cols * 2 bytes of planes (64 B per 32
+ * values: the lo plane then the hi plane, each in the byte order of the banks' code bytes), then cols / 32 fp32 scales,
+ * then cols / 32 fp32 sums of q * s; tqmoe_act_image_bytes gives the size for n rows. The image is private to the
+ * library: only tqmoe_quant_act and tqmoe_expert_gateup write it, only the decode products read it. */
 size_t  tqmoe_act_image_bytes(int32_t n, int32_t cols);
 int32_t tqmoe_quant_act(const void * x, uint32_t xtype, int32_t n, int32_t cols, void * image, void * stream,
                         tqmoe_error * err);

@@ -1,0 +1,144 @@
+// C++ face of the tqmoe C ABI with the names and error behaviour of the reference's own interfaces, header-only.
+//
+//   namespace tqmoe_hip   the free functions of `namespace tqllm_cuda` (src/experts/moe_kernels.cuh:7-81): same names,
+//                         same argument order and meaning; streams are `void *` (a hipStream_t); bad shapes throw
+//                         std::invalid_argument and device failures std::runtime_error, as moe.cu:239, 250-251, 269 do.
+//   tqmoe_hip::ExpertFormat   the expert entry points of `tqllm::WeightFormat` (weight_format.hpp:51-73) over a bank
+//                         view: a `bool false` return means "this format has no such kernel, fall back", as there.
+//
+// Differences a caller has to know, all of them in the element types (the reference's kernels speak fp16 / bf16; this
+// library takes the element type as an argument and keeps intermediate rows in fp32 or in its private activation image):
+// they are spelled out at each function.
+#pragma once
+#include <stdexcept>
+#include <string>
+
+#include "tqmoe.h"
+
+namespace tqmoe_hip {
+
+inline void check(int32_t rc, const tqmoe_error & e) {
+    if (rc == TQMOE_OK) return;
+    const std::string msg = e.message[0] ? e.message : "tqmoe call failed";
+    if (rc == TQMOE_E_ARG || rc == TQMOE_E_UNSUPPORTED || rc == TQMOE_E_WORKSPACE) throw std::invalid_argument(msg);
+    throw std::runtime_error(msg);
+}
+inline tqmoe_error fresh() {
+    tqmoe_error e{};
+    e.struct_size = sizeof(tqmoe_error);
+    return e;
+}
+
+// moe_router / moe_router_f32 (moe_kernels.cuh:7-10): fp32 router rows; x fp16 or fp32. moe_router_bf16 is the Flash-Next
+// form (bf16 router rows, bf16 x; qwen4exp.cu:1629-1659).
+inline void moe_router(const float * router, const float * shared_gate, const void * x_f16, float * logits, int hidden, int experts, int n, void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_router(router, TQMOE_F32, shared_gate, x_f16, TQMOE_F16, logits, hidden, experts, n, stream, &e), e);
+}
+inline void moe_router_f32(const float * router, const float * shared_gate, const float * x, float * logits, int hidden, int experts, int n, void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_router(router, TQMOE_F32, shared_gate, x, TQMOE_F32, logits, hidden, experts, n, stream, &e), e);
+}
+inline void moe_router_bf16(const void * router_bf16, const void * shared_gate_bf16, const void * x_bf16, float * logits, int hidden, int experts, int n,
+                            void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_router(router_bf16, TQMOE_BF16, shared_gate_bf16, x_bf16, TQMOE_BF16, logits, hidden, experts, n, stream, &e), e);
+}
+// moe_topk (moe_kernels.cuh:19-20)
+inline void moe_topk(const float * logits, int * ids, float * weights, float * shared_weights, int experts, int topk, int n, float scale, void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_topk(logits, ids, weights, shared_weights, experts, topk, n, scale, stream, &e), e);
+}
+// moe_group (moe_kernels.cuh:29): groups [experts][n], counts [experts]. The lists are ascending inside each expert
+// (the reference's device version is atomic-ordered). `scratch` holds the offsets, the permutation and the workspace:
+// moe_group_scratch_bytes() device bytes.
+inline size_t moe_group_scratch_bytes(int experts, int n, int topk) {
+    return size_t(experts + 1) * 4 + size_t(n) * topk * 4 + 512 + tqmoe_dispatch_workspace_bytes(experts, n, topk);
+}
+inline void moe_group(const int * ids, int * counts, int * groups, int experts, int n, int topk, void * scratch, void * stream) {
+    tqmoe_error e = fresh();
+    char * p = static_cast<char *>(scratch);
+    int32_t * offsets = reinterpret_cast<int32_t *>(p);
+    size_t at = (size_t(experts + 1) * 4 + 255) / 256 * 256;
+    int32_t * perm = reinterpret_cast<int32_t *>(p + at);
+    at = (at + size_t(n) * topk * 4 + 255) / 256 * 256;
+    check(tqmoe_dispatch(ids, counts, offsets, perm, groups, n, experts, n, topk, p + at, tqmoe_dispatch_workspace_bytes(experts, n, topk), stream, &e), e);
+}
+// moe_swiglu (moe_kernels.cuh:71-72), fp32 in and out here
+inline void moe_swiglu(const float * gate, const float * up, float * act, int count, void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_swiglu(gate, up, act, count, stream, &e), e);
+}
+// moe_sum (moe_kernels.cuh:73-74): routed / shared fp32 here, out bf16 as there
+inline void moe_sum(const float * routed, const float * shared, const float * weights, const float * shared_weights, void * out_bf16, int hidden, int topk, int n,
+                    void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_combine(routed, shared, weights, shared_weights, out_bf16, TQMOE_BF16, hidden, topk, n, stream, &e), e);
+}
+// moe_extend_ids (moe_kernels.cuh:77-78) without the hot / cold slot maps
+inline void moe_extend_ids(const int * ids, int * out, int k, int n, int extra, void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_extend_ids(ids, out, k, n, extra, stream, &e), e);
+}
+// moe_sum_strided (moe_kernels.cuh:80-81)
+inline void moe_sum_strided(const float * routed, int slots, const float * shared, int shared_ld, const float * weights, const float * shared_weights,
+                            void * out_bf16, int hidden, int topk, int n, void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_combine_strided(routed, slots, shared, shared_ld, weights, shared_weights, out_bf16, TQMOE_BF16, hidden, topk, n, stream, &e), e);
+}
+
+// The expert entry points of tqllm::WeightFormat over a bank view (the Mat of stacked experts, weight_format.hpp:22-28, 61).
+struct ExpertFormat {
+    // WeightFormat::load (weight_format.hpp:41): raw GGUF bytes already on the device -> the two planes (caller memory of
+    // tqmoe_bank_layout's sizes). Throws like the loaders do on a rejected row (q4.cpp:519-521) when `status` is read back
+    // by the caller; here only argument errors throw.
+    static tqmoe_bank load(uint32_t type, const void * gguf_blocks_dev, int experts, int rows, int cols, void * codes, void * aux, int32_t * status_dev, void * stream) {
+        tqmoe_error e = fresh();
+        check(tqmoe_bank_load(type, gguf_blocks_dev, int64_t(experts) * rows, cols, codes, aux, status_dev, stream, &e), e);
+        tqmoe_bank b{};
+        b.struct_size = sizeof(tqmoe_bank);
+        b.type = type; b.experts = experts; b.rows = rows; b.cols = cols; b.codes = codes; b.aux = aux;
+        return b;
+    }
+    static bool has_expert_matvec() { return true; }
+    // expert_matvec (weight_format.hpp:62-64): x arrives as the activation image of the input rows (tqmoe_quant_act);
+    // y [n * topk][rows] of ytype (TQMOE_BF16 gives the reference's output type).
+    static void expert_matvec(const tqmoe_bank & m, const void * x_image, void * y, uint32_t ytype, const int * ids, int n, int topk, bool per_expert_input,
+                              void * stream) {
+        tqmoe_error e = fresh();
+        check(tqmoe_expert_matvec(&m, x_image, y, ytype, ids, n, topk, per_expert_input ? 1 : 0, stream, &e), e);
+    }
+    // expert_matvec2 (weight_format.hpp:70-73)
+    static void expert_matvec2(const tqmoe_bank & g, const tqmoe_bank & u, const void * x_image, void * yg, void * yu, uint32_t ytype, const int * ids, int n,
+                               int topk, void * stream) {
+        tqmoe_error e = fresh();
+        check(tqmoe_expert_matvec2(&g, &u, x_image, yg, yu, ytype, ids, n, topk, stream, &e), e);
+    }
+    // expert_gemm_i8 (weight_format.hpp:54-56), mode 2 (one scale per token row), lists as counts / offsets / perm;
+    // false: no grouped int8 kernel for this format.
+    static bool expert_gemm_i8(const tqmoe_bank & m, const int8_t * xq, const float * xs, void * y_f16, const int * counts, const int * offsets, const int * perm,
+                               int n, int topk, void * stream) {
+        tqmoe_error e = fresh();
+        const int32_t rc = tqmoe_expert_gemm_i8(&m, xq, xs, counts, offsets, perm, n, topk, topk, 0, y_f16, stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
+    // expert_gemm_gateup (weight_format.hpp:57-59) on int8 rows; y [assignments][rows] half
+    static bool expert_gemm_gateup(const tqmoe_bank & g, const tqmoe_bank & u, const int8_t * xq, const float * xs, void * y_f16, const int * counts,
+                                   const int * offsets, const int * perm, int n, int topk, void * stream) {
+        tqmoe_error e = fresh();
+        const int32_t rc = tqmoe_expert_gemm_gateup_i8(&g, &u, xq, xs, counts, offsets, perm, n, topk, topk, 0, y_f16, stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
+    // dequant_rows_h (weight_format.hpp:84-86) with fp32 output: the decoded values bit for bit
+    static bool dequant_rows(const tqmoe_bank & m, float * out, int64_t row0, int64_t nrows, void * stream) {
+        tqmoe_error e = fresh();
+        check(tqmoe_bank_dequant(&m, row0, nrows, out, stream, &e), e);
+        return true;
+    }
+};
+
+}  // namespace tqmoe_hip

@@ -169,21 +169,34 @@ int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float *
 
 /* ------------------------------------------------------------------------------------------ prefill products
  * Grouped int8 x int8 -> int32 products on the matrix cores over the dispatch lists (IQ4_XS banks).
+ * counts / offsets / perm are tqmoe_dispatch's lists over ids [n][slots] with `experts` = the banks' experts.
  *
  * tqmoe_quant_rows_i8: per input row q = rint(x * 127 / amax), scale = amax / 127 (0 for a zero row): the per-token mode
  * of the reference's activation quantiser k_quant_act_rows (src/formats/weight/quant_kernels.cuh:17-19, mode 2;
- * quant_u4h.inc:790-820). q: device int8 [rows][cols] with every 32 values in the bank's byte order (private to the
- * library: only tqmoe_expert_gemm_* read it); scale: device fp32 [rows]. cols a multiple of 32.
- * tqmoe_expert_gemm_gateup_i8: act[a] = silu(gate_e x) * (up_e x) as fp16 [n * slots][gate->rows] for every assignment
- * a = t * slots + s in the lists; input row of a is t. WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59) with
- * the int8 operands of expert_gemm_i8 (weight_format.hpp:54-56).
- * tqmoe_expert_gemm_i8: y[a] = W_e x[a] as fp16 [n * slots][bank->rows]; input row of a is a itself
- * (per_expert_input). WeightFormat::expert_gemm_i8, mode 2 (per-token scales).
- * counts / offsets / perm: tqmoe_dispatch's lists over ids [n][slots] with `experts` = bank->experts. Assignments of the
- * bank's last expert use only shared_lim rows (gate / up) or columns (down) when slots > topk (the shared expert);
- * shared_lim a multiple of 256. Rows of assignments that are in no list stay untouched. */
+ * quant_u4h.inc:790-820). q: device int8 [rows][cols], every 32 values in the byte order of the banks' code bytes;
+ * scale: device fp32 [rows]. cols a multiple of 32.
+ * tqmoe_group_rows_i8: the same quantiser applied to the input row (a / xdiv) of every listed assignment a, the rows
+ * gathered expert by expert into tiles of 32 (every expert padded to whole tiles) in the operand order of the matrix
+ * instruction: the form the two products below read. q: device int8 [tqmoe_grouped_rows()][cols], scale: device, 4 bytes
+ * x tqmoe_grouped_scale_words() (the fp32 row scales, then the library's index of the tiles); the layout is private to
+ * the library. xdiv = slots for the layer input (row = token), 1 for
+ * rows that exist per assignment. This is the step the reference does with mmq_quantize_act_rows
+ * (src/experts/mmq_experts.cu:79-95: quantise and arrange the rows of every expert tile).
+ * tqmoe_expert_gemm_gateup_i8: act[a] = silu(gate_e x) * (up_e x) as fp16 [n * slots][gate->rows] for every listed
+ * assignment a = t * slots + s. WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59) with the int8 operands of
+ * expert_gemm_i8 (weight_format.hpp:54-56).
+ * tqmoe_expert_gemm_i8: y[a] = W_e x[a] as fp16 [n * slots][bank->rows]. WeightFormat::expert_gemm_i8, mode 2
+ * (per-token scales). xq / xs: tqmoe_group_rows_i8's outputs for the same lists.
+ * Assignments of the bank's last expert use only shared_lim rows (gate / up; the rest of their act row is zero) or columns
+ * (down) when slots > topk (the shared expert); shared_lim a multiple of 256. Rows of assignments that are in no list
+ * stay untouched. */
 int32_t tqmoe_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int32_t cols, int8_t * q, float * scale,
                             void * stream, tqmoe_error * err);
+int64_t tqmoe_grouped_rows(int64_t assignments, int32_t experts);
+int64_t tqmoe_grouped_scale_words(int64_t assignments, int32_t experts);
+int32_t tqmoe_group_rows_i8(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets,
+                            const int32_t * perm, int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q,
+                            float * scale, void * stream, tqmoe_error * err);
 int32_t tqmoe_expert_gemm_gateup_i8(const tqmoe_bank * gate, const tqmoe_bank * up, const int8_t * xq, const float * xs,
                                     const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t n,
                                     int32_t slots, int32_t topk, int32_t shared_lim, void * act_f16, void * stream,

@@ -30,6 +30,26 @@ def natural_order(q):
     return q.reshape(rows, cols // 32, 8, 4)[:, :, pos, :].reshape(rows, cols)
 
 
+def ungroup(q, scale, counts, perm, assignments):
+    """Grouped operand-major row tiles -> (int8 [assignments][cols] in natural order, scale [assignments]); rows of
+    assignments that are in no list stay zero. A tile is [sub-block][lane half g][row r][16 bytes]; the two 16-byte halves
+    of (row, sub-block) are the 32-byte block that natural_order() understands."""
+    cols = q.shape[1]
+    tiles = q.reshape(-1, cols // 32, 2, 32, 16)
+    rows = tiles.transpose(0, 3, 1, 2, 4).reshape(-1, cols)          # [tile * 32 + r][cols], blocks of 32 bytes
+    rows = natural_order(np.ascontiguousarray(rows))
+    out = np.zeros((assignments, cols), np.int8)
+    out_s = np.zeros(assignments, np.float32)
+    base, at = 0, 0
+    for c in counts:
+        for i in range(c):
+            out[perm[at + i]] = rows[base * 32 + i]
+            out_s[perm[at + i]] = scale[base * 32 + i]
+        at += c
+        base += (c + 31) // 32
+    return out, out_s
+
+
 @pytest.mark.parametrize("kind", ["f32", "bf16", "f16"])
 def test_quant_rows_i8_bit_exact(tq, oracle, kind):
     rng = np.random.default_rng(5)
@@ -67,7 +87,7 @@ def grouped_setup(tq, oracle, seed, experts, ff, hidden, n, k, shared):
     return decs, devb, ids, slots, banks
 
 
-@pytest.mark.parametrize("n,shared_ff", [(3, 0), (70, 256), (300, 512)])
+@pytest.mark.parametrize("n,shared_ff", [(3, 0), (70, 256), (300, 512), (900, 0)])
 def test_grouped_products_against_float64(tq, oracle, n, shared_ff):
     """gate/up + SwiGLU and down products over the dispatch lists against float64 on the decoded weights and the
     dequantised int8 rows (the integer products are exact, so only fp32 accumulation of 256-blocks and the fp16 store
@@ -77,13 +97,18 @@ def test_grouped_products_against_float64(tq, oracle, n, shared_ff):
     rng = np.random.default_rng(n)
     xb, xv = oracle.to_bf16(rng.standard_normal((n, hidden)).astype(np.float32))
     x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
-    xq, xs = tq.quant_rows_i8(x)
     counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), banks)
     want_counts = np.bincount(ids.reshape(-1), minlength=banks)
     assert np.array_equal(counts.cpu().numpy(), want_counts)
     lists = (counts, offsets, perm)
+    xq, xs = tq.group_rows_i8(x, lists, n * slots, slots)
+    # the grouped rows are the plain per-row quantiser's rows, gathered
+    pq, ps = tq.quant_rows_i8(x)
+    uq, us = ungroup(xq.cpu().numpy(), xs.cpu().numpy(), want_counts, perm.cpu().numpy(), n * slots)
+    assert np.array_equal(uq, natural_order(pq.cpu().numpy())[np.arange(n * slots) // slots])
+    assert np.array_equal(us, ps.cpu().numpy()[np.arange(n * slots) // slots])
     act = tq.expert_gemm_gateup(gate, up, xq, xs, lists, n, slots, k, shared_ff)
-    xd = natural_order(xq.cpu().numpy()).astype(np.float64) * xs.cpu().numpy().astype(np.float64)[:, None]
+    xd = natural_order(pq.cpu().numpy()).astype(np.float64) * ps.cpu().numpy().astype(np.float64)[:, None]
     got = act.float().cpu().numpy()
     for a in range(n * slots):
         e = ids.reshape(-1)[a]
@@ -93,9 +118,10 @@ def test_grouped_products_against_float64(tq, oracle, n, shared_ff):
         want = g / (1 + np.exp(-g)) * u
         assert np.abs(got[a, :lim] - want).max() < 2e-3 * max(1.0, np.abs(want).max()), a
         assert not got[a, lim:].any()
-    aq, a_s = tq.quant_rows_i8(act)
+    aq, a_s = tq.group_rows_i8(act, lists, n * slots, 1)
     y = tq.expert_gemm_i8(down, aq, a_s, lists, n, slots, k, shared_ff).float().cpu().numpy()
-    ad = natural_order(aq.cpu().numpy()).astype(np.float64) * a_s.cpu().numpy().astype(np.float64)[:, None]
+    pq, ps = tq.quant_rows_i8(act)
+    ad = natural_order(pq.cpu().numpy()).astype(np.float64) * ps.cpu().numpy().astype(np.float64)[:, None]
     for a in range(n * slots):
         e = ids.reshape(-1)[a]
         lim = shared_ff if (shared_ff and e == experts) else ff
@@ -109,8 +135,8 @@ def test_grouped_products_skip_negative_ids(tq, oracle):
     ids[5, 1] = -1
     ids[17, 0] = -1
     x = torch.randn(n, hidden, device="cuda", dtype=torch.bfloat16)
-    xq, xs = tq.quant_rows_i8(x)
     counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), banks)
+    xq, xs = tq.group_rows_i8(x, (counts, offsets, perm), n * slots, slots)
     act = tq.expert_gemm_gateup(gate, up, xq, xs, (counts, offsets, perm), n, slots, k).cpu().numpy()
     flat = ids.reshape(-1)
     assert not act[flat < 0].any()

@@ -75,6 +75,11 @@ def lib():
         l.tqmoe_combine_strided.argtypes = [p, i32, p, i64, p, p, p, u32, i32, i32, i32, p, e]
         l.tqmoe_combine_strided_f16.argtypes = [p, i32, p, i64, p, p, p, u32, i32, i32, i32, p, e]
         l.tqmoe_quant_rows_i8.argtypes = [p, u32, i64, i32, p, p, p, e]
+        l.tqmoe_grouped_rows.restype = i64
+        l.tqmoe_grouped_rows.argtypes = [i64, i32]
+        l.tqmoe_grouped_scale_words.restype = i64
+        l.tqmoe_grouped_scale_words.argtypes = [i64, i32]
+        l.tqmoe_group_rows_i8.argtypes = [p, u32, i32, p, p, p, i32, i64, i32, p, p, p, e]
         l.tqmoe_expert_gemm_gateup_i8.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_expert_gemm_i8.argtypes = [C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_swiglu.argtypes = [p, p, p, i64, p, e]
@@ -283,6 +288,21 @@ def quant_rows_i8(x):
     scale = torch.empty(rows, dtype=torch.float32, device=x.device)
     err = _err()
     _check(lib().tqmoe_quant_rows_i8(_ptr(x), _ttype(x), rows, cols, _ptr(q), _ptr(scale), _stream(x), C.byref(err)), err)
+    return q, scale
+
+
+def group_rows_i8(x, lists, assignments, xdiv):
+    """Per-row int8 quantisation of the input row (a // xdiv) of every listed assignment a, gathered expert by expert into
+    the operand-major row tiles the grouped products read (mmq_quantize_act_rows, mmq_experts.cu:79-95, in role):
+    (q int8 [grouped rows][cols], scale fp32 [grouped rows]); rows of the padding hold zeros here."""
+    counts, offsets, perm = lists
+    cols = x.shape[1]
+    rows = lib().tqmoe_grouped_rows(assignments, counts.numel())
+    q = torch.zeros((rows, cols), dtype=torch.int8, device=x.device)
+    scale = torch.zeros(lib().tqmoe_grouped_scale_words(assignments, counts.numel()), dtype=torch.float32, device=x.device)
+    err = _err()
+    _check(lib().tqmoe_group_rows_i8(_ptr(x), _ttype(x), cols, _ptr(counts), _ptr(offsets), _ptr(perm), counts.numel(), assignments, xdiv, _ptr(q),
+                                     _ptr(scale), _stream(x), C.byref(err)), err)
     return q, scale
 
 

@@ -6,9 +6,12 @@ namespace tqmoe {
 int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);  // bank.hip
 // prefill_iq4xs.hip
 int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, hipStream_t s);
-int32_t enqueue_iq4xs_gemm(int nb, const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
-                           const int * perm, int experts, int64_t assignments, int xdiv, void * out_f16, int gateup, int shared_expert, int shared_lim,
-                           hipStream_t s);
+int64_t grouped_row_tiles(int64_t assignments, int experts);
+int64_t grouped_scale_words(int64_t assignments, int experts);
+int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
+                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s);
+int32_t enqueue_iq4xs_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
+                           const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s);
 
 namespace {
 
@@ -215,6 +218,25 @@ extern "C" int32_t tqmoe_quant_rows_i8(const void * x, uint32_t xtype, int64_t r
     return launched(err, "tqmoe_quant_rows_i8");
 }
 
+extern "C" int64_t tqmoe_grouped_rows(int64_t assignments, int32_t experts) {
+    return assignments > 0 && experts > 0 ? grouped_row_tiles(assignments, experts) * 32 : 0;
+}
+
+extern "C" int64_t tqmoe_grouped_scale_words(int64_t assignments, int32_t experts) {
+    return assignments > 0 && experts > 0 ? grouped_scale_words(assignments, experts) : 0;
+}
+
+extern "C" int32_t tqmoe_group_rows_i8(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm,
+                                       int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q, float * scale, void * stream, tqmoe_error * err) {
+    if (!x || !counts || !offsets || !perm || !q || !scale || cols <= 0 || cols % 32 || experts <= 0 || experts > 4096 || assignments <= 0 || xdiv <= 0 ||
+        grouped_row_tiles(assignments, experts) > 0x7FFFFFFF)
+        return fail(err, TQMOE_E_ARG, "tqmoe_group_rows_i8: invalid shape or pointer");
+    if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_group_rows_i8: unsupported element type");
+    if (int32_t rc = need_device(err, "tqmoe_group_rows_i8")) return rc;
+    enqueue_group_rows_i8(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, static_cast<hipStream_t>(stream));
+    return launched(err, "tqmoe_group_rows_i8");
+}
+
 static int32_t gemm_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                            const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
                            tqmoe_error * err, const char * what) {
@@ -231,8 +253,8 @@ static int32_t gemm_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const i
     if (b0->experts > 4096) return fail(err, TQMOE_E_ARG, "%s: more than 4096 experts", what);
     if (int32_t rc = need_device(err, what)) return rc;
     const int shared_expert = slots > topk ? b0->experts - 1 : -1;
-    if (enqueue_iq4xs_gemm(b1 ? 2 : 1, *b0, b1, xq, xs, counts, offsets, perm, b0->experts, int64_t(n) * slots, gateup ? slots : 1, out, gateup, shared_expert,
-                           shared_lim, static_cast<hipStream_t>(stream)))
+    if (enqueue_iq4xs_gemm(*b0, b1, xq, xs, counts, offsets, perm, b0->experts, int64_t(n) * slots, out, gateup, shared_expert, shared_lim,
+                           static_cast<hipStream_t>(stream)))
         return fail(err, TQMOE_E_ARG, "%s: too many assignments for one call", what);
     return launched(err, what);
 }

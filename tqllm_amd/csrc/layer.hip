@@ -30,8 +30,9 @@ Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
     const int slots = L.topk + (L.has_shared ? 1 : 0), banks = L.n_expert + (L.has_shared ? 1 : 0);
     p.grouped = grouped_ok(L, n);
-    // the grouped products take 65535 chunks of 128 assignments a launch, the decode kernels 65535 assignments
-    const int64_t per_pass = p.grouped ? int64_t(65535 - banks) * 128 : kDecodeAssignments;
+    // the grouped products take 2^24 assignments a pass (32-bit block and byte counts stay far from their limits), the
+    // decode kernels 65535
+    const int64_t per_pass = p.grouped ? int64_t(1) << 24 : kDecodeAssignments;
     p.chunk = int(std::min<int64_t>(n, std::max<int64_t>(1, per_pass / slots)));
     size_t o = 0;
     auto take = [&](size_t bytes) { const size_t at = o; o = align_up(o + bytes, 256); return at; };
@@ -42,15 +43,17 @@ Plan plan_for(const tqmoe_layer & L, int n) {
     p.ids_ext = take(size_t(n) * slots * 4);
     const size_t c = size_t(p.chunk), a = c * slots;
     if (p.grouped) {
-        p.xq = take(c * L.hidden);
-        p.xs = take(c * 4);
+        const size_t grows = size_t(tqmoe_grouped_rows(int64_t(a), banks));
+        p.xq = take(grows * L.hidden);
+        const size_t gwords = size_t(tqmoe_grouped_scale_words(int64_t(a), banks));
+        p.xs = take(gwords * 4);
         p.counts = take(size_t(banks) * 4);
         p.offsets = take(size_t(banks + 1) * 4);
         p.perm = take(a * 4);
         p.dispatch_ws = take(tqmoe_dispatch_workspace_bytes(banks, p.chunk, slots));
         p.act16 = take(a * L.ff * 2);
-        p.aq = take(a * L.ff);
-        p.as = take(a * 4);
+        p.aq = take(grows * L.ff);
+        p.as = take(gwords * 4);
         p.y16 = take(a * L.hidden * 2);
     } else {
         p.ximage = take(tqmoe_act_image_bytes(n, L.hidden));
@@ -128,11 +131,12 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
             int32_t * counts = reinterpret_cast<int32_t *>(ws + p.counts), * offsets = reinterpret_cast<int32_t *>(ws + p.offsets),
                     * perm = reinterpret_cast<int32_t *>(ws + p.perm);
             uint16_t * act16 = reinterpret_cast<uint16_t *>(ws + p.act16), * y16 = reinterpret_cast<uint16_t *>(ws + p.y16);
-            if (int32_t rc = tqmoe_quant_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, xq, xs, stream, err)) return rc;
             if (int32_t rc = tqmoe_dispatch(cid, counts, offsets, perm, nullptr, 0, banks, c, slots, ws + p.dispatch_ws,
                                             tqmoe_dispatch_workspace_bytes(banks, c, slots), stream, err)) return rc;
+            if (int32_t rc = tqmoe_group_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq,
+                                                 xs, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_gateup_i8(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
-            if (int32_t rc = tqmoe_quant_rows_i8(act16, TQMOE_F16, int64_t(c) * slots, L.ff, aq, as, stream, err)) return rc;
+            if (int32_t rc = tqmoe_group_rows_i8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_i8(&L.down, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
             if (int32_t rc = tqmoe_combine_strided_f16(y16, slots, L.has_shared ? y16 + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, cw, csw,
                                                        cout, otype, L.hidden, L.topk, c, stream, err)) return rc;

@@ -32,6 +32,28 @@ def test_router_logits(tq, oracle, name, n):
     assert np.abs(logits - want).max() < 2e-5
 
 
+@pytest.mark.parametrize("n,e,h,shared", [(32, 512, 2048, True), (100, 33, 512, False), (4096, 512, 2048, True), (77, 64, 192, True)])
+def test_router_gemm_path(tq, oracle, n, e, h, shared):
+    """bf16 router rows and bf16 inputs from 32 tokens up take the matrix-pipe kernel: same logits to the same bar, ragged
+    token and row counts, with and without the shared-gate row; rows of a large batch equal those of a small one."""
+    rng = np.random.default_rng(n + e)
+    wb, wv = oracle.to_bf16((rng.standard_normal((e, h)) * 0.02).astype(np.float32))
+    gb, gv = oracle.to_bf16((rng.standard_normal(h) * 0.02).astype(np.float32))
+    xb, xv = oracle.to_bf16(rng.standard_normal((n, h)).astype(np.float32))
+    x = dev((xb, xv))
+    logits = tq.moe_router(dev((wb, wv)), dev((gb, gv)) if shared else None, x)
+    got = logits.cpu().numpy()
+    exact = xv.astype(np.float64) @ np.vstack([wv, gv if shared else np.zeros_like(gv)]).astype(np.float64).T
+    assert got.shape == (n, e + 1)
+    # fp32 accumulation of up to 2048 exact products: a few ulps of the largest logits (|logit| up to ~5) over 2 million samples
+    assert np.abs(got - exact).max() < 3e-6 * max(1.0, np.abs(exact).max() / 2)
+    if not shared:
+        assert not got[:, e].any()
+    if n >= 45:     # both calls on the matrix-pipe kernel: a row's sum does not depend on the batch around it
+        part = tq.moe_router(dev((wb, wv)), dev((gb, gv)) if shared else None, x[5:5 + 40].contiguous())
+        assert torch.equal(part, logits[5:45])
+
+
 def test_router_without_shared_gate_and_f16(tq, oracle):
     rng = np.random.default_rng(5)
     h, e, n = 512, 33, 7

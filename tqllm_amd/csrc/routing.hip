@@ -55,6 +55,70 @@ template <int WT> int32_t launch_router_x(uint32_t xtype, const void * w, const 
     return -1;
 }
 
+// Router logits of many tokens, bf16 rows on both sides: a GEMM on the matrix pipe. bf16 x bf16 products are exact in
+// fp32 and the matrix instruction accumulates in fp32, so the result differs from the scalar kernel's only by the order
+// of the sum. One wave per 64 tokens x 64 router rows (2 x 2 tiles of v_mfma_f32_32x32x16_bf16); no LDS: the k order
+// inside a 64-wide chunk is free, so lane half g takes columns [32 g, 32 g + 32) of the chunk and a lane reads 64
+// contiguous bytes of its row for four instructions.
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+constexpr int kRouterGemmMin = 32;   // token counts from here up (bf16 router and input) take the GEMM
+
+__global__ __launch_bounds__(256) void router_gemm_bf16_k(const uint16_t * __restrict__ w, const uint16_t * __restrict__ shared, const uint16_t * __restrict__ x,
+                                                            float * __restrict__ logits, int h, int e, int n) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, g = lane >> 5;
+    const int row_tiles = (e + 1 + 63) / 64;
+    const int unit = blockIdx.x * 4 + wave;
+    const int t0 = unit / row_tiles * 64, r0 = unit % row_tiles * 64;
+    if (t0 >= n) return;
+    // operand rows of this lane; rows past the ends repeat a valid row (their results are not stored)
+    const uint16_t * ap[2], * bp[2];
+    bool bzero[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        ap[i] = x + int64_t(min(t0 + 32 * i + r, n - 1)) * h + 32 * g;
+        const int row = min(r0 + 32 * i + r, e);
+        bzero[i] = row == e && shared == nullptr;
+        bp[i] = (row < e ? w + int64_t(row) * h : bzero[i] ? w : shared) + 32 * g;
+    }
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+    for (int k0 = 0; k0 < h; k0 += 64) {
+        v8bf a[2][4], b[2][4];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                a[i][c] = *reinterpret_cast<const v8bf *>(ap[i] + k0 + 8 * c);
+                b[i][c] = *reinterpret_cast<const v8bf *>(bp[i] + k0 + 8 * c);
+            }
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i][c], b[j][c], acc[i][j], 0, 0, 0);
+    }
+    // result register q of lane half g: token row 8 (q / 4) + 4 g + q % 4, router row r
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int row = r0 + 32 * j + r;
+            if (row > e) continue;
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const int t = t0 + 32 * i + 8 * (q >> 2) + 4 * g + (q & 3);
+                if (t < n) logits[int64_t(t) * (e + 1) + row] = bzero[j] ? 0.f : acc[i][j][q];
+            }
+        }
+}
+
 // ------------------------------------------------------------------------------------------------------ top-k
 // One wave per token. Selection rule of the reference: larger probability first, equal probabilities to the lower
 // index. Up to 1024 experts the probabilities stay in registers (lane l owns entries l, l + 64, ...) and every
@@ -340,6 +404,12 @@ extern "C" int32_t tqmoe_router(const void * router, uint32_t wtype, const void 
     if ((n + kRouterTok - 1) / kRouterTok > 65535) return fail(err, TQMOE_E_ARG, "tqmoe_router: too many tokens for one call");
     if (int32_t rc = need_device(err, "tqmoe_router")) return rc;
     const hipStream_t s = static_cast<hipStream_t>(stream);
+    if (wtype == TQMOE_BF16 && xtype == TQMOE_BF16 && n >= kRouterGemmMin && hidden % 64 == 0) {
+        const int64_t units = int64_t((n + 63) / 64) * ((experts + 1 + 63) / 64);
+        router_gemm_bf16_k<<<unsigned((units + 3) / 4), 256, 0, s>>>(static_cast<const uint16_t *>(router), static_cast<const uint16_t *>(shared_gate),
+                                                                      static_cast<const uint16_t *>(x), logits, hidden, experts, n);
+        return launched(err, "tqmoe_router");
+    }
     if (wtype == TQMOE_F32) launch_router_x<TQMOE_F32>(xtype, router, shared_gate, x, logits, hidden, experts, n, s);
     else launch_router_x<TQMOE_BF16>(xtype, router, shared_gate, x, logits, hidden, experts, n, s);
     return launched(err, "tqmoe_router");

@@ -110,7 +110,8 @@ def test_matvec2_swiglu_combine_modular_path(tq, oracle):
     layer = tq.MoeLayer(dev(inp["router"]), dev(inp["shared_gate"]), gate, up, down, cfg["topk"], shared_ff=cfg["shared_ff"])
     fused, fids, fw, flog = layer.forward(x, return_routing=True)
     assert torch.equal(fids, ids) and torch.equal(fw, w) and torch.equal(flog, logits)
-    assert torch.allclose(fused, out, rtol=0, atol=1e-5)
+    # the fused call quantises the intermediate rows per 32 values, the step-by-step one per row: both 2^-14 of a maximum
+    assert torch.allclose(fused, out, rtol=0, atol=5e-5)
     gref = g.double().cpu().numpy()
     want = gref / (1 + np.exp(-gref)) * u.double().cpu().numpy()
     assert np.abs(act.cpu().numpy() - want).max() < 1e-5
@@ -130,7 +131,9 @@ def run_layer(tq, oracle, cfg, n, seed, distinct=None):
 
 
 def check_layer(out, ids, w, want, want_ids, want_w, gaps):
-    assert (gaps > 8).all(), "seed has a near-tied token; pick another"
+    clear = gaps > 8                 # tokens whose k-th and (k+1)-th probabilities are not within a few ulps
+    assert clear.all() if len(gaps) <= 16 else clear.mean() > 0.99, "seed has a near-tied token; pick another"
+    out, ids, w, want, want_ids, want_w = out[clear], ids[clear], w[clear], want[clear], want_ids[clear], want_w[clear]
     assert np.array_equal(ids, want_ids)
     assert np.abs(w - want_w).max() < 3e-6
     mx, rel = synth.errors(out, want)
@@ -163,6 +166,12 @@ def test_layer_config4_and_5_full_shape_one_token(tq, oracle):
     check_layer(*run_layer(tq, oracle, synth.CONFIGS["c5"], 2, seed=500, distinct=4))
 
 
+@pytest.mark.parametrize("n", [64, 512])
+def test_layer_config4_crossover_token_counts(tq, oracle, n):
+    """IQ3_S bank at 64 and 512 tokens (more assignments than the per-expert de-duplication handles at 512)."""
+    check_layer(*run_layer(tq, oracle, synth.CONFIGS["c4"], n, seed=430 + n, distinct=8))
+
+
 def test_layer_linearity_and_bf16_output(tq, oracle):
     """One expert, normalised weight 1: the layer equals that expert's FFN (tests/moe.cpp:354-392); bf16 output is the
     rounded fp32 output."""
@@ -176,6 +185,6 @@ def test_layer_linearity_and_bf16_output(tq, oracle):
     img = tq.quant_act(dev(inp["x"]))
     g, u = tq.expert_matvec2(gate, up, img, ids)
     direct = tq.expert_matvec(down, tq.quant_act(tq.moe_swiglu(g, u)), ids, per_expert_input=True)
-    assert torch.allclose(out, direct, rtol=0, atol=1e-6)
+    assert torch.allclose(out, direct, rtol=0, atol=5e-5)      # intermediate rows quantised per 32 values (fused) or per row (here)
     out16 = layer.forward(dev(inp["x"]), out_type=tq.BF16)
     assert torch.equal(out16, out.to(torch.bfloat16))

@@ -40,11 +40,16 @@ __device__ __forceinline__ void zero_act_block(ActBlock & b) {
     b.sum = 0.f;
 }
 
-// 32 values (natural order) -> sub-block s of an image row
-__device__ __forceinline__ void quantise_block(const float (&v)[32], uint8_t * image_row, int S, int s) {
+__device__ __forceinline__ float block_amax(const float (&v)[32]) {
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    return amax;
+}
+
+// 32 values (natural order) -> sub-block s of an image row, quantised against `amax` (the block's own maximum, or the
+// maximum of a larger set that contains the block: the whole row for the rows tqmoe_quant_act writes)
+__device__ __forceinline__ void quantise_block(const float (&v)[32], uint8_t * image_row, int S, int s, float amax) {
     const float scale = amax * (1.f / 16383.f), inv = amax > 0.f ? 16383.f / amax : 0.f;
     uint32_t hi[8], lo[8];
     int qsum = 0;
@@ -107,22 +112,37 @@ __device__ __forceinline__ void quantise_block_lanes(float v, int i, bool live, 
     }
 }
 
-template <int XT>
-__global__ __launch_bounds__(256) void quant_act_k(const void * __restrict__ x, int n, int cols, uint8_t * __restrict__ image) {
-    const int S = cols / 32;
-    const int64_t idx = int64_t(blockIdx.x) * 256 + threadIdx.x;
-    if (idx >= int64_t(n) * S) return;
-    const int64_t row = idx / S;
-    const int s = int(idx % S);
-    float v[32];
+// One wave per row: the row's maximum first, then every sub-block against it, so that all sub-blocks of a row share one
+// scale (the products can then keep integer sums across sub-blocks and apply the row's scale once).
+template <int XT> __device__ __forceinline__ void load_block32(const void * __restrict__ x, int64_t at, float (&v)[32]) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         float t[8];
-        load8<XT>(x, row * cols + 32 * s + 8 * c, t);
+        load8<XT>(x, at + 8 * c, t);
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[8 * c + j] = t[j];
     }
-    quantise_block(v, image + row * int64_t(S) * kImageSubBytes, S, s);
+}
+template <int XT> __device__ __forceinline__ void quantise_row_wave(const void * __restrict__ x, int64_t row, int cols, uint8_t * image_row, int lane) {
+    const int S = cols / 32;
+    float amax = 0.f;
+    for (int s = lane; s < S; s += 64) {
+        float v[32];
+        load_block32<XT>(x, row * cols + 32 * s, v);
+        amax = fmaxf(amax, block_amax(v));
+    }
+    amax = wave_max(amax);
+    for (int s = lane; s < S; s += 64) {
+        float v[32];
+        load_block32<XT>(x, row * cols + 32 * s, v);
+        quantise_block(v, image_row, S, s, amax);
+    }
+}
+template <int XT>
+__global__ __launch_bounds__(256) void quant_act_k(const void * __restrict__ x, int n, int cols, uint8_t * __restrict__ image) {
+    const int64_t row = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (row >= n) return;
+    quantise_row_wave<XT>(x, row, cols, image + row * int64_t(cols / 32) * kImageSubBytes, threadIdx.x & 63);
 }
 
 }  // namespace

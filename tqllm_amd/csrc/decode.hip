@@ -110,8 +110,7 @@ extern "C" int32_t tqmoe_quant_act(const void * x, uint32_t xtype, int32_t n, in
     if (!x || !image || n <= 0 || cols <= 0 || cols % 32) return fail(err, TQMOE_E_ARG, "tqmoe_quant_act: invalid shape or pointer (cols must be a multiple of 32)");
     if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_quant_act: unsupported element type");
     if (int32_t rc = need_device(err, "tqmoe_quant_act")) return rc;
-    const int64_t subs = int64_t(n) * (cols / 32);
-    const unsigned blocks = unsigned((subs + 255) / 256);
+    const unsigned blocks = unsigned((n + 3) / 4);
     const hipStream_t s = static_cast<hipStream_t>(stream);
     uint8_t * img = static_cast<uint8_t *>(image);
     switch (xtype) {

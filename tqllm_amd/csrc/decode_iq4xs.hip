@@ -9,11 +9,13 @@
 // result registers 0..3 of lane half g are (hi, lo) of input rows 2g and 2g + 1, which one fp32 multiply-add each folds
 // into the lane's running sum with weight scale * activation scale. Waves that split a row's super-blocks add their
 // partial sums through LDS in wave order (deterministic).
+// The weight bytes are the only cold data: every wave streams its share (codes and scale records) straight into its own
+// LDS stage with direct-to-LDS loads, one super-block ahead of the one it is multiplying, so the loads of the next
+// super-block are in flight while this one is decoded.
 #include "act_image.cuh"
 #include "decode_api.cuh"
 #include "formats.cuh"
 
-#include <cstdlib>
 
 namespace tqmoe {
 namespace {
@@ -72,16 +74,22 @@ __device__ __forceinline__ v4i decode16(uint2 c, uint32_t pos) {
     return w;
 }
 
-constexpr int kStageBytes = 4096;   // codes of one (row tile, super-block) of one bank: 8 sub-blocks x 32 rows x 16 B
+constexpr int kCodeBytes = 4096;    // codes of one (row tile, super-block) of one bank: 8 sub-blocks x 32 rows x 16 B
+constexpr int kStageBytes = kCodeBytes + 256;   // then the 32 rows' 8-byte scale records
 
 // NB banks (gate and up, or one). gateup != 0: out0 is the activation image that receives silu(gate) * up; else out0 /
 // out1 receive the products as rows of `ytype`. wk waves share a row's super-blocks, tpw row tiles per block.
-// Dynamic LDS: waves * NB * kStageBytes of code staging (filled by direct-to-LDS loads, so a wave has all the bytes of
-// its share in flight at once without holding them in registers); the id list and the partial sums reuse that space.
-template <int NB>
+// Dynamic LDS: waves * nstage * NB * kStageBytes of staging (filled by direct-to-LDS loads, so a wave has the bytes of
+// a super-block in flight without holding them in registers; nstage = 2 when a wave has more than one super-block); the
+// id list and the partial sums reuse that space.
+// UNI: every sub-block of an input row has the row's one activation scale (the images tqmoe_quant_act and the top-k
+// kernel write). The 6-bit weight scales then multiply the integer results and the sums stay integers over a whole
+// super-block; otherwise (rows quantised block by block, as the fused gate / up epilogue leaves them) each sub-block's
+// result is scaled in fp32.
+template <int NB, bool UNI>
 __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * out0, void * out1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_lim, int wk,
-                                                    int tpw, int gateup) {
+                                                    int tpw, int nstage, int gateup) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t stage[];
     __shared__ int meta[2], s_tok[kTP];
     __shared__ int ql[kMaxWaves * 2][32];
@@ -101,7 +109,7 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
     const int row_lim = gateup && shared_slot ? shared_lim : rows;
     const int s_end = !gateup && shared_slot ? shared_lim / 32 : S;
     const bool valid = tile < tiles && tile * 32 < row_lim;
-    uint8_t * my_stage = stage + wave * (NB * kStageBytes);
+    uint8_t * my_stage = stage + wave * (nstage * NB * kStageBytes);
 
     float accf[NB][2];
 #pragma unroll
@@ -118,44 +126,78 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
         const int64_t tile_g = int64_t(e) * tiles + tile;
         const uint32_t pos = 0x03020100u;
         const int sb_end = s_end / 8;   // whole super-blocks only (the launcher checks)
-        for (int sb = wk_i; sb < sb_end; sb += wk) {
-            // all the code bytes of this wave's share go in flight at once, straight into LDS
+        // a super-block's cold bytes (codes, records) go in flight at once, straight into the wave's stage `slot`
+        auto issue = [&](int sb, int slot) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
+                uint8_t * dst = my_stage + (slot * NB + nb) * kStageBytes;
                 const uint8_t * src = (nb ? b1 : b0).codes + (tile_g * S + int64_t(sb) * 8) * 512 + lane * 16;
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    __builtin_amdgcn_global_load_lds(src + c * 1024, my_stage + nb * kStageBytes + c * 1024, 16, 0, 0);
+                for (int c = 0; c < 4; ++c) __builtin_amdgcn_global_load_lds(src + c * 1024, dst + c * 1024, 16, 0, 0);
+                if (lane < 16) __builtin_amdgcn_global_load_lds((nb ? b1 : b0).aux + (tile_g * NSB + sb) * 256 + lane * 16, dst + kCodeBytes, 16, 0, 0);
             }
-            uint2 rec[NB];
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) rec[nb] = *reinterpret_cast<const uint2 *>((nb ? b1 : b0).aux + ((tile_g * NSB + sb) * 32 + n) * 8);
+        };
+        if (wk_i < sb_end) issue(wk_i, 0);
+        int slot = 0;
+        for (int sb = wk_i; sb < sb_end; sb += wk) {
+            const bool more = sb + wk < sb_end;
+            // the activation side of this super-block (warm data), then the next super-block's cold bytes: those stay the
+            // youngest loads, so the wait below can leave exactly them in flight
             v4i areg[8];
 #pragma unroll
             for (int ib = 0; ib < 8; ++ib) areg[ib] = a_tok >= 0 ? *reinterpret_cast<const v4i *>(a_row + (sb * 8 + ib) * 64) : v4i{0, 0, 0, 0};
             // activation scales of the 8 sub-blocks (rows not served read row 0's: their operand A is zero anyway)
             float xs0[8], xs1[8];
-            {
+            if constexpr (!UNI) {
                 const float4 p0 = *reinterpret_cast<const float4 *>(sc0 + sb * 8), p1 = *reinterpret_cast<const float4 *>(sc0 + sb * 8 + 4);
                 const float4 q0 = *reinterpret_cast<const float4 *>(sc1 + sb * 8), q1 = *reinterpret_cast<const float4 *>(sc1 + sb * 8 + 4);
                 xs0[0] = p0.x; xs0[1] = p0.y; xs0[2] = p0.z; xs0[3] = p0.w; xs0[4] = p1.x; xs0[5] = p1.y; xs0[6] = p1.z; xs0[7] = p1.w;
                 xs1[0] = q0.x; xs1[1] = q0.y; xs1[2] = q0.z; xs1[3] = q0.w; xs1[4] = q1.x; xs1[5] = q1.y; xs1[6] = q1.z; xs1[7] = q1.w;
             }
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (more) issue(sb + wk, slot ^ 1);
+            // everything but the next super-block's loads (5 per bank, the youngest) has arrived
+            if (more) {
+                if (NB == 2) asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-                const uint8_t * cl = my_stage + nb * kStageBytes + n * 16 + g * 8;
-                const float d = half_bits_to_float(uint16_t(rec[nb].x & 0xFFFFu));
+                const uint8_t * st = my_stage + (slot * NB + nb) * kStageBytes;
+                const uint8_t * cl = st + n * 16 + g * 8;
+                const uint2 rec = *reinterpret_cast<const uint2 *>(st + kCodeBytes + n * 8);
+                const float d = half_bits_to_float(uint16_t(rec.x & 0xFFFFu));
                 const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                int si[4] = {0, 0, 0, 0};   // (hi, lo) plane sums of the two input rows, weighted by the sub-block scales
 #pragma unroll
                 for (int ib = 0; ib < 8; ++ib) {
                     const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[ib], decode16(*reinterpret_cast<const uint2 *>(cl + ib * 512), pos), zero, 0, 0, 0);
-                    const float ws = d * float(iq4xs_ls(rec[nb], ib) - 32);
-                    accf[nb][0] += float((acc[0] << 7) + acc[1]) * (ws * xs0[ib]);
-                    accf[nb][1] += float((acc[2] << 7) + acc[3]) * (ws * xs1[ib]);   // zero when that input row is not served
+                    if constexpr (UNI) {
+                        // |acc| <= 32 * 128 * 127 < 2^19 and |ls - 32| <= 32: 24-bit products, eight of them stay below 2^28
+                        const int ls = iq4xs_ls(rec, ib) - 32;
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) si[q] += __mul24(acc[q], ls);
+                    } else {
+                        const float ws = d * float(iq4xs_ls(rec, ib) - 32);
+                        accf[nb][0] += float((acc[0] << 7) + acc[1]) * (ws * xs0[ib]);
+                        accf[nb][1] += float((acc[2] << 7) + acc[3]) * (ws * xs1[ib]);   // zero when that input row is not served
+                    }
+                }
+                if constexpr (UNI) {
+                    accf[nb][0] += (float(si[0]) * 128.f + float(si[1])) * d;
+                    accf[nb][1] += (float(si[2]) * 128.f + float(si[3])) * d;
                 }
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the staged bytes are consumed before the next share overwrites them
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the staged bytes are consumed before a later share overwrites them
+            slot ^= 1;
+        }
+    }
+    if constexpr (UNI) {
+        if (valid) {   // the rows' own scales, once
+            const int t0 = s_tok[2 * g], t1 = s_tok[2 * g + 1];
+            const float x0 = image_scales(image_row_ptr(image, max(t0, 0) / xdiv, S), S)[0], x1 = image_scales(image_row_ptr(image, max(t1, 0) / xdiv, S), S)[0];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) { accf[nb][0] *= x0; accf[nb][1] *= x1; }
         }
     }
     __syncthreads();                                       // staging space is free: it now holds the partial sums
@@ -186,29 +228,43 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
 }
 
 void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0, void * out1, uint32_t ytype, const int * ids, int A, int xdiv, int mode,
-            int slots, int topk, int shared_lim, int gateup, hipStream_t s) {
+            int slots, int topk, int shared_lim, int gateup, bool uniform, hipStream_t s) {
     const int NSB = b0.cols / 256, tiles = b0.rows / 32;
-    int wk = 1, cap = kMaxWaves;
-    if (const char * v = getenv("TQMOE_WK")) cap = atoi(v) > 0 ? atoi(v) : cap;   // tuning aid
-    for (int w = 1; w <= kMaxWaves && w <= cap; ++w) if (NSB % w == 0) wk = w;      // waves that share a row's super-blocks
-    int tpw = kMaxWaves / wk;                                             // row tiles per block
+    // Waves that share a row's super-blocks: as many as it takes to put a few thousand waves in flight (a short batch
+    // is bound by the latency of one wave's chain), fewer when the batch has the waves anyway (a longer chain per
+    // wave streams with its loads one super-block ahead and saves the cross-wave sums).
+    const int64_t units = int64_t(A) * tiles;
+    const int cap = units >= 8192 ? 1 : units >= 2048 ? 2 : kMaxWaves;   // (4 shares with two stages each would leave one block per compute unit)
+    int wk = 1;
+    for (int w = 1; w <= kMaxWaves && w <= cap; ++w) if (NSB % w == 0) wk = w;
+    const int waves = wk >= 4 ? kMaxWaves : 4;                            // per block
+    int tpw = waves / wk;                                                 // row tiles per block
     if (tpw > tiles) tpw = tiles;
+    const int nstage = NSB / wk > 1 ? 2 : 1;
     const dim3 grid(unsigned((tiles + tpw - 1) / tpw), unsigned(A));
     const unsigned threads = unsigned(wk * tpw * 64);
     // staging for the codes; the same space first holds the id list (kMaxList ints) and last the partial sums
-    size_t lds = size_t(wk * tpw) * nb * kStageBytes;
+    size_t lds = size_t(wk * tpw) * nstage * nb * kStageBytes;
     if (lds < size_t(kMaxList) * sizeof(int)) lds = size_t(kMaxList) * sizeof(int);
-    if (nb == 2) iq4xs_mfma_k<2><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
-    else iq4xs_mfma_k<1><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
+    if (lds < size_t(wk * tpw) * nb * kTP * 32 * sizeof(float)) lds = size_t(wk * tpw) * nb * kTP * 32 * sizeof(float);
+    if (lds > 65536) {
+        static const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void *>(&iq4xs_mfma_k<2, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
+        static const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(&iq4xs_mfma_k<1, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
+        static const hipError_t e3 = hipFuncSetAttribute(reinterpret_cast<const void *>(&iq4xs_mfma_k<2, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
+        (void)e1; (void)e2; (void)e3;
+    }
+    if (nb == 2 && uniform) iq4xs_mfma_k<2, true><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, nstage, gateup);
+    else if (nb == 2) iq4xs_mfma_k<2, false><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, nstage, gateup);
+    else iq4xs_mfma_k<1, false><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, nstage, gateup);
 }
 
 }  // namespace
 
 template <> void DecodeLaunch<TQMOE_IQ4_XS>::matvec(Split, int nb, const MatvecArgs & k, hipStream_t s) {
-    launch(nb, k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols, 0, s);
+    launch(nb, k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols, 0, false, s);
 }
 template <> void DecodeLaunch<TQMOE_IQ4_XS>::gateup(Split, const GateupArgs & k, hipStream_t s) {
-    launch(2, k.bg, k.bu, k.ximage, k.aimage, nullptr, TQMOE_F32, k.ids, k.A, k.slots, k.mode, k.slots, k.topk, k.shared_ff, 1, s);
+    launch(2, k.bg, k.bu, k.ximage, k.aimage, nullptr, TQMOE_F32, k.ids, k.A, k.slots, k.mode, k.slots, k.topk, k.shared_ff, 1, true, s);
 }
 
 }  // namespace tqmoe

@@ -173,19 +173,7 @@ __device__ __forceinline__ void topk_finish(const TopkOut & o, const float * x_l
 }
 
 template <int XT> __device__ __forceinline__ void topk_quantise_row(const TopkOut & o, int token, int lane) {
-    const int S = o.cols / 32;
-    uint8_t * row = o.image + int64_t(token) * S * kImageSubBytes;
-    for (int s = lane; s < S; s += 64) {
-        float v[32];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            float t[8];
-            load8<XT>(o.x, int64_t(token) * o.cols + 32 * s + 8 * c, t);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) v[8 * c + j] = t[j];
-        }
-        quantise_block(v, row, S, s);
-    }
+    quantise_row_wave<XT>(o.x, token, o.cols, o.image + int64_t(token) * (o.cols / 32) * kImageSubBytes, lane);
 }
 
 template <int R, int XT>

@@ -21,6 +21,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")   # measured with rocprofv3 --pmc (see the file)
 HBM_PEAK = 8.0e12  # bytes/s, MI355X published
 INT8_PEAK = 5.0e15  # dense int8 operations/s, MI355X published
 PREFILL_MIN = 64   # token counts from here up take the grouped int8 products inside the library
@@ -118,6 +119,8 @@ def main():
     ap.add_argument("--banks", type=int, default=8, help="independent expert banks the steps rotate over")
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-mb", type=int, default=0, help="also run one plain device copy of this many MiB (a kernel of known "
+                    "traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this command)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing here uses a second GPU)" % args.gpus)
@@ -129,6 +132,12 @@ def main():
         sys.exit("bench.py: no GPU visible; the library has no CPU path")
     torch.cuda.set_device(0)
     T, R = args.tokens, args.banks
+    if args.copy_mb > 0:
+        src = torch.empty(args.copy_mb << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if args.steps is None:
         args.steps = 400 if T < PREFILL_MIN else 80
     if args.warmup is None:
@@ -253,6 +262,13 @@ def main():
                  "down_us": round(kernels["down"] * 1e3, 2), "down_hbm_frac": round(dn_bytes / (kernels["down"] * 1e-3) / HBM_PEAK, 4)}
         workload = "config 2: Flash-Next-shaped decode layer, hidden 2048, 512 IQ4_XS experts top-10 + shared (ff 512), T=%d" % T
         dtype = "int8 x int8 -> int32 MFMA, fp32 scales (IQ4_XS weights exact, bf16 activations as 2 x int8 planes)"
+
+    # HBM bytes per launch of the roofline kernel as the counters saw them (a committed measurement of this same command)
+    try:
+        with open(TRAFFIC_FILE) as f:
+            roofline["traffic"] = json.load(f).get("tokens_%d" % T, {}).get("bytes_per_launch")
+    except (OSError, ValueError):
+        pass
 
     line = {
         "metric": "MoE-layer tokens/s", "value": round(T / (ms_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,

@@ -196,17 +196,22 @@ __device__ __forceinline__ void decode_planes(uint2 c, uint4 th, uint4 tl, v4i &
 
 __device__ const int8_t kIq4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
-// dynamic LDS: [2 stages][NB][plane h, l][8 sub-blocks][64 lanes] v4i of decoded weights
+// dynamic LDS: [2 stages][NB][plane h, l][8 sub-blocks][64 lanes] v4i of decoded weights.
+// 4 * NB waves: wave = 4 * slot + row group; a wave multiplies its kMT row tiles with the weights of its operand slot
+// (gate or up; for down the two row tiles of the unit), so that two waves share a SIMD and one's vector work and loads
+// overlap the other's products.
 template <int NB>
-__global__ __launch_bounds__(256) void iq4xs_gemm_k(GemmArgs k) {
+__global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
+    constexpr int THREADS = 256 * NB;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     v4i * bs = reinterpret_cast<v4i *>(lds);
     __shared__ __attribute__((aligned(16))) uint8_t s_tab[64 * 32];   // per 6-bit scale: 16 h bytes, 16 l bytes
     __shared__ int s_asg[kChunkTiles * 32];
     __shared__ float s_scale[kChunkTiles * 32];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
+    const int mg = wave & 3, nbw = wave >> 2;     // row group, operand slot
 
-    for (int i = tid; i < 64 * 16; i += 256) {
+    for (int i = tid; i < 64 * 16; i += THREADS) {
         const int v = int(kIq4Values[i & 15]) * ((i >> 4) - 32);
         const int lo = ((v + 32) & 63) - 32, hi = (v - lo) >> 6;
         s_tab[(i >> 4) * 32 + (i & 15)] = uint8_t(hi);
@@ -215,172 +220,160 @@ __global__ __launch_bounds__(256) void iq4xs_gemm_k(GemmArgs k) {
     // Work items are (chunk of row tiles, unit of weight rows); the blocks of the grid walk them with the grid as stride.
     // Items that share operand A (one chunk, all units) have indices that agree modulo 8, so that with the round-robin of
     // blocks over the 8 XCDs (grid a multiple of 8) one XCD's L2 serves them.
-    const int items = k.plan.chunk_base[k.experts] * k.units;
-    const int items_padded = (k.plan.chunk_base[k.experts] + 7) / 8 * 8 * k.units;
-    for (int item = int(blockIdx.x); item < items_padded; item += int(gridDim.x)) {
-    const int unit = (item >> 3) % k.units, chunk = item / (8 * k.units) * 8 + (item & 7);
-    if (chunk >= k.plan.chunk_base[k.experts]) continue;
-    const int e = owner_of(k.plan.chunk_base, k.experts, chunk);
-    const Where w{e, chunk - k.plan.chunk_base[e], k.plan.tile_base[e]};
-    (void)items;
-    __syncthreads();          // the previous item's epilogue has read s_asg / s_scale
+    const int n_chunks = k.plan.chunk_base[k.experts];
+    const int items_padded = (n_chunks + 7) / 8 * 8 * k.units;
     const int S = k.b0.cols / 32, NSB = S / 8, rows = k.b0.rows, tiles_w = rows / 32;
-    const bool is_shared = e == k.shared_expert;
-    // gate / up rows of the shared expert beyond its size: no products, zeros stored (the rows are quantised whole later)
-    const bool dead = k.gateup && is_shared && unit * 32 >= k.shared_lim;
-    const int sb_end = dead ? 0 : !k.gateup && is_shared ? k.shared_lim / 256 : NSB;
-    const int cnt = k.counts[e], tiles_e = (cnt + 31) >> 5;
-    const int first_tile = w.local * kChunkTiles;                       // of this expert
-    const int live_tiles = min(kChunkTiles, tiles_e - first_tile);      // of this block
-    for (int i = tid; i < kChunkTiles * 32; i += 256) {
-        const int idx = first_tile * 32 + i;
-        const bool ok = i < live_tiles * 32 && idx < cnt;
-        s_asg[i] = ok ? k.perm[k.offsets[e] + idx] : -1;
-        s_scale[i] = ok ? k.xs[int64_t(w.tile_base + first_tile) * 32 + i] : 0.f;
-    }
-    __syncthreads();
-
-    const int my_tiles = max(0, min(kMT, live_tiles - wave * kMT));     // row tiles of this wave
-    const int8_t * a_base = k.xq + int64_t(w.tile_base + first_tile + wave * kMT) * 32 * k.b0.cols + lane * 16;
-    const int64_t a_tile = int64_t(32) * k.b0.cols;
-
-    // weight rows of operand slot nb: gate / up: the unit's 32 rows of bank nb; down: row tile NB * unit + nb of the bank
-    const uint8_t * codes[NB], * aux[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const BankView & b = nb ? k.b1 : k.b0;
-        const int64_t tile_g = int64_t(e) * tiles_w + (k.gateup ? unit : NB * unit + nb);
-        codes[nb] = b.codes + tile_g * S * 512 + n * 16 + (lane >> 5) * 8;   // sub-block s of the tile: + 512 s; lane = (row n, code half g)
-        aux[nb] = b.aux + tile_g * NSB * 256 + n * 8;            // super-block sb of the tile: + 256 sb
-    }
-
-    // The super-block loop is instantiated per number of live row tiles of the wave (0..kMT), so that its body is one
-    // straight line of code the scheduler can interleave: products, operand loads and the decode of the next stage.
-    // Every instance passes the same barriers.
-    auto body = [&](auto mt_tag) {
-        constexpr int MT = decltype(mt_tag)::value;
-        constexpr int MTA = MT ? MT : 1;
-        v16i acc_h[MTA][NB], acc_l[MTA][NB];
-        float acc_f[MTA][NB][16];
-#pragma unroll
-        for (int t = 0; t < MTA; ++t)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) { acc_f[t][nb][i] = 0.f; acc_h[t][nb][i] = 0; acc_l[t][nb][i] = 0; }
-
-        // this wave decodes sub-blocks 2 wave and 2 wave + 1 of every super-block, for each operand slot: the codes and
-        // the scale record are fetched one super-block before they are decoded, so that their latency is not waited for
-        float d_next[NB], d_cur[NB];
-        uint2 f_rec[NB], f_code[NB][2];
-        auto fetch = [&](int sb) {
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                f_rec[nb] = *reinterpret_cast<const uint2 *>(aux[nb] + int64_t(sb) * 256);
-#pragma unroll
-                for (int j = 0; j < 2; ++j) f_code[nb][j] = *reinterpret_cast<const uint2 *>(codes[nb] + (int64_t(sb) * 8 + 2 * wave + j) * 512);
-            }
-        };
-        auto decode_into = [&](int buf) {
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                d_next[nb] = half_bits_to_float(uint16_t(f_rec[nb].x & 0xFFFFu));
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int ib = 2 * wave + j;
-                    const uint4 * tab = reinterpret_cast<const uint4 *>(s_tab + iq4xs_ls(f_rec[nb], ib) * 32);
-                    v4i h, l;
-                    decode_planes(f_code[nb][j], tab[0], tab[1], h, l);
-                    bs[(((buf * NB + nb) * 2 + 0) * 8 + ib) * 64 + lane] = h;
-                    bs[(((buf * NB + nb) * 2 + 1) * 8 + ib) * 64 + lane] = l;
-                }
-            }
-        };
-        // operand A, two k-steps (sub-blocks) per slot, fetched three slots (six k-steps) before its products
-        v4i a_reg[4][MTA][2];
-        auto load_a = [&](int slot, int pair) {
-#pragma unroll
-            for (int t = 0; t < MT; ++t)
-#pragma unroll
-                for (int h = 0; h < 2; ++h) a_reg[slot][t][h] = *reinterpret_cast<const v4i *>(a_base + t * a_tile + (int64_t(pair) * 2 + h) * 1024);
-        };
-
-        if (sb_end > 0) {
-            fetch(0);
-            const int last = sb_end * 4 - 1;
-            load_a(0, 0);
-            load_a(1, min(1, last));
-            load_a(2, min(2, last));
-            decode_into(0);
-            fetch(min(1, sb_end - 1));
+    for (int item = int(blockIdx.x); item < items_padded; item += int(gridDim.x)) {
+        const int unit = (item >> 3) % k.units, chunk = item / (8 * k.units) * 8 + (item & 7);
+        if (chunk >= n_chunks) continue;
+        const int e = owner_of(k.plan.chunk_base, k.experts, chunk);
+        const int local = chunk - k.plan.chunk_base[e], tile_base = k.plan.tile_base[e];
+        __syncthreads();          // the previous item's epilogue has read s_asg / s_scale and the exchange space
+        const bool is_shared = e == k.shared_expert;
+        // gate / up rows of the shared expert beyond its size: no products, zeros stored (the rows are quantised whole later)
+        const bool dead = k.gateup && is_shared && unit * 32 >= k.shared_lim;
+        const int sb_end = dead ? 0 : !k.gateup && is_shared ? k.shared_lim / 256 : NSB;
+        const int cnt = k.counts[e], tiles_e = (cnt + 31) >> 5;
+        const int first_tile = local * kChunkTiles;                         // of this expert
+        const int live_tiles = min(kChunkTiles, tiles_e - first_tile);      // of this block
+        for (int i = tid; i < kChunkTiles * 32; i += THREADS) {
+            const int idx = first_tile * 32 + i;
+            const bool ok = i < live_tiles * 32 && idx < cnt;
+            s_asg[i] = ok ? k.perm[k.offsets[e] + idx] : -1;
+            s_scale[i] = ok ? k.xs[int64_t(tile_base + first_tile) * 32 + i] : 0.f;
         }
         __syncthreads();
-        const int pairs = sb_end * 4;
-        for (int sb = 0; sb < sb_end; ++sb) {
-            const int buf = sb & 1;
+
+        // row tiles mg and mg + 4 of the chunk: a short chunk spreads over the row groups
+        const int my_tiles = (mg < live_tiles ? 1 : 0) + (mg + 4 < live_tiles ? 1 : 0);
+        static_assert(kMT == 2 && kChunkTiles == 8, "row tile t of a wave is tile mg + 4 t of the chunk");
+        const int8_t * a_base = k.xq + int64_t(tile_base + first_tile + mg) * 32 * k.b0.cols + lane * 16;
+        const int64_t a_tile = int64_t(4) * 32 * k.b0.cols;
+
+        // weight rows of this wave's operand slot: gate / up: the unit's 32 rows of bank nbw; down: row tile NB * unit + nbw
+        const BankView & bank = nbw ? k.b1 : k.b0;
+        const int64_t tile_g = int64_t(e) * tiles_w + (k.gateup ? unit : NB * unit + nbw);
+        const uint8_t * codes = bank.codes + tile_g * S * 512 + n * 16 + g * 8;   // sub-block s of the tile: + 512 s; lane = (row n, code half g)
+        const uint8_t * aux = bank.aux + tile_g * NSB * 256 + n * 8;              // super-block sb of the tile: + 256 sb
+
+        // The super-block loop is instantiated per number of live row tiles of the wave (0..kMT), so that its body is one
+        // straight line of code the scheduler can interleave. Every instance passes the same barriers.
+        auto body = [&](auto mt_tag) {
+            constexpr int MT = decltype(mt_tag)::value;
+            constexpr int MTA = MT ? MT : 1;
+            v16i acc_h[MTA], acc_l[MTA];
+            float acc_f[MTA][16];
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) d_cur[nb] = d_next[nb];
-            // past the last super-block the fetch repeats it and the decode fills the stage nobody reads: no branches here
-            decode_into(buf ^ 1);
-            fetch(min(sb + 2, sb_end - 1));
+            for (int t = 0; t < MTA; ++t)
 #pragma unroll
-            for (int jp = 0; jp < 4; ++jp) {
-                load_a((jp + 3) & 3, min(sb * 4 + jp + 3, pairs - 1));
+                for (int i = 0; i < 16; ++i) { acc_f[t][i] = 0.f; acc_h[t][i] = 0; acc_l[t][i] = 0; }
+
+            // this wave decodes sub-blocks 2 mg and 2 mg + 1 of every super-block of its slot: the codes and the scale
+            // record are fetched one super-block before they are decoded, so that their latency is not waited for
+            float d_next = 0.f, d_cur = 0.f;
+            uint2 f_rec = {0, 0}, f_code[2] = {{0, 0}, {0, 0}};
+            auto fetch = [&](int sb) {
+                f_rec = *reinterpret_cast<const uint2 *>(aux + int64_t(sb) * 256);
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const int ib = 2 * jp + h;
-                    v4i bh[NB], bl[NB];
+                for (int j = 0; j < 2; ++j) f_code[j] = *reinterpret_cast<const uint2 *>(codes + (int64_t(sb) * 8 + 2 * mg + j) * 512);
+            };
+            auto decode_into = [&](int buf) {
+                d_next = half_bits_to_float(uint16_t(f_rec.x & 0xFFFFu));
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) {
-                        bh[nb] = bs[(((buf * NB + nb) * 2 + 0) * 8 + ib) * 64 + lane];
-                        bl[nb] = bs[(((buf * NB + nb) * 2 + 1) * 8 + ib) * 64 + lane];
+                for (int j = 0; j < 2; ++j) {
+                    const int ib = 2 * mg + j;
+                    const uint4 * tab = reinterpret_cast<const uint4 *>(s_tab + iq4xs_ls(f_rec, ib) * 32);
+                    v4i h, l;
+                    decode_planes(f_code[j], tab[0], tab[1], h, l);
+                    bs[(((buf * NB + nbw) * 2 + 0) * 8 + ib) * 64 + lane] = h;
+                    bs[(((buf * NB + nbw) * 2 + 1) * 8 + ib) * 64 + lane] = l;
+                }
+            };
+            // operand A, two k-steps (sub-blocks) per slot, fetched kSlots - 1 slots before its products
+            constexpr int kSlots = 4;
+            v4i a_reg[kSlots][MTA][2];
+            auto load_a = [&](int slot, int pair) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) a_reg[slot][t][h] = *reinterpret_cast<const v4i *>(a_base + t * a_tile + (int64_t(pair) * 2 + h) * 1024);
+            };
+
+            const int pairs = sb_end * 4;
+            if (sb_end > 0) {
+                fetch(0);
+#pragma unroll
+                for (int q = 0; q < kSlots - 1; ++q) load_a(q, min(q, pairs - 1));
+                decode_into(0);
+                fetch(min(1, sb_end - 1));
+            }
+            __syncthreads();
+            for (int sb = 0; sb < sb_end; ++sb) {
+                const int buf = sb & 1;
+                d_cur = d_next;
+                // past the last super-block the fetch repeats it and the decode fills the stage nobody reads: no branches here
+                decode_into(buf ^ 1);
+                fetch(min(sb + 2, sb_end - 1));
+#pragma unroll
+                for (int jp = 0; jp < 4; ++jp) {
+                    load_a((jp + kSlots - 1) % kSlots, min(sb * 4 + jp + kSlots - 1, pairs - 1));
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int ib = 2 * jp + h;
+                        const v4i bh = bs[(((buf * NB + nbw) * 2 + 0) * 8 + ib) * 64 + lane];
+                        const v4i bl = bs[(((buf * NB + nbw) * 2 + 1) * 8 + ib) * 64 + lane];
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) {
+                            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                            acc_h[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp % kSlots][t][h], bh, ib ? acc_h[t] : zero, 0, 0, 0);
+                            acc_l[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp % kSlots][t][h], bl, ib ? acc_l[t] : zero, 0, 0, 0);
+                        }
                     }
+                }
+                // |64 acc_h + acc_l| <= 256 * 127 * 127 * 32 < 2^28: exact in int32, then one rounding into fp32
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc_f[t][i] += float((acc_h[t][i] << 6) + acc_l[t][i]) * d_cur;
+                __syncthreads();
+            }
+            // result register i of lane half g is tile row 8 (i / 4) + 4 g + i % 4, weight row n.
+            // gate / up: the up waves hand their sums to the gate waves of the same rows through the (now idle) weight stage.
+            float * ex = reinterpret_cast<float *>(lds);
+            if (k.gateup && NB == 2) {
+                if (nbw == 1) {
 #pragma unroll
                     for (int t = 0; t < MT; ++t)
 #pragma unroll
-                        for (int nb = 0; nb < NB; ++nb) {
-                            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                            acc_h[t][nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp][t][h], bh[nb], ib ? acc_h[t][nb] : zero, 0, 0, 0);
-                            acc_l[t][nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp][t][h], bl[nb], ib ? acc_l[t][nb] : zero, 0, 0, 0);
-                        }
+                        for (int i = 0; i < 16; ++i) ex[((mg * kMT + t) * 16 + i) * 64 + lane] = acc_f[t][i];
+                }
+                __syncthreads();
+                if (nbw == 1) return;
+            }
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int m = (mg + 4 * t) * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                    const int a = s_asg[m];
+                    if (a < 0) continue;
+                    const float sc = s_scale[m];
+                    uint16_t * o = k.out + int64_t(a) * rows;
+                    if (k.gateup) {
+                        const float gv = acc_f[t][i] * sc, uv = (NB == 2 ? ex[((mg * kMT + t) * 16 + i) * 64 + lane] : acc_f[t][i]) * sc;
+                        o[unit * 32 + n] = __half_as_ushort(__float2half_rn(gv / (1.f + expf(-gv)) * uv));
+                    } else {
+                        o[(NB * unit + nbw) * 32 + n] = __half_as_ushort(__float2half_rn(acc_f[t][i] * sc));
+                    }
                 }
             }
-            // |64 acc_h + acc_l| <= 256 * 127 * 127 * 32 < 2^28: exact in int32, then one rounding into fp32
-#pragma unroll
-            for (int t = 0; t < MT; ++t)
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) acc_f[t][nb][i] += float((acc_h[t][nb][i] << 6) + acc_l[t][nb][i]) * d_cur[nb];
-            __syncthreads();
+        };
+        static_assert(kMT == 2, "the dispatch below lists the instances");
+        switch (my_tiles) {
+            case 0: body(std::integral_constant<int, 0>{}); break;
+            case 1: body(std::integral_constant<int, 1>{}); break;
+            default: body(std::integral_constant<int, 2>{}); break;
         }
-        // result register i of lane half g is tile row 8 (i / 4) + 4 g + i % 4, weight row n
-        const int g = lane >> 5;
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int m = (wave * kMT + t) * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-                const int a = s_asg[m];
-                if (a < 0) continue;
-                const float sc = s_scale[m];
-                uint16_t * o = k.out + int64_t(a) * rows;
-                if (k.gateup) {
-                    const float gv = acc_f[t][0][i] * sc, uv = acc_f[t][NB - 1][i] * sc;
-                    o[unit * 32 + n] = __half_as_ushort(__float2half_rn(gv / (1.f + expf(-gv)) * uv));
-                } else {
-#pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) o[(NB * unit + nb) * 32 + n] = __half_as_ushort(__float2half_rn(acc_f[t][nb][i] * sc));
-                }
-            }
-        }
-    };
-    static_assert(kMT == 2, "the dispatch below lists the instances");
-    switch (my_tiles) {
-        case 0: body(std::integral_constant<int, 0>{}); break;
-        case 1: body(std::integral_constant<int, 1>{}); break;
-        default: body(std::integral_constant<int, 2>{}); break;
-    }
     }   // items
 }
 
@@ -435,7 +428,7 @@ int32_t enqueue_iq4xs_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const i
     if (nb == 2) {
         static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(&iq4xs_gemm_k<2>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
         (void)once;
-        iq4xs_gemm_k<2><<<blocks, 256, lds, s>>>(k);
+        iq4xs_gemm_k<2><<<blocks, 512, lds, s>>>(k);
     } else {
         iq4xs_gemm_k<1><<<blocks, 256, lds, s>>>(k);
     }

@@ -196,7 +196,7 @@ def main():
             counts, offsets, perm, _ = tq.moe_dispatch(ext, CFG["experts"] + 1)
             lists = (counts, offsets, perm)
             xq, xsc = tq.group_rows_i8(x, lists, T * slots, slots)
-            act = tq.expert_gemm_gateup(l.gate, l.up, xq, xsc, lists, T, slots, CFG["topk"], CFG["shared_ff"])
+            act = tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, CFG["topk"], CFG["shared_ff"])
             aq, asc = tq.group_rows_i8(act, lists, T * slots, 1)
             prep.append((l, lists, xq, xsc, aq, asc))
         else:
@@ -209,7 +209,7 @@ def main():
         for item in prep:
             if prefill:
                 l, lists, xq, xsc, aq, asc = item
-                tq.expert_gemm_gateup(l.gate, l.up, xq, xsc, lists, T, slots, CFG["topk"], CFG["shared_ff"])
+                tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, CFG["topk"], CFG["shared_ff"])
             else:
                 l, ext, img, act, y = item
                 tq.expert_gateup(l.gate, l.up, img, ext, CFG["topk"], shared_ff=CFG["shared_ff"], act_image=act)

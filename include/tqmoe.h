@@ -204,6 +204,19 @@ int32_t tqmoe_expert_gemm_gateup_i8(const tqmoe_bank * gate, const tqmoe_bank * 
 int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const int32_t * counts,
                              const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk,
                              int32_t shared_lim, void * y_f16, void * stream, tqmoe_error * err);
+/* The same two products for every bank format, with fp16 operands (weights decoded and rounded to fp16, input rows
+ * converted to fp16, fp32 accumulation on the matrix cores): WeightFormat::expert_gemm (weight_format.hpp:51-53) and
+ * expert_gemm_gateup (weight_format.hpp:57-59). x: device rows of xtype with the bank's cols; the input row of
+ * assignment a is a / slots (tqmoe_expert_gemm_gateup; tqmoe_expert_gemm without per_expert_input) or a itself
+ * (per_expert_input). shared_lim a multiple of 32. act: fp16 [n * slots][rows]; y: [n * slots][rows] of ytype (F16 or F32). */
+int32_t tqmoe_expert_gemm_gateup(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x, uint32_t xtype,
+                                 const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t n,
+                                 int32_t slots, int32_t topk, int32_t shared_lim, void * act_f16, void * stream,
+                                 tqmoe_error * err);
+int32_t tqmoe_expert_gemm(const tqmoe_bank * bank, const void * x, uint32_t xtype, const int32_t * counts,
+                          const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk,
+                          int32_t shared_lim, int32_t per_expert_input, void * y, uint32_t ytype, void * stream,
+                          tqmoe_error * err);
 /* tqmoe_combine_strided with fp16 rows (the prefill products' output) */
 int32_t tqmoe_combine_strided_f16(const void * routed, int32_t slots, const void * shared, int64_t shared_ld,
                                   const float * weights, const float * shared_weights, void * out, uint32_t otype,

@@ -50,7 +50,7 @@ def make_banks(cfg, seed, distinct=None, sigma=0.02):
         per = raw.size // d
         if d < e:
             raw = np.tile(raw, (e + d - 1) // d)[: per * e].copy()
-            factors = 1.0 + (np.arange(e) // d) / 64.0
+            factors = 1.0 + 0.25 * (np.arange(e) // d) / max(1, (e - 1) // d)       # up to 1.25: all different, magnitudes as configured
             raw = _scale_field(raw, cfg["wtype"], per // oracle.BLOCK[cfg["wtype"]][1], factors)
         banks.append(raw)
     return banks

@@ -107,7 +107,7 @@ def test_grouped_products_against_float64(tq, oracle, n, shared_ff):
     uq, us = ungroup(xq.cpu().numpy(), xs.cpu().numpy(), want_counts, perm.cpu().numpy(), n * slots)
     assert np.array_equal(uq, natural_order(pq.cpu().numpy())[np.arange(n * slots) // slots])
     assert np.array_equal(us, ps.cpu().numpy()[np.arange(n * slots) // slots])
-    act = tq.expert_gemm_gateup(gate, up, xq, xs, lists, n, slots, k, shared_ff)
+    act = tq.expert_gemm_gateup_i8(gate, up, xq, xs, lists, n, slots, k, shared_ff)
     xd = natural_order(pq.cpu().numpy()).astype(np.float64) * ps.cpu().numpy().astype(np.float64)[:, None]
     got = act.float().cpu().numpy()
     for a in range(n * slots):
@@ -137,7 +137,7 @@ def test_grouped_products_skip_negative_ids(tq, oracle):
     x = torch.randn(n, hidden, device="cuda", dtype=torch.bfloat16)
     counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), banks)
     xq, xs = tq.group_rows_i8(x, (counts, offsets, perm), n * slots, slots)
-    act = tq.expert_gemm_gateup(gate, up, xq, xs, (counts, offsets, perm), n, slots, k).cpu().numpy()
+    act = tq.expert_gemm_gateup_i8(gate, up, xq, xs, (counts, offsets, perm), n, slots, k).cpu().numpy()
     flat = ids.reshape(-1)
     assert not act[flat < 0].any()
     assert act[flat >= 0].any(axis=1).all()

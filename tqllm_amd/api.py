@@ -82,6 +82,8 @@ def lib():
         l.tqmoe_group_rows_i8.argtypes = [p, u32, i32, p, p, p, i32, i64, i32, p, p, p, e]
         l.tqmoe_expert_gemm_gateup_i8.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_expert_gemm_i8.argtypes = [C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
+        l.tqmoe_expert_gemm_gateup.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, u32, p, p, p, i32, i32, i32, i32, p, p, e]
+        l.tqmoe_expert_gemm.argtypes = [C.POINTER(_Bank), p, u32, p, p, p, i32, i32, i32, i32, i32, p, u32, p, e]
         l.tqmoe_swiglu.argtypes = [p, p, p, i64, p, e]
         l.tqmoe_combine.argtypes = [p, p, p, p, p, u32, i32, i32, i32, p, e]
         l.tqmoe_layer_workspace_bytes.restype = sz
@@ -306,7 +308,30 @@ def group_rows_i8(x, lists, assignments, xdiv):
     return q, scale
 
 
-def expert_gemm_gateup(gate, up, xq, xs, lists, n, slots, topk, shared_ff=0):
+def expert_gemm_gateup(gate, up, x, lists, n, slots, topk, shared_ff=0):
+    """WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59), any bank format, fp16 operands: fp16 act [n * slots][ff];
+    rows of assignments that are in no list are zero here (the library leaves them untouched)."""
+    counts, offsets, perm = lists
+    act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=x.device)
+    err = _err()
+    g, u = gate.view(), up.view()
+    _check(lib().tqmoe_expert_gemm_gateup(C.byref(g), C.byref(u), _ptr(x), _ttype(x), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff,
+                                          _ptr(act), _stream(x), C.byref(err)), err)
+    return act
+
+
+def expert_gemm(bank, x, lists, n, slots, topk, shared_ff=0, per_expert_input=False, out_type=F16):
+    """WeightFormat::expert_gemm (weight_format.hpp:51-53), any bank format, fp16 operands: y [n * slots][rows], fp16 or fp32."""
+    counts, offsets, perm = lists
+    y = torch.zeros((n * slots, bank.rows), dtype=torch.float16 if out_type == F16 else torch.float32, device=x.device)
+    err = _err()
+    b = bank.view()
+    _check(lib().tqmoe_expert_gemm(C.byref(b), _ptr(x), _ttype(x), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff, int(per_expert_input),
+                                   _ptr(y), out_type, _stream(x), C.byref(err)), err)
+    return y
+
+
+def expert_gemm_gateup_i8(gate, up, xq, xs, lists, n, slots, topk, shared_ff=0):
     """WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59) on int8 rows: fp16 act [n * slots][ff]; rows of
     assignments that are in no list are zero here (the library leaves them untouched)."""
     counts, offsets, perm = lists

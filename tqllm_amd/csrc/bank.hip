@@ -1,6 +1,6 @@
 // Expert banks: GGUF block stream -> device layout (one thread per 32-weight sub-block), and the fp32 dequantiser
 // whose values are those of the host decoder bit for bit (no fused multiply-add, same evaluation order).
-#include "formats.cuh"
+#include "decode_sub.cuh"
 
 namespace tqmoe {
 namespace {
@@ -86,90 +86,11 @@ __global__ __launch_bounds__(256) void dequant_k(uint32_t type, const uint8_t * 
     const int S = cols / 32;
     const int64_t idx = int64_t(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= nrows * S) return;
-    const int64_t row = row0 + idx / S;
-    const int s = int(idx % S), ib = s & 7;
-    const uint8_t * cd = codes + (row * S + s) * code_bytes_per_sub(type);
-    float * y = out + idx * 32;
-    switch (type) {
-        case TQMOE_IQ4_XS: {
-            const uint2 rec = *reinterpret_cast<const uint2 *>(aux + iq4xs_aux_offset(row, S, s / 8));
-            const float dl = __fmul_rn(half_bits_to_float(uint16_t(rec.x & 0xFFFFu)), float(iq4xs_ls(rec, ib) - 32));
-            const uint4 c = *reinterpret_cast<const uint4 *>(codes + iq4xs_code_offset(row, S, s));
-            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+    float y[32];
+    decode_sub32(type, codes, aux, rows_total, cols, row0 + idx / S, int(idx % S), y);
+    float4 * o = reinterpret_cast<float4 *>(out + idx * 32);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t lo, hi;
-                lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(w[q], lo, hi);
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    y[4 * q + b] = __fmul_rn(dl, float(int8_t(lo >> (8 * b))));
-                    y[16 + 4 * q + b] = __fmul_rn(dl, float(int8_t(hi >> (8 * b))));
-                }
-            }
-            break;
-        }
-        case TQMOE_Q4_K: {
-            const uint4 rec = *reinterpret_cast<const uint4 *>(aux + (row * (S / 8) + s / 8) * 16);
-            const uint32_t sc12[3] = {rec.y, rec.z, rec.w};
-            int sc, mn;
-            q4k_scale_min(sc12, ib, sc, mn);
-            const float d1 = __fmul_rn(half_bits_to_float(uint16_t(rec.x & 0xFFFFu)), float(sc));
-            const float m1 = __fmul_rn(half_bits_to_float(uint16_t(rec.x >> 16)), float(mn));
-            const uint4 c = *reinterpret_cast<const uint4 *>(cd);
-            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    const uint32_t byte = (w[q] >> (8 * b)) & 0xFFu;
-                    y[4 * q + b] = __fsub_rn(__fmul_rn(d1, float(byte & 15u)), m1);
-                    y[16 + 4 * q + b] = __fsub_rn(__fmul_rn(d1, float(byte >> 4)), m1);
-                }
-            break;
-        }
-        case TQMOE_IQ3_S: {
-            const uint4 rec = *reinterpret_cast<const uint4 *>(aux + (row * (S / 8) + s / 8) * 16);
-            // rec: d | qh[0..1] << 16, qh[2..5], qh[6..7] | scales[0..1] << 16, scales[2..3]
-            const uint32_t qh = ib < 2 ? (rec.x >> (16 + 8 * ib)) & 0xFFu : ib < 6 ? (rec.y >> (8 * (ib - 2))) & 0xFFu : (rec.z >> (8 * (ib - 6))) & 0xFFu;
-            const uint32_t scb = (ib >> 1) < 2 ? (rec.z >> (16 + 8 * (ib >> 1))) & 0xFFu : (rec.w >> (8 * ((ib >> 1) - 2))) & 0xFFu;
-            const float db = __fmul_rn(half_bits_to_float(uint16_t(rec.x & 0xFFFFu)), float(1 + 2 * int((scb >> (4 * (ib & 1))) & 15u)));
-            const uint32_t * c = reinterpret_cast<const uint32_t *>(cd);
-            const uint32_t qs[2] = {c[0], c[1]}, sg = c[2];
-#pragma unroll
-            for (int w = 0; w < 8; ++w) {
-                const uint32_t g = d_iq3s_grid.v[((qs[w >> 2] >> (8 * (w & 3))) & 0xFFu) | (((qh >> w) & 1u) << 8)];
-                const uint32_t sn = sg >> (4 * w);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float mag = __fmul_rn(db, float((g >> (8 * j)) & 0xFFu));
-                    y[4 * w + j] = ((sn >> j) & 1u) ? -mag : mag;
-                }
-            }
-            break;
-        }
-        case TQMOE_NVFP4G: {
-            const float g = *reinterpret_cast<const float *>(aux + nvfp4_global_offset(rows_total, cols) + row * 4);
-            const uint8_t * sc = aux + row * (cols / 16) + 2 * s;
-            const float d0 = __fmul_rn(e4m3_to_float(sc[0]), g), d1 = __fmul_rn(e4m3_to_float(sc[1]), g);
-            const uint4 c = *reinterpret_cast<const uint4 *>(cd);
-            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t lo, hi;
-                lookup16<kFp4T0, kFp4T1, kFp4T2, kFp4T3>(w[q], lo, hi);
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    // table holds twice the E2M1 value; halving is exact. -0 codes give -0 * d on the host: keep the sign
-                    const uint32_t nlo = (w[q] >> (8 * b)) & 15u, nhi = (w[q] >> (8 * b + 4)) & 15u;
-                    const float vlo = nlo == 8 ? -0.f : 0.5f * float(int8_t(lo >> (8 * b)));
-                    const float vhi = nhi == 8 ? -0.f : 0.5f * float(int8_t(hi >> (8 * b)));
-                    y[4 * q + b] = __fmul_rn(vlo, d0);
-                    y[16 + 4 * q + b] = __fmul_rn(vhi, d1);
-                }
-            }
-            break;
-        }
-    }
+    for (int q = 0; q < 8; ++q) o[q] = make_float4(y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]);
 }
 
 }  // namespace

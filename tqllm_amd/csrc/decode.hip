@@ -6,6 +6,8 @@ namespace tqmoe {
 int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);  // bank.hip
 // prefill_iq4xs.hip
 int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, hipStream_t s);
+int32_t enqueue_gemm_f16(const tqmoe_bank & b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int * counts, const int * offsets, const int * perm,
+                         int experts, int64_t assignments, int xdiv, void * out, int out_f32, int gateup, int shared_expert, int shared_lim, hipStream_t s);
 int64_t grouped_row_tiles(int64_t assignments, int experts);
 int64_t grouped_scale_words(int64_t assignments, int experts);
 int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
@@ -269,4 +271,40 @@ extern "C" int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * 
                                         const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * y_f16, void * stream,
                                         tqmoe_error * err) {
     return gemm_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8");
+}
+
+static int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int32_t * counts, const int32_t * offsets,
+                               const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, int32_t xdiv, void * out, uint32_t otype, int gateup,
+                               void * stream, tqmoe_error * err, const char * what) {
+    if (int32_t rc = check_bank(b0, what, err)) return rc;
+    if (b1) {
+        if (int32_t rc = check_bank(b1, what, err)) return rc;
+        if (b1->type != b0->type || b1->rows != b0->rows || b1->cols != b0->cols || b1->experts != b0->experts)
+            return fail(err, TQMOE_E_ARG, "%s: the two banks differ in format or shape", what);
+    }
+    if (!x || !counts || !offsets || !perm || !out || n <= 0 || topk <= 0 || slots < topk) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    if (!is_act_type(xtype) || (otype != TQMOE_F16 && otype != TQMOE_F32)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported element type", what);
+    const int lim_max = gateup ? b0->rows : b0->cols;
+    if (slots > topk && (shared_lim <= 0 || shared_lim > lim_max || shared_lim % 32)) return fail(err, TQMOE_E_ARG, "%s: shared_lim must be a multiple of 32 within the bank", what);
+    if (b0->experts > 4096) return fail(err, TQMOE_E_ARG, "%s: more than 4096 experts", what);
+    if (int32_t rc = need_device(err, what)) return rc;
+    const int shared_expert = slots > topk ? b0->experts - 1 : -1;
+    if (enqueue_gemm_f16(*b0, b1, x, xtype, counts, offsets, perm, b0->experts, int64_t(n) * slots, xdiv, out, otype == TQMOE_F32, gateup, shared_expert,
+                         shared_lim, static_cast<hipStream_t>(stream)))
+        return fail(err, TQMOE_E_ARG, "%s: too many assignments for one call", what);
+    return launched(err, what);
+}
+
+extern "C" int32_t tqmoe_expert_gemm_gateup(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x, uint32_t xtype, const int32_t * counts,
+                                            const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * act_f16,
+                                            void * stream, tqmoe_error * err) {
+    if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_gemm_gateup: second bank missing");
+    return gemm_f16_common(gate, up, x, xtype, counts, offsets, perm, n, slots, topk, shared_lim, slots, act_f16, TQMOE_F16, 1, stream, err, "tqmoe_expert_gemm_gateup");
+}
+
+extern "C" int32_t tqmoe_expert_gemm(const tqmoe_bank * bank, const void * x, uint32_t xtype, const int32_t * counts, const int32_t * offsets, const int32_t * perm,
+                                     int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, int32_t per_expert_input, void * y, uint32_t ytype, void * stream,
+                                     tqmoe_error * err) {
+    return gemm_f16_common(bank, nullptr, x, xtype, counts, offsets, perm, n, slots, topk, shared_lim, per_expert_input ? 1 : slots, y, ytype, 0, stream, err,
+                           "tqmoe_expert_gemm");
 }

@@ -15,24 +15,24 @@ constexpr int kGroupedMin = 64;
 constexpr int kDecodeAssignments = 65535;   // per decode launch
 
 struct Plan {  // byte offsets into the workspace
-    bool grouped;
+    bool grouped;   // the grouped products (prefill sizes): int8 for IQ4_XS banks, fp16 for the other formats
+    bool int8;
     int chunk;   // tokens per pass of the expert stages
     size_t logits, ids, weights, shared_w, ids_ext, total;
     size_t ximage, aimage, y;                                                // decode path
     size_t xq, xs, counts, offsets, perm, dispatch_ws, act16, aq, as, y16;   // grouped path
 };
 
-bool grouped_ok(const tqmoe_layer & L, int n) {
-    return L.gate.type == TQMOE_IQ4_XS && n >= kGroupedMin && (!L.has_shared || L.shared_ff % 256 == 0);
-}
+bool int8_ok(const tqmoe_layer & L) { return L.gate.type == TQMOE_IQ4_XS && (!L.has_shared || L.shared_ff % 256 == 0); }
 
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
     const int slots = L.topk + (L.has_shared ? 1 : 0), banks = L.n_expert + (L.has_shared ? 1 : 0);
-    p.grouped = grouped_ok(L, n);
+    p.grouped = n >= kGroupedMin;
+    p.int8 = p.grouped && int8_ok(L);
     // the grouped products take 2^24 assignments a pass (32-bit block and byte counts stay far from their limits), the
     // decode kernels 65535
-    const int64_t per_pass = p.grouped ? int64_t(1) << 24 : kDecodeAssignments;
+    const int64_t per_pass = p.int8 ? int64_t(1) << 24 : p.grouped ? int64_t(65535 - banks) * 64 : kDecodeAssignments;
     p.chunk = int(std::min<int64_t>(n, std::max<int64_t>(1, per_pass / slots)));
     size_t o = 0;
     auto take = [&](size_t bytes) { const size_t at = o; o = align_up(o + bytes, 256); return at; };
@@ -43,19 +43,21 @@ Plan plan_for(const tqmoe_layer & L, int n) {
     p.ids_ext = take(size_t(n) * slots * 4);
     const size_t c = size_t(p.chunk), a = c * slots;
     if (p.grouped) {
-        const size_t grows = size_t(tqmoe_grouped_rows(int64_t(a), banks));
-        p.xq = take(grows * L.hidden);
-        const size_t gwords = size_t(tqmoe_grouped_scale_words(int64_t(a), banks));
-        p.xs = take(gwords * 4);
         p.counts = take(size_t(banks) * 4);
         p.offsets = take(size_t(banks + 1) * 4);
         p.perm = take(a * 4);
         p.dispatch_ws = take(tqmoe_dispatch_workspace_bytes(banks, p.chunk, slots));
         p.act16 = take(a * L.ff * 2);
+        p.y16 = take(a * L.hidden * 4);   // fp16 rows (int8 products) or fp32 rows (fp16 products)
+    }
+    if (p.int8) {
+        const size_t grows = size_t(tqmoe_grouped_rows(int64_t(a), banks));
+        p.xq = take(grows * L.hidden);
+        const size_t gwords = size_t(tqmoe_grouped_scale_words(int64_t(a), banks));
+        p.xs = take(gwords * 4);
         p.aq = take(grows * L.ff);
         p.as = take(gwords * 4);
-        p.y16 = take(a * L.hidden * 2);
-    } else {
+    } else if (!p.grouped) {
         p.ximage = take(tqmoe_act_image_bytes(n, L.hidden));
         p.aimage = take(tqmoe_act_image_bytes(int32_t(a), L.ff));
         p.y = take(a * L.hidden * 4);
@@ -133,11 +135,21 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
             uint16_t * act16 = reinterpret_cast<uint16_t *>(ws + p.act16), * y16 = reinterpret_cast<uint16_t *>(ws + p.y16);
             if (int32_t rc = tqmoe_dispatch(cid, counts, offsets, perm, nullptr, 0, banks, c, slots, ws + p.dispatch_ws,
                                             tqmoe_dispatch_workspace_bytes(banks, c, slots), stream, err)) return rc;
+            if (!p.int8) {
+                if (int32_t rc = tqmoe_expert_gemm_gateup(&L.gate, &L.up, xb + size_t(t0) * L.hidden * xbytes, xtype, counts, offsets, perm, c, slots, L.topk, L.shared_ff,
+                                                          act16, stream, err)) return rc;
+                float * y32 = reinterpret_cast<float *>(y16);
+                if (int32_t rc = tqmoe_expert_gemm(&L.down, act16, TQMOE_F16, counts, offsets, perm, c, slots, L.topk, L.shared_ff, 1, y32, TQMOE_F32, stream, err)) return rc;
+                if (int32_t rc = tqmoe_combine_strided(y32, slots, L.has_shared ? y32 + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, cw, csw, cout, otype,
+                                                       L.hidden, L.topk, c, stream, err)) return rc;
+                continue;
+            } else {
             if (int32_t rc = tqmoe_group_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq,
                                                  xs, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_gateup_i8(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
             if (int32_t rc = tqmoe_group_rows_i8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_i8(&L.down, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
+            }
             if (int32_t rc = tqmoe_combine_strided_f16(y16, slots, L.has_shared ? y16 + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, cw, csw,
                                                        cout, otype, L.hidden, L.topk, c, stream, err)) return rc;
         } else {

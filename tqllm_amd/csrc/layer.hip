@@ -13,6 +13,7 @@ namespace {
 // Token counts from kGroupedMin up take the grouped int8 products (IQ4_XS banks), fewer the decode kernels.
 constexpr int kGroupedMin = 64;
 constexpr int kDecodeAssignments = 65535;   // per decode launch
+constexpr int kDecodeDedup = 2048;          // assignments up to which the decode kernels serve an expert's rows together
 
 struct Plan {  // byte offsets into the workspace
     bool grouped;   // the grouped products (prefill sizes): int8 for IQ4_XS banks, fp16 for the other formats
@@ -28,8 +29,10 @@ bool int8_ok(const tqmoe_layer & L) { return L.gate.type == TQMOE_IQ4_XS && (!L.
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
     const int slots = L.topk + (L.has_shared ? 1 : 0), banks = L.n_expert + (L.has_shared ? 1 : 0);
-    p.grouped = n >= kGroupedMin;
-    p.int8 = p.grouped && int8_ok(L);
+    // the int8 grouped products from kGroupedMin tokens; the fp16 ones (other formats) once the decode kernels no longer
+    // read every expert's weights once (they group an expert's rows up to kDecodeDedup assignments a launch)
+    p.int8 = n >= kGroupedMin && int8_ok(L);
+    p.grouped = p.int8 || int64_t(n) * slots > kDecodeDedup;
     // the grouped products take 2^24 assignments a pass (32-bit block and byte counts stay far from their limits), the
     // decode kernels 65535
     const int64_t per_pass = p.int8 ? int64_t(1) << 24 : p.grouped ? int64_t(65535 - banks) * 64 : kDecodeAssignments;

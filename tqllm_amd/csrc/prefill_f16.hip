@@ -6,9 +6,9 @@
 // grouped product of their own (Q4_K, IQ3_S, NVFP4G) and IQ4_XS shapes the int8 one does not take.
 //
 // A block takes one expert, up to 64 of its assignments (the dispatch lists give them) and 64 weight rows of each bank;
-// its four waves hold one 32 x 32 quadrant each. Per 32-weight sub-block the block stages the 64 x 32 input tile and
-// the 64 x 32 weight tile(s) in LDS (each weight row's sub-block decoded by one thread with the bank's exact decoder,
-// then rounded to fp16) and every wave issues two matrix instructions per bank.
+// its four waves hold one 32 x 32 quadrant each. Per 128 weights of a row (four sub-blocks) the block stages the
+// 64 x 128 input tile and the 64 x 128 weight tile(s) in LDS (each weight row's sub-block decoded by one thread with the
+// bank's exact decoder, then rounded to fp16) and every wave issues eight matrix instructions per bank.
 #include "decode_api.cuh"
 #include "decode_sub.cuh"
 
@@ -19,7 +19,8 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kRowsPerBlock = 64;   // assignments per block
-constexpr int kPad = 40;            // halves per staged row: 32 + 8, so that 16-byte reads of consecutive rows spread over the banks
+constexpr int kKT = 128;            // weights of a row per stage
+constexpr int kPad = kKT + 8;       // halves per staged row: 16-byte reads of consecutive rows spread over the LDS banks
 
 struct F16Args {
     BankView b0, b1;
@@ -88,20 +89,27 @@ __global__ __launch_bounds__(256) void expert_gemm_f16_k(F16Args k) {
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[nb][i] = 0.f;
-    const int ar = tid >> 2, ap = tid & 3;                      // input staging: row, 8-value part of the sub-block
+    const int ar = tid >> 2, ap = tid & 3;                      // input staging: row, the sub-block of the stage's four
     const int a_asg = s_asg[ar];
-    const int64_t a_at = int64_t(max(a_asg, 0) / k.xdiv) * cols + ap * 8;
-    const int bn = tid & 63, bb = tid >> 6;                     // weight staging: row of the 64, bank
-    const bool b_live = bb < NB && row0 + bn < row_lim;
-    for (int s = 0; s < s_end; ++s) {
+    const int64_t a_at = int64_t(max(a_asg, 0) / k.xdiv) * cols + ap * 32;
+    for (int s0 = 0; s0 < s_end; s0 += kKT / 32) {
         {
-            float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            if (a_asg >= 0) load8<XT>(k.x, a_at + int64_t(s) * 32, v);
-            *reinterpret_cast<uint4 *>(&As[ar][ap * 8]) = make_uint4(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]), pack_h2(v[4], v[5]), pack_h2(v[6], v[7]));
+            uint4 h[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                if (a_asg >= 0) load8<XT>(k.x, a_at + int64_t(s0) * 32 + q * 8, v);
+                h[q] = make_uint4(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]), pack_h2(v[4], v[5]), pack_h2(v[6], v[7]));
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *reinterpret_cast<uint4 *>(&As[ar][ap * 32 + q * 8]) = h[q];
         }
-        if (bb < NB) {
+        // weight staging: NB * 64 rows x 4 sub-blocks = NB * 256 decodes over the 256 threads
+#pragma unroll
+        for (int job = 0; job < NB; ++job) {
+            const int idx = job * 256 + tid, bb = idx >> 8, bn = (idx >> 2) & 63, sub = idx & 3, s = s0 + sub;
             float y[32];
-            if (b_live) {
+            if (row0 + bn < row_lim && s < s_end) {
                 const BankView & b = bb ? k.b1 : k.b0;
                 decode_sub32(k.type, b.codes, b.aux, b.rows_total, cols, int64_t(e) * rows + row0 + bn, s, y);
             } else {
@@ -110,12 +118,12 @@ __global__ __launch_bounds__(256) void expert_gemm_f16_k(F16Args k) {
             }
 #pragma unroll
             for (int q = 0; q < 4; ++q)
-                *reinterpret_cast<uint4 *>(&Bs[bb][bn][q * 8]) =
+                *reinterpret_cast<uint4 *>(&Bs[bb][bn][sub * 32 + q * 8]) =
                     make_uint4(pack_h2(y[8 * q], y[8 * q + 1]), pack_h2(y[8 * q + 2], y[8 * q + 3]), pack_h2(y[8 * q + 4], y[8 * q + 5]), pack_h2(y[8 * q + 6], y[8 * q + 7]));
         }
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {     // operand of lane (r, g): row r, columns 16 j + 8 g .. + 7
+        for (int j = 0; j < kKT / 16; ++j) {     // operand of lane (r, g): row r, columns 16 j + 8 g .. + 7
             const v8h a = *reinterpret_cast<const v8h *>(&As[mq * 32 + r][16 * j + 8 * g]);
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {

@@ -9,13 +9,12 @@
 // result registers 0..3 of lane half g are (hi, lo) of input rows 2g and 2g + 1, which one fp32 multiply-add each folds
 // into the lane's running sum with weight scale * activation scale. Waves that split a row's super-blocks add their
 // partial sums through LDS in wave order (deterministic).
-// The weight bytes are the only cold data: every wave streams its share (codes and scale records) straight into its own
-// LDS stage with direct-to-LDS loads, one super-block ahead of the one it is multiplying, so the loads of the next
-// super-block are in flight while this one is decoded.
+// The weight bytes are the only cold data: every wave loads its share (codes and scale records) into registers one
+// super-block ahead of the one it is multiplying, so the loads of the next super-block are in flight while this one is
+// decoded.
 #include "act_image.cuh"
 #include "decode_api.cuh"
 #include "formats.cuh"
-
 
 namespace tqmoe {
 namespace {
@@ -34,12 +33,15 @@ __device__ __forceinline__ int chunk_up(const int * __restrict__ ids, int A, int
 #pragma unroll
     for (int j = 0; j < kTP; ++j) tok[j] = -1;
     if (mode == 0) { tok[0] = a; return 1; }
+    int * copy = list + kMaxList;            // the ids, fetched by the whole block in one round trip
+    for (int i = threadIdx.x; i < A; i += blockDim.x) copy[i] = ids[i];
+    __syncthreads();
     if (threadIdx.x < 64) {   // one wave walks the ids in order: ballots keep the matches ordered
         const int lane = threadIdx.x;
         int base = 0;
         for (int i0 = 0; i0 < A; i0 += 64) {
             const int i = i0 + lane;
-            const bool match = i < A && ids[i] == e;
+            const bool match = i < A && copy[i] == e;
             const unsigned long long mask = __ballot(match);
             if (match) {
                 const int r = base + __popcll(mask & ((1ull << lane) - 1ull));
@@ -74,14 +76,10 @@ __device__ __forceinline__ v4i decode16(uint2 c, uint32_t pos) {
     return w;
 }
 
-constexpr int kCodeBytes = 4096;    // codes of one (row tile, super-block) of one bank: 8 sub-blocks x 32 rows x 16 B
-constexpr int kStageBytes = kCodeBytes + 256;   // then the 32 rows' 8-byte scale records
 
 // NB banks (gate and up, or one). gateup != 0: out0 is the activation image that receives silu(gate) * up; else out0 /
 // out1 receive the products as rows of `ytype`. wk waves share a row's super-blocks, tpw row tiles per block.
-// Dynamic LDS: waves * nstage * NB * kStageBytes of staging (filled by direct-to-LDS loads, so a wave has the bytes of
-// a super-block in flight without holding them in registers; nstage = 2 when a wave has more than one super-block); the
-// id list and the partial sums reuse that space.
+// Dynamic LDS: the match list and the copy of the ids while the block finds its input rows, later the partial sums.
 // UNI: every sub-block of an input row has the row's one activation scale (the images tqmoe_quant_act and the top-k
 // kernel write). The 6-bit weight scales then multiply the integer results and the sums stay integers over a whole
 // super-block; otherwise (rows quantised block by block, as the fused gate / up epilogue leaves them) each sub-block's
@@ -89,14 +87,14 @@ constexpr int kStageBytes = kCodeBytes + 256;   // then the 32 rows' 8-byte scal
 template <int NB, bool UNI>
 __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * out0, void * out1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_lim, int wk,
-                                                    int tpw, int nstage, int gateup) {
-    extern __shared__ __attribute__((aligned(1024))) uint8_t stage[];
+                                                    int tpw, int gateup) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
     __shared__ int meta[2], s_tok[kTP];
     __shared__ int ql[kMaxWaves * 2][32];
     const int a = blockIdx.y, e = ids[a];
     if (e < 0 || int64_t(e) * b0.rows >= b0.rows_total) return;   // skipped assignment, or an id outside the bank
     int tok[kTP];
-    const int n_tok = chunk_up(ids, A, a, e, mode, reinterpret_cast<int *>(stage), meta, tok);   // the list lives in the staging space
+    const int n_tok = chunk_up(ids, A, a, e, mode, reinterpret_cast<int *>(stage), meta, tok);   // the lists live in the dynamic space
     if (n_tok == 0) return;
     if (threadIdx.x < kTP) s_tok[threadIdx.x] = tok[threadIdx.x];
     __syncthreads();
@@ -109,7 +107,6 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
     const int row_lim = gateup && shared_slot ? shared_lim : rows;
     const int s_end = !gateup && shared_slot ? shared_lim / 32 : S;
     const bool valid = tile < tiles && tile * 32 < row_lim;
-    uint8_t * my_stage = stage + wave * (nstage * NB * kStageBytes);
 
     float accf[NB][2];
 #pragma unroll
@@ -126,23 +123,23 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
         const int64_t tile_g = int64_t(e) * tiles + tile;
         const uint32_t pos = 0x03020100u;
         const int sb_end = s_end / 8;   // whole super-blocks only (the launcher checks)
-        // a super-block's cold bytes (codes, records) go in flight at once, straight into the wave's stage `slot`
-        auto issue = [&](int sb, int slot) {
+        // The weight bytes of a super-block: 8 bytes of codes per sub-block and the row's scale record, per lane, in
+        // registers. The next super-block's are loaded before this one is multiplied, so that with several waves per SIMD
+        // there are always loads in flight under the decode work.
+        struct Cold { uint2 code[NB][8]; uint2 rec[NB]; };
+        auto fetch = [&](int sb, Cold & c) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-                uint8_t * dst = my_stage + (slot * NB + nb) * kStageBytes;
-                const uint8_t * src = (nb ? b1 : b0).codes + (tile_g * S + int64_t(sb) * 8) * 512 + lane * 16;
+                const uint8_t * src = (nb ? b1 : b0).codes + (tile_g * S + int64_t(sb) * 8) * 512 + n * 16 + g * 8;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) __builtin_amdgcn_global_load_lds(src + c * 1024, dst + c * 1024, 16, 0, 0);
-                if (lane < 16) __builtin_amdgcn_global_load_lds((nb ? b1 : b0).aux + (tile_g * NSB + sb) * 256 + lane * 16, dst + kCodeBytes, 16, 0, 0);
+                for (int ib = 0; ib < 8; ++ib) c.code[nb][ib] = *reinterpret_cast<const uint2 *>(src + ib * 512);
+                c.rec[nb] = *reinterpret_cast<const uint2 *>((nb ? b1 : b0).aux + (tile_g * NSB + sb) * 256 + n * 8);
             }
         };
-        if (wk_i < sb_end) issue(wk_i, 0);
-        int slot = 0;
+        Cold cur, nxt;
+        if (wk_i < sb_end) fetch(wk_i, cur);
         for (int sb = wk_i; sb < sb_end; sb += wk) {
-            const bool more = sb + wk < sb_end;
-            // the activation side of this super-block (warm data), then the next super-block's cold bytes: those stay the
-            // youngest loads, so the wait below can leave exactly them in flight
+            if (sb + wk < sb_end) fetch(sb + wk, nxt);
             v4i areg[8];
 #pragma unroll
             for (int ib = 0; ib < 8; ++ib) areg[ib] = a_tok >= 0 ? *reinterpret_cast<const v4i *>(a_row + (sb * 8 + ib) * 64) : v4i{0, 0, 0, 0};
@@ -154,24 +151,15 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
                 xs0[0] = p0.x; xs0[1] = p0.y; xs0[2] = p0.z; xs0[3] = p0.w; xs0[4] = p1.x; xs0[5] = p1.y; xs0[6] = p1.z; xs0[7] = p1.w;
                 xs1[0] = q0.x; xs1[1] = q0.y; xs1[2] = q0.z; xs1[3] = q0.w; xs1[4] = q1.x; xs1[5] = q1.y; xs1[6] = q1.z; xs1[7] = q1.w;
             }
-            if (more) issue(sb + wk, slot ^ 1);
-            // everything but the next super-block's loads (5 per bank, the youngest) has arrived
-            if (more) {
-                if (NB == 2) asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-            } else {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            }
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-                const uint8_t * st = my_stage + (slot * NB + nb) * kStageBytes;
-                const uint8_t * cl = st + n * 16 + g * 8;
-                const uint2 rec = *reinterpret_cast<const uint2 *>(st + kCodeBytes + n * 8);
+                const uint2 rec = cur.rec[nb];
                 const float d = half_bits_to_float(uint16_t(rec.x & 0xFFFFu));
                 const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 int si[4] = {0, 0, 0, 0};   // (hi, lo) plane sums of the two input rows, weighted by the sub-block scales
 #pragma unroll
                 for (int ib = 0; ib < 8; ++ib) {
-                    const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[ib], decode16(*reinterpret_cast<const uint2 *>(cl + ib * 512), pos), zero, 0, 0, 0);
+                    const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[ib], decode16(cur.code[nb][ib], pos), zero, 0, 0, 0);
                     if constexpr (UNI) {
                         // |acc| <= 32 * 128 * 127 < 2^19 and |ls - 32| <= 32: 24-bit products, eight of them stay below 2^28
                         const int ls = iq4xs_ls(rec, ib) - 32;
@@ -188,8 +176,7 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
                     accf[nb][1] += (float(si[2]) * 128.f + float(si[3])) * d;
                 }
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the staged bytes are consumed before a later share overwrites them
-            slot ^= 1;
+            cur = nxt;
         }
     }
     if constexpr (UNI) {
@@ -200,7 +187,7 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
             for (int nb = 0; nb < NB; ++nb) { accf[nb][0] *= x0; accf[nb][1] *= x1; }
         }
     }
-    __syncthreads();                                       // staging space is free: it now holds the partial sums
+    __syncthreads();                                       // the id list is done with: the space now holds the partial sums
     float (*red)[NB][kTP][32] = reinterpret_cast<float (*)[NB][kTP][32]>(stage);
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) { red[wave][nb][2 * g][n] = accf[nb][0]; red[wave][nb][2 * g + 1][n] = accf[nb][1]; }
@@ -234,28 +221,20 @@ void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0
     // is bound by the latency of one wave's chain), fewer when the batch has the waves anyway (a longer chain per
     // wave streams with its loads one super-block ahead and saves the cross-wave sums).
     const int64_t units = int64_t(A) * tiles;
-    const int cap = units >= 8192 ? 1 : units >= 2048 ? 2 : kMaxWaves;   // (4 shares with two stages each would leave one block per compute unit)
+    const int cap = units >= 8192 ? 1 : units >= 2048 ? 2 : kMaxWaves;
     int wk = 1;
     for (int w = 1; w <= kMaxWaves && w <= cap; ++w) if (NSB % w == 0) wk = w;
     const int waves = wk >= 4 ? kMaxWaves : 4;                            // per block
     int tpw = waves / wk;                                                 // row tiles per block
     if (tpw > tiles) tpw = tiles;
-    const int nstage = NSB / wk > 1 ? 2 : 1;
     const dim3 grid(unsigned((tiles + tpw - 1) / tpw), unsigned(A));
     const unsigned threads = unsigned(wk * tpw * 64);
-    // staging for the codes; the same space first holds the id list (kMaxList ints) and last the partial sums
-    size_t lds = size_t(wk * tpw) * nstage * nb * kStageBytes;
-    if (lds < size_t(kMaxList) * sizeof(int)) lds = size_t(kMaxList) * sizeof(int);
+    // dynamic LDS: the match list and the copy of the ids (2 * kMaxList ints), later the partial sums
+    size_t lds = mode ? size_t(2) * kMaxList * sizeof(int) : 0;
     if (lds < size_t(wk * tpw) * nb * kTP * 32 * sizeof(float)) lds = size_t(wk * tpw) * nb * kTP * 32 * sizeof(float);
-    if (lds > 65536) {
-        static const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void *>(&iq4xs_mfma_k<2, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
-        static const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(&iq4xs_mfma_k<1, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
-        static const hipError_t e3 = hipFuncSetAttribute(reinterpret_cast<const void *>(&iq4xs_mfma_k<2, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
-        (void)e1; (void)e2; (void)e3;
-    }
-    if (nb == 2 && uniform) iq4xs_mfma_k<2, true><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, nstage, gateup);
-    else if (nb == 2) iq4xs_mfma_k<2, false><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, nstage, gateup);
-    else iq4xs_mfma_k<1, false><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, nstage, gateup);
+    if (nb == 2 && uniform) iq4xs_mfma_k<2, true><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
+    else if (nb == 2) iq4xs_mfma_k<2, false><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
+    else iq4xs_mfma_k<1, false><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
 }
 
 }  // namespace

@@ -109,12 +109,16 @@ int32_t tqmoe_bank_dequant(const tqmoe_bank * bank, int64_t row0, int64_t nrows,
                            tqmoe_error * err);
 
 /* ------------------------------------------------------------------------------------------ decode products
- * Activation image the decode products read: per 32 values a scale s = amax / 16383 and q = rint(x / s) held as
- * two int8 planes (q = 128 * hi + lo, 0 <= lo < 128), so that integer dot products with the integer weight codes
- * reproduce the fp32 product to 2^-15 of the block maximum. One image row is cols * 2 bytes of planes (64 B per 32
- * values: the lo plane then the hi plane, each in the byte order of the banks' code bytes), then cols / 32 fp32 scales,
- * then cols / 32 fp32 sums of q * s; tqmoe_act_image_bytes gives the size for n rows. The image is private to the
- * library: only tqmoe_quant_act and tqmoe_expert_gateup write it, only the decode products read it. */
+ * Activation image the decode products read: x = s * q with q = rint(x / s) held as two int8 planes
+ * (q = 128 * hi + lo, 0 <= lo < 128, |q| <= 16383), so that integer dot products with the integer weight codes
+ * reproduce the fp32 product to 2^-15 of the maximum the scale was taken from. tqmoe_quant_act and the top-k kernel
+ * take one scale per row (s = amax of the row / 16383: the integer sums then run over whole 256-weight super-blocks);
+ * tqmoe_expert_gateup writes its act rows with one scale per 32 values (amax of the block / 16383). Either way the
+ * row stores a scale and a sum for every block. One image row is cols * 2 bytes of planes (64 B per 32 values: the hi
+ * plane then the lo plane, each in the byte order of the banks' code bytes), then cols / 32 fp32 scales, then
+ * cols / 32 fp32 sums of q * s; tqmoe_act_image_bytes gives the size for n rows. The image is private to the library:
+ * only tqmoe_quant_act, the top-k kernel of tqmoe_layer_forward and tqmoe_expert_gateup write it, only the decode
+ * products read it. */
 size_t  tqmoe_act_image_bytes(int32_t n, int32_t cols);
 int32_t tqmoe_quant_act(const void * x, uint32_t xtype, int32_t n, int32_t cols, void * image, void * stream,
                         tqmoe_error * err);

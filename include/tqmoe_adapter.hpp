@@ -125,10 +125,29 @@ struct ExpertFormat {
         return true;
     }
     // expert_gemm_gateup (weight_format.hpp:57-59) on int8 rows; y [assignments][rows] half
-    static bool expert_gemm_gateup(const tqmoe_bank & g, const tqmoe_bank & u, const int8_t * xq, const float * xs, void * y_f16, const int * counts,
+    static bool expert_gemm_gateup_i8(const tqmoe_bank & g, const tqmoe_bank & u, const int8_t * xq, const float * xs, void * y_f16, const int * counts,
                                    const int * offsets, const int * perm, int n, int topk, void * stream) {
         tqmoe_error e = fresh();
         const int32_t rc = tqmoe_expert_gemm_gateup_i8(&g, &u, xq, xs, counts, offsets, perm, n, topk, topk, 0, y_f16, stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
+    // expert_gemm (weight_format.hpp:51-53) for any bank format: half input rows [n][cols] (or one row per assignment with
+    // per_expert_input), y [n * topk][rows] half. Weights are decoded to fp16 tiles on the fly; fp32 accumulation.
+    static bool expert_gemm(const tqmoe_bank & m, const void * x_f16, void * y_f16, const int * counts, const int * offsets, const int * perm, int n, int topk,
+                            bool per_expert_input, void * stream) {
+        tqmoe_error e = fresh();
+        const int32_t rc = tqmoe_expert_gemm(&m, x_f16, TQMOE_F16, counts, offsets, perm, n, topk, topk, 0, per_expert_input ? 1 : 0, y_f16, TQMOE_F16, stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
+    // expert_gemm_gateup (weight_format.hpp:57-59) for any bank format on half input rows; act [n * topk][rows] half
+    static bool expert_gemm_gateup(const tqmoe_bank & g, const tqmoe_bank & u, const void * x_f16, void * act_f16, const int * counts, const int * offsets,
+                                   const int * perm, int n, int topk, void * stream) {
+        tqmoe_error e = fresh();
+        const int32_t rc = tqmoe_expert_gemm_gateup(&g, &u, x_f16, TQMOE_F16, counts, offsets, perm, n, topk, topk, 0, act_f16, stream, &e);
         if (rc == TQMOE_E_UNSUPPORTED) return false;
         check(rc, e);
         return true;

@@ -6,7 +6,8 @@
 //              (natural dword d = values 4d .. 4d + 3), so that the 16 bytes [16 g, 16 g + 16) are exactly the values
 //              {8g .. 8g + 7} and {16 + 8g .. 16 + 8g + 7}: the two halves of a sub-block that pair with code bytes
 //              8g .. 8g + 7 of a 4-bit bank (low nibbles = values 0..15, high nibbles = values 16..31);
-//   [S] fp32   scale of each sub-block (amax / 16383);
+//   [S] fp32   scale of each sub-block: amax / 16383 of the block, or of the whole row (every entry the same) for the
+//              rows quantise_row_wave writes;
 //   [S] fp32   sum of the sub-block's q times its scale (the term a per-block minimum multiplies).
 #pragma once
 #include "common.cuh"

@@ -221,10 +221,10 @@ void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0
     // is bound by the latency of one wave's chain), fewer when the batch has the waves anyway (a longer chain per
     // wave streams with its loads one super-block ahead and saves the cross-wave sums).
     const int64_t units = int64_t(A) * tiles;
-    const int cap = units >= 8192 ? 1 : units >= 2048 ? 2 : kMaxWaves;
+    const int cap = units >= 8192 ? 1 : units >= 2048 ? 2 : units >= 512 ? 4 : kMaxWaves;
     int wk = 1;
     for (int w = 1; w <= kMaxWaves && w <= cap; ++w) if (NSB % w == 0) wk = w;
-    const int waves = wk >= 4 ? kMaxWaves : 4;                            // per block
+    const int waves = wk == kMaxWaves ? kMaxWaves : 4;                    // per block: small blocks, a compute unit holds several and their phases interleave
     int tpw = waves / wk;                                                 // row tiles per block
     if (tpw > tiles) tpw = tiles;
     const dim3 grid(unsigned((tiles + tpw - 1) / tpw), unsigned(A));

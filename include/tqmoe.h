@@ -74,7 +74,8 @@ int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets,
  * tqmoe_bank_load (the counterpart of WeightFormat::load, weight_format.hpp:41, and of the loaders in
  * src/formats/weight/q4.cpp:295-326, 495-530, 577-606, 802-836). Per 32 weights of a row (a sub-block):
  *   IQ4_XS  codes 16 B: byte j = weights j (low nibble) and j + 16 (high) of the sub-block (GGUF order);
- *           aux 8 B per 256 weights: d (f16), scales_h (u16), scales_l[4]. Rows are stored in tiles of 32: the 16 B
+ *           aux 8 B per 256 weights: GGUF's d (f16), scales_h, scales_l[4] repacked (the eight 6-bit scales minus 32 as
+ *           signed 6-bit fields, d in the 16 bits between them). Rows are stored in tiles of 32: the 16 B
  *           of sub-block s of the 32 rows of a tile are contiguous (512 B), tiles of a row group follow each other by
  *           sub-block, and the 8 B records likewise (256 B per tile and super-block); rows must be a multiple of 32.
  *           The other formats are row-major (codes of a row contiguous, then its records).

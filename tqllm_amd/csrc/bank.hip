@@ -35,7 +35,8 @@ __global__ __launch_bounds__(256) void load_k(uint32_t type, const uint8_t * __r
             pack_sub(codes + iq4xs_code_offset(row, S, s), [&](int j) { return j < 16 ? q[j] & 15 : q[j - 16] >> 4; });
             if ((s & 7) == 0) {
                 uint8_t * a = aux + iq4xs_aux_offset(row, S, s / 8);
-                *reinterpret_cast<uint2 *>(a) = make_uint2(rd_u32(blk), rd_u32(blk + 4));
+                const uint32_t head = rd_u32(blk);
+                *reinterpret_cast<uint2 *>(a) = iq4xs_pack_rec(head & 0xFFFFu, head >> 16, rd_u32(blk + 4));
             }
             break;
         }

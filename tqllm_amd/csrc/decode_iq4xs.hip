@@ -62,17 +62,25 @@ __device__ __forceinline__ int chunk_up(const int * __restrict__ ids, int A, int
 }
 
 // 16 four-bit codes (two dwords) -> operand B of the MFMA: the lookups of lookup16(). The selector of the third pick
-// is (bit 3 of the code at bit 2) | byte position, written as a bit-field insert so that it is one instruction.
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) { return (x & mask) | (bits & ~mask); }
-__device__ __forceinline__ v4i decode16(uint2 c, uint32_t pos) {
+// is (bit 3 of the code at bit 2) | byte position: one v_and_or_b32 when the mask and the positions sit in registers
+// (k4 in a vector register, pos in a scalar one; as literals the instruction cannot encode them and the compiler
+// splits it in two).
+struct NibbleConsts { uint32_t k4, pos; };
+__device__ __forceinline__ NibbleConsts nibble_consts() {
+    NibbleConsts c{0x04040404u, 0x03020100u};
+    asm volatile("" : "+v"(c.k4));
+    asm volatile("" : "+s"(c.pos));
+    return c;
+}
+__device__ __forceinline__ v4i decode16(uint2 c, NibbleConsts nc) {
     v4i w;
-    const uint32_t k7 = 0x07070707u, k4 = 0x04040404u;
+    const uint32_t k7 = 0x07070707u;
     const uint32_t x0 = c.x, x1 = c.y;
     const uint32_t i0 = x0 & k7, j0 = (x0 >> 4) & k7, i1 = x1 & k7, j1 = (x1 >> 4) & k7;
-    w[0] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, i0), __builtin_amdgcn_perm(kIq4T1, kIq4T0, i0), and_or(x0 >> 1, k4, pos)));
-    w[1] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, j0), __builtin_amdgcn_perm(kIq4T1, kIq4T0, j0), and_or(x0 >> 5, k4, pos)));
-    w[2] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, i1), __builtin_amdgcn_perm(kIq4T1, kIq4T0, i1), and_or(x1 >> 1, k4, pos)));
-    w[3] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, j1), __builtin_amdgcn_perm(kIq4T1, kIq4T0, j1), and_or(x1 >> 5, k4, pos)));
+    w[0] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, i0), __builtin_amdgcn_perm(kIq4T1, kIq4T0, i0), ((x0 >> 1) & nc.k4) | nc.pos));
+    w[1] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, j0), __builtin_amdgcn_perm(kIq4T1, kIq4T0, j0), ((x0 >> 5) & nc.k4) | nc.pos));
+    w[2] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, i1), __builtin_amdgcn_perm(kIq4T1, kIq4T0, i1), ((x1 >> 1) & nc.k4) | nc.pos));
+    w[3] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(kIq4T3, kIq4T2, j1), __builtin_amdgcn_perm(kIq4T1, kIq4T0, j1), ((x1 >> 5) & nc.k4) | nc.pos));
     return w;
 }
 
@@ -121,7 +129,7 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
         const float * sc0 = image_scales(image_row_ptr(image, max(t0, 0) / xdiv, S), S);
         const float * sc1 = image_scales(image_row_ptr(image, max(t1, 0) / xdiv, S), S);
         const int64_t tile_g = int64_t(e) * tiles + tile;
-        const uint32_t pos = 0x03020100u;
+        const NibbleConsts pos = nibble_consts();
         const int sb_end = s_end / 8;   // whole super-blocks only (the launcher checks)
         // The weight bytes of a super-block: 8 bytes of codes per sub-block and the row's scale record, per lane, in
         // registers. The next super-block's are loaded before this one is multiplied, so that with several waves per SIMD
@@ -154,7 +162,7 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
                 const uint2 rec = cur.rec[nb];
-                const float d = half_bits_to_float(uint16_t(rec.x & 0xFFFFu));
+                const float d = half_bits_to_float(iq4xs_d_bits(rec));
                 const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 int si[4] = {0, 0, 0, 0};   // (hi, lo) plane sums of the two input rows, weighted by the sub-block scales
 #pragma unroll
@@ -162,11 +170,11 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
                     const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[ib], decode16(cur.code[nb][ib], pos), zero, 0, 0, 0);
                     if constexpr (UNI) {
                         // |acc| <= 32 * 128 * 127 < 2^19 and |ls - 32| <= 32: 24-bit products, eight of them stay below 2^28
-                        const int ls = iq4xs_ls(rec, ib) - 32;
+                        const int ls = iq4xs_lsm32(rec, ib);
 #pragma unroll
                         for (int q = 0; q < 4; ++q) si[q] += __mul24(acc[q], ls);
                     } else {
-                        const float ws = d * float(iq4xs_ls(rec, ib) - 32);
+                        const float ws = d * float(iq4xs_lsm32(rec, ib));
                         accf[nb][0] += float((acc[0] << 7) + acc[1]) * (ws * xs0[ib]);
                         accf[nb][1] += float((acc[2] << 7) + acc[3]) * (ws * xs1[ib]);   // zero when that input row is not served
                     }

@@ -13,7 +13,7 @@ __device__ __forceinline__ void decode_sub32(uint32_t type, const uint8_t * __re
     switch (type) {
         case TQMOE_IQ4_XS: {
             const uint2 rec = *reinterpret_cast<const uint2 *>(aux + iq4xs_aux_offset(row, S, s / 8));
-            const float dl = __fmul_rn(half_bits_to_float(uint16_t(rec.x & 0xFFFFu)), float(iq4xs_ls(rec, ib) - 32));
+            const float dl = __fmul_rn(half_bits_to_float(iq4xs_d_bits(rec)), float(iq4xs_lsm32(rec, ib)));
             const uint4 c = *reinterpret_cast<const uint4 *>(codes + iq4xs_code_offset(row, S, s));
             const uint32_t w[4] = {c.x, c.y, c.z, c.w};
 #pragma unroll

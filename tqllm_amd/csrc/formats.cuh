@@ -71,9 +71,26 @@ __device__ __forceinline__ void q4k_scale_min(const uint32_t (&q)[3], int j, int
     else { sc = (byte(j + 4) & 15) | ((byte(j - 4) >> 6) << 4); mn = (byte(j + 4) >> 4) | ((byte(j) >> 6) << 4); }
 }
 
-// IQ4_XS: 6-bit scale of sub-block ib of a 256-weight record (d | scales_h << 16, scales_l[4])
-__device__ __forceinline__ int iq4xs_ls(uint2 rec, int ib) {
-    return int(((rec.y >> (4 * ib)) & 15u) | (((rec.x >> (16 + 2 * ib)) & 3u) << 4));
+// IQ4_XS: the 8-byte record of a 256-weight super-block as the device holds it. GGUF's (d, scales_h, scales_l[4]) is the
+// same 64 bits arranged for extraction in one instruction each: the eight 6-bit scales are stored minus 32 as signed
+// fields (what the decoder multiplies by), five in x at bits 6 ib, three in y at bits 14 + 6 (ib - 5); the fp16 d sits in
+// the 16 bits between them (x bits 30..31, y bits 0..13), which one alignbit brings to the low half.
+__host__ __device__ inline uint2 iq4xs_pack_rec(uint32_t d_bits, uint32_t scales_h, uint32_t scales_l) {
+    uint32_t x = 0, y = 0;
+    for (int ib = 0; ib < 8; ++ib) {
+        const uint32_t ls = ((scales_l >> (4 * ib)) & 15u) | (((scales_h >> (2 * ib)) & 3u) << 4);
+        const uint32_t f = (ls - 32u) & 63u;
+        if (ib < 5) x |= f << (6 * ib); else y |= f << (14 + 6 * (ib - 5));
+    }
+    x |= (d_bits & 3u) << 30;
+    y |= (d_bits >> 2) & 0x3FFFu;
+    return uint2{x, y};
 }
+// scale of sub-block ib minus 32, in [-32, 31]
+__device__ __forceinline__ int iq4xs_lsm32(uint2 rec, int ib) {
+    return ib < 5 ? __builtin_amdgcn_sbfe(int(rec.x), 6 * ib, 6) : __builtin_amdgcn_sbfe(int(rec.y), 14 + 6 * (ib - 5), 6);
+}
+__device__ __forceinline__ int iq4xs_ls(uint2 rec, int ib) { return iq4xs_lsm32(rec, ib) + 32; }
+__device__ __forceinline__ uint16_t iq4xs_d_bits(uint2 rec) { return uint16_t(__builtin_amdgcn_alignbit(rec.y, rec.x, 30) & 0xFFFFu); }
 
 }  // namespace tqmoe

@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
                 for (int j = 0; j < 2; ++j) f_code[j] = *reinterpret_cast<const uint2 *>(codes + (int64_t(sb) * 8 + 2 * mg + j) * 512);
             };
             auto decode_into = [&](int buf) {
-                d_next = half_bits_to_float(uint16_t(f_rec.x & 0xFFFFu));
+                d_next = half_bits_to_float(iq4xs_d_bits(f_rec));
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const int ib = 2 * mg + j;

@@ -121,9 +121,10 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
     for (int nb = 0; nb < NB; ++nb) accf[nb][0] = accf[nb][1] = 0.f;
 
     if (valid) {
-        // this lane's part of operand A: plane row n of the MFMA = plane (n & 1) of input row n >> 1 (zero past the rows served)
+        // this lane's part of operand A: plane row n of the MFMA = plane (n & 1) of input row n >> 1. Rows past the ones
+        // served read the first row's planes: their sums land in result rows that nobody reads.
         const int a_tok = n < 2 * kTP ? s_tok[n >> 1] : -1;
-        const uint8_t * a_row = image_row_ptr(image, max(a_tok, 0) / xdiv, S) + (n & 1) * 32 + g * 16;
+        const uint8_t * a_row = image_row_ptr(image, max(a_tok, s_tok[0]) / xdiv, S) + (n & 1) * 32 + g * 16;
         // the two input rows whose sums land in this lane half's result registers
         const int t0 = s_tok[2 * g], t1 = s_tok[2 * g + 1];
         const float * sc0 = image_scales(image_row_ptr(image, max(t0, 0) / xdiv, S), S);
@@ -150,8 +151,8 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
             if (sb + wk < sb_end) fetch(sb + wk, nxt);
             v4i areg[8];
 #pragma unroll
-            for (int ib = 0; ib < 8; ++ib) areg[ib] = a_tok >= 0 ? *reinterpret_cast<const v4i *>(a_row + (sb * 8 + ib) * 64) : v4i{0, 0, 0, 0};
-            // activation scales of the 8 sub-blocks (rows not served read row 0's: their operand A is zero anyway)
+            for (int ib = 0; ib < 8; ++ib) areg[ib] = *reinterpret_cast<const v4i *>(a_row + (sb * 8 + ib) * 64);
+            // activation scales of the 8 sub-blocks (rows not served read row 0's: nobody reads their sums)
             float xs0[8], xs1[8];
             if constexpr (!UNI) {
                 const float4 p0 = *reinterpret_cast<const float4 *>(sc0 + sb * 8), p1 = *reinterpret_cast<const float4 *>(sc0 + sb * 8 + 4);
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
                     } else {
                         const float ws = d * float(iq4xs_lsm32(rec, ib));
                         accf[nb][0] += float((acc[0] << 7) + acc[1]) * (ws * xs0[ib]);
-                        accf[nb][1] += float((acc[2] << 7) + acc[3]) * (ws * xs1[ib]);   // zero when that input row is not served
+                        accf[nb][1] += float((acc[2] << 7) + acc[3]) * (ws * xs1[ib]);
                     }
                 }
                 if constexpr (UNI) {

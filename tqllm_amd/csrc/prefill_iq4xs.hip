@@ -11,11 +11,15 @@
 // v_perm_b32. The two planes go through two MFMAs that accumulate over the whole 256-weight super-block, so the scales
 // cost no vector instruction per product; per super-block the results fold as acc += d * (64 * acc_h + acc_l) in fp32.
 //
-// Blocks. A block takes one expert, a chunk of up to kChunkTiles row tiles of its assignments (kMT per wave) and one
-// unit of weight rows: 32 rows of both banks (gate / up, SwiGLU fused) or 64 rows of one bank (down). Per super-block
-// the four waves decode the unit's weights once into a double-buffered LDS stage (two k-steps of both operands each)
-// that every wave then reads as operand B; decoding super-block i + 1 overlaps the products of super-block i, one barrier
-// per super-block. Operand A is prefetched into registers two k-steps ahead.
+// Blocks. A work item is one expert, a chunk of up to kChunkTiles row tiles of its assignments and one unit of weight
+// rows: 32 rows of both banks (gate / up, SwiGLU fused) or 64 rows of one bank (down). Resident blocks of eight waves
+// take items from counters (one per XCD, so that a chunk's rows stay in one L2). Per super-block the waves decode the
+// unit's weights once into a double-buffered LDS stage that every wave then reads as operand B (decoding super-block
+// i + 1 overlaps the products of super-block i, one barrier per super-block); a wave multiplies one row tile with the
+// weights of both operand slots, so a loaded piece of operand A (prefetched into registers a few k-steps ahead) serves
+// four products and SwiGLU pairs values the same lane holds. A chunk of a single row tile has nothing to share: every
+// wave then takes the tile against 32 weight rows of its own (four units per item), decoding straight into registers
+// with no barrier in the loop.
 #include "act_image.cuh"
 #include "decode_api.cuh"
 #include "formats.cuh"
@@ -29,9 +33,8 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kMT = 2;                       // row tiles (of 32 assignments) per wave
-constexpr int kGemmWaves = 4;
-constexpr int kChunkTiles = kMT * kGemmWaves;   // row tiles per block
+constexpr int kChunkTiles = 8;                // row tiles (of 32 assignments) per chunk
+constexpr int kPlanExperts = 1024;              // experts whose index a block keeps in LDS
 
 __device__ __forceinline__ v4i decode16(uint2 c) {
     v4i w;
@@ -80,14 +83,18 @@ __global__ __launch_bounds__(256) void quant_rows_i8_k(const void * __restrict__
 
 // Index of the grouped rows, kept behind the row scales: tile_base[e] = row tiles of the experts before e
 // (tiles_e = ceil(count_e / 32)), chunk_base[e] = chunks of kChunkTiles row tiles before e, both with a total at [experts].
-struct Plan { const int * tile_base, * chunk_base; };
+// Behind them 16 counters the product kernel hands work out with (zero between launches).
+constexpr int kPlanCounters = 16;
+struct Plan { const int * tile_base, * chunk_base; int * counters; };
 __host__ __device__ inline Plan plan_at(const float * scale, int64_t grouped_rows, int experts) {
     const int * p = reinterpret_cast<const int *>(scale + grouped_rows);
-    return Plan{p, p + experts + 1};
+    return Plan{p, p + experts + 1, const_cast<int *>(p) + 2 * (experts + 1)};
 }
 
-__global__ __launch_bounds__(64) void plan_k(const int * __restrict__ counts, int experts, int * __restrict__ tile_base, int * __restrict__ chunk_base) {
+__global__ __launch_bounds__(64) void plan_k(const int * __restrict__ counts, int experts, int * __restrict__ tile_base, int * __restrict__ chunk_base,
+                                             int * __restrict__ counters) {
     const int lane = threadIdx.x;
+    if (lane < kPlanCounters) counters[lane] = 0;
     int tbase = 0, cbase = 0;
     for (int e0 = 0; e0 < experts; e0 += 64) {
         const int e = e0 + lane;
@@ -194,12 +201,27 @@ __device__ __forceinline__ void decode_planes(uint2 c, uint4 th, uint4 tl, v4i &
     }
 }
 
+// The two ways through the kernel (a lone row tile, a shared chunk) must give a row the same bits: the fold of a
+// super-block and the epilogue are spelled with explicitly rounded operations, and the product that is converted to fp16
+// passes through an opaque register, so that no path turns multiply + convert into one mixed-precision instruction
+// (one rounding instead of two: different bits at ties).
+__device__ __forceinline__ float fold_sb(float acc, int h, int l, float d) { return __fmaf_rn(float((h << 6) + l), d, acc); }
+__device__ __forceinline__ uint16_t to_half_bits(float v) {
+    asm volatile("" : "+v"(v));
+    return __half_as_ushort(__float2half_rn(v));
+}
+__device__ __forceinline__ uint16_t swiglu_half(float g_acc, float u_acc, float sc) {
+    const float gv = __fmul_rn(g_acc, sc), uv = __fmul_rn(u_acc, sc);
+    const float den = __fadd_rn(1.f, __expf(-gv));
+    return to_half_bits(__fmul_rn(__fdiv_rn(gv, den), uv));
+}
+__device__ __forceinline__ uint16_t scaled_half(float acc, float sc) { return to_half_bits(__fmul_rn(acc, sc)); }
+
 __device__ const int8_t kIq4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
 // dynamic LDS: [2 stages][NB][plane h, l][8 sub-blocks][64 lanes] v4i of decoded weights.
-// 4 * NB waves: wave = 4 * slot + row group; a wave multiplies its kMT row tiles with the weights of its operand slot
-// (gate or up; for down the two row tiles of the unit), so that two waves share a SIMD and one's vector work and loads
-// overlap the other's products.
+// 4 * NB waves. Decoding: wave = 4 * slot + quarter decodes sub-blocks 2 quarter, 2 quarter + 1 of operand slot `slot`.
+// Products: a wave takes 2 / NB row tiles (tile `wave`, and tile wave + 4 when there is one slot) against every slot.
 template <int NB>
 __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
     constexpr int THREADS = 256 * NB;
@@ -208,8 +230,19 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
     __shared__ __attribute__((aligned(16))) uint8_t s_tab[64 * 32];   // per 6-bit scale: 16 h bytes, 16 l bytes
     __shared__ int s_asg[kChunkTiles * 32];
     __shared__ float s_scale[kChunkTiles * 32];
+    // the experts' index (chunk and tile prefix sums, counts, offsets), copied once: every item looks its expert up, and a
+    // binary search is a chain of dependent reads
+    __shared__ int s_cbase[kPlanExperts + 1], s_tbase[kPlanExperts + 1], s_cnt[kPlanExperts + 1], s_off[kPlanExperts + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
     const int mg = wave & 3, nbw = wave >> 2;     // row group, operand slot
+    const bool cached = k.experts <= kPlanExperts;
+    if (cached)
+        for (int i = tid; i <= k.experts; i += THREADS) {
+            s_cbase[i] = k.plan.chunk_base[i];
+            s_tbase[i] = k.plan.tile_base[i];
+            s_cnt[i] = i < k.experts ? k.counts[i] : 0;
+            s_off[i] = k.offsets[i];
+        }
 
     for (int i = tid; i < 64 * 16; i += THREADS) {
         const int v = int(kIq4Values[i & 15]) * ((i >> 4) - 32);
@@ -217,68 +250,167 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
         s_tab[(i >> 4) * 32 + (i & 15)] = uint8_t(hi);
         s_tab[(i >> 4) * 32 + 16 + (i & 15)] = uint8_t(lo);
     }
-    // Work items are (chunk of row tiles, unit of weight rows); the blocks of the grid walk them with the grid as stride.
-    // Items that share operand A (one chunk, all units) have indices that agree modulo 8, so that with the round-robin of
-    // blocks over the 8 XCDs (grid a multiple of 8) one XCD's L2 serves them.
-    const int n_chunks = k.plan.chunk_base[k.experts];
+    // Work items are (chunk of row tiles, unit of weight rows). Items that share operand A (one chunk, all units) have
+    // indices that agree modulo 8, and the blocks that the round-robin of blocks over the 8 XCDs puts on one XCD take the
+    // items of one residue from a counter of their own: one XCD's L2 serves a chunk's rows, and a block that finishes
+    // early takes more items. The next ticket is fetched under the current item's work. The last block to leave
+    // clears the counters for the next launch over these rows.
+    __syncthreads();
+    const int * cbase = cached ? s_cbase : k.plan.chunk_base, * tbase = cached ? s_tbase : k.plan.tile_base;
+    const int * cnts = cached ? s_cnt : k.counts, * offs = cached ? s_off : k.offsets;
+    const int n_chunks = cbase[k.experts];
     const int items_padded = (n_chunks + 7) / 8 * 8 * k.units;
     const int S = k.b0.cols / 32, NSB = S / 8, rows = k.b0.rows, tiles_w = rows / 32;
-    for (int item = int(blockIdx.x); item < items_padded; item += int(gridDim.x)) {
+    __shared__ int s_ticket;
+    int * ctr = k.plan.counters;
+    const int xcd = int(blockIdx.x) & 7;
+    int ticket = 0;
+    if (tid == 0) ticket = atomicAdd(&ctr[xcd], 1);
+    for (;;) {
+        __syncthreads();          // the previous item's epilogue has read s_asg / s_scale, the exchange space and s_ticket
+        if (tid == 0) s_ticket = ticket;
+        __syncthreads();
+        const int item = 8 * s_ticket + xcd;
+        if (item >= items_padded) break;
+        if (tid == 0) ticket = atomicAdd(&ctr[xcd], 1);
         const int unit = (item >> 3) % k.units, chunk = item / (8 * k.units) * 8 + (item & 7);
         if (chunk >= n_chunks) continue;
-        const int e = owner_of(k.plan.chunk_base, k.experts, chunk);
-        const int local = chunk - k.plan.chunk_base[e], tile_base = k.plan.tile_base[e];
-        __syncthreads();          // the previous item's epilogue has read s_asg / s_scale and the exchange space
+        const int e = owner_of(cbase, k.experts, chunk);
+        const int local = chunk - cbase[e], tile_base = tbase[e];
         const bool is_shared = e == k.shared_expert;
         // gate / up rows of the shared expert beyond its size: no products, zeros stored (the rows are quantised whole later)
         const bool dead = k.gateup && is_shared && unit * 32 >= k.shared_lim;
         const int sb_end = dead ? 0 : !k.gateup && is_shared ? k.shared_lim / 256 : NSB;
-        const int cnt = k.counts[e], tiles_e = (cnt + 31) >> 5;
+        const int cnt = cnts[e], tiles_e = (cnt + 31) >> 5;
         const int first_tile = local * kChunkTiles;                         // of this expert
         const int live_tiles = min(kChunkTiles, tiles_e - first_tile);      // of this block
+        // A chunk of one row tile has nothing for the waves to share: every wave then takes the tile against 32 weight
+        // rows of its own, four units per item, and the chunk's other item numbers are empty.
+        const bool lone = live_tiles == 1 && k.units % 4 == 0;
+        if (lone && unit >= k.units / 4) continue;
         for (int i = tid; i < kChunkTiles * 32; i += THREADS) {
             const int idx = first_tile * 32 + i;
             const bool ok = i < live_tiles * 32 && idx < cnt;
-            s_asg[i] = ok ? k.perm[k.offsets[e] + idx] : -1;
+            s_asg[i] = ok ? k.perm[offs[e] + idx] : -1;
             s_scale[i] = ok ? k.xs[int64_t(tile_base + first_tile) * 32 + i] : 0.f;
         }
         __syncthreads();
-
-        // row tiles mg and mg + 4 of the chunk: a short chunk spreads over the row groups
-        const int my_tiles = (mg < live_tiles ? 1 : 0) + (mg + 4 < live_tiles ? 1 : 0);
-        static_assert(kMT == 2 && kChunkTiles == 8, "row tile t of a wave is tile mg + 4 t of the chunk");
-        const int8_t * a_base = k.xq + int64_t(tile_base + first_tile + mg) * 32 * k.b0.cols + lane * 16;
+        if (lone) {
+            // weight tile of this wave: gate / up: tile 4 unit + mg of bank nbw; down: tile (4 unit + mg) NB + nbw
+            const int wt = k.gateup ? 4 * unit + mg : (4 * unit + mg) * NB + nbw;
+            const BankView & wbank = nbw ? k.b1 : k.b0;
+            const bool wdead = k.gateup && is_shared && wt * 32 >= k.shared_lim;
+            const int sbe = wdead ? 0 : !k.gateup && is_shared ? k.shared_lim / 256 : NSB;
+            const int64_t wtile_g = int64_t(e) * tiles_w + wt;
+            const uint8_t * wcodes = wbank.codes + wtile_g * S * 512 + n * 16 + g * 8;
+            const uint8_t * waux = wbank.aux + wtile_g * NSB * 256 + n * 8;
+            const int8_t * a_ptr = k.xq + int64_t(tile_base + first_tile) * 32 * k.b0.cols + lane * 16;
+            struct Stage { uint2 code[8]; uint2 rec; v4i a[8]; };
+            auto fetch1 = [&](int sb, Stage & st) {   // a super-block of the wave's weights and of the row tile
+                st.rec = *reinterpret_cast<const uint2 *>(waux + int64_t(sb) * 256);
+#pragma unroll
+                for (int ib = 0; ib < 8; ++ib) {
+                    st.code[ib] = *reinterpret_cast<const uint2 *>(wcodes + (int64_t(sb) * 8 + ib) * 512);
+                    st.a[ib] = *reinterpret_cast<const v4i *>(a_ptr + (int64_t(sb) * 8 + ib) * 1024);
+                }
+            };
+            float acc_f[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc_f[i] = 0.f;
+            auto work1 = [&](int sb, Stage & cur, Stage & nxt) {
+                fetch1(min(sb + 1, sbe - 1), nxt);   // past the last one the same again, from the cache: no branch, the same loads in flight on every path
+                __builtin_amdgcn_sched_barrier(0);
+                const float d = half_bits_to_float(iq4xs_d_bits(cur.rec));
+                v16i acc_h = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, acc_l = acc_h;
+#pragma unroll
+                for (int ib = 0; ib < 8; ++ib) {
+                    const uint4 * tab = reinterpret_cast<const uint4 *>(s_tab + iq4xs_ls(cur.rec, ib) * 32);
+                    v4i h, l;
+                    decode_planes(cur.code[ib], tab[0], tab[1], h, l);
+                    acc_h = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.a[ib], h, acc_h, 0, 0, 0);
+                    acc_l = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.a[ib], l, acc_l, 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc_f[i] = fold_sb(acc_f[i], acc_h[i], acc_l[i], d);
+            };
+            if (sbe > 0) {
+                Stage s0, s1;
+                fetch1(0, s0);
+                for (int sb = 0; sb < sbe; sb += 2) {
+                    work1(sb, s0, s1);
+                    if (sb + 1 < sbe) work1(sb + 1, s1, s0);
+                }
+            }
+            float * ex = reinterpret_cast<float *>(lds);
+            if (k.gateup && NB == 2) {   // the up waves hand their sums to the gate waves of the same weight tile
+                if (nbw == 1) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) ex[(mg * 16 + i) * 64 + lane] = acc_f[i];
+                }
+                __syncthreads();
+            }
+            if (!(k.gateup && NB == 2 && nbw == 1)) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int m = 8 * (i >> 2) + 4 * g + (i & 3);   // result register i of lane half g: row m of the tile, weight row n
+                    const int a = s_asg[m];
+                    if (a < 0) continue;
+                    const float sc = s_scale[m];
+                    uint16_t * o = k.out + int64_t(a) * rows;
+                    if (k.gateup) o[wt * 32 + n] = swiglu_half(acc_f[i], NB == 2 ? ex[(mg * 16 + i) * 64 + lane] : acc_f[i], sc);
+                    else o[wt * 32 + n] = scaled_half(acc_f[i], sc);
+                }
+            }
+            continue;
+        }
+        // Each wave takes 2 / NB row tiles of the chunk (tile `wave`; with one operand slot also tile wave + 4) against
+        // the weights of every operand slot: a loaded piece of operand A serves the products with gate and with up (or
+        // with both weight tiles of a down unit), and SwiGLU pairs values the same lane holds.
+        constexpr int TPW = 2 / NB;
+        const int my_tiles = NB == 2 ? (wave < live_tiles ? 1 : 0) : (wave < live_tiles ? 1 : 0) + (wave + 4 < live_tiles ? 1 : 0);
+        const int8_t * a_base = k.xq + int64_t(tile_base + first_tile + wave) * 32 * k.b0.cols + lane * 16;
         const int64_t a_tile = int64_t(4) * 32 * k.b0.cols;
 
-        // weight rows of this wave's operand slot: gate / up: the unit's 32 rows of bank nbw; down: row tile NB * unit + nbw
+        // the weights this wave decodes for everybody: sub-blocks 2 mg and 2 mg + 1 of operand slot nbw
+        // (gate / up: the unit's 32 rows of bank nbw; down: row tile NB * unit + nbw)
         const BankView & bank = nbw ? k.b1 : k.b0;
         const int64_t tile_g = int64_t(e) * tiles_w + (k.gateup ? unit : NB * unit + nbw);
         const uint8_t * codes = bank.codes + tile_g * S * 512 + n * 16 + g * 8;   // sub-block s of the tile: + 512 s; lane = (row n, code half g)
         const uint8_t * aux = bank.aux + tile_g * NSB * 256 + n * 8;              // super-block sb of the tile: + 256 sb
+        // the scales d of the rows of both slots, for the fold: lane's weight row n, slot b
+        const uint8_t * aux_b[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            aux_b[b] = (b ? k.b1 : k.b0).aux + (int64_t(e) * tiles_w + (k.gateup ? unit : NB * unit + b)) * NSB * 256 + n * 8;
 
-        // The super-block loop is instantiated per number of live row tiles of the wave (0..kMT), so that its body is one
+        // The super-block loop is instantiated per number of live row tiles of the wave (0..TPW), so that its body is one
         // straight line of code the scheduler can interleave. Every instance passes the same barriers.
         auto body = [&](auto mt_tag) {
             constexpr int MT = decltype(mt_tag)::value;
             constexpr int MTA = MT ? MT : 1;
-            v16i acc_h[MTA], acc_l[MTA];
-            float acc_f[MTA][16];
+            v16i acc_h[MTA][NB], acc_l[MTA][NB];
+            float acc_f[MTA][NB][16];
 #pragma unroll
             for (int t = 0; t < MTA; ++t)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) { acc_f[t][i] = 0.f; acc_h[t][i] = 0; acc_l[t][i] = 0; }
+                for (int b = 0; b < NB; ++b)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) { acc_f[t][b][i] = 0.f; acc_h[t][b][i] = 0; acc_l[t][b][i] = 0; }
 
-            // this wave decodes sub-blocks 2 mg and 2 mg + 1 of every super-block of its slot: the codes and the scale
-            // record are fetched one super-block before they are decoded, so that their latency is not waited for
-            float d_next = 0.f, d_cur = 0.f;
+            // the codes and the scale record are fetched one super-block before they are decoded, so that their latency is
+            // not waited for
             uint2 f_rec = {0, 0}, f_code[2] = {{0, 0}, {0, 0}};
+            uint2 d_rec[NB], d_rec_next[NB];
             auto fetch = [&](int sb) {
                 f_rec = *reinterpret_cast<const uint2 *>(aux + int64_t(sb) * 256);
 #pragma unroll
                 for (int j = 0; j < 2; ++j) f_code[j] = *reinterpret_cast<const uint2 *>(codes + (int64_t(sb) * 8 + 2 * mg + j) * 512);
             };
+            auto fetch_d = [&](int sb) {
+#pragma unroll
+                for (int b = 0; b < NB; ++b) d_rec_next[b] = *reinterpret_cast<const uint2 *>(aux_b[b] + int64_t(sb) * 256);
+            };
             auto decode_into = [&](int buf) {
-                d_next = half_bits_to_float(iq4xs_d_bits(f_rec));
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const int ib = 2 * mg + j;
@@ -302,6 +434,7 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
             const int pairs = sb_end * 4;
             if (sb_end > 0) {
                 fetch(0);
+                fetch_d(0);
 #pragma unroll
                 for (int q = 0; q < kSlots - 1; ++q) load_a(q, min(q, pairs - 1));
                 decode_into(0);
@@ -310,74 +443,80 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
             __syncthreads();
             for (int sb = 0; sb < sb_end; ++sb) {
                 const int buf = sb & 1;
-                d_cur = d_next;
+#pragma unroll
+                for (int b = 0; b < NB; ++b) d_rec[b] = d_rec_next[b];
                 // past the last super-block the fetch repeats it and the decode fills the stage nobody reads: no branches here
                 decode_into(buf ^ 1);
                 fetch(min(sb + 2, sb_end - 1));
+                fetch_d(min(sb + 1, sb_end - 1));
 #pragma unroll
                 for (int jp = 0; jp < 4; ++jp) {
                     load_a((jp + kSlots - 1) % kSlots, min(sb * 4 + jp + kSlots - 1, pairs - 1));
 #pragma unroll
                     for (int h = 0; h < 2; ++h) {
                         const int ib = 2 * jp + h;
-                        const v4i bh = bs[(((buf * NB + nbw) * 2 + 0) * 8 + ib) * 64 + lane];
-                        const v4i bl = bs[(((buf * NB + nbw) * 2 + 1) * 8 + ib) * 64 + lane];
 #pragma unroll
-                        for (int t = 0; t < MT; ++t) {
-                            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                            acc_h[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp % kSlots][t][h], bh, ib ? acc_h[t] : zero, 0, 0, 0);
-                            acc_l[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp % kSlots][t][h], bl, ib ? acc_l[t] : zero, 0, 0, 0);
+                        for (int b = 0; b < NB; ++b) {
+                            const v4i bh = bs[(((buf * NB + b) * 2 + 0) * 8 + ib) * 64 + lane];
+                            const v4i bl = bs[(((buf * NB + b) * 2 + 1) * 8 + ib) * 64 + lane];
+#pragma unroll
+                            for (int t = 0; t < MT; ++t) {
+                                const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                                acc_h[t][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp % kSlots][t][h], bh, ib ? acc_h[t][b] : zero, 0, 0, 0);
+                                acc_l[t][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp % kSlots][t][h], bl, ib ? acc_l[t][b] : zero, 0, 0, 0);
+                            }
                         }
                     }
                 }
                 // |64 acc_h + acc_l| <= 256 * 127 * 127 * 32 < 2^28: exact in int32, then one rounding into fp32
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) acc_f[t][i] += float((acc_h[t][i] << 6) + acc_l[t][i]) * d_cur;
-                __syncthreads();
-            }
-            // result register i of lane half g is tile row 8 (i / 4) + 4 g + i % 4, weight row n.
-            // gate / up: the up waves hand their sums to the gate waves of the same rows through the (now idle) weight stage.
-            float * ex = reinterpret_cast<float *>(lds);
-            if (k.gateup && NB == 2) {
-                if (nbw == 1) {
+                for (int b = 0; b < NB; ++b) {
+                    const float d = half_bits_to_float(iq4xs_d_bits(d_rec[b]));
 #pragma unroll
                     for (int t = 0; t < MT; ++t)
 #pragma unroll
-                        for (int i = 0; i < 16; ++i) ex[((mg * kMT + t) * 16 + i) * 64 + lane] = acc_f[t][i];
+                        for (int i = 0; i < 16; ++i) acc_f[t][b][i] = fold_sb(acc_f[t][b][i], acc_h[t][b][i], acc_l[t][b][i], d);
                 }
                 __syncthreads();
-                if (nbw == 1) return;
             }
+            // result register i of lane half g is tile row 8 (i / 4) + 4 g + i % 4, weight row n
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const int m = (mg + 4 * t) * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                    const int m = (wave + 4 * t) * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
                     const int a = s_asg[m];
                     if (a < 0) continue;
                     const float sc = s_scale[m];
                     uint16_t * o = k.out + int64_t(a) * rows;
                     if (k.gateup) {
-                        const float gv = acc_f[t][i] * sc, uv = (NB == 2 ? ex[((mg * kMT + t) * 16 + i) * 64 + lane] : acc_f[t][i]) * sc;
-                        o[unit * 32 + n] = __half_as_ushort(__float2half_rn(gv / (1.f + expf(-gv)) * uv));
+                        o[unit * 32 + n] = swiglu_half(acc_f[t][0][i], acc_f[t][NB - 1][i], sc);
                     } else {
-                        o[(NB * unit + nbw) * 32 + n] = __half_as_ushort(__float2half_rn(acc_f[t][i] * sc));
+#pragma unroll
+                        for (int b = 0; b < NB; ++b) o[(NB * unit + b) * 32 + n] = scaled_half(acc_f[t][b][i], sc);
                     }
                 }
             }
         };
-        static_assert(kMT == 2, "the dispatch below lists the instances");
-        switch (my_tiles) {
-            case 0: body(std::integral_constant<int, 0>{}); break;
-            case 1: body(std::integral_constant<int, 1>{}); break;
-            default: body(std::integral_constant<int, 2>{}); break;
+        if constexpr (NB == 2) {
+            if (my_tiles) body(std::integral_constant<int, 1>{}); else body(std::integral_constant<int, 0>{});
+        } else {
+            switch (my_tiles) {
+                case 0: body(std::integral_constant<int, 0>{}); break;
+                case 1: body(std::integral_constant<int, 1>{}); break;
+                default: body(std::integral_constant<int, 2>{}); break;
+            }
         }
     }   // items
+    if (tid == 0) {
+        __threadfence();
+        if (atomicAdd(&ctr[8], 1) == int(gridDim.x) - 1)
+            for (int i = 0; i < kPlanCounters; ++i) atomicExch(&ctr[i], 0);
+    }
 }
 
 }  // namespace
+
 
 // ---------------------------------------------------------------------------------------------- entry helpers
 int64_t grouped_row_tiles(int64_t assignments, int experts) { return (assignments + 31) / 32 + experts; }
@@ -392,13 +531,13 @@ int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int 
     return 0;
 }
 
-int64_t grouped_scale_words(int64_t assignments, int experts) { return grouped_row_tiles(assignments, experts) * 32 + 2 * (int64_t(experts) + 1); }
+int64_t grouped_scale_words(int64_t assignments, int experts) { return grouped_row_tiles(assignments, experts) * 32 + 2 * (int64_t(experts) + 1) + kPlanCounters; }
 
 int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
                               int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s) {
     const int64_t tiles = grouped_row_tiles(assignments, experts);
     const Plan plan = plan_at(scale, tiles * 32, experts);
-    plan_k<<<1, 64, 0, s>>>(counts, experts, const_cast<int *>(plan.tile_base), const_cast<int *>(plan.chunk_base));
+    plan_k<<<1, 64, 0, s>>>(counts, experts, const_cast<int *>(plan.tile_base), const_cast<int *>(plan.chunk_base), plan.counters);
     const unsigned blocks = unsigned(tiles * 4);
     switch (xtype) {
         case TQMOE_F32: group_rows_i8_k<TQMOE_F32><<<blocks, 256, 0, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan); break;

@@ -180,6 +180,13 @@ template <int R, int XT>
 __global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logits, TopkOut o, int e, int k, float scale) {
     const int token = blockIdx.x, lane = threadIdx.x;
     const float * x = logits + int64_t(token) * (e + 1);
+    // the input row's block of this lane (rows of up to 64 blocks: one per lane) is loaded now and quantised at the end, so
+    // that its latency passes under the selection
+    const int S = o.image ? o.cols / 32 : 0;
+    const bool row_in_regs = S > 0 && S <= 64;
+    float xv[32];
+    if (row_in_regs && lane < S) load_block32<XT>(o.x, int64_t(token) * o.cols + 32 * lane, xv);
+    const float shared_logit = o.shared_weights ? x[e] : 0.f;
     float p[R];
     float m = -INFINITY;
 #pragma unroll
@@ -191,7 +198,8 @@ __global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logi
     sum = wave_sum_all(sum);
 #pragma unroll
     for (int r = 0; r < R; ++r) p[r] = lane + 64 * r < e ? p[r] / sum : -2.f;   // entries past the end never win
-    float selected = 0.f;
+    float selected = 0.f, my_w = 0.f;   // lane s keeps selection s
+    int my_id = 0;
     for (int s = 0; s < k; ++s) {
         float bv = p[0];
         int bi = lane;
@@ -199,17 +207,49 @@ __global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logi
         for (int r = 1; r < R; ++r) if (p[r] > bv) { bv = p[r]; bi = lane + 64 * r; }   // strict: the lowest index of equal values
         const float top = wave_max_all(bv);
         const int best = wave_min_all(bv == top ? bi : 0x7FFFFFFF);
-        if (lane == 0) {
-            o.ids[int64_t(token) * k + s] = best;
-            o.weights[int64_t(token) * k + s] = top;
-            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + s] = best;
+        if (lane == (s & 63)) { my_id = best; my_w = top; }
+        if (k > 64 && (s & 63) == 63) {   // more selections than lanes: a full set goes out before the lanes are reused
+            o.ids[int64_t(token) * k + s - 63 + lane] = my_id;
+            o.weights[int64_t(token) * k + s - 63 + lane] = my_w;   // divided below
+            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + s - 63 + lane] = my_id;
         }
         selected += top;                       // slot order, as the host sums the selected weights
 #pragma unroll
         for (int r = 0; r < R; ++r) if (lane + 64 * r == best) p[r] = -1.f;
     }
-    topk_finish(o, x, token, lane, e, k, scale, selected);
-    if (o.image) topk_quantise_row<XT>(o, token, lane);
+    if (k <= 64) {
+        // the host divides by the clamped sum, then multiplies by the scale
+        const float total = fmaxf(selected, 6.103515625e-5f);
+        if (lane < k) {
+            float v = my_w / total;
+            if (scale != 0.f && scale != 1.f) v *= scale;
+            o.ids[int64_t(token) * k + lane] = my_id;
+            o.weights[int64_t(token) * k + lane] = v;
+            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + lane] = my_id;
+        }
+        if (lane == 0) {
+            if (o.shared_weights) o.shared_weights[token] = 1.f / (1.f + expf(-shared_logit));
+            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + k] = o.extra;
+        }
+    } else {
+        const int done = k & ~63;             // the last partial set
+        if (lane < k - done) {
+            o.ids[int64_t(token) * k + done + lane] = my_id;
+            o.weights[int64_t(token) * k + done + lane] = my_w;
+            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + done + lane] = my_id;
+        }
+        __threadfence_block();
+        topk_finish(o, x, token, lane, e, k, scale, selected);
+    }
+    if (o.image) {
+        if (row_in_regs) {
+            uint8_t * image_row = o.image + int64_t(token) * S * kImageSubBytes;
+            const float amax = wave_max(lane < S ? block_amax(xv) : 0.f);
+            if (lane < S) quantise_block(xv, image_row, S, lane, amax);
+        } else {
+            topk_quantise_row<XT>(o, token, lane);
+        }
+    }
 }
 
 template <int XT>

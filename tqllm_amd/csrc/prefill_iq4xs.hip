@@ -350,15 +350,20 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
                 __syncthreads();
             }
             if (!(k.gateup && NB == 2 && nbw == 1)) {
+                int asg[16];
+                float scl[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int m = 8 * (i >> 2) + 4 * g + (i & 3);   // result register i of lane half g: row m of the tile, weight row n
-                    const int a = s_asg[m];
-                    if (a < 0) continue;
-                    const float sc = s_scale[m];
-                    uint16_t * o = k.out + int64_t(a) * rows;
-                    if (k.gateup) o[wt * 32 + n] = swiglu_half(acc_f[i], NB == 2 ? ex[(mg * 16 + i) * 64 + lane] : acc_f[i], sc);
-                    else o[wt * 32 + n] = scaled_half(acc_f[i], sc);
+                    asg[i] = s_asg[m];
+                    scl[i] = s_scale[m];
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    if (asg[i] < 0) continue;
+                    uint16_t * o = k.out + int64_t(asg[i]) * rows;
+                    if (k.gateup) o[wt * 32 + n] = swiglu_half(acc_f[i], NB == 2 ? ex[(mg * 16 + i) * 64 + lane] : acc_f[i], scl[i]);
+                    else o[wt * 32 + n] = scaled_half(acc_f[i], scl[i]);
                 }
             }
             continue;
@@ -479,21 +484,27 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
                 }
                 __syncthreads();
             }
-            // result register i of lane half g is tile row 8 (i / 4) + 4 g + i % 4, weight row n
+            // result register i of lane half g is tile row 8 (i / 4) + 4 g + i % 4, weight row n. The rows' assignments and
+            // scales are read first, all at once: a read per element inside the store loop would serialise on LDS latency.
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
+                int asg[16];
+                float scl[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int m = (wave + 4 * t) * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-                    const int a = s_asg[m];
-                    if (a < 0) continue;
-                    const float sc = s_scale[m];
-                    uint16_t * o = k.out + int64_t(a) * rows;
+                    asg[i] = s_asg[m];
+                    scl[i] = s_scale[m];
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    if (asg[i] < 0) continue;
+                    uint16_t * o = k.out + int64_t(asg[i]) * rows;
                     if (k.gateup) {
-                        o[unit * 32 + n] = swiglu_half(acc_f[t][0][i], acc_f[t][NB - 1][i], sc);
+                        o[unit * 32 + n] = swiglu_half(acc_f[t][0][i], acc_f[t][NB - 1][i], scl[i]);
                     } else {
 #pragma unroll
-                        for (int b = 0; b < NB; ++b) o[(NB * unit + b) * 32 + n] = scaled_half(acc_f[t][b][i], sc);
+                        for (int b = 0; b < NB; ++b) o[(NB * unit + b) * 32 + n] = scaled_half(acc_f[t][b][i], scl[i]);
                     }
                 }
             }

@@ -187,6 +187,9 @@ int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float *
  * the library. xdiv = slots for the layer input (row = token), 1 for
  * rows that exist per assignment. This is the step the reference does with mmq_quantize_act_rows
  * (src/experts/mmq_experts.cu:79-95: quantise and arrange the rows of every expert tile).
+ * tqmoe_gather_rows_i8: the arranging alone, from rows tqmoe_quant_rows_i8 has quantised (rows_q [rows][cols], rows_scale
+ * [rows]): the same q / scale as tqmoe_group_rows_i8 on the unquantised rows, bit for bit, with every input row
+ * quantised once however many assignments read it (the layer input: xdiv = slots).
  * tqmoe_expert_gemm_gateup_i8: act[a] = silu(gate_e x) * (up_e x) as fp16 [n * slots][gate->rows] for every listed
  * assignment a = t * slots + s. WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59) with the int8 operands of
  * expert_gemm_i8 (weight_format.hpp:54-56).
@@ -202,6 +205,9 @@ int64_t tqmoe_grouped_scale_words(int64_t assignments, int32_t experts);
 int32_t tqmoe_group_rows_i8(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets,
                             const int32_t * perm, int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q,
                             float * scale, void * stream, tqmoe_error * err);
+int32_t tqmoe_gather_rows_i8(const int8_t * rows_q, const float * rows_scale, int32_t cols, const int32_t * counts,
+                             const int32_t * offsets, const int32_t * perm, int32_t experts, int64_t assignments,
+                             int32_t xdiv, int8_t * q, float * scale, void * stream, tqmoe_error * err);
 int32_t tqmoe_expert_gemm_gateup_i8(const tqmoe_bank * gate, const tqmoe_bank * up, const int8_t * xq, const float * xs,
                                     const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t n,
                                     int32_t slots, int32_t topk, int32_t shared_lim, void * act_f16, void * stream,

@@ -143,6 +143,27 @@ def test_grouped_products_skip_negative_ids(tq, oracle):
     assert act[flat >= 0].any(axis=1).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_gather_of_quantised_rows_equals_group_rows(tq, dtype):
+    """Quantising every input row once and gathering gives the grouped operand of the one-step kernel bit for bit (rows of
+    the padding are left as allocated by both: zeros here), with skipped assignments and a ragged expert."""
+    experts, hidden, n, slots = 9, 768, 75, 3
+    rng = np.random.default_rng(11)
+    ids = rng.integers(0, experts, size=(n, slots)).astype(np.int32)
+    ids[rng.random((n, slots)) < 0.1] = -1
+    x = torch.randn(n, hidden, device="cuda", dtype=dtype)
+    x[7] = 0          # a zero row: scale 0
+    counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), experts)
+    lists = (counts, offsets, perm)
+    q1, s1 = tq.group_rows_i8(x, lists, n * slots, slots)
+    rq, rs = tq.quant_rows_i8(x)
+    q2, s2 = tq.gather_rows_i8(rq, rs, lists, n * slots, slots)
+    assert torch.equal(q1, q2)
+    rows = q1.shape[0]
+    assert torch.equal(s1[:rows], s2[:rows])
+    assert torch.equal(s1[rows:].view(torch.int32), s2[rows:].view(torch.int32))      # the tile index behind the scales
+
+
 def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0)):
     raws = synth.make_banks(cfg, seed=seed, distinct=distinct)
     gate, up, down = banks_on_device(cfg, raws)

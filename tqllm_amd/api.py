@@ -80,6 +80,7 @@ def lib():
         l.tqmoe_grouped_scale_words.restype = i64
         l.tqmoe_grouped_scale_words.argtypes = [i64, i32]
         l.tqmoe_group_rows_i8.argtypes = [p, u32, i32, p, p, p, i32, i64, i32, p, p, p, e]
+        l.tqmoe_gather_rows_i8.argtypes = [p, p, i32, p, p, p, i32, i64, i32, p, p, p, e]
         l.tqmoe_expert_gemm_gateup_i8.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_expert_gemm_i8.argtypes = [C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_expert_gemm_gateup.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, u32, p, p, p, i32, i32, i32, i32, p, p, e]
@@ -305,6 +306,20 @@ def group_rows_i8(x, lists, assignments, xdiv):
     err = _err()
     _check(lib().tqmoe_group_rows_i8(_ptr(x), _ttype(x), cols, _ptr(counts), _ptr(offsets), _ptr(perm), counts.numel(), assignments, xdiv, _ptr(q),
                                      _ptr(scale), _stream(x), C.byref(err)), err)
+    return q, scale
+
+
+def gather_rows_i8(rows_q, rows_scale, lists, assignments, xdiv):
+    """The arranging step of group_rows_i8 alone, from rows quant_rows_i8 has quantised: the same (q, scale), every input row
+    quantised once however many assignments read it."""
+    counts, offsets, perm = lists
+    cols = rows_q.shape[1]
+    rows = lib().tqmoe_grouped_rows(assignments, counts.numel())
+    q = torch.zeros((rows, cols), dtype=torch.int8, device=rows_q.device)
+    scale = torch.zeros(lib().tqmoe_grouped_scale_words(assignments, counts.numel()), dtype=torch.float32, device=rows_q.device)
+    err = _err()
+    _check(lib().tqmoe_gather_rows_i8(_ptr(rows_q), _ptr(rows_scale), cols, _ptr(counts), _ptr(offsets), _ptr(perm), counts.numel(), assignments, xdiv,
+                                      _ptr(q), _ptr(scale), _stream(rows_q), C.byref(err)), err)
     return q, scale
 
 

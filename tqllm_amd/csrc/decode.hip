@@ -10,6 +10,8 @@ int32_t enqueue_gemm_f16(const tqmoe_bank & b0, const tqmoe_bank * b1, const voi
                          int experts, int64_t assignments, int xdiv, void * out, int out_f32, int gateup, int shared_expert, int shared_lim, hipStream_t s);
 int64_t grouped_row_tiles(int64_t assignments, int experts);
 int64_t grouped_scale_words(int64_t assignments, int experts);
+int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, const int * counts, const int * offsets, const int * perm, int experts,
+                               int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s);
 int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
                               int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s);
 int32_t enqueue_iq4xs_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
@@ -236,6 +238,17 @@ extern "C" int32_t tqmoe_group_rows_i8(const void * x, uint32_t xtype, int32_t c
     if (int32_t rc = need_device(err, "tqmoe_group_rows_i8")) return rc;
     enqueue_group_rows_i8(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, static_cast<hipStream_t>(stream));
     return launched(err, "tqmoe_group_rows_i8");
+}
+
+extern "C" int32_t tqmoe_gather_rows_i8(const int8_t * rows_q, const float * rows_scale, int32_t cols, const int32_t * counts, const int32_t * offsets,
+                                        const int32_t * perm, int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q, float * scale, void * stream,
+                                        tqmoe_error * err) {
+    if (!rows_q || !rows_scale || !counts || !offsets || !perm || !q || !scale || cols <= 0 || cols % 32 || experts <= 0 || experts > 4096 || assignments <= 0 ||
+        xdiv <= 0 || grouped_row_tiles(assignments, experts) > 0x7FFFFFFF)
+        return fail(err, TQMOE_E_ARG, "tqmoe_gather_rows_i8: invalid shape or pointer");
+    if (int32_t rc = need_device(err, "tqmoe_gather_rows_i8")) return rc;
+    enqueue_gather_rows_i8(rows_q, rows_scale, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, static_cast<hipStream_t>(stream));
+    return launched(err, "tqmoe_gather_rows_i8");
 }
 
 static int32_t gemm_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,

@@ -21,7 +21,7 @@ struct Plan {  // byte offsets into the workspace
     int chunk;   // tokens per pass of the expert stages
     size_t logits, ids, weights, shared_w, ids_ext, total;
     size_t ximage, aimage, y;                                                // decode path
-    size_t xq, xs, counts, offsets, perm, dispatch_ws, act16, aq, as, y16;   // grouped path
+    size_t xq, xs, counts, offsets, perm, dispatch_ws, act16, aq, as, y16, rq, rs;   // grouped path
 };
 
 bool int8_ok(const tqmoe_layer & L) { return L.gate.type == TQMOE_IQ4_XS && (!L.has_shared || L.shared_ff % 256 == 0); }
@@ -60,6 +60,8 @@ Plan plan_for(const tqmoe_layer & L, int n) {
         p.xs = take(gwords * 4);
         p.aq = take(grows * L.ff);
         p.as = take(gwords * 4);
+        p.rq = take(c * L.hidden);        // the chunk's input rows as int8, quantised once, then gathered per assignment
+        p.rs = take(c * 4);
     } else if (!p.grouped) {
         p.ximage = take(tqmoe_act_image_bytes(n, L.hidden));
         p.aimage = take(tqmoe_act_image_bytes(int32_t(a), L.ff));
@@ -147,8 +149,10 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
                                                        L.hidden, L.topk, c, stream, err)) return rc;
                 continue;
             } else {
-            if (int32_t rc = tqmoe_group_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq,
-                                                 xs, stream, err)) return rc;
+            int8_t * rq = reinterpret_cast<int8_t *>(ws + p.rq);
+            float * rs = reinterpret_cast<float *>(ws + p.rs);
+            if (int32_t rc = tqmoe_quant_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, rq, rs, stream, err)) return rc;
+            if (int32_t rc = tqmoe_gather_rows_i8(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_gateup_i8(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
             if (int32_t rc = tqmoe_group_rows_i8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_i8(&L.down, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;

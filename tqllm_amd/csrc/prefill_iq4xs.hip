@@ -169,6 +169,27 @@ __global__ __launch_bounds__(256) void group_rows_i8_k(const void * __restrict__
     }
 }
 
+// The same grouped operand from rows that are already int8 (quant_rows_i8_k's output: one scale per row, the bytes of every
+// 32-block in operand order): a pure copy. One block per row tile; lane (g, r) of every wave moves the 16 bytes of row r,
+// half g of one k-step at a time, so each k-step's 1 KB is written by one fully coalesced store. When several
+// assignments read one input row (xdiv > 1) the row is quantised once instead of once per assignment.
+__global__ __launch_bounds__(256) void gather_rows_i8_k(const int8_t * __restrict__ rq, const float * __restrict__ rs, int cols, const int * __restrict__ counts,
+                                                          const int * __restrict__ offsets, const int * __restrict__ perm, int experts, int xdiv,
+                                                          int8_t * __restrict__ q, float * __restrict__ scale, Plan plan) {
+    const int tile_index = int(blockIdx.x);
+    if (tile_index >= plan.tile_base[experts]) return;
+    const int e = owner_of(plan.tile_base, experts, tile_index);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, g = lane >> 5;
+    const int i = (tile_index - plan.tile_base[e]) * 32 + r;
+    if (i >= counts[e]) return;                       // rows past the expert's count are left as they are
+    const int64_t row = perm[offsets[e] + i] / xdiv;
+    if (wave == 0 && g == 0) scale[int64_t(tile_index) * 32 + r] = rs[row];
+    const uint4 * src = reinterpret_cast<const uint4 *>(rq + row * cols) + g;
+    uint4 * dst = reinterpret_cast<uint4 *>(q + int64_t(tile_index) * 32 * cols) + lane;
+    const int S = cols / 32;
+    for (int ks = wave; ks < S; ks += 4) dst[ks * 64] = src[ks * 2];
+}
+
 struct Where { int expert, local, tile_base; };
 
 struct GemmArgs {
@@ -555,6 +576,15 @@ int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const in
         case TQMOE_F16: group_rows_i8_k<TQMOE_F16><<<blocks, 256, 0, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan); break;
         default: group_rows_i8_k<TQMOE_BF16><<<blocks, 256, 0, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan); break;
     }
+    return 0;
+}
+
+int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, const int * counts, const int * offsets, const int * perm, int experts,
+                               int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s) {
+    const int64_t tiles = grouped_row_tiles(assignments, experts);
+    const Plan plan = plan_at(scale, tiles * 32, experts);
+    plan_k<<<1, 64, 0, s>>>(counts, experts, const_cast<int *>(plan.tile_base), const_cast<int *>(plan.chunk_base), plan.counters);
+    gather_rows_i8_k<<<unsigned(tiles), 256, 0, s>>>(rq, rs, cols, counts, offsets, perm, experts, xdiv, q, scale, plan);
     return 0;
 }
 

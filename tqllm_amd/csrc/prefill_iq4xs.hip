@@ -436,17 +436,15 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
 #pragma unroll
                 for (int b = 0; b < NB; ++b) d_rec_next[b] = *reinterpret_cast<const uint2 *>(aux_b[b] + int64_t(sb) * 256);
             };
-            auto decode_into = [&](int buf) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int ib = 2 * mg + j;
-                    const uint4 * tab = reinterpret_cast<const uint4 *>(s_tab + iq4xs_ls(f_rec, ib) * 32);
-                    v4i h, l;
-                    decode_planes(f_code[j], tab[0], tab[1], h, l);
-                    bs[(((buf * NB + nbw) * 2 + 0) * 8 + ib) * 64 + lane] = h;
-                    bs[(((buf * NB + nbw) * 2 + 1) * 8 + ib) * 64 + lane] = l;
-                }
+            auto decode_one = [&](int buf, int j) {
+                const int ib = 2 * mg + j;
+                const uint4 * tab = reinterpret_cast<const uint4 *>(s_tab + iq4xs_ls(f_rec, ib) * 32);
+                v4i h, l;
+                decode_planes(f_code[j], tab[0], tab[1], h, l);
+                bs[(((buf * NB + nbw) * 2 + 0) * 8 + ib) * 64 + lane] = h;
+                bs[(((buf * NB + nbw) * 2 + 1) * 8 + ib) * 64 + lane] = l;
             };
+            auto decode_into = [&](int buf) { decode_one(buf, 0); decode_one(buf, 1); };
             // operand A, two k-steps (sub-blocks) per slot, fetched kSlots - 1 slots before its products
             constexpr int kSlots = 4;
             v4i a_reg[kSlots][MTA][2];
@@ -471,12 +469,15 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
                 const int buf = sb & 1;
 #pragma unroll
                 for (int b = 0; b < NB; ++b) d_rec[b] = d_rec_next[b];
-                // past the last super-block the fetch repeats it and the decode fills the stage nobody reads: no branches here
-                decode_into(buf ^ 1);
-                fetch(min(sb + 2, sb_end - 1));
+                // The decode of the next super-block's two sub-blocks is placed between the groups of products, so that its
+                // vector work runs while the matrix pipe works through the group just issued. Past the last super-block the
+                // fetch repeats it and the decode fills the stage nobody reads: no branches here.
                 fetch_d(min(sb + 1, sb_end - 1));
 #pragma unroll
                 for (int jp = 0; jp < 4; ++jp) {
+                    if (jp == 1) { __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, 0); __builtin_amdgcn_sched_barrier(0); }
+                    if (jp == 2) { __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, 1); __builtin_amdgcn_sched_barrier(0); }
+                    if (jp == 3) { __builtin_amdgcn_sched_barrier(0); fetch(min(sb + 2, sb_end - 1)); __builtin_amdgcn_sched_barrier(0); }
                     load_a((jp + kSlots - 1) % kSlots, min(sb * 4 + jp + kSlots - 1, pairs - 1));
 #pragma unroll
                     for (int h = 0; h < 2; ++h) {

@@ -101,7 +101,7 @@ def cpu_baseline(sample_experts=24, budget_s=12.0):
     cores = max(1, min(cores, 64))
     t0 = time.time()
     t_pass, _ = oracle.cpu_expert_bench(oracle.IQ4_XS, *banks, h, f, sample_experts, cores, True, reps=1)
-    reps = int(max(1, min(50, budget_s / max(t_pass, 1e-4) - 2)))
+    reps = int(max(1, min(4000, budget_s / max(t_pass, 1e-4) - 2)))   # about budget_s seconds of CPU work
     t_pass, _ = oracle.cpu_expert_bench(oracle.IQ4_XS, *banks, h, f, sample_experts, cores, True, reps=reps)
     per_layer_token = t_pass / sample_experts * (CFG["topk"] + 1)
     return {"value": round(1.0 / per_layer_token, 2), "unit": "tokens/s", "cores": cores, "kind": "port",

@@ -129,6 +129,31 @@ def test_grouped_products_against_float64(tq, oracle, n, shared_ff):
         assert np.abs(y[a] - want).max() < 2e-3 * max(1e-3, np.abs(want).max()), a
 
 
+@pytest.mark.parametrize("rows,experts", [(96, 5), (160, 5), (128, 5), (256, 5), (64, 1100)])
+def test_gemm_i8_bank_shapes(tq, oracle, rows, experts):
+    """tqmoe_expert_gemm_i8 over banks whose row count changes the kernel's arrangement (one or two operand slots per block,
+    unit counts that do or do not allow the single-tile path) and over more experts than a block keeps an index of, against
+    float64 on the decoded weights and the dequantised int8 rows. One expert gets several row tiles, the others one."""
+    cols, n, k = 256, 150, 1
+    rng = np.random.default_rng(rows + experts)
+    w = (rng.standard_normal((experts * rows, cols)) * 0.02).astype(np.float32)
+    raw = oracle.quantize(oracle.IQ4_XS, w)
+    dec = oracle.dequantize(oracle.IQ4_XS, raw, w.size).reshape(experts, rows, cols).astype(np.float64)
+    bank = tq.ExpertBank(oracle.IQ4_XS, raw, experts, rows, cols)
+    ids = rng.integers(0, experts, size=(n, k)).astype(np.int32)
+    ids[: n // 2, 0] = 2
+    x = torch.randn(n, cols, device="cuda", dtype=torch.float16)
+    counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), experts)
+    lists = (counts, offsets, perm)
+    xq, xs = tq.group_rows_i8(x, lists, n * k, 1)
+    y = tq.expert_gemm_i8(bank, xq, xs, lists, n, k, k).float().cpu().numpy()
+    pq, ps = tq.quant_rows_i8(x)
+    xd = natural_order(pq.cpu().numpy()).astype(np.float64) * ps.cpu().numpy().astype(np.float64)[:, None]
+    for a in range(n):
+        want = dec[ids[a, 0]] @ xd[a]
+        assert np.abs(y[a] - want).max() < 2e-3 * max(1e-3, np.abs(want).max()), a
+
+
 def test_grouped_products_skip_negative_ids(tq, oracle):
     experts, ff, hidden, k, n = 4, 256, 512, 2, 40
     decs, (gate, up, down), ids, slots, banks = grouped_setup(tq, oracle, 3, experts, ff, hidden, n, k, False)

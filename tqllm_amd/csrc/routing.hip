@@ -57,65 +57,79 @@ template <int WT> int32_t launch_router_x(uint32_t xtype, const void * w, const 
 
 // Router logits of many tokens, bf16 rows on both sides: a GEMM on the matrix pipe. bf16 x bf16 products are exact in
 // fp32 and the matrix instruction accumulates in fp32, so the result differs from the scalar kernel's only by the order
-// of the sum. One wave per 64 tokens x 64 router rows (2 x 2 tiles of v_mfma_f32_32x32x16_bf16); no LDS: the k order
-// inside a 64-wide chunk is free, so lane half g takes columns [32 g, 32 g + 32) of the chunk and a lane reads 64
-// contiguous bytes of its row for four instructions.
+// of the sum. A block of four waves takes 128 tokens x 64 router rows; per 64 columns the block stages both operand
+// tiles in LDS with coalesced 16-byte loads (the next tiles are in registers while these are multiplied) and every wave
+// multiplies a 64 x 32 quadrant: two v_mfma_f32_32x32x16_bf16 per 16 columns.
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int kRouterGemmMin = 32;   // token counts from here up (bf16 router and input) take the GEMM
+constexpr int kRgTok = 128, kRgRows = 64, kRgK = 64, kRgPad = kRgK + 8;   // halves per staged row: 16-byte reads of consecutive rows spread over the banks
 
 __global__ __launch_bounds__(256) void router_gemm_bf16_k(const uint16_t * __restrict__ w, const uint16_t * __restrict__ shared, const uint16_t * __restrict__ x,
                                                             float * __restrict__ logits, int h, int e, int n) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, g = lane >> 5;
-    const int row_tiles = (e + 1 + 63) / 64;
-    const int unit = blockIdx.x * 4 + wave;
-    const int t0 = unit / row_tiles * 64, r0 = unit % row_tiles * 64;
-    if (t0 >= n) return;
-    // operand rows of this lane; rows past the ends repeat a valid row (their results are not stored)
-    const uint16_t * ap[2], * bp[2];
-    bool bzero[2];
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][kRgTok][kRgPad];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][kRgRows][kRgPad];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
+    const int t0 = int(blockIdx.x) * kRgTok, r0 = int(blockIdx.y) * kRgRows;
+    const int mq = wave & 1, nq = wave >> 1;           // quadrant: tokens 64 mq.., router rows 32 nq..
+    // staging: thread -> (row, 16-byte piece) of the tiles; A has 128 rows x 8 pieces = 4 per thread, B 64 x 8 = 2
+    const int sp = tid & 7, sr = tid >> 3;             // piece, row (0..31)
+    const uint16_t * a_src[4], * b_src[2];
+    bool b_zero[2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a_src[i] = x + int64_t(min(t0 + sr + 32 * i, n - 1)) * h + 8 * sp;   // rows past the end repeat a valid row (not stored)
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        ap[i] = x + int64_t(min(t0 + 32 * i + r, n - 1)) * h + 32 * g;
-        const int row = min(r0 + 32 * i + r, e);
-        bzero[i] = row == e && shared == nullptr;
-        bp[i] = (row < e ? w + int64_t(row) * h : bzero[i] ? w : shared) + 32 * g;
+        const int row = r0 + sr + 32 * i;
+        b_zero[i] = row > e || (row == e && shared == nullptr);
+        b_src[i] = (row < e ? w + int64_t(row) * h : (row == e && shared) ? shared : w) + 8 * sp;
     }
-    v16f acc[2][2];
+    uint4 a_st[4], b_st[2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a_st[i] = *reinterpret_cast<const uint4 *>(a_src[i] + k0);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) b_st[i] = b_zero[i] ? make_uint4(0, 0, 0, 0) : *reinterpret_cast<const uint4 *>(b_src[i] + k0);
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4 *>(&As[buf][sr + 32 * i][8 * sp]) = a_st[i];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4 *>(&Bs[buf][sr + 32 * i][8 * sp]) = b_st[i];
+    };
+    v16f acc[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int q = 0; q < 16; ++q) acc[i][q] = 0.f;
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    const int chunks = h / kRgK;
+    for (int c = 0; c < chunks; ++c) {
+        const int buf = c & 1;
+        if (c + 1 < chunks) fetch((c + 1) * kRgK);
 #pragma unroll
-            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
-    for (int k0 = 0; k0 < h; k0 += 64) {
-        v8bf a[2][4], b[2][4];
+        for (int j = 0; j < kRgK / 16; ++j) {     // operand of lane (r, g): row r, columns 16 j + 8 g .. + 7
+            const v8bf b = *reinterpret_cast<const v8bf *>(&Bs[buf][nq * 32 + r][16 * j + 8 * g]);
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                a[i][c] = *reinterpret_cast<const v8bf *>(ap[i] + k0 + 8 * c);
-                b[i][c] = *reinterpret_cast<const v8bf *>(bp[i] + k0 + 8 * c);
+            for (int i = 0; i < 2; ++i) {
+                const v8bf a = *reinterpret_cast<const v8bf *>(&As[buf][mq * 64 + 32 * i + r][16 * j + 8 * g]);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
             }
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i][c], b[j][c], acc[i][j], 0, 0, 0);
+        }
+        if (c + 1 < chunks) stage(buf ^ 1);       // the other stage: last read before the previous barrier
+        __syncthreads();
     }
-    // result register q of lane half g: token row 8 (q / 4) + 4 g + q % 4, router row r
+    // result register q of lane half g: token row 8 (q / 4) + 4 g + q % 4 of the 32-row tile, router row r
+    const int row = r0 + nq * 32 + r;
+    if (row > e) return;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int row = r0 + 32 * j + r;
-            if (row > e) continue;
-#pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                const int t = t0 + 32 * i + 8 * (q >> 2) + 4 * g + (q & 3);
-                if (t < n) logits[int64_t(t) * (e + 1) + row] = bzero[j] ? 0.f : acc[i][j][q];
-            }
+        for (int q = 0; q < 16; ++q) {
+            const int t = t0 + mq * 64 + 32 * i + 8 * (q >> 2) + 4 * g + (q & 3);
+            if (t < n) logits[int64_t(t) * (e + 1) + row] = acc[i][q];
         }
 }
 
@@ -433,8 +447,8 @@ extern "C" int32_t tqmoe_router(const void * router, uint32_t wtype, const void 
     if (int32_t rc = need_device(err, "tqmoe_router")) return rc;
     const hipStream_t s = static_cast<hipStream_t>(stream);
     if (wtype == TQMOE_BF16 && xtype == TQMOE_BF16 && n >= kRouterGemmMin && hidden % 64 == 0) {
-        const int64_t units = int64_t((n + 63) / 64) * ((experts + 1 + 63) / 64);
-        router_gemm_bf16_k<<<unsigned((units + 3) / 4), 256, 0, s>>>(static_cast<const uint16_t *>(router), static_cast<const uint16_t *>(shared_gate),
+        const dim3 grid(unsigned((n + kRgTok - 1) / kRgTok), unsigned((experts + 1 + kRgRows - 1) / kRgRows));
+        router_gemm_bf16_k<<<grid, 256, 0, s>>>(static_cast<const uint16_t *>(router), static_cast<const uint16_t *>(shared_gate),
                                                                       static_cast<const uint16_t *>(x), logits, hidden, experts, n);
         return launched(err, "tqmoe_router");
     }

@@ -6,29 +6,31 @@ namespace tqmoe {
 namespace {
 
 // ----------------------------------------------------------------------------------------------------- router
-// One wave per router row, kTok tokens per pass; each lane owns 8-element chunks lane, lane + 64, ... of the row.
+// One wave per router row, TOK tokens per pass; each lane owns 8-element chunks lane, lane + 64, ... of the row.
 // Sums in fp32; the order (chunks ascending per lane, then a butterfly over lanes) differs from a column-order host
 // sum by ordinary fp32 rounding only.
-constexpr int kRouterTok = 4;
-template <int WT, int XT>
+constexpr int kRouterTok = 4;       // tokens per pass of a wave: the router row is read once for them
+constexpr int kRouterTokFew = 1;    // decode-sized batches: a wave per (row, token), the latency of a wave's chain is what counts
+constexpr int kRouterFew = 32;      // batches up to here take kRouterTokFew
+template <int WT, int XT, int TOK>
 __global__ __launch_bounds__(256) void router_k(const void * __restrict__ w, const void * __restrict__ shared,
                                                 const void * __restrict__ x, float * __restrict__ logits, int h, int e, int n) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int row = blockIdx.x * 4 + wave;  // 0..e (e = the shared gate)
-    const int t0 = blockIdx.y * kRouterTok;
+    const int t0 = blockIdx.y * TOK;
     if (row > e) return;                     // whole waves leave together: reductions below see full waves
     const bool has_row = row < e || shared != nullptr;
     const void * wr = row < e ? w : shared;
     const int64_t wbase = row < e ? int64_t(row) * h : 0;
-    float acc[kRouterTok];
+    float acc[TOK];
 #pragma unroll
-    for (int i = 0; i < kRouterTok; ++i) acc[i] = 0.f;
+    for (int i = 0; i < TOK; ++i) acc[i] = 0.f;
     if (has_row)
         for (int c = lane * 8; c < h; c += 512) {
             float wv[8];
             load8<WT>(wr, wbase + c, wv);
 #pragma unroll
-            for (int i = 0; i < kRouterTok; ++i) {
+            for (int i = 0; i < TOK; ++i) {
                 if (t0 + i < n) {
                     float xv[8];
                     load8<XT>(x, int64_t(t0 + i) * h + c, xv);
@@ -38,7 +40,7 @@ __global__ __launch_bounds__(256) void router_k(const void * __restrict__ w, con
             }
         }
 #pragma unroll
-    for (int i = 0; i < kRouterTok; ++i) {
+    for (int i = 0; i < TOK; ++i) {
         const float s = group_sum<64>(acc[i]);
         if (lane == 0 && t0 + i < n) logits[int64_t(t0 + i) * (e + 1) + row] = s;
     }
@@ -46,11 +48,22 @@ __global__ __launch_bounds__(256) void router_k(const void * __restrict__ w, con
 
 template <int WT> int32_t launch_router_x(uint32_t xtype, const void * w, const void * sg, const void * x, float * logits,
                                           int h, int e, int n, hipStream_t s) {
-    const dim3 grid(unsigned((e + 1 + 3) / 4), unsigned((n + kRouterTok - 1) / kRouterTok));
+    const bool wide = n <= kRouterFew;   // the wide grid of one-token passes
+    const int tok = wide ? kRouterTokFew : kRouterTok;
+    const dim3 grid(unsigned((e + 1 + 3) / 4), unsigned((n + tok - 1) / tok));
     switch (xtype) {
-        case TQMOE_F32: router_k<WT, TQMOE_F32><<<grid, 256, 0, s>>>(w, sg, x, logits, h, e, n); return 0;
-        case TQMOE_F16: router_k<WT, TQMOE_F16><<<grid, 256, 0, s>>>(w, sg, x, logits, h, e, n); return 0;
-        case TQMOE_BF16: router_k<WT, TQMOE_BF16><<<grid, 256, 0, s>>>(w, sg, x, logits, h, e, n); return 0;
+        case TQMOE_F32:
+            if (wide) router_k<WT, TQMOE_F32, kRouterTokFew><<<grid, 256, 0, s>>>(w, sg, x, logits, h, e, n);
+            else router_k<WT, TQMOE_F32, kRouterTok><<<grid, 256, 0, s>>>(w, sg, x, logits, h, e, n);
+            return 0;
+        case TQMOE_F16:
+            if (wide) router_k<WT, TQMOE_F16, kRouterTokFew><<<grid, 256, 0, s>>>(w, sg, x, logits, h, e, n);
+            else router_k<WT, TQMOE_F16, kRouterTok><<<grid, 256, 0, s>>>(w, sg, x, logits, h, e, n);
+            return 0;
+        case TQMOE_BF16:
+            if (wide) router_k<WT, TQMOE_BF16, kRouterTokFew><<<grid, 256, 0, s>>>(w, sg, x, logits, h, e, n);
+            else router_k<WT, TQMOE_BF16, kRouterTok><<<grid, 256, 0, s>>>(w, sg, x, logits, h, e, n);
+            return 0;
     }
     return -1;
 }

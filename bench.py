@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""MoE-layer benchmark on one MI355X: the Flash-Next-shaped IQ4_XS layer, as decode (BASELINE config 2, the default:
+"""MoE-layer benchmark on one MI355X: the Flash-Next-shaped IQ4_XS layer, as decode (configuration 2 of the benchmark definition, the default:
 --tokens 16, also 1 and 4) or as prefill (config 3: --tokens 4096, Zipf-skewed routing, int8 MFMA grouped products).
 
 A step is one pass of the whole layer (router, top-k, gate/up + SwiGLU, down + combine, shared expert) over one batch of
@@ -115,7 +115,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 400; 80 at prefill sizes)")
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--tokens", type=int, default=16, help="decode batch of the step (BASELINE config 2 names 1, 4 and 16)")
+    ap.add_argument("--tokens", type=int, default=16, help="decode batch of the step (configuration 2 names 1, 4 and 16)")
     ap.add_argument("--banks", type=int, default=8, help="independent expert banks the steps rotate over")
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

@@ -1,5 +1,5 @@
 """Seeded synthetic MoE layers for the parity tests and the benchmark: weights N(0, sigma) quantised by the oracle's
-encoders into GGUF blocks, router weights and activations as BASELINE's configs describe them. numpy only."""
+encoders into GGUF blocks, router weights and activations as the benchmark's five configurations describe them. numpy only."""
 import numpy as np
 
 import oracle

@@ -197,7 +197,10 @@ int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float *
  * (per-token scales). xq / xs: tqmoe_group_rows_i8's outputs for the same lists.
  * Assignments of the bank's last expert use only shared_lim rows (gate / up; the rest of their act row is zero) or columns
  * (down) when slots > topk (the shared expert); shared_lim a multiple of 256. Rows of assignments that are in no list
- * stay untouched. */
+ * stay untouched. The products hand their work out through counters that live behind the grouped rows' scales (zero
+ * between launches: the grouping call clears them and every product launch leaves them cleared), so two products over
+ * the same grouped rows may follow each other on a stream, also in a replayed graph, but must not run at the same
+ * time. */
 int32_t tqmoe_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int32_t cols, int8_t * q, float * scale,
                             void * stream, tqmoe_error * err);
 int64_t tqmoe_grouped_rows(int64_t assignments, int32_t experts);

@@ -9,6 +9,7 @@ GPU is an error.
 import ctypes as C
 import os
 
+import numpy as np
 import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -189,6 +190,16 @@ class ExpertBank:
                                      C.byref(err)), err)
         if int(status.item()):
             raise TqmoeError(-1, "NVFP4G rows whose blocks carry different global scales are not loadable")
+
+    @classmethod
+    def from_gguf(cls, path, name, device="cuda"):
+        """The bank of a 3-D expert tensor [cols, rows, n_experts] of a GGUF file (ffn_{gate,up,down}_exps.weight): its
+        bytes are the stacked block stream as they lie (gguf_expert_slice, src/core/gguf.hpp:77-91)."""
+        from .gguf import GgufFile
+        wtype, experts, rows, cols, raw = GgufFile(path).expert_bank(name)
+        if wtype not in BLOCK:
+            raise TqmoeError(-1, "%s: no expert kernels for GGUF type %d" % (name, wtype))
+        return cls(wtype, torch.from_numpy(np.array(raw)), experts, rows, cols, device=device)
 
     def view(self):
         return _Bank(C.sizeof(_Bank), self.type, self.experts, self.rows, self.cols, self.codes.data_ptr(), self.aux.data_ptr())

@@ -52,6 +52,20 @@ int32_t tqmoe_router(const void * router, uint32_t wtype, const void * shared_ga
 int32_t tqmoe_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t experts,
                    int32_t topk, int32_t n, float scale, void * stream, tqmoe_error * err);
 
+/* The reference's other routing modes, moe_route (src/experts/moe.cpp:22-113) in full:
+ *   gating        TQMOE_GATE_SOFTMAX         p = softmax(logits)
+ *                 TQMOE_GATE_SIGMOID         p = 1 / (1 + exp(-logit))
+ *                 TQMOE_GATE_SOFTMAX_WEIGHT  p = logit; the weights are a softmax over the selected logits only
+ *                 TQMOE_GATE_SQRT_SOFTPLUS   p = sqrt(log(1 + exp(logit)))
+ *   probs_bias    device [experts] fp32 or NULL: added to p for the choice only (descending p + bias, ties to the lower
+ *                 index); the weights come from the unbiased p
+ *   norm_weights  nonzero: weights divided by max(their sum, 6.103515625e-5); then * (scale == 0 ? 1 : scale)
+ * The values are MoeGating's (src/experts/moe.hpp:20-26). shared_weights as in tqmoe_topk. experts <= 4096. */
+enum { TQMOE_GATE_SOFTMAX = 1, TQMOE_GATE_SIGMOID = 2, TQMOE_GATE_SOFTMAX_WEIGHT = 3, TQMOE_GATE_SQRT_SOFTPLUS = 4 };
+int32_t tqmoe_topk_gated(const float * logits, const float * probs_bias, int32_t gating, int32_t norm_weights,
+                         int32_t * ids, float * weights, float * shared_weights, int32_t experts, int32_t topk,
+                         int32_t n, float scale, void * stream, tqmoe_error * err);
+
 /* Token-to-expert dispatch of the A = n * topk assignments a = t * topk + s:
  *   counts[e]   assignments of expert e (ids < 0 skipped),
  *   offsets[e]  exclusive scan of counts, offsets[experts] = number kept,
@@ -252,6 +266,11 @@ typedef struct tqmoe_layer {
     const void * shared_gate;         /* device [hidden] of router_type, or NULL */
     uint32_t router_type;             /* TQMOE_F32 or TQMOE_BF16 */
     tqmoe_bank gate, up, down;        /* gate / up: rows ff, cols hidden; down: rows hidden, cols ff */
+    /* Routing mode, as tqmoe_topk_gated takes it. A descriptor whose struct_size ends before these fields, or that
+     * leaves them zero, routes by softmax with normalised weights and no bias. */
+    int32_t gating;                   /* 0: softmax, else a TQMOE_GATE_ value */
+    int32_t raw_weights;              /* nonzero: the selected weights are not normalised */
+    const float * probs_bias;         /* device [n_expert] fp32 selection bias, or NULL */
 } tqmoe_layer;
 
 size_t  tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t n);

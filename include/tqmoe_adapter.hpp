@@ -49,6 +49,22 @@ inline void moe_topk(const float * logits, int * ids, float * weights, float * s
     tqmoe_error e = fresh();
     check(tqmoe_topk(logits, ids, weights, shared_weights, experts, topk, n, scale, stream, &e), e);
 }
+// moe_route (src/experts/moe.hpp:28-51) for n tokens on the device: the host function's configuration with its defaults
+// (sigmoid gating, weights not normalised, no scale); logits rows hold n_expert + 1 columns as moe_router writes them,
+// probs_bias is a device array of n_expert floats or null. Throws for a gating value outside MoeGating's.
+struct MoeRouting {
+    int n_expert = 0;
+    int n_expert_used = 0;
+    int gating = TQMOE_GATE_SIGMOID;
+    bool norm_weights = false;
+    float weight_scale = 0.f;
+};
+inline void moe_route(const MoeRouting & cfg, const float * logits, const float * probs_bias, int * ids, float * weights, float * shared_weights, int n,
+                      void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_topk_gated(logits, probs_bias, cfg.gating, cfg.norm_weights ? 1 : 0, ids, weights, shared_weights, cfg.n_expert, cfg.n_expert_used, n,
+                           cfg.weight_scale, stream, &e), e);
+}
 // moe_group (moe_kernels.cuh:29): groups [experts][n], counts [experts]. The lists are ascending inside each expert
 // (the reference's device version is atomic-ordered). `scratch` holds the offsets, the permutation and the workspace:
 // moe_group_scratch_bytes() device bytes.

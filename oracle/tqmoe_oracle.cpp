@@ -433,8 +433,16 @@ void gate_probs(int gating, int n, const float * logits, std::vector<float> & pr
         float sum = 0.f;
         for (int i = 0; i < n; ++i) { probs[size_t(i)] = std::exp(logits[i] - mx); sum += probs[size_t(i)]; }
         for (int i = 0; i < n; ++i) probs[size_t(i)] /= sum;
-    } else {  // sigmoid, src/experts/moe.cpp:10-14
+    } else if (gating == TQO_GATE_SIGMOID) {  // src/experts/moe.cpp:10-14
         for (int i = 0; i < n; ++i) probs[size_t(i)] = 1.0f / (1.0f + std::exp(-logits[i]));
+    } else if (gating == TQO_GATE_SOFTMAX_WEIGHT) {  // src/experts/moe.cpp:48-50: the raw logits; softmax comes after the choice
+        for (int i = 0; i < n; ++i) probs[size_t(i)] = logits[i];
+    } else {  // sqrt(softplus), src/experts/moe.cpp:15-19 and 51-53
+        for (int i = 0; i < n; ++i) {
+            const float x = logits[i];
+            const float sp = x > 0.f ? x + std::log1p(std::exp(-x)) : std::log1p(std::exp(x));
+            probs[size_t(i)] = std::sqrt(sp);
+        }
     }
 }
 }  // namespace
@@ -442,7 +450,7 @@ void gate_probs(int gating, int n, const float * logits, std::vector<float> & pr
 int tqo_route(int gating, int n_expert, int k, int norm_weights, float weight_scale, const float * logits,
               const float * bias, int32_t * ids, float * weights) {
     if (n_expert <= 0 || k <= 0 || k > n_expert) return -1;
-    if (gating != TQO_GATE_SOFTMAX && gating != TQO_GATE_SIGMOID) return -1;
+    if (gating < TQO_GATE_SOFTMAX || gating > TQO_GATE_SQRT_SOFTPLUS) return -1;
     std::vector<float> probs;
     gate_probs(gating, n_expert, logits, probs);
     std::vector<float> sel(probs);  // selection values: bias added for the choice only (moe.cpp:63-65)
@@ -454,6 +462,13 @@ int tqo_route(int gating, int n_expert, int k, int norm_weights, float weight_sc
         return a < b;
     });
     for (int s = 0; s < k; ++s) { ids[s] = order[size_t(s)]; weights[s] = probs[size_t(order[size_t(s)])]; }
+    if (gating == TQO_GATE_SOFTMAX_WEIGHT) {  // moe.cpp:88-97: softmax over the selected weights only
+        float mx = -INFINITY;
+        for (int s = 0; s < k; ++s) mx = std::max(mx, weights[s]);
+        float sum = 0.f;
+        for (int s = 0; s < k; ++s) { weights[s] = std::exp(weights[s] - mx); sum += weights[s]; }
+        for (int s = 0; s < k; ++s) weights[s] /= sum;
+    }
     if (norm_weights) {  // moe.cpp:101-106
         float sum = 0.f;
         for (int s = 0; s < k; ++s) sum += weights[s];
@@ -661,8 +676,8 @@ int tqo_layer_forward(const tqo_layer * Lp, const float * x, const float * logit
     std::vector<int32_t> ids(static_cast<size_t>(A)), counts(static_cast<size_t>(E)), offsets(size_t(E) + 1), perm(static_cast<size_t>(A));
     std::vector<float> weights(static_cast<size_t>(A));
     for (int t = 0; t < n; ++t)
-        if (tqo_route(TQO_GATE_SOFTMAX, E, K, 1, 1.f, logits + size_t(t) * (E + 1), nullptr, ids.data() + size_t(t) * K,
-                      weights.data() + size_t(t) * K)) return -1;
+        if (tqo_route(L.gating ? L.gating : int(TQO_GATE_SOFTMAX), E, K, L.raw_weights ? 0 : 1, L.weight_scale, logits + size_t(t) * (E + 1), L.bias,
+                      ids.data() + size_t(t) * K, weights.data() + size_t(t) * K)) return -1;
     tqo_dispatch(ids.data(), A, E, counts.data(), offsets.data(), perm.data());
     if (ids_out) std::copy(ids.begin(), ids.end(), ids_out);
     if (weights_out) std::copy(weights.begin(), weights.end(), weights_out);

@@ -11,8 +11,9 @@
  *                   IQ4_XS                 src/formats/weight/dequant.cpp:176-192
  *                   IQ4_NL                 src/formats/weight/dequant.cpp:351-360
  *                   NVFP4G                 src/formats/weight/dequant.cpp:397-409
- *   tqo_route                              src/experts/moe.cpp:22-113 (softmax / sigmoid gating, selection bias,
- *                                          stable top-k, unbiased weights, clamp 6.103515625e-5, scale)
+ *   tqo_route                              src/experts/moe.cpp:22-113 (softmax / sigmoid / softmax-of-selected /
+ *                                          sqrt-softplus gating, selection bias, stable top-k, unbiased weights,
+ *                                          clamp 6.103515625e-5, scale)
  *   tqo_shared_weight                      src/experts/moe.cu:92 (sigmoid of logits column E)
  *   tqo_dispatch                           src/models/qwen/qwen4exp/prefill_plan.hpp:63-74 (ascending assignment
  *                                          order inside each expert), counts as src/experts/moe.cu:168-176
@@ -48,7 +49,7 @@ extern "C" {
 enum { TQO_F32 = 0, TQO_F16 = 1, TQO_Q4_K = 12, TQO_IQ4_NL = 20, TQO_IQ3_S = 21, TQO_IQ4_XS = 23, TQO_BF16 = 30,
        TQO_NVFP4G = 323 };
 /* gating (src/experts/moe.hpp:20-26) */
-enum { TQO_GATE_SOFTMAX = 1, TQO_GATE_SIGMOID = 2 };
+enum { TQO_GATE_SOFTMAX = 1, TQO_GATE_SIGMOID = 2, TQO_GATE_SOFTMAX_WEIGHT = 3, TQO_GATE_SQRT_SOFTPLUS = 4 };
 
 float    tqo_half_to_float(uint16_t h);
 uint16_t tqo_float_to_half(float f);
@@ -103,6 +104,8 @@ void tqo_quant_act_row_e4m3(const float * x, int cols, uint8_t * q, float * scal
  *   fp8 path; not implemented); 3 = mode 1 with the weights widened to int8 per (row, 256-weight super-block);
  *   5 = mode 1 with silu(gate) * up and the down product each rounded to fp16 (what the grouped int8 products store).
  *   out fp32 [n][H]; ids_out [n][k], weights_out [n][k] may be null. threads: worker threads over tokens.
+ *   gating (0 = softmax), raw_weights (nonzero: unnormalised), weight_scale (0 = none) and bias (or null) are
+ *   tqo_route's arguments; all zero is softmax routing with normalised weights.
  */
 typedef struct tqo_layer {
     int hidden, ff, n_expert, k, has_shared, shared_ff;
@@ -110,6 +113,9 @@ typedef struct tqo_layer {
     const void * gate, * up, * down;
     int act_mode;
     int threads;
+    int gating, raw_weights;
+    float weight_scale;
+    const float * bias;
 } tqo_layer;
 int tqo_layer_forward(const tqo_layer * L, const float * x, const float * logits, int n, float * out,
                       int32_t * ids_out, float * weights_out);

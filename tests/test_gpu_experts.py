@@ -172,6 +172,29 @@ def test_layer_config4_crossover_token_counts(tq, oracle, n):
     check_layer(*run_layer(tq, oracle, synth.CONFIGS["c4"], n, seed=430 + n, distinct=8))
 
 
+@pytest.mark.parametrize("gating,norm,biased,scale", [(2, True, True, 2.5), (2, False, False, 1.0), (4, True, True, 1.0), (3, False, True, 1.0), (1, False, True, 0.5)])
+@pytest.mark.parametrize("n", [5, 800])
+def test_layer_other_routing_modes(tq, oracle, gating, norm, biased, scale, n):
+    """Sigmoid / sqrt-softplus / selected-softmax gating, a selection bias, raw weights and a weight scale through the
+    whole layer (moe_route's modes, src/experts/moe.cpp:22-113), on the decode kernels (5 tokens) and the grouped GEMM."""
+    cfg = synth.small(synth.CONFIGS["c1"], 768, 512, 10, 3)
+    raws = synth.make_banks(cfg, seed=61)
+    gate, up, down = banks_on_device(cfg, raws)
+    inp = synth.make_inputs(cfg, n, seed=62)
+    e, k = cfg["experts"], cfg["topk"]
+    bias = np.random.default_rng(63).uniform(-0.5, 0.5, e).astype(np.float32) if biased else None
+    layer = tq.MoeLayer(dev(inp["router"]), None, gate, up, down, k, shared_ff=0, weight_scale=scale,
+                        gating=gating, probs_bias=dev(bias) if biased else None, norm_weights=norm)
+    out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
+    want, want_ids, want_w = oracle.layer_forward(inp["x"][1], logits, *raws, cfg["wtype"], cfg["hidden"], cfg["ff"], e, k, shared_ff=cfg["shared_ff"],
+                                                  act_mode=0, threads=16, gating=gating, norm=norm, scale=scale, bias=bias)
+    same = (ids == want_ids).all(axis=1)          # near-tied tokens may swap neighbours; the routing test bounds how many
+    assert same.mean() > 0.97
+    assert np.abs(w[same] - want_w[same]).max() < 4e-6 * max(1.0, float(np.abs(want_w).max()))
+    mx, rel = synth.errors(out[same], want[same])
+    assert mx < MAX_ABS * max(1.0, float(np.abs(want_w).sum(axis=1).max())) and rel < REL_RMS, (mx, rel)
+
+
 def test_layer_linearity_and_bf16_output(tq, oracle):
     """One expert, normalised weight 1: the layer equals that expert's FFN (tests/moe.cpp:354-392); bf16 output is the
     rounded fp32 output."""

@@ -97,6 +97,67 @@ def test_topk_ties_extremes_and_scale(tq, oracle):
     assert ids[0].tolist() == list(range(k)) and ids[3][0] == 10
 
 
+def selection_values(logits, gating, bias):
+    """float64 selection values of moe_route (src/experts/moe.cpp:33-65): a token is a clear case when its k + 1 largest
+    are further apart than the fp32 rounding of the gating function."""
+    lg = logits.astype(np.float64)
+    if gating == 1:
+        p = np.exp(lg - lg.max(axis=1, keepdims=True))
+        p /= p.sum(axis=1, keepdims=True)
+    elif gating == 2:
+        p = 1 / (1 + np.exp(-lg))
+    elif gating == 3:
+        p = lg
+    else:
+        p = np.sqrt(np.logaddexp(0, lg))
+    return p + bias.astype(np.float64) if bias is not None else p
+
+
+@pytest.mark.parametrize("gating", [1, 2, 3, 4])
+@pytest.mark.parametrize("e,k,n", [(256, 8, 64), (512, 10, 16), (64, 6, 33), (1500, 4, 20), (160, 70, 24), (5, 5, 12)])
+def test_topk_gated_matches_oracle(tq, oracle, gating, e, k, n):
+    rng = np.random.default_rng(e * 11 + k + gating)
+    logits = (rng.standard_normal((n, e + 1)) * 2).astype(np.float32)
+    for biased in (False, True):
+        for norm in (True, False):
+            for scale in (1.0, 2.5):
+                if gating == 1 and not biased and norm:
+                    continue                 # the plain entry point's case, tested above
+                bias = rng.uniform(-0.5, 0.5, e).astype(np.float32) if biased else None
+                ids, w, sw = (t.cpu().numpy() for t in tq.moe_topk(dev(logits), e, k, scale, gating=gating, bias=dev(bias) if biased else None,
+                                                                   norm=norm))
+                want_ids, want_w = oracle.route(logits[:, :e], k, gating, norm, scale, bias)
+                v = -np.sort(-selection_values(logits[:, :e], gating, bias), axis=1)[:, :k + 1]
+                room = 2e-6 * (np.abs(v[:, :-1]) + (float(np.abs(bias).max()) if biased else 0.0))   # fp32 rounding of value and sum
+                clear = (v[:, :-1] - v[:, 1:] > room).all(axis=1)
+                assert clear.mean() > 0.9
+                assert np.array_equal(ids[clear], want_ids[clear])
+                same = (ids == want_ids).all(axis=1)
+                assert np.abs(w[same] - want_w[same]).max() < 4e-6 * max(1.0, float(np.abs(want_w).max()))
+                want_sw = np.array([oracle.shared_weight(x) for x in logits[:, e]], np.float32)
+                assert np.abs(sw - want_sw).max() < 3e-6
+
+
+def test_topk_gated_closed_forms(tq, oracle):
+    """The cases of the reference's tests/moe.cpp:149-236 on the device: a bias moves the choice and not the weight, equal
+    values go to the lower index, underflowing sigmoids stay finite, scale 0 and 1 mean none."""
+    lg = np.array([[2, 1, 0, -1, 0.0]], np.float32)
+    ids, w, _ = (t.cpu().numpy() for t in tq.moe_topk(dev(lg), 4, 2, gating=2, bias=dev(np.array([0, 0, 0, 100], np.float32)), norm=False))
+    assert ids[0].tolist() == [3, 0] and abs(w[0, 0] - 1 / (1 + np.exp(1.0))) < 1e-6
+    ids, w, _ = (t.cpu().numpy() for t in tq.moe_topk(dev(np.full((1, 9), 0.5, np.float32)), 8, 3, gating=2, norm=False))
+    assert ids[0].tolist() == [0, 1, 2] and np.abs(w - 1 / (1 + np.exp(-0.5))).max() < 1e-6
+    ids, w, _ = (t.cpu().numpy() for t in tq.moe_topk(dev(np.array([[-200, -300, -400, -500, 0]], np.float32)), 4, 4, gating=2, norm=True))
+    assert np.isfinite(w).all() and not w.any() and ids[0].tolist() == [0, 1, 2, 3]
+    lg = np.array([[3, 1, -1, -3, 0]], np.float32)
+    w0, w1, w2 = (tq.moe_topk(dev(lg), 4, 2, s, gating=2)[1].cpu().numpy() for s in (0.0, 1.0, 2.5))
+    assert np.array_equal(w0, w1) and abs(w1.sum() - 1) < 1e-6 and np.abs(w2 - 2.5 * w1).max() < 1e-6
+    # selected-softmax: chosen by logit, weighted by a softmax over the chosen ones
+    ids, w, _ = (t.cpu().numpy() for t in tq.moe_topk(dev(np.array([[1, 3, 2, -5, 0]], np.float32)), 4, 2, gating=3, norm=False))
+    assert ids[0].tolist() == [1, 2] and np.abs(w[0] - np.array([np.e, 1]) / (np.e + 1)).max() < 1e-6
+    with pytest.raises(tq.TqmoeError):
+        tq.moe_topk(dev(lg), 4, 2, gating=7)
+
+
 @pytest.mark.parametrize("e,n,k", [(64, 1, 8), (512, 16, 10), (512, 4096, 10), (256, 8192, 9), (7, 300, 3), (4096, 700, 2), (512, 102, 10)])
 def test_dispatch_bit_exact(tq, oracle, e, n, k):
     rng = np.random.default_rng(n + e)

@@ -19,8 +19,12 @@ def max_scan_route(logits, k, gating, norm, scale, bias):
         for v in p:
             s = np.float32(s + v)
         p = (p / s).astype(np.float32)
-    else:
+    elif gating == 2:
         p = (np.float32(1) / (np.float32(1) + np.exp(-lg, dtype=np.float32))).astype(np.float32)
+    elif gating == 3:
+        p = lg
+    else:
+        p = np.sqrt(np.logaddexp(np.float64(0), lg.astype(np.float64))).astype(np.float32)   # log(1 + e^x), stable
     sel = p + bias.astype(np.float32) if bias is not None else p
     taken = np.zeros(len(lg), bool)
     ids, w = [], []
@@ -33,6 +37,8 @@ def max_scan_route(logits, k, gating, norm, scale, bias):
         ids.append(best)
         w.append(p[best])
     w = np.array(w, np.float32)
+    if gating == 3:                      # softmax over the selected logits only
+        w = softmax(w.astype(np.float64)).astype(np.float32)
     if norm:
         s = np.float32(0)
         for v in w:
@@ -45,7 +51,7 @@ def max_scan_route(logits, k, gating, norm, scale, bias):
 
 def test_route_matches_independent_max_scan(oracle):
     rng = np.random.default_rng(11)
-    for gating in (1, 2):
+    for gating in (1, 2, 3, 4):
         for norm in (False, True):
             for biased in (False, True):
                 for _ in range(60):
@@ -97,24 +103,32 @@ def test_route_closed_forms(oracle):
     # softmax with far-apart logits: exp underflows to exact zeros, ties among zeros go to the lower index
     ids, w = oracle.route(np.array([0, -200, 50, -300, -250], np.float32), 3)
     assert ids[0].tolist() == [2, 0, 1] and w[0, 0] == 1.0 and w[0, 2] == 0.0
+    # softmax over the selected logits: the choice is by logit, the weights a softmax of the chosen ones (moe.cpp:88-97)
+    ids, w = oracle.route(np.array([1.0, 3.0, 2.0, -5.0], np.float32), 2, gating=3, norm=False)
+    assert ids[0].tolist() == [1, 2] and np.abs(w[0] - np.array([np.e, 1]) / (np.e + 1)).max() < 1e-6
+    # sqrt(softplus): at 0 it is sqrt(ln 2); for large x it tends to sqrt(x); for very negative x to exp(x / 2)
+    ids, w = oracle.route(np.array([0.0, 40.0, -30.0], np.float32), 3, gating=4, norm=False)
+    assert ids[0].tolist() == [1, 0, 2]
+    assert np.abs(w[0] - np.array([np.sqrt(40.0), np.sqrt(np.log(2.0)), np.exp(-15.0)])).max() < 1e-6
     assert oracle.shared_weight(0.0) == 0.5 and oracle.shared_weight(-1e30) == 0.0
     assert abs(oracle.shared_weight(1.25) - 1 / (1 + np.exp(-1.25))) < 1e-7
 
 
 def test_route_matches_reference_objects(oracle, ref):
     rng = np.random.default_rng(13)
-    for gating in (1, 2):
+    for gating in (1, 2, 3, 4):
         for _ in range(200):
             e = int(rng.integers(2, 600))
             k = int(rng.integers(1, min(e, 16) + 1))
             lg = (rng.standard_normal(e) * rng.uniform(0.1, 6)).astype(np.float32)
             bias = rng.uniform(-1, 1, e).astype(np.float32) if rng.random() < 0.5 else None
             scale = float(np.float32(rng.choice([0.0, 1.0, 2.5])))
-            ids, w = oracle.route(lg, k, gating, True, scale, bias)
+            norm = bool(rng.random() < 0.7)
+            ids, w = oracle.route(lg, k, gating, norm, scale, bias)
             ri = np.empty(k, np.int32)
             rw = np.empty(k, np.float32)
             bp = bias.ctypes.data_as(C.c_void_p) if bias is not None else None
-            assert ref.ref_route(gating, e, k, 1, scale, lg.ctypes.data_as(C.c_void_p), bp, ri.ctypes.data_as(C.c_void_p),
+            assert ref.ref_route(gating, e, k, int(norm), scale, lg.ctypes.data_as(C.c_void_p), bp, ri.ctypes.data_as(C.c_void_p),
                                  rw.ctypes.data_as(C.c_void_p)) == 0
             assert np.array_equal(ids[0], ri)
             assert np.array_equal(w[0].view(np.uint32), rw.view(np.uint32))   # same libm, same order: bit for bit
@@ -224,6 +238,14 @@ def test_layer_forward_against_float64(oracle):
         t = 0
         want = sum(float(w[t, s]) * ffn(ids[t, s], x[t].astype(np.float64), f) for s in range(k))
         assert np.abs(out2[t] - want).max() < 2e-5 * max(1.0, np.abs(want).max())
+        # the other routing modes change the ids and weights (pinned above), nothing else
+        bias = rng.uniform(-1, 1, e).astype(np.float32)
+        out3, ids3, w3 = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=0, threads=2, gating=2, norm=False, scale=2.5, bias=bias)
+        ri, rw = oracle.route(logits[:, :e], k, 2, False, 2.5, bias)
+        assert np.array_equal(ids3, ri) and np.array_equal(w3, rw) and not np.array_equal(ids3, ids)
+        for t in range(n):
+            want = sum(float(w3[t, s]) * ffn(ids3[t, s], x[t].astype(np.float64), f) for s in range(k))
+            assert np.abs(out3[t] - want).max() < 2e-5 * max(1.0, np.abs(want).max())
 
 
 def test_declared_quantisers(oracle):

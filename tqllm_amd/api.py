@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(HERE, "libtqmoe.so")
 
 F32, F16, BF16 = 0, 1, 30
 Q4_K, IQ3_S, IQ4_XS, NVFP4G = 12, 21, 23, 323
+GATE_SOFTMAX, GATE_SIGMOID, GATE_SOFTMAX_WEIGHT, GATE_SQRT_SOFTPLUS = 1, 2, 3, 4   # MoeGating, src/experts/moe.hpp:20-26
 BLOCK = {Q4_K: (256, 144), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76)}
 _TORCH_TYPE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 _OUT_TYPE = {F32: torch.float32, BF16: torch.bfloat16}
@@ -41,7 +42,8 @@ class _Layer(C.Structure):
     _fields_ = [("struct_size", C.c_uint32), ("hidden", C.c_int32), ("ff", C.c_int32), ("n_expert", C.c_int32),
                 ("topk", C.c_int32), ("has_shared", C.c_int32), ("shared_ff", C.c_int32), ("weight_scale", C.c_float),
                 ("router", C.c_void_p), ("shared_gate", C.c_void_p), ("router_type", C.c_uint32),
-                ("gate", _Bank), ("up", _Bank), ("down", _Bank)]
+                ("gate", _Bank), ("up", _Bank), ("down", _Bank),
+                ("gating", C.c_int32), ("raw_weights", C.c_int32), ("probs_bias", C.c_void_p)]
 
 
 _lib = None
@@ -59,6 +61,7 @@ def lib():
         l.tqmoe_abi_version.restype = u32
         l.tqmoe_router.argtypes = [p, u32, p, p, u32, p, i32, i32, i32, p, e]
         l.tqmoe_topk.argtypes = [p, p, p, p, i32, i32, i32, f32, p, e]
+        l.tqmoe_topk_gated.argtypes = [p, p, i32, i32, p, p, p, i32, i32, i32, f32, p, e]
         l.tqmoe_dispatch_workspace_bytes.restype = sz
         l.tqmoe_dispatch_workspace_bytes.argtypes = [i32, i32, i32]
         l.tqmoe_dispatch.argtypes = [p, p, p, p, p, i32, i32, i32, i32, p, sz, p, e]
@@ -140,15 +143,20 @@ def moe_router(router, shared_gate, x, experts=None):
     return logits
 
 
-def moe_topk(logits, experts, topk, scale=1.0):
-    """ids [n][k] int32, weights [n][k] fp32, shared_weights [n] fp32 (moe_kernels.cuh:19-20)."""
+def moe_topk(logits, experts, topk, scale=1.0, gating=GATE_SOFTMAX, bias=None, norm=True):
+    """ids [n][k] int32, weights [n][k] fp32, shared_weights [n] fp32 (moe_kernels.cuh:19-20). gating, bias (fp32 [experts],
+    added for the choice only) and norm are moe_route's gating, probs_bias and norm_weights (src/experts/moe.cpp:22-113)."""
     n = logits.shape[0]
     ids = torch.empty((n, topk), dtype=torch.int32, device=logits.device)
     weights = torch.empty((n, topk), dtype=torch.float32, device=logits.device)
     shared = torch.empty((n,), dtype=torch.float32, device=logits.device)
     err = _err()
-    _check(lib().tqmoe_topk(_ptr(logits), _ptr(ids), _ptr(weights), _ptr(shared), experts, topk, n, float(scale), _stream(logits),
-                            C.byref(err)), err)
+    if gating == GATE_SOFTMAX and bias is None and norm:
+        _check(lib().tqmoe_topk(_ptr(logits), _ptr(ids), _ptr(weights), _ptr(shared), experts, topk, n, float(scale), _stream(logits),
+                                C.byref(err)), err)
+    else:
+        _check(lib().tqmoe_topk_gated(_ptr(logits), _ptr(bias), int(gating), int(bool(norm)), _ptr(ids), _ptr(weights), _ptr(shared), experts, topk,
+                                      n, float(scale), _stream(logits), C.byref(err)), err)
     return ids, weights, shared
 
 
@@ -402,16 +410,19 @@ def moe_combine(routed, shared, weights, shared_weights, out_type=F32):
 class MoeLayer:
     """hidden states + router weights + expert banks in, combined hidden states out, in one library call."""
 
-    def __init__(self, router, shared_gate, gate, up, down, topk, shared_ff=0, weight_scale=1.0):
+    def __init__(self, router, shared_gate, gate, up, down, topk, shared_ff=0, weight_scale=1.0, gating=GATE_SOFTMAX, probs_bias=None,
+                 norm_weights=True):
         self.router, self.shared_gate, self.gate, self.up, self.down = router, shared_gate, gate, up, down
         self.n_expert, self.hidden = router.shape
         self.ff, self.topk, self.shared_ff, self.weight_scale = gate.rows, topk, shared_ff, weight_scale
+        self.gating, self.probs_bias, self.norm_weights = gating, probs_bias, norm_weights
         self._ws = None
 
     def desc(self):
         return _Layer(C.sizeof(_Layer), self.hidden, self.ff, self.n_expert, self.topk, int(self.shared_ff > 0), self.shared_ff,
                       float(self.weight_scale), self.router.data_ptr(), self.shared_gate.data_ptr() if self.shared_gate is not None else None,
-                      _ttype(self.router), self.gate.view(), self.up.view(), self.down.view())
+                      _ttype(self.router), self.gate.view(), self.up.view(), self.down.view(), int(self.gating), int(not self.norm_weights),
+                      self.probs_bias.data_ptr() if self.probs_bias is not None else None)
 
     def workspace(self, n):
         d = self.desc()

@@ -6,7 +6,8 @@
 namespace tqmoe {
 int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);
 int32_t enqueue_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t * ext_ids, int32_t extra, const void * x,
-                     uint32_t xtype, int32_t cols, void * image, int32_t experts, int32_t topk, int32_t n, float scale, hipStream_t s);
+                     uint32_t xtype, int32_t cols, void * image, int32_t experts, int32_t topk, int32_t n, float scale, int32_t gating,
+                     const float * bias, int32_t norm, hipStream_t s);
 
 namespace {
 
@@ -71,9 +72,19 @@ Plan plan_for(const tqmoe_layer & L, int n) {
     return p;
 }
 
+// The routing fields were appended to the descriptor: one that ends before them means softmax, normalised, no bias.
+constexpr size_t kLayerBaseSize = offsetof(tqmoe_layer, gating);
+struct Routing { int32_t gating; int32_t norm; const float * bias; };
+Routing routing_of(const tqmoe_layer & L) {
+    if (L.struct_size < sizeof(tqmoe_layer)) return Routing{TQMOE_GATE_SOFTMAX, 1, nullptr};
+    return Routing{L.gating ? L.gating : int32_t(TQMOE_GATE_SOFTMAX), L.raw_weights ? 0 : 1, L.probs_bias};
+}
+
 int32_t check_layer(const tqmoe_layer * L, tqmoe_error * err) {
     const char * what = "tqmoe_layer_forward";
-    if (!L || L->struct_size < sizeof(tqmoe_layer)) return fail(err, TQMOE_E_ARG, "%s: layer descriptor missing or too small", what);
+    if (!L || L->struct_size < kLayerBaseSize) return fail(err, TQMOE_E_ARG, "%s: layer descriptor missing or too small", what);
+    const Routing rt = routing_of(*L);
+    if (rt.gating < TQMOE_GATE_SOFTMAX || rt.gating > TQMOE_GATE_SQRT_SOFTPLUS) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported gating function %d", what, rt.gating);
     if (L->hidden <= 0 || L->ff <= 0 || L->n_expert <= 0 || L->n_expert > 4096 || L->topk <= 0 || L->topk > L->n_expert || !L->router)
         return fail(err, TQMOE_E_ARG, "%s: invalid layer shape or pointer", what);
     if (L->router_type != TQMOE_F32 && L->router_type != TQMOE_BF16) return fail(err, TQMOE_E_UNSUPPORTED, "%s: router type must be F32 or BF16", what);
@@ -120,10 +131,11 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
     uint8_t * ob = static_cast<uint8_t *>(out);
 
     if (int32_t rc = tqmoe_router(L.router, L.router_type, L.shared_gate, x, xtype, logits, L.hidden, L.n_expert, n, stream, err)) return rc;
-    // one launch: softmax top-k, the ids extended by the shared expert, and (decode path) the input rows' activation image
+    // one launch: top-k, the ids extended by the shared expert, and (decode path) the input rows' activation image
     int32_t * ext = L.has_shared ? reinterpret_cast<int32_t *>(ws + p.ids_ext) : nullptr;
+    const Routing rt = routing_of(L);
     enqueue_topk(logits, ids, weights, shared_w, ext, L.n_expert, x, xtype, L.hidden, p.grouped ? nullptr : ws + p.ximage, L.n_expert, L.topk, n,
-                 L.weight_scale, static_cast<hipStream_t>(stream));
+                 L.weight_scale, rt.gating, rt.bias, rt.norm, static_cast<hipStream_t>(stream));
     if (int32_t rc = launched(err, "tqmoe_layer_forward (top-k)")) return rc;
     const int32_t * ids_ext = ext ? ext : ids;
 

@@ -319,6 +319,140 @@ template <int XT> void launch_topk(const float * logits, const TopkOut & o, int 
     else topk_lds_k<XT><<<unsigned(n), 64, size_t(e) * sizeof(float), s>>>(logits, o, e, k, scale);
 }
 
+// The reference's other gating functions (src/experts/moe.cpp:22-113): sigmoid, softmax over the selected logits only,
+// sqrt(softplus); a selection bias added for the choice but not for the weights; weights left unnormalised on request.
+// One wave per token as above; the values of lane's experts (lane, lane + 64, ...) sit in registers for up to 1024
+// experts and in LDS beyond. A taken mask replaces the "below every value" marker of the softmax kernel, since biased
+// values and raw logits have no lower bound.
+struct Gate { const float * bias; int gating, norm; };
+
+__device__ __forceinline__ float gate_value(int gating, float x) {
+    if (gating == TQMOE_GATE_SIGMOID) return 1.0f / (1.0f + expf(-x));
+    if (gating == TQMOE_GATE_SQRT_SOFTPLUS) return sqrtf(x > 0.f ? x + log1pf(expf(-x)) : log1pf(expf(x)));
+    return x;   // softmax over the selection: the logits themselves
+}
+
+// lane 0 finishes a token with more selections than lanes from the raw weights in memory, in slot order as the host does
+__device__ void gated_finish_serial(float * w, int k, const Gate & g, float scale) {
+    if (g.gating == TQMOE_GATE_SOFTMAX_WEIGHT) {
+        float mx = -INFINITY, sum = 0.f;
+        for (int s = 0; s < k; ++s) mx = fmaxf(mx, w[s]);
+        for (int s = 0; s < k; ++s) { w[s] = expf(w[s] - mx); sum += w[s]; }
+        for (int s = 0; s < k; ++s) w[s] = w[s] / sum;
+    }
+    if (g.norm) {
+        float sum = 0.f;
+        for (int s = 0; s < k; ++s) sum += w[s];
+        sum = fmaxf(sum, 6.103515625e-5f);
+        for (int s = 0; s < k; ++s) w[s] = w[s] / sum;
+    }
+    if (scale != 0.f && scale != 1.f) for (int s = 0; s < k; ++s) w[s] *= scale;
+}
+
+// sum over lanes 0 .. k - 1 in lane order (the host's slot order), k <= 64
+__device__ __forceinline__ float slot_order_sum(float v, int k) {
+    float sum = 0.f;
+    for (int s = 0; s < k; ++s) sum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), s));
+    return sum;
+}
+
+template <int R, int XT>   // R = 0: values in LDS, ceil(e / 64) per lane
+__global__ __launch_bounds__(64) void topk_gated_k(const float * __restrict__ logits, TopkOut o, Gate g, int e, int k, float scale) {
+    extern __shared__ float gated_lds[];
+    constexpr bool kLds = R == 0;
+    constexpr int kRegs = kLds ? 1 : R;
+    const int token = blockIdx.x, lane = threadIdx.x;
+    const float * x = logits + int64_t(token) * (e + 1);
+    const int per_lane = kLds ? (e + 63) / 64 : R;
+    float p_reg[kRegs], v_reg[kRegs];
+    float * p_lds = gated_lds + lane, * v_lds = gated_lds + 64 * per_lane + lane;   // entry r of a lane at [64 r]: no bank conflicts
+    auto P = [&](int r) -> float & { if constexpr (kLds) return p_lds[64 * r]; else return p_reg[r]; };
+    auto V = [&](int r) -> float & { if constexpr (kLds) return v_lds[64 * r]; else return v_reg[r]; };
+
+    const float shared_logit = o.shared_weights ? x[e] : 0.f;
+    float m = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < per_lane; ++r) { const int j = lane + 64 * r; P(r) = j < e ? x[j] : -INFINITY; m = fmaxf(m, P(r)); }
+    if (g.gating == TQMOE_GATE_SOFTMAX) {
+        m = wave_max_all(m);
+        float sum = 0.f;
+#pragma unroll
+        for (int r = 0; r < per_lane; ++r) { const int j = lane + 64 * r; P(r) = j < e ? expf(P(r) - m) : 0.f; sum += P(r); }
+        sum = wave_sum_all(sum);
+#pragma unroll
+        for (int r = 0; r < per_lane; ++r) P(r) = P(r) / sum;
+    } else {
+#pragma unroll
+        for (int r = 0; r < per_lane; ++r) P(r) = gate_value(g.gating, P(r));
+    }
+#pragma unroll
+    for (int r = 0; r < per_lane; ++r) { const int j = lane + 64 * r; V(r) = g.bias && j < e ? P(r) + g.bias[j] : P(r); }
+    uint64_t taken = 0;   // bit r: entry r of this lane is chosen already or lies past the end
+#pragma unroll
+    for (int r = 0; r < per_lane; ++r) if (lane + 64 * r >= e) taken |= uint64_t(1) << r;
+
+    float selected = 0.f, my_w = 0.f;   // lane s keeps selection s
+    int my_id = 0;
+    for (int s = 0; s < k; ++s) {
+        float bv = -INFINITY;
+        int bi = 0x7FFFFFFF;
+#pragma unroll
+        for (int r = 0; r < per_lane; ++r)   // strict: the lowest index of equal values
+            if (!(taken >> r & 1) && (bi == 0x7FFFFFFF || V(r) > bv)) { bv = V(r); bi = lane + 64 * r; }
+        const float top = wave_max_all(bv);
+        const int best = wave_min_all(bv == top && bi != 0x7FFFFFFF ? bi : 0x7FFFFFFF);
+        float wv = 0.f;
+#pragma unroll
+        for (int r = 0; r < per_lane; ++r) if (lane + 64 * r == best) { wv = P(r); taken |= uint64_t(1) << r; }
+        const float w = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv), best & 63));   // the unbiased value
+        if (lane == (s & 63)) { my_id = best; my_w = w; }
+        if (k > 64 && (s & 63) == 63) {   // more selections than lanes: a full set goes out before the lanes are reused
+            o.ids[int64_t(token) * k + s - 63 + lane] = my_id;
+            o.weights[int64_t(token) * k + s - 63 + lane] = my_w;
+            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + s - 63 + lane] = my_id;
+        }
+        selected += w;   // slot order, as the host sums the selected weights
+    }
+    if (k <= 64) {
+        if (g.gating == TQMOE_GATE_SOFTMAX_WEIGHT) {
+            const float mx = wave_max_all(lane < k ? my_w : -INFINITY);
+            my_w = lane < k ? expf(my_w - mx) : 0.f;
+            my_w = my_w / slot_order_sum(my_w, k);
+            selected = slot_order_sum(my_w, k);
+        }
+        if (g.norm) my_w = my_w / fmaxf(selected, 6.103515625e-5f);
+        if (scale != 0.f && scale != 1.f) my_w *= scale;
+        if (lane < k) {
+            o.ids[int64_t(token) * k + lane] = my_id;
+            o.weights[int64_t(token) * k + lane] = my_w;
+            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + lane] = my_id;
+        }
+    } else {
+        const int done = k & ~63;             // the last partial set
+        if (lane < k - done) {
+            o.ids[int64_t(token) * k + done + lane] = my_id;
+            o.weights[int64_t(token) * k + done + lane] = my_w;
+            if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + done + lane] = my_id;
+        }
+        __threadfence_block();
+        if (lane == 0) gated_finish_serial(o.weights + int64_t(token) * k, k, g, scale);
+    }
+    if (lane == 0) {
+        if (o.shared_weights) o.shared_weights[token] = 1.f / (1.f + expf(-shared_logit));
+        if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + k] = o.extra;
+    }
+    if (o.image) topk_quantise_row<XT>(o, token, lane);
+}
+
+template <int XT> void launch_topk_gated(const float * logits, const TopkOut & o, const Gate & g, int e, int k, int n, float scale, hipStream_t s) {
+    if (e <= 64) topk_gated_k<1, XT><<<unsigned(n), 64, 0, s>>>(logits, o, g, e, k, scale);
+    else if (e <= 128) topk_gated_k<2, XT><<<unsigned(n), 64, 0, s>>>(logits, o, g, e, k, scale);
+    else if (e <= 256) topk_gated_k<4, XT><<<unsigned(n), 64, 0, s>>>(logits, o, g, e, k, scale);
+    else if (e <= 512) topk_gated_k<8, XT><<<unsigned(n), 64, 0, s>>>(logits, o, g, e, k, scale);
+    else if (e <= 1024) topk_gated_k<16, XT><<<unsigned(n), 64, 0, s>>>(logits, o, g, e, k, scale);
+    else topk_gated_k<0, XT><<<unsigned(n), 64, size_t((e + 63) / 64) * 128 * sizeof(float), s>>>(logits, o, g, e, k, scale);
+}
+
 // --------------------------------------------------------------------------------------------------- dispatch
 // Stable counting sort of the assignments by expert. Chunks of kChunk consecutive assignments; pass 1 counts each
 // chunk's experts in LDS, pass 2 turns the per-chunk counts into exclusive prefixes (and counts / offsets), pass 3
@@ -473,12 +607,23 @@ extern "C" int32_t tqmoe_router(const void * router, uint32_t wtype, const void 
 // top-k with the optional extras of the whole-layer path: extended ids and the input rows' activation image
 namespace tqmoe {
 int32_t enqueue_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t * ext_ids, int32_t extra, const void * x,
-                     uint32_t xtype, int32_t cols, void * image, int32_t experts, int32_t topk, int32_t n, float scale, hipStream_t s) {
+                     uint32_t xtype, int32_t cols, void * image, int32_t experts, int32_t topk, int32_t n, float scale, int32_t gating,
+                     const float * bias, int32_t norm, hipStream_t s) {
     const TopkOut o{ids, weights, shared_weights, ext_ids, extra, x, static_cast<uint8_t *>(image), cols};
-    switch (image ? xtype : uint32_t(TQMOE_F32)) {
-        case TQMOE_F32: launch_topk<TQMOE_F32>(logits, o, experts, topk, n, scale, s); break;
-        case TQMOE_F16: launch_topk<TQMOE_F16>(logits, o, experts, topk, n, scale, s); break;
-        default: launch_topk<TQMOE_BF16>(logits, o, experts, topk, n, scale, s); break;
+    const uint32_t xt = image ? xtype : uint32_t(TQMOE_F32);
+    if (gating == TQMOE_GATE_SOFTMAX && !bias && norm) {   // the common case has its own kernel
+        switch (xt) {
+            case TQMOE_F32: launch_topk<TQMOE_F32>(logits, o, experts, topk, n, scale, s); break;
+            case TQMOE_F16: launch_topk<TQMOE_F16>(logits, o, experts, topk, n, scale, s); break;
+            default: launch_topk<TQMOE_BF16>(logits, o, experts, topk, n, scale, s); break;
+        }
+        return 0;
+    }
+    const Gate g{bias, gating, norm};
+    switch (xt) {
+        case TQMOE_F32: launch_topk_gated<TQMOE_F32>(logits, o, g, experts, topk, n, scale, s); break;
+        case TQMOE_F16: launch_topk_gated<TQMOE_F16>(logits, o, g, experts, topk, n, scale, s); break;
+        default: launch_topk_gated<TQMOE_BF16>(logits, o, g, experts, topk, n, scale, s); break;
     }
     return 0;
 }
@@ -489,8 +634,20 @@ extern "C" int32_t tqmoe_topk(const float * logits, int32_t * ids, float * weigh
     if (!logits || !ids || !weights || experts <= 0 || experts > 4096 || topk <= 0 || topk > experts || n <= 0)
         return fail(err, TQMOE_E_ARG, "tqmoe_topk: invalid shape or pointer");
     if (int32_t rc = need_device(err, "tqmoe_topk")) return rc;
-    enqueue_topk(logits, ids, weights, shared_weights, nullptr, 0, nullptr, TQMOE_F32, 0, nullptr, experts, topk, n, scale, static_cast<hipStream_t>(stream));
+    enqueue_topk(logits, ids, weights, shared_weights, nullptr, 0, nullptr, TQMOE_F32, 0, nullptr, experts, topk, n, scale, TQMOE_GATE_SOFTMAX, nullptr, 1,
+                 static_cast<hipStream_t>(stream));
     return launched(err, "tqmoe_topk");
+}
+
+extern "C" int32_t tqmoe_topk_gated(const float * logits, const float * probs_bias, int32_t gating, int32_t norm_weights, int32_t * ids, float * weights,
+                                    float * shared_weights, int32_t experts, int32_t topk, int32_t n, float scale, void * stream, tqmoe_error * err) {
+    if (!logits || !ids || !weights || experts <= 0 || experts > 4096 || topk <= 0 || topk > experts || n <= 0)
+        return fail(err, TQMOE_E_ARG, "tqmoe_topk_gated: invalid shape or pointer");
+    if (gating < TQMOE_GATE_SOFTMAX || gating > TQMOE_GATE_SQRT_SOFTPLUS) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_topk_gated: unsupported gating function %d", gating);
+    if (int32_t rc = need_device(err, "tqmoe_topk_gated")) return rc;
+    enqueue_topk(logits, ids, weights, shared_weights, nullptr, 0, nullptr, TQMOE_F32, 0, nullptr, experts, topk, n, scale, gating, probs_bias, norm_weights != 0,
+                 static_cast<hipStream_t>(stream));
+    return launched(err, "tqmoe_topk_gated");
 }
 
 extern "C" size_t tqmoe_dispatch_workspace_bytes(int32_t experts, int32_t n, int32_t topk) {

@@ -560,6 +560,69 @@ __global__ __launch_bounds__(256) void dispatch_place_k(const int * __restrict__
     place_chunk(ids, offsets, chunk_prefix + int64_t(blockIdx.x) * E, perm, groups, capacity, blockIdx.x * kChunk, A, E, run);
 }
 
+// Pass 2 and 3 in one launch for up to kWideExperts experts: a block of sixteen waves takes a chunk, one wave per 64
+// consecutive assignments. Every block sums the per-chunk counts itself (the chunks before it: where its assignments
+// start inside each expert; all chunks: the experts' offsets), the waves rank their assignments with ballots all at
+// once and leave their group sizes in a per-wave histogram, and a prefix over the waves in index order gives every
+// assignment its place. Nothing is left to the order of atomics.
+constexpr int kWideExperts = 1024, kWideWaves = kChunk / 64;
+
+__global__ __launch_bounds__(1024) void dispatch_place_wide_k(const int * __restrict__ ids, const int * __restrict__ chunk_counts, int * __restrict__ counts,
+                                                              int * __restrict__ offsets, int * __restrict__ perm, int * __restrict__ groups, int capacity,
+                                                              int A, int E, int chunks) {
+    extern __shared__ int sm[];   // start E + 1 | total E | scratch 1024 | hist kWideWaves x E
+    int * start = sm, * total = sm + E + 1, * scratch = total + E, * hist = scratch + 1024;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, chunk = blockIdx.x;
+    for (int j = tid; j < E; j += 1024) {
+        int before = 0, all = 0;
+        for (int b0 = 0; b0 < chunks; b0 += 16) {   // sixteen loads in flight: the loop is latency, not bandwidth
+            int v[16];
+#pragma unroll
+            for (int q = 0; q < 16; ++q) v[q] = b0 + q < chunks ? chunk_counts[int64_t(b0 + q) * E + j] : 0;
+#pragma unroll
+            for (int q = 0; q < 16; ++q) { all += v[q]; before += b0 + q < chunk ? v[q] : 0; }
+        }
+        total[j] = all;
+        hist[j] = before;          // parked here until the offsets are known
+    }
+    for (int j = tid; j < kWideWaves * E; j += 1024) if (j >= E) hist[j] = 0;
+    __syncthreads();
+    // the assignment's rank among the wave's earlier lanes of the same expert, and the size of its group
+    const int a = chunk * kChunk + tid;
+    int e = a < A ? ids[a] : -1;
+    if (e >= E) e = -1;
+    int rank = 0, size = 0;
+    bool last = false;
+    unsigned long long todo = __ballot(e >= 0);
+    while (todo) {
+        const int leader = __ffsll(todo) - 1;
+        const int v = __shfl(e, leader, 64);
+        const unsigned long long same = __ballot(e == v);
+        if (e == v) {
+            rank = __popcll(same & ((1ull << lane) - 1ull));
+            size = __popcll(same);
+            last = (63 - __clzll(same)) == lane;
+        }
+        todo &= ~same;
+    }
+    const int before_e = e >= 0 ? hist[e] : 0;   // row 0 of hist still holds the chunks before this one
+    __syncthreads();
+    for (int j = tid; j < E; j += 1024) hist[j] = 0;
+    block_exclusive_scan(total, start, E, scratch);   // ends with a barrier
+    if (e >= 0 && last) hist[wave * E + e] = size;
+    __syncthreads();
+    if (e >= 0) {
+        int slot = before_e + rank;
+        for (int w = 0; w < wave; ++w) slot += hist[w * E + e];
+        perm[start[e] + slot] = a;
+        if (groups && slot < capacity) groups[int64_t(e) * capacity + slot] = a;
+    }
+    if (chunk == 0) {
+        for (int j = tid; j < E; j += 1024) { counts[j] = total[j]; offsets[j] = start[j]; }
+        if (tid == 0) offsets[E] = start[E];
+    }
+}
+
 // A <= kChunk: everything in one block
 __global__ __launch_bounds__(256) void dispatch_small_k(const int * __restrict__ ids, int * __restrict__ counts, int * __restrict__ offsets,
                                                         int * __restrict__ perm, int * __restrict__ groups, int capacity, int A, int E) {
@@ -674,6 +737,14 @@ extern "C" int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t
         return fail(err, TQMOE_E_WORKSPACE, "tqmoe_dispatch: workspace of %zu bytes needed", tqmoe_dispatch_workspace_bytes(experts, n, topk));
     int * cc = static_cast<int *>(workspace);
     dispatch_count_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, cc, A, experts);
+    if (experts <= kWideExperts) {
+        const size_t lds = size_t(2 * experts + 1 + 1024 + kWideWaves * experts) * sizeof(int);
+        static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(&dispatch_place_wide_k), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                           int((2 * kWideExperts + 1 + 1024 + kWideWaves * kWideExperts) * sizeof(int)));
+        (void)once;
+        dispatch_place_wide_k<<<unsigned(chunks), 1024, lds, s>>>(ids, cc, counts, offsets, perm, groups, capacity, A, experts, chunks);
+        return launched(err, "tqmoe_dispatch");
+    }
     dispatch_scan_k<<<1, 1024, size_t(experts + 1024) * sizeof(int), s>>>(cc, counts, offsets, chunks, experts);
     dispatch_place_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, offsets, cc, perm, groups, capacity, A, experts);
     return launched(err, "tqmoe_dispatch");

@@ -169,6 +169,63 @@ __global__ __launch_bounds__(256) void group_rows_i8_k(const void * __restrict__
     }
 }
 
+// The same for row lengths of 512, 1024 or 2048: one block per row tile. A wave quantises eight rows out of registers
+// (one read of the input) into an LDS copy of the tile, every 32-byte block already in operand order; then lane (g, r)
+// of every wave moves the 16 bytes of row r, half g of one k-step at a time, so each k-step's 1 KB leaves as one fully
+// coalesced store instead of 256 scattered dwords.
+template <int XT, int GPL>   // groups of 8 values per lane: cols = 512 GPL
+__global__ __launch_bounds__(256) void group_rows_i8_tile_k(const void * __restrict__ x, int cols, const int * __restrict__ counts, const int * __restrict__ offsets,
+                                                              const int * __restrict__ perm, int experts, int xdiv, int8_t * __restrict__ q, float * __restrict__ scale,
+                                                              Plan plan) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t tile_rows[];   // [32][cols + 16]
+    const int tile_index = int(blockIdx.x);
+    if (tile_index >= plan.tile_base[experts]) return;
+    const int e = owner_of(plan.tile_base, experts, tile_index);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, stride = cols + 16;
+    const int cnt = counts[e], first = (tile_index - plan.tile_base[e]) * 32, off = offsets[e];
+    constexpr int kBatch = 8 / GPL;   // rows whose loads are in flight together: 64 values per lane
+    for (int r0 = wave * 8; r0 < wave * 8 + 8; r0 += kBatch) {
+        if (first + r0 >= cnt) break;
+        float v[kBatch][GPL][8];
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const int i = min(first + r0 + b, cnt - 1);          // past the count: a valid row again, not stored
+            const int64_t row = perm[off + i] / xdiv;
+#pragma unroll
+            for (int gq = 0; gq < GPL; ++gq) load8<XT>(x, row * cols + (lane + 64 * gq) * 8, v[b][gq]);
+        }
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const int r = r0 + b;
+            float amax = 0.f;
+#pragma unroll
+            for (int gq = 0; gq < GPL; ++gq)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[b][gq][j]));
+            amax = wave_max(amax);
+            const float mul = amax > 0.f ? 127.f / amax : 0.f;
+            if (first + r < cnt) {
+                if (lane == 0) scale[int64_t(tile_index) * 32 + r] = amax / 127.f;
+#pragma unroll
+                for (int gq = 0; gq < GPL; ++gq) {
+                    const int gi = lane + 64 * gq, sub = gi >> 2, d0 = 2 * (gi & 3);
+                    uint32_t wd[2] = {0, 0};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) wd[j >> 2] |= uint32_t(__float2int_rn(v[b][gq][j] * mul) & 0xFF) << (8 * (j & 3));
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) *reinterpret_cast<uint32_t *>(tile_rows + r * stride + sub * 32 + plane_pos(d0 + h) * 4) = wd[h];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int r = lane & 31, g = lane >> 5;
+    if (first + r >= cnt) return;                     // rows past the expert's count are left as they are
+    uint4 * dst = reinterpret_cast<uint4 *>(q + int64_t(tile_index) * 32 * cols) + lane;
+    const int S = cols / 32;
+    for (int ks = wave; ks < S; ks += 4) dst[ks * 64] = *reinterpret_cast<const uint4 *>(tile_rows + r * stride + ks * 32 + g * 16);
+}
+
 // The same grouped operand from rows that are already int8 (quant_rows_i8_k's output: one scale per row, the bytes of every
 // 32-block in operand order): a pure copy. One block per row tile; lane (g, r) of every wave moves the 16 bytes of row r,
 // half g of one k-step at a time, so each k-step's 1 KB is written by one fully coalesced store. When several
@@ -571,6 +628,21 @@ int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const in
     const int64_t tiles = grouped_row_tiles(assignments, experts);
     const Plan plan = plan_at(scale, tiles * 32, experts);
     plan_k<<<1, 64, 0, s>>>(counts, experts, const_cast<int *>(plan.tile_base), const_cast<int *>(plan.chunk_base), plan.counters);
+    if (cols == 512 || cols == 1024 || cols == 2048) {
+        const size_t lds = size_t(32) * size_t(cols + 16);
+        auto launch = [&](auto kernel) {
+            if (lds > 65536) (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 32 * (2048 + 16));
+            kernel<<<unsigned(tiles), 256, lds, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan);
+        };
+#define TQMOE_GROUP_TILE(XT) (cols == 512 ? launch(group_rows_i8_tile_k<XT, 1>) : cols == 1024 ? launch(group_rows_i8_tile_k<XT, 2>) : launch(group_rows_i8_tile_k<XT, 4>))
+        switch (xtype) {
+            case TQMOE_F32: TQMOE_GROUP_TILE(TQMOE_F32); break;
+            case TQMOE_F16: TQMOE_GROUP_TILE(TQMOE_F16); break;
+            default: TQMOE_GROUP_TILE(TQMOE_BF16); break;
+        }
+#undef TQMOE_GROUP_TILE
+        return 0;
+    }
     const unsigned blocks = unsigned(tiles * 4);
     switch (xtype) {
         case TQMOE_F32: group_rows_i8_k<TQMOE_F32><<<blocks, 256, 0, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan); break;

@@ -250,6 +250,26 @@ int32_t tqmoe_combine_strided_f16(const void * routed, int32_t slots, const void
                                   const float * weights, const float * shared_weights, void * out, uint32_t otype,
                                   int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err);
 
+/* tqmoe_combine_strided with the residual stream added: out = bf16(bf16(sum) + residual), the two roundings of the
+ * reference's moe_sum into bf16 followed by add_sumsq (src/models/qwen/qwen35/qwen35_forward.cpp:1248-1250,
+ * src/formats/weight/quant_tq3.inc:303-313). routed / shared: F32 or F16 rows (rtype); residual, out: device
+ * [n][hidden] bf16. out may be the residual buffer itself (every element is read before it is written). */
+int32_t tqmoe_combine_residual(const void * routed, uint32_t rtype, int32_t slots, const void * shared, int64_t shared_ld,
+                               const float * weights, const float * shared_weights, const void * residual, void * out,
+                               int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err);
+
+/* ------------------------------------------------------------------------------------- the step before the layer
+ * Residual add and RMS norm of the rows the router and the experts read, one launch for the reference's pair
+ * add_sumsq + norm_h (Qwen35Engine::ffn_block, qwen35_forward.cpp:1114-1115; quant_tq3.inc:303-313, quant.cu:647-661):
+ *   rows[t][i]   = bf16(rows[t][i] + residual[t][i])            in place; skipped when residual is NULL
+ *   normed[t][i] = bf16((rows[t][i] * inv_t) * weight[i]),      inv_t = 1 / sqrt(mean_i rows[t][i]^2 + eps)
+ * rows, residual: device [n][hidden] bf16; weight: device [hidden] fp32; normed: device [n][hidden] of ntype (BF16,
+ * or F16 holding the bf16-rounded value as the reference's fp16 activations do). hidden % 8 == 0. The sum of squares
+ * is accumulated in fp32 in this kernel's own order: normed values can differ from the reference's by one bf16 step
+ * where they sit on a rounding boundary; the updated rows are bit-exact. */
+int32_t tqmoe_add_rmsnorm(void * rows, const void * residual, const float * weight, float eps, void * normed,
+                          uint32_t ntype, int32_t hidden, int32_t n, void * stream, tqmoe_error * err);
+
 /* ---------------------------------------------------------------------------------------------- whole layer
  * hidden states + router weights + expert banks in, combined hidden states out: the sequence of
  * Qwen35Engine::ffn_block steps 2-9 (src/models/qwen/qwen35/qwen35_forward.cpp:1123-1248) and of the Flash-Next
@@ -279,6 +299,13 @@ size_t  tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t n);
 int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x, uint32_t xtype, int32_t n, void * out,
                             uint32_t otype, int32_t * ids_out, float * weights_out, float * logits_out,
                             void * workspace, size_t workspace_bytes, void * stream, tqmoe_error * err);
+
+/* tqmoe_layer_forward with the residual stream added to the result: out[t] = bf16(bf16(layer(x)[t]) + residual[t]), the
+ * add that follows the layer in the reference (qwen35_forward.cpp:1250). residual, out: device [n][hidden] bf16; out may
+ * be the residual buffer. */
+int32_t tqmoe_layer_forward_residual(const tqmoe_layer * layer, const void * x, uint32_t xtype, const void * residual,
+                                     int32_t n, void * out, int32_t * ids_out, float * weights_out, float * logits_out,
+                                     void * workspace, size_t workspace_bytes, void * stream, tqmoe_error * err);
 
 #ifdef __cplusplus
 }

@@ -65,6 +65,18 @@ inline void moe_route(const MoeRouting & cfg, const float * logits, const float 
     check(tqmoe_topk_gated(logits, probs_bias, cfg.gating, cfg.norm_weights ? 1 : 0, ids, weights, shared_weights, cfg.n_expert, cfg.n_expert_used, n,
                            cfg.weight_scale, stream, &e), e);
 }
+// The step in front of the layer, the pair add_sumsq + norm_h of Qwen35Engine::ffn_block (qwen35_forward.cpp:1114-1115) in
+// one launch: m += residual (bf16, in place; residual may be null), xh = fp16(bf16(m * inv * w)). No partial-sum buffer.
+inline void add_norm_h(void * m_bf16, const void * residual_bf16, const float * w, float eps, void * xh_f16, int hidden, int n, void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_add_rmsnorm(m_bf16, residual_bf16, w, eps, xh_f16, TQMOE_F16, hidden, n, stream, &e), e);
+}
+// moe_sum followed by the residual add (qwen35_forward.cpp:1248-1250): x = bf16(bf16(sum) + m); x may be m's buffer
+inline void moe_sum_add(const float * routed, const float * shared, const float * weights, const float * shared_weights, const void * m_bf16, void * x_bf16,
+                        int hidden, int topk, int n, void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_combine_residual(routed, TQMOE_F32, topk, shared, hidden, weights, shared_weights, m_bf16, x_bf16, hidden, topk, n, stream, &e), e);
+}
 // moe_group (moe_kernels.cuh:29): groups [experts][n], counts [experts]. The lists are ascending inside each expert
 // (the reference's device version is atomic-ordered). `scratch` holds the offsets, the permutation and the workspace:
 // moe_group_scratch_bytes() device bytes.

@@ -51,6 +51,7 @@ _lib.tqo_route_min_gap_ulps.argtypes = [C.c_int, C.c_int, _p]
 _lib.tqo_shared_weight.restype = C.c_float
 _lib.tqo_shared_weight.argtypes = [C.c_float]
 _lib.tqo_dispatch.argtypes = [_p, C.c_int, C.c_int, _p, _p, _p]
+_lib.tqo_add_rmsnorm.argtypes = [_p, _p, _p, C.c_float, C.c_int, C.c_int, _p]
 _lib.tqo_expert_ffn.restype = None
 _lib.tqo_expert_ffn.argtypes = [_p, C.c_int, _p, _p, _p, C.c_int, C.c_float, C.c_int, _p]
 _lib.tqo_combine.restype = None
@@ -107,6 +108,11 @@ def to_bf16(a):
     u = a.view(np.uint32)
     r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
     return r, (r.astype(np.uint32) << 16).view(np.float32).reshape(a.shape)
+
+
+def from_bf16(bits):
+    """uint16 bf16 bits -> fp32 values."""
+    return (np.asarray(bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
 
 
 def dequantize(wtype, raw, n):
@@ -195,6 +201,18 @@ def quant_act_row_e4m3(x):
     s = np.empty(1, np.float32)
     _lib.tqo_quant_act_row_e4m3(_ptr(x), x.size, _ptr(q), _ptr(s))
     return q, float(s[0])
+
+
+def add_rmsnorm(rows_bits, residual_bits, weight, eps):
+    """rows_bits, residual_bits: uint16 bf16 [n][H] (residual may be None); returns (updated rows bits, normed bf16 bits)."""
+    rows = np.array(rows_bits, dtype=np.uint16, order="C", copy=True)
+    res = _c(residual_bits, np.uint16) if residual_bits is not None else None
+    w = _c(weight, np.float32)
+    n, h = rows.shape
+    out = np.empty((n, h), np.uint16)
+    if _lib.tqo_add_rmsnorm(_ptr(rows), _ptr(res), _ptr(w), float(eps), h, n, _ptr(out)):
+        raise ValueError("tqo_add_rmsnorm: hidden must be a positive multiple of 256")
+    return rows, out
 
 
 def layer_forward(x, logits, gate, up, down, wtype, hidden, ff, n_expert, k, shared_ff=0, act_mode=0, threads=8, gating=GATE_SOFTMAX,

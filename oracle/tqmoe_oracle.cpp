@@ -509,6 +509,56 @@ int tqo_dispatch(const int32_t * ids, int A, int E, int32_t * counts, int32_t * 
     return 0;
 }
 
+// ------------------------------------------------------------------------- residual add and RMS norm before the layer
+namespace {
+// __shfl_xor butterfly over 32 lanes with offsets 16, 8, 4, 2, 1: every lane ends with the same value
+float butterfly32(float * v) {
+    for (int o = 16; o; o >>= 1) {
+        float t[32];
+        for (int i = 0; i < 32; ++i) t[i] = v[i] + v[i ^ o];
+        for (int i = 0; i < 32; ++i) v[i] = t[i];
+    }
+    return v[0];
+}
+}  // namespace
+
+int tqo_add_rmsnorm(uint16_t * rows, const uint16_t * residual, const float * weight, float eps, int hidden, int n,
+                    uint16_t * normed_bf16) {
+    if (hidden <= 0 || hidden % 256 || n <= 0) return -1;
+    const int nparts = hidden / 256;
+    std::vector<float> partial(static_cast<size_t>(nparts));
+    for (int t = 0; t < n; ++t) {
+        uint16_t * m = rows + size_t(t) * hidden;
+        for (int b = 0; b < nparts; ++b) {  // quant_tq3.inc:303-313 with block_sum256 (:293-301)
+            float warp_sum[8];
+            for (int w = 0; w < 8; ++w) {
+                float sq[32];
+                for (int l = 0; l < 32; ++l) {
+                    const int i = b * 256 + w * 32 + l;
+                    if (residual) m[i] = tqo_float_to_bf16(tqo_bf16_to_float(m[i]) + tqo_bf16_to_float(residual[size_t(t) * hidden + i]));
+                    const float v = tqo_bf16_to_float(m[i]);
+                    sq[l] = v * v;
+                }
+                warp_sum[w] = butterfly32(sq);
+            }
+            float s = 0.f;
+            for (int w = 0; w < 8; ++w) s += warp_sum[w];
+            partial[size_t(b)] = s;
+        }
+        float lanes[32];  // quant.cu:651-656
+        for (int l = 0; l < 32; ++l) {
+            float s = 0.f;
+            for (int i = l; i < nparts; i += 32) s += partial[size_t(i)];
+            lanes[l] = s;
+        }
+        const float total = butterfly32(lanes);
+        const float inv = 1.0f / std::sqrt(total / float(hidden) + eps);
+        for (int i = 0; i < hidden; ++i)  // quant.cu:660: rounded to bf16 whatever the storage
+            normed_bf16[size_t(t) * hidden + i] = tqo_float_to_bf16(tqo_bf16_to_float(m[i]) * inv * weight[i]);
+    }
+    return 0;
+}
+
 // -------------------------------------------------------------------------------------------- FFN and combine
 void tqo_expert_ffn(const float * x, int hidden, const float * w_gate, const float * w_up, const float * w_down,
                     int ff, float swiglu_clamp, int clamp_gate, float * out) {

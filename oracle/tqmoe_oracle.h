@@ -17,6 +17,9 @@
  *   tqo_shared_weight                      src/experts/moe.cu:92 (sigmoid of logits column E)
  *   tqo_dispatch                           src/models/qwen/qwen4exp/prefill_plan.hpp:63-74 (ascending assignment
  *                                          order inside each expert), counts as src/experts/moe.cu:168-176
+ *   tqo_add_rmsnorm                        src/formats/weight/quant_tq3.inc:293-313 (add, sums of squares) and
+ *                                          src/formats/weight/quant.cu:647-661 (norm), as called by
+ *                                          src/models/qwen/qwen35/qwen35_forward.cpp:1114-1115
  *   tqo_expert_ffn                         src/experts/moe.cpp:115-155
  *   tqo_combine                            src/experts/moe.cpp:157-163 and src/experts/moe.cu:224-234 (shared row)
  *   tqo_router_logits                      src/experts/moe.cu:17-33 (row E = shared gate), bf16 variant
@@ -30,7 +33,8 @@
  * 65,536 halves against hardware conversion; the 256 E4M3 codes against the closed form; NVFP4G against the closed
  * form value = e2m1 * e4m3(scale) * global; routing against an independent max-scan selection, scipy softmax and
  * the closed forms of the reference's tests/moe.cpp; dispatch against a brute-force stable sort; FFN / combine /
- * layer against float64 numpy on the decoded weights; and, where it builds, against the reference's own objects in
+ * layer against float64 numpy on the decoded weights; the residual add and norm against float64 numpy and closed
+ * forms (constant rows, zero rows, the eps limit); and, where it builds, against the reference's own objects in
  * oracle/_ref.
  *
  * PARITY UNPINNED: tqo_quantize (all formats). The reference holds no quantiser (it calls an external libggml that
@@ -93,6 +97,14 @@ int tqo_router_logits(const void * w, uint32_t wtype, const void * shared_gate, 
 /* Declared activation quantisers of the lossy operand paths. */
 void tqo_quant_act_row_i8(const float * x, int cols, int8_t * q, float * scale);     /* scale = amax/127 */
 void tqo_quant_act_row_e4m3(const float * x, int cols, uint8_t * q, float * scale);  /* scale = amax/448 */
+
+/* Residual add and RMS norm in front of the layer, the reference's add_sumsq + norm_h with their summation order
+ * (per 256 values: xor butterflies over 32, then the eight sums in order; the blocks' sums strided over 32 lanes and
+ * a butterfly): rows (bf16 bits, [n][hidden]) += residual in place (skipped when null), normed_bf16 = bf16((row * inv) *
+ * weight) with inv = 1 / sqrt(sum / hidden + eps) (the reference's device rsqrtf is approximate; this one is exact).
+ * hidden must be a multiple of 256. */
+int tqo_add_rmsnorm(uint16_t * rows, const uint16_t * residual, const float * weight, float eps, int hidden, int n,
+                    uint16_t * normed_bf16);
 
 /* Whole layer on the host.
  *   x fp32 [n][H] (already rounded to the activation type by the caller), logits [n][E + 1] given (so that the

@@ -78,6 +78,9 @@ def lib():
         l.tqmoe_expert_down.argtypes = [C.POINTER(_Bank), p, p, p, i32, i32, i32, i32, p, e]
         l.tqmoe_combine_strided.argtypes = [p, i32, p, i64, p, p, p, u32, i32, i32, i32, p, e]
         l.tqmoe_combine_strided_f16.argtypes = [p, i32, p, i64, p, p, p, u32, i32, i32, i32, p, e]
+        l.tqmoe_combine_residual.argtypes = [p, u32, i32, p, i64, p, p, p, p, i32, i32, i32, p, e]
+        l.tqmoe_add_rmsnorm.argtypes = [p, p, p, f32, p, u32, i32, i32, p, e]
+        l.tqmoe_layer_forward_residual.argtypes = [C.POINTER(_Layer), p, u32, p, i32, p, p, p, p, p, sz, p, e]
         l.tqmoe_quant_rows_i8.argtypes = [p, u32, i64, i32, p, p, p, e]
         l.tqmoe_grouped_rows.restype = i64
         l.tqmoe_grouped_rows.argtypes = [i64, i32]
@@ -407,6 +410,28 @@ def moe_combine(routed, shared, weights, shared_weights, out_type=F32):
     return out
 
 
+def add_rmsnorm(rows, residual, weight, eps, out_dtype=torch.bfloat16):
+    """rows (bf16 [n][H], updated in place: += residual when given) -> normed rows of out_dtype (bf16 or fp16): the
+    reference's add_sumsq + norm_h in front of the layer (qwen35_forward.cpp:1114-1115)."""
+    n, h = rows.shape
+    normed = torch.empty((n, h), dtype=out_dtype, device=rows.device)
+    err = _err()
+    _check(lib().tqmoe_add_rmsnorm(_ptr(rows), _ptr(residual), _ptr(weight), float(eps), _ptr(normed), _ttype(normed), h, n, _stream(rows), C.byref(err)), err)
+    return normed
+
+
+def moe_combine_residual(routed, shared, weights, shared_weights, residual, out=None):
+    """out = bf16(bf16(weighted sum) + residual) (moe_sum then add_sumsq, qwen35_forward.cpp:1248-1250). routed: fp32 or fp16
+    [n][topk][H]; shared: [n][H] of the same type or None."""
+    n, topk, h = routed.shape
+    if out is None:
+        out = torch.empty((n, h), dtype=torch.bfloat16, device=routed.device)
+    err = _err()
+    _check(lib().tqmoe_combine_residual(_ptr(routed), _ttype(routed), topk, _ptr(shared), h, _ptr(weights), _ptr(shared_weights), _ptr(residual), _ptr(out),
+                                        h, topk, n, _stream(routed), C.byref(err)), err)
+    return out
+
+
 class MoeLayer:
     """hidden states + router weights + expert banks in, combined hidden states out, in one library call."""
 
@@ -433,9 +458,12 @@ class MoeLayer:
             self._ws = torch.empty(need, dtype=torch.uint8, device=self.router.device)
         return self._ws
 
-    def forward(self, x, out_type=F32, return_routing=False, out=None):
+    def forward(self, x, out_type=F32, return_routing=False, out=None, residual=None):
+        """residual (bf16 [n][H]): added to the result, which is then bf16: bf16(bf16(layer(x)) + residual)."""
         n = x.shape[0]
         ws = self.workspace(n)
+        if residual is not None:
+            out_type = BF16
         if out is None:
             out = torch.empty((n, self.hidden), dtype=_OUT_TYPE[out_type], device=x.device)
         ids = weights = logits = None
@@ -445,6 +473,10 @@ class MoeLayer:
             logits = torch.empty((n, self.n_expert + 1), dtype=torch.float32, device=x.device)
         d = self.desc()
         err = _err()
-        _check(lib().tqmoe_layer_forward(C.byref(d), _ptr(x), _ttype(x), n, _ptr(out), out_type, _ptr(ids), _ptr(weights), _ptr(logits),
-                                         _ptr(ws), ws.numel(), _stream(x), C.byref(err)), err)
+        if residual is not None:
+            _check(lib().tqmoe_layer_forward_residual(C.byref(d), _ptr(x), _ttype(x), _ptr(residual), n, _ptr(out), _ptr(ids), _ptr(weights), _ptr(logits),
+                                                      _ptr(ws), ws.numel(), _stream(x), C.byref(err)), err)
+        else:
+            _check(lib().tqmoe_layer_forward(C.byref(d), _ptr(x), _ttype(x), n, _ptr(out), out_type, _ptr(ids), _ptr(weights), _ptr(logits),
+                                             _ptr(ws), ws.numel(), _stream(x), C.byref(err)), err)
         return (out, ids, weights, logits) if return_routing else out

@@ -31,10 +31,12 @@ __device__ __forceinline__ float4 load4(const uint16_t * p) {   // four fp16 val
     return make_float4(half_bits_to_float(uint16_t(v.x & 0xFFFFu)), half_bits_to_float(uint16_t(v.x >> 16)), half_bits_to_float(uint16_t(v.y & 0xFFFFu)),
                        half_bits_to_float(uint16_t(v.y >> 16)));
 }
+// With a residual (bf16 rows, bf16 out) the result is bf16(bf16(sum) + residual): the reference stores the sum as bf16
+// (moe_sum) and adds the residual stream to it afterwards (add_sumsq, qwen35_forward.cpp:1248-1250), two roundings.
 template <int OT, class RT>
 __global__ __launch_bounds__(256) void combine_k(const RT * __restrict__ routed, int slots, const RT * __restrict__ shared, int64_t shared_ld,
                                                  const float * __restrict__ weights, const float * __restrict__ shared_w, void * __restrict__ out, int h, int k,
-                                                 int64_t count) {
+                                                 int64_t count, const uint16_t * __restrict__ residual) {
     const int64_t i = (int64_t(blockIdx.x) * 256 + threadIdx.x) * 4;   // h is a multiple of 4
     if (i >= count) return;
     const int64_t t = i / h;
@@ -49,6 +51,15 @@ __global__ __launch_bounds__(256) void combine_k(const RT * __restrict__ routed,
         const float w = shared_w[t];
         const float4 v = load4(shared + t * shared_ld + j);
         sum.x += w * v.x; sum.y += w * v.y; sum.z += w * v.z; sum.w += w * v.w;
+    }
+    if constexpr (OT == TQMOE_BF16) {
+        if (residual) {
+            const uint2 r = *reinterpret_cast<const uint2 *>(residual + i);
+            sum.x = bf16_bits_to_float(float_to_bf16_bits(sum.x)) + __uint_as_float(r.x << 16);
+            sum.y = bf16_bits_to_float(float_to_bf16_bits(sum.y)) + __uint_as_float(r.x & 0xFFFF0000u);
+            sum.z = bf16_bits_to_float(float_to_bf16_bits(sum.z)) + __uint_as_float(r.y << 16);
+            sum.w = bf16_bits_to_float(float_to_bf16_bits(sum.w)) + __uint_as_float(r.y & 0xFFFF0000u);
+        }
     }
     store_out<OT>(out, i, sum.x); store_out<OT>(out, i + 1, sum.y); store_out<OT>(out, i + 2, sum.z); store_out<OT>(out, i + 3, sum.w);
 }
@@ -182,7 +193,8 @@ extern "C" int32_t tqmoe_swiglu(const float * gate, const float * up, float * ac
 
 template <class RT>
 static int32_t combine_common(const RT * routed, int32_t slots, const RT * shared, int64_t shared_ld, const float * weights, const float * shared_weights,
-                              void * out, uint32_t otype, int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err) {
+                              void * out, uint32_t otype, int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err,
+                              const uint16_t * residual = nullptr) {
     if (!routed || !weights || !out || hidden <= 0 || hidden % 4 || topk <= 0 || slots < topk || n <= 0 || (shared && (!shared_weights || shared_ld % 4)))
         return fail(err, TQMOE_E_ARG, "tqmoe_combine: invalid shape or pointer (hidden must be a multiple of 4)");
     if (otype != TQMOE_F32 && otype != TQMOE_BF16) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_combine: output type must be F32 or BF16");
@@ -190,9 +202,23 @@ static int32_t combine_common(const RT * routed, int32_t slots, const RT * share
     const int64_t count = int64_t(n) * hidden;
     const unsigned blocks = unsigned((count / 4 + 255) / 256);
     const hipStream_t s = static_cast<hipStream_t>(stream);
-    if (otype == TQMOE_F32) combine_k<TQMOE_F32, RT><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count);
-    else combine_k<TQMOE_BF16, RT><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count);
+    if (residual && otype != TQMOE_BF16) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_combine: a residual is added to BF16 output only");
+    if (otype == TQMOE_F32) combine_k<TQMOE_F32, RT><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count, nullptr);
+    else combine_k<TQMOE_BF16, RT><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count, residual);
     return launched(err, "tqmoe_combine");
+}
+
+extern "C" int32_t tqmoe_combine_residual(const void * routed, uint32_t rtype, int32_t slots, const void * shared, int64_t shared_ld, const float * weights,
+                                          const float * shared_weights, const void * residual, void * out, int32_t hidden, int32_t topk, int32_t n,
+                                          void * stream, tqmoe_error * err) {
+    if (!residual) return fail(err, TQMOE_E_ARG, "tqmoe_combine_residual: residual rows missing");
+    if (rtype == TQMOE_F32)
+        return combine_common<float>(static_cast<const float *>(routed), slots, static_cast<const float *>(shared), shared_ld, weights, shared_weights, out,
+                                     TQMOE_BF16, hidden, topk, n, stream, err, static_cast<const uint16_t *>(residual));
+    if (rtype == TQMOE_F16)
+        return combine_common<uint16_t>(static_cast<const uint16_t *>(routed), slots, static_cast<const uint16_t *>(shared), shared_ld, weights, shared_weights,
+                                        out, TQMOE_BF16, hidden, topk, n, stream, err, static_cast<const uint16_t *>(residual));
+    return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_combine_residual: routed rows are F32 or F16");
 }
 
 extern "C" int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float * shared, int64_t shared_ld, const float * weights,

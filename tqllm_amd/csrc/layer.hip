@@ -110,9 +110,9 @@ extern "C" size_t tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t
     return plan_for(*layer, n).total;
 }
 
-extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x, uint32_t xtype, int32_t n, void * out, uint32_t otype,
-                                       int32_t * ids_out, float * weights_out, float * logits_out, void * workspace, size_t workspace_bytes,
-                                       void * stream, tqmoe_error * err) {
+static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t xtype, const void * residual, int32_t n, void * out, uint32_t otype,
+                             int32_t * ids_out, float * weights_out, float * logits_out, void * workspace, size_t workspace_bytes, void * stream,
+                             tqmoe_error * err) {
     if (int32_t rc = check_layer(layer, err)) return rc;
     const tqmoe_layer & L = *layer;
     if (!x || !out || n <= 0) return fail(err, TQMOE_E_ARG, "tqmoe_layer_forward: invalid shape or pointer");
@@ -144,6 +144,16 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
         const int32_t * cid = ids_ext + size_t(t0) * slots;
         const float * cw = weights + size_t(t0) * L.topk, * csw = shared_w + t0;
         void * cout = ob + size_t(t0) * L.hidden * obytes;
+        // the weighted sum of the chunk's rows, with the residual rows added when the caller gave them
+        auto combine = [&](const void * routed, uint32_t rtype, const void * shared) -> int32_t {
+            if (residual)
+                return tqmoe_combine_residual(routed, rtype, slots, shared, int64_t(slots) * L.hidden, cw, csw,
+                                              static_cast<const uint8_t *>(residual) + size_t(t0) * L.hidden * 2, cout, L.hidden, L.topk, c, stream, err);
+            if (rtype == TQMOE_F16)
+                return tqmoe_combine_strided_f16(routed, slots, shared, int64_t(slots) * L.hidden, cw, csw, cout, otype, L.hidden, L.topk, c, stream, err);
+            return tqmoe_combine_strided(static_cast<const float *>(routed), slots, static_cast<const float *>(shared), int64_t(slots) * L.hidden, cw, csw, cout, otype,
+                                         L.hidden, L.topk, c, stream, err);
+        };
         if (p.grouped) {
             int8_t * xq = reinterpret_cast<int8_t *>(ws + p.xq), * aq = reinterpret_cast<int8_t *>(ws + p.aq);
             float * xs = reinterpret_cast<float *>(ws + p.xs), * as = reinterpret_cast<float *>(ws + p.as);
@@ -157,8 +167,7 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
                                                           act16, stream, err)) return rc;
                 float * y32 = reinterpret_cast<float *>(y16);
                 if (int32_t rc = tqmoe_expert_gemm(&L.down, act16, TQMOE_F16, counts, offsets, perm, c, slots, L.topk, L.shared_ff, 1, y32, TQMOE_F32, stream, err)) return rc;
-                if (int32_t rc = tqmoe_combine_strided(y32, slots, L.has_shared ? y32 + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, cw, csw, cout, otype,
-                                                       L.hidden, L.topk, c, stream, err)) return rc;
+                if (int32_t rc = combine(y32, TQMOE_F32, L.has_shared ? y32 + size_t(L.topk) * L.hidden : nullptr)) return rc;
                 continue;
             } else {
             int8_t * rq = reinterpret_cast<int8_t *>(ws + p.rq);
@@ -169,16 +178,27 @@ extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x
             if (int32_t rc = tqmoe_group_rows_i8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_i8(&L.down, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
             }
-            if (int32_t rc = tqmoe_combine_strided_f16(y16, slots, L.has_shared ? y16 + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, cw, csw,
-                                                       cout, otype, L.hidden, L.topk, c, stream, err)) return rc;
+            if (int32_t rc = combine(y16, TQMOE_F16, L.has_shared ? y16 + size_t(L.topk) * L.hidden : nullptr)) return rc;
         } else {
             const uint8_t * ximage = ws + p.ximage + tqmoe_act_image_bytes(1, L.hidden) * size_t(t0);
             float * y = reinterpret_cast<float *>(ws + p.y);
             if (int32_t rc = tqmoe_expert_gateup(&L.gate, &L.up, ximage, ws + p.aimage, cid, c, slots, L.topk, L.shared_ff, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_down(&L.down, ws + p.aimage, y, cid, c, slots, L.topk, L.shared_ff, stream, err)) return rc;
-            if (int32_t rc = tqmoe_combine_strided(y, slots, L.has_shared ? y + size_t(L.topk) * L.hidden : nullptr, int64_t(slots) * L.hidden, cw, csw, cout,
-                                                   otype, L.hidden, L.topk, c, stream, err)) return rc;
+            if (int32_t rc = combine(y, TQMOE_F32, L.has_shared ? y + size_t(L.topk) * L.hidden : nullptr)) return rc;
         }
     }
     return ok(err);
+}
+
+extern "C" int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x, uint32_t xtype, int32_t n, void * out, uint32_t otype,
+                                       int32_t * ids_out, float * weights_out, float * logits_out, void * workspace, size_t workspace_bytes,
+                                       void * stream, tqmoe_error * err) {
+    return layer_forward(layer, x, xtype, nullptr, n, out, otype, ids_out, weights_out, logits_out, workspace, workspace_bytes, stream, err);
+}
+
+extern "C" int32_t tqmoe_layer_forward_residual(const tqmoe_layer * layer, const void * x, uint32_t xtype, const void * residual, int32_t n, void * out,
+                                                int32_t * ids_out, float * weights_out, float * logits_out, void * workspace, size_t workspace_bytes,
+                                                void * stream, tqmoe_error * err) {
+    if (!residual) return fail(err, TQMOE_E_ARG, "tqmoe_layer_forward_residual: residual rows missing");
+    return layer_forward(layer, x, xtype, residual, n, out, TQMOE_BF16, ids_out, weights_out, logits_out, workspace, workspace_bytes, stream, err);
 }

@@ -30,7 +30,7 @@ enum { TQMOE_OK = 0, TQMOE_E_ARG = -1, TQMOE_E_UNSUPPORTED = -2, TQMOE_E_DEVICE 
 /* element types (GGUF type ids, src/core/gguf.hpp) */
 enum { TQMOE_F32 = 0, TQMOE_F16 = 1, TQMOE_BF16 = 30 };
 /* bank formats (GGUF type ids) */
-enum { TQMOE_Q4_K = 12, TQMOE_IQ3_S = 21, TQMOE_IQ4_XS = 23, TQMOE_NVFP4G = 323 };
+enum { TQMOE_Q8_0 = 8, TQMOE_Q4_K = 12, TQMOE_Q5_K = 13, TQMOE_Q6_K = 14, TQMOE_IQ4_NL = 20, TQMOE_IQ3_S = 21, TQMOE_IQ4_XS = 23, TQMOE_NVFP4G = 323 };
 
 uint32_t tqmoe_abi_version(void);
 
@@ -100,10 +100,18 @@ int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets,
  *           16 weights, [rows_total][cols / 16] bytes, then at the next multiple of 16 bytes rows_total fp32 globals
  *           (one per row; rows whose blocks disagree are rejected by the reference loader, q4.cpp:519-521, and by
  *           tqmoe_bank_load through *status).
- * cols must be a multiple of 256 (128 for NVFP4G). */
+ *   Q5_K    codes 16 B: the low four bits in the same nibble order; aux 48 B per 256 weights: d, dmin, scales[12] as in
+ *           GGUF, then one 32-bit word per sub-block with the fifth bit of its weights (bit j = weight j).
+ *   Q6_K    codes 24 B: 16 B of low nibbles in the same order, then 8 B with the upper two bits (byte k = weights
+ *           4 k .. 4 k + 3); aux 32 B per 256 weights: the sixteen int8 scales in GGUF order (two per sub-block), d (f16),
+ *           padding.
+ *   IQ4_NL  codes 16 B, GGUF's own nibble order; aux 2 B per sub-block: its d (f16).
+ *   Q8_0    codes 32 B: the int8 values; aux 2 B per sub-block: its d (f16).
+ * cols must be a multiple of 256 (128 for NVFP4G). The grouped int8 products take IQ4_XS only; every format has the
+ * decode products and the fp16 grouped products (tqmoe_expert_gemm, tqmoe_expert_gemm_gateup). */
 typedef struct tqmoe_bank {
     uint32_t struct_size;
-    uint32_t type;            /* TQMOE_Q4_K, TQMOE_IQ3_S, TQMOE_IQ4_XS or TQMOE_NVFP4G */
+    uint32_t type;            /* one of the bank formats of the enum above */
     int32_t experts;          /* matrices in the bank */
     int32_t rows, cols;       /* of one expert */
     const void * codes;       /* device, tqmoe_bank_layout's code_bytes */

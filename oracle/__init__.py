@@ -13,8 +13,9 @@ LIB_PATH = os.path.join(HERE, "libtqmoe_oracle.so")
 REF_PATH = os.path.join(HERE, "_ref", "libtqref.so")
 
 F32, F16, Q4_K, IQ4_NL, IQ3_S, IQ4_XS, BF16, NVFP4G = 0, 1, 12, 20, 21, 23, 30, 323
+Q8_0, Q5_K, Q6_K = 8, 13, 14
 GATE_SOFTMAX, GATE_SIGMOID, GATE_SOFTMAX_WEIGHT, GATE_SQRT_SOFTPLUS = 1, 2, 3, 4
-BLOCK = {Q4_K: (256, 144), IQ4_NL: (32, 18), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76)}
+BLOCK = {Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), Q8_0: (32, 34), IQ4_NL: (32, 18), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76)}
 
 
 def build(ref=True):
@@ -72,7 +73,7 @@ class _Layer(C.Structure):
     _fields_ = [("hidden", C.c_int), ("ff", C.c_int), ("n_expert", C.c_int), ("k", C.c_int), ("has_shared", C.c_int),
                 ("shared_ff", C.c_int), ("wtype", C.c_uint32), ("gate", _p), ("up", _p), ("down", _p),
                 ("act_mode", C.c_int), ("threads", C.c_int), ("gating", C.c_int), ("raw_weights", C.c_int),
-                ("weight_scale", C.c_float), ("bias", _p)]
+                ("weight_scale", C.c_float), ("bias", _p), ("wtype_down", C.c_uint32)]
 
 
 _lib.tqo_layer_forward.argtypes = [C.POINTER(_Layer), _p, _p, C.c_int, _p, _p, _p]
@@ -216,14 +217,14 @@ def add_rmsnorm(rows_bits, residual_bits, weight, eps):
 
 
 def layer_forward(x, logits, gate, up, down, wtype, hidden, ff, n_expert, k, shared_ff=0, act_mode=0, threads=8, gating=GATE_SOFTMAX,
-                  norm=True, scale=1.0, bias=None):
+                  norm=True, scale=1.0, bias=None, wtype_down=0):
     """Whole layer on the host; returns (out [n][H] fp32, ids [n][k], weights [n][k])."""
     bias = _c(bias, np.float32) if bias is not None else None
     x, logits = _c(x, np.float32), _c(logits, np.float32)
     gate, up, down = (_c(a, np.uint8) for a in (gate, up, down))
     n = x.shape[0]
     L = _Layer(hidden, ff, n_expert, k, int(shared_ff > 0), shared_ff, wtype, _ptr(gate), _ptr(up), _ptr(down), act_mode, threads,
-               int(gating), int(not norm), float(scale), _ptr(bias))
+               int(gating), int(not norm), float(scale), _ptr(bias), int(wtype_down))
     out = np.empty((n, hidden), np.float32)
     ids = np.empty((n, k), np.int32)
     w = np.empty((n, k), np.float32)

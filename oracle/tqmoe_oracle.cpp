@@ -102,7 +102,10 @@ int tqo_block_layout(uint32_t type, int * elems, int * bytes) {
     int e = 0, b = 0;
     switch (type) {  // src/core/gguf.cpp:136-152
         case TQO_Q4_K: e = 256; b = 144; break;
+        case TQO_Q5_K: e = 256; b = 176; break;
+        case TQO_Q6_K: e = 256; b = 210; break;
         case TQO_IQ4_NL: e = 32; b = 18; break;
+        case TQO_Q8_0: e = 32; b = 34; break;
         case TQO_IQ3_S: e = 256; b = 110; break;
         case TQO_IQ4_XS: e = 256; b = 136; break;
         case TQO_NVFP4G: e = 128; b = 76; break;
@@ -137,6 +140,33 @@ void decode_q4k(const uint8_t * b, float * y) {
     }
 }
 
+void decode_q5k(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:102-116: (d * sc) * v - dmin * m
+    const float d = tqo_half_to_float(rd16(b)), dmin = tqo_half_to_float(rd16(b + 2));
+    const uint8_t * qh = b + 16, * q = b + 48;
+    for (int j = 0; j < 8; ++j) {
+        int sc, mn;
+        q4k_scale_min(b + 4, j, sc, mn);
+        for (int l = 0; l < 32; ++l) {
+            const int v = ((j & 1) ? q[32 * (j / 2) + l] >> 4 : q[32 * (j / 2) + l] & 15) + ((qh[l] >> j) & 1) * 16;
+            y[32 * j + l] = d * float(sc) * float(v) - dmin * float(mn);
+        }
+    }
+}
+
+void decode_q6k(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:194-208: (d * sc) * (q - 32)
+    const uint8_t * ql = b, * qh = b + 128;
+    const int8_t * sc = reinterpret_cast<const int8_t *>(b + 192);
+    const float d = tqo_half_to_float(rd16(b + 208));
+    for (int n = 0; n < 2; ++n, y += 128, ql += 64, qh += 32, sc += 8)
+        for (int l = 0; l < 32; ++l) {
+            const int is = l / 16;
+            y[l] = d * float(sc[is]) * float(((ql[l] & 15) | (((qh[l] >> 0) & 3) << 4)) - 32);
+            y[l + 32] = d * float(sc[is + 2]) * float(((ql[l + 32] & 15) | (((qh[l] >> 2) & 3) << 4)) - 32);
+            y[l + 64] = d * float(sc[is + 4]) * float(((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32);
+            y[l + 96] = d * float(sc[is + 6]) * float(((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32);
+        }
+}
+
 inline int iq4xs_subscale(const uint8_t * b, int ib) {  // 6-bit scale of sub-block ib, before the -32 offset
     const uint16_t sh = rd16(b + 2);
     return ((b[4 + ib / 2] >> (4 * (ib & 1))) & 15) | (((sh >> (2 * ib)) & 3) << 4);
@@ -160,6 +190,11 @@ void decode_iq4nl(const uint8_t * b, float * y) {
         y[j] = d * float(kIq4Values[b[2 + j] & 15]);
         y[16 + j] = d * float(kIq4Values[b[2 + j] >> 4]);
     }
+}
+
+void decode_q8_0(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:555-562
+    const float d = tqo_half_to_float(rd16(b));
+    for (int j = 0; j < 32; ++j) y[j] = d * float(int8_t(b[2 + j]));
 }
 
 void decode_iq3s(const uint8_t * b, float * y) {
@@ -199,8 +234,11 @@ int tqo_dequantize(uint32_t type, const void * src, float * dst, int64_t n) {
     const uint8_t * s = static_cast<const uint8_t *>(src);
     for (int64_t b = 0; b < n / elems; ++b, s += bytes, dst += elems) switch (type) {
         case TQO_Q4_K: decode_q4k(s, dst); break;
+        case TQO_Q5_K: decode_q5k(s, dst); break;
+        case TQO_Q6_K: decode_q6k(s, dst); break;
         case TQO_IQ4_XS: decode_iq4xs(s, dst); break;
         case TQO_IQ4_NL: decode_iq4nl(s, dst); break;
+        case TQO_Q8_0: decode_q8_0(s, dst); break;
         case TQO_IQ3_S: decode_iq3s(s, dst); break;
         case TQO_NVFP4G: decode_nvfp4g(s, dst); break;
     }
@@ -225,6 +263,15 @@ inline float iq4_block_scale(const float * x) {
     float amax = 0.f, vmax = 0.f;
     for (int i = 0; i < 32; ++i) if (std::fabs(x[i]) > amax) { amax = std::fabs(x[i]); vmax = x[i]; }
     return vmax / -127.f;
+}
+
+void encode_q8_0(const float * x, uint8_t * b) {  // d = amax / 127, q = rint(x / d)
+    float amax = 0.f;
+    for (int j = 0; j < 32; ++j) amax = std::max(amax, std::fabs(x[j]));
+    const uint16_t hd = tqo_float_to_half(amax / 127.f);
+    const float d = tqo_half_to_float(hd), inv = d != 0.f ? 1.f / d : 0.f;
+    std::memcpy(b, &hd, 2);
+    for (int j = 0; j < 32; ++j) b[2 + j] = uint8_t(int8_t(std::max(-127.f, std::min(127.f, std::nearbyint(x[j] * inv)))));
 }
 
 void encode_iq4nl(const float * x, uint8_t * b) {
@@ -293,6 +340,71 @@ void encode_q4k(const float * x, uint8_t * b) {
                 code[h] = step > 0.f ? std::min(15, std::max(0, int(std::nearbyint((v + off) / step)))) : 0;
             }
             b[16 + 32 * c + l] = uint8_t(code[0] | (code[1] << 4));
+        }
+}
+
+void encode_q5k(const float * x, uint8_t * b) {  // encode_q4k with 32 levels and the high-bit plane
+    float sc[8], mn[8], smax = 0.f, mmax = 0.f;
+    for (int i = 0; i < 8; ++i) {
+        float lo = 0.f, hi = 0.f;
+        for (int l = 0; l < 32; ++l) { lo = std::min(lo, x[32 * i + l]); hi = std::max(hi, x[32 * i + l]); }
+        sc[i] = (hi - lo) / 31.f;
+        mn[i] = -lo;
+        smax = std::max(smax, sc[i]);
+        mmax = std::max(mmax, mn[i]);
+    }
+    const uint16_t hd = tqo_float_to_half(smax / 63.f), hm = tqo_float_to_half(mmax / 63.f);
+    const float d = tqo_half_to_float(hd), dm = tqo_half_to_float(hm);
+    std::memset(b, 0, 176);
+    std::memcpy(b, &hd, 2);
+    std::memcpy(b + 2, &hm, 2);
+    int s6[8], m6[8];
+    for (int i = 0; i < 8; ++i) {
+        s6[i] = d > 0.f ? std::min(63, std::max(0, int(std::nearbyint(sc[i] / d)))) : 0;
+        m6[i] = dm > 0.f ? std::min(63, std::max(0, int(std::nearbyint(mn[i] / dm)))) : 0;
+    }
+    uint8_t * q = b + 4;
+    for (int j = 0; j < 4; ++j) {
+        q[j] = uint8_t(s6[j] | ((s6[j + 4] >> 4) << 6));
+        q[j + 4] = uint8_t(m6[j] | ((m6[j + 4] >> 4) << 6));
+        q[j + 8] = uint8_t((s6[j + 4] & 15) | ((m6[j + 4] & 15) << 4));
+    }
+    for (int i = 0; i < 8; ++i)
+        for (int l = 0; l < 32; ++l) {
+            const float step = d * float(s6[i]), off = dm * float(m6[i]);
+            const int code = step > 0.f ? std::min(31, std::max(0, int(std::nearbyint((x[32 * i + l] + off) / step)))) : 0;
+            b[48 + 32 * (i / 2) + l] |= uint8_t((code & 15) << (4 * (i & 1)));
+            b[16 + l] |= uint8_t((code >> 4) << i);
+        }
+}
+
+void encode_q6k(const float * x, uint8_t * b) {  // 16 groups of 16: scale amax / 31, super scale max / 127
+    float gs[16], big = 0.f;
+    for (int g = 0; g < 16; ++g) {
+        float amax = 0.f;
+        for (int l = 0; l < 16; ++l) amax = std::max(amax, std::fabs(x[16 * g + l]));
+        gs[g] = amax / 31.f;
+        big = std::max(big, gs[g]);
+    }
+    const uint16_t hd = tqo_float_to_half(big / 127.f);
+    const float d = tqo_half_to_float(hd);
+    std::memset(b, 0, 210);
+    std::memcpy(b + 208, &hd, 2);
+    int code[256];
+    for (int g = 0; g < 16; ++g) {
+        const int sc = d > 0.f ? std::min(127, std::max(0, int(std::nearbyint(gs[g] / d)))) : 0;
+        // weights 16 g .. of the block: sub-block i = g / 2 = 4 n + j, half is = g % 2: scale index 8 n + 2 j + is = g
+        b[192 + g] = uint8_t(int8_t(sc));
+        const float step = d * float(sc);
+        for (int l = 0; l < 16; ++l)
+            code[16 * g + l] = step > 0.f ? std::min(63, std::max(0, int(std::nearbyint(x[16 * g + l] / step)) + 32)) : 32;
+    }
+    for (int n = 0; n < 2; ++n)
+        for (int l = 0; l < 32; ++l) {
+            const int c0 = code[128 * n + l], c1 = code[128 * n + 32 + l], c2 = code[128 * n + 64 + l], c3 = code[128 * n + 96 + l];
+            b[64 * n + l] = uint8_t((c0 & 15) | ((c2 & 15) << 4));
+            b[64 * n + 32 + l] = uint8_t((c1 & 15) | ((c3 & 15) << 4));
+            b[128 + 32 * n + l] = uint8_t((c0 >> 4) | ((c1 >> 4) << 2) | ((c2 >> 4) << 4) | ((c3 >> 4) << 6));
         }
 }
 
@@ -416,8 +528,11 @@ int tqo_quantize(uint32_t type, const float * src, void * dst, int64_t n, int64_
     }
     for (int64_t b = 0; b < n / elems; ++b, src += elems, o += bytes) switch (type) {
         case TQO_Q4_K: encode_q4k(src, o); break;
+        case TQO_Q5_K: encode_q5k(src, o); break;
+        case TQO_Q6_K: encode_q6k(src, o); break;
         case TQO_IQ4_XS: encode_iq4xs(src, o); break;
         case TQO_IQ4_NL: encode_iq4nl(src, o); break;
+        case TQO_Q8_0: encode_q8_0(src, o); break;
         case TQO_IQ3_S: encode_iq3s(src, o); break;
     }
     return 0;
@@ -675,11 +790,14 @@ int decode_expert(const tqo_layer & L, int e, int ff, Decoded & d) {
     // gate / up: the first ff rows of expert e
     if (tqo_dequantize(L.wtype, static_cast<const uint8_t *>(L.gate) + stride * e, d.gate.data(), int64_t(ff) * L.hidden)) return -1;
     if (tqo_dequantize(L.wtype, static_cast<const uint8_t *>(L.up) + stride * e, d.up.data(), int64_t(ff) * L.hidden)) return -1;
-    // down: rows of L.ff columns, the first ff columns kept
+    // down: rows of L.ff columns, the first ff columns kept; its bank may have a format of its own
+    const uint32_t dtype = L.wtype_down ? L.wtype_down : L.wtype;
+    int delems, dbytes;
+    if (!tqo_block_layout(dtype, &delems, &dbytes) || L.ff % delems) return -1;
     std::vector<float> row(static_cast<size_t>(L.ff));
-    const size_t row_bytes = size_t(L.ff / elems) * bytes;
+    const size_t row_bytes = size_t(L.ff / delems) * dbytes, dstride = size_t(gu / delems) * dbytes;
     for (int r = 0; r < L.hidden; ++r) {
-        if (tqo_dequantize(L.wtype, static_cast<const uint8_t *>(L.down) + stride * e + row_bytes * r, row.data(), L.ff)) return -1;
+        if (tqo_dequantize(dtype, static_cast<const uint8_t *>(L.down) + dstride * e + row_bytes * r, row.data(), L.ff)) return -1;
         std::copy(row.begin(), row.begin() + ff, d.down.begin() + size_t(r) * ff);
     }
     if (L.act_mode == 3) {

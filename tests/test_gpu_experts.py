@@ -19,7 +19,7 @@ def tq():
     return tqllm_amd
 
 
-@pytest.mark.parametrize("wtype", [12, 21, 23, 323])
+@pytest.mark.parametrize("wtype", [12, 21, 23, 323, 20, 8, 13, 14])
 def test_bank_decode_bit_exact(tq, oracle, wtype):
     rng = np.random.default_rng(wtype)
     experts, rows, cols = 3, (64 if wtype == 23 else 40), 1024      # IQ4_XS banks are tiled by 32 rows
@@ -27,7 +27,7 @@ def test_bank_decode_bit_exact(tq, oracle, wtype):
     nb = experts * rows * cols // el
     # random block bytes with sane scale fields, as the reference's device tests make them (tests/moe_device.cu:121-138)
     raw = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
-    for off in {12: [0, 2], 21: [0], 23: [0]}.get(wtype, []):
+    for off in {12: [0, 2], 21: [0], 23: [0], 20: [0], 8: [0], 13: [0, 2], 14: [208]}.get(wtype, []):
         raw[:, off:off + 2] = np.float16(rng.uniform(1e-3, 5e-2, nb) * rng.choice([-1, 1], nb)).view(np.uint8).reshape(nb, 2)
     if wtype == 323:
         g = rng.uniform(1e-3, 2e-2, experts * rows).astype(np.float32)
@@ -147,6 +147,34 @@ def test_layer_small_shapes(tq, oracle, name, n):
     base = synth.CONFIGS[name]
     cfg = synth.small(base, 768 if name != "c5" else 384, 512 if name != "c5" else 256, 10, 3)
     check_layer(*run_layer(tq, oracle, cfg, n, seed=50 + n))
+
+
+@pytest.mark.parametrize("wtype", [20, 8, 13, 14])
+@pytest.mark.parametrize("n", [1, 5, 300])
+def test_layer_iq4nl_q8_0_q5k_q6k_banks(tq, oracle, wtype, n):
+    """IQ4_NL (the CPU bench's format), Q8_0, Q5_K and Q6_K through the same decode kernels and grouped GEMM as the
+    others, with a shared expert."""
+    cfg = dict(hidden=768, ff=512, experts=10, topk=3, shared_ff=256, wtype=wtype, rtype="bf16", xtype="bf16")
+    check_layer(*run_layer(tq, oracle, cfg, n, seed=90 + n + wtype))
+
+
+@pytest.mark.parametrize("gu_type,down_type", [(12, 14), (23, 14), (13, 8)])
+@pytest.mark.parametrize("n", [4, 300])
+def test_layer_down_bank_of_another_format(tq, oracle, gu_type, down_type, n):
+    """Mixed checkpoints (the K-quant mixes keep ffn_down_exps in a wider format than gate / up): the down bank may have a
+    format of its own, on the decode kernels and on the grouped GEMM."""
+    cfg = dict(hidden=768, ff=512, experts=10, topk=3, shared_ff=256, wtype=gu_type, rtype="bf16", xtype="bf16")
+    raws = synth.make_banks(cfg, seed=120 + n)
+    raws[2] = synth.make_banks(dict(cfg, wtype=down_type), seed=121 + n)[2]
+    e = cfg["experts"] + 1
+    gate, up = (tq.ExpertBank(gu_type, r, e, cfg["ff"], cfg["hidden"]) for r in raws[:2])
+    down = tq.ExpertBank(down_type, raws[2], e, cfg["hidden"], cfg["ff"])
+    inp = synth.make_inputs(cfg, n, seed=122 + n)
+    layer = tq.MoeLayer(dev(inp["router"]), dev(inp["shared_gate"]), gate, up, down, cfg["topk"], shared_ff=cfg["shared_ff"])
+    out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
+    want, want_ids, want_w = oracle.layer_forward(inp["x"][1], logits, *raws, gu_type, cfg["hidden"], cfg["ff"], cfg["experts"], cfg["topk"],
+                                                  shared_ff=cfg["shared_ff"], act_mode=0, threads=16, wtype_down=down_type)
+    check_layer(out, ids, w, want, want_ids, want_w, oracle.route_min_gap_ulps(logits[:, :cfg["experts"]], cfg["topk"]))
 
 
 @pytest.mark.parametrize("n", [1, 4, 16])

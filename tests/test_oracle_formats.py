@@ -139,13 +139,73 @@ def test_iq4xs_independent_decode(oracle):
     assert np.array_equal(got, want.astype(np.float32))
 
 
-@pytest.mark.parametrize("wtype", [12, 20, 21, 23, 323])
+def test_q8_0_closed_form(oracle):
+    """Q8_0 (dequant.cpp:555-562): 34 bytes = fp16 d, 32 int8; value d * q, every code from -128 to 127."""
+    rng = np.random.default_rng(5)
+    nb = 16
+    raw = np.empty((nb, 34), np.uint8)
+    d = np.float16(rng.uniform(1e-3, 5e-2, nb) * rng.choice([-1, 1], nb))
+    raw[:, 0:2] = d.view(np.uint8).reshape(nb, 2)
+    q = rng.integers(-128, 128, (nb, 32)).astype(np.int8)
+    q[0] = np.arange(-128, -96)
+    q[1] = np.arange(96, 128)
+    raw[:, 2:] = q.view(np.uint8)
+    got = oracle.dequantize(oracle.Q8_0, raw, nb * 32).reshape(nb, 32)
+    assert np.array_equal(got, d.astype(np.float32)[:, None] * q.astype(np.float32))
+    # the encoder's round trip: within half a step of d = amax / 127
+    x = rng.standard_normal((8, 32)).astype(np.float32)
+    back = oracle.dequantize(oracle.Q8_0, oracle.quantize(oracle.Q8_0, x), x.size).reshape(8, 32)
+    assert (np.abs(back - x) <= np.abs(x).max(axis=1, keepdims=True) / 127 * 0.51 + 1e-6).all()
+
+
+@pytest.mark.parametrize("wtype,bits", [(13, 5), (14, 6)])
+def test_q5k_q6k_independent_decode_and_round_trip(oracle, wtype, bits):
+    """Q5_K / Q6_K: the codes are plain integers, so a block built from known codes and scales must decode to the closed
+    form (scale * code - min, scale * (code - 32)); the encoders' round trip stays within a step."""
+    rng = np.random.default_rng(wtype)
+    if wtype == 13:
+        b = np.zeros(176, np.uint8)
+        b[0:2] = np.array([np.float16(0.5)]).view(np.uint8)
+        b[2:4] = np.array([np.float16(0.25)]).view(np.uint8)
+        b[4:8] = [3, 5, 7, 9]            # scales of sub-blocks 0..3 (6-bit), mins follow
+        b[8:12] = [1, 2, 3, 4]
+        code = rng.integers(0, 32, 256)
+        for i in range(4):               # the first four sub-blocks: scale b[4 + i], min b[8 + i]
+            for l in range(32):
+                c = int(code[32 * i + l])
+                b[48 + 32 * (i // 2) + l] |= (c & 15) << (4 * (i & 1))
+                b[16 + l] |= (c >> 4) << i
+        got = oracle.dequantize(13, b, 256)
+        for i in range(4):
+            want = np.float32(0.5) * np.float32(b[4 + i]) * code[32 * i:32 * i + 32].astype(np.float32) - np.float32(0.25) * np.float32(b[8 + i])
+            assert np.array_equal(got[32 * i:32 * i + 32], want.astype(np.float32))
+    else:
+        b = np.zeros(210, np.uint8)
+        b[208:210] = np.array([np.float16(0.125)]).view(np.uint8)
+        sc = rng.integers(-20, 21, 16).astype(np.int8)
+        b[192:208] = sc.view(np.uint8)
+        code = rng.integers(0, 64, 256)
+        for n in range(2):
+            for l in range(32):
+                c = [int(code[128 * n + 32 * j + l]) for j in range(4)]
+                b[64 * n + l] = (c[0] & 15) | ((c[2] & 15) << 4)
+                b[64 * n + 32 + l] = (c[1] & 15) | ((c[3] & 15) << 4)
+                b[128 + 32 * n + l] = (c[0] >> 4) | ((c[1] >> 4) << 2) | ((c[2] >> 4) << 4) | ((c[3] >> 4) << 6)
+        got = oracle.dequantize(14, b, 256)
+        want = np.float32(0.125) * np.repeat(sc, 16).astype(np.float32) * (code - 32).astype(np.float32)
+        assert np.array_equal(got, want.astype(np.float32))
+    x = (rng.standard_normal((4, 256)) * 0.05).astype(np.float32)
+    back = oracle.dequantize(wtype, oracle.quantize(wtype, x), x.size).reshape(4, 256)
+    assert np.abs(back - x).max() < np.abs(x).max() / (2 ** bits - 1) * 1.6
+
+
+@pytest.mark.parametrize("wtype", [8, 12, 13, 14, 20, 21, 23, 323])
 def test_decoders_match_reference_objects(oracle, ref, wtype):
     rng = np.random.default_rng(wtype)
     el, bb = oracle.BLOCK[wtype]
     nb = 64
     raw = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
-    halves = {12: [0, 2], 20: [0], 21: [0], 23: [0]}.get(wtype, [])
+    halves = {8: [0], 12: [0, 2], 13: [0, 2], 14: [208], 20: [0], 21: [0], 23: [0]}.get(wtype, [])
     for off in halves:
         raw[:, off:off + 2] = np.float16(rng.uniform(1e-3, 5e-2, nb) * rng.choice([-1, 1], nb)).view(np.uint8).reshape(nb, 2)
     if wtype == 323:

@@ -65,6 +65,52 @@ __global__ __launch_bounds__(256) void load_k(uint32_t type, const uint8_t * __r
             }
             break;
         }
+        case TQMOE_Q5_K: {  // 176 B per 256: d, dmin, scales[12], qh[32] (bit j of byte l: weight l of sub-block j), qs[128] as Q4_K
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 176;
+            const int ib = s & 7;
+            const uint8_t * q = blk + 48 + 32 * (ib >> 1);
+            pack_sub(cd, [&](int j) { return (ib & 1) ? q[j] >> 4 : q[j] & 15; });
+            uint8_t * a = aux + (row * (S / 8) + s / 8) * 48;
+            uint32_t hb = 0;
+#pragma unroll
+            for (int l = 0; l < 32; ++l) hb |= uint32_t((blk[16 + l] >> ib) & 1) << l;
+            *reinterpret_cast<uint32_t *>(a + 16 + 4 * ib) = hb;
+            if (ib == 0) *reinterpret_cast<uint4 *>(a) = make_uint4(rd_u32(blk), rd_u32(blk + 4), rd_u32(blk + 8), rd_u32(blk + 12));
+            break;
+        }
+        case TQMOE_Q6_K: {  // 210 B per 256: ql[128], qh[64], scales[16], d; sub-block i = 4 n + j holds weights 128 n + 32 j ..
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 210;
+            const int ib = s & 7, n = ib >> 2, j = ib & 3;
+            const uint8_t * ql = blk + 64 * n + 32 * (j & 1), * qh = blk + 128 + 32 * n;
+            __attribute__((aligned(16))) uint8_t low[16];   // 24-byte code records are 8-byte aligned: stored as three 8-byte pieces
+            pack_sub(low, [&](int l) { return (j & 2) ? ql[l] >> 4 : ql[l] & 15; });
+            reinterpret_cast<uint2 *>(cd)[0] = reinterpret_cast<const uint2 *>(low)[0];
+            reinterpret_cast<uint2 *>(cd)[1] = reinterpret_cast<const uint2 *>(low)[1];
+            uint32_t hi[2] = {0, 0};   // two bits per weight, byte k = weights 4 k .. 4 k + 3
+#pragma unroll
+            for (int l = 0; l < 32; ++l) hi[l >> 4] |= uint32_t((qh[l] >> (2 * j)) & 3) << (2 * (l & 15));
+            *reinterpret_cast<uint2 *>(cd + 16) = make_uint2(hi[0], hi[1]);
+            if (ib == 0) {
+                uint8_t * a = aux + (row * (S / 8) + s / 8) * 32;
+                *reinterpret_cast<uint4 *>(a) = make_uint4(rd_u32(blk + 192), rd_u32(blk + 196), rd_u32(blk + 200), rd_u32(blk + 204));
+                *reinterpret_cast<uint4 *>(a + 16) = make_uint4(rd_u16(blk + 208), 0, 0, 0);
+            }
+            break;
+        }
+        case TQMOE_IQ4_NL: {  // 18 B per 32: d, qs[16] (byte j = weight j | weight j + 16 << 4: the canonical order)
+            const uint8_t * blk = src + (row * S + s) * 18;
+            pack_sub(cd, [&](int j) { return j < 16 ? blk[2 + j] & 15 : blk[2 + j - 16] >> 4; });
+            *reinterpret_cast<uint16_t *>(aux + (row * S + s) * 2) = uint16_t(rd_u16(blk));
+            break;
+        }
+        case TQMOE_Q8_0: {  // 34 B per 32: d, 32 int8
+            const uint8_t * blk = src + (row * S + s) * 34;
+            uint32_t * o = reinterpret_cast<uint32_t *>(cd);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) o[q] = rd_u16(blk + 2 + 4 * q) | rd_u16(blk + 4 + 4 * q) << 16;
+            *reinterpret_cast<uint16_t *>(aux + (row * S + s) * 2) = uint16_t(rd_u16(blk));
+            break;
+        }
         case TQMOE_NVFP4G: {  // 76 B per 128: global f32, 8 E4M3 scales, 64 code bytes (byte i of a 16-group: weights 2i, 2i + 1)
             const uint8_t * blk = src + (row * (S / 4) + s / 4) * 76;
             const int q4 = s & 3;

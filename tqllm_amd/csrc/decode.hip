@@ -76,6 +76,10 @@ void dispatch_matvec(uint32_t type, Split sp, int nb, const MatvecArgs & k, hipS
         case TQMOE_IQ4_XS: DecodeLaunch<TQMOE_IQ4_XS>::matvec(sp, nb, k, s); break;
         case TQMOE_Q4_K: DecodeLaunch<TQMOE_Q4_K>::matvec(sp, nb, k, s); break;
         case TQMOE_IQ3_S: DecodeLaunch<TQMOE_IQ3_S>::matvec(sp, nb, k, s); break;
+        case TQMOE_IQ4_NL: DecodeLaunch<TQMOE_IQ4_NL>::matvec(sp, nb, k, s); break;
+        case TQMOE_Q8_0: DecodeLaunch<TQMOE_Q8_0>::matvec(sp, nb, k, s); break;
+        case TQMOE_Q5_K: DecodeLaunch<TQMOE_Q5_K>::matvec(sp, nb, k, s); break;
+        case TQMOE_Q6_K: DecodeLaunch<TQMOE_Q6_K>::matvec(sp, nb, k, s); break;
         default: DecodeLaunch<TQMOE_NVFP4G>::matvec(sp, nb, k, s); break;
     }
 }
@@ -84,6 +88,10 @@ void dispatch_gateup(uint32_t type, Split sp, const GateupArgs & k, hipStream_t 
         case TQMOE_IQ4_XS: DecodeLaunch<TQMOE_IQ4_XS>::gateup(sp, k, s); break;
         case TQMOE_Q4_K: DecodeLaunch<TQMOE_Q4_K>::gateup(sp, k, s); break;
         case TQMOE_IQ3_S: DecodeLaunch<TQMOE_IQ3_S>::gateup(sp, k, s); break;
+        case TQMOE_IQ4_NL: DecodeLaunch<TQMOE_IQ4_NL>::gateup(sp, k, s); break;
+        case TQMOE_Q8_0: DecodeLaunch<TQMOE_Q8_0>::gateup(sp, k, s); break;
+        case TQMOE_Q5_K: DecodeLaunch<TQMOE_Q5_K>::gateup(sp, k, s); break;
+        case TQMOE_Q6_K: DecodeLaunch<TQMOE_Q6_K>::gateup(sp, k, s); break;
         default: DecodeLaunch<TQMOE_NVFP4G>::gateup(sp, k, s); break;
     }
 }

@@ -44,5 +44,9 @@ template <> void DecodeLaunch<TQMOE_IQ4_XS>::gateup(Split sp, const GateupArgs &
 extern template struct DecodeLaunch<TQMOE_Q4_K>;
 extern template struct DecodeLaunch<TQMOE_IQ3_S>;
 extern template struct DecodeLaunch<TQMOE_NVFP4G>;
+extern template struct DecodeLaunch<TQMOE_IQ4_NL>;
+extern template struct DecodeLaunch<TQMOE_Q8_0>;
+extern template struct DecodeLaunch<TQMOE_Q5_K>;
+extern template struct DecodeLaunch<TQMOE_Q6_K>;
 
 }  // namespace tqmoe

@@ -87,6 +87,97 @@ template <> struct Sub<TQMOE_Q4_K> {
     }
 };
 
+template <> struct Sub<TQMOE_Q5_K> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint4 c; uint4 rec; uint32_t hb; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        v.c = *reinterpret_cast<const uint4 *>(t.codes + (r * S + s) * 16u);
+        const uint8_t * a = t.aux + (r * (S >> 3) + (s >> 3)) * 48u;
+        v.rec = *reinterpret_cast<const uint4 *>(a);
+        v.hb = *reinterpret_cast<const uint32_t *>(a + 16u + 4u * (s & 7u));
+        return v;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int s, const uint32_t *, Dec & d) {
+        const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            nibbles(w[q], d.w[q], d.w[4 + q]);
+            d.w[q] |= spread4(r.hb >> (4 * q)) << 4;            // the fifth bit of weights 4 q ..
+            d.w[4 + q] |= spread4(r.hb >> (16 + 4 * q)) << 4;   // and of weights 16 + 4 q ..
+        }
+        const uint32_t sc12[3] = {r.rec.y, r.rec.z, r.rec.w};
+        int sc, mn;
+        q4k_scale_min(sc12, s & 7, sc, mn);
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.rec.x & 0xFFFFu)) * float(sc);
+        d.mn = half_bits_to_float(uint16_t(r.rec.x >> 16)) * float(mn);
+    }
+};
+
+template <> struct Sub<TQMOE_Q6_K> {
+    static constexpr bool kSplit = true;   // one scale per 16 weights: the sub-block's halves
+    struct Raw { uint2 c[3]; uint32_t sc; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        const uint2 * cp = reinterpret_cast<const uint2 *>(t.codes + (r * S + s) * 24u);
+        v.c[0] = cp[0]; v.c[1] = cp[1]; v.c[2] = cp[2];
+        const uint8_t * a = t.aux + (r * (S >> 3) + (s >> 3)) * 32u;
+        v.sc = *reinterpret_cast<const uint16_t *>(a + 2u * (s & 7u));
+        v.d = *reinterpret_cast<const uint16_t *>(a + 16u);
+        return v;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t *, Dec & d) {
+        const uint32_t w[4] = {r.c[0].x, r.c[0].y, r.c[1].x, r.c[1].y};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t lo, hi;
+            nibbles(w[q], lo, hi);
+            d.w[q] = minus32(lo | spread2x4(r.c[2].x >> (8 * q)) << 4);
+            d.w[4 + q] = minus32(hi | spread2x4(r.c[2].y >> (8 * q)) << 4);
+        }
+        const float dd = half_bits_to_float(uint16_t(r.d));
+        d.s0 = dd * float(int8_t(r.sc & 0xFFu));
+        d.s1 = dd * float(int8_t(r.sc >> 8));
+        d.mn = 0.f;
+    }
+};
+
+template <> struct Sub<TQMOE_IQ4_NL> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint4 c; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        v.c = *reinterpret_cast<const uint4 *>(t.codes + (r * S + s) * 16u);
+        v.d = *reinterpret_cast<const uint16_t *>(t.aux + (r * S + s) * 2u);
+        return v;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t *, Dec & d) {
+        const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(w[q], d.w[q], d.w[4 + q]);
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.d));
+        d.mn = 0.f;
+    }
+};
+
+template <> struct Sub<TQMOE_Q8_0> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint4 c0, c1; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        const uint4 * cp = reinterpret_cast<const uint4 *>(t.codes + (r * S + s) * 32u);
+        v.c0 = cp[0]; v.c1 = cp[1];
+        v.d = *reinterpret_cast<const uint16_t *>(t.aux + (r * S + s) * 2u);
+        return v;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t *, Dec & d) {   // the codes are the values
+        d.w[0] = r.c0.x; d.w[1] = r.c0.y; d.w[2] = r.c0.z; d.w[3] = r.c0.w;
+        d.w[4] = r.c1.x; d.w[5] = r.c1.y; d.w[6] = r.c1.z; d.w[7] = r.c1.w;
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.d));
+        d.mn = 0.f;
+    }
+};
+
 template <> struct Sub<TQMOE_NVFP4G> {
     static constexpr bool kSplit = true;
     struct Raw { uint4 c; uint32_t sc; float g; };

@@ -67,6 +67,75 @@ __device__ __forceinline__ void decode_sub32(uint32_t type, const uint8_t * __re
             }
             break;
         }
+        case TQMOE_Q5_K: {  // dequant.cpp:102-116: (d * sc) * v - dmin * m, v = nibble + 16 * high bit
+            const uint8_t * a = aux + (row * (S / 8) + s / 8) * 48;
+            const uint4 rec = *reinterpret_cast<const uint4 *>(a);
+            const uint32_t hb = *reinterpret_cast<const uint32_t *>(a + 16 + 4 * ib);
+            const uint32_t sc12[3] = {rec.y, rec.z, rec.w};
+            int sc, mn;
+            q4k_scale_min(sc12, ib, sc, mn);
+            const float d1 = __fmul_rn(half_bits_to_float(uint16_t(rec.x & 0xFFFFu)), float(sc));
+            const float m1 = __fmul_rn(half_bits_to_float(uint16_t(rec.x >> 16)), float(mn));
+            const uint4 c = *reinterpret_cast<const uint4 *>(cd);
+            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const uint32_t byte = (w[q] >> (8 * b)) & 0xFFu;
+                    const int j = 4 * q + b;
+                    y[j] = __fsub_rn(__fmul_rn(d1, float((byte & 15u) + 16u * ((hb >> j) & 1u))), m1);
+                    y[16 + j] = __fsub_rn(__fmul_rn(d1, float((byte >> 4) + 16u * ((hb >> (16 + j)) & 1u))), m1);
+                }
+            break;
+        }
+        case TQMOE_Q6_K: {  // dequant.cpp:194-208: (d * sc) * (q - 32), one int8 scale per 16 weights
+            const uint8_t * a = aux + (row * (S / 8) + s / 8) * 32;
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(a + 16));
+            const float d0 = __fmul_rn(d, float(int8_t(a[2 * ib]))), d1 = __fmul_rn(d, float(int8_t(a[2 * ib + 1])));
+            const uint2 c0 = *reinterpret_cast<const uint2 *>(cd), c1 = *reinterpret_cast<const uint2 *>(cd + 8), hi = *reinterpret_cast<const uint2 *>(cd + 16);
+            const uint32_t w[4] = {c0.x, c0.y, c1.x, c1.y};
+            const uint32_t h2[2] = {hi.x, hi.y};
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const uint32_t byte = (w[q] >> (8 * b)) & 0xFFu;
+                    const int j = 4 * q + b;
+                    const int lo = int((byte & 15u) | (((h2[0] >> (2 * j)) & 3u) << 4)) - 32;
+                    const int up = int((byte >> 4) | (((h2[1] >> (2 * j)) & 3u) << 4)) - 32;
+                    y[j] = __fmul_rn(d0, float(lo));
+                    y[16 + j] = __fmul_rn(d1, float(up));
+                }
+            break;
+        }
+        case TQMOE_IQ4_NL: {  // dequant.cpp:351-360: d * kv[q]
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(aux + (row * S + s) * 2));
+            const uint4 c = *reinterpret_cast<const uint4 *>(cd);
+            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t lo, hi;
+                lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(w[q], lo, hi);
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    y[4 * q + b] = __fmul_rn(d, float(int8_t(lo >> (8 * b))));
+                    y[16 + 4 * q + b] = __fmul_rn(d, float(int8_t(hi >> (8 * b))));
+                }
+            }
+            break;
+        }
+        case TQMOE_Q8_0: {  // dequant.cpp:555-562: d * q
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(aux + (row * S + s) * 2));
+            const uint32_t * c = reinterpret_cast<const uint32_t *>(cd);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const uint32_t w = c[q];
+#pragma unroll
+                for (int b = 0; b < 4; ++b) y[4 * q + b] = __fmul_rn(d, float(int8_t(w >> (8 * b))));
+            }
+            break;
+        }
         case TQMOE_NVFP4G: {
             const float g = *reinterpret_cast<const float *>(aux + nvfp4_global_offset(rows_total, cols) + row * 4);
             const uint8_t * sc = aux + row * (cols / 16) + 2 * s;

@@ -7,9 +7,11 @@
 namespace tqmoe {
 
 // code bytes per sub-block
-__host__ __device__ constexpr int code_bytes_per_sub(uint32_t type) { return type == TQMOE_IQ3_S ? 12 : 16; }
-// aux record bytes per 256 weights (NVFP4G keeps bytes per 16 weights instead: see aux_row_bytes)
-__host__ __device__ constexpr int aux_record_bytes(uint32_t type) { return type == TQMOE_IQ4_XS ? 8 : 16; }
+__host__ __device__ constexpr int code_bytes_per_sub(uint32_t type) { return type == TQMOE_IQ3_S ? 12 : type == TQMOE_Q8_0 ? 32 : type == TQMOE_Q6_K ? 24 : 16; }
+// aux record bytes per 256 weights (NVFP4G keeps bytes per 16 weights instead: see aux_row_bytes; IQ4_NL and Q8_0 hold
+// the eight fp16 scales of their 32-weight blocks)
+// Q5_K: the Q4_K header and the eight sub-blocks' high-bit words; Q6_K: sixteen int8 scales, d, padding
+__host__ __device__ constexpr int aux_record_bytes(uint32_t type) { return type == TQMOE_IQ4_XS ? 8 : type == TQMOE_Q5_K ? 48 : type == TQMOE_Q6_K ? 32 : 16; }
 __host__ __device__ constexpr int64_t code_row_bytes(uint32_t type, int cols) { return int64_t(cols / 32) * code_bytes_per_sub(type); }
 __host__ __device__ constexpr int64_t aux_row_bytes(uint32_t type, int cols) {
     return type == TQMOE_NVFP4G ? int64_t(cols / 16) : int64_t(cols / 256) * aux_record_bytes(type);
@@ -63,6 +65,13 @@ __device__ __forceinline__ float e4m3_to_float(uint32_t b) {
     else v = __uint_as_float(uint32_t(e + 120) << 23 | uint32_t(m) << 20);  // (1 + m/8) * 2^(e - 7)
     return (b & 0x80u) ? -v : v;
 }
+
+// four bits -> the low bit of four bytes
+__device__ __forceinline__ uint32_t spread4(uint32_t bits) { return ((bits & 15u) * 0x00204081u) & 0x01010101u; }
+// eight bits (four 2-bit fields) -> the low two bits of four bytes
+__device__ __forceinline__ uint32_t spread2x4(uint32_t x) { x &= 0xFFu; return (x | x << 6 | x << 12 | x << 18) & 0x03030303u; }
+// bytes q in [0, 63] -> int8 bytes q - 32
+__device__ __forceinline__ uint32_t minus32(uint32_t v) { return ((v | 0x80808080u) - 0x20202020u) ^ 0x80808080u; }
 
 // Q4_K: 6-bit (scale, min) of sub-block j from the 12-byte field held as three dwords
 __device__ __forceinline__ void q4k_scale_min(const uint32_t (&q)[3], int j, int & sc, int & mn) {

@@ -25,7 +25,7 @@ struct Plan {  // byte offsets into the workspace
     size_t xq, xs, counts, offsets, perm, dispatch_ws, act16, aq, as, y16, rq, rs;   // grouped path
 };
 
-bool int8_ok(const tqmoe_layer & L) { return L.gate.type == TQMOE_IQ4_XS && (!L.has_shared || L.shared_ff % 256 == 0); }
+bool int8_ok(const tqmoe_layer & L) { return L.gate.type == TQMOE_IQ4_XS && L.down.type == TQMOE_IQ4_XS && (!L.has_shared || L.shared_ff % 256 == 0); }
 
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
@@ -90,7 +90,7 @@ int32_t check_layer(const tqmoe_layer * L, tqmoe_error * err) {
     if (L->router_type != TQMOE_F32 && L->router_type != TQMOE_BF16) return fail(err, TQMOE_E_UNSUPPORTED, "%s: router type must be F32 or BF16", what);
     for (const tqmoe_bank * b : {&L->gate, &L->up, &L->down}) if (int32_t rc = check_bank(b, what, err)) return rc;
     const int banks = L->n_expert + (L->has_shared ? 1 : 0);
-    if (L->gate.type != L->up.type || L->gate.type != L->down.type) return fail(err, TQMOE_E_UNSUPPORTED, "%s: the three banks must share one format", what);
+    if (L->gate.type != L->up.type) return fail(err, TQMOE_E_UNSUPPORTED, "%s: the gate and up banks must share one format (down may have its own)", what);
     if (L->gate.rows != L->ff || L->gate.cols != L->hidden || L->up.rows != L->ff || L->up.cols != L->hidden || L->down.rows != L->hidden ||
         L->down.cols != L->ff || L->gate.experts != banks || L->up.experts != banks || L->down.experts != banks)
         return fail(err, TQMOE_E_ARG, "%s: bank shapes do not match the layer (%d experts of %d x %d expected)", what, banks, L->ff, L->hidden);

@@ -2,6 +2,8 @@
 // follows in the reference and how it is pinned). Nothing in the product library links or loads this file.
 #include "tqmoe_oracle.h"
 #include "iq3s_lattice.h"
+#include "iq3xxs_lattice.h"
+#include "iq2s_lattice.h"
 
 #include <algorithm>
 #include <atomic>
@@ -107,6 +109,8 @@ int tqo_block_layout(uint32_t type, int * elems, int * bytes) {
         case TQO_IQ4_NL: e = 32; b = 18; break;
         case TQO_Q8_0: e = 32; b = 34; break;
         case TQO_IQ3_S: e = 256; b = 110; break;
+        case TQO_IQ3_XXS: e = 256; b = 98; break;
+        case TQO_IQ2_S: e = 256; b = 82; break;
         case TQO_IQ4_XS: e = 256; b = 136; break;
         case TQO_NVFP4G: e = 128; b = 76; break;
         default: return 0;
@@ -192,6 +196,37 @@ void decode_iq4nl(const uint8_t * b, float * y) {
     }
 }
 
+void decode_iq3xxs(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:157-174
+    const float d = tqo_half_to_float(rd16(b));
+    const uint8_t * qs = b + 2;
+    for (int ib = 0; ib < 8; ++ib) {
+        uint32_t a;
+        std::memcpy(&a, b + 66 + 4 * ib, 4);
+        const float db = d * (0.5f + float(a >> 28)) * 0.5f;
+        for (int l = 0; l < 4; ++l) {
+            // seven stored sign bits for eight weights; the eighth makes the number of minus signs even
+            const uint32_t i7 = (a >> (7 * l)) & 127u, sg = i7 | ((uint32_t(__builtin_popcount(i7)) & 1u) << 7);
+            for (int h = 0; h < 2; ++h, y += 4) {
+                const uint32_t g = tq_iq3xxs_point(qs[ib * 8 + 2 * l + h]);
+                for (int j = 0; j < 4; ++j) y[j] = db * float((g >> (8 * j)) & 0xFFu) * (((sg >> (4 * h + j)) & 1u) ? -1.f : 1.f);
+            }
+        }
+    }
+}
+
+void decode_iq2s(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:271-287
+    const float d = tqo_half_to_float(rd16(b));
+    const uint8_t * qs = b + 2, * signs = b + 34, * qh = b + 66, * sc = b + 74;
+    for (int ib = 0; ib < 8; ++ib) {
+        const float db[2] = {d * (0.5f + float(sc[ib] & 15)) * 0.25f, d * (0.5f + float(sc[ib] >> 4)) * 0.25f};
+        for (int l = 0; l < 4; ++l) {
+            const uint64_t g = tq_iq2s_point(qs[4 * ib + l] | ((qh[ib] << (8 - 2 * l)) & 0x300));
+            for (int j = 0; j < 8; ++j)
+                y[32 * ib + 8 * l + j] = db[l / 2] * float((g >> (8 * j)) & 0xFFu) * ((signs[4 * ib + l] >> j) & 1 ? -1.f : 1.f);
+        }
+    }
+}
+
 void decode_q8_0(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:555-562
     const float d = tqo_half_to_float(rd16(b));
     for (int j = 0; j < 32; ++j) y[j] = d * float(int8_t(b[2 + j]));
@@ -240,6 +275,8 @@ int tqo_dequantize(uint32_t type, const void * src, float * dst, int64_t n) {
         case TQO_IQ4_NL: decode_iq4nl(s, dst); break;
         case TQO_Q8_0: decode_q8_0(s, dst); break;
         case TQO_IQ3_S: decode_iq3s(s, dst); break;
+        case TQO_IQ3_XXS: decode_iq3xxs(s, dst); break;
+        case TQO_IQ2_S: decode_iq2s(s, dst); break;
         case TQO_NVFP4G: decode_nvfp4g(s, dst); break;
     }
     return 0;

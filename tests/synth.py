@@ -13,6 +13,10 @@ CONFIGS = {
 }
 
 
+# formats the oracle has no encoder for: offset of the fp16 block scale and the range it is drawn from (weights of about 0.02)
+RANDOM_BLOCKS = {oracle.IQ3_XXS: (0, 1.5e-4, 4e-4), oracle.IQ2_S: (0, 4e-4, 1e-3)}
+
+
 def small(cfg, hidden, ff, experts, topk=None):
     c = dict(cfg)
     c.update(hidden=hidden, ff=ff, experts=experts, topk=min(topk or cfg["topk"], experts))
@@ -45,8 +49,16 @@ def make_banks(cfg, seed, distinct=None, sigma=0.02):
     rng = np.random.default_rng(seed)
     banks = []
     for rows, cols in ((f, h), (f, h), (h, f)):
-        w = (rng.standard_normal((d * rows, cols)) * sigma).astype(np.float32)
-        raw = oracle.quantize(cfg["wtype"], w)
+        if cfg["wtype"] in RANDOM_BLOCKS:     # no encoder for this format: random valid blocks with scales of the same size
+            el, nbytes = oracle.BLOCK[cfg["wtype"]]
+            blocks = rng.integers(0, 256, (d * rows * cols // el, nbytes), dtype=np.uint8)
+            off, lo, hi = RANDOM_BLOCKS[cfg["wtype"]]
+            dd = np.float16(rng.uniform(lo, hi, len(blocks)) * rng.choice([-1, 1], len(blocks)))
+            blocks[:, off:off + 2] = dd.view(np.uint8).reshape(-1, 2)
+            raw = blocks.reshape(-1)
+        else:
+            w = (rng.standard_normal((d * rows, cols)) * sigma).astype(np.float32)
+            raw = oracle.quantize(cfg["wtype"], w)
         per = raw.size // d
         if d < e:
             raw = np.tile(raw, (e + d - 1) // d)[: per * e].copy()

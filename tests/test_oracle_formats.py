@@ -199,13 +199,69 @@ def test_q5k_q6k_independent_decode_and_round_trip(oracle, wtype, bits):
     assert np.abs(back - x).max() < np.abs(x).max() / (2 ** bits - 1) * 1.6
 
 
-@pytest.mark.parametrize("wtype", [8, 12, 13, 14, 20, 21, 23, 323])
+def test_iq3xxs_closed_form(oracle):
+    """IQ3_XXS (dequant.cpp:157-174): lattice index 0 is the point (4, 4, 4, 4); the scale nibble s gives d (0.5 + s) / 2;
+    the seven stored sign bits are completed by a parity bit, so one stored minus sign makes the eighth weight negative too."""
+    b = np.zeros(98, np.uint8)
+    b[0:2] = np.array([np.float16(0.25)]).view(np.uint8)
+    words = np.zeros(8, np.uint32)
+    words[0] = 3 << 28                        # sub-block 0: scale nibble 3, no minus signs
+    words[1] = (1 << 28) | 0b0000001          # sub-block 1: first group has weight 0 negative -> parity makes weight 7 negative
+    words[2] = (15 << 28) | (0b0000011 << 7)  # sub-block 2: second group, weights 0 and 1 negative, parity even
+    b[66:98] = words.view(np.uint8)
+    got = oracle.dequantize(oracle.IQ3_XXS, b, 256)
+    assert np.array_equal(got[0:32], np.full(32, 0.25 * 3.5 * 0.5 * 4, np.float32))
+    want1 = np.full(32, 0.25 * 1.5 * 0.5 * 4, np.float32)
+    want1[[0, 7]] *= -1
+    assert np.array_equal(got[32:64], want1)
+    want2 = np.full(32, 0.25 * 15.5 * 0.5 * 4, np.float32)
+    want2[[8, 9]] *= -1
+    assert np.array_equal(got[64:96], want2)
+    # every lattice point has magnitudes from the eight levels, and the table's points are distinct
+    idx = np.zeros(98, np.uint8)
+    idx[0:2] = np.array([np.float16(1.0)]).view(np.uint8)
+    pts = set()
+    for base in range(0, 256, 64):
+        idx[2:66] = np.arange(base, base + 64, dtype=np.uint8)
+        v = oracle.dequantize(oracle.IQ3_XXS, idx, 256) * 4        # d (0.5 + 0) / 2 = 0.25
+        assert set(np.unique(v).tolist()) <= {4.0, 12.0, 20.0, 28.0, 36.0, 44.0, 52.0, 62.0}
+        pts |= {tuple(r) for r in v.reshape(64, 4).tolist()}
+    assert len(pts) == 256
+
+
+def test_iq2s_closed_form(oracle):
+    """IQ2_S (dequant.cpp:271-287): lattice index 0 is the point of eight 8s; the low scale nibble serves the first 16 weights
+    of a sub-block, the high one the other 16; a sign byte's bit j negates weight j of its group; qh adds 256 per two bits."""
+    b = np.zeros(82, np.uint8)
+    b[0:2] = np.array([np.float16(0.5)]).view(np.uint8)
+    b[74] = 0x53                 # sub-block 0: nibble 3 for weights 0..15, 5 for 16..31
+    b[34] = 0b10000001           # group 0: weights 0 and 7 negative
+    got = oracle.dequantize(oracle.IQ2_S, b, 256)
+    want = np.concatenate([np.full(16, 0.5 * 3.5 * 0.25 * 8), np.full(16, 0.5 * 5.5 * 0.25 * 8)]).astype(np.float32)
+    want[[0, 7]] *= -1
+    assert np.array_equal(got[:32], want)
+    assert np.array_equal(got[32:], np.full(224, 0.5 * 0.5 * 0.25 * 8, np.float32))
+    # the index reaches all 1024 points through qh; they are distinct and their magnitudes are the three levels
+    pts = set()
+    blk = np.zeros(82, np.uint8)
+    blk[0:2] = np.array([np.float16(1.0)]).view(np.uint8)
+    for hi in range(4):
+        blk[66:74] = hi * 0x55                       # the same two high bits for the four groups of every sub-block
+        for base in range(0, 256, 32):
+            blk[2:34] = np.arange(base, base + 32, dtype=np.uint8)
+            v = oracle.dequantize(oracle.IQ2_S, blk, 256) * 8          # d (0.5 + 0) / 4 = 0.125
+            assert set(np.unique(v).tolist()) <= {8.0, 25.0, 43.0}
+            pts |= {tuple(r) for r in v.reshape(32, 8).tolist()}
+    assert len(pts) == 1024
+
+
+@pytest.mark.parametrize("wtype", [8, 12, 13, 14, 18, 20, 21, 22, 23, 323])
 def test_decoders_match_reference_objects(oracle, ref, wtype):
     rng = np.random.default_rng(wtype)
     el, bb = oracle.BLOCK[wtype]
     nb = 64
     raw = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
-    halves = {8: [0], 12: [0, 2], 13: [0, 2], 14: [208], 20: [0], 21: [0], 23: [0]}.get(wtype, [])
+    halves = {8: [0], 12: [0, 2], 13: [0, 2], 14: [208], 18: [0], 20: [0], 21: [0], 22: [0], 23: [0]}.get(wtype, [])
     for off in halves:
         raw[:, off:off + 2] = np.float16(rng.uniform(1e-3, 5e-2, nb) * rng.choice([-1, 1], nb)).view(np.uint8).reshape(nb, 2)
     if wtype == 323:

@@ -65,6 +65,26 @@ __global__ __launch_bounds__(256) void load_k(uint32_t type, const uint8_t * __r
             }
             break;
         }
+        case TQMOE_IQ3_XXS: {  // 98 B per 256: d, qs[64] (lattice indices), 8 words of 4 x 7 sign bits + 4-bit scale
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 98;
+            const int ib = s & 7;
+            uint32_t * o = reinterpret_cast<uint32_t *>(cd);
+            o[0] = rd_u32(blk + 2 + 8 * ib);
+            o[1] = rd_u32(blk + 2 + 8 * ib + 4);
+            o[2] = rd_u32(blk + 66 + 4 * ib);
+            if (ib == 0) *reinterpret_cast<uint4 *>(aux + (row * (S / 8) + s / 8) * 16) = make_uint4(rd_u16(blk), 0, 0, 0);
+            break;
+        }
+        case TQMOE_IQ2_S: {  // 82 B per 256: d, qs[32] (low index bytes), signs[32], qh[8], scales[8]
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 82;
+            const int ib = s & 7;
+            uint32_t * o = reinterpret_cast<uint32_t *>(cd);
+            o[0] = rd_u32(blk + 2 + 4 * ib);
+            o[1] = rd_u32(blk + 34 + 4 * ib);
+            o[2] = uint32_t(blk[66 + ib]) | uint32_t(blk[74 + ib]) << 8;
+            if (ib == 0) *reinterpret_cast<uint4 *>(aux + (row * (S / 8) + s / 8) * 16) = make_uint4(rd_u16(blk), 0, 0, 0);
+            break;
+        }
         case TQMOE_Q5_K: {  // 176 B per 256: d, dmin, scales[12], qh[32] (bit j of byte l: weight l of sub-block j), qs[128] as Q4_K
             const uint8_t * blk = src + (row * (S / 8) + s / 8) * 176;
             const int ib = s & 7;

@@ -80,6 +80,8 @@ void dispatch_matvec(uint32_t type, Split sp, int nb, const MatvecArgs & k, hipS
         case TQMOE_Q8_0: DecodeLaunch<TQMOE_Q8_0>::matvec(sp, nb, k, s); break;
         case TQMOE_Q5_K: DecodeLaunch<TQMOE_Q5_K>::matvec(sp, nb, k, s); break;
         case TQMOE_Q6_K: DecodeLaunch<TQMOE_Q6_K>::matvec(sp, nb, k, s); break;
+        case TQMOE_IQ3_XXS: DecodeLaunch<TQMOE_IQ3_XXS>::matvec(sp, nb, k, s); break;
+        case TQMOE_IQ2_S: DecodeLaunch<TQMOE_IQ2_S>::matvec(sp, nb, k, s); break;
         default: DecodeLaunch<TQMOE_NVFP4G>::matvec(sp, nb, k, s); break;
     }
 }
@@ -92,6 +94,8 @@ void dispatch_gateup(uint32_t type, Split sp, const GateupArgs & k, hipStream_t 
         case TQMOE_Q8_0: DecodeLaunch<TQMOE_Q8_0>::gateup(sp, k, s); break;
         case TQMOE_Q5_K: DecodeLaunch<TQMOE_Q5_K>::gateup(sp, k, s); break;
         case TQMOE_Q6_K: DecodeLaunch<TQMOE_Q6_K>::gateup(sp, k, s); break;
+        case TQMOE_IQ3_XXS: DecodeLaunch<TQMOE_IQ3_XXS>::gateup(sp, k, s); break;
+        case TQMOE_IQ2_S: DecodeLaunch<TQMOE_IQ2_S>::gateup(sp, k, s); break;
         default: DecodeLaunch<TQMOE_NVFP4G>::gateup(sp, k, s); break;
     }
 }

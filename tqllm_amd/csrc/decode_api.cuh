@@ -48,5 +48,7 @@ extern template struct DecodeLaunch<TQMOE_IQ4_NL>;
 extern template struct DecodeLaunch<TQMOE_Q8_0>;
 extern template struct DecodeLaunch<TQMOE_Q5_K>;
 extern template struct DecodeLaunch<TQMOE_Q6_K>;
+extern template struct DecodeLaunch<TQMOE_IQ3_XXS>;
+extern template struct DecodeLaunch<TQMOE_IQ2_S>;
 
 }  // namespace tqmoe

@@ -87,6 +87,57 @@ template <> struct Sub<TQMOE_Q4_K> {
     }
 };
 
+template <> struct Sub<TQMOE_IQ3_XXS> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint32_t c[3]; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        const uint32_t * cp = reinterpret_cast<const uint32_t *>(t.codes + (r * S + s) * 12u);
+        v.c[0] = cp[0]; v.c[1] = cp[1]; v.c[2] = cp[2];
+        v.d = *reinterpret_cast<const uint16_t *>(t.aux + (r * (S >> 3) + (s >> 3)) * 16u);
+        return v;
+    }
+    // grid: the 256-entry lattice in LDS
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t * grid, Dec & d) {
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            const uint32_t g = grid[(r.c[w >> 2] >> (8 * (w & 3))) & 0xFFu];
+            const uint32_t bits = spread4(iq3xxs_signs(r.c[2], w >> 1) >> (4 * (w & 1)));
+            const uint32_t m = (bits << 8) - bits;   // byte masks 0xFF; negate the selected bytes: (g ^ m) + bits, no carry leaves a byte
+            d.w[w] = (g ^ m) + bits;
+        }
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.d)) * (0.5f + float(r.c[2] >> 28)) * 0.5f;
+        d.mn = 0.f;
+    }
+};
+
+template <> struct Sub<TQMOE_IQ2_S> {
+    static constexpr bool kSplit = true;   // one scale nibble per 16 weights: the sub-block's halves
+    struct Raw { uint32_t c[3]; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        const uint32_t * cp = reinterpret_cast<const uint32_t *>(t.codes + (r * S + s) * 12u);
+        v.c[0] = cp[0]; v.c[1] = cp[1]; v.c[2] = cp[2];
+        v.d = *reinterpret_cast<const uint16_t *>(t.aux + (r * (S >> 3) + (s >> 3)) * 16u);
+        return v;
+    }
+    // grid: the 1024-point lattice in LDS, two dwords per point
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t * grid, Dec & d) {
+        const uint32_t qh = r.c[2] & 0xFFu, sc = (r.c[2] >> 8) & 0xFFu;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {   // group l = w / 2 of eight weights, half h = w % 2
+            const uint32_t g = grid[2 * iq2s_index(r.c[0], qh, w >> 1) + (w & 1)];
+            const uint32_t bits = spread4(r.c[1] >> (8 * (w >> 1) + 4 * (w & 1)));
+            const uint32_t m = (bits << 8) - bits;
+            d.w[w] = (g ^ m) + bits;
+        }
+        const float dd = half_bits_to_float(uint16_t(r.d));
+        d.s0 = dd * (0.5f + float(sc & 15u)) * 0.25f;
+        d.s1 = dd * (0.5f + float(sc >> 4)) * 0.25f;
+        d.mn = 0.f;
+    }
+};
+
 template <> struct Sub<TQMOE_Q5_K> {
     static constexpr bool kSplit = false;
     struct Raw { uint4 c; uint4 rec; uint32_t hb; };
@@ -233,6 +284,14 @@ template <uint32_t FMT> __device__ __forceinline__ const uint32_t * stage_grid(u
         for (int i = threadIdx.x; i < 512; i += blockDim.x) lds[i] = d_iq3s_grid.v[i];
         __syncthreads();
         return lds;
+    } else if constexpr (FMT == TQMOE_IQ2_S) {
+        for (int i = threadIdx.x; i < 2048; i += blockDim.x) lds[i] = d_iq2s_grid.v[i];
+        __syncthreads();
+        return lds;
+    } else if constexpr (FMT == TQMOE_IQ3_XXS) {
+        for (int i = threadIdx.x; i < 256; i += blockDim.x) lds[i] = d_iq3xxs_grid.v[i];
+        __syncthreads();
+        return lds;
     } else {
         return nullptr;
     }
@@ -332,7 +391,7 @@ __device__ __forceinline__ void load_x(const uint8_t * __restrict__ image, const
 template <uint32_t FMT, int LPR, int M, int NB, int NJ, int NW>
 __global__ __launch_bounds__(NW * 64) void matvec_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * y0, void * y1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_cols) {
-    __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : 1];
+    __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : FMT == TQMOE_IQ3_XXS ? 256 : FMT == TQMOE_IQ2_S ? 2048 : 1];
     __shared__ int meta[2];
     const uint32_t * grid = stage_grid<FMT>(grid_lds);
     const int a = blockIdx.y, e = ids[a];
@@ -374,7 +433,7 @@ __global__ __launch_bounds__(NW * 64) void gateup_k(BankView bg, BankView bu, co
                                                     const int * __restrict__ ids, int A, int slots, int topk, int shared_ff, int mode) {
     constexpr int RW = 64 / LPR, NJ = 32 / (NW * RW);
     static_assert(NJ >= 1 && NJ * NW * RW == 32, "a block makes exactly 32 rows");
-    __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : 1];
+    __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : FMT == TQMOE_IQ3_XXS ? 256 : FMT == TQMOE_IQ2_S ? 2048 : 1];
     __shared__ int meta[2];
     __shared__ float gl[2][32], ul[2][32];
     __shared__ int ql[2][32];

@@ -67,6 +67,39 @@ __device__ __forceinline__ void decode_sub32(uint32_t type, const uint8_t * __re
             }
             break;
         }
+        case TQMOE_IQ3_XXS: {  // dequant.cpp:157-174: ((d * (0.5 + s)) * 0.5) * magnitude, sign applied last
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(aux + (row * (S / 8) + s / 8) * 16));
+            const uint32_t * c = reinterpret_cast<const uint32_t *>(cd);
+            const uint32_t qs[2] = {c[0], c[1]}, word = c[2];
+            const float db = __fmul_rn(__fmul_rn(d, __fadd_rn(0.5f, float(word >> 28))), 0.5f);
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {   // group l = w / 2 of eight weights, half h = w % 2
+                const uint32_t g = d_iq3xxs_grid.v[(qs[w >> 2] >> (8 * (w & 3))) & 0xFFu];
+                const uint32_t sn = iq3xxs_signs(word, w >> 1) >> (4 * (w & 1));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float mag = __fmul_rn(db, float((g >> (8 * j)) & 0xFFu));
+                    y[4 * w + j] = ((sn >> j) & 1u) ? -mag : mag;
+                }
+            }
+            break;
+        }
+        case TQMOE_IQ2_S: {  // dequant.cpp:271-287: ((d * (0.5 + nibble)) * 0.25) * magnitude, one nibble per 16 weights
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(aux + (row * (S / 8) + s / 8) * 16));
+            const uint32_t * c = reinterpret_cast<const uint32_t *>(cd);
+            const uint32_t low = c[0], sg = c[1], qh = c[2] & 0xFFu, sc = (c[2] >> 8) & 0xFFu;
+            const float db[2] = {__fmul_rn(__fmul_rn(d, __fadd_rn(0.5f, float(sc & 15u))), 0.25f), __fmul_rn(__fmul_rn(d, __fadd_rn(0.5f, float(sc >> 4))), 0.25f)};
+#pragma unroll
+            for (int l = 0; l < 4; ++l) {
+                const uint32_t idx = iq2s_index(low, qh, l), sn = (sg >> (8 * l)) & 0xFFu;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float mag = __fmul_rn(db[l >> 1], float((d_iq2s_grid.v[2 * idx + (j >> 2)] >> (8 * (j & 3))) & 0xFFu));
+                    y[8 * l + j] = ((sn >> j) & 1u) ? -mag : mag;
+                }
+            }
+            break;
+        }
         case TQMOE_Q5_K: {  // dequant.cpp:102-116: (d * sc) * v - dmin * m, v = nibble + 16 * high bit
             const uint8_t * a = aux + (row * (S / 8) + s / 8) * 48;
             const uint4 rec = *reinterpret_cast<const uint4 *>(a);

@@ -3,11 +3,13 @@
 #pragma once
 #include "common.cuh"
 #include "iq3s_lattice.h"
+#include "iq3xxs_lattice.h"
+#include "iq2s_lattice.h"
 
 namespace tqmoe {
 
 // code bytes per sub-block
-__host__ __device__ constexpr int code_bytes_per_sub(uint32_t type) { return type == TQMOE_IQ3_S ? 12 : type == TQMOE_Q8_0 ? 32 : type == TQMOE_Q6_K ? 24 : 16; }
+__host__ __device__ constexpr int code_bytes_per_sub(uint32_t type) { return type == TQMOE_IQ3_S || type == TQMOE_IQ3_XXS || type == TQMOE_IQ2_S ? 12 : type == TQMOE_Q8_0 ? 32 : type == TQMOE_Q6_K ? 24 : 16; }
 // aux record bytes per 256 weights (NVFP4G keeps bytes per 16 weights instead: see aux_row_bytes; IQ4_NL and Q8_0 hold
 // the eight fp16 scales of their 32-weight blocks)
 // Q5_K: the Q4_K header and the eight sub-blocks' high-bit words; Q6_K: sixteen int8 scales, d, padding
@@ -55,6 +57,43 @@ constexpr Iq3sGrid make_iq3s_grid() {
     return g;
 }
 __device__ const Iq3sGrid d_iq3s_grid = make_iq3s_grid();
+
+// IQ3_XXS lattice points in the classic form
+struct Iq3xxsGrid { uint32_t v[256]; };
+constexpr uint32_t iq3xxs_level(uint32_t l) { return l < 7u ? 8u * l + 4u : 62u; }
+constexpr Iq3xxsGrid make_iq3xxs_grid() {
+    constexpr uint16_t codes[256] = {TQMOE_IQ3XXS_LATTICE12};
+    Iq3xxsGrid g{};
+    for (int i = 0; i < 256; ++i) {
+        const uint32_t c = codes[i];
+        g.v[i] = iq3xxs_level(c & 7u) | (iq3xxs_level((c >> 3) & 7u) << 8) | (iq3xxs_level((c >> 6) & 7u) << 16) | (iq3xxs_level((c >> 9) & 7u) << 24);
+    }
+    return g;
+}
+__device__ const Iq3xxsGrid d_iq3xxs_grid = make_iq3xxs_grid();
+// IQ2_S lattice points: two dwords per point (magnitudes of weights 0..3, 4..7 of the group of eight)
+struct Iq2sGrid { uint32_t v[2048]; };
+constexpr Iq2sGrid make_iq2s_grid() {
+    constexpr uint16_t codes[1024] = {TQMOE_IQ2S_LATTICE16};
+    constexpr uint32_t level[4] = {8, 25, 43, 0};
+    Iq2sGrid g{};
+    for (int i = 0; i < 1024; ++i)
+        for (int h = 0; h < 2; ++h) {
+            uint32_t w = 0;
+            for (int j = 0; j < 4; ++j) w |= level[(codes[i] >> (2 * (4 * h + j))) & 3u] << (8 * j);
+            g.v[2 * i + h] = w;
+        }
+    return g;
+}
+__device__ const Iq2sGrid d_iq2s_grid = make_iq2s_grid();
+// lattice index of group l of an IQ2_S sub-block: its low byte and two bits of the sub-block's qh byte
+__device__ __forceinline__ uint32_t iq2s_index(uint32_t low4, uint32_t qh, int l) { return ((low4 >> (8 * l)) & 0xFFu) | ((qh << (8 - 2 * l)) & 0x300u); }
+
+// the eight sign bits of a group of eight weights from its seven stored ones: the eighth makes their count even
+__device__ __forceinline__ uint32_t iq3xxs_signs(uint32_t word, int l) {
+    const uint32_t i7 = (word >> (7 * l)) & 127u;
+    return i7 | ((uint32_t(__popc(i7)) & 1u) << 7);
+}
 
 // E4M3 byte -> float: (1 + m/8) 2^(e-7), subnormal m/8 2^-6, 0x7F / 0xFF NaN
 __device__ __forceinline__ float e4m3_to_float(uint32_t b) {

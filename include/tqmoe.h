@@ -30,7 +30,8 @@ enum { TQMOE_OK = 0, TQMOE_E_ARG = -1, TQMOE_E_UNSUPPORTED = -2, TQMOE_E_DEVICE 
 /* element types (GGUF type ids, src/core/gguf.hpp) */
 enum { TQMOE_F32 = 0, TQMOE_F16 = 1, TQMOE_BF16 = 30 };
 /* bank formats (GGUF type ids) */
-enum { TQMOE_Q8_0 = 8, TQMOE_Q4_K = 12, TQMOE_Q5_K = 13, TQMOE_Q6_K = 14, TQMOE_IQ3_XXS = 18, TQMOE_IQ4_NL = 20, TQMOE_IQ3_S = 21, TQMOE_IQ2_S = 22, TQMOE_IQ4_XS = 23, TQMOE_NVFP4G = 323 };
+enum { TQMOE_Q4_0 = 2, TQMOE_Q8_0 = 8, TQMOE_Q3_K = 11, TQMOE_Q4_K = 12, TQMOE_Q5_K = 13, TQMOE_Q6_K = 14, TQMOE_IQ2_XXS = 16, TQMOE_IQ2_XS = 17,
+       TQMOE_IQ3_XXS = 18, TQMOE_IQ4_NL = 20, TQMOE_IQ3_S = 21, TQMOE_IQ2_S = 22, TQMOE_IQ4_XS = 23, TQMOE_NVFP4G = 323 };
 
 uint32_t tqmoe_abi_version(void);
 
@@ -109,7 +110,14 @@ int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets,
  *           256 weights: d (f16), padding.
  *   IQ2_S   codes 12 B: 4 low index bytes, 4 sign bytes, the sub-block's qh byte, its scale byte, 2 B padding; aux as
  *           IQ3_XXS.
+ *   IQ2_XS  codes 12 B: GGUF's four 16-bit fields (9-bit lattice index, 7 sign bits), the sub-block's scale byte, 3 B
+ *           padding; aux as IQ3_XXS.
+ *   IQ2_XXS codes 8 B: 4 lattice index bytes, then GGUF's word of four 7-bit sign fields and the 4-bit scale; aux as IQ3_XXS.
+ *   Q3_K    codes 12 B: 8 B with the low two bits (byte k = weights 4 k .. 4 k + 3), then 4 B with the third bit (bit j =
+ *           weight j; the weight is the three-bit value minus 4); aux 32 B per 256 weights: the sixteen 6-bit scales minus
+ *           32 as int8 (two per sub-block), d (f16), padding.
  *   IQ4_NL  codes 16 B, GGUF's own nibble order; aux 2 B per sub-block: its d (f16).
+ *   Q4_0    as IQ4_NL (the weight is the nibble minus 8).
  *   Q8_0    codes 32 B: the int8 values; aux 2 B per sub-block: its d (f16).
  * cols must be a multiple of 256 (128 for NVFP4G). The grouped int8 products take IQ4_XS only; every format has the
  * decode products and the fp16 grouped products (tqmoe_expert_gemm, tqmoe_expert_gemm_gateup). */

@@ -4,6 +4,8 @@
 #include "iq3s_lattice.h"
 #include "iq3xxs_lattice.h"
 #include "iq2s_lattice.h"
+#include "iq2xxs_lattice.h"
+#include "iq2xs_lattice.h"
 
 #include <algorithm>
 #include <atomic>
@@ -111,6 +113,10 @@ int tqo_block_layout(uint32_t type, int * elems, int * bytes) {
         case TQO_IQ3_S: e = 256; b = 110; break;
         case TQO_IQ3_XXS: e = 256; b = 98; break;
         case TQO_IQ2_S: e = 256; b = 82; break;
+        case TQO_IQ2_XXS: e = 256; b = 66; break;
+        case TQO_IQ2_XS: e = 256; b = 74; break;
+        case TQO_Q3_K: e = 256; b = 110; break;
+        case TQO_Q4_0: e = 32; b = 18; break;
         case TQO_IQ4_XS: e = 256; b = 136; break;
         case TQO_NVFP4G: e = 128; b = 76; break;
         default: return 0;
@@ -227,6 +233,66 @@ void decode_iq2s(const uint8_t * b, float * y) {  // src/formats/weight/dequant.
     }
 }
 
+// the eight sign bits of a group of eight weights from a 7-bit field: the eighth makes the count of minus signs even
+// (ksigns_iq2xs of the reference, src/formats/weight/ksigns_iq2xs.inc: entry i is i | parity(i) << 7)
+inline uint32_t signs8(uint32_t i7) { return i7 | ((uint32_t(__builtin_popcount(i7)) & 1u) << 7); }
+
+void decode_iq2xxs(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:233-249
+    const float d = tqo_half_to_float(rd16(b));
+    for (int ib = 0; ib < 8; ++ib) {
+        uint32_t a[2];
+        std::memcpy(a, b + 2 + 8 * ib, 8);
+        const float db = d * (0.5f + float(a[1] >> 28)) * 0.25f;
+        for (int l = 0; l < 4; ++l) {
+            const uint64_t g = tq_iq2xxs_point((a[0] >> (8 * l)) & 0xFFu);
+            const uint32_t sg = signs8((a[1] >> (7 * l)) & 127u);
+            for (int j = 0; j < 8; ++j) y[32 * ib + 8 * l + j] = db * float((g >> (8 * j)) & 0xFFu) * (((sg >> j) & 1u) ? -1.f : 1.f);
+        }
+    }
+}
+
+void decode_iq2xs(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:252-268
+    const float d = tqo_half_to_float(rd16(b));
+    const uint8_t * sc = b + 66;
+    for (int ib = 0; ib < 8; ++ib) {
+        const float db[2] = {d * (0.5f + float(sc[ib] & 15)) * 0.25f, d * (0.5f + float(sc[ib] >> 4)) * 0.25f};
+        for (int l = 0; l < 4; ++l) {
+            const uint32_t q = rd16(b + 2 + 2 * (4 * ib + l));
+            const uint64_t g = tq_iq2xs_point(q & 511u);
+            const uint32_t sg = signs8(q >> 9);
+            for (int j = 0; j < 8; ++j) y[32 * ib + 8 * l + j] = db[l / 2] * float((g >> (8 * j)) & 0xFFu) * (((sg >> j) & 1u) ? -1.f : 1.f);
+        }
+    }
+}
+
+void q3k_scales(const uint8_t * p, int8_t * sc) {  // src/formats/weight/dequant.cpp:66-76: 12 bytes -> 16 six-bit scales minus 32
+    // scale i: low four bits in byte i % 8 (low nibble for i < 8, high for i >= 8), upper two bits in byte 8 + i % 4 at 2 (i / 4)
+    for (int i = 0; i < 16; ++i) {
+        const int lo = i < 8 ? p[i] & 15 : p[i - 8] >> 4;
+        const int hi = (p[8 + (i & 3)] >> (2 * (i >> 2))) & 3;
+        sc[i] = int8_t((lo | (hi << 4)) - 32);
+    }
+}
+
+void decode_q3k(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:118-131: (d * sc) * q, q = two bits - (mask bit ? 0 : 4)
+    int8_t sc[16];
+    q3k_scales(b + 96, sc);
+    const float d = tqo_half_to_float(rd16(b + 108));
+    for (int e = 0; e < 256; ++e) {
+        const int n = e / 128, j = (e % 128) / 32, w = e % 32;
+        const int q = ((b[32 + 32 * n + w] >> (2 * j)) & 3) - (((b[w] >> (4 * n + j)) & 1) ? 0 : 4);
+        y[e] = d * float(sc[8 * n + 2 * j + (w >= 16)]) * float(q);
+    }
+}
+
+void decode_q4_0(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:480-491: (q - 8) * d
+    const float d = tqo_half_to_float(rd16(b));
+    for (int j = 0; j < 16; ++j) {
+        y[j] = float(int(b[2 + j] & 15) - 8) * d;
+        y[16 + j] = float(int(b[2 + j] >> 4) - 8) * d;
+    }
+}
+
 void decode_q8_0(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:555-562
     const float d = tqo_half_to_float(rd16(b));
     for (int j = 0; j < 32; ++j) y[j] = d * float(int8_t(b[2 + j]));
@@ -277,6 +343,10 @@ int tqo_dequantize(uint32_t type, const void * src, float * dst, int64_t n) {
         case TQO_IQ3_S: decode_iq3s(s, dst); break;
         case TQO_IQ3_XXS: decode_iq3xxs(s, dst); break;
         case TQO_IQ2_S: decode_iq2s(s, dst); break;
+        case TQO_IQ2_XXS: decode_iq2xxs(s, dst); break;
+        case TQO_IQ2_XS: decode_iq2xs(s, dst); break;
+        case TQO_Q3_K: decode_q3k(s, dst); break;
+        case TQO_Q4_0: decode_q4_0(s, dst); break;
         case TQO_NVFP4G: decode_nvfp4g(s, dst); break;
     }
     return 0;

@@ -14,7 +14,23 @@ CONFIGS = {
 
 
 # formats the oracle has no encoder for: offset of the fp16 block scale and the range it is drawn from (weights of about 0.02)
-RANDOM_BLOCKS = {oracle.IQ3_XXS: (0, 1.5e-4, 4e-4), oracle.IQ2_S: (0, 4e-4, 1e-3)}
+RANDOM_BLOCKS = {oracle.IQ3_XXS: (0, 1.5e-4, 4e-4), oracle.IQ2_S: (0, 4e-4, 1e-3), oracle.Q4_0: (0, 2e-3, 6e-3), oracle.Q3_K: (108, 3e-4, 7e-4),
+                 oracle.IQ2_XXS: (0, 2e-4, 5e-4), oracle.IQ2_XS: (0, 2e-4, 5e-4)}
+# byte offset of the fp16 block scale where it is not the block's first field
+SCALE_OFFSET = {oracle.Q6_K: 208, oracle.Q3_K: 108}
+
+
+def bank_blocks(wtype, rows, cols, rng, sigma=0.02):
+    """GGUF blocks of a [rows][cols] matrix with weights of about `sigma`: encoded N(0, sigma) values, or, for a format the
+    oracle has no encoder for, random valid blocks with block scales that give weights of that size."""
+    if wtype in RANDOM_BLOCKS:
+        el, nbytes = oracle.BLOCK[wtype]
+        blocks = rng.integers(0, 256, (rows * cols // el, nbytes), dtype=np.uint8)
+        off, lo, hi = RANDOM_BLOCKS[wtype]
+        dd = np.float16(rng.uniform(lo, hi, len(blocks)) * (sigma / 0.02) * rng.choice([-1, 1], len(blocks)))
+        blocks[:, off:off + 2] = dd.view(np.uint8).reshape(-1, 2)
+        return blocks.reshape(-1)
+    return oracle.quantize(wtype, (rng.standard_normal((rows, cols)) * sigma).astype(np.float32))
 
 
 def small(cfg, hidden, ff, experts, topk=None):
@@ -33,8 +49,9 @@ def _scale_field(raw, wtype, per_expert_blocks, factors):
         g = blocks[:, :, 0:4].copy().view(np.float32)
         blocks[:, :, 0:4] = (g * factors[:, None, None].astype(np.float32)).view(np.uint8)
     else:
-        d = blocks[:, :, 0:2].copy().view(np.float16).astype(np.float32)
-        blocks[:, :, 0:2] = (d * factors[:, None, None]).astype(np.float16).view(np.uint8)
+        o = SCALE_OFFSET.get(wtype, 0)
+        d = blocks[:, :, o:o + 2].copy().view(np.float16).astype(np.float32)
+        blocks[:, :, o:o + 2] = (d * factors[:, None, None]).astype(np.float16).view(np.uint8)
         if wtype == oracle.Q4_K:
             m = blocks[:, :, 2:4].copy().view(np.float16).astype(np.float32)
             blocks[:, :, 2:4] = (m * factors[:, None, None]).astype(np.float16).view(np.uint8)
@@ -49,16 +66,7 @@ def make_banks(cfg, seed, distinct=None, sigma=0.02):
     rng = np.random.default_rng(seed)
     banks = []
     for rows, cols in ((f, h), (f, h), (h, f)):
-        if cfg["wtype"] in RANDOM_BLOCKS:     # no encoder for this format: random valid blocks with scales of the same size
-            el, nbytes = oracle.BLOCK[cfg["wtype"]]
-            blocks = rng.integers(0, 256, (d * rows * cols // el, nbytes), dtype=np.uint8)
-            off, lo, hi = RANDOM_BLOCKS[cfg["wtype"]]
-            dd = np.float16(rng.uniform(lo, hi, len(blocks)) * rng.choice([-1, 1], len(blocks)))
-            blocks[:, off:off + 2] = dd.view(np.uint8).reshape(-1, 2)
-            raw = blocks.reshape(-1)
-        else:
-            w = (rng.standard_normal((d * rows, cols)) * sigma).astype(np.float32)
-            raw = oracle.quantize(cfg["wtype"], w)
+        raw = bank_blocks(cfg["wtype"], d * rows, cols, rng, sigma)
         per = raw.size // d
         if d < e:
             raw = np.tile(raw, (e + d - 1) // d)[: per * e].copy()

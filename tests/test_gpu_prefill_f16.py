@@ -19,7 +19,7 @@ def tq():
     return tqllm_amd
 
 
-@pytest.mark.parametrize("wtype", [12, 21, 23, 323, 20, 8, 13, 14])
+@pytest.mark.parametrize("wtype", [12, 21, 23, 323, 20, 8, 13, 14, 11, 17])
 @pytest.mark.parametrize("n,shared_ff", [(70, 0), (200, 128)])
 def test_grouped_f16_products_against_float64(tq, oracle, wtype, n, shared_ff):
     rng = np.random.default_rng(wtype + n)
@@ -27,9 +27,8 @@ def test_grouped_f16_products_against_float64(tq, oracle, wtype, n, shared_ff):
     banks = experts + (1 if shared_ff else 0)
     decs, devb = [], []
     for rows, cols in ((ff, hidden), (ff, hidden), (hidden, ff)):
-        w = (rng.standard_normal((banks * rows, cols)) * 0.02).astype(np.float32)
-        raw = oracle.quantize(wtype, w)
-        decs.append(oracle.dequantize(wtype, raw, w.size).reshape(banks, rows, cols).astype(np.float64))
+        raw = synth.bank_blocks(wtype, banks * rows, cols, rng)
+        decs.append(oracle.dequantize(wtype, raw, banks * rows * cols).reshape(banks, rows, cols).astype(np.float64))
         devb.append(tq.ExpertBank(wtype, raw, banks, rows, cols))
     gate, up, down = devb
     slots = k + (1 if shared_ff else 0)

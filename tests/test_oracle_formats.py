@@ -255,13 +255,88 @@ def test_iq2s_closed_form(oracle):
     assert len(pts) == 1024
 
 
-@pytest.mark.parametrize("wtype", [8, 12, 13, 14, 18, 20, 21, 22, 23, 323])
+def test_q4_0_closed_form(oracle):
+    """Q4_0 (dequant.cpp:480-491): byte j of a block holds weight j (low nibble) and weight j + 16 (high), value (q - 8) d."""
+    b = np.zeros(18, np.uint8)
+    b[0:2] = np.array([np.float16(0.5)]).view(np.uint8)
+    b[2:18] = np.arange(16, dtype=np.uint8) | ((15 - np.arange(16, dtype=np.uint8)) << 4)
+    got = oracle.dequantize(oracle.Q4_0, b, 32)
+    want = np.concatenate([np.arange(16) - 8, 7 - np.arange(16)]).astype(np.float32) * 0.5
+    assert np.array_equal(got, want)
+
+
+def test_q3k_closed_form(oracle):
+    """Q3_K (dequant.cpp:66-76, 118-131): weight 128 n + 32 j + w takes two bits of qs[32 n + w] at 2 j and its third bit from
+    hmask[w] at 4 n + j (set: +0, clear: -4); scale 8 n + 2 j + (w >= 16) of sixteen 6-bit scales, each taken minus 32."""
+    rng = np.random.default_rng(3)
+    hm = rng.integers(0, 256, 32, dtype=np.uint8)
+    qs = rng.integers(0, 256, 64, dtype=np.uint8)
+    sc6 = rng.integers(0, 64, 16)
+    packed = np.zeros(12, np.uint8)
+    for i in range(16):           # the layout the reference unpacks: low nibbles in bytes 0..7, upper two bits in bytes 8..11
+        packed[i % 8] |= (sc6[i] & 15) << (4 * (i // 8))
+        packed[8 + i % 4] |= (sc6[i] >> 4) << (2 * (i // 4))
+    b = np.concatenate([hm, qs, packed, np.array([np.float16(0.25)]).view(np.uint8)])
+    got = oracle.dequantize(oracle.Q3_K, b, 256)
+    e = np.arange(256)
+    n, j, w = e // 128, (e % 128) // 32, e % 32
+    q = ((qs[32 * n + w] >> (2 * j)) & 3).astype(np.int32) - 4 * (1 - ((hm[w] >> (4 * n + j)) & 1).astype(np.int32))
+    want = (np.float32(0.25) * (sc6[8 * n + 2 * j + (w >= 16)] - 32).astype(np.float32)) * q.astype(np.float32)
+    assert np.array_equal(got, want.astype(np.float32))
+    assert q.min() == -4 and q.max() == 3
+
+
+@pytest.mark.parametrize("wtype,points", [(16, 256), (17, 512)])
+def test_iq2xxs_iq2xs_closed_form(oracle, wtype, points):
+    """IQ2_XXS (dequant.cpp:233-249) and IQ2_XS (252-268): lattice index 0 is the point of eight 8s; d (0.5 + s) / 4 with s
+    the word's top nibble (IQ2_XXS) or a nibble per 16 weights (IQ2_XS); seven stored sign bits completed by a parity bit."""
+    el, bb = oracle.BLOCK[wtype]
+    b = np.zeros(bb, np.uint8)
+    b[0:2] = np.array([np.float16(0.5)]).view(np.uint8)
+    if wtype == 16:
+        w = np.zeros(16, np.uint32)
+        w[1] = (3 << 28) | 0b0000001             # sub-block 0: scale 3, group 0 weight 0 negative -> weight 7 too
+        w[3] = (5 << 28) | (0b0000011 << 14)     # sub-block 1: scale 5, group 2 weights 0 and 1 negative
+        b[2:66] = w.view(np.uint8)
+        want0 = np.full(32, 0.5 * 3.5 * 0.25 * 8, np.float32)
+        want1 = np.full(32, 0.5 * 5.5 * 0.25 * 8, np.float32)
+    else:
+        q = np.zeros(32, np.uint16)
+        q[0] = 0b0000001 << 9
+        q[6] = 0b0000011 << 9
+        b[2:66] = q.view(np.uint8)
+        b[66], b[67] = 0x73, 0x95                # sub-block 0: nibbles 3 | 7, sub-block 1: 5 | 9
+        want0 = np.concatenate([np.full(16, 0.5 * 3.5 * 0.25 * 8), np.full(16, 0.5 * 7.5 * 0.25 * 8)]).astype(np.float32)
+        want1 = np.concatenate([np.full(16, 0.5 * 5.5 * 0.25 * 8), np.full(16, 0.5 * 9.5 * 0.25 * 8)]).astype(np.float32)
+    want0[[0, 7]] *= -1
+    want1[[16, 17]] *= -1
+    got = oracle.dequantize(wtype, b, 256)
+    assert np.array_equal(got[0:32], want0) and np.array_equal(got[32:64], want1)
+    assert np.array_equal(got[64:], np.full(192, 0.5 * 0.5 * 0.25 * 8, np.float32))
+    # every point of the lattice is reached, the points are distinct and their magnitudes are the three levels
+    blk = np.zeros(bb, np.uint8)
+    blk[0:2] = np.array([np.float16(1.0)]).view(np.uint8)
+    pts = set()
+    for base in range(0, points, 32):
+        if wtype == 16:
+            idx = np.zeros((8, 8), np.uint8)
+            idx[:, 0:4] = np.arange(base, base + 32, dtype=np.uint8).reshape(8, 4)
+            blk[2:66] = idx.reshape(-1)
+        else:
+            blk[2:66] = np.arange(base, base + 32, dtype=np.uint16).view(np.uint8)
+        v = oracle.dequantize(wtype, blk, 256) * 8
+        assert set(np.unique(v).tolist()) <= {8.0, 25.0, 43.0}
+        pts |= {tuple(r) for r in v.reshape(32, 8).tolist()}
+    assert len(pts) == points
+
+
+@pytest.mark.parametrize("wtype", [2, 8, 11, 12, 13, 14, 16, 17, 18, 20, 21, 22, 23, 323])
 def test_decoders_match_reference_objects(oracle, ref, wtype):
     rng = np.random.default_rng(wtype)
     el, bb = oracle.BLOCK[wtype]
     nb = 64
     raw = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
-    halves = {8: [0], 12: [0, 2], 13: [0, 2], 14: [208], 18: [0], 20: [0], 21: [0], 22: [0], 23: [0]}.get(wtype, [])
+    halves = {2: [0], 11: [108], 16: [0], 17: [0], 8: [0], 12: [0, 2], 13: [0, 2], 14: [208], 18: [0], 20: [0], 21: [0], 22: [0], 23: [0]}.get(wtype, [])
     for off in halves:
         raw[:, off:off + 2] = np.float16(rng.uniform(1e-3, 5e-2, nb) * rng.choice([-1, 1], nb)).view(np.uint8).reshape(nb, 2)
     if wtype == 323:

@@ -85,6 +85,56 @@ __global__ __launch_bounds__(256) void load_k(uint32_t type, const uint8_t * __r
             if (ib == 0) *reinterpret_cast<uint4 *>(aux + (row * (S / 8) + s / 8) * 16) = make_uint4(rd_u16(blk), 0, 0, 0);
             break;
         }
+        case TQMOE_IQ2_XXS: {  // 66 B per 256: d, per sub-block four lattice index bytes and a word of 4 x 7 sign bits + 4-bit scale
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 66;
+            const int ib = s & 7;
+            *reinterpret_cast<uint2 *>(cd) = make_uint2(rd_u32(blk + 2 + 8 * ib), rd_u32(blk + 2 + 8 * ib + 4));
+            if (ib == 0) *reinterpret_cast<uint4 *>(aux + (row * (S / 8) + s / 8) * 16) = make_uint4(rd_u16(blk), 0, 0, 0);
+            break;
+        }
+        case TQMOE_IQ2_XS: {  // 74 B per 256: d, 32 x (9-bit lattice index | 7 sign bits << 9), scales[8] (a nibble per 16 weights)
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 74;
+            const int ib = s & 7;
+            uint32_t * o = reinterpret_cast<uint32_t *>(cd);
+            o[0] = rd_u32(blk + 2 + 8 * ib);
+            o[1] = rd_u32(blk + 2 + 8 * ib + 4);
+            o[2] = blk[66 + ib];
+            if (ib == 0) *reinterpret_cast<uint4 *>(aux + (row * (S / 8) + s / 8) * 16) = make_uint4(rd_u16(blk), 0, 0, 0);
+            break;
+        }
+        case TQMOE_Q3_K: {  // 110 B per 256: hmask[32], qs[64], scales[12], d; sub-block i = 4 n + j holds weights 128 n + 32 j ..
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 110;
+            const int ib = s & 7, n = ib >> 2, j = ib & 3;
+            const uint8_t * qs = blk + 32 + 32 * n;
+            uint32_t lo[2] = {0, 0}, hb = 0;   // two low bits per weight (byte k = weights 4 k .. 4 k + 3), the third bit per weight
+#pragma unroll
+            for (int l = 0; l < 32; ++l) {
+                lo[l >> 4] |= uint32_t((qs[l] >> (2 * j)) & 3) << (2 * (l & 15));
+                hb |= uint32_t((blk[l] >> ib) & 1) << l;
+            }
+            uint32_t * o = reinterpret_cast<uint32_t *>(cd);
+            o[0] = lo[0]; o[1] = lo[1]; o[2] = hb;
+            if (ib == 0) {   // the sixteen 6-bit scales, stored minus 32 as int8 (what the decoder multiplies by), then d
+                const uint8_t * p = blk + 96;
+                uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const uint32_t l4 = i < 8 ? p[i] & 15u : uint32_t(p[i - 8]) >> 4;
+                    const uint32_t h2 = (uint32_t(p[8 + (i & 3)]) >> (2 * (i >> 2))) & 3u;
+                    w[i >> 2] |= (((l4 | h2 << 4) - 32u) & 0xFFu) << (8 * (i & 3));
+                }
+                uint8_t * a = aux + (row * (S / 8) + s / 8) * 32;
+                *reinterpret_cast<uint4 *>(a) = make_uint4(w[0], w[1], w[2], w[3]);
+                *reinterpret_cast<uint4 *>(a + 16) = make_uint4(rd_u16(blk + 108), 0, 0, 0);
+            }
+            break;
+        }
+        case TQMOE_Q4_0: {  // 18 B per 32: d, qs[16] (byte j = weight j | weight j + 16 << 4: the canonical order)
+            const uint8_t * blk = src + (row * S + s) * 18;
+            pack_sub(cd, [&](int j) { return j < 16 ? blk[2 + j] & 15 : blk[2 + j - 16] >> 4; });
+            *reinterpret_cast<uint16_t *>(aux + (row * S + s) * 2) = uint16_t(rd_u16(blk));
+            break;
+        }
         case TQMOE_Q5_K: {  // 176 B per 256: d, dmin, scales[12], qh[32] (bit j of byte l: weight l of sub-block j), qs[128] as Q4_K
             const uint8_t * blk = src + (row * (S / 8) + s / 8) * 176;
             const int ib = s & 7;

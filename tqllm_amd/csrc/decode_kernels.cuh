@@ -138,6 +138,102 @@ template <> struct Sub<TQMOE_IQ2_S> {
     }
 };
 
+template <> struct Sub<TQMOE_IQ2_XXS> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint2 c; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        v.c = *reinterpret_cast<const uint2 *>(t.codes + (r * S + s) * 8u);
+        v.d = *reinterpret_cast<const uint16_t *>(t.aux + (r * (S >> 3) + (s >> 3)) * 16u);
+        return v;
+    }
+    // grid: the 256-point lattice in LDS, two dwords per point
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t * grid, Dec & d) {
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const uint2 g = *reinterpret_cast<const uint2 *>(grid + 2u * ((r.c.x >> (8 * l)) & 0xFFu));
+            const uint32_t sn = iq3xxs_signs(r.c.y, l);
+            d.w[2 * l] = apply_signs4(g.x, sn);
+            d.w[2 * l + 1] = apply_signs4(g.y, sn >> 4);
+        }
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.d)) * (0.5f + float(r.c.y >> 28)) * 0.25f;
+        d.mn = 0.f;
+    }
+};
+
+template <> struct Sub<TQMOE_IQ2_XS> {
+    static constexpr bool kSplit = true;   // one scale nibble per 16 weights: the sub-block's halves
+    struct Raw { uint32_t c[3]; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        const uint32_t * cp = reinterpret_cast<const uint32_t *>(t.codes + (r * S + s) * 12u);
+        v.c[0] = cp[0]; v.c[1] = cp[1]; v.c[2] = cp[2];
+        v.d = *reinterpret_cast<const uint16_t *>(t.aux + (r * (S >> 3) + (s >> 3)) * 16u);
+        return v;
+    }
+    // grid: the 512-point lattice in LDS, two dwords per point
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t * grid, Dec & d) {
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const uint32_t q = (r.c[l >> 1] >> (16 * (l & 1))) & 0xFFFFu;
+            const uint2 g = *reinterpret_cast<const uint2 *>(grid + 2u * (q & 511u));
+            const uint32_t sn = signs8(q >> 9);
+            d.w[2 * l] = apply_signs4(g.x, sn);
+            d.w[2 * l + 1] = apply_signs4(g.y, sn >> 4);
+        }
+        const float dd = half_bits_to_float(uint16_t(r.d));
+        d.s0 = dd * (0.5f + float(r.c[2] & 15u)) * 0.25f;
+        d.s1 = dd * (0.5f + float((r.c[2] >> 4) & 15u)) * 0.25f;
+        d.mn = 0.f;
+    }
+};
+
+template <> struct Sub<TQMOE_Q3_K> {
+    static constexpr bool kSplit = true;   // one scale per 16 weights: the sub-block's halves
+    struct Raw { uint32_t c[3]; uint32_t sc; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        const uint32_t * cp = reinterpret_cast<const uint32_t *>(t.codes + (r * S + s) * 12u);
+        v.c[0] = cp[0]; v.c[1] = cp[1]; v.c[2] = cp[2];
+        const uint8_t * a = t.aux + (r * (S >> 3) + (s >> 3)) * 32u;
+        v.sc = *reinterpret_cast<const uint16_t *>(a + 2u * (s & 7u));
+        v.d = *reinterpret_cast<const uint16_t *>(a + 16u);
+        return v;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t *, Dec & d) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q)   // weights 4 q ..: two low bits from byte q of the low plane, the third from four mask bits
+            d.w[q] = minus_k<4>(spread2x4(r.c[q >> 2] >> (8 * (q & 3))) | spread4(r.c[2] >> (4 * q)) << 2);
+        const float dd = half_bits_to_float(uint16_t(r.d));
+        d.s0 = dd * float(int8_t(r.sc & 0xFFu));
+        d.s1 = dd * float(int8_t(r.sc >> 8));
+        d.mn = 0.f;
+    }
+};
+
+template <> struct Sub<TQMOE_Q4_0> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint4 c; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        v.c = *reinterpret_cast<const uint4 *>(t.codes + (r * S + s) * 16u);
+        v.d = *reinterpret_cast<const uint16_t *>(t.aux + (r * S + s) * 2u);
+        return v;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t *, Dec & d) {
+        const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t lo, hi;
+            nibbles(w[q], lo, hi);
+            d.w[q] = minus_k<8>(lo);
+            d.w[4 + q] = minus_k<8>(hi);
+        }
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.d));
+        d.mn = 0.f;
+    }
+};
+
 template <> struct Sub<TQMOE_Q5_K> {
     static constexpr bool kSplit = false;
     struct Raw { uint4 c; uint4 rec; uint32_t hb; };
@@ -280,16 +376,14 @@ template <> struct Sub<TQMOE_IQ3_S> {
 };
 
 template <uint32_t FMT> __device__ __forceinline__ const uint32_t * stage_grid(uint32_t * lds) {
-    if constexpr (FMT == TQMOE_IQ3_S) {
-        for (int i = threadIdx.x; i < 512; i += blockDim.x) lds[i] = d_iq3s_grid.v[i];
-        __syncthreads();
-        return lds;
-    } else if constexpr (FMT == TQMOE_IQ2_S) {
-        for (int i = threadIdx.x; i < 2048; i += blockDim.x) lds[i] = d_iq2s_grid.v[i];
-        __syncthreads();
-        return lds;
-    } else if constexpr (FMT == TQMOE_IQ3_XXS) {
-        for (int i = threadIdx.x; i < 256; i += blockDim.x) lds[i] = d_iq3xxs_grid.v[i];
+    const uint32_t * src = nullptr;
+    if constexpr (FMT == TQMOE_IQ3_S) src = d_iq3s_grid.v;
+    else if constexpr (FMT == TQMOE_IQ3_XXS) src = d_iq3xxs_grid.v;
+    else if constexpr (FMT == TQMOE_IQ2_S) src = d_iq2s_grid.v;
+    else if constexpr (FMT == TQMOE_IQ2_XS) src = d_iq2xs_grid.v;
+    else if constexpr (FMT == TQMOE_IQ2_XXS) src = d_iq2xxs_grid.v;
+    if constexpr (lattice_dwords(FMT) > 1) {
+        for (int i = threadIdx.x; i < lattice_dwords(FMT); i += blockDim.x) lds[i] = src[i];
         __syncthreads();
         return lds;
     } else {
@@ -391,7 +485,7 @@ __device__ __forceinline__ void load_x(const uint8_t * __restrict__ image, const
 template <uint32_t FMT, int LPR, int M, int NB, int NJ, int NW>
 __global__ __launch_bounds__(NW * 64) void matvec_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * y0, void * y1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_cols) {
-    __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : FMT == TQMOE_IQ3_XXS ? 256 : FMT == TQMOE_IQ2_S ? 2048 : 1];
+    __shared__ __attribute__((aligned(8))) uint32_t grid_lds[lattice_dwords(FMT)];
     __shared__ int meta[2];
     const uint32_t * grid = stage_grid<FMT>(grid_lds);
     const int a = blockIdx.y, e = ids[a];
@@ -433,7 +527,7 @@ __global__ __launch_bounds__(NW * 64) void gateup_k(BankView bg, BankView bu, co
                                                     const int * __restrict__ ids, int A, int slots, int topk, int shared_ff, int mode) {
     constexpr int RW = 64 / LPR, NJ = 32 / (NW * RW);
     static_assert(NJ >= 1 && NJ * NW * RW == 32, "a block makes exactly 32 rows");
-    __shared__ uint32_t grid_lds[FMT == TQMOE_IQ3_S ? 512 : FMT == TQMOE_IQ3_XXS ? 256 : FMT == TQMOE_IQ2_S ? 2048 : 1];
+    __shared__ __attribute__((aligned(8))) uint32_t grid_lds[lattice_dwords(FMT)];
     __shared__ int meta[2];
     __shared__ float gl[2][32], ul[2][32];
     __shared__ int ql[2][32];

@@ -100,6 +100,64 @@ __device__ __forceinline__ void decode_sub32(uint32_t type, const uint8_t * __re
             }
             break;
         }
+        case TQMOE_IQ2_XXS: {  // dequant.cpp:233-249: ((d * (0.5 + s)) * 0.25) * magnitude, sign applied last
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(aux + (row * (S / 8) + s / 8) * 16));
+            const uint2 c = *reinterpret_cast<const uint2 *>(cd);
+            const float db = __fmul_rn(__fmul_rn(d, __fadd_rn(0.5f, float(c.y >> 28))), 0.25f);
+#pragma unroll
+            for (int l = 0; l < 4; ++l) {
+                const uint32_t idx = (c.x >> (8 * l)) & 0xFFu, sn = iq3xxs_signs(c.y, l);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float mag = __fmul_rn(db, float((d_iq2xxs_grid.v[2 * idx + (j >> 2)] >> (8 * (j & 3))) & 0xFFu));
+                    y[8 * l + j] = ((sn >> j) & 1u) ? -mag : mag;
+                }
+            }
+            break;
+        }
+        case TQMOE_IQ2_XS: {  // dequant.cpp:252-268: ((d * (0.5 + nibble)) * 0.25) * magnitude, one nibble per 16 weights
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(aux + (row * (S / 8) + s / 8) * 16));
+            const uint32_t * c = reinterpret_cast<const uint32_t *>(cd);
+            const uint32_t q2[2] = {c[0], c[1]}, sc = c[2] & 0xFFu;
+            const float db[2] = {__fmul_rn(__fmul_rn(d, __fadd_rn(0.5f, float(sc & 15u))), 0.25f), __fmul_rn(__fmul_rn(d, __fadd_rn(0.5f, float(sc >> 4))), 0.25f)};
+#pragma unroll
+            for (int l = 0; l < 4; ++l) {
+                const uint32_t q = (q2[l >> 1] >> (16 * (l & 1))) & 0xFFFFu, idx = q & 511u, sn = signs8(q >> 9);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float mag = __fmul_rn(db[l >> 1], float((d_iq2xs_grid.v[2 * idx + (j >> 2)] >> (8 * (j & 3))) & 0xFFu));
+                    y[8 * l + j] = ((sn >> j) & 1u) ? -mag : mag;
+                }
+            }
+            break;
+        }
+        case TQMOE_Q3_K: {  // dequant.cpp:118-131: (d * sc) * (q - 4), q = two low bits | mask bit << 2, one int8 scale per 16 weights
+            const uint8_t * a = aux + (row * (S / 8) + s / 8) * 32;
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(a + 16));
+            const float ds[2] = {__fmul_rn(d, float(int8_t(a[2 * ib]))), __fmul_rn(d, float(int8_t(a[2 * ib + 1])))};
+            const uint32_t * c = reinterpret_cast<const uint32_t *>(cd);
+            const uint32_t lo[2] = {c[0], c[1]}, hb = c[2];
+#pragma unroll
+            for (int j = 0; j < 32; ++j) {
+                const int q = int(((lo[j >> 4] >> (2 * (j & 15))) & 3u) | (((hb >> j) & 1u) << 2)) - 4;
+                y[j] = __fmul_rn(ds[j >> 4], float(q));
+            }
+            break;
+        }
+        case TQMOE_Q4_0: {  // dequant.cpp:480-491: (q - 8) * d
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(aux + (row * S + s) * 2));
+            const uint4 c = *reinterpret_cast<const uint4 *>(cd);
+            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const uint32_t byte = (w[q] >> (8 * b)) & 0xFFu;
+                    y[4 * q + b] = __fmul_rn(float(int(byte & 15u) - 8), d);
+                    y[16 + 4 * q + b] = __fmul_rn(float(int(byte >> 4) - 8), d);
+                }
+            break;
+        }
         case TQMOE_Q5_K: {  // dequant.cpp:102-116: (d * sc) * v - dmin * m, v = nibble + 16 * high bit
             const uint8_t * a = aux + (row * (S / 8) + s / 8) * 48;
             const uint4 rec = *reinterpret_cast<const uint4 *>(a);

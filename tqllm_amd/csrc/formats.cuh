@@ -5,15 +5,20 @@
 #include "iq3s_lattice.h"
 #include "iq3xxs_lattice.h"
 #include "iq2s_lattice.h"
+#include "iq2xxs_lattice.h"
+#include "iq2xs_lattice.h"
 
 namespace tqmoe {
 
 // code bytes per sub-block
-__host__ __device__ constexpr int code_bytes_per_sub(uint32_t type) { return type == TQMOE_IQ3_S || type == TQMOE_IQ3_XXS || type == TQMOE_IQ2_S ? 12 : type == TQMOE_Q8_0 ? 32 : type == TQMOE_Q6_K ? 24 : 16; }
-// aux record bytes per 256 weights (NVFP4G keeps bytes per 16 weights instead: see aux_row_bytes; IQ4_NL and Q8_0 hold
-// the eight fp16 scales of their 32-weight blocks)
-// Q5_K: the Q4_K header and the eight sub-blocks' high-bit words; Q6_K: sixteen int8 scales, d, padding
-__host__ __device__ constexpr int aux_record_bytes(uint32_t type) { return type == TQMOE_IQ4_XS ? 8 : type == TQMOE_Q5_K ? 48 : type == TQMOE_Q6_K ? 32 : 16; }
+__host__ __device__ constexpr int code_bytes_per_sub(uint32_t type) {
+    return type == TQMOE_IQ3_S || type == TQMOE_IQ3_XXS || type == TQMOE_IQ2_S || type == TQMOE_IQ2_XS || type == TQMOE_Q3_K ? 12
+         : type == TQMOE_IQ2_XXS ? 8 : type == TQMOE_Q8_0 ? 32 : type == TQMOE_Q6_K ? 24 : 16;
+}
+// aux record bytes per 256 weights (NVFP4G keeps bytes per 16 weights instead: see aux_row_bytes; IQ4_NL, Q4_0 and Q8_0
+// hold the eight fp16 scales of their 32-weight blocks)
+// Q5_K: the Q4_K header and the eight sub-blocks' high-bit words; Q6_K and Q3_K: sixteen int8 scales, d, padding
+__host__ __device__ constexpr int aux_record_bytes(uint32_t type) { return type == TQMOE_IQ4_XS ? 8 : type == TQMOE_Q5_K ? 48 : type == TQMOE_Q6_K || type == TQMOE_Q3_K ? 32 : 16; }
 __host__ __device__ constexpr int64_t code_row_bytes(uint32_t type, int cols) { return int64_t(cols / 32) * code_bytes_per_sub(type); }
 __host__ __device__ constexpr int64_t aux_row_bytes(uint32_t type, int cols) {
     return type == TQMOE_NVFP4G ? int64_t(cols / 16) : int64_t(cols / 256) * aux_record_bytes(type);
@@ -71,13 +76,12 @@ constexpr Iq3xxsGrid make_iq3xxs_grid() {
     return g;
 }
 __device__ const Iq3xxsGrid d_iq3xxs_grid = make_iq3xxs_grid();
-// IQ2_S lattice points: two dwords per point (magnitudes of weights 0..3, 4..7 of the group of eight)
-struct Iq2sGrid { uint32_t v[2048]; };
-constexpr Iq2sGrid make_iq2s_grid() {
-    constexpr uint16_t codes[1024] = {TQMOE_IQ2S_LATTICE16};
+// IQ2_S / IQ2_XS / IQ2_XXS lattice points: two dwords per point (magnitudes of weights 0..3, 4..7 of the group of eight)
+template <int N> struct Iq2Grid { uint32_t v[2 * N]; };
+template <int N> constexpr Iq2Grid<N> make_iq2_grid(const uint16_t (&codes)[N]) {
     constexpr uint32_t level[4] = {8, 25, 43, 0};
-    Iq2sGrid g{};
-    for (int i = 0; i < 1024; ++i)
+    Iq2Grid<N> g{};
+    for (int i = 0; i < N; ++i)
         for (int h = 0; h < 2; ++h) {
             uint32_t w = 0;
             for (int j = 0; j < 4; ++j) w |= level[(codes[i] >> (2 * (4 * h + j))) & 3u] << (8 * j);
@@ -85,15 +89,25 @@ constexpr Iq2sGrid make_iq2s_grid() {
         }
     return g;
 }
-__device__ const Iq2sGrid d_iq2s_grid = make_iq2s_grid();
+constexpr uint16_t kIq2sCodes[1024] = {TQMOE_IQ2S_LATTICE16};
+constexpr uint16_t kIq2xsCodes[512] = {TQMOE_IQ2XS_LATTICE16};
+constexpr uint16_t kIq2xxsCodes[256] = {TQMOE_IQ2XXS_LATTICE16};
+__device__ const Iq2Grid<1024> d_iq2s_grid = make_iq2_grid(kIq2sCodes);
+__device__ const Iq2Grid<512> d_iq2xs_grid = make_iq2_grid(kIq2xsCodes);
+__device__ const Iq2Grid<256> d_iq2xxs_grid = make_iq2_grid(kIq2xxsCodes);
+// dwords of a format's lattice as the kernels stage it in LDS (1: the format has none)
+__host__ __device__ constexpr int lattice_dwords(uint32_t type) {
+    return type == TQMOE_IQ3_S ? 512 : type == TQMOE_IQ3_XXS ? 256 : type == TQMOE_IQ2_S ? 2048 : type == TQMOE_IQ2_XS ? 1024 : type == TQMOE_IQ2_XXS ? 512 : 1;
+}
 // lattice index of group l of an IQ2_S sub-block: its low byte and two bits of the sub-block's qh byte
 __device__ __forceinline__ uint32_t iq2s_index(uint32_t low4, uint32_t qh, int l) { return ((low4 >> (8 * l)) & 0xFFu) | ((qh << (8 - 2 * l)) & 0x300u); }
 
 // the eight sign bits of a group of eight weights from its seven stored ones: the eighth makes their count even
-__device__ __forceinline__ uint32_t iq3xxs_signs(uint32_t word, int l) {
-    const uint32_t i7 = (word >> (7 * l)) & 127u;
-    return i7 | ((uint32_t(__popc(i7)) & 1u) << 7);
-}
+__device__ __forceinline__ uint32_t signs8(uint32_t i7) { return i7 | ((uint32_t(__popc(i7)) & 1u) << 7); }
+__device__ __forceinline__ uint32_t iq3xxs_signs(uint32_t word, int l) { return signs8((word >> (7 * l)) & 127u); }
+// the magnitudes g of four weights with the signs of four bits applied: negate the selected bytes, (g ^ m) + bits with m
+// the byte masks 0xFF of the set bits; no carry leaves a byte
+__device__ __forceinline__ uint32_t apply_signs4(uint32_t g, uint32_t bits4);
 
 // E4M3 byte -> float: (1 + m/8) 2^(e-7), subnormal m/8 2^-6, 0x7F / 0xFF NaN
 __device__ __forceinline__ float e4m3_to_float(uint32_t b) {
@@ -111,6 +125,12 @@ __device__ __forceinline__ uint32_t spread4(uint32_t bits) { return ((bits & 15u
 __device__ __forceinline__ uint32_t spread2x4(uint32_t x) { x &= 0xFFu; return (x | x << 6 | x << 12 | x << 18) & 0x03030303u; }
 // bytes q in [0, 63] -> int8 bytes q - 32
 __device__ __forceinline__ uint32_t minus32(uint32_t v) { return ((v | 0x80808080u) - 0x20202020u) ^ 0x80808080u; }
+// bytes q in [0, 127] -> int8 bytes q - K
+template <uint32_t K> __device__ __forceinline__ uint32_t minus_k(uint32_t v) { return ((v | 0x80808080u) - K * 0x01010101u) ^ 0x80808080u; }
+__device__ __forceinline__ uint32_t apply_signs4(uint32_t g, uint32_t bits4) {
+    const uint32_t bits = spread4(bits4), m = (bits << 8) - bits;
+    return (g ^ m) + bits;
+}
 
 // Q4_K: 6-bit (scale, min) of sub-block j from the 12-byte field held as three dwords
 __device__ __forceinline__ void q4k_scale_min(const uint32_t (&q)[3], int j, int & sc, int & mn) {

@@ -30,8 +30,8 @@ enum { TQMOE_OK = 0, TQMOE_E_ARG = -1, TQMOE_E_UNSUPPORTED = -2, TQMOE_E_DEVICE 
 /* element types (GGUF type ids, src/core/gguf.hpp) */
 enum { TQMOE_F32 = 0, TQMOE_F16 = 1, TQMOE_BF16 = 30 };
 /* bank formats (GGUF type ids) */
-enum { TQMOE_Q4_0 = 2, TQMOE_Q8_0 = 8, TQMOE_Q3_K = 11, TQMOE_Q4_K = 12, TQMOE_Q5_K = 13, TQMOE_Q6_K = 14, TQMOE_IQ2_XXS = 16, TQMOE_IQ2_XS = 17,
-       TQMOE_IQ3_XXS = 18, TQMOE_IQ4_NL = 20, TQMOE_IQ3_S = 21, TQMOE_IQ2_S = 22, TQMOE_IQ4_XS = 23, TQMOE_NVFP4G = 323 };
+enum { TQMOE_Q4_0 = 2, TQMOE_Q8_0 = 8, TQMOE_Q2_K = 10, TQMOE_Q3_K = 11, TQMOE_Q4_K = 12, TQMOE_Q5_K = 13, TQMOE_Q6_K = 14, TQMOE_IQ2_XXS = 16, TQMOE_IQ2_XS = 17,
+       TQMOE_IQ3_XXS = 18, TQMOE_IQ1_S = 19, TQMOE_IQ4_NL = 20, TQMOE_IQ3_S = 21, TQMOE_IQ2_S = 22, TQMOE_IQ4_XS = 23, TQMOE_NVFP4G = 323 };
 
 uint32_t tqmoe_abi_version(void);
 
@@ -116,6 +116,10 @@ int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets,
  *   Q3_K    codes 12 B: 8 B with the low two bits (byte k = weights 4 k .. 4 k + 3), then 4 B with the third bit (bit j =
  *           weight j; the weight is the three-bit value minus 4); aux 32 B per 256 weights: the sixteen 6-bit scales minus
  *           32 as int8 (two per sub-block), d (f16), padding.
+ *   Q2_K    codes 8 B: two bits per weight (byte k = weights 4 k .. 4 k + 3); aux 32 B per 256 weights: GGUF's sixteen
+ *           (scale | min << 4) bytes (two per sub-block), d, dmin (f16), padding.
+ *   IQ1_S   codes 8 B: 4 low lattice index bytes, then GGUF's 16-bit qh of the sub-block (4 x 3 upper index bits, the 3-bit
+ *           scale, the sign of the shift), 2 B padding; aux as IQ3_XXS.
  *   IQ4_NL  codes 16 B, GGUF's own nibble order; aux 2 B per sub-block: its d (f16).
  *   Q4_0    as IQ4_NL (the weight is the nibble minus 8).
  *   Q8_0    codes 32 B: the int8 values; aux 2 B per sub-block: its d (f16).

@@ -15,8 +15,9 @@ REF_PATH = os.path.join(HERE, "_ref", "libtqref.so")
 F32, F16, Q4_K, IQ4_NL, IQ3_S, IQ4_XS, BF16, NVFP4G = 0, 1, 12, 20, 21, 23, 30, 323
 Q8_0, Q5_K, Q6_K, IQ3_XXS, IQ2_S = 8, 13, 14, 18, 22
 Q4_0, Q3_K, IQ2_XXS, IQ2_XS = 2, 11, 16, 17
+Q2_K, IQ1_S = 10, 19
 GATE_SOFTMAX, GATE_SIGMOID, GATE_SOFTMAX_WEIGHT, GATE_SQRT_SOFTPLUS = 1, 2, 3, 4
-BLOCK = {Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), IQ3_XXS: (256, 98), IQ2_S: (256, 82), Q4_0: (32, 18), Q3_K: (256, 110), IQ2_XXS: (256, 66), IQ2_XS: (256, 74), Q8_0: (32, 34), IQ4_NL: (32, 18), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76)}
+BLOCK = {Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), IQ3_XXS: (256, 98), IQ2_S: (256, 82), Q4_0: (32, 18), Q3_K: (256, 110), IQ2_XXS: (256, 66), IQ2_XS: (256, 74), Q2_K: (256, 84), IQ1_S: (256, 50), Q8_0: (32, 34), IQ4_NL: (32, 18), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76)}
 
 
 def build(ref=True):

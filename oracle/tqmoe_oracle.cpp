@@ -6,6 +6,7 @@
 #include "iq2s_lattice.h"
 #include "iq2xxs_lattice.h"
 #include "iq2xs_lattice.h"
+#include "iq1s_lattice.h"
 
 #include <algorithm>
 #include <atomic>
@@ -117,6 +118,8 @@ int tqo_block_layout(uint32_t type, int * elems, int * bytes) {
         case TQO_IQ2_XS: e = 256; b = 74; break;
         case TQO_Q3_K: e = 256; b = 110; break;
         case TQO_Q4_0: e = 32; b = 18; break;
+        case TQO_Q2_K: e = 256; b = 84; break;
+        case TQO_IQ1_S: e = 256; b = 50; break;
         case TQO_IQ4_XS: e = 256; b = 136; break;
         case TQO_NVFP4G: e = 128; b = 76; break;
         default: return 0;
@@ -285,6 +288,28 @@ void decode_q3k(const uint8_t * b, float * y) {  // src/formats/weight/dequant.c
     }
 }
 
+void decode_q2k(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:289-310: (d * scale) * q - dmin * min per 16 weights
+    const float d = tqo_half_to_float(rd16(b + 80)), dmin = tqo_half_to_float(rd16(b + 82));
+    for (int e = 0; e < 256; ++e) {
+        const int n = e / 128, j = (e % 128) / 32, w = e % 32;
+        const uint8_t sc = b[8 * n + 2 * j + (w >= 16)];
+        const float dl = d * float(sc & 15), ml = dmin * float(sc >> 4);
+        y[e] = dl * float((b[16 + 32 * n + w] >> (2 * j)) & 3) - ml;
+    }
+}
+
+void decode_iq1s(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:311-326: (d * (2 s + 1)) * (value + delta)
+    const float d = tqo_half_to_float(rd16(b));
+    for (int ib = 0; ib < 8; ++ib) {
+        const uint32_t qh = rd16(b + 34 + 2 * ib);
+        const float dl = d * float(2 * ((qh >> 12) & 7) + 1), delta = (qh & 0x8000u) ? -0.125f : 0.125f;
+        for (int l = 0; l < 4; ++l) {
+            const uint64_t g = tq_iq1s_point(b[2 + 4 * ib + l] | (((qh >> (3 * l)) & 7u) << 8));
+            for (int j = 0; j < 8; ++j) y[32 * ib + 8 * l + j] = dl * (float(int8_t((g >> (8 * j)) & 0xFFu)) + delta);
+        }
+    }
+}
+
 void decode_q4_0(const uint8_t * b, float * y) {  // src/formats/weight/dequant.cpp:480-491: (q - 8) * d
     const float d = tqo_half_to_float(rd16(b));
     for (int j = 0; j < 16; ++j) {
@@ -347,6 +372,8 @@ int tqo_dequantize(uint32_t type, const void * src, float * dst, int64_t n) {
         case TQO_IQ2_XS: decode_iq2xs(s, dst); break;
         case TQO_Q3_K: decode_q3k(s, dst); break;
         case TQO_Q4_0: decode_q4_0(s, dst); break;
+        case TQO_Q2_K: decode_q2k(s, dst); break;
+        case TQO_IQ1_S: decode_iq1s(s, dst); break;
         case TQO_NVFP4G: decode_nvfp4g(s, dst); break;
     }
     return 0;

@@ -17,6 +17,8 @@
  *                   IQ2_XXS, IQ2_XS        src/formats/weight/dequant.cpp:233-249, 252-268 (likewise)
  *                   Q3_K                   src/formats/weight/dequant.cpp:66-76, 118-131 (likewise)
  *                   Q4_0                   src/formats/weight/dequant.cpp:480-491 (likewise)
+ *                   Q2_K                   src/formats/weight/dequant.cpp:289-310 (likewise)
+ *                   IQ1_S                  src/formats/weight/dequant.cpp:311-326 (likewise)
  *                   Q6_K                   src/formats/weight/dequant.cpp:194-208
  *                   NVFP4G                 src/formats/weight/dequant.cpp:397-409
  *   tqo_route                              src/experts/moe.cpp:22-113 (softmax / sigmoid / softmax-of-selected /
@@ -58,7 +60,7 @@ extern "C" {
 #endif
 
 /* GGUF tensor type ids (src/core/gguf.hpp) */
-enum { TQO_F32 = 0, TQO_F16 = 1, TQO_Q4_0 = 2, TQO_Q8_0 = 8, TQO_Q3_K = 11, TQO_Q4_K = 12, TQO_Q5_K = 13, TQO_Q6_K = 14, TQO_IQ2_XXS = 16, TQO_IQ2_XS = 17, TQO_IQ3_XXS = 18, TQO_IQ2_S = 22, TQO_IQ4_NL = 20, TQO_IQ3_S = 21, TQO_IQ4_XS = 23, TQO_BF16 = 30,
+enum { TQO_F32 = 0, TQO_F16 = 1, TQO_Q4_0 = 2, TQO_Q8_0 = 8, TQO_Q2_K = 10, TQO_Q3_K = 11, TQO_Q4_K = 12, TQO_Q5_K = 13, TQO_Q6_K = 14, TQO_IQ2_XXS = 16, TQO_IQ2_XS = 17, TQO_IQ3_XXS = 18, TQO_IQ1_S = 19, TQO_IQ2_S = 22, TQO_IQ4_NL = 20, TQO_IQ3_S = 21, TQO_IQ4_XS = 23, TQO_BF16 = 30,
        TQO_NVFP4G = 323 };
 /* gating (src/experts/moe.hpp:20-26) */
 enum { TQO_GATE_SOFTMAX = 1, TQO_GATE_SIGMOID = 2, TQO_GATE_SOFTMAX_WEIGHT = 3, TQO_GATE_SQRT_SOFTPLUS = 4 };

@@ -14,10 +14,11 @@ CONFIGS = {
 
 
 # formats the oracle has no encoder for: offset of the fp16 block scale and the range it is drawn from (weights of about 0.02)
-RANDOM_BLOCKS = {oracle.IQ3_XXS: (0, 1.5e-4, 4e-4), oracle.IQ2_S: (0, 4e-4, 1e-3), oracle.Q4_0: (0, 2e-3, 6e-3), oracle.Q3_K: (108, 3e-4, 7e-4),
-                 oracle.IQ2_XXS: (0, 2e-4, 5e-4), oracle.IQ2_XS: (0, 2e-4, 5e-4)}
+RANDOM_BLOCKS = {oracle.IQ3_XXS: [(0, 1.5e-4, 4e-4)], oracle.IQ2_S: [(0, 4e-4, 1e-3)], oracle.Q4_0: [(0, 2e-3, 6e-3)], oracle.Q3_K: [(108, 3e-4, 7e-4)],
+                 oracle.IQ2_XXS: [(0, 2e-4, 5e-4)], oracle.IQ2_XS: [(0, 2e-4, 5e-4)], oracle.Q2_K: [(80, 1e-3, 3e-3), (82, 1.5e-3, 4.5e-3)],
+                 oracle.IQ1_S: [(0, 2e-3, 4e-3)]}
 # byte offset of the fp16 block scale where it is not the block's first field
-SCALE_OFFSET = {oracle.Q6_K: 208, oracle.Q3_K: 108}
+SCALE_OFFSET = {oracle.Q6_K: 208, oracle.Q3_K: 108, oracle.Q2_K: 80}
 
 
 def bank_blocks(wtype, rows, cols, rng, sigma=0.02):
@@ -26,9 +27,9 @@ def bank_blocks(wtype, rows, cols, rng, sigma=0.02):
     if wtype in RANDOM_BLOCKS:
         el, nbytes = oracle.BLOCK[wtype]
         blocks = rng.integers(0, 256, (rows * cols // el, nbytes), dtype=np.uint8)
-        off, lo, hi = RANDOM_BLOCKS[wtype]
-        dd = np.float16(rng.uniform(lo, hi, len(blocks)) * (sigma / 0.02) * rng.choice([-1, 1], len(blocks)))
-        blocks[:, off:off + 2] = dd.view(np.uint8).reshape(-1, 2)
+        for off, lo, hi in RANDOM_BLOCKS[wtype]:
+            dd = np.float16(rng.uniform(lo, hi, len(blocks)) * (sigma / 0.02) * rng.choice([-1, 1], len(blocks)))
+            blocks[:, off:off + 2] = dd.view(np.uint8).reshape(-1, 2)
         return blocks.reshape(-1)
     return oracle.quantize(wtype, (rng.standard_normal((rows, cols)) * sigma).astype(np.float32))
 
@@ -52,9 +53,9 @@ def _scale_field(raw, wtype, per_expert_blocks, factors):
         o = SCALE_OFFSET.get(wtype, 0)
         d = blocks[:, :, o:o + 2].copy().view(np.float16).astype(np.float32)
         blocks[:, :, o:o + 2] = (d * factors[:, None, None]).astype(np.float16).view(np.uint8)
-        if wtype == oracle.Q4_K:
-            m = blocks[:, :, 2:4].copy().view(np.float16).astype(np.float32)
-            blocks[:, :, 2:4] = (m * factors[:, None, None]).astype(np.float16).view(np.uint8)
+        if wtype in (oracle.Q4_K, oracle.Q5_K, oracle.Q2_K):       # the minimums' scale follows the block scale
+            m = blocks[:, :, o + 2:o + 4].copy().view(np.float16).astype(np.float32)
+            blocks[:, :, o + 2:o + 4] = (m * factors[:, None, None]).astype(np.float16).view(np.uint8)
     return blocks.reshape(-1)
 
 

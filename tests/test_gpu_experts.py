@@ -19,7 +19,7 @@ def tq():
     return tqllm_amd
 
 
-@pytest.mark.parametrize("wtype", [12, 21, 23, 323, 20, 8, 13, 14, 18, 22, 2, 11, 16, 17])
+@pytest.mark.parametrize("wtype", [12, 21, 23, 323, 20, 8, 13, 14, 18, 22, 2, 11, 16, 17, 10, 19])
 def test_bank_decode_bit_exact(tq, oracle, wtype):
     rng = np.random.default_rng(wtype)
     experts, rows, cols = 3, (64 if wtype == 23 else 40), 1024      # IQ4_XS banks are tiled by 32 rows
@@ -27,7 +27,7 @@ def test_bank_decode_bit_exact(tq, oracle, wtype):
     nb = experts * rows * cols // el
     # random block bytes with sane scale fields, as the reference's device tests make them (tests/moe_device.cu:121-138)
     raw = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
-    for off in {12: [0, 2], 21: [0], 23: [0], 20: [0], 8: [0], 13: [0, 2], 14: [208], 18: [0], 22: [0], 2: [0], 11: [108], 16: [0], 17: [0]}.get(wtype, []):
+    for off in {12: [0, 2], 21: [0], 23: [0], 20: [0], 8: [0], 13: [0, 2], 14: [208], 18: [0], 22: [0], 2: [0], 11: [108], 16: [0], 17: [0], 10: [80, 82], 19: [0]}.get(wtype, []):
         raw[:, off:off + 2] = np.float16(rng.uniform(1e-3, 5e-2, nb) * rng.choice([-1, 1], nb)).view(np.uint8).reshape(nb, 2)
     if wtype == 323:
         g = rng.uniform(1e-3, 2e-2, experts * rows).astype(np.float32)
@@ -149,7 +149,7 @@ def test_layer_small_shapes(tq, oracle, name, n):
     check_layer(*run_layer(tq, oracle, cfg, n, seed=50 + n))
 
 
-@pytest.mark.parametrize("wtype", [20, 8, 13, 14, 18, 22, 2, 11, 16, 17])
+@pytest.mark.parametrize("wtype", [20, 8, 13, 14, 18, 22, 2, 11, 16, 17, 10, 19])
 @pytest.mark.parametrize("n", [1, 5, 300])
 def test_layer_further_bank_formats(tq, oracle, wtype, n):
     """IQ4_NL (the CPU bench's format), Q8_0, Q5_K, Q6_K, IQ3_XXS and IQ2_S through the same decode kernels and grouped

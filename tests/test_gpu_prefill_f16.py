@@ -19,7 +19,7 @@ def tq():
     return tqllm_amd
 
 
-@pytest.mark.parametrize("wtype", [12, 21, 23, 323, 20, 8, 13, 14, 11, 17])
+@pytest.mark.parametrize("wtype", [12, 21, 23, 323, 20, 8, 13, 14, 11, 17, 10, 19])
 @pytest.mark.parametrize("n,shared_ff", [(70, 0), (200, 128)])
 def test_grouped_f16_products_against_float64(tq, oracle, wtype, n, shared_ff):
     rng = np.random.default_rng(wtype + n)

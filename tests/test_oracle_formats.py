@@ -286,6 +286,45 @@ def test_q3k_closed_form(oracle):
     assert q.min() == -4 and q.max() == 3
 
 
+def test_q2k_closed_form(oracle):
+    """Q2_K (dequant.cpp:289-310): weight 128 n + 32 j + w takes two bits of qs[32 n + w] at 2 j; byte 8 n + 2 j + (w >= 16) of
+    the sixteen holds its scale (low nibble) and minimum (high): (d scale) q - dmin minimum."""
+    rng = np.random.default_rng(4)
+    sc = rng.integers(0, 256, 16, dtype=np.uint8)
+    qs = rng.integers(0, 256, 64, dtype=np.uint8)
+    b = np.concatenate([sc, qs, np.array([np.float16(0.25), np.float16(0.5)]).view(np.uint8)])
+    got = oracle.dequantize(oracle.Q2_K, b, 256)
+    e = np.arange(256)
+    n, j, w = e // 128, (e % 128) // 32, e % 32
+    s = sc[8 * n + 2 * j + (w >= 16)]
+    q = (qs[32 * n + w] >> (2 * j)) & 3
+    want = (np.float32(0.25) * (s & 15).astype(np.float32)) * q.astype(np.float32) - np.float32(0.5) * (s >> 4).astype(np.float32)
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+def test_iq1s_closed_form(oracle):
+    """IQ1_S (dequant.cpp:311-326): values -1, 0, 1 shifted by +-1/8 (bit 15 of the sub-block's qh: minus), times d (2 s + 1)
+    with s in bits 12..14; the lattice index is the qs byte plus three bits of qh per group of eight weights."""
+    blk = np.zeros(50, np.uint8)
+    blk[0:2] = np.array([np.float16(1.0)]).view(np.uint8)
+    qh = np.zeros(8, np.uint16)
+    qh[1] = (5 << 12) | 0x8000
+    pts = set()
+    for hi in range(8):
+        qh[0] = hi | hi << 3 | hi << 6 | hi << 9
+        blk[34:50] = qh.view(np.uint8)
+        for base in range(0, 256, 4):
+            blk[2:6] = np.arange(base, base + 4, dtype=np.uint8)
+            v = oracle.dequantize(oracle.IQ1_S, blk, 256)
+            assert set(np.unique(v[:32]).tolist()) <= {-0.875, 0.125, 1.125}
+            pts |= {tuple(r) for r in v[:32].reshape(4, 8).tolist()}
+    assert len(pts) == 2048
+    first = oracle.dequantize(oracle.IQ1_S, blk, 256)
+    g0 = first[64:72] - np.float32(0.125)                     # lattice point 0 (sub-block 2: index 0, scale 1, plus shift)
+    assert set(np.unique(g0).tolist()) <= {-1.0, 0.0, 1.0}
+    assert np.array_equal(first[32:40], np.float32(11.0) * (g0 - np.float32(0.125)))
+
+
 @pytest.mark.parametrize("wtype,points", [(16, 256), (17, 512)])
 def test_iq2xxs_iq2xs_closed_form(oracle, wtype, points):
     """IQ2_XXS (dequant.cpp:233-249) and IQ2_XS (252-268): lattice index 0 is the point of eight 8s; d (0.5 + s) / 4 with s
@@ -330,13 +369,13 @@ def test_iq2xxs_iq2xs_closed_form(oracle, wtype, points):
     assert len(pts) == points
 
 
-@pytest.mark.parametrize("wtype", [2, 8, 11, 12, 13, 14, 16, 17, 18, 20, 21, 22, 23, 323])
+@pytest.mark.parametrize("wtype", [2, 8, 10, 11, 12, 13, 14, 16, 17, 18, 19, 20, 21, 22, 23, 323])
 def test_decoders_match_reference_objects(oracle, ref, wtype):
     rng = np.random.default_rng(wtype)
     el, bb = oracle.BLOCK[wtype]
     nb = 64
     raw = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
-    halves = {2: [0], 11: [108], 16: [0], 17: [0], 8: [0], 12: [0, 2], 13: [0, 2], 14: [208], 18: [0], 20: [0], 21: [0], 22: [0], 23: [0]}.get(wtype, [])
+    halves = {2: [0], 10: [80, 82], 19: [0], 11: [108], 16: [0], 17: [0], 8: [0], 12: [0, 2], 13: [0, 2], 14: [208], 18: [0], 20: [0], 21: [0], 22: [0], 23: [0]}.get(wtype, [])
     for off in halves:
         raw[:, off:off + 2] = np.float16(rng.uniform(1e-3, 5e-2, nb) * rng.choice([-1, 1], nb)).view(np.uint8).reshape(nb, 2)
     if wtype == 323:

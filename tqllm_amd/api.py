@@ -19,8 +19,9 @@ F32, F16, BF16 = 0, 1, 30
 Q4_K, IQ3_S, IQ4_XS, NVFP4G = 12, 21, 23, 323
 Q8_0, IQ4_NL, Q5_K, Q6_K, IQ3_XXS, IQ2_S = 8, 20, 13, 14, 18, 22
 Q4_0, Q3_K, IQ2_XXS, IQ2_XS = 2, 11, 16, 17
+Q2_K, IQ1_S = 10, 19
 GATE_SOFTMAX, GATE_SIGMOID, GATE_SOFTMAX_WEIGHT, GATE_SQRT_SOFTPLUS = 1, 2, 3, 4   # MoeGating, src/experts/moe.hpp:20-26
-BLOCK = {Q4_K: (256, 144), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76), IQ4_NL: (32, 18), Q8_0: (32, 34), Q5_K: (256, 176), Q6_K: (256, 210), IQ3_XXS: (256, 98), IQ2_S: (256, 82), Q4_0: (32, 18), Q3_K: (256, 110), IQ2_XXS: (256, 66), IQ2_XS: (256, 74)}
+BLOCK = {Q4_K: (256, 144), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76), IQ4_NL: (32, 18), Q8_0: (32, 34), Q5_K: (256, 176), Q6_K: (256, 210), IQ3_XXS: (256, 98), IQ2_S: (256, 82), Q4_0: (32, 18), Q3_K: (256, 110), IQ2_XXS: (256, 66), IQ2_XS: (256, 74), Q2_K: (256, 84), IQ1_S: (256, 50)}
 _TORCH_TYPE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 _OUT_TYPE = {F32: torch.float32, BF16: torch.bfloat16}
 

@@ -129,6 +129,28 @@ __global__ __launch_bounds__(256) void load_k(uint32_t type, const uint8_t * __r
             }
             break;
         }
+        case TQMOE_Q2_K: {  // 84 B per 256: scales[16] (scale | min << 4), qs[64], d, dmin; sub-block i = 4 n + j holds weights 128 n + 32 j ..
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 84;
+            const int ib = s & 7, n = ib >> 2, j = ib & 3;
+            const uint8_t * qs = blk + 16 + 32 * n;
+            uint32_t lo[2] = {0, 0};   // two bits per weight, byte k = weights 4 k .. 4 k + 3
+#pragma unroll
+            for (int l = 0; l < 32; ++l) lo[l >> 4] |= uint32_t((qs[l] >> (2 * j)) & 3) << (2 * (l & 15));
+            *reinterpret_cast<uint2 *>(cd) = make_uint2(lo[0], lo[1]);
+            if (ib == 0) {
+                uint8_t * a = aux + (row * (S / 8) + s / 8) * 32;
+                *reinterpret_cast<uint4 *>(a) = make_uint4(rd_u32(blk), rd_u32(blk + 4), rd_u32(blk + 8), rd_u32(blk + 12));
+                *reinterpret_cast<uint4 *>(a + 16) = make_uint4(rd_u32(blk + 80), 0, 0, 0);
+            }
+            break;
+        }
+        case TQMOE_IQ1_S: {  // 50 B per 256: d, qs[32] (low index bytes), qh[8] (4 x 3 index bits, 3-bit scale, delta sign)
+            const uint8_t * blk = src + (row * (S / 8) + s / 8) * 50;
+            const int ib = s & 7;
+            *reinterpret_cast<uint2 *>(cd) = make_uint2(rd_u32(blk + 2 + 4 * ib), rd_u16(blk + 34 + 2 * ib));
+            if (ib == 0) *reinterpret_cast<uint4 *>(aux + (row * (S / 8) + s / 8) * 16) = make_uint4(rd_u16(blk), 0, 0, 0);
+            break;
+        }
         case TQMOE_Q4_0: {  // 18 B per 32: d, qs[16] (byte j = weight j | weight j + 16 << 4: the canonical order)
             const uint8_t * blk = src + (row * S + s) * 18;
             pack_sub(cd, [&](int j) { return j < 16 ? blk[2 + j] & 15 : blk[2 + j - 16] >> 4; });

@@ -46,7 +46,7 @@ inline int32_t need_device(tqmoe_error * err, const char * what) {
     return 0;
 }
 inline bool is_act_type(uint32_t t) { return t == TQMOE_F32 || t == TQMOE_F16 || t == TQMOE_BF16; }
-inline bool is_bank_type(uint32_t t) { return t == TQMOE_Q4_0 || t == TQMOE_Q3_K || t == TQMOE_IQ2_XXS || t == TQMOE_IQ2_XS || t == TQMOE_Q4_K || t == TQMOE_IQ3_S || t == TQMOE_IQ4_XS || t == TQMOE_NVFP4G || t == TQMOE_IQ4_NL || t == TQMOE_Q8_0 ||
+inline bool is_bank_type(uint32_t t) { return t == TQMOE_Q2_K || t == TQMOE_IQ1_S || t == TQMOE_Q4_0 || t == TQMOE_Q3_K || t == TQMOE_IQ2_XXS || t == TQMOE_IQ2_XS || t == TQMOE_Q4_K || t == TQMOE_IQ3_S || t == TQMOE_IQ4_XS || t == TQMOE_NVFP4G || t == TQMOE_IQ4_NL || t == TQMOE_Q8_0 ||
            t == TQMOE_Q5_K || t == TQMOE_Q6_K || t == TQMOE_IQ3_XXS || t == TQMOE_IQ2_S;
 }
 inline size_t elem_bytes(uint32_t t) { return t == TQMOE_F32 ? 4 : 2; }

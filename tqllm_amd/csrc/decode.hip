@@ -82,6 +82,8 @@ void dispatch_matvec(uint32_t type, Split sp, int nb, const MatvecArgs & k, hipS
         case TQMOE_Q6_K: DecodeLaunch<TQMOE_Q6_K>::matvec(sp, nb, k, s); break;
         case TQMOE_IQ3_XXS: DecodeLaunch<TQMOE_IQ3_XXS>::matvec(sp, nb, k, s); break;
         case TQMOE_IQ2_S: DecodeLaunch<TQMOE_IQ2_S>::matvec(sp, nb, k, s); break;
+        case TQMOE_Q2_K: DecodeLaunch<TQMOE_Q2_K>::matvec(sp, nb, k, s); break;
+        case TQMOE_IQ1_S: DecodeLaunch<TQMOE_IQ1_S>::matvec(sp, nb, k, s); break;
         case TQMOE_Q4_0: DecodeLaunch<TQMOE_Q4_0>::matvec(sp, nb, k, s); break;
         case TQMOE_Q3_K: DecodeLaunch<TQMOE_Q3_K>::matvec(sp, nb, k, s); break;
         case TQMOE_IQ2_XXS: DecodeLaunch<TQMOE_IQ2_XXS>::matvec(sp, nb, k, s); break;
@@ -100,6 +102,8 @@ void dispatch_gateup(uint32_t type, Split sp, const GateupArgs & k, hipStream_t 
         case TQMOE_Q6_K: DecodeLaunch<TQMOE_Q6_K>::gateup(sp, k, s); break;
         case TQMOE_IQ3_XXS: DecodeLaunch<TQMOE_IQ3_XXS>::gateup(sp, k, s); break;
         case TQMOE_IQ2_S: DecodeLaunch<TQMOE_IQ2_S>::gateup(sp, k, s); break;
+        case TQMOE_Q2_K: DecodeLaunch<TQMOE_Q2_K>::gateup(sp, k, s); break;
+        case TQMOE_IQ1_S: DecodeLaunch<TQMOE_IQ1_S>::gateup(sp, k, s); break;
         case TQMOE_Q4_0: DecodeLaunch<TQMOE_Q4_0>::gateup(sp, k, s); break;
         case TQMOE_Q3_K: DecodeLaunch<TQMOE_Q3_K>::gateup(sp, k, s); break;
         case TQMOE_IQ2_XXS: DecodeLaunch<TQMOE_IQ2_XXS>::gateup(sp, k, s); break;

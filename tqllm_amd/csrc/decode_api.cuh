@@ -50,6 +50,8 @@ extern template struct DecodeLaunch<TQMOE_Q5_K>;
 extern template struct DecodeLaunch<TQMOE_Q6_K>;
 extern template struct DecodeLaunch<TQMOE_IQ3_XXS>;
 extern template struct DecodeLaunch<TQMOE_IQ2_S>;
+extern template struct DecodeLaunch<TQMOE_Q2_K>;
+extern template struct DecodeLaunch<TQMOE_IQ1_S>;
 extern template struct DecodeLaunch<TQMOE_Q4_0>;
 extern template struct DecodeLaunch<TQMOE_Q3_K>;
 extern template struct DecodeLaunch<TQMOE_IQ2_XXS>;

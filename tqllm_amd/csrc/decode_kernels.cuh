@@ -26,8 +26,9 @@ namespace {
 // of the activation planes (Dec), and multiplied with any number of activation blocks.
 struct Dec {
     uint32_t w[8];   // int8 x 4 each; w[q] = values 4q .. 4q + 3 of the sub-block
-    float s0, s1;    // scale of dwords 0..3 and of dwords 4..7 (equal except for NVFP4G's two 16-weight groups)
-    float mn;        // coefficient of the block's activation sum (Q4_K minimum), else 0
+    float s0, s1;    // scale of dwords 0..3 and of dwords 4..7 (equal unless the format scales 16-weight groups)
+    float mn;        // coefficient of the block's activation sum (a K-quant minimum), else 0; with half minimums (Q2_K): of
+    float mn1;       // the first 16 weights' sum, and mn1 of the other 16's
 };
 
 // w: natural dwords d0 .. d0 + 3 of a sub-block's values; x: a plane indexed by plane position
@@ -37,8 +38,18 @@ template <int D0> __device__ __forceinline__ int dot4x(const uint32_t * w, const
     for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_sdot4(int(w[q]), x[plane_pos(D0 + q)], acc, false);
     return acc;
 }
-template <bool SPLIT> __device__ __forceinline__ float dot_block(const Dec & d, const ActBlock & x) {
-    if constexpr (SPLIT) {
+// a format whose traits declare kHalfMins has a minimum per 16 weights
+template <class F, class = void> struct HalfMins { static constexpr bool value = false; };
+template <class F> struct HalfMins<F, decltype(void(F::kHalfMins))> { static constexpr bool value = true; };
+
+template <bool SPLIT, bool HALF_MINS = false> __device__ __forceinline__ float dot_block(const Dec & d, const ActBlock & x) {
+    if constexpr (HALF_MINS) {
+        const int t0 = (dot4x<0>(d.w, x.hi) << 7) + dot4x<0>(d.w, x.lo);
+        const int t1 = (dot4x<4>(d.w + 4, x.hi) << 7) + dot4x<4>(d.w + 4, x.lo);
+        const uint32_t ones[4] = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};
+        const float u0 = float((dot4x<0>(ones, x.hi) << 7) + dot4x<0>(ones, x.lo)) * x.scale;   // the first half's activation sum
+        return (float(t0) * d.s0 + float(t1) * d.s1) * x.scale - d.mn * u0 - d.mn1 * (x.sum - u0);
+    } else if constexpr (SPLIT) {
         const int t0 = (dot4x<0>(d.w, x.hi) << 7) + dot4x<0>(d.w, x.lo);
         const int t1 = (dot4x<4>(d.w + 4, x.hi) << 7) + dot4x<4>(d.w + 4, x.lo);
         return (float(t0) * d.s0 + float(t1) * d.s1) * x.scale;
@@ -208,6 +219,55 @@ template <> struct Sub<TQMOE_Q3_K> {
         d.s0 = dd * float(int8_t(r.sc & 0xFFu));
         d.s1 = dd * float(int8_t(r.sc >> 8));
         d.mn = 0.f;
+    }
+};
+
+template <> struct Sub<TQMOE_Q2_K> {
+    static constexpr bool kSplit = true;      // one scale and one minimum per 16 weights: the sub-block's halves
+    static constexpr bool kHalfMins = true;
+    struct Raw { uint2 c; uint32_t sc; uint32_t dm; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        v.c = *reinterpret_cast<const uint2 *>(t.codes + (r * S + s) * 8u);
+        const uint8_t * a = t.aux + (r * (S >> 3) + (s >> 3)) * 32u;
+        v.sc = *reinterpret_cast<const uint16_t *>(a + 2u * (s & 7u));
+        v.dm = *reinterpret_cast<const uint32_t *>(a + 16u);
+        return v;
+    }
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t *, Dec & d) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            d.w[q] = spread2x4(r.c.x >> (8 * q));
+            d.w[4 + q] = spread2x4(r.c.y >> (8 * q));
+        }
+        const float dd = half_bits_to_float(uint16_t(r.dm & 0xFFFFu)), dmin = half_bits_to_float(uint16_t(r.dm >> 16));
+        d.s0 = dd * float(r.sc & 15u);
+        d.s1 = dd * float((r.sc >> 8) & 15u);
+        d.mn = dmin * float((r.sc >> 4) & 15u);
+        d.mn1 = dmin * float((r.sc >> 12) & 15u);
+    }
+};
+
+template <> struct Sub<TQMOE_IQ1_S> {
+    static constexpr bool kSplit = false;
+    struct Raw { uint2 c; uint32_t d; };
+    static __device__ __forceinline__ Raw load(const Tile & t, uint32_t r, uint32_t S, uint32_t s) {
+        Raw v;
+        v.c = *reinterpret_cast<const uint2 *>(t.codes + (r * S + s) * 8u);
+        v.d = *reinterpret_cast<const uint16_t *>(t.aux + (r * (S >> 3) + (s >> 3)) * 16u);
+        return v;
+    }
+    // grid: the 2048-point lattice in LDS, two dwords per point of int8 values; value + delta is split into the integer
+    // product and delta times the block's activation sum
+    static __device__ __forceinline__ void decode(const Raw & r, int, const uint32_t * grid, Dec & d) {
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const uint2 g = *reinterpret_cast<const uint2 *>(grid + 2u * (((r.c.x >> (8 * l)) & 0xFFu) | (((r.c.y >> (3 * l)) & 7u) << 8)));
+            d.w[2 * l] = g.x;
+            d.w[2 * l + 1] = g.y;
+        }
+        d.s0 = d.s1 = half_bits_to_float(uint16_t(r.d)) * float(2 * int((r.c.y >> 12) & 7u) + 1);
+        d.mn = (r.c.y & 0x8000u) ? 0.125f * d.s0 : -0.125f * d.s0;
     }
 };
 
@@ -382,6 +442,7 @@ template <uint32_t FMT> __device__ __forceinline__ const uint32_t * stage_grid(u
     else if constexpr (FMT == TQMOE_IQ2_S) src = d_iq2s_grid.v;
     else if constexpr (FMT == TQMOE_IQ2_XS) src = d_iq2xs_grid.v;
     else if constexpr (FMT == TQMOE_IQ2_XXS) src = d_iq2xxs_grid.v;
+    else if constexpr (FMT == TQMOE_IQ1_S) src = d_iq1s_grid.v;
     if constexpr (lattice_dwords(FMT) > 1) {
         for (int i = threadIdx.x; i < lattice_dwords(FMT); i += blockDim.x) lds[i] = src[i];
         __syncthreads();
@@ -457,7 +518,7 @@ __device__ __forceinline__ void block_rows(const Tile (&tile)[NB], int S, int ro
                     Dec d;
                     F::decode(raw[u][nb][m], min(sl + LPR * m, S - 1), grid, d);
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) acc[nt] += dot_block<F::kSplit>(d, x[nt][m]);   // blocks past the row's end are zero
+                    for (int nt = 0; nt < NT; ++nt) acc[nt] += dot_block<F::kSplit, HalfMins<F>::value>(d, x[nt][m]);   // blocks past the row's end are zero
                 }
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {

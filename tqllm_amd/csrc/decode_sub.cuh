@@ -144,6 +144,31 @@ __device__ __forceinline__ void decode_sub32(uint32_t type, const uint8_t * __re
             }
             break;
         }
+        case TQMOE_Q2_K: {  // dequant.cpp:289-310: (d * scale) * q - dmin * min, a (scale, min) byte per 16 weights
+            const uint8_t * a = aux + (row * (S / 8) + s / 8) * 32;
+            const uint32_t dm = *reinterpret_cast<const uint32_t *>(a + 16);
+            const float d = half_bits_to_float(uint16_t(dm & 0xFFFFu)), dmin = half_bits_to_float(uint16_t(dm >> 16));
+            const float dl[2] = {__fmul_rn(d, float(a[2 * ib] & 15)), __fmul_rn(d, float(a[2 * ib + 1] & 15))};
+            const float ml[2] = {__fmul_rn(dmin, float(a[2 * ib] >> 4)), __fmul_rn(dmin, float(a[2 * ib + 1] >> 4))};
+            const uint2 c = *reinterpret_cast<const uint2 *>(cd);
+            const uint32_t lo[2] = {c.x, c.y};
+#pragma unroll
+            for (int j = 0; j < 32; ++j) y[j] = __fsub_rn(__fmul_rn(dl[j >> 4], float((lo[j >> 4] >> (2 * (j & 15))) & 3u)), ml[j >> 4]);
+            break;
+        }
+        case TQMOE_IQ1_S: {  // dequant.cpp:311-326: (d * (2 s + 1)) * (value + delta)
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(aux + (row * (S / 8) + s / 8) * 16));
+            const uint2 c = *reinterpret_cast<const uint2 *>(cd);
+            const float dl = __fmul_rn(d, float(2 * int((c.y >> 12) & 7u) + 1)), delta = (c.y & 0x8000u) ? -0.125f : 0.125f;
+#pragma unroll
+            for (int l = 0; l < 4; ++l) {
+                const uint32_t idx = ((c.x >> (8 * l)) & 0xFFu) | (((c.y >> (3 * l)) & 7u) << 8);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    y[8 * l + j] = __fmul_rn(dl, __fadd_rn(float(int8_t((d_iq1s_grid.v[2 * idx + (j >> 2)] >> (8 * (j & 3))) & 0xFFu)), delta));
+            }
+            break;
+        }
         case TQMOE_Q4_0: {  // dequant.cpp:480-491: (q - 8) * d
             const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(aux + (row * S + s) * 2));
             const uint4 c = *reinterpret_cast<const uint4 *>(cd);

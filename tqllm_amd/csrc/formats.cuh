@@ -7,18 +7,20 @@
 #include "iq2s_lattice.h"
 #include "iq2xxs_lattice.h"
 #include "iq2xs_lattice.h"
+#include "iq1s_lattice.h"
 
 namespace tqmoe {
 
 // code bytes per sub-block
 __host__ __device__ constexpr int code_bytes_per_sub(uint32_t type) {
     return type == TQMOE_IQ3_S || type == TQMOE_IQ3_XXS || type == TQMOE_IQ2_S || type == TQMOE_IQ2_XS || type == TQMOE_Q3_K ? 12
-         : type == TQMOE_IQ2_XXS ? 8 : type == TQMOE_Q8_0 ? 32 : type == TQMOE_Q6_K ? 24 : 16;
+         : type == TQMOE_IQ2_XXS || type == TQMOE_Q2_K || type == TQMOE_IQ1_S ? 8 : type == TQMOE_Q8_0 ? 32 : type == TQMOE_Q6_K ? 24 : 16;
 }
 // aux record bytes per 256 weights (NVFP4G keeps bytes per 16 weights instead: see aux_row_bytes; IQ4_NL, Q4_0 and Q8_0
 // hold the eight fp16 scales of their 32-weight blocks)
-// Q5_K: the Q4_K header and the eight sub-blocks' high-bit words; Q6_K and Q3_K: sixteen int8 scales, d, padding
-__host__ __device__ constexpr int aux_record_bytes(uint32_t type) { return type == TQMOE_IQ4_XS ? 8 : type == TQMOE_Q5_K ? 48 : type == TQMOE_Q6_K || type == TQMOE_Q3_K ? 32 : 16; }
+// Q5_K: the Q4_K header and the eight sub-blocks' high-bit words; Q6_K and Q3_K: sixteen int8 scales, d, padding;
+// Q2_K: sixteen (scale | min << 4) bytes, d, dmin, padding
+__host__ __device__ constexpr int aux_record_bytes(uint32_t type) { return type == TQMOE_IQ4_XS ? 8 : type == TQMOE_Q5_K ? 48 : type == TQMOE_Q6_K || type == TQMOE_Q3_K || type == TQMOE_Q2_K ? 32 : 16; }
 __host__ __device__ constexpr int64_t code_row_bytes(uint32_t type, int cols) { return int64_t(cols / 32) * code_bytes_per_sub(type); }
 __host__ __device__ constexpr int64_t aux_row_bytes(uint32_t type, int cols) {
     return type == TQMOE_NVFP4G ? int64_t(cols / 16) : int64_t(cols / 256) * aux_record_bytes(type);
@@ -95,9 +97,23 @@ constexpr uint16_t kIq2xxsCodes[256] = {TQMOE_IQ2XXS_LATTICE16};
 __device__ const Iq2Grid<1024> d_iq2s_grid = make_iq2_grid(kIq2sCodes);
 __device__ const Iq2Grid<512> d_iq2xs_grid = make_iq2_grid(kIq2xsCodes);
 __device__ const Iq2Grid<256> d_iq2xxs_grid = make_iq2_grid(kIq2xxsCodes);
+// IQ1_S lattice points: two dwords per point, int8 values from {-1, 0, 1}
+constexpr Iq2Grid<2048> make_iq1s_grid() {
+    constexpr uint16_t codes[2048] = {TQMOE_IQ1S_LATTICE16};
+    constexpr uint32_t value[4] = {0x00, 0x01, 0xFF, 0};
+    Iq2Grid<2048> g{};
+    for (int i = 0; i < 2048; ++i)
+        for (int h = 0; h < 2; ++h) {
+            uint32_t w = 0;
+            for (int j = 0; j < 4; ++j) w |= value[(codes[i] >> (2 * (4 * h + j))) & 3u] << (8 * j);
+            g.v[2 * i + h] = w;
+        }
+    return g;
+}
+__device__ const Iq2Grid<2048> d_iq1s_grid = make_iq1s_grid();
 // dwords of a format's lattice as the kernels stage it in LDS (1: the format has none)
 __host__ __device__ constexpr int lattice_dwords(uint32_t type) {
-    return type == TQMOE_IQ3_S ? 512 : type == TQMOE_IQ3_XXS ? 256 : type == TQMOE_IQ2_S ? 2048 : type == TQMOE_IQ2_XS ? 1024 : type == TQMOE_IQ2_XXS ? 512 : 1;
+    return type == TQMOE_IQ3_S ? 512 : type == TQMOE_IQ3_XXS ? 256 : type == TQMOE_IQ2_S ? 2048 : type == TQMOE_IQ2_XS ? 1024 : type == TQMOE_IQ2_XXS ? 512 : type == TQMOE_IQ1_S ? 4096 : 1;
 }
 // lattice index of group l of an IQ2_S sub-block: its low byte and two bits of the sub-block's qh byte
 __device__ __forceinline__ uint32_t iq2s_index(uint32_t low4, uint32_t qh, int l) { return ((low4 >> (8 * l)) & 0xFFu) | ((qh << (8 - 2 * l)) & 0x300u); }

@@ -34,6 +34,27 @@ struct GateupArgs {
     int A, slots, topk, shared_ff, mode;
 };
 
+// arguments of the grouped fp16 products (prefill_f16_kernels.cuh)
+struct F16Args {
+    BankView b0, b1;
+    const void * x;           // input rows of xtype, cols = bank cols
+    uint32_t xtype;
+    const int * counts;       // [experts]
+    const int * offsets;      // [experts + 1]
+    const int * perm;         // assignment indices grouped by expert
+    int experts;
+    int xdiv;                 // input row of assignment a = a / xdiv
+    void * out;               // [assignments][rows], fp16 or fp32
+    int out_f32;
+    int gateup;
+    int shared_expert;        // the expert whose rows (gate / up) or columns (down) stop at shared_lim, or -1
+    int shared_lim;
+};
+// the grouped fp16 product of one bank format; wide: the 128 x 128 tile (grid of 128-row units), else 64 x 64
+template <uint32_t FMT> struct F16Launch {
+    static void run(const F16Args & k, bool two_banks, bool wide, dim3 grid, hipStream_t s);
+};
+
 // launch tables, one explicit instantiation per bank format (decode_<format>.hip)
 template <uint32_t FMT> struct DecodeLaunch {
     static void matvec(Split sp, int nb, const MatvecArgs & k, hipStream_t s);
@@ -56,5 +77,21 @@ extern template struct DecodeLaunch<TQMOE_Q4_0>;
 extern template struct DecodeLaunch<TQMOE_Q3_K>;
 extern template struct DecodeLaunch<TQMOE_IQ2_XXS>;
 extern template struct DecodeLaunch<TQMOE_IQ2_XS>;
+extern template struct F16Launch<TQMOE_IQ4_XS>;
+extern template struct F16Launch<TQMOE_Q4_K>;
+extern template struct F16Launch<TQMOE_IQ3_S>;
+extern template struct F16Launch<TQMOE_NVFP4G>;
+extern template struct F16Launch<TQMOE_IQ4_NL>;
+extern template struct F16Launch<TQMOE_Q8_0>;
+extern template struct F16Launch<TQMOE_Q5_K>;
+extern template struct F16Launch<TQMOE_Q6_K>;
+extern template struct F16Launch<TQMOE_IQ3_XXS>;
+extern template struct F16Launch<TQMOE_IQ2_S>;
+extern template struct F16Launch<TQMOE_Q2_K>;
+extern template struct F16Launch<TQMOE_IQ1_S>;
+extern template struct F16Launch<TQMOE_Q4_0>;
+extern template struct F16Launch<TQMOE_Q3_K>;
+extern template struct F16Launch<TQMOE_IQ2_XXS>;
+extern template struct F16Launch<TQMOE_IQ2_XS>;
 
 }  // namespace tqmoe

@@ -1,3 +1,5 @@
-// Decode kernels of one bank format (see decode_kernels.cuh).
+// Decode kernels and grouped fp16 products of one bank format (see decode_kernels.cuh, prefill_f16_kernels.cuh).
 #include "decode_kernels.cuh"
+#include "prefill_f16_kernels.cuh"
 template struct tqmoe::DecodeLaunch<TQMOE_IQ4_NL>;
+template struct tqmoe::F16Launch<TQMOE_IQ4_NL>;

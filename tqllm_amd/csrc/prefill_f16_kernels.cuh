@@ -1,0 +1,229 @@
+// Prefill-sized expert products of any bank format: a grouped fp16 x fp16 -> fp32 GEMM on the matrix pipe (the kernels;
+// prefill_f16.hip holds the entry, and one translation unit per bank format instantiates F16Launch<FMT>).
+//
+// The counterpart of the reference's WeightFormat::expert_gemm / expert_gemm_gateup (weight_format.hpp:51-59): weights
+// turned into fp16 tiles in LDS, input rows converted to fp16, products accumulated in fp32 by
+// v_mfma_f32_32x32x16_f16, gate and up in one launch with the SwiGLU epilogue.
+//
+// A block takes one expert, up to 64 W of its assignments (the dispatch lists give them) and 64 W weight rows of each
+// bank, W = 1 or 2; its four waves hold a (32 W) x (32 W) tile each as W x W matrix instructions. Per stage of 128 / W
+// weights of a row the block puts the input tile and the weight tile(s) in LDS and every wave issues 8 W
+// matrix instructions per bank. With W = 2 an operand read from LDS feeds two instructions and a weight tile serves twice
+// the rows; two such blocks fit a CU, one staging while the other multiplies.
+//
+// Weight values. A thread takes one 32-weight sub-block through the format's decode-kernel traits (Sub<FMT>: the int8
+// values q, the scale(s) and the minimum(s)) and makes fp16(q * scale - minimum) with one fp32 multiply-add per weight:
+// the product and the difference are rounded once in fp32 (2^-24) and once to fp16, where the exact decoder of the
+// fp32 dequantiser rounds them separately; the difference is far below the fp16 step.
+#pragma once
+#include "decode_kernels.cuh"
+
+namespace tqmoe {
+namespace {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// the expert whose run of ROWS-row blocks holds `unit`; local = the block inside the expert; expert = -1 past the last
+struct Where { int expert, local; };
+template <int ROWS> __device__ __forceinline__ Where locate(const int * __restrict__ counts, int experts, int unit) {
+    __shared__ Where w;
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        if (lane == 0) w.expert = -1;
+        int base = 0;
+        for (int e0 = 0; e0 < experts; e0 += 64) {
+            const int e = e0 + lane;
+            const int units = e < experts ? (max(counts[e], 0) + ROWS - 1) / ROWS : 0;
+            int ui = units;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) { const int a = __shfl_up(ui, d, 64); if (lane >= d) ui += a; }
+            if (units > 0 && unit >= base + ui - units && unit < base + ui) { w.expert = e; w.local = unit - (base + ui - units); }
+            base += __shfl(ui, 63, 64);
+            if (unit < base) break;
+        }
+    }
+    __syncthreads();
+    return w;
+}
+
+typedef float v2f __attribute__((ext_vector_type(2)));
+// two floats -> two halves, round to nearest even (one packed conversion)
+__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
+    const v2f v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2h));
+}
+
+// four int8 values -> four halves fp16(q * scale - minimum) (two dwords): the bytes are biased to unsigned so that each
+// converts to fp32 in one instruction, and the bias goes into the constant of the multiply-add, c = -(128 scale + minimum)
+__device__ __forceinline__ uint2 i8x4_to_h4(uint32_t w, float scale, float c) {
+    const uint32_t u = w ^ 0x80808080u;
+    const float f0 = float(u & 0xFFu), f1 = float((u >> 8) & 0xFFu), f2 = float((u >> 16) & 0xFFu), f3 = float(u >> 24);
+    return make_uint2(pack_h2(fmaf(f0, scale, c), fmaf(f1, scale, c)), pack_h2(fmaf(f2, scale, c), fmaf(f3, scale, c)));
+}
+
+// The fp16 values of sub-block s of weight row `row` (an index into the stacked bank), as 16 dwords in weight order.
+template <uint32_t FMT> struct F16Sub {
+    static __device__ __forceinline__ void get(const BankView & b, int64_t row, int s, const uint32_t * grid, uint32_t (&h)[16]) {
+        Tile t;
+        t.codes = b.codes + row * code_row_bytes(FMT, b.cols);
+        t.aux = b.aux + row * aux_row_bytes(FMT, b.cols);
+        t.aux2 = FMT == TQMOE_NVFP4G ? b.aux + nvfp4_global_offset(b.rows_total, b.cols) + row * 4 : nullptr;
+        const typename Sub<FMT>::Raw raw = Sub<FMT>::load(t, 0u, uint32_t(b.cols / 32), uint32_t(s));
+        Dec d;
+        d.mn1 = 0.f;
+        Sub<FMT>::decode(raw, s, grid, d);
+        const float c0 = -(128.f * d.s0 + d.mn), c1 = -(128.f * d.s1 + (HalfMins<Sub<FMT>>::value ? d.mn1 : d.mn));
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const uint2 v = i8x4_to_h4(d.w[q], q < 4 ? d.s0 : d.s1, q < 4 ? c0 : c1);
+            h[2 * q] = v.x;
+            h[2 * q + 1] = v.y;
+        }
+    }
+};
+// IQ4_XS banks are tile-major and have kernels of their own for the decode-sized products: the same steps from the
+// tile-major offsets
+template <> struct F16Sub<TQMOE_IQ4_XS> {
+    static __device__ __forceinline__ void get(const BankView & b, int64_t row, int s, const uint32_t *, uint32_t (&h)[16]) {
+        const int S = b.cols / 32;
+        const uint4 c = *reinterpret_cast<const uint4 *>(b.codes + iq4xs_code_offset(row, S, s));
+        const uint2 rec = *reinterpret_cast<const uint2 *>(b.aux + iq4xs_aux_offset(row, S, s / 8));
+        const float sc = half_bits_to_float(iq4xs_d_bits(rec)) * float(iq4xs_lsm32(rec, s & 7)), c0 = -128.f * sc;
+        const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t lo, hi;
+            lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(w[q], lo, hi);
+            const uint2 a = i8x4_to_h4(lo, sc, c0), z = i8x4_to_h4(hi, sc, c0);
+            h[2 * q] = a.x; h[2 * q + 1] = a.y;
+            h[8 + 2 * q] = z.x; h[8 + 2 * q + 1] = z.y;
+        }
+    }
+};
+
+// 32 input values of a row as 16 dwords of halves
+__device__ __forceinline__ void load_x32(const void * x, uint32_t xtype, int64_t at, uint32_t (&h)[16]) {
+    float v[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        if (xtype == TQMOE_F32) load8<TQMOE_F32>(x, at + q * 8, v);
+        else if (xtype == TQMOE_F16) load8<TQMOE_F16>(x, at + q * 8, v);
+        else load8<TQMOE_BF16>(x, at + q * 8, v);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) h[4 * q + j] = pack_h2(v[2 * j], v[2 * j + 1]);
+    }
+}
+
+template <uint32_t FMT, int NB, int W>
+__global__ __launch_bounds__(256, W == 2 ? 2 : 1) void expert_gemm_f16_k(F16Args k) {
+    constexpr int kM = 64 * W, kN = 64 * W, kK = 128 / W, kPad = kK + 8;   // padded rows: 16-byte reads of consecutive rows spread over the LDS banks
+    constexpr int kSubs = kK / 32;                                           // sub-blocks of a row per stage; 256 threads = kN rows x kSubs
+    __shared__ __attribute__((aligned(16))) uint16_t As[kM][kPad];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[NB][kN][kPad];
+    __shared__ __attribute__((aligned(8))) uint32_t grid_lds[lattice_dwords(FMT)];
+    __shared__ int s_asg[kM];
+    const Where w = locate<kM>(k.counts, k.experts, int(blockIdx.y));
+    const int e = w.expert;
+    if (e < 0) return;
+    const uint32_t * grid = stage_grid<FMT>(grid_lds);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
+    const int mq = wave & 1, nq = wave >> 1;                   // wave tile: input rows 32 W mq.., weight rows 32 W nq.. of the block's tile
+    const BankView & b0 = k.b0;
+    const int rows = b0.rows, cols = b0.cols, S = cols / 32, row0 = int(blockIdx.x) * kN;
+    const bool is_shared = e == k.shared_expert;
+    const int row_lim = k.gateup && is_shared ? k.shared_lim : rows;     // weight rows this expert has
+    const int s_end = !k.gateup && is_shared ? k.shared_lim / 32 : S;    // sub-blocks of the input rows it reads
+    const int cnt = k.counts[e], first = w.local * kM;
+    if (tid < kM) s_asg[tid] = first + tid < cnt ? k.perm[k.offsets[e] + first + tid] : -1;
+    __syncthreads();
+    const bool wave_has_rows = first + mq * 32 * W < cnt;      // a wave whose input rows are all past the list multiplies nothing
+
+    v16f acc[NB][W][W];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int t = 0; t < W * W; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[nb][t / W][t % W][i] = 0.f;
+    const int tr = tid / kSubs, tp = tid % kSubs;               // staging: row of the tile, the sub-block of the stage's kSubs
+    const int a_asg = s_asg[tr];
+    const int64_t a_at = int64_t(max(a_asg, 0) / k.xdiv) * cols + tp * 32;
+    const bool b_row = row0 + tr < row_lim;
+    for (int s0 = 0; s0 < s_end; s0 += kSubs) {
+        const bool in_k = s0 + tp < s_end;
+        {
+            uint32_t h[16];
+            if (a_asg >= 0 && in_k) load_x32(k.x, k.xtype, a_at + int64_t(s0) * 32, h);
+            else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) h[i] = 0u;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *reinterpret_cast<uint4 *>(&As[tr][tp * 32 + q * 8]) = make_uint4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3]);
+        }
+#pragma unroll
+        for (int bb = 0; bb < NB; ++bb) {
+            uint32_t h[16];
+            if (b_row && in_k) F16Sub<FMT>::get(bb ? k.b1 : k.b0, int64_t(e) * rows + row0 + tr, s0 + tp, grid, h);
+            else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) h[i] = 0u;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *reinterpret_cast<uint4 *>(&Bs[bb][tr][tp * 32 + q * 8]) = make_uint4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3]);
+        }
+        __syncthreads();
+        if (wave_has_rows) {
+#pragma unroll
+            for (int j = 0; j < kK / 16; ++j) {     // operand of lane (r, g): row r, columns 16 j + 8 g .. + 7
+                v8h a[W];
+#pragma unroll
+                for (int mi = 0; mi < W; ++mi) a[mi] = *reinterpret_cast<const v8h *>(&As[(mq * W + mi) * 32 + r][16 * j + 8 * g]);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    v8h b[W];
+#pragma unroll
+                    for (int ni = 0; ni < W; ++ni) b[ni] = *reinterpret_cast<const v8h *>(&Bs[nb][(nq * W + ni) * 32 + r][16 * j + 8 * g]);
+#pragma unroll
+                    for (int mi = 0; mi < W; ++mi)
+#pragma unroll
+                        for (int ni = 0; ni < W; ++ni) acc[nb][mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b[ni], acc[nb][mi][ni], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (!wave_has_rows) return;
+    // result register i of lane half g: input row 8 (i / 4) + 4 g + i % 4 of the 32 x 32 tile, weight row r
+#pragma unroll
+    for (int ni = 0; ni < W; ++ni) {
+        const int col = row0 + (nq * W + ni) * 32 + r;
+        if (col >= rows) continue;
+#pragma unroll
+        for (int mi = 0; mi < W; ++mi)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int a = s_asg[(mq * W + mi) * 32 + 8 * (i >> 2) + 4 * g + (i & 3)];
+                if (a < 0) continue;
+                float v = acc[0][mi][ni][i];
+                if (k.gateup) v = v / (1.f + expf(-v)) * acc[NB - 1][mi][ni][i];
+                v = col < row_lim ? v : 0.f;
+                if (k.out_f32) static_cast<float *>(k.out)[int64_t(a) * rows + col] = v;
+                else static_cast<uint16_t *>(k.out)[int64_t(a) * rows + col] = __half_as_ushort(__float2half_rn(v));
+            }
+    }
+}
+
+}  // namespace
+
+template <uint32_t FMT> void F16Launch<FMT>::run(const F16Args & k, bool two_banks, bool wide, dim3 grid, hipStream_t s) {
+    if (wide) {
+        if (two_banks) expert_gemm_f16_k<FMT, 2, 2><<<grid, 256, 0, s>>>(k); else expert_gemm_f16_k<FMT, 1, 2><<<grid, 256, 0, s>>>(k);
+    } else {
+        if (two_banks) expert_gemm_f16_k<FMT, 2, 1><<<grid, 256, 0, s>>>(k); else expert_gemm_f16_k<FMT, 1, 1><<<grid, 256, 0, s>>>(k);
+    }
+}
+
+}  // namespace tqmoe

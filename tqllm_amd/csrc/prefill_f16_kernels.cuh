@@ -63,14 +63,19 @@ __device__ __forceinline__ uint2 i8x4_to_h4(uint32_t w, float scale, float c) {
     return make_uint2(pack_h2(fmaf(f0, scale, c), fmaf(f1, scale, c)), pack_h2(fmaf(f2, scale, c), fmaf(f3, scale, c)));
 }
 
-// The fp16 values of sub-block s of weight row `row` (an index into the stacked bank), as 16 dwords in weight order.
+// The fp16 values of sub-block s of weight row `row` (an index into the stacked bank), as 16 dwords in weight order, in two
+// steps so that the loads of a stage can be in flight during the products of the one before: load() issues the loads,
+// finish() turns what they brought into halves.
 template <uint32_t FMT> struct F16Sub {
-    static __device__ __forceinline__ void get(const BankView & b, int64_t row, int s, const uint32_t * grid, uint32_t (&h)[16]) {
+    typedef typename Sub<FMT>::Raw Raw;
+    static __device__ __forceinline__ Raw load(const BankView & b, int64_t row, int s) {
         Tile t;
         t.codes = b.codes + row * code_row_bytes(FMT, b.cols);
         t.aux = b.aux + row * aux_row_bytes(FMT, b.cols);
         t.aux2 = FMT == TQMOE_NVFP4G ? b.aux + nvfp4_global_offset(b.rows_total, b.cols) + row * 4 : nullptr;
-        const typename Sub<FMT>::Raw raw = Sub<FMT>::load(t, 0u, uint32_t(b.cols / 32), uint32_t(s));
+        return Sub<FMT>::load(t, 0u, uint32_t(b.cols / 32), uint32_t(s));
+    }
+    static __device__ __forceinline__ void finish(const Raw & raw, int s, const uint32_t * grid, uint32_t (&h)[16]) {
         Dec d;
         d.mn1 = 0.f;
         Sub<FMT>::decode(raw, s, grid, d);
@@ -86,12 +91,17 @@ template <uint32_t FMT> struct F16Sub {
 // IQ4_XS banks are tile-major and have kernels of their own for the decode-sized products: the same steps from the
 // tile-major offsets
 template <> struct F16Sub<TQMOE_IQ4_XS> {
-    static __device__ __forceinline__ void get(const BankView & b, int64_t row, int s, const uint32_t *, uint32_t (&h)[16]) {
+    struct Raw { uint4 c; uint2 rec; };
+    static __device__ __forceinline__ Raw load(const BankView & b, int64_t row, int s) {
         const int S = b.cols / 32;
-        const uint4 c = *reinterpret_cast<const uint4 *>(b.codes + iq4xs_code_offset(row, S, s));
-        const uint2 rec = *reinterpret_cast<const uint2 *>(b.aux + iq4xs_aux_offset(row, S, s / 8));
-        const float sc = half_bits_to_float(iq4xs_d_bits(rec)) * float(iq4xs_lsm32(rec, s & 7)), c0 = -128.f * sc;
-        const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+        Raw r;
+        r.c = *reinterpret_cast<const uint4 *>(b.codes + iq4xs_code_offset(row, S, s));
+        r.rec = *reinterpret_cast<const uint2 *>(b.aux + iq4xs_aux_offset(row, S, s / 8));
+        return r;
+    }
+    static __device__ __forceinline__ void finish(const Raw & r, int s, const uint32_t *, uint32_t (&h)[16]) {
+        const float sc = half_bits_to_float(iq4xs_d_bits(r.rec)) * float(iq4xs_lsm32(r.rec, s & 7)), c0 = -128.f * sc;
+        const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             uint32_t lo, hi;
@@ -103,16 +113,38 @@ template <> struct F16Sub<TQMOE_IQ4_XS> {
     }
 };
 
-// 32 input values of a row as 16 dwords of halves
-__device__ __forceinline__ void load_x32(const void * x, uint32_t xtype, int64_t at, uint32_t (&h)[16]) {
-    float v[8];
+// 32 input values of a row: 16-bit types are fetched a stage ahead as four 16-byte pieces, fp32 rows at the time of use
+struct RawX { uint4 v[4]; };
+__device__ __forceinline__ RawX load_x32(const void * x, uint32_t xtype, int64_t at) {
+    RawX r;
+    if (xtype != TQMOE_F32) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        if (xtype == TQMOE_F32) load8<TQMOE_F32>(x, at + q * 8, v);
-        else if (xtype == TQMOE_F16) load8<TQMOE_F16>(x, at + q * 8, v);
-        else load8<TQMOE_BF16>(x, at + q * 8, v);
+        for (int q = 0; q < 4; ++q) r.v[q] = reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(x) + at)[q];
+    } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) h[4 * q + j] = pack_h2(v[2 * j], v[2 * j + 1]);
+        for (int q = 0; q < 4; ++q) r.v[q] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    return r;
+}
+__device__ __forceinline__ void finish_x32(const RawX & r, const void * x, uint32_t xtype, int64_t at, uint32_t (&h)[16]) {
+    if (xtype == TQMOE_F16) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { h[4 * q] = r.v[q].x; h[4 * q + 1] = r.v[q].y; h[4 * q + 2] = r.v[q].z; h[4 * q + 3] = r.v[q].w; }
+    } else if (xtype == TQMOE_BF16) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t w[4] = {r.v[q].x, r.v[q].y, r.v[q].z, r.v[q].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) h[4 * q + j] = pack_h2(__uint_as_float(w[j] << 16), __uint_as_float(w[j] & 0xFFFF0000u));
+        }
+    } else {
+        float v[8];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            load8<TQMOE_F32>(x, at + q * 8, v);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) h[4 * q + j] = pack_h2(v[2 * j], v[2 * j + 1]);
+        }
     }
 }
 
@@ -151,12 +183,18 @@ __global__ __launch_bounds__(256, W == 2 ? 2 : 1) void expert_gemm_f16_k(F16Args
     const int a_asg = s_asg[tr];
     const int64_t a_at = int64_t(max(a_asg, 0) / k.xdiv) * cols + tp * 32;
     const bool b_row = row0 + tr < row_lim;
+    // loads run one stage ahead of their use; past the last sub-block they repeat it (the values are not used)
+    const int64_t b_row_at = int64_t(e) * rows + row0 + (b_row ? tr : 0);
+    RawX raw_a = load_x32(k.x, k.xtype, a_at + int64_t(min(tp, S - 1) - tp) * 32);
+    typename F16Sub<FMT>::Raw raw_b[NB];
+#pragma unroll
+    for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(tp, S - 1));
     for (int s0 = 0; s0 < s_end; s0 += kSubs) {
         const bool in_k = s0 + tp < s_end;
         {
             uint32_t h[16];
-            if (a_asg >= 0 && in_k) load_x32(k.x, k.xtype, a_at + int64_t(s0) * 32, h);
-            else {
+            finish_x32(raw_a, k.x, k.xtype, a_at + int64_t(min(s0 + tp, S - 1) - tp) * 32, h);
+            if (!(a_asg >= 0 && in_k)) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) h[i] = 0u;
             }
@@ -166,13 +204,19 @@ __global__ __launch_bounds__(256, W == 2 ? 2 : 1) void expert_gemm_f16_k(F16Args
 #pragma unroll
         for (int bb = 0; bb < NB; ++bb) {
             uint32_t h[16];
-            if (b_row && in_k) F16Sub<FMT>::get(bb ? k.b1 : k.b0, int64_t(e) * rows + row0 + tr, s0 + tp, grid, h);
-            else {
+            F16Sub<FMT>::finish(raw_b[bb], min(s0 + tp, S - 1), grid, h);
+            if (!(b_row && in_k)) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) h[i] = 0u;
             }
 #pragma unroll
             for (int q = 0; q < 4; ++q) *reinterpret_cast<uint4 *>(&Bs[bb][tr][tp * 32 + q * 8]) = make_uint4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3]);
+        }
+        {
+            const int sn = min(s0 + kSubs + tp, S - 1);
+            raw_a = load_x32(k.x, k.xtype, a_at + int64_t(sn - tp) * 32);
+#pragma unroll
+            for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, sn);
         }
         __syncthreads();
         if (wave_has_rows) {

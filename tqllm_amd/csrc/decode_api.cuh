@@ -50,7 +50,7 @@ struct F16Args {
     int shared_expert;        // the expert whose rows (gate / up) or columns (down) stop at shared_lim, or -1
     int shared_lim;
 };
-// the grouped fp16 product of one bank format; wide: the 128 x 128 tile (grid of 128-row units), else 64 x 64
+// the grouped fp16 product of one bank format; wide: 128 input rows per block (grid.y counts such units), else 64
 template <uint32_t FMT> struct F16Launch {
     static void run(const F16Args & k, bool two_banks, bool wide, dim3 grid, hipStream_t s);
 };

@@ -400,8 +400,8 @@ template <> struct Sub<TQMOE_NVFP4G> {
 #pragma unroll
         for (int q = 0; q < 4; ++q) lookup16<kFp4T0, kFp4T1, kFp4T2, kFp4T3>(w[q], d.w[q], d.w[4 + q]);
         // low nibbles = the first 16-weight group, high nibbles = the second; table values are twice the E2M1 value
-        d.s0 = e4m3_to_float(r.sc & 0xFFu) * (0.5f * r.g);
-        d.s1 = e4m3_to_float(r.sc >> 8) * (0.5f * r.g);
+        d.s0 = e4m3_to_float_fast(r.sc & 0xFFu) * (0.5f * r.g);
+        d.s1 = e4m3_to_float_fast(r.sc >> 8) * (0.5f * r.g);
         d.mn = 0.f;
     }
 };

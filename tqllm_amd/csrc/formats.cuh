@@ -135,6 +135,13 @@ __device__ __forceinline__ float e4m3_to_float(uint32_t b) {
     return (b & 0x80u) ? -v : v;
 }
 
+// the same through the fp16 conversion: the seven low bits moved to fp16's exponent and mantissa fields are the value
+// times 2^-8, subnormals included (one conversion and one multiply); the NaN codes are kept
+__device__ __forceinline__ float e4m3_to_float_fast(uint32_t b) {
+    const float v = half_bits_to_float(uint16_t(((b & 0x80u) << 8) | ((b & 0x7Fu) << 7))) * 256.f;
+    return (b & 0x7Fu) == 0x7Fu ? __uint_as_float(0x7FC00000u) : v;
+}
+
 // four bits -> the low bit of four bytes
 __device__ __forceinline__ uint32_t spread4(uint32_t bits) { return ((bits & 15u) * 0x00204081u) & 0x01010101u; }
 // eight bits (four 2-bit fields) -> the low two bits of four bytes

@@ -9,7 +9,7 @@ template struct F16Launch<TQMOE_IQ4_XS>;
 
 namespace {
 
-constexpr int kWideFrom = 64;   // assignments per expert, on average, from which the 128 x 128 tile is used
+constexpr int kWideFrom = 64;   // assignments per expert, on average, from which a block takes 128 input rows
 
 void dispatch_f16(uint32_t type, const F16Args & k, bool two, bool wide, dim3 grid, hipStream_t s) {
     switch (type) {
@@ -28,10 +28,10 @@ int32_t enqueue_gemm_f16(const tqmoe_bank & b0, const tqmoe_bank * b1, const voi
                          int experts, int64_t assignments, int xdiv, void * out, int out_f32, int gateup, int shared_expert, int shared_lim, hipStream_t s) {
     const F16Args k{view(b0), b1 ? view(*b1) : view(b0), x, xtype, counts, offsets, perm, experts, xdiv, out, out_f32, gateup, shared_expert, shared_lim};
     const bool wide = assignments >= int64_t(experts) * kWideFrom;   // half a wide tile filled on average
-    const int tile = wide ? 128 : 64;
+    const int tile = wide ? 128 : 64;                                // input rows of a block
     const int64_t units = assignments / tile + experts;              // sum of ceil(count / tile) never exceeds this
     if (units > 65535) return -1;
-    dispatch_f16(b0.type, k, b1 != nullptr, wide, dim3(unsigned((b0.rows + tile - 1) / tile), unsigned(units)), s);
+    dispatch_f16(b0.type, k, b1 != nullptr, wide, dim3(unsigned((b0.rows + 127) / 128), unsigned(units)), s);
     return 0;
 }
 

@@ -2,14 +2,15 @@
 // prefill_f16.hip holds the entry, and one translation unit per bank format instantiates F16Launch<FMT>).
 //
 // The counterpart of the reference's WeightFormat::expert_gemm / expert_gemm_gateup (weight_format.hpp:51-59): weights
-// turned into fp16 tiles in LDS, input rows converted to fp16, products accumulated in fp32 by
+// turned into fp16 operands in registers, input rows converted to fp16 tiles in LDS, products accumulated in fp32 by
 // v_mfma_f32_32x32x16_f16, gate and up in one launch with the SwiGLU epilogue.
 //
-// A block takes one expert, up to 64 W of its assignments (the dispatch lists give them) and 64 W weight rows of each
-// bank, W = 1 or 2; its four waves hold a (32 W) x (32 W) tile each as W x W matrix instructions. Per stage of 128 / W
-// weights of a row the block puts the input tile and the weight tile(s) in LDS and every wave issues 8 W
-// matrix instructions per bank. With W = 2 an operand read from LDS feeds two instructions and a weight tile serves twice
-// the rows; two such blocks fit a CU, one staging while the other multiplies.
+// A block takes one expert, up to 128 (or 64) of its assignments (the dispatch lists give them) and 128 weight rows of
+// each bank; each of its four waves owns 32 of the weight rows and all the block's input rows, four (two) 32 x 32 tiles per
+// bank. Per stage of 64 weights of a row, lane (r, g) of a wave decodes sub-block g of its weight row r: those sixteen
+// dwords ARE its weight operands of the stage's four matrix instructions per tile, so weights never pass through LDS.
+// The input tile does (double-buffered, one barrier per stage), each 16-byte operand read feeding one instruction per
+// bank. Weight and input loads are issued one stage ahead of their use.
 //
 // Weight values. A thread takes one 32-weight sub-block through the format's decode-kernel traits (Sub<FMT>: the int8
 // values q, the scale(s) and the minimum(s)) and makes fp16(q * scale - minimum) with one fp32 multiply-add per weight:
@@ -75,14 +76,16 @@ template <uint32_t FMT> struct F16Sub {
         t.aux2 = FMT == TQMOE_NVFP4G ? b.aux + nvfp4_global_offset(b.rows_total, b.cols) + row * 4 : nullptr;
         return Sub<FMT>::load(t, 0u, uint32_t(b.cols / 32), uint32_t(s));
     }
-    static __device__ __forceinline__ void finish(const Raw & raw, int s, const uint32_t * grid, uint32_t (&h)[16]) {
+    // valid false: all zeros (a row or a sub-block past the end), through a zero scale and constant
+    static __device__ __forceinline__ void finish(const Raw & raw, int s, const uint32_t * grid, bool valid, uint32_t (&h)[16]) {
         Dec d;
         d.mn1 = 0.f;
         Sub<FMT>::decode(raw, s, grid, d);
-        const float c0 = -(128.f * d.s0 + d.mn), c1 = -(128.f * d.s1 + (HalfMins<Sub<FMT>>::value ? d.mn1 : d.mn));
+        const float s0 = valid ? d.s0 : 0.f, s1 = valid ? d.s1 : 0.f;
+        const float c0 = valid ? -(128.f * d.s0 + d.mn) : 0.f, c1 = valid ? -(128.f * d.s1 + (HalfMins<Sub<FMT>>::value ? d.mn1 : d.mn)) : 0.f;
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
-            const uint2 v = i8x4_to_h4(d.w[q], q < 4 ? d.s0 : d.s1, q < 4 ? c0 : c1);
+            const uint2 v = i8x4_to_h4(d.w[q], q < 4 ? s0 : s1, q < 4 ? c0 : c1);
             h[2 * q] = v.x;
             h[2 * q + 1] = v.y;
         }
@@ -99,8 +102,8 @@ template <> struct F16Sub<TQMOE_IQ4_XS> {
         r.rec = *reinterpret_cast<const uint2 *>(b.aux + iq4xs_aux_offset(row, S, s / 8));
         return r;
     }
-    static __device__ __forceinline__ void finish(const Raw & r, int s, const uint32_t *, uint32_t (&h)[16]) {
-        const float sc = half_bits_to_float(iq4xs_d_bits(r.rec)) * float(iq4xs_lsm32(r.rec, s & 7)), c0 = -128.f * sc;
+    static __device__ __forceinline__ void finish(const Raw & r, int s, const uint32_t *, bool valid, uint32_t (&h)[16]) {
+        const float sc = valid ? half_bits_to_float(iq4xs_d_bits(r.rec)) * float(iq4xs_lsm32(r.rec, s & 7)) : 0.f, c0 = -128.f * sc;
         const uint32_t w[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -148,12 +151,10 @@ __device__ __forceinline__ void finish_x32(const RawX & r, const void * x, uint3
     }
 }
 
-template <uint32_t FMT, int NB, int W>
-__global__ __launch_bounds__(256, W == 2 ? 2 : 1) void expert_gemm_f16_k(F16Args k) {
-    constexpr int kM = 64 * W, kN = 64 * W, kK = 128 / W, kPad = kK + 8;   // padded rows: 16-byte reads of consecutive rows spread over the LDS banks
-    constexpr int kSubs = kK / 32;                                           // sub-blocks of a row per stage; 256 threads = kN rows x kSubs
-    __shared__ __attribute__((aligned(16))) uint16_t As[kM][kPad];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[NB][kN][kPad];
+template <uint32_t FMT, int NB, int MT>
+__global__ __launch_bounds__(256, 2) void expert_gemm_f16_k(F16Args k) {
+    constexpr int kM = 32 * MT, kN = 128, kK = 64, kPad = kK + 8;   // padded rows: 16-byte reads of consecutive rows spread over the LDS banks
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][kM][kPad];
     __shared__ __attribute__((aligned(8))) uint32_t grid_lds[lattice_dwords(FMT)];
     __shared__ int s_asg[kM];
     const Where w = locate<kM>(k.counts, k.experts, int(blockIdx.y));
@@ -161,7 +162,6 @@ __global__ __launch_bounds__(256, W == 2 ? 2 : 1) void expert_gemm_f16_k(F16Args
     if (e < 0) return;
     const uint32_t * grid = stage_grid<FMT>(grid_lds);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
-    const int mq = wave & 1, nq = wave >> 1;                   // wave tile: input rows 32 W mq.., weight rows 32 W nq.. of the block's tile
     const BankView & b0 = k.b0;
     const int rows = b0.rows, cols = b0.cols, S = cols / 32, row0 = int(blockIdx.x) * kN;
     const bool is_shared = e == k.shared_expert;
@@ -169,104 +169,97 @@ __global__ __launch_bounds__(256, W == 2 ? 2 : 1) void expert_gemm_f16_k(F16Args
     const int s_end = !k.gateup && is_shared ? k.shared_lim / 32 : S;    // sub-blocks of the input rows it reads
     const int cnt = k.counts[e], first = w.local * kM;
     if (tid < kM) s_asg[tid] = first + tid < cnt ? k.perm[k.offsets[e] + first + tid] : -1;
+    for (int i = tid; i < 2 * kM * kPad / 8; i += 256) reinterpret_cast<uint4 *>(&As[0][0][0])[i] = make_uint4(0u, 0u, 0u, 0u);
     __syncthreads();
-    const bool wave_has_rows = first + mq * 32 * W < cnt;      // a wave whose input rows are all past the list multiplies nothing
+    const int m_tiles = min(MT, (cnt - first + 31) / 32);      // 32-row tiles of the block that hold assignments
 
-    v16f acc[NB][W][W];
+    v16f acc[NB][MT];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int t = 0; t < W * W; ++t)
+        for (int mi = 0; mi < MT; ++mi)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) acc[nb][t / W][t % W][i] = 0.f;
-    const int tr = tid / kSubs, tp = tid % kSubs;               // staging: row of the tile, the sub-block of the stage's kSubs
-    const int a_asg = s_asg[tr];
-    const int64_t a_at = int64_t(max(a_asg, 0) / k.xdiv) * cols + tp * 32;
-    const bool b_row = row0 + tr < row_lim;
+            for (int i = 0; i < 16; ++i) acc[nb][mi][i] = 0.f;
+    // input staging: thread -> (row, sub-block of the stage's two); with fewer than 128 rows the upper threads idle
+    const int tr = tid >> 1, tp = tid & 1;
+    const bool a_thread = tr < kM;
+    const int a_asg = a_thread ? s_asg[tr] : -1;
+    const int64_t a_at = int64_t(max(a_asg, 0) / k.xdiv) * cols;
+    // weights: lane (r, g) of wave w decodes sub-block g of the stage for weight row row0 + 32 w + r: its operand registers
+    const int col = row0 + 32 * wave + r;
+    const bool b_row = col < row_lim;
+    const int64_t b_row_at = int64_t(e) * rows + (b_row ? col : row0);
     // loads run one stage ahead of their use; past the last sub-block they repeat it (the values are not used)
-    const int64_t b_row_at = int64_t(e) * rows + row0 + (b_row ? tr : 0);
-    RawX raw_a = load_x32(k.x, k.xtype, a_at + int64_t(min(tp, S - 1) - tp) * 32);
+    RawX raw_a = load_x32(k.x, k.xtype, a_at + int64_t(min(tp, S - 1)) * 32);
     typename F16Sub<FMT>::Raw raw_b[NB];
 #pragma unroll
-    for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(tp, S - 1));
-    for (int s0 = 0; s0 < s_end; s0 += kSubs) {
-        const bool in_k = s0 + tp < s_end;
-        {
+    for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(g, S - 1));
+    int buf = 0;
+    for (int s0 = 0; s0 < s_end; s0 += 2, buf ^= 1) {
+        if (a_asg >= 0) {                       // rows without an assignment stay zero
             uint32_t h[16];
-            finish_x32(raw_a, k.x, k.xtype, a_at + int64_t(min(s0 + tp, S - 1) - tp) * 32, h);
-            if (!(a_asg >= 0 && in_k)) {
+            finish_x32(raw_a, k.x, k.xtype, a_at + int64_t(min(s0 + tp, S - 1)) * 32, h);
+            if (s0 + 2 > s_end) {               // the last stage of an odd number of sub-blocks (uniform)
+                if (s0 + tp >= s_end) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) h[i] = 0u;
+                    for (int i = 0; i < 16; ++i) h[i] = 0u;
+                }
             }
 #pragma unroll
-            for (int q = 0; q < 4; ++q) *reinterpret_cast<uint4 *>(&As[tr][tp * 32 + q * 8]) = make_uint4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3]);
+            for (int q = 0; q < 4; ++q) *reinterpret_cast<uint4 *>(&As[buf][tr][tp * 32 + q * 8]) = make_uint4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3]);
         }
+        uint32_t hb[NB][16];
 #pragma unroll
         for (int bb = 0; bb < NB; ++bb) {
-            uint32_t h[16];
-            F16Sub<FMT>::finish(raw_b[bb], min(s0 + tp, S - 1), grid, h);
-            if (!(b_row && in_k)) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) h[i] = 0u;
-            }
-#pragma unroll
-            for (int q = 0; q < 4; ++q) *reinterpret_cast<uint4 *>(&Bs[bb][tr][tp * 32 + q * 8]) = make_uint4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3]);
+            F16Sub<FMT>::finish(raw_b[bb], min(s0 + g, S - 1), grid, b_row && s0 + g < s_end, hb[bb]);
         }
         {
-            const int sn = min(s0 + kSubs + tp, S - 1);
-            raw_a = load_x32(k.x, k.xtype, a_at + int64_t(sn - tp) * 32);
+            raw_a = load_x32(k.x, k.xtype, a_at + int64_t(min(s0 + 2 + tp, S - 1)) * 32);
 #pragma unroll
-            for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, sn);
+            for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(s0 + 2 + g, S - 1));
         }
+        // one barrier per stage: the tile written now was last read two stages ago, before the barrier of the stage between
         __syncthreads();
-        if (wave_has_rows) {
+        // product j of a stage takes weights 8 j .. 8 j + 7 of the lane's sub-block; the input operand of lane (m, g) is the same
+        // eight columns 32 g + 8 j .. of input row m (the order of the sum inside a stage is free as long as both agree)
 #pragma unroll
-            for (int j = 0; j < kK / 16; ++j) {     // operand of lane (r, g): row r, columns 16 j + 8 g .. + 7
-                v8h a[W];
+        for (int j = 0; j < 4; ++j) {
 #pragma unroll
-                for (int mi = 0; mi < W; ++mi) a[mi] = *reinterpret_cast<const v8h *>(&As[(mq * W + mi) * 32 + r][16 * j + 8 * g]);
+            for (int mi = 0; mi < MT; ++mi) {
+                if (mi < m_tiles) {
+                    const v8h a = *reinterpret_cast<const v8h *>(&As[buf][mi * 32 + r][32 * g + 8 * j]);
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    v8h b[W];
-#pragma unroll
-                    for (int ni = 0; ni < W; ++ni) b[ni] = *reinterpret_cast<const v8h *>(&Bs[nb][(nq * W + ni) * 32 + r][16 * j + 8 * g]);
-#pragma unroll
-                    for (int mi = 0; mi < W; ++mi)
-#pragma unroll
-                        for (int ni = 0; ni < W; ++ni) acc[nb][mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b[ni], acc[nb][mi][ni], 0, 0, 0);
+                    for (int nb = 0; nb < NB; ++nb) {
+                        const uint4 bw = make_uint4(hb[nb][4 * j], hb[nb][4 * j + 1], hb[nb][4 * j + 2], hb[nb][4 * j + 3]);
+                        acc[nb][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, __builtin_bit_cast(v8h, bw), acc[nb][mi], 0, 0, 0);
+                    }
                 }
             }
         }
-        __syncthreads();
     }
-    if (!wave_has_rows) return;
     // result register i of lane half g: input row 8 (i / 4) + 4 g + i % 4 of the 32 x 32 tile, weight row r
+    if (col >= rows) return;
 #pragma unroll
-    for (int ni = 0; ni < W; ++ni) {
-        const int col = row0 + (nq * W + ni) * 32 + r;
-        if (col >= rows) continue;
+    for (int mi = 0; mi < MT; ++mi)
 #pragma unroll
-        for (int mi = 0; mi < W; ++mi)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int a = s_asg[(mq * W + mi) * 32 + 8 * (i >> 2) + 4 * g + (i & 3)];
-                if (a < 0) continue;
-                float v = acc[0][mi][ni][i];
-                if (k.gateup) v = v / (1.f + expf(-v)) * acc[NB - 1][mi][ni][i];
-                v = col < row_lim ? v : 0.f;
-                if (k.out_f32) static_cast<float *>(k.out)[int64_t(a) * rows + col] = v;
-                else static_cast<uint16_t *>(k.out)[int64_t(a) * rows + col] = __half_as_ushort(__float2half_rn(v));
-            }
-    }
+        for (int i = 0; i < 16; ++i) {
+            const int a = s_asg[mi * 32 + 8 * (i >> 2) + 4 * g + (i & 3)];
+            if (a < 0) continue;
+            float v = acc[0][mi][i];
+            if (k.gateup) v = v * __builtin_amdgcn_rcpf(1.f + __expf(-v)) * acc[NB - 1][mi][i];
+            v = col < row_lim ? v : 0.f;
+            if (k.out_f32) static_cast<float *>(k.out)[int64_t(a) * rows + col] = v;
+            else static_cast<uint16_t *>(k.out)[int64_t(a) * rows + col] = __half_as_ushort(__float2half_rn(v));
+        }
 }
 
 }  // namespace
 
 template <uint32_t FMT> void F16Launch<FMT>::run(const F16Args & k, bool two_banks, bool wide, dim3 grid, hipStream_t s) {
     if (wide) {
-        if (two_banks) expert_gemm_f16_k<FMT, 2, 2><<<grid, 256, 0, s>>>(k); else expert_gemm_f16_k<FMT, 1, 2><<<grid, 256, 0, s>>>(k);
+        if (two_banks) expert_gemm_f16_k<FMT, 2, 4><<<grid, 256, 0, s>>>(k); else expert_gemm_f16_k<FMT, 1, 4><<<grid, 256, 0, s>>>(k);
     } else {
-        if (two_banks) expert_gemm_f16_k<FMT, 2, 1><<<grid, 256, 0, s>>>(k); else expert_gemm_f16_k<FMT, 1, 1><<<grid, 256, 0, s>>>(k);
+        if (two_banks) expert_gemm_f16_k<FMT, 2, 2><<<grid, 256, 0, s>>>(k); else expert_gemm_f16_k<FMT, 1, 2><<<grid, 256, 0, s>>>(k);
     }
 }
 

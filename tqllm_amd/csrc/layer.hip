@@ -15,6 +15,7 @@ namespace {
 constexpr int kGroupedMin = 64;
 constexpr int kDecodeAssignments = 65535;   // per decode launch
 constexpr int kDecodeDedup = 2048;          // assignments up to which the decode kernels serve an expert's rows together
+constexpr int kGroupedPerBank = 3;          // assignments per expert from which the fp16 grouped products are the faster path
 
 struct Plan {  // byte offsets into the workspace
     bool grouped;   // the grouped products (prefill sizes): int8 for IQ4_XS banks, fp16 for the other formats
@@ -30,10 +31,12 @@ bool int8_ok(const tqmoe_layer & L) { return L.gate.type == TQMOE_IQ4_XS && L.do
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
     const int slots = L.topk + (L.has_shared ? 1 : 0), banks = L.n_expert + (L.has_shared ? 1 : 0);
-    // the int8 grouped products from kGroupedMin tokens; the fp16 ones (other formats) once the decode kernels no longer
-    // read every expert's weights once (they group an expert's rows up to kDecodeDedup assignments a launch)
+    // the int8 grouped products from kGroupedMin tokens; the fp16 ones (other formats) from kGroupedPerBank assignments per
+    // bank matrix on average (measured: the decode kernels' time grows with the assignments, the grouped products' with
+    // the experts they decode, and the two cross at about three assignments per expert), and in any case once the decode
+    // kernels no longer read every expert's weights once (they group an expert's rows up to kDecodeDedup assignments a launch)
     p.int8 = n >= kGroupedMin && int8_ok(L);
-    p.grouped = p.int8 || int64_t(n) * slots > kDecodeDedup;
+    p.grouped = p.int8 || int64_t(n) * slots > std::min<int64_t>(kDecodeDedup, int64_t(kGroupedPerBank) * banks);
     // the grouped products take 2^24 assignments a pass (32-bit block and byte counts stay far from their limits), the
     // decode kernels 65535
     const int64_t per_pass = p.int8 ? int64_t(1) << 24 : p.grouped ? int64_t(65535 - banks) * 64 : kDecodeAssignments;

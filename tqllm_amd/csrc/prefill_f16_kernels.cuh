@@ -196,6 +196,11 @@ __global__ __launch_bounds__(256, 2) void expert_gemm_f16_k(F16Args k) {
     for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(g, S - 1));
     int buf = 0;
     for (int s0 = 0; s0 < s_end; s0 += 2, buf ^= 1) {
+        // the loads of the next stage go out before this stage's conversions: a whole stage to arrive in
+        const RawX next_a = load_x32(k.x, k.xtype, a_at + int64_t(min(s0 + 2 + tp, S - 1)) * 32);
+        typename F16Sub<FMT>::Raw next_b[NB];
+#pragma unroll
+        for (int bb = 0; bb < NB; ++bb) next_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(s0 + 2 + g, S - 1));
         if (a_asg >= 0) {                       // rows without an assignment stay zero
             uint32_t h[16];
             finish_x32(raw_a, k.x, k.xtype, a_at + int64_t(min(s0 + tp, S - 1)) * 32, h);
@@ -213,11 +218,9 @@ __global__ __launch_bounds__(256, 2) void expert_gemm_f16_k(F16Args k) {
         for (int bb = 0; bb < NB; ++bb) {
             F16Sub<FMT>::finish(raw_b[bb], min(s0 + g, S - 1), grid, b_row && s0 + g < s_end, hb[bb]);
         }
-        {
-            raw_a = load_x32(k.x, k.xtype, a_at + int64_t(min(s0 + 2 + tp, S - 1)) * 32);
+        raw_a = next_a;
 #pragma unroll
-            for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(s0 + 2 + g, S - 1));
-        }
+        for (int bb = 0; bb < NB; ++bb) raw_b[bb] = next_b[bb];
         // one barrier per stage: the tile written now was last read two stages ago, before the barrier of the stage between
         __syncthreads();
         // product j of a stage takes weights 8 j .. 8 j + 7 of the lane's sub-block; the input operand of lane (m, g) is the same

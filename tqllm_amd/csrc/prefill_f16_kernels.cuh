@@ -171,7 +171,6 @@ __global__ __launch_bounds__(256, 2) void expert_gemm_f16_k(F16Args k) {
     if (tid < kM) s_asg[tid] = first + tid < cnt ? k.perm[k.offsets[e] + first + tid] : -1;
     for (int i = tid; i < 2 * kM * kPad / 8; i += 256) reinterpret_cast<uint4 *>(&As[0][0][0])[i] = make_uint4(0u, 0u, 0u, 0u);
     __syncthreads();
-    const int m_tiles = min(MT, (cnt - first + 31) / 32);      // 32-row tiles of the block that hold assignments
 
     v16f acc[NB][MT];
 #pragma unroll
@@ -196,11 +195,16 @@ __global__ __launch_bounds__(256, 2) void expert_gemm_f16_k(F16Args k) {
     for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(g, S - 1));
     int buf = 0;
     for (int s0 = 0; s0 < s_end; s0 += 2, buf ^= 1) {
-        // the loads of the next stage go out before this stage's conversions: a whole stage to arrive in
-        const RawX next_a = load_x32(k.x, k.xtype, a_at + int64_t(min(s0 + 2 + tp, S - 1)) * 32);
+        // the loads of the next stage go out before this stage's conversions (a whole stage to arrive in) where the registers
+        // allow a second set, else behind them
+        constexpr bool kEarly = NB * MT < 8;
+        RawX next_a;
         typename F16Sub<FMT>::Raw next_b[NB];
+        if constexpr (kEarly) {
+            next_a = load_x32(k.x, k.xtype, a_at + int64_t(min(s0 + 2 + tp, S - 1)) * 32);
 #pragma unroll
-        for (int bb = 0; bb < NB; ++bb) next_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(s0 + 2 + g, S - 1));
+            for (int bb = 0; bb < NB; ++bb) next_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(s0 + 2 + g, S - 1));
+        }
         if (a_asg >= 0) {                       // rows without an assignment stay zero
             uint32_t h[16];
             finish_x32(raw_a, k.x, k.xtype, a_at + int64_t(min(s0 + tp, S - 1)) * 32, h);
@@ -218,25 +222,37 @@ __global__ __launch_bounds__(256, 2) void expert_gemm_f16_k(F16Args k) {
         for (int bb = 0; bb < NB; ++bb) {
             F16Sub<FMT>::finish(raw_b[bb], min(s0 + g, S - 1), grid, b_row && s0 + g < s_end, hb[bb]);
         }
-        raw_a = next_a;
+        if constexpr (kEarly) {
+            raw_a = next_a;
 #pragma unroll
-        for (int bb = 0; bb < NB; ++bb) raw_b[bb] = next_b[bb];
+            for (int bb = 0; bb < NB; ++bb) raw_b[bb] = next_b[bb];
+        } else {
+            raw_a = load_x32(k.x, k.xtype, a_at + int64_t(min(s0 + 2 + tp, S - 1)) * 32);
+#pragma unroll
+            for (int bb = 0; bb < NB; ++bb) raw_b[bb] = F16Sub<FMT>::load(bb ? k.b1 : k.b0, b_row_at, min(s0 + 2 + g, S - 1));
+        }
         // one barrier per stage: the tile written now was last read two stages ago, before the barrier of the stage between
         __syncthreads();
         // product j of a stage takes weights 8 j .. 8 j + 7 of the lane's sub-block; the input operand of lane (m, g) is the same
         // eight columns 32 g + 8 j .. of input row m (the order of the sum inside a stage is free as long as both agree)
+        // all the block's tiles in straight-line code, also those without assignments (their input rows are zero): a branch per
+        // tile would make every operand read wait by itself, and a second code path costs registers (and occupancy)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
 #pragma unroll
-            for (int mi = 0; mi < MT; ++mi) {
-                if (mi < m_tiles) {
-                    const v8h a = *reinterpret_cast<const v8h *>(&As[buf][mi * 32 + r][32 * g + 8 * j]);
+            for (int m0 = 0; m0 < MT; m0 += 2) {   // two operand reads in flight, then their products
+                constexpr int kPair = MT > 1 ? 2 : 1;
+                v8h a[kPair];
+#pragma unroll
+                for (int mi = 0; mi < kPair; ++mi) a[mi] = *reinterpret_cast<const v8h *>(&As[buf][(m0 + mi) * 32 + r][32 * g + 8 * j]);
+#pragma unroll
+                for (int mi = 0; mi < kPair; ++mi)
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) {
                         const uint4 bw = make_uint4(hb[nb][4 * j], hb[nb][4 * j + 1], hb[nb][4 * j + 2], hb[nb][4 * j + 3]);
-                        acc[nb][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, __builtin_bit_cast(v8h, bw), acc[nb][mi], 0, 0, 0);
+                        acc[nb][m0 + mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], __builtin_bit_cast(v8h, bw), acc[nb][m0 + mi], 0, 0, 0);
                     }
-                }
+                __builtin_amdgcn_sched_barrier(0);   // later reads stay behind these products (reading far ahead spills)
             }
         }
     }

@@ -69,6 +69,34 @@ def test_grouped_f16_products_against_float64(tq, oracle, wtype, n, shared_ff):
         assert synth.errors(y[a], want)[1] < 1.5e-3, a
 
 
+@pytest.mark.parametrize("rows", [40, 200, 333])
+@pytest.mark.parametrize("n,xdtype", [(50, "f32"), (900, "f16"), (900, "bf16")])
+def test_grouped_f16_product_ragged_rows_and_input_types(tq, oracle, rows, n, xdtype):
+    """Weight-row counts that fill the kernel's 128-row blocks only partly, each input type, lists short (64-row blocks) and long
+    (128-row blocks), one input row per token shared by its assignments."""
+    rng = np.random.default_rng(rows + n)
+    experts, cols, k = 5, 512, 2
+    raw = synth.bank_blocks(12, experts * rows, cols, rng)
+    dec = oracle.dequantize(12, raw, experts * rows * cols).reshape(experts, rows, cols).astype(np.float64)
+    bank = tq.ExpertBank(12, raw, experts, rows, cols)
+    ids = np.stack([rng.permutation(experts)[:k] for _ in range(n)]).astype(np.int32)
+    x32 = rng.standard_normal((n, cols)).astype(np.float32)
+    if xdtype == "f32":
+        x, xv = torch.from_numpy(x32).cuda(), x32
+    elif xdtype == "f16":
+        x = torch.from_numpy(x32).cuda().half()
+        xv = x.float().cpu().numpy()
+    else:
+        xb, xv = oracle.to_bf16(x32)
+        x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
+    counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), experts)
+    y = tq.expert_gemm(bank, x, (counts, offsets, perm), n, k, k, out_type=tq.F32).cpu().numpy()
+    flat = ids.reshape(-1)
+    for a in range(0, n * k, 7):
+        want = dec[flat[a]] @ xv[a // k].astype(np.float64)
+        assert synth.errors(y[a], want)[1] < 1.5e-3, a
+
+
 def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, head=None):
     raws = synth.make_banks(cfg, seed=seed, distinct=distinct)
     gate, up, down = banks_on_device(cfg, raws)

@@ -32,10 +32,12 @@ def test_router_logits(tq, oracle, name, n):
     assert np.abs(logits - want).max() < 2e-5
 
 
-@pytest.mark.parametrize("n,e,h,shared", [(32, 512, 2048, True), (100, 33, 512, False), (4096, 512, 2048, True), (77, 64, 192, True)])
+@pytest.mark.parametrize("n,e,h,shared", [(32, 512, 2048, True), (100, 33, 512, False), (4096, 512, 2048, True), (77, 64, 192, True),
+                                          (250, 600, 512, False), (1000, 130, 192, True), (9000, 1100, 256, True)])
 def test_router_gemm_path(tq, oracle, n, e, h, shared):
-    """bf16 router rows and bf16 inputs from 32 tokens up take the matrix-pipe kernel: same logits to the same bar, ragged
-    token and row counts, with and without the shared-gate row; rows of a large batch equal those of a small one."""
+    """bf16 router rows and bf16 inputs take the matrix-pipe kernel from about 120,000 tokens x rows (64-token blocks, 128-token
+    blocks for the largest grids), the wave-per-row kernel below: same logits to the same bar, ragged token and row counts,
+    with and without the shared-gate row; on the matrix-pipe kernel the rows of a large batch equal those of a smaller one."""
     rng = np.random.default_rng(n + e)
     wb, wv = oracle.to_bf16((rng.standard_normal((e, h)) * 0.02).astype(np.float32))
     gb, gv = oracle.to_bf16((rng.standard_normal(h) * 0.02).astype(np.float32))
@@ -49,9 +51,10 @@ def test_router_gemm_path(tq, oracle, n, e, h, shared):
     assert np.abs(got - exact).max() < 3e-6 * max(1.0, np.abs(exact).max() / 2)
     if not shared:
         assert not got[:, e].any()
-    if n >= 45:     # both calls on the matrix-pipe kernel: a row's sum does not depend on the batch around it
-        part = tq.moe_router(dev((wb, wv)), dev((gb, gv)) if shared else None, x[5:5 + 40].contiguous())
-        assert torch.equal(part, logits[5:45])
+    m = -(-130000 // (e + 1))
+    if n >= m + 5:     # both calls on the matrix-pipe kernel: a row's sum does not depend on the batch around it
+        part = tq.moe_router(dev((wb, wv)), dev((gb, gv)) if shared else None, x[5:5 + m].contiguous())
+        assert torch.equal(part, logits[5:5 + m])
 
 
 def test_router_without_shared_gate_and_f16(tq, oracle):

@@ -75,7 +75,9 @@ template <int WT> int32_t launch_router_x(uint32_t xtype, const void * w, const 
 // multiplies a 64 x 32 quadrant: two v_mfma_f32_32x32x16_bf16 per 16 columns.
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-constexpr int kRouterGemmMin = 32;   // token counts from here up (bf16 router and input) take the GEMM
+constexpr int kRouterGemmMin = 120000;   // tokens x router rows from which a bf16 router and input take the GEMM (measured crossover: the
+                                         // GEMM's chain of 64-column stages over the hidden size sets a floor of about 30 us at hidden 2048,
+                                         // the wave-per-row kernel takes 10 us up to 16,000 and grows with tokens x rows)
 constexpr int kRgTok = 128, kRgRows = 64, kRgK = 64, kRgPad = kRgK + 8;   // halves per staged row: 16-byte reads of consecutive rows spread over the banks
 
 __global__ __launch_bounds__(256) void router_gemm_bf16_k(const uint16_t * __restrict__ w, const uint16_t * __restrict__ shared, const uint16_t * __restrict__ x,
@@ -656,7 +658,7 @@ extern "C" int32_t tqmoe_router(const void * router, uint32_t wtype, const void 
     if ((n + kRouterTok - 1) / kRouterTok > 65535) return fail(err, TQMOE_E_ARG, "tqmoe_router: too many tokens for one call");
     if (int32_t rc = need_device(err, "tqmoe_router")) return rc;
     const hipStream_t s = static_cast<hipStream_t>(stream);
-    if (wtype == TQMOE_BF16 && xtype == TQMOE_BF16 && n >= kRouterGemmMin && hidden % 64 == 0) {
+    if (wtype == TQMOE_BF16 && xtype == TQMOE_BF16 && int64_t(n) * (experts + 1) >= kRouterGemmMin && hidden % 64 == 0) {
         const dim3 grid(unsigned((n + kRgTok - 1) / kRgTok), unsigned((experts + 1 + kRgRows - 1) / kRgRows));
         router_gemm_bf16_k<<<grid, 256, 0, s>>>(static_cast<const uint16_t *>(router), static_cast<const uint16_t *>(shared_gate),
                                                                       static_cast<const uint16_t *>(x), logits, hidden, experts, n);

@@ -51,6 +51,30 @@ def test_host_only_entry_points(tq):
     assert lib.tqmoe_dispatch_workspace_bytes(512, 4096, 10) > 0
 
 
+def test_bank_format_ids_and_layouts_agree(tq):
+    """Every bank format of the header's enum has the same GGUF type id in the Python mirror and in the oracle, the same GGUF
+    block size in both, and a device layout whose code and aux sizes follow the header's description."""
+    import oracle
+    text = open(HEADER).read()
+    ids = {m.group(1): int(m.group(2)) for m in re.finditer(r"TQMOE_((?:I?Q\d\w*)|NVFP4G)\s*=\s*(\d+)", text)}
+    assert len(ids) == 16 and ids["IQ4_XS"] == 23 and ids["NVFP4G"] == 323
+    # bytes per 32 weights of the code plane, and of the aux plane per 256 weights (NVFP4G: per 16 weights a byte, plus 4 per row)
+    code_per_sub = {"IQ4_XS": 16, "Q4_K": 16, "Q5_K": 16, "IQ4_NL": 16, "Q4_0": 16, "NVFP4G": 16, "IQ3_S": 12, "IQ3_XXS": 12, "IQ2_S": 12,
+                    "IQ2_XS": 12, "Q3_K": 12, "IQ2_XXS": 8, "Q2_K": 8, "IQ1_S": 8, "Q6_K": 24, "Q8_0": 32}
+    aux_per_256 = {"IQ4_XS": 8, "Q5_K": 48, "Q6_K": 32, "Q3_K": 32, "Q2_K": 32}
+    lib = tq.lib()
+    for name, tid in ids.items():
+        assert getattr(tq, name) == tid and getattr(oracle, name) == tid, name
+        assert tq.api.BLOCK[tid] == oracle.BLOCK[tid], name
+        code, aux = C.c_size_t(), C.c_size_t()
+        err = tq.api._err()
+        rows, cols = 64, 1024
+        assert lib.tqmoe_bank_layout(tid, rows, cols, C.byref(code), C.byref(aux), C.byref(err)) == 0, name
+        assert code.value == rows * cols // 32 * code_per_sub[name], name
+        want_aux = rows * cols // 16 + rows * 4 if name == "NVFP4G" else rows * cols // 256 * aux_per_256.get(name, 16)
+        assert aux.value == want_aux, name
+
+
 def test_errors_are_reported_not_swallowed(tq):
     lib = tq.lib()
     err = tq.api._err()

@@ -51,6 +51,7 @@ _lib.tqo_quantize.argtypes = [C.c_uint32, _p, _p, C.c_int64, C.c_int64]
 _lib.tqo_route.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _p, _p, _p, _p]
 _lib.tqo_route_min_gap_ulps.restype = C.c_double
 _lib.tqo_route_min_gap_ulps.argtypes = [C.c_int, C.c_int, _p]
+_lib.tqo_route_softmax_collision.argtypes = [C.c_int, C.c_int, _p]
 _lib.tqo_shared_weight.restype = C.c_float
 _lib.tqo_shared_weight.argtypes = [C.c_float]
 _lib.tqo_dispatch.argtypes = [_p, C.c_int, C.c_int, _p, _p, _p]
@@ -64,8 +65,6 @@ _lib.tqo_quant_act_row_i8.restype = None
 _lib.tqo_quant_act_row_i8.argtypes = [_p, C.c_int, _p, _p]
 _lib.tqo_quant_act_row_e4m3.restype = None
 _lib.tqo_quant_act_row_e4m3.argtypes = [_p, C.c_int, _p, _p]
-_lib.tqo_widen_i8_256.restype = None
-_lib.tqo_widen_i8_256.argtypes = [_p, _p, _p]
 _lib.tqo_cpu_expert_bench.restype = C.c_double
 _lib.tqo_cpu_expert_bench.argtypes = [C.c_uint32, _p, _p, _p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _p]
 _lib.tqo_hardware_threads.restype = C.c_int
@@ -151,6 +150,12 @@ def route(logits, k, gating=GATE_SOFTMAX, norm=True, scale=1.0, bias=None):
 def route_min_gap_ulps(logits, k):
     lg = np.atleast_2d(_c(logits, np.float32))
     return np.array([_lib.tqo_route_min_gap_ulps(lg.shape[1], k, _ptr(lg[t])) for t in range(lg.shape[0])])
+
+
+def route_softmax_collision(logits, k):
+    """bool per token: the reference's choice rests on a tie of rounded probabilities between different logits"""
+    lg = np.atleast_2d(_c(logits, np.float32))
+    return np.array([bool(_lib.tqo_route_softmax_collision(lg.shape[1], k, _ptr(lg[t]))) for t in range(lg.shape[0])])
 
 
 def shared_weight(logit):

@@ -742,6 +742,26 @@ double tqo_route_min_gap_ulps(int n_expert, int k, const float * logits) {
     return best;
 }
 
+int tqo_route_softmax_collision(int n_expert, int k, const float * logits) {
+    std::vector<float> probs;
+    gate_probs(TQO_GATE_SOFTMAX, n_expert, logits, probs);
+    std::vector<int> order(static_cast<size_t>(n_expert));
+    std::iota(order.begin(), order.end(), 0);
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
+        if (probs[size_t(a)] != probs[size_t(b)]) return probs[size_t(a)] > probs[size_t(b)];
+        return a < b;
+    });
+    int found = 0;
+    for (int s = 0; s < k && s + 1 < n_expert; ++s) {
+        const int a = order[size_t(s)], b = order[size_t(s) + 1];
+        const float pa = probs[size_t(a)], pb = probs[size_t(b)];
+        // a probability below the smallest normal number sits where exp() implementations flush differently
+        if ((pa != 0.f && pa < 1.17549435e-38f) || (pb != 0.f && pb < 1.17549435e-38f)) found = 1;
+        if (pa == pb && pa != 0.f && logits[a] != logits[b]) found = 1;
+    }
+    return found;
+}
+
 float tqo_shared_weight(float logit) { return 1.f / (1.f + std::exp(-logit)); }
 
 int tqo_dispatch(const int32_t * ids, int A, int E, int32_t * counts, int32_t * offsets, int32_t * perm) {
@@ -884,14 +904,6 @@ void tqo_quant_act_row_e4m3(const float * x, int cols, uint8_t * q, float * scal
     for (int i = 0; i < cols; ++i) q[i] = tqo_float_to_e4m3(x[i] * mul);
 }
 
-void tqo_widen_i8_256(const float * w, int8_t * q, float * scale) {
-    float m = 0.f;
-    for (int i = 0; i < 256; ++i) m = std::max(m, std::fabs(w[i]));
-    *scale = m / 127.f;
-    const float mul = m > 0.f ? 127.f / m : 0.f;
-    for (int i = 0; i < 256; ++i) q[i] = int8_t(std::nearbyint(w[i] * mul));
-}
-
 // ------------------------------------------------------------------------------------------------ whole layer
 namespace {
 
@@ -900,15 +912,6 @@ void requant_row_i8(float * x, int cols) {  // x <- dequantised per-row int8 ima
     float s;
     tqo_quant_act_row_i8(x, cols, q.data(), &s);
     for (int i = 0; i < cols; ++i) x[i] = float(q[size_t(i)]) * s;
-}
-
-void widen_matrix_i8(float * w, int64_t n) {
-    int8_t q[256];
-    float s;
-    for (int64_t b = 0; b < n / 256; ++b) {
-        tqo_widen_i8_256(w + b * 256, q, &s);
-        for (int i = 0; i < 256; ++i) w[b * 256 + i] = float(q[i]) * s;
-    }
 }
 
 struct Decoded { std::vector<float> gate, up, down; };
@@ -933,12 +936,6 @@ int decode_expert(const tqo_layer & L, int e, int ff, Decoded & d) {
     for (int r = 0; r < L.hidden; ++r) {
         if (tqo_dequantize(dtype, static_cast<const uint8_t *>(L.down) + dstride * e + row_bytes * r, row.data(), L.ff)) return -1;
         std::copy(row.begin(), row.begin() + ff, d.down.begin() + size_t(r) * ff);
-    }
-    if (L.act_mode == 3) {
-        if (ff % 256 || L.hidden % 256) return -1;
-        widen_matrix_i8(d.gate.data(), int64_t(ff) * L.hidden);
-        widen_matrix_i8(d.up.data(), int64_t(ff) * L.hidden);
-        widen_matrix_i8(d.down.data(), int64_t(L.hidden) * ff);
     }
     return 0;
 }
@@ -972,7 +969,7 @@ int tqo_layer_forward(const tqo_layer * Lp, const float * x, const float * logit
     int elems, bytes;
     if (!tqo_block_layout(L.wtype, &elems, &bytes)) return -1;
     if (L.hidden % elems || L.ff % elems || n <= 0 || L.k <= 0 || L.k > L.n_expert) return -1;
-    if (L.act_mode != 0 && L.act_mode != 1 && L.act_mode != 3 && L.act_mode != 5) return -1;
+    if (L.act_mode != 0 && L.act_mode != 1 && L.act_mode != 5) return -1;
     if (L.has_shared && (L.shared_ff <= 0 || L.shared_ff > L.ff || L.shared_ff % elems)) return -1;
     const int E = L.n_expert, K = L.k, A = n * K, H = L.hidden;
     std::vector<int32_t> ids(static_cast<size_t>(A)), counts(static_cast<size_t>(E)), offsets(size_t(E) + 1), perm(static_cast<size_t>(A));

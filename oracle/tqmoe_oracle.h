@@ -88,6 +88,12 @@ int tqo_route(int gating, int n_expert, int k, int norm_weights, float weight_sc
  * (softmax probabilities as tqo_route computes them); a token with a gap of a few ulp is a near tie, where an
  * exp() that rounds differently may order the pair differently. Equal values (true ties) are skipped. */
 double tqo_route_min_gap_ulps(int n_expert, int k, const float * logits);
+/* 1 when, among the k + 1 largest softmax probabilities as tqo_route computes them (ties to the lower index), two
+ * neighbours have the same nonzero fp32 probability although their logits differ, or one of them is a subnormal number:
+ * the tokens on which a selection by logit (what a kernel with another exp() can reproduce exactly) and the reference's
+ * selection by rounded probability may differ. Equal logits, and probabilities that underflowed to zero, are ordered by
+ * index on both sides and are no collision. */
+int tqo_route_softmax_collision(int n_expert, int k, const float * logits);
 float tqo_shared_weight(float logit);
 
 /* stable dispatch: counts[E], offsets[E + 1] (exclusive scan), perm[A] = assignment indices grouped by expert in
@@ -121,10 +127,10 @@ int tqo_add_rmsnorm(uint16_t * rows, const uint16_t * residual, const float * we
  *   routing of a device run can be replayed on the device's own logits), banks = GGUF blocks [E (+1)][rows][cols]
  *   for gate, up ([F][H]) and down ([H][F]); shared expert = expert index E of the same banks when has_shared,
  *   its FFN size shared_ff <= F (the first shared_ff rows / columns), weighted by sigmoid(logits[.][E]).
- *   act_mode: 0 = fp32 activations (oracle A); 1 = gate/up inputs and down inputs per-row int8 (oracle B of the
- *   int8 path); 2 = per-row E4M3 inputs and weights rounded to E4M3 after a power-of-two row scale (oracle B of the
- *   fp8 path; not implemented); 3 = mode 1 with the weights widened to int8 per (row, 256-weight super-block);
- *   5 = mode 1 with silu(gate) * up and the down product each rounded to fp16 (what the grouped int8 products store).
+ *   act_mode: 0 = fp32 activations (oracle A); 1 = the inputs of both products (the token row, the act row) passed
+ *   through tqo_quant_act_row_i8 (oracle B of an int8 path that keeps fp32 intermediate rows); 5 = mode 1 with
+ *   silu(gate) * up and the down product each rounded to fp16 (oracle B of the grouped int8 products, which store
+ *   fp16 rows).
  *   out fp32 [n][H]; ids_out [n][k], weights_out [n][k] may be null. threads: worker threads over tokens.
  *   gating (0 = softmax), raw_weights (nonzero: unnormalised), weight_scale (0 = none) and bias (or null) are
  *   tqo_route's arguments; all zero is softmax routing with normalised weights.
@@ -142,10 +148,6 @@ typedef struct tqo_layer {
 } tqo_layer;
 int tqo_layer_forward(const tqo_layer * L, const float * x, const float * logits, int n, float * out,
                       int32_t * ids_out, float * weights_out);
-
-/* int8 widening of one decoded weight row segment (256 weights): q = rint(w * 127 / amax), scale = amax / 127
- * (scale 0 and q 0 for an all-zero segment). The declared weight operand of the int8 MFMA path. */
-void tqo_widen_i8_256(const float * w, int8_t * q, float * scale);
 
 /* CPU baseline (port of the reference's tests/bench_cpu_expert_mt.cpp scheme onto an arbitrary bank format):
  * `threads` workers pull experts from an atomic counter; each expert = gate, up, down matvec of one token with

@@ -24,3 +24,16 @@ def banks_on_device(cfg, raws):
 
 def oracle_type(kind):
     return {"f32": oracle.F32, "bf16": oracle.BF16, "f16": oracle.F16}[kind]
+
+
+def clear_tokens(oracle, logits, experts, k, ids=None, want_ids=None, label=""):
+    """Tokens on which the routing ids must equal the reference's bit for bit: all but those where the reference's own
+    choice rests on two different logits rounding to one fp32 probability (or on subnormal probabilities), which no
+    other exp() implementation can be asked to reproduce. Prints how many tokens are exempt and, when the ids are given,
+    how many of the exempt ones actually differ; at most one token in 500 may be exempt."""
+    import numpy as np
+    tie = oracle.route_softmax_collision(logits[:, :experts], k)
+    differ = int((ids[tie] != want_ids[tie]).any(axis=1).sum()) if ids is not None and tie.any() else 0
+    print("%srouting: %d of %d tokens exempt (probability ties between different logits), %d of them differ" % (label and label + ": ", int(tie.sum()), len(tie), differ))
+    assert tie.sum() <= max(1, len(tie) // 500), "too many exempt tokens: pick another seed"
+    return ~tie

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import synth
-from gpu_util import banks_on_device, dev
+from gpu_util import banks_on_device, clear_tokens, dev
 
 pytestmark = pytest.mark.gpu
 
@@ -107,9 +107,7 @@ def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, head=None):
     sel = slice(None) if head is None else slice(0, head)
     want, want_ids, want_w = oracle.layer_forward(inp["x"][1][sel], logits[sel], *raws, cfg["wtype"], cfg["hidden"], cfg["ff"], cfg["experts"],
                                                   cfg["topk"], shared_ff=cfg["shared_ff"], act_mode=0, threads=16)
-    gaps = oracle.route_min_gap_ulps(logits[sel, :cfg["experts"]], cfg["topk"])
-    clear = gaps > 8
-    assert clear.mean() > 0.99
+    clear = clear_tokens(oracle, logits[sel], cfg["experts"], cfg["topk"], ids[sel], want_ids)
     assert np.array_equal(ids[sel][clear], want_ids[clear])
     assert np.abs(w[sel][clear] - want_w[clear]).max() < 3e-6
     mx, rel = synth.errors(out[sel][clear], want[clear])

@@ -257,10 +257,90 @@ def test_declared_quantisers(oracle):
     assert np.array_equal(q, np.rint(x * (np.float32(127) / m)).astype(np.int8))
     q0, s0 = oracle.quant_act_row_i8(np.zeros(64, np.float32))
     assert s0 == 0 and not q0.any()
+    # E4M3 rows: scale amax / 448, every code the nearest E4M3 value of x * (448 / amax), found here by brute force over
+    # the 254 finite codes (ties to the even mantissa), so a truncating or biased conversion fails
     q8, s8 = oracle.quant_act_row_e4m3(x)
-    back = np.array([oracle.e4m3_to_float(b) for b in q8]) * s8
-    assert np.abs(back - x).max() <= m / 448 * 16 + 1e-6      # half a step at the top binade (step 32 of 448)
+    assert s8 == np.float32(m / np.float32(448))
+    codes = np.array([b for b in range(256) if (b & 0x7F) != 0x7F], np.uint8)
+    vals = np.array([oracle.e4m3_to_float(b) for b in codes], np.float64)
+    scaled = (x * (np.float32(448) / m)).astype(np.float32).astype(np.float64)
+    for v, got in zip(scaled, q8):
+        d = np.abs(vals - v)
+        best = codes[np.flatnonzero(d == d.min())]
+        best = [b for b in best if (v < 0) == bool(b & 0x80) or v == 0]
+        want = [b for b in best if not b & 1] if len(best) > 1 else best
+        assert got in want, (v, got, best)
     assert max(oracle.e4m3_to_float(b & 0x7F) for b in q8) == 448.0
+    q0, s0 = oracle.quant_act_row_e4m3(np.zeros(64, np.float32))
+    assert s0 == 0 and not (q0 & 0x7F).any()
+
+
+def _half(a):
+    return np.asarray(a, np.float64).astype(np.float16).astype(np.float64)
+
+
+def _requant_i8(v):
+    """float64 restatement of the per-row int8 quantiser: fp32 scale amax / 127, q = rint(v * (127 / amax)), value q * scale"""
+    v32 = np.asarray(v, np.float64).astype(np.float32)
+    m = np.abs(v32).max()
+    if m == 0:
+        return np.zeros_like(v, np.float64)
+    q = np.rint(v32 * (np.float32(127) / m))
+    return q.astype(np.float64) * np.float64(np.float32(m / np.float32(127)))
+
+
+def test_layer_forward_lossy_operand_modes_against_float64(oracle):
+    """act_mode 1 and 5 of tqo_layer_forward (the gates of the grouped int8 products) rebuilt step by step in float64
+    numpy: per-row int8 on the token row, [mode 5: fp16 rounding of silu(g) * u], per-row int8 on the act row, the down
+    product [mode 5: rounded to fp16], the weighted sum in fp32. The same rebuild with any one of those steps left out
+    must be far from the oracle, so an oracle that skipped a step would fail."""
+    rng = np.random.default_rng(23)
+    h, f, e, k, n = 256, 256, 6, 2, 6
+    for wtype, sf in ((oracle.IQ4_XS, 256), (oracle.Q4_K, 0), (oracle.IQ3_S, 256)):
+        banks = [oracle.quantize(wtype, (rng.standard_normal(((e + 1) * r, c)) * 0.05).astype(np.float32))
+                 for r, c in ((f, h), (f, h), (h, f))]
+        dec = [oracle.dequantize(wtype, b, (e + 1) * f * h).astype(np.float64) for b in banks]
+        wg, wu, wd = dec[0].reshape(e + 1, f, h), dec[1].reshape(e + 1, f, h), dec[2].reshape(e + 1, h, f)
+        x = rng.standard_normal((n, h)).astype(np.float32)
+        logits = rng.standard_normal((n, e + 1)).astype(np.float32)
+
+        def rebuild(ids, w, mode, skip=None):
+            out = np.zeros((n, h))
+            for t in range(n):
+                xq = _requant_i8(x[t]) if skip != "x" else x[t].astype(np.float64)
+
+                def ffn(j, ff):
+                    g, u = wg[j, :ff] @ xq, wu[j, :ff] @ xq
+                    act = g / (1 + np.exp(-g)) * u
+                    if mode == 5 and skip != "act16":
+                        act = _half(act)
+                    if skip != "act":
+                        act = _requant_i8(act)
+                    y = wd[j, :, :ff] @ act
+                    return _half(y) if mode == 5 and skip != "y16" else y
+
+                out[t] = sum(float(w[t, s]) * ffn(ids[t, s], f) for s in range(k))
+                if sf:
+                    out[t] += 1 / (1 + np.exp(-float(logits[t, e]))) * ffn(e, sf)
+            return out
+
+        for mode in (1, 5):
+            got, ids, w = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=sf, act_mode=mode, threads=3)
+            ri, rw = oracle.route(logits[:, :e], k)
+            assert np.array_equal(ids, ri) and np.array_equal(w, rw)
+            want = rebuild(ids, w, mode)
+            tol = 2e-5 * max(1.0, np.abs(want).max())
+            # fp32 sums in the oracle against float64 here: a value on a rounding boundary of the int8 or fp16 steps may
+            # fall the other way, so a few elements may be off by one such step; everything else agrees to fp32 accuracy
+            off = np.abs(got - want) > tol
+            assert off.mean() < 0.01, (wtype, mode, off.mean())
+            assert np.abs(got - want).max() < 5e-4 * np.abs(want).max(), (wtype, mode)
+            for skip in ("x", "act") + (("act16", "y16") if mode == 5 else ()):
+                other = rebuild(ids, w, mode, skip)
+                assert (np.abs(got - other) > tol).mean() > 0.3, (wtype, mode, skip)
+        # the fp32 oracle is none of them either
+        a, _, _ = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=sf, act_mode=0, threads=1)
+        assert (np.abs(a - want) > tol).mean() > 0.5
 
 
 def test_cpu_baseline_kernels_agree_with_decode(oracle, ref):

@@ -174,6 +174,24 @@ __device__ __forceinline__ int wave_min_all(int v) {
     v = min(v, dpp_keep_i<0x143, 0xC>(v));
     return __builtin_amdgcn_readlane(v, 63);
 }
+__device__ __forceinline__ int wave_max_all_i(int v) {
+    v = max(v, dpp_i<kDppXor1>(v));
+    v = max(v, dpp_i<kDppXor2>(v));
+    v = max(v, dpp_i<kDppHalfMirror>(v));
+    v = max(v, dpp_i<kDppMirror>(v));
+    v = max(v, dpp_keep_i<0x142, 0xA>(v));
+    v = max(v, dpp_keep_i<0x143, 0xC>(v));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+// Selection keys of the softmax top-k. The reference orders by rounded probability, ties to the lower index
+// (src/experts/moe.cpp:73-78); exp and the division by the common sum are monotone, so ordering by logit gives the same
+// choice whatever exp() the device has, except where two different logits round to one probability. Entries whose
+// probability underflowed to zero are all tied there and go by index: they share one key below every logit's.
+// A finite float maps to an integer with the same order (-0 counts as +0); the map is its own inverse.
+constexpr int kKeyGone = INT_MIN, kKeyZero = INT_MIN + 1;
+__device__ __forceinline__ int order_key(float x) { const int i = __float_as_int(x + 0.f); return i ^ ((i >> 31) & 0x7FFFFFFF); }
+__device__ __forceinline__ float key_value(int k) { return __int_as_float(k ^ ((k >> 31) & 0x7FFFFFFF)); }
+
 __device__ __forceinline__ float wave_sum_all(float v) {
     v = row_sum16(v);
     v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));
@@ -216,26 +234,31 @@ __global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logi
     float xv[32];
     if (row_in_regs && lane < S) load_block32<XT>(o.x, int64_t(token) * o.cols + 32 * lane, xv);
     const float shared_logit = o.shared_weights ? x[e] : 0.f;
-    float p[R];
-    float m = -INFINITY;
+    int key[R];
+    float m = -INFINITY, sum = 0.f;
+    {
+        float l[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) { const int j = lane + 64 * r; p[r] = j < e ? x[j] : -INFINITY; m = fmaxf(m, p[r]); }
-    m = wave_max_all(m);
-    float sum = 0.f;
+        for (int r = 0; r < R; ++r) { const int j = lane + 64 * r; l[r] = j < e ? x[j] : -INFINITY; m = fmaxf(m, l[r]); }
+        m = wave_max_all(m);
 #pragma unroll
-    for (int r = 0; r < R; ++r) { const int j = lane + 64 * r; p[r] = j < e ? expf(p[r] - m) : 0.f; sum += p[r]; }
-    sum = wave_sum_all(sum);
-#pragma unroll
-    for (int r = 0; r < R; ++r) p[r] = lane + 64 * r < e ? p[r] / sum : -2.f;   // entries past the end never win
+        for (int r = 0; r < R; ++r) {
+            const int j = lane + 64 * r;
+            const float ex = j < e ? expf(l[r] - m) : 0.f;
+            sum += ex;
+            key[r] = j < e ? (ex > 0.f ? order_key(l[r]) : kKeyZero) : kKeyGone;   // entries past the end never win
+        }
+        sum = wave_sum_all(sum);
+    }
     float selected = 0.f, my_w = 0.f;   // lane s keeps selection s
     int my_id = 0;
     for (int s = 0; s < k; ++s) {
-        float bv = p[0];
-        int bi = lane;
+        int bk = key[0], bi = lane;
 #pragma unroll
-        for (int r = 1; r < R; ++r) if (p[r] > bv) { bv = p[r]; bi = lane + 64 * r; }   // strict: the lowest index of equal values
-        const float top = wave_max_all(bv);
-        const int best = wave_min_all(bv == top ? bi : 0x7FFFFFFF);
+        for (int r = 1; r < R; ++r) if (key[r] > bk) { bk = key[r]; bi = lane + 64 * r; }   // strict: the lowest index of equal keys
+        const int topkey = wave_max_all_i(bk);
+        const int best = wave_min_all(bk == topkey ? bi : 0x7FFFFFFF);
+        const float top = topkey == kKeyZero ? 0.f : expf(key_value(topkey) - m) / sum;   // the probability, as every entry's would be computed
         if (lane == (s & 63)) { my_id = best; my_w = top; }
         if (k > 64 && (s & 63) == 63) {   // more selections than lanes: a full set goes out before the lanes are reused
             o.ids[int64_t(token) * k + s - 63 + lane] = my_id;
@@ -244,7 +267,7 @@ __global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logi
         }
         selected += top;                       // slot order, as the host sums the selected weights
 #pragma unroll
-        for (int r = 0; r < R; ++r) if (lane + 64 * r == best) p[r] = -1.f;
+        for (int r = 0; r < R; ++r) if (lane + 64 * r == best) key[r] = kKeyGone;
     }
     if (k <= 64) {
         // the host divides by the clamped sum, then multiplies by the scale
@@ -283,30 +306,29 @@ __global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logi
 
 template <int XT>
 __global__ __launch_bounds__(64) void topk_lds_k(const float * __restrict__ logits, TopkOut o, int e, int k, float scale) {
-    extern __shared__ float probs[];
+    extern __shared__ int keys[];
     const int token = blockIdx.x, lane = threadIdx.x;
     const float * x = logits + int64_t(token) * (e + 1);
     float m = -INFINITY;
     for (int j = lane; j < e; j += 64) m = fmaxf(m, x[j]);
     m = wave_max_all(m);
     float sum = 0.f;
-    for (int j = lane; j < e; j += 64) { const float p = expf(x[j] - m); probs[j] = p; sum += p; }
+    for (int j = lane; j < e; j += 64) { const float ex = expf(x[j] - m); keys[j] = ex > 0.f ? order_key(x[j]) : kKeyZero; sum += ex; }
     sum = wave_sum_all(sum);
-    for (int j = lane; j < e; j += 64) probs[j] = probs[j] / sum;
     float selected = 0.f;
     for (int s = 0; s < k; ++s) {
-        float bv = -INFINITY;
-        int bi = 0x7FFFFFFF;
-        for (int j = lane; j < e; j += 64) if (probs[j] > bv) { bv = probs[j]; bi = j; }
-        const float top = wave_max_all(bv);
-        const int best = wave_min_all(bv == top ? bi : 0x7FFFFFFF);
+        int bk = kKeyGone, bi = 0x7FFFFFFF;
+        for (int j = lane; j < e; j += 64) if (keys[j] > bk) { bk = keys[j]; bi = j; }
+        const int topkey = wave_max_all_i(bk);
+        const int best = wave_min_all(bk == topkey ? bi : 0x7FFFFFFF);
+        const float top = topkey == kKeyZero ? 0.f : expf(key_value(topkey) - m) / sum;
         if (lane == 0) {
             o.ids[int64_t(token) * k + s] = best;
             o.weights[int64_t(token) * k + s] = top;
             if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + s] = best;
         }
         selected += top;
-        if ((best & 63) == lane) probs[best] = -1.f;
+        if ((best & 63) == lane) keys[best] = kKeyGone;
     }
     topk_finish(o, x, token, lane, e, k, scale, selected);
     if (o.image) topk_quantise_row<XT>(o, token, lane);
@@ -721,6 +743,31 @@ extern "C" size_t tqmoe_dispatch_workspace_bytes(int32_t experts, int32_t n, int
     return chunks <= 1 ? 16 : size_t(chunks) * size_t(experts) * sizeof(int);
 }
 
+namespace tqmoe {
+namespace {
+// the launches of tqmoe_dispatch; cc: chunks x experts ints of scratch for more than one chunk
+int32_t enqueue_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets, int32_t * perm, int32_t * groups, int32_t capacity, int32_t experts,
+                         int A, int chunks, int * cc, hipStream_t s, tqmoe_error * err, const char * what) {
+    if (chunks == 1) {
+        dispatch_small_k<<<1, 256, size_t(2 * experts + 1 + 256) * sizeof(int), s>>>(ids, counts, offsets, perm, groups, capacity, A, experts);
+        return launched(err, what);
+    }
+    dispatch_count_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, cc, A, experts);
+    if (experts <= kWideExperts) {
+        const size_t lds = size_t(2 * experts + 1 + 1024 + kWideWaves * experts) * sizeof(int);
+        static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(&dispatch_place_wide_k), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                           int((2 * kWideExperts + 1 + 1024 + kWideWaves * kWideExperts) * sizeof(int)));
+        (void)once;
+        dispatch_place_wide_k<<<unsigned(chunks), 1024, lds, s>>>(ids, cc, counts, offsets, perm, groups, capacity, A, experts, chunks);
+        return launched(err, what);
+    }
+    dispatch_scan_k<<<1, 1024, size_t(experts + 1024) * sizeof(int), s>>>(cc, counts, offsets, chunks, experts);
+    dispatch_place_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, offsets, cc, perm, groups, capacity, A, experts);
+    return launched(err, what);
+}
+}  // namespace
+}  // namespace tqmoe
+
 extern "C" int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets, int32_t * perm, int32_t * groups,
                                   int32_t capacity, int32_t experts, int32_t n, int32_t topk, void * workspace, size_t workspace_bytes,
                                   void * stream, tqmoe_error * err) {
@@ -731,23 +778,7 @@ extern "C" int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t
     const int A = int(A64), chunks = (A + kChunk - 1) / kChunk;
     if (int32_t rc = need_device(err, "tqmoe_dispatch")) return rc;
     const hipStream_t s = static_cast<hipStream_t>(stream);
-    if (chunks == 1) {
-        dispatch_small_k<<<1, 256, size_t(2 * experts + 1 + 256) * sizeof(int), s>>>(ids, counts, offsets, perm, groups, capacity, A, experts);
-        return launched(err, "tqmoe_dispatch");
-    }
-    if (!workspace || workspace_bytes < tqmoe_dispatch_workspace_bytes(experts, n, topk))
+    if (chunks > 1 && (!workspace || workspace_bytes < tqmoe_dispatch_workspace_bytes(experts, n, topk)))
         return fail(err, TQMOE_E_WORKSPACE, "tqmoe_dispatch: workspace of %zu bytes needed", tqmoe_dispatch_workspace_bytes(experts, n, topk));
-    int * cc = static_cast<int *>(workspace);
-    dispatch_count_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, cc, A, experts);
-    if (experts <= kWideExperts) {
-        const size_t lds = size_t(2 * experts + 1 + 1024 + kWideWaves * experts) * sizeof(int);
-        static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(&dispatch_place_wide_k), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                           int((2 * kWideExperts + 1 + 1024 + kWideWaves * kWideExperts) * sizeof(int)));
-        (void)once;
-        dispatch_place_wide_k<<<unsigned(chunks), 1024, lds, s>>>(ids, cc, counts, offsets, perm, groups, capacity, A, experts, chunks);
-        return launched(err, "tqmoe_dispatch");
-    }
-    dispatch_scan_k<<<1, 1024, size_t(experts + 1024) * sizeof(int), s>>>(cc, counts, offsets, chunks, experts);
-    dispatch_place_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, offsets, cc, perm, groups, capacity, A, experts);
-    return launched(err, "tqmoe_dispatch");
+    return enqueue_dispatch(ids, counts, offsets, perm, groups, capacity, experts, A, chunks, static_cast<int *>(workspace), s, err, "tqmoe_dispatch");
 }

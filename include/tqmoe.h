@@ -82,6 +82,16 @@ int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets,
                        int32_t capacity, int32_t experts, int32_t n, int32_t topk, void * workspace,
                        size_t workspace_bytes, void * stream, tqmoe_error * err);
 
+/* tqmoe_dispatch for callers that cannot allocate or carry a workspace (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid allocation). It has no counterpart in the reference. Same lists, same kernels; the
+ * per-chunk counts live in a 4 MiB array inside the library's device image (one copy per GPU, held until the process
+ * ends), whose address is looked up on the first call on a device. Limit: ceil(n * topk / 1024) * experts <= 1,048,576
+ * (for 512 experts about two million assignments), beyond it TQMOE_E_WORKSPACE. Calls on one GPU share that array:
+ * two calls that overlap in time on the same GPU (different streams) race; calls on one stream are ordered. Nothing
+ * in the array needs clearing between calls (every entry a call reads, it has written first). */
+int32_t tqmoe_dispatch_static(const int32_t * ids, int32_t * counts, int32_t * offsets, int32_t * perm, int32_t * groups,
+                              int32_t capacity, int32_t experts, int32_t n, int32_t topk, void * stream, tqmoe_error * err);
+
 /* -------------------------------------------------------------------------------------------------- banks
  * A bank is one projection of every expert: `experts` matrices of rows x cols stacked row-wise, expert e at row
  * e * rows (weight_format.hpp:61 "Stacked weights [experts * rows][cols]"); a non-owning view like tqllm::Mat

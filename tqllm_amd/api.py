@@ -68,6 +68,7 @@ def lib():
         l.tqmoe_dispatch_workspace_bytes.restype = sz
         l.tqmoe_dispatch_workspace_bytes.argtypes = [i32, i32, i32]
         l.tqmoe_dispatch.argtypes = [p, p, p, p, p, i32, i32, i32, i32, p, sz, p, e]
+        l.tqmoe_dispatch_static.argtypes = [p, p, p, p, p, i32, i32, i32, i32, p, e]
         l.tqmoe_bank_layout.argtypes = [u32, i64, i32, C.POINTER(sz), C.POINTER(sz), e]
         l.tqmoe_bank_load.argtypes = [u32, p, i64, i32, p, p, p, p, e]
         l.tqmoe_bank_dequant.argtypes = [C.POINTER(_Bank), i64, i64, p, p, e]
@@ -181,6 +182,14 @@ def moe_dispatch(ids, experts, capacity=0):
     _check(lib().tqmoe_dispatch(_ptr(ids), _ptr(counts), _ptr(offsets), _ptr(perm), _ptr(groups), capacity, experts, n, topk, _ptr(ws),
                                 wsb, _stream(ids), C.byref(err)), err)
     return counts, offsets, perm, groups
+
+
+def moe_dispatch_into(ids, experts, counts, offsets, perm, groups=None, capacity=0):
+    """tqmoe_dispatch_static into tensors the caller already holds: the library's built-in scratch, nothing allocated."""
+    n, topk = ids.shape
+    err = _err()
+    _check(lib().tqmoe_dispatch_static(_ptr(ids), _ptr(counts), _ptr(offsets), _ptr(perm), _ptr(groups), capacity, experts, n, topk,
+                                       _stream(ids), C.byref(err)), err)
 
 
 class ExpertBank:

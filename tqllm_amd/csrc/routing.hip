@@ -1,4 +1,6 @@
 // Router logits, softmax + top-k, and the stable token-to-expert dispatch.
+#include <mutex>
+
 #include "act_image.cuh"
 #include "common.cuh"
 
@@ -743,6 +745,12 @@ extern "C" size_t tqmoe_dispatch_workspace_bytes(int32_t experts, int32_t n, int
     return chunks <= 1 ? 16 : size_t(chunks) * size_t(experts) * sizeof(int);
 }
 
+// Scratch of tqmoe_dispatch_static: the per-chunk counts, in the library's own device image (every GPU the library runs
+// on holds its copy until the process ends). In host code the array's name is not a device address: the address on the
+// current device comes from hipGetSymbolAddress, once per device, and only that pointer is handed to the kernels.
+constexpr int kStaticInts = 1 << 20;                 // 4 MiB: chunks x experts may not exceed it
+static __device__ __align__(256) int scratch[kStaticInts];
+
 namespace tqmoe {
 namespace {
 // the launches of tqmoe_dispatch; cc: chunks x experts ints of scratch for more than one chunk
@@ -765,6 +773,24 @@ int32_t enqueue_dispatch(const int32_t * ids, int32_t * counts, int32_t * offset
     dispatch_place_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, offsets, cc, perm, groups, capacity, A, experts);
     return launched(err, what);
 }
+
+constexpr int kMaxDevices = 64;
+int * g_scratch_ptr[kMaxDevices];                    // address of ::scratch on each device, looked up on first use
+std::mutex g_scratch_mutex;
+
+int32_t static_scratch(int ** out, tqmoe_error * err) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(err, TQMOE_E_DEVICE, "tqmoe_dispatch_static: no usable current device");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void * p = nullptr;
+        const hipError_t rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (rc != hipSuccess || !p) return fail(err, TQMOE_E_DEVICE, "tqmoe_dispatch_static: hipGetSymbolAddress: %s", hipGetErrorString(rc));
+        g_scratch_ptr[dev] = static_cast<int *>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
 }  // namespace
 }  // namespace tqmoe
 
@@ -781,4 +807,18 @@ extern "C" int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t
     if (chunks > 1 && (!workspace || workspace_bytes < tqmoe_dispatch_workspace_bytes(experts, n, topk)))
         return fail(err, TQMOE_E_WORKSPACE, "tqmoe_dispatch: workspace of %zu bytes needed", tqmoe_dispatch_workspace_bytes(experts, n, topk));
     return enqueue_dispatch(ids, counts, offsets, perm, groups, capacity, experts, A, chunks, static_cast<int *>(workspace), s, err, "tqmoe_dispatch");
+}
+
+extern "C" int32_t tqmoe_dispatch_static(const int32_t * ids, int32_t * counts, int32_t * offsets, int32_t * perm, int32_t * groups,
+                                         int32_t capacity, int32_t experts, int32_t n, int32_t topk, void * stream, tqmoe_error * err) {
+    if (!ids || !counts || !offsets || !perm || experts <= 0 || experts > 4096 || n <= 0 || topk <= 0 || (groups && capacity <= 0))
+        return fail(err, TQMOE_E_ARG, "tqmoe_dispatch_static: invalid shape or pointer");
+    const int64_t A64 = int64_t(n) * topk, chunks64 = (A64 + kChunk - 1) / kChunk;
+    if (chunks64 > 1 && chunks64 * experts > kStaticInts)
+        return fail(err, TQMOE_E_WORKSPACE, "tqmoe_dispatch_static: %lld assignments x %d experts need %lld scratch ints, the built-in scratch holds %d "
+                    "(use tqmoe_dispatch with a workspace)", (long long)A64, experts, (long long)(chunks64 * experts), kStaticInts);
+    int * cc = nullptr;
+    if (int32_t rc = static_scratch(&cc, err)) return rc;
+    return enqueue_dispatch(ids, counts, offsets, perm, groups, capacity, experts, int(A64), int(chunks64), cc, static_cast<hipStream_t>(stream), err,
+                            "tqmoe_dispatch_static");
 }

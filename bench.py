@@ -1,19 +1,27 @@
 #!/usr/bin/env python3
-"""MoE-layer benchmark on one MI355X: the Flash-Next-shaped IQ4_XS layer, as decode (configuration 2 of the benchmark definition, the default:
---tokens 16, also 1 and 4) or as prefill (config 3: --tokens 4096, Zipf-skewed routing, int8 MFMA grouped products).
+"""MoE-layer benchmark on one MI355X.
 
-A step is one pass of the whole layer (router, top-k, gate/up + SwiGLU, down + combine, shared expert) over one batch of
-T tokens, with every input already resident in HBM. Steps rotate over several independent expert banks so that the
-weights of a step stream from HBM, not from the 256 MB last-level cache. One JSON line is printed:
-  value     MoE-layer tokens/s (T / mean step time), whole job = this one GPU
-  roofline  the dominant kernel (fused gate/up + SwiGLU) over its mean duration, measured with HIP events around
-            back-to-back launches of that kernel alone: decode = algorithmic bytes of the distinct experts it must read
-            against 8 TB/s; prefill = int8 operations (2 per multiply-add) of its assignments against 5.0 POP/s
-  cpu_baseline  the CPU expert path (port of the reference's tests/bench_cpu_expert_mt.cpp scheme to IQ4_XS at this
-            layer's shape) timed on this box's host cores on a bounded sample
+The default run measures the metric of the benchmark definition, "MoE-layer tokens/s at 1 and 4096 tokens", on the
+Flash-Next-shaped IQ4_XS layer: decode batches of 1 and 16 tokens (configuration 2) and the 4096-token prefill with
+Zipf-skewed routing (configuration 3). The headline fields of the JSON line are the 4096-token point; `points` carries
+every measured point with its own step time, tokens/s, roofline and layer figures. `--config 1|4|5` measures the other
+configurations at their own token counts, `--tokens T` one point only (what the profiling commands use).
+
+A step is one pass of the whole layer (router, top-k, gate/up + SwiGLU, down, combine, shared expert) over one batch of
+T tokens with every input already resident in HBM. Steps rotate over several independent expert banks so that a step's
+weights stream from HBM, not from the 256 MB last-level cache. Per point:
+  tokens_per_s  T / mean step time, a HIP graph of one step per bank replayed
+  roofline      the dominant kernel (gate + up + SwiGLU) over its mean duration, measured with events on the launching
+                stream around back-to-back launches of that kernel alone. Decode kernels: the bytes of the distinct
+                experts the launch must read against 8 TB/s. Grouped products: 2 operations per multiply-add of their
+                assignments against the dense matrix peak of the operand type
+  layer         the whole step's algorithmic bytes and operations against the same peaks
+cpu_baseline: the CPU expert path (the scheme of the reference's tests/bench_cpu_expert_mt.cpp at this layer's shape)
+timed on this box's host cores on a bounded sample.
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -23,139 +31,129 @@ sys.path.insert(0, ROOT)
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")   # measured with rocprofv3 --pmc (see the file)
 HBM_PEAK = 8.0e12  # bytes/s, MI355X published
-INT8_PEAK = 5.0e15  # dense int8 operations/s, MI355X published
-PREFILL_MIN = 64   # token counts from here up take the grouped int8 products inside the library
+PEAK = {"int8": 5.0e15, "fp8": 5.0e15, "fp16": 2.5e15}   # dense matrix operations/s, MI355X published
 ZIPF_S = 1.1
-CFG = dict(hidden=2048, ff=512, experts=512, topk=10, shared_ff=512)
-IQ4_XS_BYTES_PER_WEIGHT = 136.0 / 256.0
+MIN_ROUNDS = 50    # graph replays timed per point at least
+
+# GGUF type ids and block sizes (weights, bytes)
+Q4_K, IQ3_S, IQ4_XS, NVFP4G = 12, 21, 23, 323
+BLOCK = {Q4_K: (256, 144), IQ3_S: (256, 110), IQ4_XS: (256, 136), NVFP4G: (128, 76)}
+CONFIGS = {
+    "2": dict(label="config 2 / 3: Flash-Next-shaped layer, hidden 2048, 512 IQ4_XS experts top-10 + shared (ff 512), bf16 router and activations",
+              hidden=2048, ff=512, experts=512, topk=10, shared_ff=512, wtype=IQ4_XS, fmt="IQ4_XS", rtype="bf16", xtype="bf16",
+              points=(1, 16, 4096), zipf_from=64),
+    "1": dict(label="config 1: hidden 2048, 64 Q4_K experts top-8 (ff 768), fp32 router and activations",
+              hidden=2048, ff=768, experts=64, topk=8, shared_ff=0, wtype=Q4_K, fmt="Q4_K", rtype="f32", xtype="f32", points=(1, 16), zipf_from=None),
+    "4": dict(label="config 4: hidden 2048, 256 IQ3_S experts top-8 (ff 768), bf16 router and activations",
+              hidden=2048, ff=768, experts=256, topk=8, shared_ff=0, wtype=IQ3_S, fmt="IQ3_S", rtype="bf16", xtype="bf16", points=(1, 64, 512),
+              zipf_from=None),
+    "5": dict(label="config 5: hidden 3072, 256 NVFP4 experts top-8 + shared (ff 1536), bf16 router and activations, router logits N(0,1)",
+              hidden=3072, ff=1536, experts=256, topk=8, shared_ff=1536, wtype=NVFP4G, fmt="NVFP4G", rtype="bf16", xtype="bf16", points=(8192,),
+              zipf_from=None, unit_logits=True),
+}
 
 
-def random_iq4xs_bank(torch, experts, rows, cols, gen):
-    """GGUF IQ4_XS block stream of random valid blocks on the device (random codes and sub-scales, small finite fp16
-    super-scales, as the reference's device tests make their banks: tests/moe_device.cu:121-138)."""
-    nb = experts * rows * cols // 256
-    raw = torch.randint(0, 256, (nb, 136), dtype=torch.uint8, device="cuda", generator=gen)
-    d = (torch.rand(nb, device="cuda", generator=gen) * 4e-5 + 4e-5).to(torch.float16)
-    d = d * (torch.randint(0, 2, (nb,), device="cuda", generator=gen) * 2 - 1).to(torch.float16)
-    raw[:, 0:2] = d.view(torch.uint8).reshape(nb, 2)
+def random_bank(torch, wtype, experts, rows, cols, gen):
+    """GGUF block stream of random valid blocks on the device, block scales sized for weights of about 0.02 (random
+    codes and sub-scales, small finite super-scales, as the reference's device tests make their banks:
+    tests/moe_device.cu:121-138, tests/nvfp4_expert.cu:34-50)."""
+    elems, nbytes = BLOCK[wtype]
+    nb = experts * rows * cols // elems
+    raw = torch.randint(0, 256, (nb, nbytes), dtype=torch.uint8, device="cuda", generator=gen)
+
+    def half_field(lo, hi, signed):
+        d = (torch.rand(nb, device="cuda", generator=gen) * (hi - lo) + lo).to(torch.float16)
+        if signed:
+            d = d * (torch.randint(0, 2, (nb,), device="cuda", generator=gen) * 2 - 1).to(torch.float16)
+        return d.view(torch.uint8).reshape(nb, 2)
+
+    if wtype == IQ4_XS:
+        raw[:, 0:2] = half_field(4e-5, 8e-5, True)
+    elif wtype == Q4_K:
+        raw[:, 0:2] = half_field(1e-4, 2e-4, False)
+        raw[:, 2:4] = half_field(1e-4, 2e-4, False)
+    elif wtype == IQ3_S:
+        raw[:, 0:2] = half_field(1.5e-4, 3e-4, True)
+    elif wtype == NVFP4G:
+        per_row = cols // elems
+        g = (torch.rand(experts * rows, device="cuda", generator=gen) * 2e-3 + 5e-4).float()      # one global per row
+        raw[:, 0:4] = g.repeat_interleave(per_row).view(torch.uint8).reshape(nb, 4)
+        raw[:, 4:12] = (0x28 + torch.randint(0, 0x30, (nb, 8), device="cuda", generator=gen)).to(torch.uint8)   # E4M3 0.125 .. 16
     return raw.reshape(-1)
 
 
-def build_layers(torch, tq, banks, tokens, seed):
+def build_banks(torch, tq, cfg, banks, seed):
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
-    h, f, e = CFG["hidden"], CFG["ff"], CFG["experts"] + 1
-    layers, xs = [], []
+    h, f, e = cfg["hidden"], cfg["ff"], cfg["experts"] + (1 if cfg["shared_ff"] else 0)
+    out = []
     for _ in range(banks):
         trio = []
         for rows, cols in ((f, h), (f, h), (h, f)):
-            raw = random_iq4xs_bank(torch, e, rows, cols, gen)
-            trio.append(tq.ExpertBank(tq.IQ4_XS, raw, e, rows, cols))
+            raw = random_bank(torch, cfg["wtype"], e, rows, cols, gen)
+            trio.append(tq.ExpertBank(cfg["wtype"], raw, e, rows, cols))
             del raw
-        skew = tokens >= PREFILL_MIN
-        router = torch.randn((CFG["experts"], h), device="cuda", generator=gen) * (h ** -0.5 if skew else 0.02)
+        out.append(trio)
+    torch.cuda.synchronize()
+    return out, gen
+
+
+def build_point(torch, tq, cfg, trios, gen, tokens):
+    """One layer and one input batch per bank for a point of `tokens` tokens."""
+    h = cfg["hidden"]
+    skew = cfg["zipf_from"] is not None and tokens >= cfg["zipf_from"]
+    unit = skew or cfg.get("unit_logits")
+    rdt = torch.bfloat16 if cfg["rtype"] == "bf16" else torch.float32
+    xdt = torch.bfloat16 if cfg["xtype"] == "bf16" else torch.float32
+    layers, xs = [], []
+    for trio in trios:
+        router = torch.randn((cfg["experts"], h), device="cuda", generator=gen) * (h ** -0.5 if unit else 0.02)
         x = torch.randn((tokens, h), device="cuda", generator=gen)
         if skew:
             # logits = N(0, 1) + ln p_e, p_e ~ rank^-1.1 over a random permutation of the experts: the bias rides in the
             # last router column against a constant 1 in the last activation
-            p = 1.0 / torch.arange(1, CFG["experts"] + 1, device="cuda", dtype=torch.float64) ** ZIPF_S
-            p = (p / p.sum())[torch.randperm(CFG["experts"], device="cuda", generator=gen)]
+            p = 1.0 / torch.arange(1, cfg["experts"] + 1, device="cuda", dtype=torch.float64) ** ZIPF_S
+            p = (p / p.sum())[torch.randperm(cfg["experts"], device="cuda", generator=gen)]
             router[:, -1] = torch.log(p).float()
             x[:, -1] = 1.0
-        sgate = (torch.randn((h,), device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
-        layers.append(tq.MoeLayer(router.to(torch.bfloat16), sgate, *trio, CFG["topk"], shared_ff=CFG["shared_ff"]))
-        xs.append(x.to(torch.bfloat16))
+        sgate = (torch.randn((h,), device="cuda", generator=gen) * 0.02).to(rdt) if cfg["shared_ff"] else None
+        layers.append(tq.MoeLayer(router.to(rdt), sgate, *trio, cfg["topk"], shared_ff=cfg["shared_ff"]))
+        xs.append(x.to(xdt))
     torch.cuda.synchronize()
-    return layers, xs
+    return layers, xs, skew
 
 
-def time_steps(torch, fn, steps, warmup):
+def time_calls(torch, fn, calls, warmup):
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     a.record()
-    for _ in range(steps):
+    for _ in range(calls):
         fn()
     b.record()
     torch.cuda.synchronize()
-    return a.elapsed_time(b) / steps  # ms per call
+    return a.elapsed_time(b) / calls  # ms per call
 
 
-def cpu_baseline(sample_experts=24, budget_s=12.0):
-    """CPU expert path on this box's cores: `sample_experts` IQ4_XS experts (gate, up 512x2048; down 2048x512), one token
-    each, int8 activations per 32-block, all hardware threads pulling experts from a shared counter."""
-    import numpy as np
-
-    import oracle
-    rng = np.random.default_rng(7)
-    h, f = CFG["hidden"], CFG["ff"]
-    banks = []
-    for rows, cols in ((f, h), (f, h), (h, f)):
-        nb = sample_experts * rows * cols // 256
-        raw = rng.integers(0, 256, (nb, 136), dtype=np.uint8)
-        raw[:, 0:2] = np.float16(rng.uniform(4e-5, 8e-5, nb)).view(np.uint8).reshape(nb, 2)
-        banks.append(raw.reshape(-1))
-    # the GPU box reports every core of its host; a job's share is what the affinity mask allows
-    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else oracle.hardware_threads()
-    cores = max(1, min(cores, 64))
-    t0 = time.time()
-    t_pass, _ = oracle.cpu_expert_bench(oracle.IQ4_XS, *banks, h, f, sample_experts, cores, True, reps=1)
-    reps = int(max(1, min(4000, budget_s / max(t_pass, 1e-4) - 2)))   # about budget_s seconds of CPU work
-    t_pass, _ = oracle.cpu_expert_bench(oracle.IQ4_XS, *banks, h, f, sample_experts, cores, True, reps=reps)
-    per_layer_token = t_pass / sample_experts * (CFG["topk"] + 1)
-    return {"value": round(1.0 / per_layer_token, 2), "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": "%d IQ4_XS experts (gate/up 512x2048, down 2048x512), one token, int8 activations per 32-block, %d threads on an "
-                      "atomic expert queue, %d timed passes of %.1f ms; tokens/s = 1 / (11 experts x mean time per expert); %.1f s of CPU work"
-                      % (sample_experts, cores, reps, t_pass * 1e3, time.time() - t0)}
-
-
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None, help="timed steps (default 400; 80 at prefill sizes)")
-    ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--tokens", type=int, default=16, help="decode batch of the step (configuration 2 names 1, 4 and 16)")
-    ap.add_argument("--banks", type=int, default=8, help="independent expert banks the steps rotate over")
-    ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--copy-mb", type=int, default=0, help="also run one plain device copy of this many MiB (a kernel of known "
-                    "traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this command)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing here uses a second GPU)" % args.gpus)
-
-    import torch
-
-    import tqllm_amd as tq
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible; the library has no CPU path")
-    torch.cuda.set_device(0)
-    T, R = args.tokens, args.banks
-    if args.copy_mb > 0:
-        src = torch.empty(args.copy_mb << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
-    if args.steps is None:
-        args.steps = 400 if T < PREFILL_MIN else 80
-    if args.warmup is None:
-        args.warmup = 40 if T < PREFILL_MIN else 8
-    layers, xs = build_layers(torch, tq, R, T, seed=1234)
-    outs = [torch.empty((T, CFG["hidden"]), dtype=torch.float32, device="cuda") for _ in range(R)]
+def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
+    R = len(trios)
+    layers, xs, skew = build_point(torch, tq, cfg, trios, gen, T)
+    h, f, k = cfg["hidden"], cfg["ff"], cfg["topk"]
+    slots = k + (1 if cfg["shared_ff"] else 0)
+    outs = [torch.empty((T, h), dtype=torch.float32, device="cuda") for _ in range(R)]
     for l in layers:
         l.workspace(T)
+    path = layers[0].path(T)
 
-    # ---- whole layer: K steps, rotating banks; a HIP graph of R steps is replayed so that the host is not the bound
+    # ---- whole layer: a HIP graph of one step per bank is replayed so that the host is not the bound
     def eager_round():
         for l, x, o in zip(layers, xs, outs):
             l.forward(x, out=o)
 
-    steps = max(R, args.steps // R * R)
-    warm = max(R, args.warmup // R * R)
-    launch = "eager"
-    round_fn = eager_round
+    rounds = max(MIN_ROUNDS if not args.no_graph else 1, math.ceil(args.steps / R))
+    warm_rounds = max(2, math.ceil(args.warmup / R))
+    launch, round_fn = "eager", eager_round
     if not args.no_graph:
         try:
             eager_round()
@@ -173,8 +171,7 @@ def main():
             round_fn, launch = g.replay, "hipgraph(%d steps)" % R
         except Exception as ex:  # noqa: BLE001
             print("bench.py: HIP graph path unavailable (%s); timing eager launches" % ex, file=sys.stderr)
-    ms_round = time_steps(torch, round_fn, steps // R, warm // R)
-    ms_step = ms_round / R
+    ms_step = time_calls(torch, round_fn, rounds, warm_rounds) / R
 
     # ---- routing statistics of the steps (distinct experts a step must read)
     uniq, routing = [], []
@@ -183,103 +180,168 @@ def main():
         uniq.append(int(torch.unique(ids).numel()))
         routing.append(ids)
     u_mean = sum(uniq) / len(uniq)
-    per_expert = 3 * CFG["ff"] * CFG["hidden"] * IQ4_XS_BYTES_PER_WEIGHT
-    layer_bytes = (u_mean + 1) * per_expert + (CFG["experts"] + 1) * CFG["hidden"] * 2 + T * CFG["hidden"] * 2 * 2
-    slots = CFG["topk"] + 1
-    prefill = T >= PREFILL_MIN
+    bpw = BLOCK[cfg["wtype"]][1] / BLOCK[cfg["wtype"]][0]
+    shared = 1 if cfg["shared_ff"] else 0
+    rbytes = 2 if cfg["rtype"] == "bf16" else 4
+    xbytes = 2 if cfg["xtype"] == "bf16" else 4
+    layer_bytes = (u_mean + shared) * 3 * f * h * bpw + (cfg["experts"] + shared) * h * rbytes + T * h * xbytes * 2
+    gu_bytes = (u_mean + shared) * 2 * f * h * bpw
+    dn_bytes = (u_mean + shared) * f * h * bpw
+    gu_ops = T * slots * 2 * f * h * 2.0      # multiply-adds of gate and up, 2 operations each
+    dn_ops = T * slots * f * h * 2.0
 
     # ---- dominant kernels alone: back-to-back launches over the rotating banks, inputs prepared once
     prep = []
     for l, x, ids in zip(layers, xs, routing):
-        ext = tq.moe_extend_ids(ids, CFG["experts"])
-        if prefill:
-            counts, offsets, perm, _ = tq.moe_dispatch(ext, CFG["experts"] + 1)
-            lists = (counts, offsets, perm)
-            xq, xsc = tq.group_rows_i8(x, lists, T * slots, slots)
-            act = tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, CFG["topk"], CFG["shared_ff"])
-            aq, asc = tq.group_rows_i8(act, lists, T * slots, 1)
-            prep.append((l, lists, xq, xsc, aq, asc))
-        else:
+        ext = tq.moe_extend_ids(ids, cfg["experts"]) if shared else ids
+        if path == "decode":
             img = tq.quant_act(x)
-            act = tq.expert_gateup(l.gate, l.up, img, ext, CFG["topk"], shared_ff=CFG["shared_ff"])
-            y = tq.expert_down(l.down, act, ext, CFG["topk"], shared_ff=CFG["shared_ff"])
+            act = tq.expert_gateup(l.gate, l.up, img, ext, k, shared_ff=cfg["shared_ff"])
+            y = tq.expert_down(l.down, act, ext, k, shared_ff=cfg["shared_ff"])
             prep.append((l, ext, img, act, y))
+        else:
+            counts, offsets, perm, _ = tq.moe_dispatch(ext, cfg["experts"] + shared)
+            lists = (counts, offsets, perm)
+            if path == "grouped_i8":
+                xq, xsc = tq.group_rows_i8(x, lists, T * slots, slots)
+                act = tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, k, cfg["shared_ff"])
+                aq, asc = tq.group_rows_i8(act, lists, T * slots, 1)
+                prep.append((l, lists, xq, xsc, aq, asc))
+            else:
+                act = tq.expert_gemm_gateup(l.gate, l.up, x, lists, T, slots, k, cfg["shared_ff"])
+                prep.append((l, lists, x, act))
 
     def gateup_round():
         for item in prep:
-            if prefill:
-                l, lists, xq, xsc, aq, asc = item
-                tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, CFG["topk"], CFG["shared_ff"])
-            else:
+            if path == "decode":
                 l, ext, img, act, y = item
-                tq.expert_gateup(l.gate, l.up, img, ext, CFG["topk"], shared_ff=CFG["shared_ff"], act_image=act)
+                tq.expert_gateup(l.gate, l.up, img, ext, k, shared_ff=cfg["shared_ff"], act_image=act)
+            elif path == "grouped_i8":
+                l, lists, xq, xsc, aq, asc = item
+                tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, k, cfg["shared_ff"])
+            else:
+                l, lists, x, act = item
+                tq.expert_gemm_gateup(l.gate, l.up, x, lists, T, slots, k, cfg["shared_ff"])
 
     def down_round():
         for item in prep:
-            if prefill:
-                l, lists, xq, xsc, aq, asc = item
-                tq.expert_gemm_i8(l.down, aq, asc, lists, T, slots, CFG["topk"], CFG["shared_ff"])
-            else:
+            if path == "decode":
                 l, ext, img, act, y = item
-                tq.expert_down(l.down, act, ext, CFG["topk"], shared_ff=CFG["shared_ff"], y=y)
+                tq.expert_down(l.down, act, ext, k, shared_ff=cfg["shared_ff"], y=y)
+            elif path == "grouped_i8":
+                l, lists, xq, xsc, aq, asc = item
+                tq.expert_gemm_i8(l.down, aq, asc, lists, T, slots, k, cfg["shared_ff"])
+            else:
+                l, lists, x, act = item
+                tq.expert_gemm(l.down, act, lists, T, slots, k, cfg["shared_ff"], per_expert_input=True, out_type=tq.F32)
 
     kernels = {}
-    reps = 1 if prefill else 4
+    small = path == "decode"
+    reps = 4 if small else 1
     for name, fn in (("gateup", gateup_round), ("down", down_round)):
         fn()
         torch.cuda.synchronize()
         timed = fn
-        if not prefill:   # microsecond kernels: replay a graph of them so that the host is not the bound
+        if small and not args.no_graph:   # microsecond kernels: replay a graph of them so that the host is not the bound
             gk = torch.cuda.CUDAGraph()
             with torch.cuda.graph(gk):
                 for _ in range(reps):
                     fn()
             timed = gk.replay
-        kernels[name] = time_steps(torch, timed, max(4, steps // (reps * R)), 2) / (reps * R)  # ms per launch
-    gu_bytes = (u_mean + 1) * 2 * CFG["ff"] * CFG["hidden"] * IQ4_XS_BYTES_PER_WEIGHT
-    dn_bytes = (u_mean + 1) * CFG["ff"] * CFG["hidden"] * IQ4_XS_BYTES_PER_WEIGHT
-    gu_ops = T * slots * 2 * CFG["ff"] * CFG["hidden"] * 2.0      # int8 multiply-adds of gate and up, 2 operations each
-    dn_ops = T * slots * CFG["ff"] * CFG["hidden"] * 2.0
+        n_calls = max(4, rounds // reps) if small else max(4, min(rounds, 20))
+        kernels[name] = time_calls(torch, timed, n_calls, 2) / ((reps if timed is not fn else 1) * R)  # ms per launch
 
-    if prefill:
-        achieved = gu_ops / (kernels["gateup"] * 1e-3)
-        roofline = {"bound": "mfma", "kernel": "iq4xs_gemm_k<2> (grouped gate + up int8 MFMA product + SwiGLU)", "achieved": round(achieved / 1e12, 2),
-                    "peak": INT8_PEAK / 1e12, "unit": "TFLOP/s", "frac": round(achieved / INT8_PEAK, 4), "traffic": None,
-                    "ops": "int8 multiply-add = 2 operations; peak = dense int8 5.0 POP/s",
-                    "algorithmic_ops_per_launch": int(gu_ops), "us_per_launch": round(kernels["gateup"] * 1e3, 2)}
-        layer = {"algorithmic_ops_per_step": int(gu_ops + dn_ops), "mfma_frac": round((gu_ops + dn_ops) / (ms_step * 1e-3) / INT8_PEAK, 4),
-                 "algorithmic_bytes_per_step": int(layer_bytes), "hbm_frac": round(layer_bytes / (ms_step * 1e-3) / HBM_PEAK, 4),
-                 "down_us": round(kernels["down"] * 1e3, 2), "down_mfma_frac": round(dn_ops / (kernels["down"] * 1e-3) / INT8_PEAK, 4)}
-        workload = ("config 3: Flash-Next-shaped prefill layer, hidden 2048, 512 IQ4_XS experts top-10 + shared (ff 512), T=%d, router logits N(0,1) + "
-                    "Zipf(%.1f) popularity bias, per-row int8 activations" % (T, ZIPF_S))
-        dtype = "int8 x int8 -> int32 MFMA, fp32 scales (IQ4_XS weights exact, per-row int8 activations)"
+    gu_s, dn_s, step_s = kernels["gateup"] * 1e-3, kernels["down"] * 1e-3, ms_step * 1e-3
+    if path == "decode":
+        kname = "iq4xs_mfma_k<2> (gate + up + SwiGLU)" if cfg["wtype"] == IQ4_XS else "gateup_k<%s> (gate + up + SwiGLU)" % cfg["fmt"]
+        roofline = {"bound": "hbm", "kernel": kname, "achieved": round(gu_bytes / gu_s / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                    "frac": round(gu_bytes / gu_s / HBM_PEAK, 4), "traffic": None, "algorithmic_bytes_per_launch": int(gu_bytes),
+                    "us_per_launch": round(gu_s * 1e6, 2)}
+        layer = {"algorithmic_bytes_per_step": int(layer_bytes), "hbm_frac": round(layer_bytes / step_s / HBM_PEAK, 4),
+                 "down_us": round(dn_s * 1e6, 2), "down_hbm_frac": round(dn_bytes / dn_s / HBM_PEAK, 4)}
+        dtype = "int8 x int8 -> int32 (weights exact, activations as two int8 planes), fp32 scales"
     else:
-        achieved = gu_bytes / (kernels["gateup"] * 1e-3)
-        roofline = {"bound": "hbm", "kernel": "iq4xs_mfma_k<2> (gate + up + SwiGLU)", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
-                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4), "traffic": None,
-                    "algorithmic_bytes_per_launch": int(gu_bytes), "us_per_launch": round(kernels["gateup"] * 1e3, 2)}
-        layer = {"algorithmic_bytes_per_step": int(layer_bytes), "hbm_frac": round(layer_bytes / (ms_step * 1e-3) / HBM_PEAK, 4),
-                 "down_us": round(kernels["down"] * 1e3, 2), "down_hbm_frac": round(dn_bytes / (kernels["down"] * 1e-3) / HBM_PEAK, 4)}
-        workload = "config 2: Flash-Next-shaped decode layer, hidden 2048, 512 IQ4_XS experts top-10 + shared (ff 512), T=%d" % T
-        dtype = "int8 x int8 -> int32 MFMA, fp32 scales (IQ4_XS weights exact, bf16 activations as 2 x int8 planes)"
+        op = {"grouped_i8": "int8", "grouped_f16": "fp16", "grouped_fp8": "fp8"}[path]
+        kname = {"grouped_i8": "iq4xs_gemm_k<2> (grouped gate + up int8 MFMA product + SwiGLU)",
+                 "grouped_f16": "expert_gemm_f16_k<%s,2> (grouped gate + up fp16 MFMA product + SwiGLU)" % cfg["fmt"],
+                 "grouped_fp8": "expert_gemm_fp8_k<2> (grouped gate + up fp8 MFMA product + SwiGLU)"}[path]
+        roofline = {"bound": "mfma", "kernel": kname, "achieved": round(gu_ops / gu_s / 1e12, 2), "peak": PEAK[op] / 1e12, "unit": "TFLOP/s",
+                    "frac": round(gu_ops / gu_s / PEAK[op], 4), "traffic": None,
+                    "ops": "multiply-add = 2 operations; peak = dense %s %.1f POP/s" % (op, PEAK[op] / 1e15),
+                    "algorithmic_ops_per_launch": int(gu_ops), "us_per_launch": round(gu_s * 1e6, 2),
+                    "hbm_frac": round(gu_bytes / gu_s / HBM_PEAK, 4)}
+        layer = {"algorithmic_ops_per_step": int(gu_ops + dn_ops), "mfma_frac": round((gu_ops + dn_ops) / step_s / PEAK[op], 4),
+                 "algorithmic_bytes_per_step": int(layer_bytes), "hbm_frac": round(layer_bytes / step_s / HBM_PEAK, 4),
+                 "down_us": round(dn_s * 1e6, 2), "down_mfma_frac": round(dn_ops / dn_s / PEAK[op], 4)}
+        dtype = {"int8": "int8 x int8 -> int32 MFMA (weights exact, per-row int8 activations), fp32 scales",
+                 "fp16": "fp16 x fp16 -> fp32 MFMA (weights and activations rounded to fp16)",
+                 "fp8": "E4M3 x E4M3 -> fp32 MFMA (weights and activations rounded to E4M3), fp32 scales"}[op]
+    # HBM bytes per launch of the roofline kernel as the counters saw them (a committed measurement of this same point)
+    roofline["traffic"] = traffic.get("config%s_tokens_%d" % (key, T), {}).get("bytes_per_launch")
+    del layers, xs, outs, prep
+    torch.cuda.empty_cache()
+    return {"tokens": T, "tokens_per_s": round(T / step_s, 1), "ms_per_step": round(ms_step, 5), "steps": rounds * R, "warmup": warm_rounds * R,
+            "path": path, "launch": launch, "routing": "N(0,1) logits + Zipf(%.1f) popularity bias" % ZIPF_S if skew else "random router",
+            "distinct_experts_per_step": round(u_mean, 1), "dtype": dtype, "roofline": roofline, "layer": layer}
 
-    # HBM bytes per launch of the roofline kernel as the counters saw them (a committed measurement of this same command)
+
+def cpu_baseline(cfg, budget_s=12.0):
+    """CPU expert path on this box's cores at the layer's shape and format (see oracle.cpu_baseline_sweep)."""
+    import oracle
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else oracle.hardware_threads()
+    return oracle.cpu_baseline_sweep(cfg["wtype"], cfg["hidden"], cfg["ff"], cfg["topk"] + (1 if cfg["shared_ff"] else 0), max(1, min(cores, 64)), budget_s)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400, help="timed steps per point; rounded up to whole rounds over the banks, at least %d rounds" % MIN_ROUNDS)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--config", default="2", choices=sorted(CONFIGS), help="benchmark configuration (2 covers configurations 2 and 3)")
+    ap.add_argument("--tokens", type=int, default=None, help="measure this one point instead of the configuration's list")
+    ap.add_argument("--banks", type=int, default=8, help="independent expert banks the steps rotate over")
+    ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-mb", type=int, default=0, help="also run one plain device copy of this many MiB (a kernel of known "
+                    "traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this command)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing here uses a second GPU)" % args.gpus)
+
+    import torch
+
+    import tqllm_amd as tq
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the library has no CPU path")
+    torch.cuda.set_device(0)
+    if args.copy_mb > 0:
+        src = torch.empty(args.copy_mb << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    cfg = CONFIGS[args.config]
     try:
         with open(TRAFFIC_FILE) as f:
-            roofline["traffic"] = json.load(f).get("tokens_%d" % T, {}).get("bytes_per_launch")
+            traffic = json.load(f)
     except (OSError, ValueError):
-        pass
-
+        traffic = {}
+    trios, gen = build_banks(torch, tq, cfg, args.banks, seed=1234)
+    tokens = (args.tokens,) if args.tokens else cfg["points"]
+    points = [measure_point(torch, tq, cfg, args.config, trios, gen, T, args, traffic) for T in tokens]
+    head = points[-1]   # the largest point: 4096 tokens in the default run
     line = {
-        "metric": "MoE-layer tokens/s", "value": round(T / (ms_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
-        "steps": steps, "warmup": warm, "ms_per_step": round(ms_step, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": dtype,
-        "data": "synthetic: random valid IQ4_XS blocks, bf16 router, bf16 N(0,1) activations; %d rotating banks" % R,
-        "config": {"workload": workload, "tokens": T, "launch": launch, "distinct_experts_per_step": round(u_mean, 1)},
-        "roofline": roofline, "layer": layer,
+        "metric": "MoE-layer tokens/s", "value": head["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
+        "steps": head["steps"], "warmup": head["warmup"], "steps_requested": args.steps, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
+        "data": "synthetic: random valid %s blocks (weights of about 0.02), N(0,1) activations; %d rotating banks" % (cfg["fmt"], args.banks),
+        "config": {"workload": "%s; T=%d, %s" % (cfg["label"], head["tokens"], head["routing"]), "tokens": head["tokens"], "launch": head["launch"],
+                   "path": head["path"], "distinct_experts_per_step": head["distinct_experts_per_step"],
+                   "points": "tokens " + ", ".join(str(p["tokens"]) for p in points)},
+        "roofline": head["roofline"], "layer": head["layer"], "points": points,
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline()
+        line["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(line))
 
 

@@ -328,6 +328,13 @@ typedef struct tqmoe_layer {
 } tqmoe_layer;
 
 size_t  tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t n);
+/* Which expert products tqmoe_layer_forward runs for n tokens of this layer (the choice depends on the batch and the
+ * bank formats only, never on the data, so that a token's result does not depend on what else is routed; the reference
+ * makes its switch slot-independent for the same reason, src/models/qwen/qwen4exp/fn_layer_forward.cpp:408-414):
+ * the decode kernels (one read of every distinct expert), the grouped int8 products, or the grouped fp16 products.
+ * Negative: the descriptor is invalid. */
+enum { TQMOE_PATH_DECODE = 0, TQMOE_PATH_GROUPED_I8 = 1, TQMOE_PATH_GROUPED_F16 = 2, TQMOE_PATH_GROUPED_FP8 = 3 };
+int32_t tqmoe_layer_path(const tqmoe_layer * layer, int32_t n);
 /* x: device [n][hidden] of xtype; out: device [n][hidden] of otype (F32 or BF16); ids_out [n][topk], weights_out
  * [n][topk], logits_out [n][n_expert + 1] optional device outputs (NULL to skip). */
 int32_t tqmoe_layer_forward(const tqmoe_layer * layer, const void * x, uint32_t xtype, int32_t n, void * out,

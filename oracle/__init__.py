@@ -67,6 +67,9 @@ _lib.tqo_quant_act_row_e4m3.restype = None
 _lib.tqo_quant_act_row_e4m3.argtypes = [_p, C.c_int, _p, _p]
 _lib.tqo_cpu_expert_bench.restype = C.c_double
 _lib.tqo_cpu_expert_bench.argtypes = [C.c_uint32, _p, _p, _p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _p]
+_lib.tqo_cpu_expert_latency.restype = C.c_double
+_lib.tqo_cpu_expert_latency.argtypes = [C.c_uint32, _p, _p, _p, C.c_int, C.c_int, C.c_int, C.c_int, _p]
+_lib.tqo_cpu_matvec.argtypes = [C.c_uint32, _p, C.c_int, C.c_int, _p, C.c_int, _p]
 _lib.tqo_hardware_threads.restype = C.c_int
 
 
@@ -249,8 +252,86 @@ def cpu_expert_bench(wtype, gate, up, down, hidden, ff, n_expert, threads, int8_
     return t, float(chk[0])
 
 
+def cpu_expert_latency(wtype, gate, up, down, hidden, ff, threads, reps=20):
+    """seconds per expert with the rows of one expert split over persistent workers (int8 activations)"""
+    gate, up, down = (_c(a, np.uint8) for a in (gate, up, down))
+    chk = np.zeros(1, np.float32)
+    t = _lib.tqo_cpu_expert_latency(wtype, _ptr(gate), _ptr(up), _ptr(down), hidden, ff, threads, reps, _ptr(chk))
+    if t < 0:
+        raise ValueError("tqo_cpu_expert_latency: bad configuration")
+    return t, float(chk[0])
+
+
+def cpu_matvec(wtype, w, rows, cols, x, mode):
+    """y [rows] = W x with the baseline's kernels: mode 0 fp32, 1 int8 activations (AVX2), 2 int8 activations (scalar)"""
+    w, x = _c(w, np.uint8), _c(x, np.float32)
+    y = np.empty(rows, np.float32)
+    if _lib.tqo_cpu_matvec(wtype, _ptr(w), rows, cols, _ptr(x), mode, _ptr(y)):
+        raise ValueError("tqo_cpu_matvec: bad configuration")
+    return y
+
+
 def hardware_threads():
     return _lib.tqo_hardware_threads()
+
+
+def random_blocks(wtype, rows, cols, rng):
+    """GGUF blocks of a [rows][cols] matrix: random codes and sub-scales, block scales sized for weights of about 0.02"""
+    elems, nbytes = BLOCK[wtype]
+    nb = rows * cols // elems
+    raw = rng.integers(0, 256, (nb, nbytes), dtype=np.uint8)
+    if wtype == NVFP4G:
+        g = np.repeat(rng.uniform(5e-4, 2.5e-3, rows).astype(np.float32), cols // elems)
+        raw[:, 0:4] = g.view(np.uint8).reshape(nb, 4)
+        raw[:, 4:12] = 0x28 + rng.integers(0, 0x30, (nb, 8), dtype=np.uint8)
+    else:
+        lo, hi = {IQ4_XS: (4e-5, 8e-5), IQ4_NL: (1.5e-4, 3e-4), Q4_K: (1e-4, 2e-4), IQ3_S: (1.5e-4, 3e-4)}[wtype]
+        raw[:, 0:2] = np.float16(rng.uniform(lo, hi, nb)).view(np.uint8).reshape(nb, 2)
+        if wtype == Q4_K:
+            raw[:, 2:4] = np.float16(rng.uniform(lo, hi, nb)).view(np.uint8).reshape(nb, 2)
+    return raw.reshape(-1)
+
+
+def cpu_baseline_sweep(wtype, hidden, ff, experts_per_token, cores, budget_s=12.0, sample_experts=24):
+    """The CPU expert path on this machine's cores, as the reference's tests/bench_cpu_expert_mt.cpp runs it: thread counts
+    1, 2, 4, ... up to `cores`, fp32 and int8-activation variants over `sample_experts` experts of the layer's shape pulled
+    from an atomic queue; then the rows of one expert split over persistent workers. Returns the benchmark's cpu_baseline
+    record: value = MoE-layer tokens/s of the best (threads, variant) = 1 / (experts_per_token x its mean time per expert)."""
+    import time
+    rng = np.random.default_rng(7)
+    banks = [random_blocks(wtype, sample_experts * rows, cols, rng) for rows, cols in ((ff, hidden), (ff, hidden), (hidden, ff))]
+    expert_bytes = sum(b.size for b in banks) / sample_experts
+    t_start = time.time()
+    counts = sorted({min(cores, 1 << i) for i in range(cores.bit_length() + 1)} | {cores})
+    sweep, best = [], None
+    for nt in counts:
+        for int8 in (False, True):
+            t_pass, _ = cpu_expert_bench(wtype, *banks, hidden, ff, sample_experts, nt, int8, reps=2)
+            row = {"threads": nt, "variant": "int8" if int8 else "fp32", "ms_per_expert": round(t_pass / sample_experts * 1e3, 4),
+                   "gb_per_s": round(expert_bytes * sample_experts / t_pass / 1e9, 2)}
+            sweep.append(row)
+            if best is None or t_pass < best[0]:
+                best = (t_pass, nt, int8)
+    # the best setting again, for what is left of the budget
+    spent = time.time() - t_start
+    reps = int(max(3, min(4000, (budget_s - spent) / max(best[0], 1e-4))))
+    t_pass, _ = cpu_expert_bench(wtype, *banks, hidden, ff, sample_experts, best[1], best[2], reps=reps)
+    per_expert = t_pass / sample_experts
+    one = [b[: b.size // sample_experts] for b in banks]
+    latency = {}
+    for nt in counts:
+        t_one, _ = cpu_expert_latency(wtype, *one, hidden, ff, nt, reps=30)
+        latency[str(nt)] = round(t_one * 1e3, 4)
+    name = {IQ4_XS: "IQ4_XS", IQ4_NL: "IQ4_NL", Q4_K: "Q4_K", IQ3_S: "IQ3_S", NVFP4G: "NVFP4G"}[wtype]
+    return {"value": round(1.0 / (per_expert * experts_per_token), 2), "unit": "tokens/s", "cores": best[1], "kind": "port",
+            "variant": "int8" if best[2] else "fp32", "ms_per_expert": round(per_expert * 1e3, 4),
+            "gb_per_s": round(expert_bytes / per_expert / 1e9, 2), "cores_available": cores,
+            "sample": "%d %s experts (gate/up %dx%d, down %dx%d), one token each, workers on an atomic expert queue, thread counts %s x {fp32, "
+                      "int8 activations per 32-block with AVX2 integer dots}; value = best setting (%d threads, %s) re-timed over %d passes: "
+                      "tokens/s = 1 / (%d experts x mean time per expert); %.1f s of CPU work"
+                      % (sample_experts, name, ff, hidden, hidden, ff, counts, best[1], "int8" if best[2] else "fp32", reps, experts_per_token,
+                         time.time() - t_start),
+            "sweep": sweep, "row_split_ms_per_expert": latency}
 
 
 def ref_lib():

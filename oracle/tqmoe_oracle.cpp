@@ -8,11 +8,14 @@
 #include "iq2xs_lattice.h"
 #include "iq1s_lattice.h"
 
+#include <immintrin.h>
+
 #include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <cmath>
 #include <cstring>
+#include <functional>
 #include <limits>
 #include <mutex>
 #include <numeric>
@@ -1025,50 +1028,124 @@ int tqo_layer_forward(const tqo_layer * Lp, const float * x, const float * logit
 }
 
 // ---------------------------------------------------------------------------------------------- CPU baseline
-// Scheme of the reference's tests/bench_cpu_expert_mt.cpp:69-116 (workers pull whole experts from an atomic counter,
-// gate -> up -> down per expert, one warm pass, `reps` timed passes), on this build's bank formats. The int8 variant
-// quantises the input per 32-block (scale amax/127) and takes integer dots with the block's integer codes, as
-// src/experts/cpu_expert_matvec.cpp:200-280 does for IQ4_NL; the fp32 variant decodes and multiplies in fp32.
+// Scheme of the reference's tests/bench_cpu_expert_mt.cpp: table 1 (:69-116) has workers pull whole experts from an
+// atomic counter, gate -> up -> down per expert, one warm pass, `reps` timed passes, for thread counts 1, 2, 4, ...;
+// table 2 (:130-199) splits the rows of ONE expert's three matrices over persistent workers woken by a generation
+// counter (single-expert latency). Both on this build's bank formats. The int8 variant quantises the input per
+// 32-block (scale amax / 127) and takes integer dots with the block's integer codes on AVX2 (unsigned x signed byte
+// products summed in pairs, then widened: the instruction pair the reference's K-quant dots use,
+// src/experts/cpu_kquant.cpp:85-101, 154-172; its IQ4_NL kernel, src/experts/cpu_expert_matvec.cpp:200-280, takes the
+// 16-bit route to the same sums). The fp32 variant decodes a block and multiplies in fp32 (eight partial sums).
 namespace {
 
-// integer image of one 32-weight block: w = scale * q + offset (offset only for Q4_K)
-struct BlockI8 { int8_t q[32]; float scale, offset; };
+// integer image of one 32-weight block: w[i] = scale[i / 16] * q[i] + offset
+struct BlockI8 { int8_t q[32]; float scale[2], offset; };
 
-inline void block_image(uint32_t type, const uint8_t * super, int ib, BlockI8 & o) {
+// scalar decode of a block's integer codes: every format the baseline runs (the vector decoders below are checked against it)
+inline void block_image(uint32_t type, const uint8_t * blk, int ib, BlockI8 & o) {
     o.offset = 0.f;
     switch (type) {
         case TQO_IQ4_XS: {
-            o.scale = tqo_half_to_float(rd16(super)) * float(iq4xs_subscale(super, ib) - 32);
-            const uint8_t * q = super + 8 + 16 * ib;
+            o.scale[0] = o.scale[1] = tqo_half_to_float(rd16(blk)) * float(iq4xs_subscale(blk, ib) - 32);
+            const uint8_t * q = blk + 8 + 16 * ib;
             for (int j = 0; j < 16; ++j) { o.q[j] = kIq4Values[q[j] & 15]; o.q[16 + j] = kIq4Values[q[j] >> 4]; }
             break;
         }
         case TQO_IQ4_NL: {
-            o.scale = tqo_half_to_float(rd16(super));
-            for (int j = 0; j < 16; ++j) { o.q[j] = kIq4Values[super[2 + j] & 15]; o.q[16 + j] = kIq4Values[super[2 + j] >> 4]; }
+            o.scale[0] = o.scale[1] = tqo_half_to_float(rd16(blk));
+            for (int j = 0; j < 16; ++j) { o.q[j] = kIq4Values[blk[2 + j] & 15]; o.q[16 + j] = kIq4Values[blk[2 + j] >> 4]; }
             break;
         }
         case TQO_Q4_K: {
             int sc, mn;
-            q4k_scale_min(super + 4, ib, sc, mn);
-            o.scale = tqo_half_to_float(rd16(super)) * float(sc);
-            o.offset = -(tqo_half_to_float(rd16(super + 2)) * float(mn));
-            const uint8_t * q = super + 16 + 32 * (ib / 2);
+            q4k_scale_min(blk + 4, ib, sc, mn);
+            o.scale[0] = o.scale[1] = tqo_half_to_float(rd16(blk)) * float(sc);
+            o.offset = -(tqo_half_to_float(rd16(blk + 2)) * float(mn));
+            const uint8_t * q = blk + 16 + 32 * (ib / 2);
             for (int l = 0; l < 32; ++l) o.q[l] = int8_t((ib & 1) ? q[l] >> 4 : q[l] & 15);
             break;
         }
         case TQO_IQ3_S: {
-            o.scale = tqo_half_to_float(rd16(super)) * float(1 + 2 * ((super[106 + ib / 2] >> (4 * (ib & 1))) & 15));
+            o.scale[0] = o.scale[1] = tqo_half_to_float(rd16(blk)) * float(1 + 2 * ((blk[106 + ib / 2] >> (4 * (ib & 1))) & 15));
             for (int w = 0; w < 8; ++w) {
-                const uint32_t g = tq_iq3s_point(super[2 + 8 * ib + w] | (((super[66 + ib] >> w) & 1) << 8));
-                const int sg = super[74 + 4 * ib + w / 2] >> (4 * (w & 1));
+                const uint32_t g = tq_iq3s_point(blk[2 + 8 * ib + w] | (((blk[66 + ib] >> w) & 1) << 8));
+                const int sg = blk[74 + 4 * ib + w / 2] >> (4 * (w & 1));
                 for (int j = 0; j < 4; ++j) { const int m = (g >> (8 * j)) & 255; o.q[4 * w + j] = int8_t(((sg >> j) & 1) ? -m : m); }
             }
             break;
         }
-        default: {  // NVFP4G: two 16-groups per 32 weights are handled by the caller through the fp32 path
-            o.scale = 0.f;
-            std::memset(o.q, 0, 32);
+        default: {  // NVFP4G (128-weight block): q = 2 * e2m1, one scale per 16 weights
+            float g;
+            std::memcpy(&g, blk, 4);
+            for (int h = 0; h < 2; ++h) {
+                o.scale[h] = 0.5f * (tqo_e4m3_to_float(blk[4 + 2 * ib + h]) * g);
+                for (int i = 0; i < 8; ++i) {
+                    const uint8_t c = blk[12 + 8 * (2 * ib + h) + i];
+                    o.q[16 * h + 2 * i] = int8_t(std::lrintf(2.f * kE2M1[c & 15]));
+                    o.q[16 * h + 2 * i + 1] = int8_t(std::lrintf(2.f * kE2M1[c >> 4]));
+                }
+            }
+        }
+    }
+}
+
+// the same block as a 32-byte vector (AVX2)
+struct Iq3Table { uint32_t v[512]; Iq3Table() { for (int i = 0; i < 512; ++i) v[i] = tq_iq3s_point(i); } };
+inline __m256i block_codes_avx2(uint32_t type, const uint8_t * blk, int ib) {
+    switch (type) {
+        case TQO_IQ4_XS: case TQO_IQ4_NL: {
+            const __m128i table = _mm_loadu_si128(reinterpret_cast<const __m128i *>(kIq4Values));
+            const __m128i q = _mm_loadu_si128(reinterpret_cast<const __m128i *>(type == TQO_IQ4_XS ? blk + 8 + 16 * ib : blk + 2));
+            const __m128i m4 = _mm_set1_epi8(15);
+            return _mm256_set_m128i(_mm_shuffle_epi8(table, _mm_and_si128(_mm_srli_epi16(q, 4), m4)), _mm_shuffle_epi8(table, _mm_and_si128(q, m4)));
+        }
+        case TQO_Q4_K: {
+            const __m256i q = _mm256_loadu_si256(reinterpret_cast<const __m256i *>(blk + 16 + 32 * (ib / 2)));
+            return _mm256_and_si256((ib & 1) ? _mm256_srli_epi16(q, 4) : q, _mm256_set1_epi8(15));
+        }
+        case TQO_IQ3_S: {
+            static const Iq3Table table;
+            // eight lattice indices: the byte, and bit w of the sub-block's qh byte as bit 8
+            const __m256i low = _mm256_cvtepu8_epi32(_mm_loadl_epi64(reinterpret_cast<const __m128i *>(blk + 2 + 8 * ib)));
+            const __m256i bit = _mm256_and_si256(_mm256_srlv_epi32(_mm256_set1_epi32(blk[66 + ib]), _mm256_setr_epi32(0, 1, 2, 3, 4, 5, 6, 7)), _mm256_set1_epi32(1));
+            const __m256i mag = _mm256_i32gather_epi32(reinterpret_cast<const int *>(table.v), _mm256_or_si256(low, _mm256_slli_epi32(bit, 8)), 4);
+            // sign bit 4 w + j of the sub-block's 32 sign bits belongs to byte 4 w + j: spread the four sign bytes over the
+            // vector, pick each byte's bit, and negate where it is set
+            uint32_t sg;
+            std::memcpy(&sg, blk + 74 + 4 * ib, 4);
+            const __m256i bytes = _mm256_shuffle_epi8(_mm256_set1_epi32(int(sg)), _mm256_setr_epi8(0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1, 1, 1, 2, 2, 2, 2, 2, 2, 2, 2, 3, 3, 3, 3, 3, 3, 3, 3));
+            const __m256i pick = _mm256_set1_epi64x(int64_t(0x8040201008040201ull));
+            const __m256i neg = _mm256_cmpeq_epi8(_mm256_and_si256(bytes, pick), pick);
+            return _mm256_sub_epi8(_mm256_xor_si256(mag, neg), neg);
+        }
+        default: {  // NVFP4G: byte i of a group = weights 2 i (low nibble) and 2 i + 1
+            static const int8_t two_e2m1[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+            const __m128i table = _mm_loadu_si128(reinterpret_cast<const __m128i *>(two_e2m1));
+            const __m128i q = _mm_loadu_si128(reinterpret_cast<const __m128i *>(blk + 12 + 16 * ib));
+            const __m128i m4 = _mm_set1_epi8(15);
+            const __m128i even = _mm_shuffle_epi8(table, _mm_and_si128(q, m4)), odd = _mm_shuffle_epi8(table, _mm_and_si128(_mm_srli_epi16(q, 4), m4));
+            return _mm256_set_m128i(_mm_unpackhi_epi8(even, odd), _mm_unpacklo_epi8(even, odd));
+        }
+    }
+}
+inline float half_hw(const uint8_t * p) { return _cvtsh_ss(rd16(p)); }   // the hardware conversion (equal to tqo_half_to_float on all 65,536 halves)
+inline void block_scales(uint32_t type, const uint8_t * blk, int ib, float (&scale)[2], float & offset) {
+    offset = 0.f;
+    switch (type) {
+        case TQO_IQ4_XS: scale[0] = scale[1] = half_hw(blk) * float(iq4xs_subscale(blk, ib) - 32); break;
+        case TQO_IQ4_NL: scale[0] = scale[1] = half_hw(blk); break;
+        case TQO_Q4_K: {
+            int sc, mn;
+            q4k_scale_min(blk + 4, ib, sc, mn);
+            scale[0] = scale[1] = half_hw(blk) * float(sc);
+            offset = -(half_hw(blk + 2) * float(mn));
+            break;
+        }
+        case TQO_IQ3_S: scale[0] = scale[1] = half_hw(blk) * float(1 + 2 * ((blk[106 + ib / 2] >> (4 * (ib & 1))) & 15)); break;
+        default: {
+            float g;
+            std::memcpy(&g, blk, 4);
+            for (int h = 0; h < 2; ++h) scale[h] = 0.5f * (tqo_e4m3_to_float(blk[4 + 2 * ib + h]) * g);
         }
     }
 }
@@ -1090,45 +1167,141 @@ void quant_x_blocks(const float * x, int cols, XQ & o) {
     }
 }
 
-void matvec(uint32_t type, const uint8_t * W, int rows, int cols, const float * x, const XQ * xq, float * y) {
+inline float hsum8(__m256 v) {
+    __m128 s = _mm_add_ps(_mm256_castps256_ps128(v), _mm256_extractf128_ps(v, 1));
+    s = _mm_add_ps(s, _mm_movehl_ps(s, s));
+    s = _mm_add_ss(s, _mm_shuffle_ps(s, s, 1));
+    return _mm_cvtss_f32(s);
+}
+
+// rows [r0, r1) of y = W x. mode 0: fp32 (decode, fp32 products, eight partial sums); 1: int8 activations, AVX2 integer
+// dots; 2: int8 activations, scalar integer dots (the check of mode 1)
+__attribute__((optimize("O3"))) void matvec_rows(uint32_t type, const uint8_t * W, int cols, const float * x, const XQ * xq, int mode, int r0, int r1, float * y) {
     int elems, bytes;
     tqo_block_layout(type, &elems, &bytes);
     const size_t row_bytes = size_t(cols / elems) * bytes;
-    std::vector<float> dec(static_cast<size_t>(elems));
-    for (int r = 0; r < rows; ++r) {
+    const __m256i ones = _mm256_set1_epi16(1);
+    std::vector<float> xsum;   // fp32 path: the sum of every 32-block of x (what a block's offset multiplies)
+    if (mode == 0) {
+        xsum.resize(size_t(cols / 32));
+        for (int b = 0; b < cols / 32; ++b) { float t = 0.f; for (int i = 0; i < 32; ++i) t += x[32 * b + i]; xsum[size_t(b)] = t; }
+    }
+    for (int r = r0; r < r1; ++r) {
         const uint8_t * row = W + row_bytes * r;
-        float acc = 0.f;
-        if (xq && type != TQO_NVFP4G) {
+        float result;
+        if (mode == 1) {
+            __m256 acc = _mm256_setzero_ps();
+            float off = 0.f;
+            for (int b = 0; b < cols / 32; ++b) {
+                const uint8_t * blk = row + size_t((32 * b) / elems) * bytes;
+                const int ib = (32 * b % elems) / 32;
+                float sc[2], offset;
+                block_scales(type, blk, ib, sc, offset);
+                const __m256i w = block_codes_avx2(type, blk, ib);
+                const __m256i q = _mm256_loadu_si256(reinterpret_cast<const __m256i *>(xq->q.data() + 32 * b));
+                // |w| as the unsigned operand, q with w's sign as the signed one: pair sums stay below 2^15 (|w|, |q| <= 127)
+                const __m256i dot = _mm256_madd_epi16(_mm256_maddubs_epi16(_mm256_sign_epi8(w, w), _mm256_sign_epi8(q, w)), ones);
+                const float xs = xq->scale[size_t(b)];
+                const __m256 scale = _mm256_set_m128(_mm_set1_ps(sc[1] * xs), _mm_set1_ps(sc[0] * xs));   // weights 0..15 in the low half
+                acc = _mm256_fmadd_ps(_mm256_cvtepi32_ps(dot), scale, acc);
+                off += offset * (xs * float(xq->sum[size_t(b)]));
+            }
+            result = hsum8(acc) + off;
+        } else if (mode == 2) {
+            float acc = 0.f;
             BlockI8 bi;
             for (int b = 0; b < cols / 32; ++b) {
-                const uint8_t * super = row + size_t((32 * b) / elems) * bytes;
-                block_image(type, super, (32 * b % elems) / 32, bi);
+                const uint8_t * blk = row + size_t((32 * b) / elems) * bytes;
+                block_image(type, blk, (32 * b % elems) / 32, bi);
                 const int8_t * q = xq->q.data() + 32 * b;
-                int dot = 0;
-                for (int i = 0; i < 32; ++i) dot += int(bi.q[i]) * int(q[i]);
-                acc += xq->scale[size_t(b)] * (bi.scale * float(dot) + bi.offset * float(xq->sum[size_t(b)]));
+                int d0 = 0, d1 = 0;
+                for (int i = 0; i < 16; ++i) { d0 += int(bi.q[i]) * int(q[i]); d1 += int(bi.q[16 + i]) * int(q[16 + i]); }
+                acc += xq->scale[size_t(b)] * (bi.scale[0] * float(d0) + bi.scale[1] * float(d1) + bi.offset * float(xq->sum[size_t(b)]));
             }
+            result = acc;
         } else {
-            for (int b = 0; b < cols / elems; ++b) {
-                tqo_dequantize(type, row + size_t(b) * bytes, dec.data(), elems);
-                float part = 0.f;
-                for (int i = 0; i < elems; ++i) part += dec[size_t(i)] * x[b * elems + i];
-                acc += part;
+            // fp32: the block's integer codes widened to fp32, four fused multiply-adds of eight products each, then the block's
+            // scale (w = scale * q + offset, so the offset meets the plain sum of the block's x)
+            __m256 acc = _mm256_setzero_ps();
+            float off = 0.f;
+            for (int b = 0; b < cols / 32; ++b) {
+                const uint8_t * blk = row + size_t((32 * b) / elems) * bytes;
+                const int ib = (32 * b % elems) / 32;
+                float sc[2], offset;
+                block_scales(type, blk, ib, sc, offset);
+                const __m256i w = block_codes_avx2(type, blk, ib);
+                const __m128i lo = _mm256_castsi256_si128(w), hi = _mm256_extracti128_si256(w, 1);
+                const float * xb = x + 32 * b;
+                __m256 p0 = _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi8_epi32(lo)), _mm256_loadu_ps(xb));
+                p0 = _mm256_fmadd_ps(_mm256_cvtepi32_ps(_mm256_cvtepi8_epi32(_mm_srli_si128(lo, 8))), _mm256_loadu_ps(xb + 8), p0);
+                __m256 p1 = _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi8_epi32(hi)), _mm256_loadu_ps(xb + 16));
+                p1 = _mm256_fmadd_ps(_mm256_cvtepi32_ps(_mm256_cvtepi8_epi32(_mm_srli_si128(hi, 8))), _mm256_loadu_ps(xb + 24), p1);
+                acc = _mm256_fmadd_ps(p0, _mm256_set1_ps(sc[0]), acc);
+                acc = _mm256_fmadd_ps(p1, _mm256_set1_ps(sc[1]), acc);
+                if (offset != 0.f) off += offset * xsum[size_t(b)];
             }
+            result = hsum8(acc) + off;
         }
-        y[r] = acc;
+        y[r] = result;
     }
 }
+
+bool baseline_type(uint32_t t) { return t == TQO_IQ4_XS || t == TQO_IQ4_NL || t == TQO_Q4_K || t == TQO_IQ3_S || t == TQO_NVFP4G; }
+
+// persistent workers woken by a generation counter (tests/bench_cpu_expert_mt.cpp:130-165); worker 0 is the caller
+struct RowPool {
+    std::vector<std::thread> th;
+    std::atomic<long> gen{0};
+    std::atomic<int> done{0};
+    std::atomic<bool> stop{false};
+    const std::function<void(int)> * work = nullptr;
+    int n;
+    explicit RowPool(int n_) : n(n_) {
+        for (int i = 1; i < n; ++i) th.emplace_back([this, i]() {
+            long seen = 0;
+            for (;;) {
+                const long g = gen.load(std::memory_order_acquire);
+                if (g == seen) { if (stop.load(std::memory_order_acquire)) return; std::this_thread::yield(); continue; }
+                seen = g;
+                if (stop.load(std::memory_order_acquire)) return;
+                (*work)(i);
+                done.fetch_add(1, std::memory_order_release);
+            }
+        });
+    }
+    void run(const std::function<void(int)> & w) {
+        work = &w;
+        done.store(0, std::memory_order_release);
+        gen.fetch_add(1, std::memory_order_release);
+        w(0);
+        while (done.load(std::memory_order_acquire) < n - 1) std::this_thread::yield();
+    }
+    ~RowPool() {
+        stop.store(true, std::memory_order_release);
+        gen.fetch_add(1, std::memory_order_release);
+        for (auto & t : th) t.join();
+    }
+};
 
 }  // namespace
 
 int tqo_hardware_threads(void) { return int(std::thread::hardware_concurrency()); }
 
+int tqo_cpu_matvec(uint32_t wtype, const void * W, int rows, int cols, const float * x, int mode, float * y) {
+    int elems, bytes;
+    if (!baseline_type(wtype) || !tqo_block_layout(wtype, &elems, &bytes) || cols % elems || cols % 32 || rows <= 0 || mode < 0 || mode > 2) return -1;
+    XQ xq;
+    if (mode) quant_x_blocks(x, cols, xq);
+    matvec_rows(wtype, static_cast<const uint8_t *>(W), cols, x, mode ? &xq : nullptr, mode, 0, rows, y);
+    return 0;
+}
+
 double tqo_cpu_expert_bench(uint32_t wtype, const void * gate, const void * up, const void * down, int hidden, int ff,
                             int n_expert, int threads, int int8_act, int reps, float * checksum) {
     int elems, bytes;
-    if (!tqo_block_layout(wtype, &elems, &bytes) || hidden % elems || ff % elems || n_expert <= 0 || threads <= 0 || reps <= 0) return -1.0;
+    if (!baseline_type(wtype) || !tqo_block_layout(wtype, &elems, &bytes) || hidden % elems || ff % elems || n_expert <= 0 || threads <= 0 || reps <= 0) return -1.0;
     const size_t stride = size_t(int64_t(ff) * hidden / elems) * bytes;
+    const int mode = int8_act ? 1 : 0;
     std::vector<float> sums(static_cast<size_t>(n_expert), 0.f);
     auto pass = [&]() {
         std::atomic<int> next{0};
@@ -1140,11 +1313,11 @@ double tqo_cpu_expert_bench(uint32_t wtype, const void * gate, const void * up, 
                 if (e >= n_expert) break;
                 for (int i = 0; i < hidden; ++i) x[size_t(i)] = 0.5f + 0.001f * float((i + e) & 15);
                 if (int8_act) quant_x_blocks(x.data(), hidden, xq);
-                matvec(wtype, static_cast<const uint8_t *>(gate) + stride * e, ff, hidden, x.data(), int8_act ? &xq : nullptr, g.data());
-                matvec(wtype, static_cast<const uint8_t *>(up) + stride * e, ff, hidden, x.data(), int8_act ? &xq : nullptr, u.data());
+                matvec_rows(wtype, static_cast<const uint8_t *>(gate) + stride * e, hidden, x.data(), &xq, mode, 0, ff, g.data());
+                matvec_rows(wtype, static_cast<const uint8_t *>(up) + stride * e, hidden, x.data(), &xq, mode, 0, ff, u.data());
                 for (int o = 0; o < ff; ++o) act[size_t(o)] = (g[size_t(o)] / (1.f + std::exp(-g[size_t(o)]))) * u[size_t(o)];
                 if (int8_act) quant_x_blocks(act.data(), ff, aq);
-                matvec(wtype, static_cast<const uint8_t *>(down) + stride * e, hidden, ff, act.data(), int8_act ? &aq : nullptr, y.data());
+                matvec_rows(wtype, static_cast<const uint8_t *>(down) + stride * e, ff, act.data(), &aq, mode, 0, hidden, y.data());
                 float s = 0.f;
                 for (int i = 0; i < hidden; ++i) s += y[size_t(i)];
                 sums[size_t(e)] = s;
@@ -1160,5 +1333,37 @@ double tqo_cpu_expert_bench(uint32_t wtype, const void * gate, const void * up, 
     for (int r = 0; r < reps; ++r) pass();
     const auto t1 = std::chrono::steady_clock::now();
     if (checksum) { float s = 0.f; for (float v : sums) s += v; *checksum = s; }
+    return std::chrono::duration<double>(t1 - t0).count() / reps;
+}
+
+double tqo_cpu_expert_latency(uint32_t wtype, const void * gate, const void * up, const void * down, int hidden, int ff,
+                              int threads, int reps, float * checksum) {
+    int elems, bytes;
+    if (!baseline_type(wtype) || !tqo_block_layout(wtype, &elems, &bytes) || hidden % elems || ff % elems || threads <= 0 || reps <= 0) return -1.0;
+    std::vector<float> x(static_cast<size_t>(hidden)), g(static_cast<size_t>(ff)), u(static_cast<size_t>(ff)), act(static_cast<size_t>(ff)), y(static_cast<size_t>(hidden));
+    for (int i = 0; i < hidden; ++i) x[size_t(i)] = 0.5f + 0.001f * float(i & 15);
+    XQ xq, aq;
+    RowPool pool(threads);
+    const std::function<void(int)> gate_up = [&](int t) {
+        const int lo = int(int64_t(ff) * t / threads), hi = int(int64_t(ff) * (t + 1) / threads);
+        matvec_rows(wtype, static_cast<const uint8_t *>(gate), hidden, x.data(), &xq, 1, lo, hi, g.data());
+        matvec_rows(wtype, static_cast<const uint8_t *>(up), hidden, x.data(), &xq, 1, lo, hi, u.data());
+    };
+    const std::function<void(int)> down_rows = [&](int t) {
+        const int lo = int(int64_t(hidden) * t / threads), hi = int(int64_t(hidden) * (t + 1) / threads);
+        matvec_rows(wtype, static_cast<const uint8_t *>(down), ff, act.data(), &aq, 1, lo, hi, y.data());
+    };
+    auto expert = [&]() {   // the act row depends on every gate / up row: two phases, as the engine's miss pool runs them
+        quant_x_blocks(x.data(), hidden, xq);
+        pool.run(gate_up);
+        for (int o = 0; o < ff; ++o) act[size_t(o)] = (g[size_t(o)] / (1.f + std::exp(-g[size_t(o)]))) * u[size_t(o)];
+        quant_x_blocks(act.data(), ff, aq);
+        pool.run(down_rows);
+    };
+    expert();
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int r = 0; r < reps; ++r) expert();
+    const auto t1 = std::chrono::steady_clock::now();
+    if (checksum) { float s = 0.f; for (float v : y) s += v; *checksum = s; }
     return std::chrono::duration<double>(t1 - t0).count() / reps;
 }

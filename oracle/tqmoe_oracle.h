@@ -149,12 +149,20 @@ typedef struct tqo_layer {
 int tqo_layer_forward(const tqo_layer * L, const float * x, const float * logits, int n, float * out,
                       int32_t * ids_out, float * weights_out);
 
-/* CPU baseline (port of the reference's tests/bench_cpu_expert_mt.cpp scheme onto an arbitrary bank format):
- * `threads` workers pull experts from an atomic counter; each expert = gate, up, down matvec of one token with
- * per-32-block int8 activations (int8_act = 1) or fp32 activations (0). Returns seconds per pass over n_expert
- * experts, averaged over `reps` passes after one warm pass. */
+/* CPU baseline: the scheme of the reference's tests/bench_cpu_expert_mt.cpp on this build's bank formats (IQ4_XS,
+ * IQ4_NL, Q4_K, IQ3_S, NVFP4G).
+ * tqo_cpu_expert_bench: table 1 (:69-116). `threads` workers pull experts from an atomic counter; each expert = gate,
+ * up, down matvec of one token with per-32-block int8 activations and AVX2 integer dots (int8_act = 1) or fp32
+ * activations (0). Returns seconds per pass over n_expert experts, averaged over `reps` passes after one warm pass.
+ * tqo_cpu_expert_latency: table 2 (:130-199). One expert (index 0 of the banks), its rows split over `threads`
+ * persistent workers woken by a generation counter, int8 activations; seconds per expert.
+ * tqo_cpu_matvec: one matvec y[rows] = W x with the kernels the two benches run. mode 0 fp32, 1 int8 activations
+ * with AVX2 integer dots, 2 int8 activations with scalar integer dots. */
 double tqo_cpu_expert_bench(uint32_t wtype, const void * gate, const void * up, const void * down, int hidden, int ff,
                             int n_expert, int threads, int int8_act, int reps, float * checksum);
+double tqo_cpu_expert_latency(uint32_t wtype, const void * gate, const void * up, const void * down, int hidden, int ff,
+                              int threads, int reps, float * checksum);
+int tqo_cpu_matvec(uint32_t wtype, const void * W, int rows, int cols, const float * x, int mode, float * y);
 int tqo_hardware_threads(void);
 
 #ifdef __cplusplus

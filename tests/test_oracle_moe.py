@@ -344,24 +344,45 @@ def test_layer_forward_lossy_operand_modes_against_float64(oracle):
 
 
 def test_cpu_baseline_kernels_agree_with_decode(oracle, ref):
-    """The CPU-baseline matvecs: fp32 variant vs decode + float64 dot; int8 variant within 1e-2 rms-rel (the gates of
-    the reference's tests/test_cpu_expert_matvec.cpp:117-118); the reference's own IQ4_NL kernels agree likewise."""
+    """The CPU-baseline matvecs, row by row, with the gates of the reference's tests/test_cpu_expert_matvec.cpp:117-118, 178-195:
+    fp32 variant vs decode + float64 dot rms-rel <= 1e-5; int8 variant <= 1e-2; and the AVX2 integer dots against the scalar
+    ones (the integer sums are exact on both sides, so they agree to fp32 rounding of the scale products). Then the two bench
+    schemes' checksums against float64; the reference's own IQ4_NL kernels agree likewise."""
     rng = np.random.default_rng(19)
+    rel = lambda y, want: np.sqrt(np.mean((y - want) ** 2) / np.mean(want ** 2))
+    for wtype in (oracle.IQ4_XS, oracle.Q4_K, oracle.IQ3_S, oracle.IQ4_NL, oracle.NVFP4G):
+        rows, cols = 96, 768 if wtype != oracle.NVFP4G else 640
+        for raw in (oracle.random_blocks(wtype, rows, cols, rng),
+                    oracle.quantize(wtype, (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32))):
+            x = rng.standard_normal(cols).astype(np.float32)
+            want = oracle.dequantize(wtype, raw, rows * cols).reshape(rows, cols).astype(np.float64) @ x.astype(np.float64)
+            y32, y8, y8s = (oracle.cpu_matvec(wtype, raw, rows, cols, x, mode) for mode in (0, 1, 2))
+            assert rel(y32, want) < 1e-5, (wtype, rel(y32, want))
+            assert rel(y8, want) < 1e-2, (wtype, rel(y8, want))
+            assert np.abs(y8 - y8s).max() < 2e-6 * np.abs(want).max(), wtype
     h, f, ne = 512, 256, 2
-    for wtype in (oracle.IQ4_XS, oracle.Q4_K, oracle.IQ3_S, oracle.IQ4_NL):
+    for wtype in (oracle.IQ4_XS, oracle.Q4_K, oracle.IQ3_S, oracle.IQ4_NL, oracle.NVFP4G):
+        if wtype == oracle.NVFP4G:
+            h, f = 640, 256
         banks = [oracle.quantize(wtype, (rng.standard_normal((ne * r, c)) * 0.02).astype(np.float32))
                  for r, c in ((f, h), (f, h), (h, f))]
         t0, c0 = oracle.cpu_expert_bench(wtype, *banks, h, f, ne, 2, False, reps=1)
         t1, c1 = oracle.cpu_expert_bench(wtype, *banks, h, f, ne, 2, True, reps=1)
         dec = [oracle.dequantize(wtype, b, ne * f * h).astype(np.float64) for b in banks]
-        want = 0.0
+        want, first = 0.0, None
         for e in range(ne):
             x = 0.5 + 0.001 * ((np.arange(h) + e) & 15)
             g, u = dec[0].reshape(ne, f, h)[e] @ x, dec[1].reshape(ne, f, h)[e] @ x
-            want += (dec[2].reshape(ne, h, f)[e] @ (g / (1 + np.exp(-g)) * u)).sum()
+            y = (dec[2].reshape(ne, h, f)[e] @ (g / (1 + np.exp(-g)) * u)).sum()
+            first = y if first is None else first
+            want += y
         assert abs(c0 - want) < 1e-4 * max(1.0, abs(want)), (wtype, c0, want)
         assert abs(c1 - want) < 3e-2 * max(1.0, abs(want)), (wtype, c1, want)
         assert t0 > 0 and t1 > 0
+        # one expert with its rows split over persistent workers: the same result whatever the number of workers
+        one = [b[: b.size // ne] for b in banks]
+        lat = [oracle.cpu_expert_latency(wtype, *one, h, f, nt, reps=2) for nt in (1, 3)]
+        assert lat[0][1] == lat[1][1] and abs(lat[0][1] - first) < 3e-2 * max(1.0, abs(first)), (wtype, lat, first)
     # the reference's IQ4_NL kernels on the same blocks
     rows, cols = 64, 512
     raw = oracle.quantize(oracle.IQ4_NL, (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32))

@@ -101,6 +101,7 @@ def lib():
         l.tqmoe_layer_workspace_bytes.restype = sz
         l.tqmoe_layer_workspace_bytes.argtypes = [C.POINTER(_Layer), i32]
         l.tqmoe_layer_forward.argtypes = [C.POINTER(_Layer), p, u32, i32, p, u32, p, p, p, p, sz, p, e]
+        l.tqmoe_layer_path.argtypes = [C.POINTER(_Layer), i32]
         for name in ("tqmoe_router", "tqmoe_topk", "tqmoe_dispatch", "tqmoe_bank_layout", "tqmoe_bank_load", "tqmoe_bank_dequant",
                      "tqmoe_quant_act", "tqmoe_expert_matvec", "tqmoe_expert_matvec2", "tqmoe_extend_ids", "tqmoe_expert_gateup", "tqmoe_expert_down", "tqmoe_combine_strided", "tqmoe_swiglu", "tqmoe_combine",
                      "tqmoe_layer_forward"):
@@ -460,6 +461,14 @@ class MoeLayer:
                       float(self.weight_scale), self.router.data_ptr(), self.shared_gate.data_ptr() if self.shared_gate is not None else None,
                       _ttype(self.router), self.gate.view(), self.up.view(), self.down.view(), int(self.gating), int(not self.norm_weights),
                       self.probs_bias.data_ptr() if self.probs_bias is not None else None)
+
+    def path(self, n):
+        """'decode', 'grouped_i8', 'grouped_f16' or 'grouped_fp8': the expert products a batch of n tokens takes"""
+        d = self.desc()
+        rc = lib().tqmoe_layer_path(C.byref(d), n)
+        if rc < 0:
+            raise TqmoeError(rc, "layer descriptor rejected")
+        return ("decode", "grouped_i8", "grouped_f16", "grouped_fp8")[rc]
 
     def workspace(self, n):
         d = self.desc()

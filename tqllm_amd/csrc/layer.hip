@@ -113,6 +113,12 @@ extern "C" size_t tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t
     return plan_for(*layer, n).total;
 }
 
+extern "C" int32_t tqmoe_layer_path(const tqmoe_layer * layer, int32_t n) {
+    if (!layer || n <= 0 || check_layer(layer, nullptr)) return TQMOE_E_ARG;
+    const Plan p = plan_for(*layer, n);
+    return p.int8 ? TQMOE_PATH_GROUPED_I8 : p.grouped ? TQMOE_PATH_GROUPED_F16 : TQMOE_PATH_DECODE;
+}
+
 static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t xtype, const void * residual, int32_t n, void * out, uint32_t otype,
                              int32_t * ids_out, float * weights_out, float * logits_out, void * workspace, size_t workspace_bytes, void * stream,
                              tqmoe_error * err) {

@@ -182,6 +182,18 @@ int32_t tqmoe_expert_matvec2(const tqmoe_bank * gate, const tqmoe_bank * up, con
                              void * y_up, uint32_t ytype, const int32_t * ids, int32_t n, int32_t topk, void * stream,
                              tqmoe_error * err);
 
+/* The same two products on the rows the reference's callers hold (fp16 rows; any of F32 / F16 / BF16 here): exactly
+ * WeightFormat::expert_matvec(const Mat &, const __half * x, bf16 * y, int rows, const int * ids, int n, int topk,
+ * bool per_expert_input, stream) and expert_matvec2 (weight_format.hpp:62-64, 70-73). x: device [n][cols], or
+ * [n * topk][cols] with per_expert_input. The activation image is made in `scratch` (caller-owned device memory of
+ * tqmoe_act_image_bytes(input rows, cols); one enqueue order: image, then product) and is dead after the call. */
+int32_t tqmoe_expert_matvec_rows(const tqmoe_bank * bank, const void * x, uint32_t xtype, void * y, uint32_t ytype,
+                                 const int32_t * ids, int32_t n, int32_t topk, int32_t per_expert_input, void * scratch,
+                                 size_t scratch_bytes, void * stream, tqmoe_error * err);
+int32_t tqmoe_expert_matvec2_rows(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x, uint32_t xtype,
+                                  void * y_gate, void * y_up, uint32_t ytype, const int32_t * ids, int32_t n, int32_t topk,
+                                  void * scratch, size_t scratch_bytes, void * stream, tqmoe_error * err);
+
 /* Decode stages of the layer (tqmoe_layer_forward is router, top-k, tqmoe_extend_ids, tqmoe_quant_act, these two and
  * tqmoe_combine_strided). `ids` holds the expert of every (token, slot), [n][slots]: the routed ids and, when
  * slots == topk + 1, the shared expert's bank index in the last slot (tqmoe_extend_ids makes it). One block serves every
@@ -270,7 +282,8 @@ int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * xq, const f
  * converted to fp16, fp32 accumulation on the matrix cores): WeightFormat::expert_gemm (weight_format.hpp:51-53) and
  * expert_gemm_gateup (weight_format.hpp:57-59). x: device rows of xtype with the bank's cols; the input row of
  * assignment a is a / slots (tqmoe_expert_gemm_gateup; tqmoe_expert_gemm without per_expert_input) or a itself
- * (per_expert_input). shared_lim a multiple of 32. act: fp16 [n * slots][rows]; y: [n * slots][rows] of ytype (F16 or F32). */
+ * (per_expert_input). shared_lim a multiple of 32. act: fp16 [n * slots][rows]; y: [n * slots][rows] of ytype (F16, BF16 or F32).
+ * n * slots only bounds the number of listed assignments (it sizes the launch): any upper bound will do. */
 int32_t tqmoe_expert_gemm_gateup(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x, uint32_t xtype,
                                  const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t n,
                                  int32_t slots, int32_t topk, int32_t shared_lim, void * act_f16, void * stream,
@@ -279,6 +292,14 @@ int32_t tqmoe_expert_gemm(const tqmoe_bank * bank, const void * x, uint32_t xtyp
                           const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk,
                           int32_t shared_lim, int32_t per_expert_input, void * y, uint32_t ytype, void * stream,
                           tqmoe_error * err);
+/* The reference's form of the dispatch lists, counts [experts] + groups [experts][capacity] (what its grouped products
+ * take: weight_format.hpp:51-59; filled by moe_group, moe.cu:168-176, or on the host, prefill_plan.hpp:63-74), as the
+ * lists the grouped products above read: offsets [experts + 1] = exclusive scan of min(counts, capacity), perm = the
+ * experts' lists one behind the other (perm needs room for the sum of the counts; experts * capacity always suffices).
+ * The order inside an expert is kept; the products do not depend on it. */
+int32_t tqmoe_lists_from_groups(const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts,
+                                int32_t * offsets, int32_t * perm, void * stream, tqmoe_error * err);
+
 /* tqmoe_combine_strided with fp16 rows (the prefill products' output) */
 int32_t tqmoe_combine_strided_f16(const void * routed, int32_t slots, const void * shared, int64_t shared_ld,
                                   const float * weights, const float * shared_weights, void * out, uint32_t otype,

@@ -188,4 +188,88 @@ struct ExpertFormat {
     }
 };
 
+// The expert virtuals of tqllm::WeightFormat with the base class's exact signatures (weight_format.hpp:51-73), as a mixin
+// over the reference's own types, so that a maintainer derives the HIP format from it and the `override`s compile:
+//
+//   struct HipExperts final : tqmoe_hip::ExpertOverrides<tqllm::WeightFormat, tqllm::Mat, __half, __nv_bfloat16, cudaStream_t> { ... };
+//
+// Mat is read as the reference fills it for stacked experts (weight_format.hpp:22-28, 61): p = code plane, aux = aux
+// plane, type = GGUF type id, rows = experts * rows of one expert, cols. The base signatures carry no scratch memory and
+// no token count, so the object holds them: `scratch` is engine-owned device memory (set_scratch) for the activation
+// image of a decode call and for the offsets / permutation form of a grouped call's lists
+// (expert_scratch_bytes(rows, cols, assignments, experts) bytes); `max_assignments` bounds the listed assignments of a
+// grouped call (n * topk of the pass; 0 = experts * capacity, always safe, costs idle blocks). Return values and
+// exceptions are the base's: false = "no such kernel for this format, fall back", std::invalid_argument on bad shapes,
+// std::runtime_error on device errors.
+inline size_t expert_scratch_bytes(int cols, int input_rows, int max_assignments, int experts) {
+    const size_t image = tqmoe_act_image_bytes(input_rows, cols);
+    const size_t lists = (size_t(experts) + 1 + size_t(max_assignments)) * 4 + 512;
+    return image > lists ? image : lists;
+}
+
+template <class Base, class MatT, class HalfT, class Bf16T, class StreamT>
+struct ExpertOverrides : Base {
+    void * scratch = nullptr;
+    size_t scratch_bytes = 0;
+    int max_assignments = 0;
+    void set_scratch(void * device_memory, size_t bytes) { scratch = device_memory; scratch_bytes = bytes; }
+
+    static tqmoe_bank bank_of(const MatT & m, int rows) {
+        tqmoe_bank b{};
+        b.struct_size = sizeof(tqmoe_bank);
+        b.type = m.type; b.experts = rows > 0 ? m.rows / rows : 0; b.rows = rows; b.cols = m.cols; b.codes = m.p; b.aux = m.aux;
+        return b;
+    }
+    bool has_expert_matvec() const override { return true; }
+
+    void expert_matvec(const MatT & m, const HalfT * x, Bf16T * y, int rows, const int * ids, int n, int topk, bool per_expert_input, StreamT stream) const override {
+        tqmoe_error e = fresh();
+        const tqmoe_bank b = bank_of(m, rows);
+        check(tqmoe_expert_matvec_rows(&b, x, TQMOE_F16, y, TQMOE_BF16, ids, n, topk, per_expert_input ? 1 : 0, scratch, scratch_bytes, (void *)stream, &e), e);
+    }
+    void expert_matvec2(const MatT & g, const MatT & u, const HalfT * x, Bf16T * yg, Bf16T * yu, int rows, const int * ids, int n, int topk,
+                        StreamT stream) const override {
+        tqmoe_error e = fresh();
+        const tqmoe_bank bg = bank_of(g, rows), bu = bank_of(u, rows);
+        check(tqmoe_expert_matvec2_rows(&bg, &bu, x, TQMOE_F16, yg, yu, TQMOE_BF16, ids, n, topk, scratch, scratch_bytes, (void *)stream, &e), e);
+    }
+    // the lists in this library's form, in the scratch: offsets [experts + 1], then perm
+    bool lists(const int * counts, const int * groups, int capacity, int experts, int32_t *& offsets, int32_t *& perm, int64_t & bound, StreamT stream) const {
+        bound = max_assignments > 0 ? max_assignments : int64_t(experts) * capacity;
+        const size_t at = (size_t(experts + 1) * 4 + 255) / 256 * 256;
+        if (!scratch || scratch_bytes < at + size_t(bound) * 4) throw std::invalid_argument("tqmoe adapter: scratch too small for the dispatch lists");
+        offsets = static_cast<int32_t *>(scratch);
+        perm = reinterpret_cast<int32_t *>(static_cast<char *>(scratch) + at);
+        tqmoe_error e = fresh();
+        check(tqmoe_lists_from_groups(counts, groups, capacity, experts, offsets, perm, (void *)stream, &e), e);
+        return true;
+    }
+    bool expert_gemm(const MatT & m, const HalfT * x, Bf16T * y, int rows, const int * counts, const int * groups, int capacity, int experts, int topk,
+                     bool per_expert_input, StreamT stream) const override {
+        int32_t * offsets, * perm;
+        int64_t bound;
+        lists(counts, groups, capacity, experts, offsets, perm, bound, stream);
+        tqmoe_error e = fresh();
+        const tqmoe_bank b = bank_of(m, rows);
+        const int32_t n = int32_t((bound + topk - 1) / topk);
+        const int32_t rc = tqmoe_expert_gemm(&b, x, TQMOE_F16, counts, offsets, perm, n, topk, topk, 0, per_expert_input ? 1 : 0, y, TQMOE_BF16, (void *)stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
+    bool expert_gemm_gateup(const MatT & g, const MatT & u, const HalfT * x, HalfT * y, int rows, const int * counts, const int * groups, int capacity,
+                            int experts, int topk, StreamT stream) const override {
+        int32_t * offsets, * perm;
+        int64_t bound;
+        lists(counts, groups, capacity, experts, offsets, perm, bound, stream);
+        tqmoe_error e = fresh();
+        const tqmoe_bank bg = bank_of(g, rows), bu = bank_of(u, rows);
+        const int32_t n = int32_t((bound + topk - 1) / topk);
+        const int32_t rc = tqmoe_expert_gemm_gateup(&bg, &bu, x, TQMOE_F16, counts, offsets, perm, n, topk, topk, 0, y, (void *)stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
+};
+
 }  // namespace tqmoe_hip

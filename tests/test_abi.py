@@ -105,6 +105,11 @@ def test_adapter_header_compiles(tmp_path):
     src.write_text('#include "tqmoe_adapter.hpp"\n'
                    "int main() { tqmoe_error e = tqmoe_hip::fresh(); (void)e; return tqmoe_hip::ExpertFormat::has_expert_matvec() ? 0 : 1; }\n")
     subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), str(src)])
+    # the override mixin against a base class that restates the reference's expert virtuals (tests/adapter_check.cpp): a
+    # signature that does not match the base fails to compile there; the GPU test runs the program
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(rocm, "include"),
+                           "-I", os.path.join(ROOT, "include"), os.path.join(ROOT, "tests", "adapter_check.cpp")])
     # the C header alone is plain C
     csrc = tmp_path / "use.c"
     csrc.write_text('#include "tqmoe.h"\nint main(void) { return (int)sizeof(tqmoe_layer) == 0; }\n')

@@ -77,6 +77,9 @@ def lib():
         l.tqmoe_quant_act.argtypes = [p, u32, i32, i32, p, p, e]
         l.tqmoe_expert_matvec.argtypes = [C.POINTER(_Bank), p, p, u32, p, i32, i32, i32, p, e]
         l.tqmoe_expert_matvec2.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, u32, p, i32, i32, p, e]
+        l.tqmoe_expert_matvec_rows.argtypes = [C.POINTER(_Bank), p, u32, p, u32, p, i32, i32, i32, p, sz, p, e]
+        l.tqmoe_expert_matvec2_rows.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, u32, p, p, u32, p, i32, i32, p, sz, p, e]
+        l.tqmoe_lists_from_groups.argtypes = [p, p, i32, i32, p, p, p, e]
         l.tqmoe_extend_ids.argtypes = [p, p, i32, i32, i32, p, e]
         l.tqmoe_expert_gateup.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, i32, i32, i32, i32, p, e]
         l.tqmoe_expert_down.argtypes = [C.POINTER(_Bank), p, p, p, i32, i32, i32, i32, p, e]

@@ -7,7 +7,7 @@ int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err); 
 // prefill_iq4xs.hip
 int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, hipStream_t s);
 int32_t enqueue_gemm_f16(const tqmoe_bank & b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int * counts, const int * offsets, const int * perm,
-                         int experts, int64_t assignments, int xdiv, void * out, int out_f32, int gateup, int shared_expert, int shared_lim, hipStream_t s);
+                         int experts, int64_t assignments, int xdiv, void * out, uint32_t out_type, int gateup, int shared_expert, int shared_lim, hipStream_t s);
 int64_t grouped_row_tiles(int64_t assignments, int experts);
 int64_t grouped_scale_words(int64_t assignments, int experts);
 int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, const int * counts, const int * offsets, const int * perm, int experts,
@@ -69,6 +69,36 @@ __global__ __launch_bounds__(256) void extend_ids_k(const int * __restrict__ ids
     if (i >= count) return;
     const int t = i / (topk + 1), s = i % (topk + 1);
     ext[i] = s < topk ? ids[t * topk + s] : extra;
+}
+
+// The reference's dispatch lists (counts [E], groups [E][capacity]) as the lists this library's grouped products read:
+// offsets = exclusive scan of the counts, perm = the experts' lists one behind the other. One block; the order inside an
+// expert is kept as it is (the reference's device lists are in no particular order, its host lists ascending).
+__global__ __launch_bounds__(1024) void lists_from_groups_k(const int * __restrict__ counts, const int * __restrict__ groups, int capacity, int E,
+                                                            int * __restrict__ offsets, int * __restrict__ perm) {
+    __shared__ int part[1024];
+    extern __shared__ int start[];   // E + 1
+    const int tid = threadIdx.x, per = (E + 1023) / 1024, lo = min(tid * per, E), hi = min(lo + per, E);
+    int sum = 0;
+    for (int e = lo; e < hi; ++e) sum += min(max(counts[e], 0), capacity);
+    part[tid] = sum;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const int v = tid >= d ? part[tid - d] : 0;
+        __syncthreads();
+        part[tid] += v;
+        __syncthreads();
+    }
+    int base = tid ? part[tid - 1] : 0;
+    for (int e = lo; e < hi; ++e) { start[e] = base; base += min(max(counts[e], 0), capacity); }
+    if (tid == 1023) start[E] = part[1023];
+    __syncthreads();
+    for (int e = tid; e <= E; e += 1024) offsets[e] = start[e];
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int e = wave; e < E; e += 16) {   // a wave per expert: coalesced reads of its list
+        const int c = start[e + 1] - start[e];
+        for (int i = lane; i < c; i += 64) perm[start[e] + i] = groups[int64_t(e) * capacity + i];
+    }
 }
 
 void dispatch_matvec(uint32_t type, Split sp, int nb, const MatvecArgs & k, hipStream_t s) {
@@ -170,6 +200,40 @@ extern "C" int32_t tqmoe_expert_matvec2(const tqmoe_bank * gate, const tqmoe_ban
                                         const int32_t * ids, int32_t n, int32_t topk, void * stream, tqmoe_error * err) {
     if (!up || n <= 0 || topk <= 0) return fail(err, TQMOE_E_ARG, "tqmoe_expert_matvec2: invalid shape or second bank missing");
     return matvec_common(gate, up, image, y_gate, y_up, ytype, ids, int64_t(n) * topk, topk, 1, 1, 0, stream, err, "tqmoe_expert_matvec2");
+}
+
+// the decode products on the caller's own rows: the image is made in the caller's scratch and read by the product behind it
+static int32_t matvec_rows_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, void * y0, void * y1, uint32_t ytype,
+                                  const int32_t * ids, int32_t n, int32_t topk, int32_t per_expert_input, void * scratch, size_t scratch_bytes, void * stream,
+                                  tqmoe_error * err, const char * what) {
+    if (!b0 || n <= 0 || topk <= 0 || int64_t(n) * topk > 65535) return fail(err, TQMOE_E_ARG, "%s: invalid shape", what);
+    const int32_t rows_in = per_expert_input ? n * topk : n;
+    const size_t need = tqmoe_act_image_bytes(rows_in, b0->cols);
+    if (!need) return fail(err, TQMOE_E_ARG, "%s: cols must be a positive multiple of 32", what);
+    if (!scratch || scratch_bytes < need) return fail(err, TQMOE_E_WORKSPACE, "%s: scratch of %zu bytes needed (tqmoe_act_image_bytes of the input rows)", what, need);
+    if (int32_t rc = tqmoe_quant_act(x, xtype, rows_in, b0->cols, scratch, stream, err)) return rc;
+    return matvec_common(b0, b1, scratch, y0, y1, ytype, ids, int64_t(n) * topk, per_expert_input ? 1 : topk, 1, 1, 0, stream, err, what);
+}
+
+extern "C" int32_t tqmoe_expert_matvec_rows(const tqmoe_bank * bank, const void * x, uint32_t xtype, void * y, uint32_t ytype, const int32_t * ids, int32_t n,
+                                            int32_t topk, int32_t per_expert_input, void * scratch, size_t scratch_bytes, void * stream, tqmoe_error * err) {
+    return matvec_rows_common(bank, nullptr, x, xtype, y, nullptr, ytype, ids, n, topk, per_expert_input, scratch, scratch_bytes, stream, err, "tqmoe_expert_matvec_rows");
+}
+
+extern "C" int32_t tqmoe_expert_matvec2_rows(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x, uint32_t xtype, void * y_gate, void * y_up,
+                                             uint32_t ytype, const int32_t * ids, int32_t n, int32_t topk, void * scratch, size_t scratch_bytes, void * stream,
+                                             tqmoe_error * err) {
+    if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_matvec2_rows: second bank missing");
+    return matvec_rows_common(gate, up, x, xtype, y_gate, y_up, ytype, ids, n, topk, 0, scratch, scratch_bytes, stream, err, "tqmoe_expert_matvec2_rows");
+}
+
+extern "C" int32_t tqmoe_lists_from_groups(const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts, int32_t * offsets, int32_t * perm,
+                                           void * stream, tqmoe_error * err) {
+    if (!counts || !groups || !offsets || !perm || capacity <= 0 || experts <= 0 || experts > 4096)
+        return fail(err, TQMOE_E_ARG, "tqmoe_lists_from_groups: invalid shape or pointer");
+    if (int32_t rc = need_device(err, "tqmoe_lists_from_groups")) return rc;
+    lists_from_groups_k<<<1, 1024, size_t(experts + 1) * sizeof(int), static_cast<hipStream_t>(stream)>>>(counts, groups, capacity, experts, offsets, perm);
+    return launched(err, "tqmoe_lists_from_groups");
 }
 
 extern "C" int32_t tqmoe_extend_ids(const int32_t * ids, int32_t * out, int32_t topk, int32_t n, int32_t extra, void * stream, tqmoe_error * err) {
@@ -346,13 +410,13 @@ static int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, con
             return fail(err, TQMOE_E_ARG, "%s: the two banks differ in format or shape", what);
     }
     if (!x || !counts || !offsets || !perm || !out || n <= 0 || topk <= 0 || slots < topk) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
-    if (!is_act_type(xtype) || (otype != TQMOE_F16 && otype != TQMOE_F32)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported element type", what);
+    if (!is_act_type(xtype) || !is_act_type(otype)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported element type", what);
     const int lim_max = gateup ? b0->rows : b0->cols;
     if (slots > topk && (shared_lim <= 0 || shared_lim > lim_max || shared_lim % 32)) return fail(err, TQMOE_E_ARG, "%s: shared_lim must be a multiple of 32 within the bank", what);
     if (b0->experts > 4096) return fail(err, TQMOE_E_ARG, "%s: more than 4096 experts", what);
     if (int32_t rc = need_device(err, what)) return rc;
     const int shared_expert = slots > topk ? b0->experts - 1 : -1;
-    if (enqueue_gemm_f16(*b0, b1, x, xtype, counts, offsets, perm, b0->experts, int64_t(n) * slots, xdiv, out, otype == TQMOE_F32, gateup, shared_expert,
+    if (enqueue_gemm_f16(*b0, b1, x, xtype, counts, offsets, perm, b0->experts, int64_t(n) * slots, xdiv, out, otype, gateup, shared_expert,
                          shared_lim, static_cast<hipStream_t>(stream)))
         return fail(err, TQMOE_E_ARG, "%s: too many assignments for one call", what);
     return launched(err, what);

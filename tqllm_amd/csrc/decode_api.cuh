@@ -44,8 +44,8 @@ struct F16Args {
     const int * perm;         // assignment indices grouped by expert
     int experts;
     int xdiv;                 // input row of assignment a = a / xdiv
-    void * out;               // [assignments][rows], fp16 or fp32
-    int out_f32;
+    void * out;               // [assignments][rows]
+    uint32_t out_type;        // TQMOE_F16, TQMOE_BF16 or TQMOE_F32
     int gateup;
     int shared_expert;        // the expert whose rows (gate / up) or columns (down) stop at shared_lim, or -1
     int shared_lim;

@@ -267,7 +267,8 @@ __global__ __launch_bounds__(256, 2) void expert_gemm_f16_k(F16Args k) {
             float v = acc[0][mi][i];
             if (k.gateup) v = v * __builtin_amdgcn_rcpf(1.f + __expf(-v)) * acc[NB - 1][mi][i];
             v = col < row_lim ? v : 0.f;
-            if (k.out_f32) static_cast<float *>(k.out)[int64_t(a) * rows + col] = v;
+            if (k.out_type == TQMOE_F32) static_cast<float *>(k.out)[int64_t(a) * rows + col] = v;
+            else if (k.out_type == TQMOE_BF16) static_cast<uint16_t *>(k.out)[int64_t(a) * rows + col] = float_to_bf16_bits(v);
             else static_cast<uint16_t *>(k.out)[int64_t(a) * rows + col] = __half_as_ushort(__float2half_rn(v));
         }
 }

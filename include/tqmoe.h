@@ -331,7 +331,9 @@ int32_t tqmoe_add_rmsnorm(void * rows, const void * residual, const float * weig
  * layer (src/models/qwen/qwen4exp/fn_layer_forward.cpp:311-336, 447-520) in one call.
  * The shared expert, when has_shared, is expert index n_expert of the three banks (so banks hold n_expert + 1
  * matrices), uses the first shared_ff rows of gate / up and the first shared_ff columns of down, and is weighted by
- * sigmoid(router logit column n_expert). */
+ * sigmoid(router logit column n_expert), or by 1 when shared_gate is NULL (an always-on shared expert without a gate row).
+ * MoeConfig::swiglu_clamp (src/experts/moe.hpp) is not carried: the fused SwiGLU is unclamped, a model that clamps runs
+ * the modular entry points with its own activation step. */
 typedef struct tqmoe_layer {
     uint32_t struct_size;
     int32_t hidden, ff, n_expert, topk;

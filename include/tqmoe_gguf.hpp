@@ -80,29 +80,42 @@ inline bool gguf_block_layout(uint32_t type, uint64_t & elems, uint64_t & bytes)
 
 inline uint64_t gguf_expert_count(const GgufTensor & t) { return t.ne.size() == 3 ? t.ne[2] : 0; }
 
+// One expert of a 3-D expert tensor [cols, rows, n_experts] as a 2-D tensor view of its own (the job of the reference's
+// gguf_expert_slice, src/core/gguf.hpp:77-91). Fails closed: a tensor that is not 3-D, an empty expert axis, an index past
+// it, a type without a block layout, rows that do not end on a block boundary (a row is what the loaders read, so the
+// check is per row, not per expert), sizes that overflow 64 bits, or a byte count that disagrees with the one recorded
+// when the file was opened all throw std::runtime_error naming the tensor.
+struct ExpertGeometry { uint64_t experts, cols, rows, bytes_each; };
+inline ExpertGeometry gguf_expert_geometry(const GgufTensor & t, const std::string & name) {
+    auto fail = [&](const std::string & why) -> ExpertGeometry { throw std::runtime_error(name + ": " + why); };
+    if (t.ne.size() != 3) return fail("expected a 3-D tensor [cols, rows, experts], found " + std::to_string(t.ne.size()) + " dimension(s)");
+    ExpertGeometry g{t.ne[2], t.ne[0], t.ne[1], 0};
+    if (g.experts == 0) return fail("the expert axis is empty");
+    uint64_t block_elems = 0, block_bytes = 0;
+    if (!gguf_block_layout(t.type, block_elems, block_bytes)) return fail("GGUF type " + std::to_string(t.type) + " has no block layout here");
+    if (g.cols == 0 || g.rows == 0) return fail("an expert matrix of " + std::to_string(g.rows) + " x " + std::to_string(g.cols) + " holds nothing");
+    if (g.cols % block_elems)
+        return fail("rows of " + std::to_string(g.cols) + " weights do not end on the " + std::to_string(block_elems) + "-weight blocks of type " +
+                    std::to_string(t.type));
+    uint64_t row_bytes = 0, each = 0, all = 0;
+    if (__builtin_mul_overflow(g.cols / block_elems, block_bytes, &row_bytes) || __builtin_mul_overflow(row_bytes, g.rows, &each) ||
+        __builtin_mul_overflow(each, g.experts, &all))
+        return fail("tensor size overflows 64 bits");
+    if (all != t.bytes)
+        return fail(std::to_string(g.experts) + " experts of " + std::to_string(each) + " bytes make " + std::to_string(all) + " bytes, the file records " +
+                    std::to_string(t.bytes));
+    g.bytes_each = each;
+    return g;
+}
 inline GgufTensor gguf_expert_slice(const GgufTensor & t, uint64_t idx, const std::string & name) {
-    if (t.ne.size() != 3) throw std::runtime_error(name + ": not a 3-D expert tensor (ne.size()=" + std::to_string(t.ne.size()) + ")");
-    const uint64_t n_experts = t.ne[2];
-    if (n_experts == 0) throw std::runtime_error(name + ": expert tensor with zero experts");
-    if (idx >= n_experts) throw std::runtime_error(name + ": expert index " + std::to_string(idx) + " out of range (" + std::to_string(n_experts) + " experts)");
-    uint64_t blk = 0, bpb = 0;
-    if (!gguf_block_layout(t.type, blk, bpb)) throw std::runtime_error(name + ": unsupported expert tensor type " + std::to_string(t.type));
-    // an expert boundary inside a block could not be addressed
-    const uint64_t per_expert_elems = t.ne[0] * t.ne[1];
-    if (per_expert_elems == 0 || per_expert_elems % blk)
-        throw std::runtime_error(name + ": per-expert element count " + std::to_string(per_expert_elems) + " is not a multiple of the " + std::to_string(blk) +
-                                 "-element block of type " + std::to_string(t.type));
-    const uint64_t per_expert_bytes = per_expert_elems / blk * bpb;
-    // against the byte count the file records: if they disagree every expert would be read from the wrong place
-    if (per_expert_bytes * n_experts != t.bytes)
-        throw std::runtime_error(name + ": expert slice bytes (" + std::to_string(per_expert_bytes) + " x " + std::to_string(n_experts) + ") != tensor bytes (" +
-                                 std::to_string(t.bytes) + ")");
-    GgufTensor s;
-    s.type = t.type;
-    s.ne = {t.ne[0], t.ne[1]};
-    s.offset = t.offset + idx * per_expert_bytes;
-    s.bytes = per_expert_bytes;
-    return s;
+    const ExpertGeometry g = gguf_expert_geometry(t, name);
+    if (idx >= g.experts) throw std::runtime_error(name + ": expert " + std::to_string(idx) + " requested, the tensor holds " + std::to_string(g.experts));
+    GgufTensor view;
+    view.type = t.type;
+    view.ne = {g.cols, g.rows};
+    view.bytes = g.bytes_each;
+    view.offset = t.offset + idx * g.bytes_each;
+    return view;
 }
 
 namespace gguf_detail {

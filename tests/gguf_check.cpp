@@ -1,74 +1,98 @@
-// Host check of include/tqmoe_gguf.hpp against a synthetic GGUF file written by tests/test_gguf.py: the cases of the
-// reference's tests/moe_experts.cpp (every slice must read ITS OWN expert; inconsistencies must throw).
-// usage: gguf_check <file> <cols> <rows> <experts>   tensors: experts.f32 (value e * 10000 + r * 100 + c), experts.q2k
-// (every byte of expert e is 0xE0 + e). Prints one line per check; exit code = number of failures.
+// Host check of include/tqmoe_gguf.hpp on the synthetic GGUF file tests/test_gguf.py writes. The property under test is
+// the one the reference's tests/moe_experts.cpp is about: slicing a stacked expert tensor must hand back each expert's
+// own bytes (a wrong stride reads a neighbour), and every inconsistent descriptor must be refused.
+// usage: gguf_check <file> <cols> <rows> <experts>
+// The file holds "experts.f32" (element value = expert * 10000 + row * 100 + col) and "experts.q2k" (every byte of expert
+// e is 0xE0 + e). One line per check; the exit code is the number of failed checks.
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 
 #include "tqmoe_gguf.hpp"
 
 using namespace tqmoe_hip;
 
-static int failures = 0;
-static void check(bool ok, const char * what) {
+static int failed = 0;
+static void report(const char * what, bool ok) {
     std::printf("   %s %s\n", ok ? "ok  " : "FAIL", what);
-    if (!ok) ++failures;
+    failed += ok ? 0 : 1;
 }
-static bool throws(const GgufTensor & t, uint64_t idx) {
-    try { gguf_expert_slice(t, idx, "t"); return false; } catch (const std::runtime_error &) { return true; }
+static bool refused(const std::function<void()> & f) {
+    try { f(); } catch (const std::runtime_error &) { return true; }
+    return false;
 }
 
 int main(int argc, char ** argv) {
     if (argc < 5) return 100;
-    const uint64_t COLS = std::strtoull(argv[2], nullptr, 10), ROWS = std::strtoull(argv[3], nullptr, 10), N_EXP = std::strtoull(argv[4], nullptr, 10);
-    const GgufFile f = gguf_open(argv[1]);
-    const GgufTensor & t = f.tensors.at("experts.f32");
-    check(gguf_expert_count(t) == N_EXP, "expert count");
-    check(t.ne.size() == 3 && t.ne[0] == COLS && t.ne[1] == ROWS && t.ne[2] == N_EXP, "tensor dims are [COLS][ROWS][N_EXP]");
-    const std::vector<char> whole = f.read(t);
-    check(whole.size() == COLS * ROWS * N_EXP * 4, "whole tensor byte count");
-    bool all_ok = true, values_ok = true;
-    for (uint64_t e = 0; e < N_EXP; ++e) {
-        const GgufTensor s = gguf_expert_slice(t, e, "experts.f32");
-        if (s.ne.size() != 2 || s.ne[0] != COLS || s.ne[1] != ROWS || s.bytes != COLS * ROWS * 4) { all_ok = false; break; }
-        const std::vector<char> got = f.read(s);
-        if (got.size() != s.bytes || std::memcmp(got.data(), whole.data() + e * s.bytes, s.bytes) != 0) { all_ok = false; break; }
-        const float * v = reinterpret_cast<const float *>(got.data());
-        if (v[0] != float(e * 10000) || v[COLS * ROWS - 1] != float(e * 10000 + (ROWS - 1) * 100 + (COLS - 1))) values_ok = false;
+    const uint64_t cols = std::strtoull(argv[2], nullptr, 10), rows = std::strtoull(argv[3], nullptr, 10), experts = std::strtoull(argv[4], nullptr, 10);
+    const GgufFile file = gguf_open(argv[1]);
+
+    // ---- fp32 tensor: every element names its expert, row and column
+    const GgufTensor & plain = file.tensors.at("experts.f32");
+    report("fp32 tensor: three dimensions, cols x rows x experts", plain.ne == std::vector<uint64_t>{cols, rows, experts});
+    report("fp32 tensor: expert count", gguf_expert_count(plain) == experts);
+    const std::vector<char> everything = file.read(plain);
+    report("fp32 tensor: bytes of the whole tensor", everything.size() == cols * rows * experts * sizeof(float));
+    bool shape = true, bytes = true, values = true;
+    for (uint64_t e = 0; e < experts; ++e) {
+        const GgufTensor one = gguf_expert_slice(plain, e, "experts.f32");
+        shape = shape && one.ne == std::vector<uint64_t>{cols, rows} && one.bytes == cols * rows * sizeof(float) && one.type == plain.type;
+        const std::vector<char> data = file.read(one);
+        bytes = bytes && data.size() == one.bytes && !std::memcmp(data.data(), everything.data() + e * one.bytes, one.bytes);
+        if (data.size() != one.bytes) break;
+        float first, last;
+        std::memcpy(&first, data.data(), 4);
+        std::memcpy(&last, data.data() + one.bytes - 4, 4);
+        values = values && first == float(e * 10000) && last == float(e * 10000 + (rows - 1) * 100 + (cols - 1));
     }
-    check(all_ok, "every slice is byte-identical to its own expert span");
-    check(values_ok, "sliced values identify the correct expert (first and last element)");
-    const GgufTensor & q = f.tensors.at("experts.q2k");
-    bool q_ok = gguf_expert_count(q) == N_EXP;
-    for (uint64_t e = 0; e < N_EXP && q_ok; ++e) {
-        const GgufTensor s = gguf_expert_slice(q, e, "experts.q2k");
-        if (s.bytes != COLS * ROWS / 256 * 84) { q_ok = false; break; }
-        for (char c : f.read(s)) if (uint8_t(c) != uint8_t(0xE0 + e)) { q_ok = false; break; }
+    report("fp32 slices: 2-D views of one expert's size", shape);
+    report("fp32 slices: the bytes of the expert's own span of the tensor", bytes);
+    report("fp32 slices: first and last value carry the slice's expert number", values);
+
+    // ---- Q2_K tensor: block format, every byte names its expert
+    const GgufTensor & blocks = file.tensors.at("experts.q2k");
+    bool own = gguf_expert_count(blocks) == experts;
+    for (uint64_t e = 0; e < experts && own; ++e) {
+        const GgufTensor one = gguf_expert_slice(blocks, e, "experts.q2k");
+        own = one.bytes == cols * rows / 256 * 84;
+        for (char c : file.read(one)) own = own && uint8_t(c) == uint8_t(0xE0 + e);
     }
-    check(q_ok, "each Q2_K slice reads exactly its own expert's bytes");
-    const GgufExpertBank b = gguf_expert_bank(f, "experts.q2k");
-    check(b.type == 10 && uint64_t(b.experts) == N_EXP && uint64_t(b.rows) == ROWS && uint64_t(b.cols) == COLS && b.bytes == q.bytes && b.offset == q.offset,
-          "bank descriptor of the whole tensor");
-    // fail-closed behaviour
-    GgufTensor good;
-    good.type = 0; good.ne = {COLS, ROWS, N_EXP}; good.offset = 0; good.bytes = COLS * ROWS * N_EXP * 4;
-    check(!throws(good, 0), "a consistent descriptor does not throw");
-    check(throws(good, N_EXP), "index == n_experts throws");
-    check(throws(good, N_EXP + 100), "index far out of range throws");
-    GgufTensor two_d = good; two_d.ne = {COLS, ROWS};
-    check(throws(two_d, 0), "2-D tensor throws");
-    GgufTensor zero_exp = good; zero_exp.ne = {COLS, ROWS, 0};
-    check(throws(zero_exp, 0), "zero experts throws");
-    GgufTensor bad_bytes = good; bad_bytes.bytes = good.bytes + 4;
-    check(throws(bad_bytes, 0), "byte-count mismatch throws");
-    GgufTensor bad_block; bad_block.type = 10; bad_block.ne = {100, 7, N_EXP}; bad_block.offset = 0; bad_block.bytes = 100 * 7 * N_EXP;
-    check(throws(bad_block, 0), "per-expert count not block-aligned throws");
-    GgufTensor four_d = good; four_d.ne = {COLS, ROWS, N_EXP, 2};
-    check(throws(four_d, 0), "4-D tensor throws");
-    GgufTensor bad_type = good; bad_type.type = 9999;
-    check(throws(bad_type, 0), "unknown type throws");
-    bool no_file = false;
-    try { gguf_open(std::string(argv[1]) + ".missing"); } catch (const std::runtime_error &) { no_file = true; }
-    check(no_file, "a missing file throws");
-    return failures;
+    report("Q2_K slices: 84 bytes per 256 weights, all of them the expert's own", own);
+    const GgufExpertBank bank = gguf_expert_bank(file, "experts.q2k");
+    report("Q2_K bank: the whole tensor as one stacked bank", bank.type == 10 && uint64_t(bank.experts) == experts && uint64_t(bank.rows) == rows &&
+                                                                   uint64_t(bank.cols) == cols && bank.offset == blocks.offset && bank.bytes == blocks.bytes);
+
+    // ---- descriptors that must be refused (built here, no file behind them)
+    GgufTensor sound;
+    sound.type = 0;
+    sound.ne = {cols, rows, experts};
+    sound.offset = 0;
+    sound.bytes = cols * rows * experts * 4;
+    auto slice_refused = [](GgufTensor t, uint64_t idx) { return refused([&] { gguf_expert_slice(t, idx, "t"); }); };
+    report("accepted: a consistent descriptor", !slice_refused(sound, 0) && !slice_refused(sound, experts - 1));
+    report("refused: the index one past the last expert", slice_refused(sound, experts));
+    report("refused: an index far past the end", slice_refused(sound, experts + 100));
+    { GgufTensor t = sound; t.ne = {cols, rows}; report("refused: a 2-D tensor", slice_refused(t, 0)); }
+    { GgufTensor t = sound; t.ne = {cols, rows, experts, 2}; report("refused: a 4-D tensor", slice_refused(t, 0)); }
+    { GgufTensor t = sound; t.ne = {cols, rows, 0}; report("refused: an empty expert axis", slice_refused(t, 0)); }
+    { GgufTensor t = sound; t.bytes += 4; report("refused: a byte count other than experts x expert size", slice_refused(t, 0)); }
+    { GgufTensor t = sound; t.type = 9999; report("refused: a type without a block layout", slice_refused(t, 0)); }
+    {
+        GgufTensor t;   // Q2_K rows of 100 weights: no whole number of 256-weight blocks
+        t.type = 10; t.ne = {100, 7, experts}; t.offset = 0; t.bytes = 100 * 7 * experts;
+        report("refused: rows that do not end on a block boundary", slice_refused(t, 0));
+    }
+    {
+        GgufTensor t;   // 128 x 2 weights fill one Q2_K block per expert, but a row of 128 does not: rows are what loaders read
+        t.type = 10; t.ne = {128, 2, experts}; t.offset = 0; t.bytes = 84 * experts;
+        report("refused: an expert of whole blocks whose rows are not", slice_refused(t, 0));
+    }
+    {
+        GgufTensor t = sound;   // sizes whose product leaves 64 bits
+        t.ne = {uint64_t(1) << 40, uint64_t(1) << 30, 4};
+        t.bytes = 0;
+        report("refused: dimensions whose byte count overflows", slice_refused(t, 0));
+    }
+    report("refused: a file that does not exist", refused([&] { gguf_open(std::string(argv[1]) + ".missing"); }));
+    return failed;
 }

@@ -11,7 +11,7 @@ import pytest
 import synth
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-COLS, ROWS, N_EXP = 32, 8, 5
+COLS, ROWS, N_EXP = 256, 8, 5      # rows of one Q2_K block: rows must end on block boundaries
 
 
 def put_str(b, s):
@@ -81,7 +81,9 @@ def test_python_slicer_fails_closed():
     gguf_expert_slice(good, N_EXP - 1, "t")
     cases = [(good, N_EXP), (good, N_EXP + 100), (GgufTensor(0, [COLS, ROWS], 0, good.bytes), 0), (GgufTensor(0, [COLS, ROWS, 0], 0, good.bytes), 0),
              (GgufTensor(0, [COLS, ROWS, N_EXP], 0, good.bytes + 4), 0), (GgufTensor(10, [100, 7, N_EXP], 0, 100 * 7 * N_EXP), 0),
-             (GgufTensor(0, [COLS, ROWS, N_EXP, 2], 0, good.bytes), 0), (GgufTensor(9999, [COLS, ROWS, N_EXP], 0, good.bytes), 0)]
+             (GgufTensor(0, [COLS, ROWS, N_EXP, 2], 0, good.bytes), 0), (GgufTensor(9999, [COLS, ROWS, N_EXP], 0, good.bytes), 0),
+             (GgufTensor(10, [128, 2, N_EXP], 0, 84 * N_EXP), 0),                       # whole blocks per expert, but not per row
+             (GgufTensor(0, [1 << 40, 1 << 30, 4], 0, 0), 0), (good, -1)]               # a byte count past 64 bits; a negative index
     for t, idx in cases:
         with pytest.raises(GgufError):
             gguf_expert_slice(t, idx, "t")

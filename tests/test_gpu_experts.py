@@ -237,3 +237,21 @@ def test_layer_linearity_and_bf16_output(tq, oracle):
     assert torch.allclose(out, direct, rtol=0, atol=5e-5)      # intermediate rows quantised per 32 values (fused) or per row (here)
     out16 = layer.forward(dev(inp["x"]), out_type=tq.BF16)
     assert torch.equal(out16, out.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("n", [3, 200])
+def test_layer_shared_expert_without_a_gate_row(tq, oracle, n):
+    """An always-on shared expert with no gate row (shared_gate NULL) is weighted by 1, on the decode kernels and on the
+    grouped products: the oracle gets there through a shared-gate logit whose sigmoid is exactly 1."""
+    cfg = synth.small(synth.CONFIGS["c2"], 512, 256, 12, 3)
+    raws = synth.make_banks(cfg, seed=140 + n)
+    gate, up, down = banks_on_device(cfg, raws)
+    inp = synth.make_inputs(cfg, n, seed=141 + n)
+    layer = tq.MoeLayer(dev(inp["router"]), None, gate, up, down, cfg["topk"], shared_ff=cfg["shared_ff"])
+    out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
+    assert not logits[:, cfg["experts"]].any()
+    logits[:, cfg["experts"]] = 100.0
+    mode = 0 if layer.path(n) == "decode" else 5
+    want, want_ids, want_w = oracle.layer_forward(inp["x"][1], logits, *raws, cfg["wtype"], cfg["hidden"], cfg["ff"], cfg["experts"], cfg["topk"],
+                                                  shared_ff=cfg["shared_ff"], act_mode=mode, threads=8)
+    check_layer(out, ids, w, want, want_ids, want_w, clear_tokens(oracle, logits, cfg["experts"], cfg["topk"], ids, want_ids))

@@ -4,10 +4,14 @@
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <set>
+#include <utility>
 
 #include "../../include/tqmoe.h"
 
@@ -45,6 +49,34 @@ inline int32_t need_device(tqmoe_error * err, const char * what) {
     }
     return 0;
 }
+// Per-device facts and one-time settings. The library keeps no state a caller could observe; these only remember what has
+// already been asked of the runtime, per device, so that repeated launches do not ask again.
+inline int current_device() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) { (void)hipGetLastError(); dev = 0; }
+    return dev;
+}
+inline int cu_count() {   // compute units of the current device
+    static std::atomic<int> known[64];
+    const int dev = current_device() & 63;
+    int n = known[dev].load(std::memory_order_relaxed);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) { (void)hipGetLastError(); n = 256; }
+        known[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+// raises a kernel's dynamic LDS limit, once per kernel and device
+inline void allow_dynamic_lds(const void * kernel, int bytes) {
+    static std::mutex guard;
+    static std::set<std::pair<const void *, int>> done;
+    const std::pair<const void *, int> key(kernel, current_device());
+    std::lock_guard<std::mutex> lock(guard);
+    if (done.count(key)) return;
+    (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    done.insert(key);
+}
+
 inline bool is_act_type(uint32_t t) { return t == TQMOE_F32 || t == TQMOE_F16 || t == TQMOE_BF16; }
 inline bool is_bank_type(uint32_t t) { return t == TQMOE_Q2_K || t == TQMOE_IQ1_S || t == TQMOE_Q4_0 || t == TQMOE_Q3_K || t == TQMOE_IQ2_XXS || t == TQMOE_IQ2_XS || t == TQMOE_Q4_K || t == TQMOE_IQ3_S || t == TQMOE_IQ4_XS || t == TQMOE_NVFP4G || t == TQMOE_IQ4_NL || t == TQMOE_Q8_0 ||
            t == TQMOE_Q5_K || t == TQMOE_Q6_K || t == TQMOE_IQ3_XXS || t == TQMOE_IQ2_S;

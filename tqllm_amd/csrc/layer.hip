@@ -7,7 +7,7 @@ namespace tqmoe {
 int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);
 int32_t enqueue_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t * ext_ids, int32_t extra, const void * x,
                      uint32_t xtype, int32_t cols, void * image, int32_t experts, int32_t topk, int32_t n, float scale, int32_t gating,
-                     const float * bias, int32_t norm, hipStream_t s);
+                     const float * bias, int32_t norm, hipStream_t s, int32_t shared_ungated);
 
 namespace {
 
@@ -144,7 +144,7 @@ static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t
     int32_t * ext = L.has_shared ? reinterpret_cast<int32_t *>(ws + p.ids_ext) : nullptr;
     const Routing rt = routing_of(L);
     enqueue_topk(logits, ids, weights, shared_w, ext, L.n_expert, x, xtype, L.hidden, p.grouped ? nullptr : ws + p.ximage, L.n_expert, L.topk, n,
-                 L.weight_scale, rt.gating, rt.bias, rt.norm, static_cast<hipStream_t>(stream));
+                 L.weight_scale, rt.gating, rt.bias, rt.norm, static_cast<hipStream_t>(stream), L.has_shared && !L.shared_gate);
     if (int32_t rc = launched(err, "tqmoe_layer_forward (top-k)")) return rc;
     const int32_t * ids_ext = ext ? ext : ids;
 

@@ -631,7 +631,7 @@ int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const in
     if (cols == 512 || cols == 1024 || cols == 2048) {
         const size_t lds = size_t(32) * size_t(cols + 16);
         auto launch = [&](auto kernel) {
-            if (lds > 65536) (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 32 * (2048 + 16));
+            if (lds > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kernel), 32 * (2048 + 16));
             kernel<<<unsigned(tiles), 256, lds, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan);
         };
 #define TQMOE_GROUP_TILE(XT) (cols == 512 ? launch(group_rows_i8_tile_k<XT, 1>) : cols == 1024 ? launch(group_rows_i8_tile_k<XT, 2>) : launch(group_rows_i8_tile_k<XT, 4>))
@@ -670,17 +670,12 @@ int32_t enqueue_iq4xs_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const i
     GemmArgs k{view(b0), b1 ? view(*b1) : view(b0), xq, xs, counts, offsets, perm, plan_at(xs, tiles * 32, experts), experts, static_cast<uint16_t *>(out_f16),
                gateup, units, shared_expert, shared_lim};
     // one block per compute unit (the kernel's registers and LDS allow no second one), walking the work items
-    static const int cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        return n;
-    }();
+    const int cus = cu_count();
     const int64_t most = (tiles / kChunkTiles + experts + 7) / 8 * 8 * units;     // an upper bound of the items
     const unsigned blocks = unsigned(std::min<int64_t>((cus + 7) / 8 * 8, most));
     const size_t lds = size_t(2) * nb * 2 * 8 * 64 * sizeof(v4i);
     if (nb == 2) {
-        static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(&iq4xs_gemm_k<2>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-        (void)once;
+        allow_dynamic_lds(reinterpret_cast<const void *>(&iq4xs_gemm_k<2>), 65536);
         iq4xs_gemm_k<2><<<blocks, 512, lds, s>>>(k);
     } else {
         iq4xs_gemm_k<1><<<blocks, 256, lds, s>>>(k);

@@ -206,7 +206,9 @@ struct TopkOut {
     int * ext_ids; int extra;          // optional [n][k + 1] copy of the ids with `extra` in the last slot
     const void * x; uint8_t * image;   // optional: the token's input row is written as an activation image row
     int cols;
+    int shared_ungated;                // the shared expert has no gate row: its weight is 1, not sigmoid(0)
 };
+__device__ __forceinline__ float shared_weight_of(const TopkOut & o, float logit) { return o.shared_ungated ? 1.f : 1.f / (1.f + expf(-logit)); }
 
 __device__ __forceinline__ void topk_finish(const TopkOut & o, const float * x_logits, int token, int lane, int e, int k, float scale, float selected) {
     if (lane == 0) {
@@ -216,7 +218,7 @@ __device__ __forceinline__ void topk_finish(const TopkOut & o, const float * x_l
             if (scale != 0.f && scale != 1.f) v *= scale;
             o.weights[int64_t(token) * k + s] = v;
         }
-        if (o.shared_weights) o.shared_weights[token] = 1.f / (1.f + expf(-x_logits[e]));
+        if (o.shared_weights) o.shared_weights[token] = shared_weight_of(o, x_logits[e]);
         if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + k] = o.extra;
     }
 }
@@ -282,7 +284,7 @@ __global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logi
             if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + lane] = my_id;
         }
         if (lane == 0) {
-            if (o.shared_weights) o.shared_weights[token] = 1.f / (1.f + expf(-shared_logit));
+            if (o.shared_weights) o.shared_weights[token] = shared_weight_of(o, shared_logit);
             if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + k] = o.extra;
         }
     } else {
@@ -464,7 +466,7 @@ __global__ __launch_bounds__(64) void topk_gated_k(const float * __restrict__ lo
         if (lane == 0) gated_finish_serial(o.weights + int64_t(token) * k, k, g, scale);
     }
     if (lane == 0) {
-        if (o.shared_weights) o.shared_weights[token] = 1.f / (1.f + expf(-shared_logit));
+        if (o.shared_weights) o.shared_weights[token] = shared_weight_of(o, shared_logit);
         if (o.ext_ids) o.ext_ids[int64_t(token) * (k + 1) + k] = o.extra;
     }
     if (o.image) topk_quantise_row<XT>(o, token, lane);
@@ -697,8 +699,8 @@ extern "C" int32_t tqmoe_router(const void * router, uint32_t wtype, const void 
 namespace tqmoe {
 int32_t enqueue_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t * ext_ids, int32_t extra, const void * x,
                      uint32_t xtype, int32_t cols, void * image, int32_t experts, int32_t topk, int32_t n, float scale, int32_t gating,
-                     const float * bias, int32_t norm, hipStream_t s) {
-    const TopkOut o{ids, weights, shared_weights, ext_ids, extra, x, static_cast<uint8_t *>(image), cols};
+                     const float * bias, int32_t norm, hipStream_t s, int32_t shared_ungated) {
+    const TopkOut o{ids, weights, shared_weights, ext_ids, extra, x, static_cast<uint8_t *>(image), cols, shared_ungated};
     const uint32_t xt = image ? xtype : uint32_t(TQMOE_F32);
     if (gating == TQMOE_GATE_SOFTMAX && !bias && norm) {   // the common case has its own kernel
         switch (xt) {
@@ -724,7 +726,7 @@ extern "C" int32_t tqmoe_topk(const float * logits, int32_t * ids, float * weigh
         return fail(err, TQMOE_E_ARG, "tqmoe_topk: invalid shape or pointer");
     if (int32_t rc = need_device(err, "tqmoe_topk")) return rc;
     enqueue_topk(logits, ids, weights, shared_weights, nullptr, 0, nullptr, TQMOE_F32, 0, nullptr, experts, topk, n, scale, TQMOE_GATE_SOFTMAX, nullptr, 1,
-                 static_cast<hipStream_t>(stream));
+                 static_cast<hipStream_t>(stream), 0);
     return launched(err, "tqmoe_topk");
 }
 
@@ -735,7 +737,7 @@ extern "C" int32_t tqmoe_topk_gated(const float * logits, const float * probs_bi
     if (gating < TQMOE_GATE_SOFTMAX || gating > TQMOE_GATE_SQRT_SOFTPLUS) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_topk_gated: unsupported gating function %d", gating);
     if (int32_t rc = need_device(err, "tqmoe_topk_gated")) return rc;
     enqueue_topk(logits, ids, weights, shared_weights, nullptr, 0, nullptr, TQMOE_F32, 0, nullptr, experts, topk, n, scale, gating, probs_bias, norm_weights != 0,
-                 static_cast<hipStream_t>(stream));
+                 static_cast<hipStream_t>(stream), 0);
     return launched(err, "tqmoe_topk_gated");
 }
 
@@ -763,9 +765,7 @@ int32_t enqueue_dispatch(const int32_t * ids, int32_t * counts, int32_t * offset
     dispatch_count_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, cc, A, experts);
     if (experts <= kWideExperts) {
         const size_t lds = size_t(2 * experts + 1 + 1024 + kWideWaves * experts) * sizeof(int);
-        static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(&dispatch_place_wide_k), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                           int((2 * kWideExperts + 1 + 1024 + kWideWaves * kWideExperts) * sizeof(int)));
-        (void)once;
+        allow_dynamic_lds(reinterpret_cast<const void *>(&dispatch_place_wide_k), int((2 * kWideExperts + 1 + 1024 + kWideWaves * kWideExperts) * sizeof(int)));
         dispatch_place_wide_k<<<unsigned(chunks), 1024, lds, s>>>(ids, cc, counts, offsets, perm, groups, capacity, A, experts, chunks);
         return launched(err, what);
     }

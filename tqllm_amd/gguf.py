@@ -30,27 +30,38 @@ def gguf_expert_count(t):
     return t.ne[2] if len(t.ne) == 3 else 0
 
 
-def gguf_expert_slice(t, idx, name):
-    """Descriptor of expert idx of a 3-D expert tensor: ne reduced to [cols, rows], offset / bytes of its span. Raises
-    GgufError on any inconsistency (gguf.cpp:174-200): a wrong slice would silently read a neighbouring expert."""
+def gguf_expert_geometry(t, name):
+    """(experts, cols, rows, bytes of one expert) of a 3-D expert tensor [cols, rows, experts], or GgufError: not 3-D, an empty
+    expert axis, a type without a block layout, rows that do not end on a block boundary (a row is what the loaders read),
+    a size past 64 bits, or a byte count other than the one recorded when the file was opened."""
     if len(t.ne) != 3:
-        raise GgufError("%s: not a 3-D expert tensor (ne.size()=%d)" % (name, len(t.ne)))
-    n_experts = t.ne[2]
-    if n_experts == 0:
-        raise GgufError("%s: expert tensor with zero experts" % name)
-    if idx >= n_experts or idx < 0:
-        raise GgufError("%s: expert index %d out of range (%d experts)" % (name, idx, n_experts))
+        raise GgufError("%s: expected a 3-D tensor [cols, rows, experts], found %d dimension(s)" % (name, len(t.ne)))
+    cols, rows, experts = t.ne
+    if experts == 0:
+        raise GgufError("%s: the expert axis is empty" % name)
     layout = gguf_block_layout(t.type)
     if layout is None:
-        raise GgufError("%s: unsupported expert tensor type %d" % (name, t.type))
-    blk, bpb = layout
-    per_expert_elems = t.ne[0] * t.ne[1]
-    if per_expert_elems == 0 or per_expert_elems % blk:
-        raise GgufError("%s: per-expert element count %d is not a multiple of the %d-element block of type %d" % (name, per_expert_elems, blk, t.type))
-    per_expert_bytes = per_expert_elems // blk * bpb
-    if per_expert_bytes * n_experts != t.bytes:
-        raise GgufError("%s: expert slice bytes (%d x %d) != tensor bytes (%d)" % (name, per_expert_bytes, n_experts, t.bytes))
-    return GgufTensor(t.type, t.ne[:2], t.offset + idx * per_expert_bytes, per_expert_bytes)
+        raise GgufError("%s: GGUF type %d has no block layout here" % (name, t.type))
+    block_elems, block_bytes = layout
+    if cols == 0 or rows == 0:
+        raise GgufError("%s: an expert matrix of %d x %d holds nothing" % (name, rows, cols))
+    if cols % block_elems:
+        raise GgufError("%s: rows of %d weights do not end on the %d-weight blocks of type %d" % (name, cols, block_elems, t.type))
+    each = cols // block_elems * block_bytes * rows
+    if each * experts >= 1 << 64:
+        raise GgufError("%s: tensor size overflows 64 bits" % name)
+    if each * experts != t.bytes:
+        raise GgufError("%s: %d experts of %d bytes make %d bytes, the file records %d" % (name, experts, each, each * experts, t.bytes))
+    return experts, cols, rows, each
+
+
+def gguf_expert_slice(t, idx, name):
+    """Expert idx of a 3-D expert tensor as a 2-D tensor view of its own (gguf_expert_slice of src/core/gguf.hpp:77-91 in role).
+    Fails closed: a wrong slice would silently read a neighbouring expert."""
+    experts, cols, rows, each = gguf_expert_geometry(t, name)
+    if not 0 <= idx < experts:
+        raise GgufError("%s: expert %d requested, the tensor holds %d" % (name, idx, experts))
+    return GgufTensor(t.type, [cols, rows], t.offset + idx * each, each)
 
 
 class GgufFile:

@@ -233,7 +233,9 @@ int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float *
                               int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err);
 
 /* ------------------------------------------------------------------------------------------ prefill products
- * Grouped int8 x int8 -> int32 products on the matrix cores over the dispatch lists (IQ4_XS banks).
+ * Grouped int8 x int8 -> int32 products on the matrix cores over the dispatch lists: IQ4_XS, IQ3_S and Q4_K banks, with
+ * exact weights (the reference's int8 path covers its u4h formats the same way, quant_u4h.inc:783-789, 839-845, and its
+ * MMQ path the IQ formats, mmq_experts.cu:193-196). Rows a multiple of 32, columns of 256.
  * counts / offsets / perm are tqmoe_dispatch's lists over ids [n][slots] with `experts` = the banks' experts.
  *
  * tqmoe_quant_rows_i8: per input row q = rint(x * 127 / amax), scale = amax / 127 (0 for a zero row): the per-token mode
@@ -278,6 +280,24 @@ int32_t tqmoe_expert_gemm_gateup_i8(const tqmoe_bank * gate, const tqmoe_bank * 
 int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const int32_t * counts,
                              const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk,
                              int32_t shared_lim, void * y_f16, void * stream, tqmoe_error * err);
+/* The E4M3 form of the same steps for NVFP4G banks (fp8 x fp8 -> fp32 on the matrix cores): the input rows as E4M3 with
+ * one scale per row, amax / 448 (the reference's fp8_quant_rows, src/core/fp8_gemm.cuh:19-31: scales applied after the
+ * product); the weights widened to E4M3 bytes, e2m1 * (E4M3 scale of the 16 weights) / 8 rounded to nearest even (a
+ * declared lossy operand: up to six significant bits into four; the 8 keeps 6 * 448 inside the format), 8 * the row's
+ * fp32 global applied to the result. q: E4M3 bytes in the layout of tqmoe_group_rows_i8's; tqmoe_gather_rows_i8 arranges rows that
+ * tqmoe_quant_rows_fp8 has quantised (it copies bytes). Rows a multiple of 32, columns of 256. */
+int32_t tqmoe_quant_rows_fp8(const void * x, uint32_t xtype, int64_t rows, int32_t cols, uint8_t * q, float * scale,
+                             void * stream, tqmoe_error * err);
+int32_t tqmoe_group_rows_fp8(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets,
+                             const int32_t * perm, int32_t experts, int64_t assignments, int32_t xdiv, uint8_t * q,
+                             float * scale, void * stream, tqmoe_error * err);
+int32_t tqmoe_expert_gemm_gateup_fp8(const tqmoe_bank * gate, const tqmoe_bank * up, const uint8_t * xq, const float * xs,
+                                     const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t n,
+                                     int32_t slots, int32_t topk, int32_t shared_lim, void * act_f16, void * stream,
+                                     tqmoe_error * err);
+int32_t tqmoe_expert_gemm_fp8(const tqmoe_bank * bank, const uint8_t * xq, const float * xs, const int32_t * counts,
+                              const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk,
+                              int32_t shared_lim, void * y_f16, void * stream, tqmoe_error * err);
 /* The same two products for every bank format, with fp16 operands (weights decoded and rounded to fp16, input rows
  * converted to fp16, fp32 accumulation on the matrix cores): WeightFormat::expert_gemm (weight_format.hpp:51-53) and
  * expert_gemm_gateup (weight_format.hpp:57-59). x: device rows of xtype with the bank's cols; the input row of

@@ -63,6 +63,8 @@ _lib.tqo_combine.argtypes = [C.c_int, _p, _p, C.c_int, _p]
 _lib.tqo_router_logits.argtypes = [_p, C.c_uint32, _p, _p, C.c_uint32, C.c_int, C.c_int, C.c_int, _p]
 _lib.tqo_quant_act_row_i8.restype = None
 _lib.tqo_quant_act_row_i8.argtypes = [_p, C.c_int, _p, _p]
+_lib.tqo_dequantize_nvfp4_widened.restype = C.c_int
+_lib.tqo_dequantize_nvfp4_widened.argtypes = [_p, _p, C.c_int64]
 _lib.tqo_quant_act_row_e4m3.restype = None
 _lib.tqo_quant_act_row_e4m3.argtypes = [_p, C.c_int, _p, _p]
 _lib.tqo_cpu_expert_bench.restype = C.c_double
@@ -125,6 +127,15 @@ def dequantize(wtype, raw, n):
     out = np.empty(int(n), np.float32)
     if _lib.tqo_dequantize(wtype, _ptr(raw), _ptr(out), int(n)):
         raise ValueError("tqo_dequantize: bad type or size")
+    return out
+
+
+def dequantize_nvfp4_widened(raw, n):
+    """NVFP4G blocks with e2m1 * scale rounded to E4M3 before the global multiplies it (the fp8 products' weights)."""
+    raw = _c(raw, np.uint8)
+    out = np.empty(int(n), np.float32)
+    if _lib.tqo_dequantize_nvfp4_widened(_ptr(raw), _ptr(out), int(n)):
+        raise ValueError("tqo_dequantize_nvfp4_widened: bad size")
     return out
 
 

@@ -357,6 +357,27 @@ void decode_nvfp4g(const uint8_t * b, float * y) {
 
 }  // namespace
 
+// NVFP4G with the weights as an fp8 matrix pipe takes them: e2m1 * E4M3 scale / 8 rounded to E4M3 (nearest even; the
+// division keeps the largest product, 6 * 448 / 8 = 336, inside the format), 8 * the row's fp32 global applied to the rounded
+// value (src/core/fp8_gemm.cuh:19-31 keeps scales outside the operand the same way)
+int tqo_dequantize_nvfp4_widened(const void * src, float * dst, int64_t n) {
+    if (n % 128) return -1;
+    const uint8_t * b = static_cast<const uint8_t *>(src);
+    for (int64_t blk = 0; blk < n / 128; ++blk, b += 76, dst += 128) {
+        float g;
+        std::memcpy(&g, b, 4);
+        for (int grp = 0; grp < 8; ++grp) {
+            const float sc = tqo_e4m3_to_float(b[4 + grp]);
+            for (int i = 0; i < 8; ++i) {
+                const uint8_t q = b[12 + 8 * grp + i];
+                dst[16 * grp + 2 * i] = tqo_e4m3_to_float(tqo_float_to_e4m3(kE2M1[q & 15] * sc * 0.125f)) * (8.f * g);
+                dst[16 * grp + 2 * i + 1] = tqo_e4m3_to_float(tqo_float_to_e4m3(kE2M1[q >> 4] * sc * 0.125f)) * (8.f * g);
+            }
+        }
+    }
+    return 0;
+}
+
 int tqo_dequantize(uint32_t type, const void * src, float * dst, int64_t n) {
     int elems, bytes;
     if (!tqo_block_layout(type, &elems, &bytes) || n < 0 || n % elems) return -1;
@@ -917,6 +938,18 @@ void requant_row_i8(float * x, int cols) {  // x <- dequantised per-row int8 ima
     for (int i = 0; i < cols; ++i) x[i] = float(q[size_t(i)]) * s;
 }
 
+void requant_row_e4m3(float * x, int cols) {  // x <- dequantised per-row E4M3 image of x
+    std::vector<uint8_t> q(static_cast<size_t>(cols));
+    float s;
+    tqo_quant_act_row_e4m3(x, cols, q.data(), &s);
+    for (int i = 0; i < cols; ++i) x[i] = tqo_e4m3_to_float(q[size_t(i)]) * s;
+}
+void requant_row(int act_mode, float * x, int cols) { if (act_mode == 2) requant_row_e4m3(x, cols); else requant_row_i8(x, cols); }
+// act_mode 2 reads the banks as the fp8 products do
+int decode_weights(const tqo_layer & L, uint32_t type, const void * src, float * dst, int64_t n) {
+    return L.act_mode == 2 ? tqo_dequantize_nvfp4_widened(src, dst, n) : tqo_dequantize(type, src, dst, n);
+}
+
 struct Decoded { std::vector<float> gate, up, down; };
 
 int decode_expert(const tqo_layer & L, int e, int ff, Decoded & d) {
@@ -928,8 +961,8 @@ int decode_expert(const tqo_layer & L, int e, int ff, Decoded & d) {
     d.up.resize(size_t(ff) * L.hidden);
     d.down.resize(size_t(L.hidden) * ff);
     // gate / up: the first ff rows of expert e
-    if (tqo_dequantize(L.wtype, static_cast<const uint8_t *>(L.gate) + stride * e, d.gate.data(), int64_t(ff) * L.hidden)) return -1;
-    if (tqo_dequantize(L.wtype, static_cast<const uint8_t *>(L.up) + stride * e, d.up.data(), int64_t(ff) * L.hidden)) return -1;
+    if (decode_weights(L, L.wtype, static_cast<const uint8_t *>(L.gate) + stride * e, d.gate.data(), int64_t(ff) * L.hidden)) return -1;
+    if (decode_weights(L, L.wtype, static_cast<const uint8_t *>(L.up) + stride * e, d.up.data(), int64_t(ff) * L.hidden)) return -1;
     // down: rows of L.ff columns, the first ff columns kept; its bank may have a format of its own
     const uint32_t dtype = L.wtype_down ? L.wtype_down : L.wtype;
     int delems, dbytes;
@@ -937,7 +970,7 @@ int decode_expert(const tqo_layer & L, int e, int ff, Decoded & d) {
     std::vector<float> row(static_cast<size_t>(L.ff));
     const size_t row_bytes = size_t(L.ff / delems) * dbytes, dstride = size_t(gu / delems) * dbytes;
     for (int r = 0; r < L.hidden; ++r) {
-        if (tqo_dequantize(dtype, static_cast<const uint8_t *>(L.down) + dstride * e + row_bytes * r, row.data(), L.ff)) return -1;
+        if (decode_weights(L, dtype, static_cast<const uint8_t *>(L.down) + dstride * e + row_bytes * r, row.data(), L.ff)) return -1;
         std::copy(row.begin(), row.begin() + ff, d.down.begin() + size_t(r) * ff);
     }
     return 0;
@@ -953,9 +986,9 @@ void ffn_mode(const tqo_layer & L, const float * x, const Decoded & d, int ff, f
         for (int i = 0; i < L.hidden; ++i) { g += wg[i] * x[i]; u += wu[i] * x[i]; }
         act[size_t(o)] = (g / (1.f + std::exp(-g))) * u;
     }
-    const bool f16 = L.act_mode == 5;   // the grouped products keep act and y as fp16 rows
+    const bool f16 = L.act_mode == 5 || L.act_mode == 2;   // the grouped products keep act and y as fp16 rows
     if (f16) for (float & v : act) v = tqo_half_to_float(tqo_float_to_half(v));
-    requant_row_i8(act.data(), ff);
+    requant_row(L.act_mode, act.data(), ff);
     for (int i = 0; i < L.hidden; ++i) {
         float s = 0.f;
         const float * wd = d.down.data() + size_t(i) * ff;
@@ -972,7 +1005,8 @@ int tqo_layer_forward(const tqo_layer * Lp, const float * x, const float * logit
     int elems, bytes;
     if (!tqo_block_layout(L.wtype, &elems, &bytes)) return -1;
     if (L.hidden % elems || L.ff % elems || n <= 0 || L.k <= 0 || L.k > L.n_expert) return -1;
-    if (L.act_mode != 0 && L.act_mode != 1 && L.act_mode != 5) return -1;
+    if (L.act_mode != 0 && L.act_mode != 1 && L.act_mode != 2 && L.act_mode != 5) return -1;
+    if (L.act_mode == 2 && (L.wtype != TQO_NVFP4G || (L.wtype_down && L.wtype_down != TQO_NVFP4G))) return -1;
     if (L.has_shared && (L.shared_ff <= 0 || L.shared_ff > L.ff || L.shared_ff % elems)) return -1;
     const int E = L.n_expert, K = L.k, A = n * K, H = L.hidden;
     std::vector<int32_t> ids(static_cast<size_t>(A)), counts(static_cast<size_t>(E)), offsets(size_t(E) + 1), perm(static_cast<size_t>(A));
@@ -985,7 +1019,7 @@ int tqo_layer_forward(const tqo_layer * Lp, const float * x, const float * logit
     if (weights_out) std::copy(weights.begin(), weights.end(), weights_out);
 
     std::vector<float> xin(x, x + size_t(n) * H);
-    if (L.act_mode) for (int t = 0; t < n; ++t) requant_row_i8(xin.data() + size_t(t) * H, H);
+    if (L.act_mode) for (int t = 0; t < n; ++t) requant_row(L.act_mode, xin.data() + size_t(t) * H, H);
 
     std::vector<float> routed(size_t(A) * H), shared(L.has_shared ? size_t(n) * H : 0);
     std::atomic<int> next{0}, failed{0};

@@ -113,6 +113,10 @@ int tqo_router_logits(const void * w, uint32_t wtype, const void * shared_gate, 
 /* Declared activation quantisers of the lossy operand paths. */
 void tqo_quant_act_row_i8(const float * x, int cols, int8_t * q, float * scale);     /* scale = amax/127 */
 void tqo_quant_act_row_e4m3(const float * x, int cols, uint8_t * q, float * scale);  /* scale = amax/448 */
+/* NVFP4G blocks -> fp32 with e2m1 * (E4M3 scale) / 8 rounded to E4M3 before 8 * the row's global multiplies it: the
+ * weights of an fp8 matrix product that keeps the global outside the operand (the 8 keeps 6 * 448 inside E4M3). n a
+ * multiple of 128. */
+int  tqo_dequantize_nvfp4_widened(const void * src, float * dst, int64_t n);
 
 /* Residual add and RMS norm in front of the layer, the reference's add_sumsq + norm_h with their summation order
  * (per 256 values: xor butterflies over 32, then the eight sums in order; the blocks' sums strided over 32 lanes and
@@ -130,7 +134,8 @@ int tqo_add_rmsnorm(uint16_t * rows, const uint16_t * residual, const float * we
  *   act_mode: 0 = fp32 activations (oracle A); 1 = the inputs of both products (the token row, the act row) passed
  *   through tqo_quant_act_row_i8 (oracle B of an int8 path that keeps fp32 intermediate rows); 5 = mode 1 with
  *   silu(gate) * up and the down product each rounded to fp16 (oracle B of the grouped int8 products, which store
- *   fp16 rows).
+ *   fp16 rows); 2 = NVFP4G banks on fp8 operands (oracle B of the grouped fp8 products): both product inputs passed
+ *   through tqo_quant_act_row_e4m3, the weights through tqo_dequantize_nvfp4_widened, fp16 roundings as in mode 5.
  *   out fp32 [n][H]; ids_out [n][k], weights_out [n][k] may be null. threads: worker threads over tokens.
  *   gating (0 = softmax), raw_weights (nonzero: unnormalised), weight_scale (0 = none) and bias (or null) are
  *   tqo_route's arguments; all zero is softmax routing with normalised weights.

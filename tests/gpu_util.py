@@ -37,3 +37,9 @@ def clear_tokens(oracle, logits, experts, k, ids=None, want_ids=None, label=""):
     print("%srouting: %d of %d tokens exempt (probability ties between different logits), %d of them differ" % (label and label + ": ", int(tie.sum()), len(tie), differ))
     assert tie.sum() <= max(1, len(tie) // 500), "too many exempt tokens: pick another seed"
     return ~tie
+
+
+def oracle_mode(layer, n):
+    """the oracle's operand mode for the products a batch of n tokens takes: fp32 activations for the decode kernels and
+    the fp16 grouped products, the declared 8-bit quantisers for the int8 and fp8 grouped products"""
+    return {"decode": 0, "grouped_f16": 0, "grouped_i8": 5, "grouped_fp8": 2}[layer.path(n)]

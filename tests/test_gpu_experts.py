@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import synth
-from gpu_util import banks_on_device, clear_tokens, dev
+from gpu_util import banks_on_device, clear_tokens, dev, oracle_mode
 
 pytestmark = pytest.mark.gpu
 
@@ -125,7 +125,7 @@ def run_layer(tq, oracle, cfg, n, seed, distinct=None):
                         shared_ff=cfg["shared_ff"])
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
     want, want_ids, want_w = oracle.layer_forward(inp["x"][1], logits, *raws, cfg["wtype"], cfg["hidden"], cfg["ff"], cfg["experts"],
-                                                  cfg["topk"], shared_ff=cfg["shared_ff"], act_mode=0, threads=16)
+                                                  cfg["topk"], shared_ff=cfg["shared_ff"], act_mode=oracle_mode(layer, n), threads=16)
     clear = clear_tokens(oracle, logits, cfg["experts"], cfg["topk"], ids, want_ids)
     return out, ids, w, want, want_ids, want_w, clear
 
@@ -171,7 +171,7 @@ def test_layer_down_bank_of_another_format(tq, oracle, gu_type, down_type, n):
     layer = tq.MoeLayer(dev(inp["router"]), dev(inp["shared_gate"]), gate, up, down, cfg["topk"], shared_ff=cfg["shared_ff"])
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
     want, want_ids, want_w = oracle.layer_forward(inp["x"][1], logits, *raws, gu_type, cfg["hidden"], cfg["ff"], cfg["experts"], cfg["topk"],
-                                                  shared_ff=cfg["shared_ff"], act_mode=0, threads=16, wtype_down=down_type)
+                                                  shared_ff=cfg["shared_ff"], act_mode=oracle_mode(layer, n), threads=16, wtype_down=down_type)
     check_layer(out, ids, w, want, want_ids, want_w, clear_tokens(oracle, logits, cfg["experts"], cfg["topk"], ids, want_ids))
 
 
@@ -213,7 +213,7 @@ def test_layer_other_routing_modes(tq, oracle, gating, norm, biased, scale, n):
                         gating=gating, probs_bias=dev(bias) if biased else None, norm_weights=norm)
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
     want, want_ids, want_w = oracle.layer_forward(inp["x"][1], logits, *raws, cfg["wtype"], cfg["hidden"], cfg["ff"], e, k, shared_ff=cfg["shared_ff"],
-                                                  act_mode=0, threads=16, gating=gating, norm=norm, scale=scale, bias=bias)
+                                                  act_mode=oracle_mode(layer, n), threads=16, gating=gating, norm=norm, scale=scale, bias=bias)
     same = (ids == want_ids).all(axis=1)          # near-tied tokens may swap neighbours; the routing test bounds how many
     assert same.mean() > 0.97
     assert np.abs(w[same] - want_w[same]).max() < 4e-6 * max(1.0, float(np.abs(want_w).max()))
@@ -251,7 +251,7 @@ def test_layer_shared_expert_without_a_gate_row(tq, oracle, n):
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
     assert not logits[:, cfg["experts"]].any()
     logits[:, cfg["experts"]] = 100.0
-    mode = 0 if layer.path(n) == "decode" else 5
+    mode = oracle_mode(layer, n)
     want, want_ids, want_w = oracle.layer_forward(inp["x"][1], logits, *raws, cfg["wtype"], cfg["hidden"], cfg["ff"], cfg["experts"], cfg["topk"],
                                                   shared_ff=cfg["shared_ff"], act_mode=mode, threads=8)
     check_layer(out, ids, w, want, want_ids, want_w, clear_tokens(oracle, logits, cfg["experts"], cfg["topk"], ids, want_ids))

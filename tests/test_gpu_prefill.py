@@ -66,16 +66,19 @@ def test_quant_rows_i8_bit_exact(tq, oracle, kind):
         assert s[r] == np.float32(ws)
 
 
-def grouped_setup(tq, oracle, seed, experts, ff, hidden, n, k, shared):
+def grouped_setup(tq, oracle, seed, experts, ff, hidden, n, k, shared, wtype=None, widened=False):
+    """widened: the decoded weights as the fp8 products take them (NVFP4G)"""
+    wtype = oracle.IQ4_XS if wtype is None else wtype
     rng = np.random.default_rng(seed)
     banks = experts + (1 if shared else 0)
     raws, decs, devb = [], [], []
     for rows, cols in ((ff, hidden), (ff, hidden), (hidden, ff)):
         w = (rng.standard_normal((banks * rows, cols)) * 0.02).astype(np.float32)
-        raw = oracle.quantize(oracle.IQ4_XS, w)
+        raw = oracle.quantize(wtype, w)
         raws.append(raw)
-        decs.append(oracle.dequantize(oracle.IQ4_XS, raw, w.size).reshape(banks, rows, cols).astype(np.float64))
-        devb.append(tq.ExpertBank(oracle.IQ4_XS, raw, banks, rows, cols))
+        dec = oracle.dequantize_nvfp4_widened(raw, w.size) if widened else oracle.dequantize(wtype, raw, w.size)
+        decs.append(dec.reshape(banks, rows, cols).astype(np.float64))
+        devb.append(tq.ExpertBank(wtype, raw, banks, rows, cols))
     slots = k + (1 if shared else 0)
     ids = np.stack([rng.permutation(experts)[:k] for _ in range(n)]).astype(np.int32)
     ids[:, 0] = np.where(rng.random(n) < 0.7, 1, ids[:, 0])            # a crowded expert (several 128-chunks when n is large)
@@ -87,13 +90,42 @@ def grouped_setup(tq, oracle, seed, experts, ff, hidden, n, k, shared):
     return decs, devb, ids, slots, banks
 
 
+def e4m3_values(oracle, q):
+    table = np.array([oracle.e4m3_to_float(c) for c in range(256)], np.float64)
+    return table[q.view(np.uint8)]
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16", "f16"])
+def test_quant_rows_fp8_bit_exact(tq, oracle, kind):
+    """Per-row E4M3 (scale amax / 448, nearest even) against the oracle's quantiser, byte for byte."""
+    rng = np.random.default_rng(6)
+    rows, cols = 41, 768
+    x = rng.standard_normal((rows, cols)).astype(np.float32) * rng.uniform(1e-3, 300, (rows, 1)).astype(np.float32)
+    x[7] = 0
+    x[9, :200] *= 1e-4          # values far below the row's maximum: E4M3 subnormals and zeros
+    t = torch.from_numpy(x).cuda().to({"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[kind])
+    xv = t.float().cpu().numpy()
+    q, s = tq.quant_rows_fp8(t)
+    q, s = natural_order(q.cpu().numpy()).view(np.uint8), s.cpu().numpy()
+    for r in range(rows):
+        wq, ws = oracle.quant_act_row_e4m3(xv[r])
+        same = q[r] == wq
+        assert (same | ((q[r] & 0x7F) == 0) & ((wq & 0x7F) == 0)).all(), r      # a zero's sign is free
+        assert s[r] == np.float32(ws)
+
+
+@pytest.mark.parametrize("wtype", ["IQ4_XS", "IQ3_S", "Q4_K", "NVFP4G"])
 @pytest.mark.parametrize("n,shared_ff", [(3, 0), (70, 256), (300, 512), (900, 0)])
-def test_grouped_products_against_float64(tq, oracle, n, shared_ff):
+def test_grouped_products_against_float64(tq, oracle, n, shared_ff, wtype):
     """gate/up + SwiGLU and down products over the dispatch lists against float64 on the decoded weights and the
-    dequantised int8 rows (the integer products are exact, so only fp32 accumulation of 256-blocks and the fp16 store
-    separate the two)."""
+    dequantised 8-bit rows (the integer products are exact, so only fp32 accumulation of 256-blocks and the fp16 store
+    separate the two; the fp8 products accumulate in fp32 on the decoded E4M3 operands)."""
     experts, ff, hidden, k = 7, 512, 768, 3
-    decs, (gate, up, down), ids, slots, banks = grouped_setup(tq, oracle, 11 + n, experts, ff, hidden, n, k, shared_ff > 0)
+    fp8 = wtype == "NVFP4G"
+    wtype = getattr(oracle, wtype)
+    decs, (gate, up, down), ids, slots, banks = grouped_setup(tq, oracle, 11 + n, experts, ff, hidden, n, k, shared_ff > 0, wtype, widened=fp8)
+    if fp8:
+        return grouped_products_fp8(tq, oracle, decs, gate, up, down, ids, slots, banks, n, k, shared_ff, experts, ff, hidden)
     rng = np.random.default_rng(n)
     xb, xv = oracle.to_bf16(rng.standard_normal((n, hidden)).astype(np.float32))
     x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
@@ -129,26 +161,76 @@ def test_grouped_products_against_float64(tq, oracle, n, shared_ff):
         assert np.abs(y[a] - want).max() < 2e-3 * max(1e-3, np.abs(want).max()), a
 
 
+def grouped_products_fp8(tq, oracle, decs, gate, up, down, ids, slots, banks, n, k, shared_ff, experts, ff, hidden):
+    rng = np.random.default_rng(n)
+    xb, xv = oracle.to_bf16(rng.standard_normal((n, hidden)).astype(np.float32))
+    x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
+    counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), banks)
+    lists = (counts, offsets, perm)
+    xq, xs = tq.group_rows_fp8(x, lists, n * slots, slots)
+    pq, ps = tq.quant_rows_fp8(x)
+    uq, us = ungroup(xq.cpu().numpy(), xs.cpu().numpy(), np.bincount(ids.reshape(-1), minlength=banks), perm.cpu().numpy(), n * slots)
+    assert np.array_equal(uq, natural_order(pq.cpu().numpy())[np.arange(n * slots) // slots])
+    assert np.array_equal(us, ps.cpu().numpy()[np.arange(n * slots) // slots])
+    act = tq.expert_gemm_gateup_fp8(gate, up, xq, xs, lists, n, slots, k, shared_ff)
+    xd = e4m3_values(oracle, natural_order(pq.cpu().numpy())) * ps.cpu().numpy().astype(np.float64)[:, None]
+    got = act.float().cpu().numpy()
+    for a in range(n * slots):
+        e = ids.reshape(-1)[a]
+        lim = shared_ff if (shared_ff and e == experts) else ff
+        g = decs[0][e][:lim] @ xd[a // slots]
+        u = decs[1][e][:lim] @ xd[a // slots]
+        want = g / (1 + np.exp(-g)) * u
+        assert np.abs(got[a, :lim] - want).max() < 2e-3 * max(1.0, np.abs(want).max()), a
+        assert not got[a, lim:].any()
+    aq, a_s = tq.group_rows_fp8(act, lists, n * slots, 1)
+    y = tq.expert_gemm_fp8(down, aq, a_s, lists, n, slots, k, shared_ff).float().cpu().numpy()
+    pq, ps = tq.quant_rows_fp8(act)
+    ad = e4m3_values(oracle, natural_order(pq.cpu().numpy())) * ps.cpu().numpy().astype(np.float64)[:, None]
+    for a in range(n * slots):
+        e = ids.reshape(-1)[a]
+        lim = shared_ff if (shared_ff and e == experts) else ff
+        want = decs[2][e][:, :lim] @ ad[a, :lim]
+        assert np.abs(y[a] - want).max() < 2e-3 * max(1e-3, np.abs(want).max()), a
+
+
+def test_grouped_products_refuse_the_wrong_operand_type(tq, oracle):
+    """int8 rows for an NVFP4G bank, E4M3 rows for an int8 format, a format with neither: refused, nothing enqueued."""
+    rng = np.random.default_rng(1)
+    mk = lambda t: tq.ExpertBank(t, oracle.quantize(t, (rng.standard_normal((2 * 64, 256)) * 0.02).astype(np.float32)), 2, 64, 256)
+    ids = np.zeros((4, 1), np.int32)
+    counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), 2)
+    x = torch.randn(4, 256, device="cuda", dtype=torch.float16)
+    xq, xs = tq.group_rows_i8(x, (counts, offsets, perm), 4, 1)
+    for bank, fn in ((mk(oracle.NVFP4G), tq.expert_gemm_i8), (mk(oracle.IQ4_XS), tq.expert_gemm_fp8), (mk(oracle.IQ4_NL), tq.expert_gemm_i8)):
+        with pytest.raises(tq.TqmoeError):
+            fn(bank, xq, xs, (counts, offsets, perm), 4, 1, 1)
+
+
+@pytest.mark.parametrize("wtype", ["IQ4_XS", "IQ3_S", "Q4_K", "NVFP4G"])
 @pytest.mark.parametrize("rows,experts", [(96, 5), (160, 5), (128, 5), (256, 5), (64, 1100)])
-def test_gemm_i8_bank_shapes(tq, oracle, rows, experts):
+def test_gemm_i8_bank_shapes(tq, oracle, rows, experts, wtype):
     """tqmoe_expert_gemm_i8 over banks whose row count changes the kernel's arrangement (one or two operand slots per block,
     unit counts that do or do not allow the single-tile path) and over more experts than a block keeps an index of, against
     float64 on the decoded weights and the dequantised int8 rows. One expert gets several row tiles, the others one."""
     cols, n, k = 256, 150, 1
+    fp8 = wtype == "NVFP4G"
+    wtype = getattr(oracle, wtype)
     rng = np.random.default_rng(rows + experts)
     w = (rng.standard_normal((experts * rows, cols)) * 0.02).astype(np.float32)
-    raw = oracle.quantize(oracle.IQ4_XS, w)
-    dec = oracle.dequantize(oracle.IQ4_XS, raw, w.size).reshape(experts, rows, cols).astype(np.float64)
-    bank = tq.ExpertBank(oracle.IQ4_XS, raw, experts, rows, cols)
+    raw = oracle.quantize(wtype, w)
+    dec = (oracle.dequantize_nvfp4_widened(raw, w.size) if fp8 else oracle.dequantize(wtype, raw, w.size)).reshape(experts, rows, cols).astype(np.float64)
+    bank = tq.ExpertBank(wtype, raw, experts, rows, cols)
     ids = rng.integers(0, experts, size=(n, k)).astype(np.int32)
     ids[: n // 2, 0] = 2
     x = torch.randn(n, cols, device="cuda", dtype=torch.float16)
     counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), experts)
     lists = (counts, offsets, perm)
-    xq, xs = tq.group_rows_i8(x, lists, n * k, 1)
-    y = tq.expert_gemm_i8(bank, xq, xs, lists, n, k, k).float().cpu().numpy()
-    pq, ps = tq.quant_rows_i8(x)
-    xd = natural_order(pq.cpu().numpy()).astype(np.float64) * ps.cpu().numpy().astype(np.float64)[:, None]
+    xq, xs = tq.group_rows_i8(x, lists, n * k, 1, fp8=fp8)
+    y = tq.expert_gemm_i8(bank, xq, xs, lists, n, k, k, fp8=fp8).float().cpu().numpy()
+    pq, ps = tq.quant_rows_i8(x, fp8=fp8)
+    rows_q = natural_order(pq.cpu().numpy())
+    xd = (e4m3_values(oracle, rows_q) if fp8 else rows_q.astype(np.float64)) * ps.cpu().numpy().astype(np.float64)[:, None]
     for a in range(n):
         want = dec[ids[a, 0]] @ xd[a]
         assert np.abs(y[a] - want).max() < 2e-3 * max(1e-3, np.abs(want).max()), a
@@ -189,12 +271,13 @@ def test_gather_of_quantised_rows_equals_group_rows(tq, dtype):
     assert torch.equal(s1[rows:].view(torch.int32), s2[rows:].view(torch.int32))      # the tile index behind the scales
 
 
-def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0)):
+def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0), path="grouped_i8"):
     raws = synth.make_banks(cfg, seed=seed, distinct=distinct)
     gate, up, down = banks_on_device(cfg, raws)
     inp = synth.make_inputs(cfg, n, seed=seed + 1, zipf=zipf)
     layer = tq.MoeLayer(dev(inp["router"]), dev(inp["shared_gate"]) if cfg["shared_ff"] else None, gate, up, down, cfg["topk"],
                         shared_ff=cfg["shared_ff"])
+    assert layer.path(n) == path
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
     wants = {}
     for mode in modes:
@@ -205,15 +288,20 @@ def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0)):
 
 
 def check_layer(out, ids, w, wants, clear):
-    want, want_ids, want_w = wants[5]
+    fp8 = 5 not in wants
+    want, want_ids, want_w = wants[2] if fp8 else wants[5]
     assert np.array_equal(ids[clear], want_ids[clear])
     assert np.abs(w[clear] - want_w[clear]).max() < 3e-6
     mx, rel = synth.errors(out[clear], want[clear])
-    assert mx < MAX_ABS and rel < REL_RMS, (mx, rel)
-    if 0 in wants:                       # distance to the fp32-activation result: the price of the int8 operand format
+    # E4M3 keeps four significant bits: where the two sides' act values differ in their last fp16 bit (fp32 sums in another
+    # order) and straddle an E4M3 step, the quantised value moves by 6 to 12 %. About 1e-4 of the act values do, which alone
+    # is a relative RMS of about 1e-3 on the output, so the fp8 layer is gated at 3e-3 and at 1e-2 of the largest value; the
+    # products on given operands are held to float64 in test_grouped_products_against_float64.
+    assert mx < MAX_ABS * (max(1.0, float(np.abs(want[clear]).max())) if fp8 else 1.0) and rel < (3e-3 if fp8 else REL_RMS), (mx, rel)
+    if 0 in wants:                       # distance to the fp32-activation result: the price of the 8-bit operand format
         mxa, rela = synth.errors(out[clear], wants[0][0][clear])
-        print("vs fp32 activations: max-abs %.3g rel-rms %.3g; vs int8-activation oracle: max-abs %.3g rel-rms %.3g" % (mxa, rela, mx, rel))
-        assert rela < 3e-2
+        print("vs fp32 activations: max-abs %.3g rel-rms %.3g; vs the %s-operand oracle: max-abs %.3g rel-rms %.3g" % (mxa, rela, "E4M3" if fp8 else "int8", mx, rel))
+        assert rela < (1e-1 if fp8 else 3e-2)
     return mx, rel
 
 
@@ -221,6 +309,17 @@ def check_layer(out, ids, w, wants, clear):
 def test_layer_grouped_small_shapes(tq, oracle, n):
     cfg = synth.small(synth.CONFIGS["c2"], 768, 512, 10, 3)
     check_layer(*run_layer(tq, oracle, cfg, n, seed=60 + n))
+
+
+@pytest.mark.parametrize("name,fmt,path,mode", [("c1", "Q4_K", "grouped_i8", 5), ("c4", "IQ3_S", "grouped_i8", 5), ("c5", "NVFP4G", "grouped_fp8", 2)])
+@pytest.mark.parametrize("n", [64, 300])
+def test_layer_grouped_other_formats(tq, oracle, name, fmt, path, mode, n):
+    """Q4_K and IQ3_S banks on the int8 products, NVFP4G banks on the fp8 products, against the oracle with the same
+    declared operand quantisers (the distance to the fp32-activation oracle printed beside it)."""
+    base = synth.CONFIGS[name]
+    assert base["wtype"] == getattr(oracle, fmt)
+    cfg = synth.small(base, 768, 512, 10, 3)
+    check_layer(*run_layer(tq, oracle, cfg, n, seed=160 + n, modes=(mode, 0), path=path))
 
 
 def test_layer_grouped_small_skewed(tq, oracle):

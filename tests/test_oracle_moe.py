@@ -289,6 +289,97 @@ def _requant_i8(v):
     return q.astype(np.float64) * np.float64(np.float32(m / np.float32(127)))
 
 
+def test_nvfp4_widened_weights_closed_form(oracle):
+    """tqo_dequantize_nvfp4_widened against the closed form on every (scale byte, code) pair: the E4M3 value nearest to
+    e2m1 * scale / 8 (found by brute force over the 256 codes, ties to the even code), times 8 * the global."""
+    codes = np.arange(256, dtype=np.uint8)
+    vals = np.array([oracle.e4m3_to_float(c) for c in codes], np.float64)
+    finite = ~np.isnan(vals)
+    e2m1 = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6])
+
+    def nearest(v):   # the value only (the sign of a zero is not observable in a product)
+        v = float(np.clip(v, -448, 448))
+        d = np.abs(vals[finite] - v)
+        best = np.flatnonzero(d == d.min())
+        cands = codes[finite][best]
+        return vals[finite][best][np.argmin(cands & 1)] if len(set(vals[finite][best])) > 1 else vals[finite][best][0]
+
+    scales = [s for s in range(256) if not np.isnan(oracle.e4m3_to_float(s))]
+    g = np.float32(0.37)
+    for s0 in range(0, len(scales), 8):
+        blk = np.zeros(76, np.uint8)
+        blk[:4] = np.frombuffer(g.tobytes(), np.uint8)
+        blk[4:12] = scales[s0:s0 + 8] + [0] * (8 - len(scales[s0:s0 + 8]))
+        blk[12:76] = np.tile(np.array([0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE], np.uint8), 8)   # codes 0..15 in every group
+        got = oracle.dequantize_nvfp4_widened(blk, 128).reshape(8, 16)
+        for grp in range(8):
+            sc = oracle.e4m3_to_float(int(blk[4 + grp]))
+            want = np.array([nearest(e2m1[c] * sc / 8) for c in range(16)]) * np.float64(np.float32(8) * g)
+            assert np.array_equal(got[grp].astype(np.float64), np.float32(want).astype(np.float64)), (grp, int(blk[4 + grp]))
+    # where the product needs no rounding the widened bank is the plain one
+    rng = np.random.default_rng(2)
+    raw = oracle.quantize(oracle.NVFP4G, (rng.standard_normal((4, 256)) * 0.02).astype(np.float32))
+    plain, wide = oracle.dequantize(oracle.NVFP4G, raw, 1024), oracle.dequantize_nvfp4_widened(raw, 1024)
+    assert (np.abs(wide - plain) <= np.abs(plain) * 2.0 ** -4 + 1e-7).all()   # four significant bits kept
+    assert (wide != plain).mean() > 0.05   # and it is lossy
+
+
+def _requant_e4m3(oracle, v):
+    v = np.asarray(v, np.float32)
+    m = np.float32(np.abs(v).max())
+    if m == 0:
+        return v.astype(np.float64)
+    mul = np.float32(448) / m
+    q = np.array([oracle.e4m3_to_float(oracle.float_to_e4m3(np.float32(t * mul))) for t in v], np.float64)
+    return q * np.float64(np.float32(m / np.float32(448)))
+
+
+def test_layer_forward_fp8_mode_against_float64(oracle):
+    """act_mode 2 (the gate of the grouped fp8 products) rebuilt in float64 numpy from the pinned pieces: widened weights,
+    per-row E4M3 on the token row, fp16 rounding of silu(g) * u, per-row E4M3 on the act row, the down product rounded to
+    fp16. Leaving any one step out must land far from the oracle."""
+    rng = np.random.default_rng(29)
+    h, f, e, k, n, sf = 256, 256, 5, 2, 5, 128
+    wtype = oracle.NVFP4G
+    banks = [oracle.quantize(wtype, (rng.standard_normal(((e + 1) * r, c)) * 0.05).astype(np.float32)) for r, c in ((f, h), (f, h), (h, f))]
+    wide = [oracle.dequantize_nvfp4_widened(b, (e + 1) * f * h).astype(np.float64) for b in banks]
+    plain = [oracle.dequantize(wtype, b, (e + 1) * f * h).astype(np.float64) for b in banks]
+    x = rng.standard_normal((n, h)).astype(np.float32)
+    logits = rng.standard_normal((n, e + 1)).astype(np.float32)
+    got, ids, w = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=sf, act_mode=2, threads=3)
+
+    def rebuild(skip=None):
+        dec = plain if skip == "w" else wide
+        wg, wu, wd = dec[0].reshape(e + 1, f, h), dec[1].reshape(e + 1, f, h), dec[2].reshape(e + 1, h, f)
+        out = np.zeros((n, h))
+        for t in range(n):
+            xq = _requant_e4m3(oracle, x[t]) if skip != "x" else x[t].astype(np.float64)
+
+            def ffn(j, ff):
+                g, u = wg[j, :ff] @ xq, wu[j, :ff] @ xq
+                act = g / (1 + np.exp(-g)) * u
+                if skip != "act16":
+                    act = _half(act)
+                if skip != "act":
+                    act = _requant_e4m3(oracle, act)
+                y = wd[j, :, :ff] @ act
+                return _half(y) if skip != "y16" else y
+
+            out[t] = sum(float(w[t, s]) * ffn(ids[t, s], f) for s in range(k)) + 1 / (1 + np.exp(-float(logits[t, e]))) * ffn(e, sf)
+        return out
+
+    want = rebuild()
+    tol = 2e-5 * max(1.0, np.abs(want).max())
+    off = np.abs(got - want) > tol
+    assert off.mean() < 0.02, off.mean()
+    assert np.abs(got - want).max() < 2e-3 * np.abs(want).max()
+    for skip in ("w", "x", "act", "act16", "y16"):
+        assert (np.abs(got - rebuild(skip)) > tol).mean() > 0.3, skip
+    # banks of another format have no such mode
+    with pytest.raises(Exception):
+        oracle.layer_forward(x, logits, *banks, oracle.IQ4_XS, h, f, e, k, act_mode=2)
+
+
 def test_layer_forward_lossy_operand_modes_against_float64(oracle):
     """act_mode 1 and 5 of tqo_layer_forward (the gates of the grouped int8 products) rebuilt step by step in float64
     numpy: per-row int8 on the token row, [mode 5: fp16 rounding of silu(g) * u], per-row int8 on the act row, the down

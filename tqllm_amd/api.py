@@ -97,6 +97,10 @@ def lib():
         l.tqmoe_gather_rows_i8.argtypes = [p, p, i32, p, p, p, i32, i64, i32, p, p, p, e]
         l.tqmoe_expert_gemm_gateup_i8.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_expert_gemm_i8.argtypes = [C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
+        l.tqmoe_quant_rows_fp8.argtypes = l.tqmoe_quant_rows_i8.argtypes
+        l.tqmoe_group_rows_fp8.argtypes = l.tqmoe_group_rows_i8.argtypes
+        l.tqmoe_expert_gemm_gateup_fp8.argtypes = l.tqmoe_expert_gemm_gateup_i8.argtypes
+        l.tqmoe_expert_gemm_fp8.argtypes = l.tqmoe_expert_gemm_i8.argtypes
         l.tqmoe_expert_gemm_gateup.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, u32, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_expert_gemm.argtypes = [C.POINTER(_Bank), p, u32, p, p, p, i32, i32, i32, i32, i32, p, u32, p, e]
         l.tqmoe_swiglu.argtypes = [p, p, p, i64, p, e]
@@ -321,18 +325,23 @@ def moe_combine_strided(y, slots, weights, shared_weights=None, out_type=F32, ou
     return out
 
 
-def quant_rows_i8(x):
+def quant_rows_i8(x, fp8=False):
     """Per-row int8 activations (k_quant_act_rows mode 2, quant_kernels.cuh:17-19): (q int8 [rows][cols] in the library's
-    byte order, scale fp32 [rows])."""
+    byte order, scale fp32 [rows]). fp8: E4M3 bytes with scale amax / 448 (fp8_quant_rows, fp8_gemm.cuh:19-31)."""
     rows, cols = x.shape
     q = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
     scale = torch.empty(rows, dtype=torch.float32, device=x.device)
     err = _err()
-    _check(lib().tqmoe_quant_rows_i8(_ptr(x), _ttype(x), rows, cols, _ptr(q), _ptr(scale), _stream(x), C.byref(err)), err)
+    fn = lib().tqmoe_quant_rows_fp8 if fp8 else lib().tqmoe_quant_rows_i8
+    _check(fn(_ptr(x), _ttype(x), rows, cols, _ptr(q), _ptr(scale), _stream(x), C.byref(err)), err)
     return q, scale
 
 
-def group_rows_i8(x, lists, assignments, xdiv):
+def quant_rows_fp8(x):
+    return quant_rows_i8(x, fp8=True)
+
+
+def group_rows_i8(x, lists, assignments, xdiv, fp8=False):
     """Per-row int8 quantisation of the input row (a // xdiv) of every listed assignment a, gathered expert by expert into
     the operand-major row tiles the grouped products read (mmq_quantize_act_rows, mmq_experts.cu:79-95, in role):
     (q int8 [grouped rows][cols], scale fp32 [grouped rows]); rows of the padding hold zeros here."""
@@ -342,9 +351,15 @@ def group_rows_i8(x, lists, assignments, xdiv):
     q = torch.zeros((rows, cols), dtype=torch.int8, device=x.device)
     scale = torch.zeros(lib().tqmoe_grouped_scale_words(assignments, counts.numel()), dtype=torch.float32, device=x.device)
     err = _err()
-    _check(lib().tqmoe_group_rows_i8(_ptr(x), _ttype(x), cols, _ptr(counts), _ptr(offsets), _ptr(perm), counts.numel(), assignments, xdiv, _ptr(q),
-                                     _ptr(scale), _stream(x), C.byref(err)), err)
+    fn = lib().tqmoe_group_rows_fp8 if fp8 else lib().tqmoe_group_rows_i8
+    _check(fn(_ptr(x), _ttype(x), cols, _ptr(counts), _ptr(offsets), _ptr(perm), counts.numel(), assignments, xdiv, _ptr(q), _ptr(scale), _stream(x),
+              C.byref(err)), err)
     return q, scale
+
+
+def group_rows_fp8(x, lists, assignments, xdiv):
+    """group_rows_i8 with E4M3 bytes (scale amax / 448): the operand of the NVFP4G grouped products."""
+    return group_rows_i8(x, lists, assignments, xdiv, fp8=True)
 
 
 def gather_rows_i8(rows_q, rows_scale, lists, assignments, xdiv):
@@ -384,28 +399,38 @@ def expert_gemm(bank, x, lists, n, slots, topk, shared_ff=0, per_expert_input=Fa
     return y
 
 
-def expert_gemm_gateup_i8(gate, up, xq, xs, lists, n, slots, topk, shared_ff=0):
+def expert_gemm_gateup_i8(gate, up, xq, xs, lists, n, slots, topk, shared_ff=0, fp8=False):
     """WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59) on int8 rows: fp16 act [n * slots][ff]; rows of
     assignments that are in no list are zero here (the library leaves them untouched)."""
     counts, offsets, perm = lists
     act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=xq.device)
     err = _err()
     g, u = gate.view(), up.view()
-    _check(lib().tqmoe_expert_gemm_gateup_i8(C.byref(g), C.byref(u), _ptr(xq), _ptr(xs), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk,
-                                             shared_ff, _ptr(act), _stream(xq), C.byref(err)), err)
+    fn = lib().tqmoe_expert_gemm_gateup_fp8 if fp8 else lib().tqmoe_expert_gemm_gateup_i8
+    _check(fn(C.byref(g), C.byref(u), _ptr(xq), _ptr(xs), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff, _ptr(act), _stream(xq),
+              C.byref(err)), err)
     return act
 
 
-def expert_gemm_i8(bank, xq, xs, lists, n, slots, topk, shared_ff=0):
+def expert_gemm_gateup_fp8(gate, up, xq, xs, lists, n, slots, topk, shared_ff=0):
+    """The gate / up product with SwiGLU on E4M3 rows (NVFP4G banks, weights widened to E4M3)."""
+    return expert_gemm_gateup_i8(gate, up, xq, xs, lists, n, slots, topk, shared_ff, fp8=True)
+
+
+def expert_gemm_i8(bank, xq, xs, lists, n, slots, topk, shared_ff=0, fp8=False):
     """WeightFormat::expert_gemm_i8 (weight_format.hpp:54-56), per-token scales, one input row per assignment: fp16
     y [n * slots][rows]."""
     counts, offsets, perm = lists
     y = torch.zeros((n * slots, bank.rows), dtype=torch.float16, device=xq.device)
     err = _err()
     b = bank.view()
-    _check(lib().tqmoe_expert_gemm_i8(C.byref(b), _ptr(xq), _ptr(xs), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff, _ptr(y),
-                                      _stream(xq), C.byref(err)), err)
+    fn = lib().tqmoe_expert_gemm_fp8 if fp8 else lib().tqmoe_expert_gemm_i8
+    _check(fn(C.byref(b), _ptr(xq), _ptr(xs), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff, _ptr(y), _stream(xq), C.byref(err)), err)
     return y
+
+
+def expert_gemm_fp8(bank, xq, xs, lists, n, slots, topk, shared_ff=0):
+    return expert_gemm_i8(bank, xq, xs, lists, n, slots, topk, shared_ff, fp8=True)
 
 
 def moe_swiglu(gate, up):

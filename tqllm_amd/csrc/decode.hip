@@ -4,8 +4,8 @@
 
 namespace tqmoe {
 int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);  // bank.hip
-// prefill_iq4xs.hip
-int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, hipStream_t s);
+// prefill_planes.hip (f8: E4M3 operand bytes in place of int8)
+int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, hipStream_t s, bool f8);
 int32_t enqueue_gemm_f16(const tqmoe_bank & b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int * counts, const int * offsets, const int * perm,
                          int experts, int64_t assignments, int xdiv, void * out, uint32_t out_type, int gateup, int shared_expert, int shared_lim, hipStream_t s);
 int64_t grouped_row_tiles(int64_t assignments, int experts);
@@ -13,8 +13,10 @@ int64_t grouped_scale_words(int64_t assignments, int experts);
 int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, const int * counts, const int * offsets, const int * perm, int experts,
                                int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s);
 int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
-                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s);
-int32_t enqueue_iq4xs_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
+                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8);
+bool plane_gemm_has(uint32_t type);
+bool plane_gemm_is_fp8(uint32_t type);
+int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
                            const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s);
 
 namespace {
@@ -327,12 +329,21 @@ extern "C" int32_t tqmoe_combine(const float * routed, const float * shared, con
     return tqmoe_combine_strided(routed, topk, shared, hidden, weights, shared_weights, out, otype, hidden, topk, n, stream, err);
 }
 
+static int32_t quant_rows_common(const void * x, uint32_t xtype, int64_t rows, int32_t cols, void * q, float * scale, void * stream, tqmoe_error * err, bool f8,
+                                 const char * what) {
+    if (!x || !q || !scale || rows <= 0 || cols <= 0 || cols % 32 || (rows + 3) / 4 > 0x7FFFFFFF) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported element type", what);
+    if (int32_t rc = need_device(err, what)) return rc;
+    enqueue_quant_rows_i8(x, xtype, rows, cols, static_cast<int8_t *>(q), scale, static_cast<hipStream_t>(stream), f8);
+    return launched(err, what);
+}
+
 extern "C" int32_t tqmoe_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int32_t cols, int8_t * q, float * scale, void * stream, tqmoe_error * err) {
-    if (!x || !q || !scale || rows <= 0 || cols <= 0 || cols % 32 || (rows + 3) / 4 > 0x7FFFFFFF) return fail(err, TQMOE_E_ARG, "tqmoe_quant_rows_i8: invalid shape or pointer");
-    if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_quant_rows_i8: unsupported element type");
-    if (int32_t rc = need_device(err, "tqmoe_quant_rows_i8")) return rc;
-    enqueue_quant_rows_i8(x, xtype, rows, cols, q, scale, static_cast<hipStream_t>(stream));
-    return launched(err, "tqmoe_quant_rows_i8");
+    return quant_rows_common(x, xtype, rows, cols, q, scale, stream, err, false, "tqmoe_quant_rows_i8");
+}
+
+extern "C" int32_t tqmoe_quant_rows_fp8(const void * x, uint32_t xtype, int64_t rows, int32_t cols, uint8_t * q, float * scale, void * stream, tqmoe_error * err) {
+    return quant_rows_common(x, xtype, rows, cols, q, scale, stream, err, true, "tqmoe_quant_rows_fp8");
 }
 
 extern "C" int64_t tqmoe_grouped_rows(int64_t assignments, int32_t experts) {
@@ -343,15 +354,25 @@ extern "C" int64_t tqmoe_grouped_scale_words(int64_t assignments, int32_t expert
     return assignments > 0 && experts > 0 ? grouped_scale_words(assignments, experts) : 0;
 }
 
-extern "C" int32_t tqmoe_group_rows_i8(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm,
-                                       int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q, float * scale, void * stream, tqmoe_error * err) {
+static int32_t group_rows_common(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t experts,
+                                 int64_t assignments, int32_t xdiv, void * q, float * scale, void * stream, tqmoe_error * err, bool f8, const char * what) {
     if (!x || !counts || !offsets || !perm || !q || !scale || cols <= 0 || cols % 32 || experts <= 0 || experts > 4096 || assignments <= 0 || xdiv <= 0 ||
         grouped_row_tiles(assignments, experts) > 0x7FFFFFFF)
-        return fail(err, TQMOE_E_ARG, "tqmoe_group_rows_i8: invalid shape or pointer");
-    if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_group_rows_i8: unsupported element type");
-    if (int32_t rc = need_device(err, "tqmoe_group_rows_i8")) return rc;
-    enqueue_group_rows_i8(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, static_cast<hipStream_t>(stream));
-    return launched(err, "tqmoe_group_rows_i8");
+        return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported element type", what);
+    if (int32_t rc = need_device(err, what)) return rc;
+    enqueue_group_rows_i8(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, static_cast<int8_t *>(q), scale, static_cast<hipStream_t>(stream), f8);
+    return launched(err, what);
+}
+
+extern "C" int32_t tqmoe_group_rows_i8(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm,
+                                       int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q, float * scale, void * stream, tqmoe_error * err) {
+    return group_rows_common(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, stream, err, false, "tqmoe_group_rows_i8");
+}
+
+extern "C" int32_t tqmoe_group_rows_fp8(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm,
+                                        int32_t experts, int64_t assignments, int32_t xdiv, uint8_t * q, float * scale, void * stream, tqmoe_error * err) {
+    return group_rows_common(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, stream, err, true, "tqmoe_group_rows_fp8");
 }
 
 extern "C" int32_t tqmoe_gather_rows_i8(const int8_t * rows_q, const float * rows_scale, int32_t cols, const int32_t * counts, const int32_t * offsets,
@@ -367,21 +388,24 @@ extern "C" int32_t tqmoe_gather_rows_i8(const int8_t * rows_q, const float * row
 
 static int32_t gemm_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                            const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
-                           tqmoe_error * err, const char * what) {
+                           tqmoe_error * err, const char * what, bool fp8) {
     if (int32_t rc = check_bank(b0, what, err)) return rc;
     if (b1) {
         if (int32_t rc = check_bank(b1, what, err)) return rc;
         if (b1->type != b0->type || b1->rows != b0->rows || b1->cols != b0->cols || b1->experts != b0->experts)
             return fail(err, TQMOE_E_ARG, "%s: the two banks differ in format or shape", what);
     }
-    if (b0->type != TQMOE_IQ4_XS) return fail(err, TQMOE_E_UNSUPPORTED, "%s: no int8 grouped product for bank type %u (false in the reference's terms: use the decode products)", what, b0->type);
+    if (!plane_gemm_has(b0->type) || plane_gemm_is_fp8(b0->type) != fp8)
+        return fail(err, TQMOE_E_UNSUPPORTED, "%s: no %s grouped product for bank type %u (false in the reference's terms: use the fp16 grouped or the decode products)", what,
+                    fp8 ? "fp8" : "int8", b0->type);
+    if (b0->cols % 256 || b0->rows % 32) return fail(err, TQMOE_E_UNSUPPORTED, "%s: the bank's rows must be a multiple of 32 and its columns of 256", what);
     if (!xq || !xs || !counts || !offsets || !perm || !out || n <= 0 || topk <= 0 || slots < topk) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
     const int lim_max = gateup ? b0->rows : b0->cols;
     if (slots > topk && (shared_lim <= 0 || shared_lim > lim_max || shared_lim % 256)) return fail(err, TQMOE_E_ARG, "%s: shared_lim must be a multiple of 256 within the bank", what);
     if (b0->experts > 4096) return fail(err, TQMOE_E_ARG, "%s: more than 4096 experts", what);
     if (int32_t rc = need_device(err, what)) return rc;
     const int shared_expert = slots > topk ? b0->experts - 1 : -1;
-    if (enqueue_iq4xs_gemm(*b0, b1, xq, xs, counts, offsets, perm, b0->experts, int64_t(n) * slots, out, gateup, shared_expert, shared_lim,
+    if (enqueue_plane_gemm(*b0, b1, xq, xs, counts, offsets, perm, b0->experts, int64_t(n) * slots, out, gateup, shared_expert, shared_lim,
                            static_cast<hipStream_t>(stream)))
         return fail(err, TQMOE_E_ARG, "%s: too many assignments for one call", what);
     return launched(err, what);
@@ -391,13 +415,28 @@ extern "C" int32_t tqmoe_expert_gemm_gateup_i8(const tqmoe_bank * gate, const tq
                                                const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim,
                                                void * act_f16, void * stream, tqmoe_error * err) {
     if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_gemm_gateup_i8: second bank missing");
-    return gemm_common(gate, up, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err, "tqmoe_expert_gemm_gateup_i8");
+    return gemm_common(gate, up, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err, "tqmoe_expert_gemm_gateup_i8", false);
 }
 
 extern "C" int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                                         const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * y_f16, void * stream,
                                         tqmoe_error * err) {
-    return gemm_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8");
+    return gemm_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8", false);
+}
+
+extern "C" int32_t tqmoe_expert_gemm_gateup_fp8(const tqmoe_bank * gate, const tqmoe_bank * up, const uint8_t * xq, const float * xs, const int32_t * counts,
+                                                const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim,
+                                                void * act_f16, void * stream, tqmoe_error * err) {
+    if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_gemm_gateup_fp8: second bank missing");
+    return gemm_common(gate, up, reinterpret_cast<const int8_t *>(xq), xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err,
+                       "tqmoe_expert_gemm_gateup_fp8", true);
+}
+
+extern "C" int32_t tqmoe_expert_gemm_fp8(const tqmoe_bank * bank, const uint8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
+                                         const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * y_f16, void * stream,
+                                         tqmoe_error * err) {
+    return gemm_common(bank, nullptr, reinterpret_cast<const int8_t *>(xq), xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err,
+                       "tqmoe_expert_gemm_fp8", true);
 }
 
 static int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int32_t * counts, const int32_t * offsets,

@@ -8,6 +8,8 @@ int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err);
 int32_t enqueue_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t * ext_ids, int32_t extra, const void * x,
                      uint32_t xtype, int32_t cols, void * image, int32_t experts, int32_t topk, int32_t n, float scale, int32_t gating,
                      const float * bias, int32_t norm, hipStream_t s, int32_t shared_ungated);
+bool plane_gemm_has(uint32_t type);
+bool plane_gemm_is_fp8(uint32_t type);
 
 namespace {
 
@@ -26,7 +28,11 @@ struct Plan {  // byte offsets into the workspace
     size_t xq, xs, counts, offsets, perm, dispatch_ws, act16, aq, as, y16, rq, rs;   // grouped path
 };
 
-bool int8_ok(const tqmoe_layer & L) { return L.gate.type == TQMOE_IQ4_XS && L.down.type == TQMOE_IQ4_XS && (!L.has_shared || L.shared_ff % 256 == 0); }
+// the 8-bit grouped products: both banks' formats have one with the same operand type (int8, or E4M3 for NVFP4G)
+bool int8_ok(const tqmoe_layer & L) {
+    return plane_gemm_has(L.gate.type) && plane_gemm_has(L.down.type) && plane_gemm_is_fp8(L.gate.type) == plane_gemm_is_fp8(L.down.type) &&
+           L.hidden % 256 == 0 && L.ff % 256 == 0 && (!L.has_shared || L.shared_ff % 256 == 0);
+}
 
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
@@ -116,7 +122,7 @@ extern "C" size_t tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t
 extern "C" int32_t tqmoe_layer_path(const tqmoe_layer * layer, int32_t n) {
     if (!layer || n <= 0 || check_layer(layer, nullptr)) return TQMOE_E_ARG;
     const Plan p = plan_for(*layer, n);
-    return p.int8 ? TQMOE_PATH_GROUPED_I8 : p.grouped ? TQMOE_PATH_GROUPED_F16 : TQMOE_PATH_DECODE;
+    return p.int8 ? (plane_gemm_is_fp8(layer->gate.type) ? TQMOE_PATH_GROUPED_FP8 : TQMOE_PATH_GROUPED_I8) : p.grouped ? TQMOE_PATH_GROUPED_F16 : TQMOE_PATH_DECODE;
 }
 
 static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t xtype, const void * residual, int32_t n, void * out, uint32_t otype,
@@ -181,11 +187,20 @@ static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t
             } else {
             int8_t * rq = reinterpret_cast<int8_t *>(ws + p.rq);
             float * rs = reinterpret_cast<float *>(ws + p.rs);
+            if (plane_gemm_is_fp8(L.gate.type)) {
+                uint8_t * xq8 = reinterpret_cast<uint8_t *>(xq), * aq8 = reinterpret_cast<uint8_t *>(aq);
+                if (int32_t rc = tqmoe_quant_rows_fp8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, reinterpret_cast<uint8_t *>(rq), rs, stream, err)) return rc;
+                if (int32_t rc = tqmoe_gather_rows_i8(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, stream, err)) return rc;
+                if (int32_t rc = tqmoe_expert_gemm_gateup_fp8(&L.gate, &L.up, xq8, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
+                if (int32_t rc = tqmoe_group_rows_fp8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq8, as, stream, err)) return rc;
+                if (int32_t rc = tqmoe_expert_gemm_fp8(&L.down, aq8, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
+            } else {
             if (int32_t rc = tqmoe_quant_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, rq, rs, stream, err)) return rc;
             if (int32_t rc = tqmoe_gather_rows_i8(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_gateup_i8(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
             if (int32_t rc = tqmoe_group_rows_i8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_i8(&L.down, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
+            }
             }
             if (int32_t rc = combine(y16, TQMOE_F16, L.has_shared ? y16 + size_t(L.topk) * L.hidden : nullptr)) return rc;
         } else {

@@ -1,15 +1,22 @@
-// Prefill-sized expert products of IQ4_XS banks: a grouped int8 x int8 -> int32 GEMM on the matrix pipe.
+// Prefill-sized expert products on the matrix pipe with 8-bit operands: grouped int8 x int8 -> int32 GEMMs for IQ4_XS,
+// IQ3_S and Q4_K banks (exact weights), and an fp8 x fp8 -> fp32 GEMM for NVFP4G banks (weights widened to E4M3).
 //
-// Operands. Activations are int8 per input row (one fp32 scale per row, amax / 127). The rows of every expert's
-// assignments are gathered into tiles of 32 rows, experts in order, each expert padded to whole tiles, and stored
-// operand-major: the 1 KB that the 64 lanes of a wave feed to one v_mfma_i32_32x32x32_i8 as operand A (lane = 32 g + r
-// holds, for row r and 32-weight sub-block j, the 16 values {8g..8g+7} and {16+8g..16+8g+7} in the byte order of the
-// bank's code bytes) is contiguous, sub-blocks in order. A wave then loads its operand with one fully coalesced
-// instruction and no shuffle.
-// Weights stay exact. An IQ4_XS value is d * (ls - 32) * kv[q]: the product (ls - 32) * kv[q] (13 bits) is split as
-// 64 * h + l with h, l int8, taken per sub-block from a 64-entry table of 16-value lookup tables in LDS and applied with
-// v_perm_b32. The two planes go through two MFMAs that accumulate over the whole 256-weight super-block, so the scales
-// cost no vector instruction per product; per super-block the results fold as acc += d * (64 * acc_h + acc_l) in fp32.
+// Operands. Activations are 8 bits per input row with one fp32 scale per row: int8 (amax / 127) or E4M3 (amax / 448). The
+// rows of every expert's assignments are gathered into tiles of 32 rows, experts in order, each expert padded to whole
+// tiles, and stored operand-major: the 1 KB that the 64 lanes of a wave feed to one v_mfma_i32_32x32x32_i8 as operand A
+// (lane = 32 g + r holds, for row r and 32-weight sub-block j, the 16 values {8g..8g+7} and {16+8g..16+8g+7} in the byte
+// order of the bank's code bytes) is contiguous, sub-blocks in order. A wave then loads its operand with one fully
+// coalesced instruction and no shuffle. The two 8-byte halves of that operand are the operands of two
+// v_mfma_f32_32x32x16_fp8_fp8, so the fp8 path shares the layout.
+// Integer weights stay exact. A value is d * p with an integer p per weight of up to 13 bits (IQ4_XS: (ls - 32) * kv[q];
+// IQ3_S: (1 + 2 ls) * (+-lattice magnitude); Q4_K: sc * q, with the minimum's coefficient mn as a further plane that
+// is constant over a sub-block). p is split as 64 * h + l with h, l int8, taken per sub-block from 16-entry lookup
+// tables in LDS (one pair per scale value) and applied with v_perm_b32. The planes go through one MFMA each that
+// accumulate over the whole 256-weight super-block, so the scales cost no vector instruction per product; per
+// super-block the results fold as acc += d * (64 * acc_h + acc_l) - dmin * acc_m in fp32.
+// NVFP4G weights are e2m1 * E4M3 scale (per 16 weights) * fp32 global (per row): the product of the first two is rounded
+// to E4M3 (a declared lossy operand: six significant bits into four), again through a 16-entry table per scale byte; the
+// fp8 MFMA accumulates in fp32 over the whole row and the global multiplies the result.
 //
 // Blocks. A work item is one expert, a chunk of up to kChunkTiles row tiles of its assignments and one unit of weight
 // rows: 32 rows of both banks (gate / up, SwiGLU fused) or 64 rows of one bank (down). Resident blocks of eight waves
@@ -17,9 +24,9 @@
 // unit's weights once into a double-buffered LDS stage that every wave then reads as operand B (decoding super-block
 // i + 1 overlaps the products of super-block i, one barrier per super-block); a wave multiplies one row tile with the
 // weights of both operand slots, so a loaded piece of operand A (prefetched into registers a few k-steps ahead) serves
-// four products and SwiGLU pairs values the same lane holds. A chunk of a single row tile has nothing to share: every
-// wave then takes the tile against 32 weight rows of its own (four units per item), decoding straight into registers
-// with no barrier in the loop.
+// every product with it and SwiGLU pairs values the same lane holds. A chunk of a single row tile has nothing to share:
+// every wave then takes the tile against 32 weight rows of its own (four units per item), decoding straight into
+// registers with no barrier in the loop.
 #include "act_image.cuh"
 #include "decode_api.cuh"
 #include "formats.cuh"
@@ -36,19 +43,24 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kChunkTiles = 8;                // row tiles (of 32 assignments) per chunk
 constexpr int kPlanExperts = 1024;              // experts whose index a block keeps in LDS
 
-__device__ __forceinline__ v4i decode16(uint2 c) {
-    v4i w;
-    uint32_t lo, hi;
-    lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(c.x, lo, hi);
-    w[0] = int(lo); w[1] = int(hi);
-    lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(c.y, lo, hi);
-    w[2] = int(lo); w[3] = int(hi);
-    return w;
+// four scaled values -> four operand bytes: int8 (round to nearest) or E4M3 (round to nearest even; the values are
+// clamped to +-448 first, so the conversion never leaves the finite codes)
+template <bool F8> __device__ __forceinline__ uint32_t pack4_q(float a, float b, float c, float d) {
+    if constexpr (F8) {
+        auto clamp = [](float v) { return fminf(fmaxf(v, -448.f), 448.f); };
+        int w = __builtin_amdgcn_cvt_pk_fp8_f32(clamp(a), clamp(b), 0, false);
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(clamp(c), clamp(d), w, true);
+        return uint32_t(w);
+    } else {
+        return uint32_t(__float2int_rn(a) & 0xFF) | uint32_t(__float2int_rn(b) & 0xFF) << 8 | uint32_t(__float2int_rn(c) & 0xFF) << 16 |
+               uint32_t(__float2int_rn(d) & 0xFF) << 24;
+    }
 }
+template <bool F8> constexpr float kOperandMax = F8 ? 448.f : 127.f;
 
-// rows of int8 activations: q = rint(x * 127 / amax) per row, scale = amax / 127; one wave per row
-template <int XT>
-__global__ __launch_bounds__(256) void quant_rows_i8_k(const void * __restrict__ x, int64_t rows, int cols, int8_t * __restrict__ q, float * __restrict__ scale) {
+// rows of 8-bit activations: q = rint(x * 127 / amax) per row, scale = amax / 127 (E4M3: 448 in place of 127); one wave per row
+template <int XT, bool F8>
+__global__ __launch_bounds__(256) void quant_rows_k(const void * __restrict__ x, int64_t rows, int cols, int8_t * __restrict__ q, float * __restrict__ scale) {
     const int lane = threadIdx.x & 63;
     const int64_t row = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -66,15 +78,13 @@ __global__ __launch_bounds__(256) void quant_rows_i8_k(const void * __restrict__
     amax = fmaxf(amax, dpp_f<kDppMirror>(amax));
     amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
     amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-    const float mul = amax > 0.f ? 127.f / amax : 0.f;
-    if (lane == 0) scale[row] = amax / 127.f;
+    const float mul = amax > 0.f ? kOperandMax<F8> / amax : 0.f;
+    if (lane == 0) scale[row] = amax / kOperandMax<F8>;
     uint32_t * out = reinterpret_cast<uint32_t *>(q + row * cols);
     for (int gi = lane; gi < groups; gi += 64) {
         float v[8];
         load8<XT>(x, row * cols + gi * 8, v);
-        uint32_t w[2] = {0, 0};
-#pragma unroll
-        for (int j = 0; j < 8; ++j) w[j >> 2] |= uint32_t(__float2int_rn(v[j] * mul) & 0xFF) << (8 * (j & 3));
+        const uint32_t w[2] = {pack4_q<F8>(v[0] * mul, v[1] * mul, v[2] * mul, v[3] * mul), pack4_q<F8>(v[4] * mul, v[5] * mul, v[6] * mul, v[7] * mul)};
         const int blk = gi >> 2, d0 = 2 * (gi & 3);
         out[blk * 8 + plane_pos(d0)] = w[0];
         out[blk * 8 + plane_pos(d0 + 1)] = w[1];
@@ -127,8 +137,8 @@ __device__ __forceinline__ int owner_of(const int * __restrict__ base, int exper
 // Rows of the grouped operand: block b takes rows [8 (b % 4), +8) of row tile b / 4, one wave per two rows. Row i of
 // expert e's tiles is assignment perm[offsets[e] + i], its source row a / xdiv. Rows past the expert's count are left as
 // they are (their products are never stored).
-template <int XT>
-__global__ __launch_bounds__(256) void group_rows_i8_k(const void * __restrict__ x, int cols, const int * __restrict__ counts, const int * __restrict__ offsets,
+template <int XT, bool F8>
+__global__ __launch_bounds__(256) void group_rows_k(const void * __restrict__ x, int cols, const int * __restrict__ counts, const int * __restrict__ offsets,
                                                          const int * __restrict__ perm, int experts, int xdiv, int8_t * __restrict__ q, float * __restrict__ scale,
                                                          Plan plan) {
     const int tile_index = int(blockIdx.x >> 2);
@@ -151,14 +161,12 @@ __global__ __launch_bounds__(256) void group_rows_i8_k(const void * __restrict__
             for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
         }
         amax = wave_max(amax);
-        const float mul = amax > 0.f ? 127.f / amax : 0.f;
-        if (lane == 0) scale[int64_t(tile_index) * 32 + r] = amax / 127.f;
+        const float mul = amax > 0.f ? kOperandMax<F8> / amax : 0.f;
+        if (lane == 0) scale[int64_t(tile_index) * 32 + r] = amax / kOperandMax<F8>;
         for (int gi = lane; gi < groups; gi += 64) {
             float v[8];
             load8<XT>(x, row * cols + gi * 8, v);
-            uint32_t wd[2] = {0, 0};
-#pragma unroll
-            for (int j = 0; j < 8; ++j) wd[j >> 2] |= uint32_t(__float2int_rn(v[j] * mul) & 0xFF) << (8 * (j & 3));
+            const uint32_t wd[2] = {pack4_q<F8>(v[0] * mul, v[1] * mul, v[2] * mul, v[3] * mul), pack4_q<F8>(v[4] * mul, v[5] * mul, v[6] * mul, v[7] * mul)};
             const int sub = gi >> 2, d0 = 2 * (gi & 3);
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
@@ -173,8 +181,8 @@ __global__ __launch_bounds__(256) void group_rows_i8_k(const void * __restrict__
 // (one read of the input) into an LDS copy of the tile, every 32-byte block already in operand order; then lane (g, r)
 // of every wave moves the 16 bytes of row r, half g of one k-step at a time, so each k-step's 1 KB leaves as one fully
 // coalesced store instead of 256 scattered dwords.
-template <int XT, int GPL>   // groups of 8 values per lane: cols = 512 GPL
-__global__ __launch_bounds__(256) void group_rows_i8_tile_k(const void * __restrict__ x, int cols, const int * __restrict__ counts, const int * __restrict__ offsets,
+template <int XT, int GPL, bool F8>   // groups of 8 values per lane: cols = 512 GPL
+__global__ __launch_bounds__(256) void group_rows_tile_k(const void * __restrict__ x, int cols, const int * __restrict__ counts, const int * __restrict__ offsets,
                                                               const int * __restrict__ perm, int experts, int xdiv, int8_t * __restrict__ q, float * __restrict__ scale,
                                                               Plan plan) {
     extern __shared__ __attribute__((aligned(16))) uint8_t tile_rows[];   // [32][cols + 16]
@@ -203,15 +211,14 @@ __global__ __launch_bounds__(256) void group_rows_i8_tile_k(const void * __restr
 #pragma unroll
                 for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[b][gq][j]));
             amax = wave_max(amax);
-            const float mul = amax > 0.f ? 127.f / amax : 0.f;
+            const float mul = amax > 0.f ? kOperandMax<F8> / amax : 0.f;
             if (first + r < cnt) {
-                if (lane == 0) scale[int64_t(tile_index) * 32 + r] = amax / 127.f;
+                if (lane == 0) scale[int64_t(tile_index) * 32 + r] = amax / kOperandMax<F8>;
 #pragma unroll
                 for (int gq = 0; gq < GPL; ++gq) {
                     const int gi = lane + 64 * gq, sub = gi >> 2, d0 = 2 * (gi & 3);
-                    uint32_t wd[2] = {0, 0};
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) wd[j >> 2] |= uint32_t(__float2int_rn(v[b][gq][j] * mul) & 0xFF) << (8 * (j & 3));
+                    const float * vv = v[b][gq];
+                    const uint32_t wd[2] = {pack4_q<F8>(vv[0] * mul, vv[1] * mul, vv[2] * mul, vv[3] * mul), pack4_q<F8>(vv[4] * mul, vv[5] * mul, vv[6] * mul, vv[7] * mul)};
 #pragma unroll
                     for (int h = 0; h < 2; ++h) *reinterpret_cast<uint32_t *>(tile_rows + r * stride + sub * 32 + plane_pos(d0 + h) * 4) = wd[h];
                 }
@@ -247,8 +254,6 @@ __global__ __launch_bounds__(256) void gather_rows_i8_k(const int8_t * __restric
     for (int ks = wave; ks < S; ks += 4) dst[ks * 64] = src[ks * 2];
 }
 
-struct Where { int expert, local, tile_base; };
-
 struct GemmArgs {
     BankView b0, b1;          // gate and up; down: the same bank twice
     const int8_t * xq;        // grouped operand-major row tiles
@@ -265,18 +270,36 @@ struct GemmArgs {
     int shared_lim;
 };
 
-// 16 codes (two dwords) through the two 16-entry tables of their sub-block scale: h and l planes, 16 int8 each
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+// four codes (bytes of idx3: index within a table half; sel: position + 4 * half) through a 16-entry byte table
+__device__ __forceinline__ int pick16(uint4 t, uint32_t idx3, uint32_t sel) {
+    return int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(t.w, t.z, idx3), __builtin_amdgcn_perm(t.y, t.x, idx3), sel));
+}
+// the eight 4-bit codes of a dword as lookup keys: low nibbles (weights j) and high nibbles (weights j + 16)
+struct NibbleKeys { uint32_t i_lo, s_lo, i_hi, s_hi; };
+__device__ __forceinline__ NibbleKeys nibble_keys(uint32_t c) {
+    return NibbleKeys{c & 0x07070707u, ((c >> 1) & 0x04040404u) | 0x03020100u, (c >> 4) & 0x07070707u, ((c >> 5) & 0x04040404u) | 0x03020100u};
+}
+// 16 codes (two dwords) through the two 16-entry tables of their sub-block scale: h and l planes, 16 int8 each, in operand
+// order (values 8g.., 16 + 8g.., 8g + 4.., 16 + 8g + 4..)
 __device__ __forceinline__ void decode_planes(uint2 c, uint4 th, uint4 tl, v4i & h, v4i & l) {
     const uint32_t cw[2] = {c.x, c.y};
 #pragma unroll
     for (int w = 0; w < 2; ++w) {
-        const uint32_t i_lo = cw[w] & 0x07070707u, i_hi = (cw[w] >> 4) & 0x07070707u;
-        const uint32_t s_lo = ((cw[w] >> 1) & 0x04040404u) | 0x03020100u, s_hi = ((cw[w] >> 5) & 0x04040404u) | 0x03020100u;
-        h[2 * w] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(th.w, th.z, i_lo), __builtin_amdgcn_perm(th.y, th.x, i_lo), s_lo));
-        h[2 * w + 1] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(th.w, th.z, i_hi), __builtin_amdgcn_perm(th.y, th.x, i_hi), s_hi));
-        l[2 * w] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(tl.w, tl.z, i_lo), __builtin_amdgcn_perm(tl.y, tl.x, i_lo), s_lo));
-        l[2 * w + 1] = int(__builtin_amdgcn_perm(__builtin_amdgcn_perm(tl.w, tl.z, i_hi), __builtin_amdgcn_perm(tl.y, tl.x, i_hi), s_hi));
+        const NibbleKeys k = nibble_keys(cw[w]);
+        h[2 * w] = pick16(th, k.i_lo, k.s_lo);
+        h[2 * w + 1] = pick16(th, k.i_hi, k.s_hi);
+        l[2 * w] = pick16(tl, k.i_lo, k.s_lo);
+        l[2 * w + 1] = pick16(tl, k.i_hi, k.s_hi);
     }
+}
+// an integer of up to 13 bits as 64 * hi + lo with lo in [-32, 32) and both in int8
+__device__ __forceinline__ void split_planes(int v, uint8_t & hi, uint8_t & lo) {
+    const int l = ((v + 32) & 63) - 32;
+    lo = uint8_t(l);
+    hi = uint8_t((v - l) >> 6);
 }
 
 // The two ways through the kernel (a lone row tile, a shared chunk) must give a row the same bits: the fold of a
@@ -297,15 +320,210 @@ __device__ __forceinline__ uint16_t scaled_half(float acc, float sc) { return to
 
 __device__ const int8_t kIq4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
-// dynamic LDS: [2 stages][NB][plane h, l][8 sub-blocks][64 lanes] v4i of decoded weights.
+// ------------------------------------------------------------------------------------------------ bank formats
+// What the kernel needs of a format. Lane (n, g) of a wave holds, of weight row n of a 32-row tile and one sub-block, the
+// 16 weights {8g..8g+7} and {16+8g..16+8g+7}: Src are its base pointers, Code what it loads per sub-block, Rec what
+// decoding needs of the sub-block's super-block, DRec what the fold needs of it (the lane's row, any g).
+// planes() turns a Code into kPlanes operand registers; tables() fills the lookup tables (and the lattice) in LDS.
+struct WIq4xs {   // tile-major codes (512 B per sub-block of a tile), 8-byte records (256 B per super-block of a tile)
+    static constexpr int kPlanes = 2, kTabBytes = 64 * 32, kLattice = 1;
+    static constexpr bool kFp8 = false, kMin = false, kRowMul = false;
+    struct Code { uint2 c; };
+    typedef uint2 Rec;
+    typedef uint2 DRec;
+    struct Src { const uint8_t * codes, * aux; };
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t *, int tid, int threads) {   // per 6-bit scale: 16 h bytes, 16 l bytes
+        for (int i = tid; i < 64 * 16; i += threads) split_planes(int(kIq4Values[i & 15]) * ((i >> 4) - 32), tab[(i >> 4) * 32 + (i & 15)], tab[(i >> 4) * 32 + 16 + (i & 15)]);
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int g) {
+        const int S = b.cols / 32;
+        const int64_t tile_g = int64_t(e) * (b.rows / 32) + wtile;
+        return Src{b.codes + tile_g * S * 512 + n * 16 + g * 8, b.aux + tile_g * (S / 8) * 256 + n * 8};
+    }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) { return Code{*reinterpret_cast<const uint2 *>(s.codes + int64_t(sub) * 512)}; }
+    static __device__ __forceinline__ Rec rec(const Src & s, int sb) { return *reinterpret_cast<const uint2 *>(s.aux + int64_t(sb) * 256); }
+    static __device__ __forceinline__ DRec drec(const Src & s, int sb) { return rec(s, sb); }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec & r, int ib, int, const uint8_t * tab, const uint32_t *, v4i * p) {
+        const uint4 * t = reinterpret_cast<const uint4 *>(tab + iq4xs_ls(r, ib) * 32);
+        decode_planes(c.c, t[0], t[1], p[0], p[1]);
+    }
+    static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(iq4xs_d_bits(r)); }
+    static __device__ __forceinline__ float dmin(const DRec &) { return 0.f; }
+    static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
+};
+
+struct WQ4k {   // row-major: 16 code bytes per sub-block, a 16-byte record (d | dmin << 16, twelve bytes of 6-bit scales and minimums) per super-block
+    static constexpr int kPlanes = 3, kTabBytes = 64 * 32, kLattice = 1;
+    static constexpr bool kFp8 = false, kMin = true, kRowMul = false;
+    struct Code { uint2 c; };
+    typedef uint4 Rec;
+    typedef uint32_t DRec;
+    struct Src { const uint8_t * codes, * aux; };
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t *, int tid, int threads) {   // per 6-bit scale sc: sc * q for the 16 codes
+        for (int i = tid; i < 64 * 16; i += threads) split_planes((i & 15) * (i >> 4), tab[(i >> 4) * 32 + (i & 15)], tab[(i >> 4) * 32 + 16 + (i & 15)]);
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int g) {
+        const int S = b.cols / 32;
+        const int64_t row = int64_t(e) * b.rows + wtile * 32 + n;
+        return Src{b.codes + row * S * 16 + g * 8, b.aux + row * (S / 8) * 16};
+    }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) { return Code{*reinterpret_cast<const uint2 *>(s.codes + int64_t(sub) * 16)}; }
+    static __device__ __forceinline__ Rec rec(const Src & s, int sb) { return *reinterpret_cast<const uint4 *>(s.aux + int64_t(sb) * 16); }
+    static __device__ __forceinline__ DRec drec(const Src & s, int sb) { return *reinterpret_cast<const uint32_t *>(s.aux + int64_t(sb) * 16); }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec & r, int ib, int, const uint8_t * tab, const uint32_t *, v4i * p) {
+        const uint32_t sc12[3] = {r.y, r.z, r.w};
+        int sc, mn;
+        q4k_scale_min(sc12, ib, sc, mn);
+        const uint4 * t = reinterpret_cast<const uint4 *>(tab + sc * 32);
+        decode_planes(c.c, t[0], t[1], p[0], p[1]);
+        const int m = mn * 0x01010101;   // the minimum's coefficient, the same for the sub-block's 32 weights
+        p[2] = v4i{m, m, m, m};
+    }
+    static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(uint16_t(r & 0xFFFFu)); }
+    static __device__ __forceinline__ float dmin(const DRec & r) { return half_bits_to_float(uint16_t(r >> 16)); }
+    static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
+};
+
+struct WIq3s {   // row-major: 12 code bytes per sub-block (8 lattice indices, 32 sign bits), a 16-byte record per super-block
+    static constexpr int kPlanes = 2, kTabBytes = 16 * 32, kLattice = 512;
+    static constexpr bool kFp8 = false, kMin = false, kRowMul = false;
+    struct Code { uint32_t qs0, qs1, sg; };
+    typedef uint4 Rec;       // d | qh[0..1] << 16, qh[2..5], qh[6..7] | scales[0..1] << 16, scales[2..3]
+    typedef uint32_t DRec;
+    struct Src { const uint8_t * codes, * aux; };
+    // per 4-bit scale ls the 16 products (1 + 2 ls) * (+-(2 j + 1)): code = sign << 3 | magnitude index j
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t * lat, int tid, int threads) {
+        for (int i = tid; i < 16 * 16; i += threads) {
+            const int mag = (1 + 2 * (i >> 4)) * (2 * (i & 7) + 1);
+            split_planes((i & 8) ? -mag : mag, tab[(i >> 4) * 32 + (i & 15)], tab[(i >> 4) * 32 + 16 + (i & 15)]);
+        }
+        for (int i = tid; i < 512; i += threads) lat[i] = d_iq3s_grid.v[i];
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int) {
+        const int S = b.cols / 32;
+        const int64_t row = int64_t(e) * b.rows + wtile * 32 + n;
+        return Src{b.codes + row * S * 12, b.aux + row * (S / 8) * 16};
+    }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) {
+        const uint32_t * c = reinterpret_cast<const uint32_t *>(s.codes + int64_t(sub) * 12);
+        return Code{c[0], c[1], c[2]};
+    }
+    static __device__ __forceinline__ Rec rec(const Src & s, int sb) { return *reinterpret_cast<const uint4 *>(s.aux + int64_t(sb) * 16); }
+    static __device__ __forceinline__ DRec drec(const Src & s, int sb) { return *reinterpret_cast<const uint32_t *>(s.aux + int64_t(sb) * 16); }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec & r, int ib, int g, const uint8_t * tab, const uint32_t * lat, v4i * p) {
+        const uint32_t qh = ib < 2 ? (r.x >> (16 + 8 * ib)) & 0xFFu : ib < 6 ? (r.y >> (8 * (ib - 2))) & 0xFFu : (r.z >> (8 * (ib - 6))) & 0xFFu;
+        const uint32_t scb = (ib >> 1) < 2 ? (r.z >> (16 + 8 * (ib >> 1))) & 0xFFu : (r.w >> (8 * ((ib >> 1) - 2))) & 0xFFu;
+        const uint4 * t = reinterpret_cast<const uint4 *>(tab + ((scb >> (4 * (ib & 1))) & 15u) * 32);
+        const uint4 th = t[0], tl = t[1];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {   // operand dword q = the group of four weights 2 g + q / 2 (+ 4 for odd q)
+            const int w = 2 * g + (q >> 1) + 4 * (q & 1);
+            const uint32_t idx = (((w < 4 ? c.qs0 : c.qs1) >> (8 * (w & 3))) & 0xFFu) | (((qh >> w) & 1u) << 8);
+            const uint32_t mag = lat[idx];                                      // bytes 1, 3, .., 15
+            const uint32_t i3 = (mag >> 1) & 0x07070707u, sel = (spread4(c.sg >> (4 * w)) << 2) | 0x03020100u;
+            p[0][q] = pick16(th, i3, sel);
+            p[1][q] = pick16(tl, i3, sel);
+        }
+    }
+    static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(uint16_t(r & 0xFFFFu)); }
+    static __device__ __forceinline__ float dmin(const DRec &) { return 0.f; }
+    static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
+};
+
+struct WNvfp4 {   // row-major: 16 code bytes per sub-block, one E4M3 scale byte per 16 weights, one fp32 global per row
+    static constexpr int kPlanes = 1, kTabBytes = 256 * 16, kLattice = 1;
+    static constexpr bool kFp8 = true, kMin = false, kRowMul = true;
+    struct Code { uint2 c; };
+    typedef uint4 Rec;       // the 16 scale bytes of the row's super-block
+    typedef uint32_t DRec;   // unused: nothing is folded
+    struct Src { const uint8_t * codes, * aux; };
+    // per scale byte the 16 products e2m1(code) * e4m3(scale) / 8, rounded to E4M3 (nearest even); the division keeps the
+    // largest product (6 * 448) inside the format, and rowmul() gives the 8 back
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t *, int tid, int threads) {
+        uint32_t * t32 = reinterpret_cast<uint32_t *>(tab);
+        for (int i = tid; i < 256 * 4; i += threads) {
+            const float sc = e4m3_to_float(uint32_t(i >> 2));
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = 4 * (i & 3) + j;
+                const uint32_t tb = ((c < 4 ? kFp4T0 : c < 8 ? kFp4T1 : c < 12 ? kFp4T2 : kFp4T3) >> (8 * (c & 3))) & 0xFFu;   // twice the e2m1 value
+                v[j] = float(int8_t(tb)) * 0.0625f * sc;
+            }
+            t32[i] = pack4_q<true>(v[0], v[1], v[2], v[3]);
+        }
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int g) {
+        const int S = b.cols / 32;
+        const int64_t row = int64_t(e) * b.rows + wtile * 32 + n;
+        return Src{b.codes + row * S * 16 + g * 8, b.aux + row * (b.cols / 16)};
+    }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) { return Code{*reinterpret_cast<const uint2 *>(s.codes + int64_t(sub) * 16)}; }
+    static __device__ __forceinline__ Rec rec(const Src & s, int sb) { return *reinterpret_cast<const uint4 *>(s.aux + int64_t(sb) * 16); }
+    static __device__ __forceinline__ DRec drec(const Src &, int) { return 0; }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec & r, int ib, int, const uint8_t * tab, const uint32_t *, v4i * p) {
+        const uint32_t pair = ((ib >> 1) == 0 ? r.x : (ib >> 1) == 1 ? r.y : (ib >> 1) == 2 ? r.z : r.w) >> (16 * (ib & 1));
+        const uint4 t0 = *reinterpret_cast<const uint4 *>(tab + (pair & 0xFFu) * 16), t1 = *reinterpret_cast<const uint4 *>(tab + ((pair >> 8) & 0xFFu) * 16);
+        const uint32_t cw[2] = {c.c.x, c.c.y};
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {   // low nibbles: the sub-block's first 16 weights (first scale), high nibbles: the other 16
+            const NibbleKeys k = nibble_keys(cw[w]);
+            p[0][2 * w] = pick16(t0, k.i_lo, k.s_lo);
+            p[0][2 * w + 1] = pick16(t1, k.i_hi, k.s_hi);
+        }
+    }
+    static __device__ __forceinline__ float d(const DRec &) { return 1.f; }
+    static __device__ __forceinline__ float dmin(const DRec &) { return 0.f; }
+    static __device__ __forceinline__ float rowmul(const BankView & b, int e, int wtile, int n) {
+        return 8.f * *reinterpret_cast<const float *>(b.aux + nvfp4_global_offset(b.rows_total, b.cols) + (int64_t(e) * b.rows + wtile * 32 + n) * 4);
+    }
+};
+
+// one sub-block's products of a row tile with the planes of a weight tile
+template <class W> struct Acc {
+    v16i plane[W::kFp8 ? 1 : W::kPlanes];   // int32 sums of the current super-block (unused by the fp8 path)
+    v16f sum;                               // fp32 result so far
+};
+template <class W> __device__ __forceinline__ void acc_clear(Acc<W> & a) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a.sum[i] = 0.f;
+}
+template <class W> __device__ __forceinline__ void acc_step(Acc<W> & a, v4i x, const v4i * w, bool first_of_sb) {
+    if constexpr (W::kFp8) {
+        const long x0 = __builtin_bit_cast(long, v2i{x[0], x[1]}), x1 = __builtin_bit_cast(long, v2i{x[2], x[3]});
+        const long w0 = __builtin_bit_cast(long, v2i{w[0][0], w[0][1]}), w1 = __builtin_bit_cast(long, v2i{w[0][2], w[0][3]});
+        a.sum = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(x0, w0, a.sum, 0, 0, 0);
+        a.sum = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(x1, w1, a.sum, 0, 0, 0);
+    } else {
+        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int p = 0; p < W::kPlanes; ++p) a.plane[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, w[p], first_of_sb ? zero : a.plane[p], 0, 0, 0);
+    }
+}
+// |64 acc_h + acc_l| <= 256 * 127 * 2^12 < 2^28: exact in int32, then one rounding into fp32
+template <class W> __device__ __forceinline__ void acc_fold(Acc<W> & a, const typename W::DRec & r) {
+    if constexpr (!W::kFp8) {
+        const float d = W::d(r);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) a.sum[i] = fold_sb(a.sum[i], a.plane[0][i], a.plane[1][i], d);
+        if constexpr (W::kMin) {
+            const float m = -W::dmin(r);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) a.sum[i] = __fmaf_rn(float(a.plane[2][i]), m, a.sum[i]);
+        }
+    }
+}
+
+// dynamic LDS: [2 stages][NB][planes][8 sub-blocks][64 lanes] v4i of decoded weights.
 // 4 * NB waves. Decoding: wave = 4 * slot + quarter decodes sub-blocks 2 quarter, 2 quarter + 1 of operand slot `slot`.
 // Products: a wave takes 2 / NB row tiles (tile `wave`, and tile wave + 4 when there is one slot) against every slot.
-template <int NB>
-__global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
-    constexpr int THREADS = 256 * NB;
+template <int NB, class W>
+__global__ __launch_bounds__(256 * NB) void plane_gemm_k(GemmArgs k) {
+    constexpr int THREADS = 256 * NB, P = W::kPlanes;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     v4i * bs = reinterpret_cast<v4i *>(lds);
-    __shared__ __attribute__((aligned(16))) uint8_t s_tab[64 * 32];   // per 6-bit scale: 16 h bytes, 16 l bytes
+    __shared__ __attribute__((aligned(16))) uint8_t s_tab[W::kTabBytes];
+    __shared__ uint32_t s_lat[W::kLattice];
     __shared__ int s_asg[kChunkTiles * 32];
     __shared__ float s_scale[kChunkTiles * 32];
     // the experts' index (chunk and tile prefix sums, counts, offsets), copied once: every item looks its expert up, and a
@@ -321,13 +539,7 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
             s_cnt[i] = i < k.experts ? k.counts[i] : 0;
             s_off[i] = k.offsets[i];
         }
-
-    for (int i = tid; i < 64 * 16; i += THREADS) {
-        const int v = int(kIq4Values[i & 15]) * ((i >> 4) - 32);
-        const int lo = ((v + 32) & 63) - 32, hi = (v - lo) >> 6;
-        s_tab[(i >> 4) * 32 + (i & 15)] = uint8_t(hi);
-        s_tab[(i >> 4) * 32 + 16 + (i & 15)] = uint8_t(lo);
-    }
+    W::tables(s_tab, s_lat, tid, THREADS);
     // Work items are (chunk of row tiles, unit of weight rows). Items that share operand A (one chunk, all units) have
     // indices that agree modulo 8, and the blocks that the round-robin of blocks over the 8 XCDs puts on one XCD take the
     // items of one residue from a counter of their own: one XCD's L2 serves a chunk's rows, and a block that finishes
@@ -338,7 +550,7 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
     const int * cnts = cached ? s_cnt : k.counts, * offs = cached ? s_off : k.offsets;
     const int n_chunks = cbase[k.experts];
     const int items_padded = (n_chunks + 7) / 8 * 8 * k.units;
-    const int S = k.b0.cols / 32, NSB = S / 8, rows = k.b0.rows, tiles_w = rows / 32;
+    const int NSB = k.b0.cols / 256, rows = k.b0.rows;
     __shared__ int s_ticket;
     int * ctr = k.plan.counters;
     const int xcd = int(blockIdx.x) & 7;
@@ -379,37 +591,30 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
             const BankView & wbank = nbw ? k.b1 : k.b0;
             const bool wdead = k.gateup && is_shared && wt * 32 >= k.shared_lim;
             const int sbe = wdead ? 0 : !k.gateup && is_shared ? k.shared_lim / 256 : NSB;
-            const int64_t wtile_g = int64_t(e) * tiles_w + wt;
-            const uint8_t * wcodes = wbank.codes + wtile_g * S * 512 + n * 16 + g * 8;
-            const uint8_t * waux = wbank.aux + wtile_g * NSB * 256 + n * 8;
+            const typename W::Src wsrc = W::src(wbank, e, wt, n, g);
             const int8_t * a_ptr = k.xq + int64_t(tile_base + first_tile) * 32 * k.b0.cols + lane * 16;
-            struct Stage { uint2 code[8]; uint2 rec; v4i a[8]; };
+            struct Stage { typename W::Code code[8]; typename W::Rec rec; typename W::DRec drec; v4i a[8]; };
             auto fetch1 = [&](int sb, Stage & st) {   // a super-block of the wave's weights and of the row tile
-                st.rec = *reinterpret_cast<const uint2 *>(waux + int64_t(sb) * 256);
+                st.rec = W::rec(wsrc, sb);
+                if constexpr (!W::kFp8) st.drec = W::drec(wsrc, sb);
 #pragma unroll
                 for (int ib = 0; ib < 8; ++ib) {
-                    st.code[ib] = *reinterpret_cast<const uint2 *>(wcodes + (int64_t(sb) * 8 + ib) * 512);
+                    st.code[ib] = W::code(wsrc, sb * 8 + ib);
                     st.a[ib] = *reinterpret_cast<const v4i *>(a_ptr + (int64_t(sb) * 8 + ib) * 1024);
                 }
             };
-            float acc_f[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc_f[i] = 0.f;
+            Acc<W> acc;
+            acc_clear(acc);
             auto work1 = [&](int sb, Stage & cur, Stage & nxt) {
                 fetch1(min(sb + 1, sbe - 1), nxt);   // past the last one the same again, from the cache: no branch, the same loads in flight on every path
                 __builtin_amdgcn_sched_barrier(0);
-                const float d = half_bits_to_float(iq4xs_d_bits(cur.rec));
-                v16i acc_h = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, acc_l = acc_h;
 #pragma unroll
                 for (int ib = 0; ib < 8; ++ib) {
-                    const uint4 * tab = reinterpret_cast<const uint4 *>(s_tab + iq4xs_ls(cur.rec, ib) * 32);
-                    v4i h, l;
-                    decode_planes(cur.code[ib], tab[0], tab[1], h, l);
-                    acc_h = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.a[ib], h, acc_h, 0, 0, 0);
-                    acc_l = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.a[ib], l, acc_l, 0, 0, 0);
+                    v4i w[P];
+                    W::planes(cur.code[ib], cur.rec, ib, g, s_tab, s_lat, w);
+                    acc_step(acc, cur.a[ib], w, ib == 0);
                 }
-#pragma unroll
-                for (int i = 0; i < 16; ++i) acc_f[i] = fold_sb(acc_f[i], acc_h[i], acc_l[i], d);
+                acc_fold(acc, cur.drec);
             };
             if (sbe > 0) {
                 Stage s0, s1;
@@ -419,11 +624,16 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
                     if (sb + 1 < sbe) work1(sb + 1, s1, s0);
                 }
             }
+            if constexpr (W::kRowMul) {
+                const float rm = W::rowmul(wbank, e, wt, n);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc.sum[i] = __fmul_rn(acc.sum[i], rm);
+            }
             float * ex = reinterpret_cast<float *>(lds);
             if (k.gateup && NB == 2) {   // the up waves hand their sums to the gate waves of the same weight tile
                 if (nbw == 1) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) ex[(mg * 16 + i) * 64 + lane] = acc_f[i];
+                    for (int i = 0; i < 16; ++i) ex[(mg * 16 + i) * 64 + lane] = acc.sum[i];
                 }
                 __syncthreads();
             }
@@ -440,8 +650,8 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
                 for (int i = 0; i < 16; ++i) {
                     if (asg[i] < 0) continue;
                     uint16_t * o = k.out + int64_t(asg[i]) * rows;
-                    if (k.gateup) o[wt * 32 + n] = swiglu_half(acc_f[i], NB == 2 ? ex[(mg * 16 + i) * 64 + lane] : acc_f[i], scl[i]);
-                    else o[wt * 32 + n] = scaled_half(acc_f[i], scl[i]);
+                    if (k.gateup) o[wt * 32 + n] = swiglu_half(acc.sum[i], NB == 2 ? ex[(mg * 16 + i) * 64 + lane] : acc.sum[i], scl[i]);
+                    else o[wt * 32 + n] = scaled_half(acc.sum[i], scl[i]);
                 }
             }
             continue;
@@ -456,50 +666,45 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
 
         // the weights this wave decodes for everybody: sub-blocks 2 mg and 2 mg + 1 of operand slot nbw
         // (gate / up: the unit's 32 rows of bank nbw; down: row tile NB * unit + nbw)
-        const BankView & bank = nbw ? k.b1 : k.b0;
-        const int64_t tile_g = int64_t(e) * tiles_w + (k.gateup ? unit : NB * unit + nbw);
-        const uint8_t * codes = bank.codes + tile_g * S * 512 + n * 16 + g * 8;   // sub-block s of the tile: + 512 s; lane = (row n, code half g)
-        const uint8_t * aux = bank.aux + tile_g * NSB * 256 + n * 8;              // super-block sb of the tile: + 256 sb
-        // the scales d of the rows of both slots, for the fold: lane's weight row n, slot b
-        const uint8_t * aux_b[NB];
+        const typename W::Src wsrc = W::src(nbw ? k.b1 : k.b0, e, k.gateup ? unit : NB * unit + nbw, n, g);
+        // lane's weight row n of both slots, for the fold: its super-blocks' scales
+        typename W::Src src_b[NB];
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
-            aux_b[b] = (b ? k.b1 : k.b0).aux + (int64_t(e) * tiles_w + (k.gateup ? unit : NB * unit + b)) * NSB * 256 + n * 8;
+        for (int b = 0; b < NB; ++b) src_b[b] = W::src(b ? k.b1 : k.b0, e, k.gateup ? unit : NB * unit + b, n, g);
 
         // The super-block loop is instantiated per number of live row tiles of the wave (0..TPW), so that its body is one
         // straight line of code the scheduler can interleave. Every instance passes the same barriers.
         auto body = [&](auto mt_tag) {
             constexpr int MT = decltype(mt_tag)::value;
             constexpr int MTA = MT ? MT : 1;
-            v16i acc_h[MTA][NB], acc_l[MTA][NB];
-            float acc_f[MTA][NB][16];
+            Acc<W> acc[MTA][NB];
 #pragma unroll
             for (int t = 0; t < MTA; ++t)
 #pragma unroll
-                for (int b = 0; b < NB; ++b)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) { acc_f[t][b][i] = 0.f; acc_h[t][b][i] = 0; acc_l[t][b][i] = 0; }
+                for (int b = 0; b < NB; ++b) acc_clear(acc[t][b]);
 
             // the codes and the scale record are fetched one super-block before they are decoded, so that their latency is
             // not waited for
-            uint2 f_rec = {0, 0}, f_code[2] = {{0, 0}, {0, 0}};
-            uint2 d_rec[NB], d_rec_next[NB];
+            typename W::Rec f_rec = {};
+            typename W::Code f_code[2] = {};
+            typename W::DRec d_rec[NB] = {}, d_rec_next[NB] = {};
             auto fetch = [&](int sb) {
-                f_rec = *reinterpret_cast<const uint2 *>(aux + int64_t(sb) * 256);
+                f_rec = W::rec(wsrc, sb);
 #pragma unroll
-                for (int j = 0; j < 2; ++j) f_code[j] = *reinterpret_cast<const uint2 *>(codes + (int64_t(sb) * 8 + 2 * mg + j) * 512);
+                for (int j = 0; j < 2; ++j) f_code[j] = W::code(wsrc, sb * 8 + 2 * mg + j);
             };
             auto fetch_d = [&](int sb) {
+                if constexpr (!W::kFp8) {
 #pragma unroll
-                for (int b = 0; b < NB; ++b) d_rec_next[b] = *reinterpret_cast<const uint2 *>(aux_b[b] + int64_t(sb) * 256);
+                    for (int b = 0; b < NB; ++b) d_rec_next[b] = W::drec(src_b[b], sb);
+                }
             };
             auto decode_one = [&](int buf, int j) {
                 const int ib = 2 * mg + j;
-                const uint4 * tab = reinterpret_cast<const uint4 *>(s_tab + iq4xs_ls(f_rec, ib) * 32);
-                v4i h, l;
-                decode_planes(f_code[j], tab[0], tab[1], h, l);
-                bs[(((buf * NB + nbw) * 2 + 0) * 8 + ib) * 64 + lane] = h;
-                bs[(((buf * NB + nbw) * 2 + 1) * 8 + ib) * 64 + lane] = l;
+                v4i w[P];
+                W::planes(f_code[j], f_rec, ib, g, s_tab, s_lat, w);
+#pragma unroll
+                for (int p = 0; p < P; ++p) bs[(((buf * NB + nbw) * P + p) * 8 + ib) * 64 + lane] = w[p];
             };
             auto decode_into = [&](int buf) { decode_one(buf, 0); decode_one(buf, 1); };
             // operand A, two k-steps (sub-blocks) per slot, fetched kSlots - 1 slots before its products
@@ -541,27 +746,29 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
                         const int ib = 2 * jp + h;
 #pragma unroll
                         for (int b = 0; b < NB; ++b) {
-                            const v4i bh = bs[(((buf * NB + b) * 2 + 0) * 8 + ib) * 64 + lane];
-                            const v4i bl = bs[(((buf * NB + b) * 2 + 1) * 8 + ib) * 64 + lane];
+                            v4i w[P];
 #pragma unroll
-                            for (int t = 0; t < MT; ++t) {
-                                const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                                acc_h[t][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp % kSlots][t][h], bh, ib ? acc_h[t][b] : zero, 0, 0, 0);
-                                acc_l[t][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[jp % kSlots][t][h], bl, ib ? acc_l[t][b] : zero, 0, 0, 0);
-                            }
+                            for (int p = 0; p < P; ++p) w[p] = bs[(((buf * NB + b) * P + p) * 8 + ib) * 64 + lane];
+#pragma unroll
+                            for (int t = 0; t < MT; ++t) acc_step(acc[t][b], a_reg[jp % kSlots][t][h], w, ib == 0);
                         }
                     }
                 }
-                // |64 acc_h + acc_l| <= 256 * 127 * 127 * 32 < 2^28: exact in int32, then one rounding into fp32
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) acc_fold(acc[t][b], d_rec[b]);
+                __syncthreads();
+            }
+            if constexpr (W::kRowMul) {
 #pragma unroll
                 for (int b = 0; b < NB; ++b) {
-                    const float d = half_bits_to_float(iq4xs_d_bits(d_rec[b]));
+                    const float rm = W::rowmul(b ? k.b1 : k.b0, e, k.gateup ? unit : NB * unit + b, n);
 #pragma unroll
                     for (int t = 0; t < MT; ++t)
 #pragma unroll
-                        for (int i = 0; i < 16; ++i) acc_f[t][b][i] = fold_sb(acc_f[t][b][i], acc_h[t][b][i], acc_l[t][b][i], d);
+                        for (int i = 0; i < 16; ++i) acc[t][b].sum[i] = __fmul_rn(acc[t][b].sum[i], rm);
                 }
-                __syncthreads();
             }
             // result register i of lane half g is tile row 8 (i / 4) + 4 g + i % 4, weight row n. The rows' assignments and
             // scales are read first, all at once: a read per element inside the store loop would serialise on LDS latency.
@@ -580,10 +787,10 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
                     if (asg[i] < 0) continue;
                     uint16_t * o = k.out + int64_t(asg[i]) * rows;
                     if (k.gateup) {
-                        o[unit * 32 + n] = swiglu_half(acc_f[t][0][i], acc_f[t][NB - 1][i], scl[i]);
+                        o[unit * 32 + n] = swiglu_half(acc[t][0].sum[i], acc[t][NB - 1].sum[i], scl[i]);
                     } else {
 #pragma unroll
-                        for (int b = 0; b < NB; ++b) o[(NB * unit + b) * 32 + n] = scaled_half(acc_f[t][b][i], scl[i]);
+                        for (int b = 0; b < NB; ++b) o[(NB * unit + b) * 32 + n] = scaled_half(acc[t][b].sum[i], scl[i]);
                     }
                 }
             }
@@ -611,44 +818,49 @@ __global__ __launch_bounds__(256 * NB) void iq4xs_gemm_k(GemmArgs k) {
 // ---------------------------------------------------------------------------------------------- entry helpers
 int64_t grouped_row_tiles(int64_t assignments, int experts) { return (assignments + 31) / 32 + experts; }
 
-int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, hipStream_t s) {
+// f8: E4M3 bytes with scale amax / 448 in place of int8 bytes with scale amax / 127
+int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, hipStream_t s, bool f8) {
     const unsigned blocks = unsigned((rows + 3) / 4);
+#define TQMOE_QUANT(XT) (f8 ? quant_rows_k<XT, true><<<blocks, 256, 0, s>>>(x, rows, cols, q, scale) : quant_rows_k<XT, false><<<blocks, 256, 0, s>>>(x, rows, cols, q, scale))
     switch (xtype) {
-        case TQMOE_F32: quant_rows_i8_k<TQMOE_F32><<<blocks, 256, 0, s>>>(x, rows, cols, q, scale); break;
-        case TQMOE_F16: quant_rows_i8_k<TQMOE_F16><<<blocks, 256, 0, s>>>(x, rows, cols, q, scale); break;
-        default: quant_rows_i8_k<TQMOE_BF16><<<blocks, 256, 0, s>>>(x, rows, cols, q, scale); break;
+        case TQMOE_F32: TQMOE_QUANT(TQMOE_F32); break;
+        case TQMOE_F16: TQMOE_QUANT(TQMOE_F16); break;
+        default: TQMOE_QUANT(TQMOE_BF16); break;
     }
+#undef TQMOE_QUANT
     return 0;
 }
 
 int64_t grouped_scale_words(int64_t assignments, int experts) { return grouped_row_tiles(assignments, experts) * 32 + 2 * (int64_t(experts) + 1) + kPlanCounters; }
 
-int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
-                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s) {
-    const int64_t tiles = grouped_row_tiles(assignments, experts);
-    const Plan plan = plan_at(scale, tiles * 32, experts);
-    plan_k<<<1, 64, 0, s>>>(counts, experts, const_cast<int *>(plan.tile_base), const_cast<int *>(plan.chunk_base), plan.counters);
+template <int XT, bool F8>
+static void group_rows_launch(const void * x, int cols, const int * counts, const int * offsets, const int * perm, int experts, int64_t tiles, int xdiv, int8_t * q,
+                              float * scale, const Plan & plan, hipStream_t s) {
     if (cols == 512 || cols == 1024 || cols == 2048) {
         const size_t lds = size_t(32) * size_t(cols + 16);
         auto launch = [&](auto kernel) {
             if (lds > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kernel), 32 * (2048 + 16));
             kernel<<<unsigned(tiles), 256, lds, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan);
         };
-#define TQMOE_GROUP_TILE(XT) (cols == 512 ? launch(group_rows_i8_tile_k<XT, 1>) : cols == 1024 ? launch(group_rows_i8_tile_k<XT, 2>) : launch(group_rows_i8_tile_k<XT, 4>))
-        switch (xtype) {
-            case TQMOE_F32: TQMOE_GROUP_TILE(TQMOE_F32); break;
-            case TQMOE_F16: TQMOE_GROUP_TILE(TQMOE_F16); break;
-            default: TQMOE_GROUP_TILE(TQMOE_BF16); break;
-        }
-#undef TQMOE_GROUP_TILE
-        return 0;
+        if (cols == 512) launch(group_rows_tile_k<XT, 1, F8>); else if (cols == 1024) launch(group_rows_tile_k<XT, 2, F8>); else launch(group_rows_tile_k<XT, 4, F8>);
+        return;
     }
-    const unsigned blocks = unsigned(tiles * 4);
+    group_rows_k<XT, F8><<<unsigned(tiles * 4), 256, 0, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan);
+}
+
+int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
+                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8) {
+    const int64_t tiles = grouped_row_tiles(assignments, experts);
+    const Plan plan = plan_at(scale, tiles * 32, experts);
+    plan_k<<<1, 64, 0, s>>>(counts, experts, const_cast<int *>(plan.tile_base), const_cast<int *>(plan.chunk_base), plan.counters);
+#define TQMOE_GROUP(XT) (f8 ? group_rows_launch<XT, true>(x, cols, counts, offsets, perm, experts, tiles, xdiv, q, scale, plan, s) \
+                            : group_rows_launch<XT, false>(x, cols, counts, offsets, perm, experts, tiles, xdiv, q, scale, plan, s))
     switch (xtype) {
-        case TQMOE_F32: group_rows_i8_k<TQMOE_F32><<<blocks, 256, 0, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan); break;
-        case TQMOE_F16: group_rows_i8_k<TQMOE_F16><<<blocks, 256, 0, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan); break;
-        default: group_rows_i8_k<TQMOE_BF16><<<blocks, 256, 0, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan); break;
+        case TQMOE_F32: TQMOE_GROUP(TQMOE_F32); break;
+        case TQMOE_F16: TQMOE_GROUP(TQMOE_F16); break;
+        default: TQMOE_GROUP(TQMOE_BF16); break;
     }
+#undef TQMOE_GROUP
     return 0;
 }
 
@@ -661,8 +873,22 @@ int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, co
     return 0;
 }
 
+// bank formats with a plane GEMM: int8 operands (IQ4_XS, IQ3_S, Q4_K) or E4M3 operands (NVFP4G)
+bool plane_gemm_has(uint32_t type) { return type == TQMOE_IQ4_XS || type == TQMOE_IQ3_S || type == TQMOE_Q4_K || type == TQMOE_NVFP4G; }
+bool plane_gemm_is_fp8(uint32_t type) { return type == TQMOE_NVFP4G; }
+
+template <class W> static void plane_gemm_launch(int nb, const GemmArgs & k, unsigned blocks, hipStream_t s) {
+    const size_t lds = size_t(2) * nb * W::kPlanes * 8 * 64 * sizeof(v4i);
+    if (nb == 2) {
+        if (lds > 65536 - 24576) allow_dynamic_lds(reinterpret_cast<const void *>(&plane_gemm_k<2, W>), 2 * 2 * 3 * 8 * 64 * sizeof(v4i));
+        plane_gemm_k<2, W><<<blocks, 512, lds, s>>>(k);
+    } else {
+        plane_gemm_k<1, W><<<blocks, 256, lds, s>>>(k);
+    }
+}
+
 // assignments = total entries of perm (it fixes where the index behind the scales lies)
-int32_t enqueue_iq4xs_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
+int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
                            const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s) {
     const int nb = gateup || b0.rows % 64 == 0 ? 2 : 1;
     const int units = gateup ? b0.rows / 32 : b0.rows / (32 * nb);
@@ -673,12 +899,12 @@ int32_t enqueue_iq4xs_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const i
     const int cus = cu_count();
     const int64_t most = (tiles / kChunkTiles + experts + 7) / 8 * 8 * units;     // an upper bound of the items
     const unsigned blocks = unsigned(std::min<int64_t>((cus + 7) / 8 * 8, most));
-    const size_t lds = size_t(2) * nb * 2 * 8 * 64 * sizeof(v4i);
-    if (nb == 2) {
-        allow_dynamic_lds(reinterpret_cast<const void *>(&iq4xs_gemm_k<2>), 65536);
-        iq4xs_gemm_k<2><<<blocks, 512, lds, s>>>(k);
-    } else {
-        iq4xs_gemm_k<1><<<blocks, 256, lds, s>>>(k);
+    switch (b0.type) {
+        case TQMOE_IQ4_XS: plane_gemm_launch<WIq4xs>(nb, k, blocks, s); break;
+        case TQMOE_IQ3_S: plane_gemm_launch<WIq3s>(nb, k, blocks, s); break;
+        case TQMOE_Q4_K: plane_gemm_launch<WQ4k>(nb, k, blocks, s); break;
+        case TQMOE_NVFP4G: plane_gemm_launch<WNvfp4>(nb, k, blocks, s); break;
+        default: return -1;
     }
     return 0;
 }

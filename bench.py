@@ -43,7 +43,7 @@ CONFIGS = {
               hidden=2048, ff=512, experts=512, topk=10, shared_ff=512, wtype=IQ4_XS, fmt="IQ4_XS", rtype="bf16", xtype="bf16",
               points=(1, 16, 4096), zipf_from=64),
     "1": dict(label="config 1: hidden 2048, 64 Q4_K experts top-8 (ff 768), fp32 router and activations",
-              hidden=2048, ff=768, experts=64, topk=8, shared_ff=0, wtype=Q4_K, fmt="Q4_K", rtype="f32", xtype="f32", points=(1, 16), zipf_from=None),
+              hidden=2048, ff=768, experts=64, topk=8, shared_ff=0, wtype=Q4_K, fmt="Q4_K", rtype="f32", xtype="f32", points=(1, 16, 4096), zipf_from=None),
     "4": dict(label="config 4: hidden 2048, 256 IQ3_S experts top-8 (ff 768), bf16 router and activations",
               hidden=2048, ff=768, experts=256, topk=8, shared_ff=0, wtype=IQ3_S, fmt="IQ3_S", rtype="bf16", xtype="bf16", points=(1, 64, 512),
               zipf_from=None),
@@ -192,6 +192,7 @@ def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
 
     # ---- dominant kernels alone: back-to-back launches over the rotating banks, inputs prepared once
     prep = []
+    fp8 = path == "grouped_fp8"
     for l, x, ids in zip(layers, xs, routing):
         ext = tq.moe_extend_ids(ids, cfg["experts"]) if shared else ids
         if path == "decode":
@@ -202,10 +203,10 @@ def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
         else:
             counts, offsets, perm, _ = tq.moe_dispatch(ext, cfg["experts"] + shared)
             lists = (counts, offsets, perm)
-            if path == "grouped_i8":
-                xq, xsc = tq.group_rows_i8(x, lists, T * slots, slots)
-                act = tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, k, cfg["shared_ff"])
-                aq, asc = tq.group_rows_i8(act, lists, T * slots, 1)
+            if path in ("grouped_i8", "grouped_fp8"):
+                xq, xsc = tq.group_rows_i8(x, lists, T * slots, slots, fp8=fp8)
+                act = tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, k, cfg["shared_ff"], fp8=fp8)
+                aq, asc = tq.group_rows_i8(act, lists, T * slots, 1, fp8=fp8)
                 prep.append((l, lists, xq, xsc, aq, asc))
             else:
                 act = tq.expert_gemm_gateup(l.gate, l.up, x, lists, T, slots, k, cfg["shared_ff"])
@@ -216,9 +217,9 @@ def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
             if path == "decode":
                 l, ext, img, act, y = item
                 tq.expert_gateup(l.gate, l.up, img, ext, k, shared_ff=cfg["shared_ff"], act_image=act)
-            elif path == "grouped_i8":
+            elif path in ("grouped_i8", "grouped_fp8"):
                 l, lists, xq, xsc, aq, asc = item
-                tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, k, cfg["shared_ff"])
+                tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, k, cfg["shared_ff"], fp8=fp8)
             else:
                 l, lists, x, act = item
                 tq.expert_gemm_gateup(l.gate, l.up, x, lists, T, slots, k, cfg["shared_ff"])
@@ -228,9 +229,9 @@ def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
             if path == "decode":
                 l, ext, img, act, y = item
                 tq.expert_down(l.down, act, ext, k, shared_ff=cfg["shared_ff"], y=y)
-            elif path == "grouped_i8":
+            elif path in ("grouped_i8", "grouped_fp8"):
                 l, lists, xq, xsc, aq, asc = item
-                tq.expert_gemm_i8(l.down, aq, asc, lists, T, slots, k, cfg["shared_ff"])
+                tq.expert_gemm_i8(l.down, aq, asc, lists, T, slots, k, cfg["shared_ff"], fp8=fp8)
             else:
                 l, lists, x, act = item
                 tq.expert_gemm(l.down, act, lists, T, slots, k, cfg["shared_ff"], per_expert_input=True, out_type=tq.F32)
@@ -262,9 +263,9 @@ def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
         dtype = "int8 x int8 -> int32 (weights exact, activations as two int8 planes), fp32 scales"
     else:
         op = {"grouped_i8": "int8", "grouped_f16": "fp16", "grouped_fp8": "fp8"}[path]
-        kname = {"grouped_i8": "iq4xs_gemm_k<2> (grouped gate + up int8 MFMA product + SwiGLU)",
+        kname = {"grouped_i8": "plane_gemm_k<2, %s> (grouped gate + up int8 MFMA product + SwiGLU)" % cfg["fmt"],
                  "grouped_f16": "expert_gemm_f16_k<%s,2> (grouped gate + up fp16 MFMA product + SwiGLU)" % cfg["fmt"],
-                 "grouped_fp8": "expert_gemm_fp8_k<2> (grouped gate + up fp8 MFMA product + SwiGLU)"}[path]
+                 "grouped_fp8": "plane_gemm_k<2, %s> (grouped gate + up fp8 MFMA product + SwiGLU)" % cfg["fmt"]}[path]
         roofline = {"bound": "mfma", "kernel": kname, "achieved": round(gu_ops / gu_s / 1e12, 2), "peak": PEAK[op] / 1e12, "unit": "TFLOP/s",
                     "frac": round(gu_ops / gu_s / PEAK[op], 4), "traffic": None,
                     "ops": "multiply-add = 2 operations; peak = dense %s %.1f POP/s" % (op, PEAK[op] / 1e15),

@@ -37,12 +37,14 @@ bool int8_ok(const tqmoe_layer & L) {
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
     const int slots = L.topk + (L.has_shared ? 1 : 0), banks = L.n_expert + (L.has_shared ? 1 : 0);
-    // the int8 grouped products from kGroupedMin tokens; the fp16 ones (other formats) from kGroupedPerBank assignments per
-    // bank matrix on average (measured: the decode kernels' time grows with the assignments, the grouped products' with
-    // the experts they decode, and the two cross at about three assignments per expert), and in any case once the decode
-    // kernels no longer read every expert's weights once (they group an expert's rows up to kDecodeDedup assignments a launch)
-    p.int8 = n >= kGroupedMin && int8_ok(L);
-    p.grouped = p.int8 || int64_t(n) * slots > std::min<int64_t>(kDecodeDedup, int64_t(kGroupedPerBank) * banks);
+    // IQ4_XS banks (tile-major): the int8 grouped products from kGroupedMin tokens. Every other format, on the 8-bit or the
+    // fp16 grouped products: from kGroupedPerBank assignments per bank matrix on average (measured: the decode kernels' time
+    // grows with the assignments, the grouped products' with the experts they decode, and the two cross at about three
+    // assignments per expert), and in any case once the decode kernels no longer read every expert's weights once (they
+    // group an expert's rows up to kDecodeDedup assignments a launch)
+    const bool many = int64_t(n) * slots > std::min<int64_t>(kDecodeDedup, int64_t(kGroupedPerBank) * banks);
+    p.int8 = int8_ok(L) && (L.gate.type == TQMOE_IQ4_XS && L.down.type == TQMOE_IQ4_XS ? n >= kGroupedMin : many);
+    p.grouped = p.int8 || many;
     // the grouped products take 2^24 assignments a pass (32-bit block and byte counts stay far from their limits), the
     // decode kernels 65535
     const int64_t per_pass = p.int8 ? int64_t(1) << 24 : p.grouped ? int64_t(65535 - banks) * 64 : kDecodeAssignments;

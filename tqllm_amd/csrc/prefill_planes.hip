@@ -266,6 +266,7 @@ struct GemmArgs {
     uint16_t * out;           // fp16 [assignments][rows]: silu(gate) * up, or the plain product
     int gateup;
     int units;                // weight-row units per expert: rows / 32 (gate / up, and down with NB = 1), rows / 64 (down, NB = 2)
+    int unit_group;           // consecutive units an item runs through (a divisor of units): short rows get more per item
     int shared_expert;        // index of the expert whose rows (gate / up) or columns (down) stop at shared_lim, or -1
     int shared_lim;
 };
@@ -432,7 +433,7 @@ struct WIq3s {   // row-major: 12 code bytes per sub-block (8 lattice indices, 3
 
 struct WNvfp4 {   // row-major: 16 code bytes per sub-block, one E4M3 scale byte per 16 weights, one fp32 global per row
     static constexpr int kPlanes = 1, kTabBytes = 256 * 16, kLattice = 1;
-    static constexpr bool kFp8 = true, kMin = false, kRowMul = true;
+    static constexpr bool kFp8 = true, kRowMul = true;
     struct Code { uint2 c; };
     typedef uint4 Rec;       // the 16 scale bytes of the row's super-block
     typedef uint32_t DRec;   // unused: nothing is folded
@@ -515,11 +516,16 @@ template <class W> __device__ __forceinline__ void acc_fold(Acc<W> & a, const ty
 }
 
 // dynamic LDS: [2 stages][NB][planes][8 sub-blocks][64 lanes] v4i of decoded weights.
-// 4 * NB waves. Decoding: wave = 4 * slot + quarter decodes sub-blocks 2 quarter, 2 quarter + 1 of operand slot `slot`.
-// Products: a wave takes 2 / NB row tiles (tile `wave`, and tile wave + 4 when there is one slot) against every slot.
-template <int NB, class W>
-__global__ __launch_bounds__(256 * NB) void plane_gemm_k(GemmArgs k) {
-    constexpr int THREADS = 256 * NB, P = W::kPlanes;
+// WAVES waves (8 with two operand slots, 4 with one). Decoding: the 8 * NB (slot, sub-block) pieces of a super-block are
+// dealt to the waves in order, 8 NB / WAVES each. Products: a wave takes 8 / WAVES row tiles (tile `wave`, then every
+// WAVES-th) against every slot.
+template <int NB, class W, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
+    constexpr int THREADS = 64 * WAVES, P = W::kPlanes;
+    constexpr int TPW = 8 / WAVES;           // row tiles per wave of a shared chunk
+    constexpr int PIECES = 8 * NB / WAVES;   // (slot, sub-block) pieces a wave decodes per super-block
+    constexpr int SPW = 4 * NB / WAVES;      // operand slots per wave on a lone row tile
+    static_assert(kChunkTiles == 8 && (PIECES == 2 || PIECES == 4) && (SPW == 1 || SPW == 2), "wave arrangement");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     v4i * bs = reinterpret_cast<v4i *>(lds);
     __shared__ __attribute__((aligned(16))) uint8_t s_tab[W::kTabBytes];
@@ -530,7 +536,7 @@ __global__ __launch_bounds__(256 * NB) void plane_gemm_k(GemmArgs k) {
     // binary search is a chain of dependent reads
     __shared__ int s_cbase[kPlanExperts + 1], s_tbase[kPlanExperts + 1], s_cnt[kPlanExperts + 1], s_off[kPlanExperts + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
-    const int mg = wave & 3, nbw = wave >> 2;     // row group, operand slot
+    const int mg = wave & 3, nbw = wave >> 2;     // lone row tile: weight tile of the wave within the item, operand slot (SPW == 1)
     const bool cached = k.experts <= kPlanExperts;
     if (cached)
         for (int i = tid; i <= k.experts; i += THREADS) {
@@ -549,7 +555,8 @@ __global__ __launch_bounds__(256 * NB) void plane_gemm_k(GemmArgs k) {
     const int * cbase = cached ? s_cbase : k.plan.chunk_base, * tbase = cached ? s_tbase : k.plan.tile_base;
     const int * cnts = cached ? s_cnt : k.counts, * offs = cached ? s_off : k.offsets;
     const int n_chunks = cbase[k.experts];
-    const int items_padded = (n_chunks + 7) / 8 * 8 * k.units;
+    const int groups = k.units / k.unit_group;                  // unit groups per chunk
+    const int items_padded = (n_chunks + 7) / 8 * 8 * groups;
     const int NSB = k.b0.cols / 256, rows = k.b0.rows;
     __shared__ int s_ticket;
     int * ctr = k.plan.counters;
@@ -563,58 +570,86 @@ __global__ __launch_bounds__(256 * NB) void plane_gemm_k(GemmArgs k) {
         const int item = 8 * s_ticket + xcd;
         if (item >= items_padded) break;
         if (tid == 0) ticket = atomicAdd(&ctr[xcd], 1);
-        const int unit = (item >> 3) % k.units, chunk = item / (8 * k.units) * 8 + (item & 7);
+        const int ug = (item >> 3) % groups, chunk = item / (8 * groups) * 8 + (item & 7);
         if (chunk >= n_chunks) continue;
         const int e = owner_of(cbase, k.experts, chunk);
         const int local = chunk - cbase[e], tile_base = tbase[e];
         const bool is_shared = e == k.shared_expert;
+        const int u0 = ug * k.unit_group;                                   // the item's first unit
         // gate / up rows of the shared expert beyond its size: no products, zeros stored (the rows are quantised whole later)
-        const bool dead = k.gateup && is_shared && unit * 32 >= k.shared_lim;
-        const int sb_end = dead ? 0 : !k.gateup && is_shared ? k.shared_lim / 256 : NSB;
+        const int live_units = k.gateup && is_shared ? min(max(k.shared_lim / 32 - u0, 0), k.unit_group) : k.unit_group;
+        const int sb_full = !k.gateup && is_shared ? k.shared_lim / 256 : NSB;   // super-blocks of a live unit's products
         const int cnt = cnts[e], tiles_e = (cnt + 31) >> 5;
         const int first_tile = local * kChunkTiles;                         // of this expert
         const int live_tiles = min(kChunkTiles, tiles_e - first_tile);      // of this block
         // A chunk of one row tile has nothing for the waves to share: every wave then takes the tile against 32 weight
-        // rows of its own, four units per item, and the chunk's other item numbers are empty.
+        // rows of its own (of every slot it has), four units a pass, the chunk's items taking passes in turn.
         const bool lone = live_tiles == 1 && k.units % 4 == 0;
-        if (lone && unit >= k.units / 4) continue;
-        for (int i = tid; i < kChunkTiles * 32; i += THREADS) {
-            const int idx = first_tile * 32 + i;
-            const bool ok = i < live_tiles * 32 && idx < cnt;
-            s_asg[i] = ok ? k.perm[offs[e] + idx] : -1;
-            s_scale[i] = ok ? k.xs[int64_t(tile_base + first_tile) * 32 + i] : 0.f;
+        if (lone && ug >= k.units / 4) continue;
+        // the rows' assignments and scales are only read when the results are stored: their loads are issued here and land
+        // in LDS after the products, so that nothing waits for them
+        static_assert(kChunkTiles * 32 == 256 && THREADS >= 256, "one row per thread");
+        int row_asg = -1;
+        float row_scale = 0.f;
+        if (tid < kChunkTiles * 32) {
+            const int idx = first_tile * 32 + tid;
+            if (tid < live_tiles * 32 && idx < cnt) {
+                row_asg = k.perm[offs[e] + idx];
+                row_scale = k.xs[int64_t(tile_base + first_tile) * 32 + tid];
+            }
         }
-        __syncthreads();
-        if (lone) {
-            // weight tile of this wave: gate / up: tile 4 unit + mg of bank nbw; down: tile (4 unit + mg) NB + nbw
-            const int wt = k.gateup ? 4 * unit + mg : (4 * unit + mg) * NB + nbw;
-            const BankView & wbank = nbw ? k.b1 : k.b0;
-            const bool wdead = k.gateup && is_shared && wt * 32 >= k.shared_lim;
-            const int sbe = wdead ? 0 : !k.gateup && is_shared ? k.shared_lim / 256 : NSB;
-            const typename W::Src wsrc = W::src(wbank, e, wt, n, g);
+        auto rows_to_lds = [&]() {
+            if (tid < kChunkTiles * 32) { s_asg[tid] = row_asg; s_scale[tid] = row_scale; }
+            __syncthreads();
+        };
+        if (lone) for (int unit = ug; unit < k.units / 4; unit += groups) {
+            // weight tiles of this wave: gate / up: tile 4 unit + mg of bank b; down: tile (4 unit + mg) NB + b; b = the wave's
+            // slot, or both slots
+            int wt[SPW];
+            typename W::Src wsrc[SPW];
+            int sbe = 0;
+#pragma unroll
+            for (int q = 0; q < SPW; ++q) {
+                const int b = SPW == 1 ? nbw : q;
+                wt[q] = k.gateup ? 4 * unit + mg : (4 * unit + mg) * NB + b;
+                wsrc[q] = W::src(b ? k.b1 : k.b0, e, wt[q], n, g);
+            }
+            {
+                const bool wdead = k.gateup && is_shared && wt[0] * 32 >= k.shared_lim;   // gate / up: the slots share the tile number
+                sbe = wdead ? 0 : !k.gateup && is_shared ? k.shared_lim / 256 : NSB;
+            }
             const int8_t * a_ptr = k.xq + int64_t(tile_base + first_tile) * 32 * k.b0.cols + lane * 16;
-            struct Stage { typename W::Code code[8]; typename W::Rec rec; typename W::DRec drec; v4i a[8]; };
+            struct Stage { typename W::Code code[SPW][8]; typename W::Rec rec[SPW]; typename W::DRec drec[SPW]; v4i a[8]; };
             auto fetch1 = [&](int sb, Stage & st) {   // a super-block of the wave's weights and of the row tile
-                st.rec = W::rec(wsrc, sb);
-                if constexpr (!W::kFp8) st.drec = W::drec(wsrc, sb);
+#pragma unroll
+                for (int q = 0; q < SPW; ++q) {
+                    st.rec[q] = W::rec(wsrc[q], sb);
+                    if constexpr (!W::kFp8) st.drec[q] = W::drec(wsrc[q], sb);
+                }
 #pragma unroll
                 for (int ib = 0; ib < 8; ++ib) {
-                    st.code[ib] = W::code(wsrc, sb * 8 + ib);
+#pragma unroll
+                    for (int q = 0; q < SPW; ++q) st.code[q][ib] = W::code(wsrc[q], sb * 8 + ib);
                     st.a[ib] = *reinterpret_cast<const v4i *>(a_ptr + (int64_t(sb) * 8 + ib) * 1024);
                 }
             };
-            Acc<W> acc;
-            acc_clear(acc);
+            Acc<W> acc[SPW];
+#pragma unroll
+            for (int q = 0; q < SPW; ++q) acc_clear(acc[q]);
             auto work1 = [&](int sb, Stage & cur, Stage & nxt) {
                 fetch1(min(sb + 1, sbe - 1), nxt);   // past the last one the same again, from the cache: no branch, the same loads in flight on every path
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ib = 0; ib < 8; ++ib) {
-                    v4i w[P];
-                    W::planes(cur.code[ib], cur.rec, ib, g, s_tab, s_lat, w);
-                    acc_step(acc, cur.a[ib], w, ib == 0);
+#pragma unroll
+                    for (int q = 0; q < SPW; ++q) {
+                        v4i w[P];
+                        W::planes(cur.code[q][ib], cur.rec[q], ib, g, s_tab, s_lat, w);
+                        acc_step(acc[q], cur.a[ib], w, ib == 0);
+                    }
                 }
-                acc_fold(acc, cur.drec);
+#pragma unroll
+                for (int q = 0; q < SPW; ++q) acc_fold(acc[q], cur.drec[q]);
             };
             if (sbe > 0) {
                 Stage s0, s1;
@@ -625,19 +660,24 @@ __global__ __launch_bounds__(256 * NB) void plane_gemm_k(GemmArgs k) {
                 }
             }
             if constexpr (W::kRowMul) {
-                const float rm = W::rowmul(wbank, e, wt, n);
 #pragma unroll
-                for (int i = 0; i < 16; ++i) acc.sum[i] = __fmul_rn(acc.sum[i], rm);
+                for (int q = 0; q < SPW; ++q) {
+                    const float rm = W::rowmul((SPW == 1 ? nbw : q) ? k.b1 : k.b0, e, wt[q], n);
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[q].sum[i] = __fmul_rn(acc[q].sum[i], rm);
+                }
             }
+            rows_to_lds();
             float * ex = reinterpret_cast<float *>(lds);
-            if (k.gateup && NB == 2) {   // the up waves hand their sums to the gate waves of the same weight tile
+            constexpr bool kExchange = SPW == 1 && NB == 2;   // gate and up of a weight tile sit in two waves
+            if (k.gateup && kExchange) {   // the up waves hand their sums to the gate waves of the same weight tile
                 if (nbw == 1) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) ex[(mg * 16 + i) * 64 + lane] = acc.sum[i];
+                    for (int i = 0; i < 16; ++i) ex[(mg * 16 + i) * 64 + lane] = acc[0].sum[i];
                 }
                 __syncthreads();
             }
-            if (!(k.gateup && NB == 2 && nbw == 1)) {
+            if (!(k.gateup && kExchange && nbw == 1)) {
                 int asg[16];
                 float scl[16];
 #pragma unroll
@@ -650,30 +690,35 @@ __global__ __launch_bounds__(256 * NB) void plane_gemm_k(GemmArgs k) {
                 for (int i = 0; i < 16; ++i) {
                     if (asg[i] < 0) continue;
                     uint16_t * o = k.out + int64_t(asg[i]) * rows;
-                    if (k.gateup) o[wt * 32 + n] = swiglu_half(acc.sum[i], NB == 2 ? ex[(mg * 16 + i) * 64 + lane] : acc.sum[i], scl[i]);
-                    else o[wt * 32 + n] = scaled_half(acc.sum[i], scl[i]);
+                    if (k.gateup) {
+                        const float up = kExchange ? ex[(mg * 16 + i) * 64 + lane] : acc[SPW - 1].sum[i];
+                        o[wt[0] * 32 + n] = swiglu_half(acc[0].sum[i], up, scl[i]);
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < SPW; ++q) o[wt[q] * 32 + n] = scaled_half(acc[q].sum[i], scl[i]);
+                    }
                 }
             }
-            continue;
         }
-        // Each wave takes 2 / NB row tiles of the chunk (tile `wave`; with one operand slot also tile wave + 4) against
-        // the weights of every operand slot: a loaded piece of operand A serves the products with gate and with up (or
-        // with both weight tiles of a down unit), and SwiGLU pairs values the same lane holds.
-        constexpr int TPW = 2 / NB;
-        const int my_tiles = NB == 2 ? (wave < live_tiles ? 1 : 0) : (wave < live_tiles ? 1 : 0) + (wave + 4 < live_tiles ? 1 : 0);
-        const int8_t * a_base = k.xq + int64_t(tile_base + first_tile + wave) * 32 * k.b0.cols + lane * 16;
-        const int64_t a_tile = int64_t(4) * 32 * k.b0.cols;
-
-        // the weights this wave decodes for everybody: sub-blocks 2 mg and 2 mg + 1 of operand slot nbw
-        // (gate / up: the unit's 32 rows of bank nbw; down: row tile NB * unit + nbw)
-        const typename W::Src wsrc = W::src(nbw ? k.b1 : k.b0, e, k.gateup ? unit : NB * unit + nbw, n, g);
-        // lane's weight row n of both slots, for the fold: its super-blocks' scales
-        typename W::Src src_b[NB];
+        if (lone) continue;
+        // Each wave takes TPW row tiles of the chunk (tile `wave`, then every WAVES-th) against the weights of every operand
+        // slot: a loaded piece of operand A serves the products with gate and with up (or with both weight tiles of a down
+        // unit), and SwiGLU pairs values the same lane holds. The item's units follow each other as one stream of
+        // super-blocks: the first weights of unit u + 1 are fetched and decoded under the last products of unit u, so that only
+        // the item's first super-block is waited for.
+        int my_tiles = 0;
 #pragma unroll
-        for (int b = 0; b < NB; ++b) src_b[b] = W::src(b ? k.b1 : k.b0, e, k.gateup ? unit : NB * unit + b, n, g);
+        for (int t = 0; t < TPW; ++t) my_tiles += wave + WAVES * t < live_tiles ? 1 : 0;
+        const int8_t * a_base = k.xq + int64_t(tile_base + first_tile + wave) * 32 * k.b0.cols + lane * 16;
+        const int64_t a_tile = int64_t(WAVES) * 32 * k.b0.cols;
 
-        // The super-block loop is instantiated per number of live row tiles of the wave (0..TPW), so that its body is one
-        // straight line of code the scheduler can interleave. Every instance passes the same barriers.
+        // the weights this wave decodes for everybody: pieces wave * PIECES + q, piece = (slot, sub-block) = (id / 8, id % 8)
+        // (gate / up: the unit's 32 rows of the slot's bank; down: row tile NB * unit + slot)
+        const int my_slot = wave * PIECES / 8, my_ib0 = wave * PIECES % 8;
+        auto weight_tile = [&](int u, int b) { return k.gateup ? u : NB * u + b; };
+
+        // The stream is instantiated per number of live row tiles of the wave (0..TPW), so that its body is one straight
+        // line of code the scheduler can interleave. Every instance passes the same barriers.
         auto body = [&](auto mt_tag) {
             constexpr int MT = decltype(mt_tag)::value;
             constexpr int MTA = MT ? MT : 1;
@@ -682,120 +727,177 @@ __global__ __launch_bounds__(256 * NB) void plane_gemm_k(GemmArgs k) {
             for (int t = 0; t < MTA; ++t)
 #pragma unroll
                 for (int b = 0; b < NB; ++b) acc_clear(acc[t][b]);
-
-            // the codes and the scale record are fetched one super-block before they are decoded, so that their latency is
-            // not waited for
-            typename W::Rec f_rec = {};
-            typename W::Code f_code[2] = {};
-            typename W::DRec d_rec[NB] = {}, d_rec_next[NB] = {};
-            auto fetch = [&](int sb) {
-                f_rec = W::rec(wsrc, sb);
+            // the results of unit u (acc) to memory; result register i of lane half g is tile row 8 (i / 4) + 4 g + i % 4, weight
+            // row n. The rows' assignments and scales are read first, all at once: a read per element inside the store loop
+            // would serialise on LDS latency.
+            auto store_unit = [&](int u, bool zero) {
+                if constexpr (W::kRowMul) {
 #pragma unroll
-                for (int j = 0; j < 2; ++j) f_code[j] = W::code(wsrc, sb * 8 + 2 * mg + j);
-            };
-            auto fetch_d = [&](int sb) {
-                if constexpr (!W::kFp8) {
+                    for (int b = 0; b < NB; ++b) {
+                        const float rm = W::rowmul(b ? k.b1 : k.b0, e, weight_tile(u, b), n);
 #pragma unroll
-                    for (int b = 0; b < NB; ++b) d_rec_next[b] = W::drec(src_b[b], sb);
+                        for (int t = 0; t < MT; ++t)
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) acc[t][b].sum[i] = __fmul_rn(acc[t][b].sum[i], rm);
+                    }
                 }
-            };
-            auto decode_one = [&](int buf, int j) {
-                const int ib = 2 * mg + j;
-                v4i w[P];
-                W::planes(f_code[j], f_rec, ib, g, s_tab, s_lat, w);
 #pragma unroll
-                for (int p = 0; p < P; ++p) bs[(((buf * NB + nbw) * P + p) * 8 + ib) * 64 + lane] = w[p];
-            };
-            auto decode_into = [&](int buf) { decode_one(buf, 0); decode_one(buf, 1); };
-            // operand A, two k-steps (sub-blocks) per slot, fetched kSlots - 1 slots before its products
-            constexpr int kSlots = 4;
-            v4i a_reg[kSlots][MTA][2];
-            auto load_a = [&](int slot, int pair) {
+                for (int t = 0; t < MT; ++t) {
+                    int asg[16];
+                    float scl[16];
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
+                    for (int i = 0; i < 16; ++i) {
+                        const int m = (wave + WAVES * t) * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                        asg[i] = s_asg[m];
+                        scl[i] = s_scale[m];
+                    }
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) a_reg[slot][t][h] = *reinterpret_cast<const v4i *>(a_base + t * a_tile + (int64_t(pair) * 2 + h) * 1024);
-            };
-
-            const int pairs = sb_end * 4;
-            if (sb_end > 0) {
-                fetch(0);
-                fetch_d(0);
+                    for (int i = 0; i < 16; ++i) {
+                        if (asg[i] < 0) continue;
+                        uint16_t * o = k.out + int64_t(asg[i]) * rows;
+                        if (k.gateup) {
+                            o[u * 32 + n] = zero ? uint16_t(0) : swiglu_half(acc[t][0].sum[i], acc[t][NB - 1].sum[i], scl[i]);
+                        } else {
 #pragma unroll
-                for (int q = 0; q < kSlots - 1; ++q) load_a(q, min(q, pairs - 1));
-                decode_into(0);
-                fetch(min(1, sb_end - 1));
-            }
-            __syncthreads();
-            for (int sb = 0; sb < sb_end; ++sb) {
-                const int buf = sb & 1;
-#pragma unroll
-                for (int b = 0; b < NB; ++b) d_rec[b] = d_rec_next[b];
-                // The decode of the next super-block's two sub-blocks is placed between the groups of products, so that its
-                // vector work runs while the matrix pipe works through the group just issued. Past the last super-block the
-                // fetch repeats it and the decode fills the stage nobody reads: no branches here.
-                fetch_d(min(sb + 1, sb_end - 1));
-#pragma unroll
-                for (int jp = 0; jp < 4; ++jp) {
-                    if (jp == 1) { __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, 0); __builtin_amdgcn_sched_barrier(0); }
-                    if (jp == 2) { __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, 1); __builtin_amdgcn_sched_barrier(0); }
-                    if (jp == 3) { __builtin_amdgcn_sched_barrier(0); fetch(min(sb + 2, sb_end - 1)); __builtin_amdgcn_sched_barrier(0); }
-                    load_a((jp + kSlots - 1) % kSlots, min(sb * 4 + jp + kSlots - 1, pairs - 1));
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        const int ib = 2 * jp + h;
-#pragma unroll
-                        for (int b = 0; b < NB; ++b) {
-                            v4i w[P];
-#pragma unroll
-                            for (int p = 0; p < P; ++p) w[p] = bs[(((buf * NB + b) * P + p) * 8 + ib) * 64 + lane];
-#pragma unroll
-                            for (int t = 0; t < MT; ++t) acc_step(acc[t][b], a_reg[jp % kSlots][t][h], w, ib == 0);
+                            for (int b = 0; b < NB; ++b) o[(NB * u + b) * 32 + n] = zero ? uint16_t(0) : scaled_half(acc[t][b].sum[i], scl[i]);
                         }
                     }
                 }
+            };
+
+            // a stream over the units [ub, ub + nu) of the item
+            auto run = [&](int ub, int nu) {
+            const int total = nu * sb_full, pairs_u = sb_full * 4;
+
+            // Loads run ahead of the products through the item's (unit, super-block) steps: codes and scale records two
+            // steps (decoded one step ahead), the fold's scales one step, operand A kSlots - 1 pairs of sub-blocks. Past a
+            // unit's last step they go on into the next unit's first ones; past the item's last step they repeat it (from
+            // the cache, feeding nothing): selects between two base pointers, no branches around loads.
+            typename W::Rec f_rec = {};
+            typename W::Code f_code[PIECES] = {};
+            typename W::DRec d_rec[NB] = {}, d_rec_next[NB] = {};
+            typename W::Src src_cur = W::src(my_slot ? k.b1 : k.b0, e, weight_tile(ub, my_slot), n, g), src_nxt = src_cur;
+            typename W::Src dsrc_cur[NB], dsrc_nxt[NB];
 #pragma unroll
-                for (int b = 0; b < NB; ++b)
+            for (int b = 0; b < NB; ++b) dsrc_nxt[b] = dsrc_cur[b] = W::src(b ? k.b1 : k.b0, e, weight_tile(ub, b), n, g);
+            bool last = nu <= 1;
+            // step `ahead` steps after super-block sb of the current unit: in this unit, in the next one, or the item's last
+            auto fetch = [&](int sb, int ahead) {
+                const int t = sb + ahead;
+                const bool here = t < sb_full || last;
+                const typename W::Src & src = here ? src_cur : src_nxt;
+                const int at = t < sb_full ? t : last ? sb_full - 1 : t - sb_full;
+                f_rec = W::rec(src, at);
 #pragma unroll
-                    for (int t = 0; t < MT; ++t) acc_fold(acc[t][b], d_rec[b]);
-                __syncthreads();
-            }
-            if constexpr (W::kRowMul) {
+                for (int j = 0; j < PIECES; ++j) f_code[j] = W::code(src, at * 8 + my_ib0 + j);
+            };
+            auto fetch_d = [&](int sb, int ahead) {
+                if constexpr (!W::kFp8) {
+                    const int t = sb + ahead;
+                    const bool here = t < sb_full || last;
+                    const int at = t < sb_full ? t : last ? sb_full - 1 : t - sb_full;
 #pragma unroll
-                for (int b = 0; b < NB; ++b) {
-                    const float rm = W::rowmul(b ? k.b1 : k.b0, e, k.gateup ? unit : NB * unit + b, n);
-#pragma unroll
-                    for (int t = 0; t < MT; ++t)
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) acc[t][b].sum[i] = __fmul_rn(acc[t][b].sum[i], rm);
+                    for (int b = 0; b < NB; ++b) d_rec_next[b] = W::drec(here ? dsrc_cur[b] : dsrc_nxt[b], at);
                 }
-            }
-            // result register i of lane half g is tile row 8 (i / 4) + 4 g + i % 4, weight row n. The rows' assignments and
-            // scales are read first, all at once: a read per element inside the store loop would serialise on LDS latency.
+            };
+            auto decode_one = [&](int buf, int j) {
+                const int ib = my_ib0 + j;
+                v4i w[P];
+                W::planes(f_code[j], f_rec, ib, g, s_tab, s_lat, w);
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                int asg[16];
-                float scl[16];
+                for (int p = 0; p < P; ++p) bs[(((buf * NB + my_slot) * P + p) * 8 + ib) * 64 + lane] = w[p];
+            };
+            // operand A (the same rows for every unit), two k-steps (sub-blocks) per slot
+            constexpr int kSlots = 4;
+            v4i a_reg[kSlots][MTA][2];
+            auto load_a = [&](int slot, int pair) {   // pair counted from the current unit's first
+                const int at = pair < pairs_u ? pair : last ? pairs_u - 1 : pair - pairs_u;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int m = (wave + 4 * t) * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-                    asg[i] = s_asg[m];
-                    scl[i] = s_scale[m];
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) a_reg[slot][t][h] = *reinterpret_cast<const v4i *>(a_base + t * a_tile + (int64_t(at) * 2 + h) * 1024);
+            };
+            if (total > 0) {
+                if (!last) {
+                    src_nxt = W::src(my_slot ? k.b1 : k.b0, e, weight_tile(ub + 1, my_slot), n, g);
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) dsrc_nxt[b] = W::src(b ? k.b1 : k.b0, e, weight_tile(ub + 1, b), n, g);
                 }
+                fetch(0, 0);
+                fetch_d(0, 0);
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    if (asg[i] < 0) continue;
-                    uint16_t * o = k.out + int64_t(asg[i]) * rows;
-                    if (k.gateup) {
-                        o[unit * 32 + n] = swiglu_half(acc[t][0].sum[i], acc[t][NB - 1].sum[i], scl[i]);
-                    } else {
+                for (int q = 0; q < kSlots - 1; ++q) load_a(q, q);
 #pragma unroll
-                        for (int b = 0; b < NB; ++b) o[(NB * unit + b) * 32 + n] = scaled_half(acc[t][b].sum[i], scl[i]);
+                for (int j = 0; j < PIECES; ++j) decode_one(0, j);
+                fetch(0, 1);
+            }
+            __syncthreads();
+            int parity = 0;   // stage that holds the current unit's first super-block
+            for (int uu = 0; uu < (total > 0 ? nu : 0); ++uu) {
+                for (int sb = 0; sb < sb_full; ++sb) {
+                    const int buf = (parity + sb) & 1;
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) d_rec[b] = d_rec_next[b];
+                    // The decode of the next step's pieces is placed between the groups of products, so that its vector
+                    // work runs while the matrix pipe works through the group just issued.
+                    fetch_d(sb, 1);
+#pragma unroll
+                    for (int jp = 0; jp < 4; ++jp) {
+                        if constexpr (PIECES == 2) {
+                            if (jp == 1) { __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, 0); __builtin_amdgcn_sched_barrier(0); }
+                            if (jp == 2) { __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, 1); __builtin_amdgcn_sched_barrier(0); }
+                        } else {
+                            __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, jp); __builtin_amdgcn_sched_barrier(0);
+                        }
+                        if (jp == 3) { __builtin_amdgcn_sched_barrier(0); fetch(sb, 2); __builtin_amdgcn_sched_barrier(0); }
+                        load_a((jp + kSlots - 1) % kSlots, sb * 4 + jp + kSlots - 1);
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int ib = 2 * jp + h;
+#pragma unroll
+                            for (int b = 0; b < NB; ++b) {
+                                v4i w[P];
+#pragma unroll
+                                for (int p = 0; p < P; ++p) w[p] = bs[(((buf * NB + b) * P + p) * 8 + ib) * 64 + lane];
+#pragma unroll
+                                for (int t = 0; t < MT; ++t) acc_step(acc[t][b], a_reg[jp % kSlots][t][h], w, ib == 0);
+                            }
+                        }
                     }
+#pragma unroll
+                    for (int b = 0; b < NB; ++b)
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) acc_fold(acc[t][b], d_rec[b]);
+                    __syncthreads();
                 }
+                if (uu == 0) rows_to_lds();   // the rows' assignments and scales: long arrived
+                store_unit(ub + uu, false);
+#pragma unroll
+                for (int t = 0; t < MTA; ++t)
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) acc_clear(acc[t][b]);
+                // on to the next unit: its first super-block sits in the stage already, its first pairs of operand A in registers
+                parity = (parity + sb_full) & 1;
+                src_cur = src_nxt;
+#pragma unroll
+                for (int b = 0; b < NB; ++b) dsrc_cur[b] = dsrc_nxt[b];
+                last = uu + 2 >= nu;
+                if (!last) {
+                    src_nxt = W::src(my_slot ? k.b1 : k.b0, e, weight_tile(ub + uu + 2, my_slot), n, g);
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) dsrc_nxt[b] = W::src(b ? k.b1 : k.b0, e, weight_tile(ub + uu + 2, b), n, g);
+                }
+            }
+            };
+            // (units of a single super-block cannot look two steps ahead into one next unit: they run one by one)
+            if (sb_full >= 2) run(u0, live_units);
+            else for (int i = 0; i < live_units; ++i) run(u0 + i, 1);
+            if (live_units < k.unit_group) {   // units past the shared expert's size: zeros
+                if (live_units * sb_full == 0) rows_to_lds();
+                for (int u = u0 + live_units; u < u0 + k.unit_group; ++u) store_unit(u, true);
             }
         };
-        if constexpr (NB == 2) {
+        if constexpr (TPW == 1) {
             if (my_tiles) body(std::integral_constant<int, 1>{}); else body(std::integral_constant<int, 0>{});
         } else {
             switch (my_tiles) {
@@ -877,13 +979,17 @@ int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, co
 bool plane_gemm_has(uint32_t type) { return type == TQMOE_IQ4_XS || type == TQMOE_IQ3_S || type == TQMOE_Q4_K || type == TQMOE_NVFP4G; }
 bool plane_gemm_is_fp8(uint32_t type) { return type == TQMOE_NVFP4G; }
 
+// Two operand slots run on eight waves (a row tile each). The four-wave arrangement of the same kernel (two row tiles a wave,
+// half the LDS reads per product, twice the registers) measured 15 to 20 % slower on every format: one wave per SIMD leaves
+// nothing to issue while that wave waits.
 template <class W> static void plane_gemm_launch(int nb, const GemmArgs & k, unsigned blocks, hipStream_t s) {
     const size_t lds = size_t(2) * nb * W::kPlanes * 8 * 64 * sizeof(v4i);
+    constexpr size_t kLdsMost = size_t(2) * 2 * 3 * 8 * 64 * sizeof(v4i);
     if (nb == 2) {
-        if (lds > 65536 - 24576) allow_dynamic_lds(reinterpret_cast<const void *>(&plane_gemm_k<2, W>), 2 * 2 * 3 * 8 * 64 * sizeof(v4i));
-        plane_gemm_k<2, W><<<blocks, 512, lds, s>>>(k);
+        if (lds > 65536 - 24576) allow_dynamic_lds(reinterpret_cast<const void *>(&plane_gemm_k<2, W, 8>), kLdsMost);
+        plane_gemm_k<2, W, 8><<<blocks, 512, lds, s>>>(k);
     } else {
-        plane_gemm_k<1, W><<<blocks, 256, lds, s>>>(k);
+        plane_gemm_k<1, W, 4><<<blocks, 256, lds, s>>>(k);
     }
 }
 
@@ -893,11 +999,14 @@ int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const i
     const int nb = gateup || b0.rows % 64 == 0 ? 2 : 1;
     const int units = gateup ? b0.rows / 32 : b0.rows / (32 * nb);
     const int64_t tiles = grouped_row_tiles(assignments, experts);
+    // units per item: about sixteen super-block steps of products behind one item's start-up, in a divisor of the units
+    int unit_group = std::max(1, std::min(8, 16 / std::max(1, b0.cols / 256)));
+    while (units % unit_group) --unit_group;
     GemmArgs k{view(b0), b1 ? view(*b1) : view(b0), xq, xs, counts, offsets, perm, plan_at(xs, tiles * 32, experts), experts, static_cast<uint16_t *>(out_f16),
-               gateup, units, shared_expert, shared_lim};
+               gateup, units, unit_group, shared_expert, shared_lim};
     // one block per compute unit (the kernel's registers and LDS allow no second one), walking the work items
     const int cus = cu_count();
-    const int64_t most = (tiles / kChunkTiles + experts + 7) / 8 * 8 * units;     // an upper bound of the items
+    const int64_t most = (tiles / kChunkTiles + experts + 7) / 8 * 8 * (units / unit_group);     // an upper bound of the items
     const unsigned blocks = unsigned(std::min<int64_t>((cus + 7) / 8 * 8, most));
     switch (b0.type) {
         case TQMOE_IQ4_XS: plane_gemm_launch<WIq4xs>(nb, k, blocks, s); break;

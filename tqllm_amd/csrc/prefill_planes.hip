@@ -177,11 +177,11 @@ __global__ __launch_bounds__(256) void group_rows_k(const void * __restrict__ x,
     }
 }
 
-// The same for row lengths of 512, 1024 or 2048: one block per row tile. A wave quantises eight rows out of registers
+// The same for row lengths that are a multiple of 256 up to 2048: one block per row tile. A wave quantises eight rows out of registers
 // (one read of the input) into an LDS copy of the tile, every 32-byte block already in operand order; then lane (g, r)
 // of every wave moves the 16 bytes of row r, half g of one k-step at a time, so each k-step's 1 KB leaves as one fully
 // coalesced store instead of 256 scattered dwords.
-template <int XT, int GPL, bool F8>   // groups of 8 values per lane: cols = 512 GPL
+template <int XT, int GPL, bool F8>   // groups of 8 values per lane: 512 (GPL - 1) < cols <= 512 GPL
 __global__ __launch_bounds__(256) void group_rows_tile_k(const void * __restrict__ x, int cols, const int * __restrict__ counts, const int * __restrict__ offsets,
                                                               const int * __restrict__ perm, int experts, int xdiv, int8_t * __restrict__ q, float * __restrict__ scale,
                                                               Plan plan) {
@@ -191,7 +191,8 @@ __global__ __launch_bounds__(256) void group_rows_tile_k(const void * __restrict
     const int e = owner_of(plan.tile_base, experts, tile_index);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, stride = cols + 16;
     const int cnt = counts[e], first = (tile_index - plan.tile_base[e]) * 32, off = offsets[e];
-    constexpr int kBatch = 8 / GPL;   // rows whose loads are in flight together: 64 values per lane
+    constexpr int kBatch = GPL == 3 ? 2 : 8 / GPL;   // rows whose loads are in flight together: about 64 values per lane
+    const int groups = cols / 8;
     for (int r0 = wave * 8; r0 < wave * 8 + 8; r0 += kBatch) {
         if (first + r0 >= cnt) break;
         float v[kBatch][GPL][8];
@@ -200,7 +201,12 @@ __global__ __launch_bounds__(256) void group_rows_tile_k(const void * __restrict
             const int i = min(first + r0 + b, cnt - 1);          // past the count: a valid row again, not stored
             const int64_t row = perm[off + i] / xdiv;
 #pragma unroll
-            for (int gq = 0; gq < GPL; ++gq) load8<XT>(x, row * cols + (lane + 64 * gq) * 8, v[b][gq]);
+            for (int gq = 0; gq < GPL; ++gq) {
+                if (lane + 64 * gq < groups) load8<XT>(x, row * cols + (lane + 64 * gq) * 8, v[b][gq]);
+                else
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[b][gq][j] = 0.f;
+            }
         }
 #pragma unroll
         for (int b = 0; b < kBatch; ++b) {
@@ -217,6 +223,7 @@ __global__ __launch_bounds__(256) void group_rows_tile_k(const void * __restrict
 #pragma unroll
                 for (int gq = 0; gq < GPL; ++gq) {
                     const int gi = lane + 64 * gq, sub = gi >> 2, d0 = 2 * (gi & 3);
+                    if (gi >= groups) break;
                     const float * vv = v[b][gq];
                     const uint32_t wd[2] = {pack4_q<F8>(vv[0] * mul, vv[1] * mul, vv[2] * mul, vv[3] * mul), pack4_q<F8>(vv[4] * mul, vv[5] * mul, vv[6] * mul, vv[7] * mul)};
 #pragma unroll
@@ -264,7 +271,6 @@ struct GemmArgs {
     Plan plan;
     int experts;
     uint16_t * out;           // fp16 [assignments][rows]: silu(gate) * up, or the plain product
-    int gateup;
     int units;                // weight-row units per expert: rows / 32 (gate / up, and down with NB = 1), rows / 64 (down, NB = 2)
     int unit_group;           // consecutive units an item runs through (a divisor of units): short rows get more per item
     int shared_expert;        // index of the expert whose rows (gate / up) or columns (down) stop at shared_lim, or -1
@@ -519,7 +525,9 @@ template <class W> __device__ __forceinline__ void acc_fold(Acc<W> & a, const ty
 // WAVES waves (8 with two operand slots, 4 with one). Decoding: the 8 * NB (slot, sub-block) pieces of a super-block are
 // dealt to the waves in order, 8 NB / WAVES each. Products: a wave takes 8 / WAVES row tiles (tile `wave`, then every
 // WAVES-th) against every slot.
-template <int NB, class W, int WAVES>
+// GATEUP: the two slots are the gate and the up bank and SwiGLU joins them; else a plain product (a kernel name of its own
+// for each, so that a trace tells them apart)
+template <int NB, class W, int WAVES, bool GATEUP>
 __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
     constexpr int THREADS = 64 * WAVES, P = W::kPlanes;
     constexpr int TPW = 8 / WAVES;           // row tiles per wave of a shared chunk
@@ -577,8 +585,8 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
         const bool is_shared = e == k.shared_expert;
         const int u0 = ug * k.unit_group;                                   // the item's first unit
         // gate / up rows of the shared expert beyond its size: no products, zeros stored (the rows are quantised whole later)
-        const int live_units = k.gateup && is_shared ? min(max(k.shared_lim / 32 - u0, 0), k.unit_group) : k.unit_group;
-        const int sb_full = !k.gateup && is_shared ? k.shared_lim / 256 : NSB;   // super-blocks of a live unit's products
+        const int live_units = GATEUP && is_shared ? min(max(k.shared_lim / 32 - u0, 0), k.unit_group) : k.unit_group;
+        const int sb_full = !GATEUP && is_shared ? k.shared_lim / 256 : NSB;   // super-blocks of a live unit's products
         const int cnt = cnts[e], tiles_e = (cnt + 31) >> 5;
         const int first_tile = local * kChunkTiles;                         // of this expert
         const int live_tiles = min(kChunkTiles, tiles_e - first_tile);      // of this block
@@ -611,12 +619,12 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
 #pragma unroll
             for (int q = 0; q < SPW; ++q) {
                 const int b = SPW == 1 ? nbw : q;
-                wt[q] = k.gateup ? 4 * unit + mg : (4 * unit + mg) * NB + b;
+                wt[q] = GATEUP ? 4 * unit + mg : (4 * unit + mg) * NB + b;
                 wsrc[q] = W::src(b ? k.b1 : k.b0, e, wt[q], n, g);
             }
             {
-                const bool wdead = k.gateup && is_shared && wt[0] * 32 >= k.shared_lim;   // gate / up: the slots share the tile number
-                sbe = wdead ? 0 : !k.gateup && is_shared ? k.shared_lim / 256 : NSB;
+                const bool wdead = GATEUP && is_shared && wt[0] * 32 >= k.shared_lim;   // gate / up: the slots share the tile number
+                sbe = wdead ? 0 : !GATEUP && is_shared ? k.shared_lim / 256 : NSB;
             }
             const int8_t * a_ptr = k.xq + int64_t(tile_base + first_tile) * 32 * k.b0.cols + lane * 16;
             struct Stage { typename W::Code code[SPW][8]; typename W::Rec rec[SPW]; typename W::DRec drec[SPW]; v4i a[8]; };
@@ -670,14 +678,14 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
             rows_to_lds();
             float * ex = reinterpret_cast<float *>(lds);
             constexpr bool kExchange = SPW == 1 && NB == 2;   // gate and up of a weight tile sit in two waves
-            if (k.gateup && kExchange) {   // the up waves hand their sums to the gate waves of the same weight tile
+            if (GATEUP && kExchange) {   // the up waves hand their sums to the gate waves of the same weight tile
                 if (nbw == 1) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) ex[(mg * 16 + i) * 64 + lane] = acc[0].sum[i];
                 }
                 __syncthreads();
             }
-            if (!(k.gateup && kExchange && nbw == 1)) {
+            if (!(GATEUP && kExchange && nbw == 1)) {
                 int asg[16];
                 float scl[16];
 #pragma unroll
@@ -690,7 +698,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                 for (int i = 0; i < 16; ++i) {
                     if (asg[i] < 0) continue;
                     uint16_t * o = k.out + int64_t(asg[i]) * rows;
-                    if (k.gateup) {
+                    if (GATEUP) {
                         const float up = kExchange ? ex[(mg * 16 + i) * 64 + lane] : acc[SPW - 1].sum[i];
                         o[wt[0] * 32 + n] = swiglu_half(acc[0].sum[i], up, scl[i]);
                     } else {
@@ -715,7 +723,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
         // the weights this wave decodes for everybody: pieces wave * PIECES + q, piece = (slot, sub-block) = (id / 8, id % 8)
         // (gate / up: the unit's 32 rows of the slot's bank; down: row tile NB * unit + slot)
         const int my_slot = wave * PIECES / 8, my_ib0 = wave * PIECES % 8;
-        auto weight_tile = [&](int u, int b) { return k.gateup ? u : NB * u + b; };
+        auto weight_tile = [&](int u, int b) { return GATEUP ? u : NB * u + b; };
 
         // The stream is instantiated per number of live row tiles of the wave (0..TPW), so that its body is one straight
         // line of code the scheduler can interleave. Every instance passes the same barriers.
@@ -755,7 +763,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                     for (int i = 0; i < 16; ++i) {
                         if (asg[i] < 0) continue;
                         uint16_t * o = k.out + int64_t(asg[i]) * rows;
-                        if (k.gateup) {
+                        if (GATEUP) {
                             o[u * 32 + n] = zero ? uint16_t(0) : swiglu_half(acc[t][0].sum[i], acc[t][NB - 1].sum[i], scl[i]);
                         } else {
 #pragma unroll
@@ -938,13 +946,16 @@ int64_t grouped_scale_words(int64_t assignments, int experts) { return grouped_r
 template <int XT, bool F8>
 static void group_rows_launch(const void * x, int cols, const int * counts, const int * offsets, const int * perm, int experts, int64_t tiles, int xdiv, int8_t * q,
                               float * scale, const Plan & plan, hipStream_t s) {
-    if (cols == 512 || cols == 1024 || cols == 2048) {
+    if (cols % 256 == 0 && cols <= 2048) {
         const size_t lds = size_t(32) * size_t(cols + 16);
         auto launch = [&](auto kernel) {
-            if (lds > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kernel), 32 * (2048 + 16));
+            if (lds > 65536 - 1024) allow_dynamic_lds(reinterpret_cast<const void *>(kernel), 32 * (2048 + 16));
             kernel<<<unsigned(tiles), 256, lds, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan);
         };
-        if (cols == 512) launch(group_rows_tile_k<XT, 1, F8>); else if (cols == 1024) launch(group_rows_tile_k<XT, 2, F8>); else launch(group_rows_tile_k<XT, 4, F8>);
+        if (cols <= 512) launch(group_rows_tile_k<XT, 1, F8>);
+        else if (cols <= 1024) launch(group_rows_tile_k<XT, 2, F8>);
+        else if (cols <= 1536) launch(group_rows_tile_k<XT, 3, F8>);
+        else launch(group_rows_tile_k<XT, 4, F8>);
         return;
     }
     group_rows_k<XT, F8><<<unsigned(tiles * 4), 256, 0, s>>>(x, cols, counts, offsets, perm, experts, xdiv, q, scale, plan);
@@ -982,15 +993,16 @@ bool plane_gemm_is_fp8(uint32_t type) { return type == TQMOE_NVFP4G; }
 // Two operand slots run on eight waves (a row tile each). The four-wave arrangement of the same kernel (two row tiles a wave,
 // half the LDS reads per product, twice the registers) measured 15 to 20 % slower on every format: one wave per SIMD leaves
 // nothing to issue while that wave waits.
-template <class W> static void plane_gemm_launch(int nb, const GemmArgs & k, unsigned blocks, hipStream_t s) {
+template <class W> static void plane_gemm_launch(int nb, bool gateup, const GemmArgs & k, unsigned blocks, hipStream_t s) {
     const size_t lds = size_t(2) * nb * W::kPlanes * 8 * 64 * sizeof(v4i);
     constexpr size_t kLdsMost = size_t(2) * 2 * 3 * 8 * 64 * sizeof(v4i);
-    if (nb == 2) {
-        if (lds > 65536 - 24576) allow_dynamic_lds(reinterpret_cast<const void *>(&plane_gemm_k<2, W, 8>), kLdsMost);
-        plane_gemm_k<2, W, 8><<<blocks, 512, lds, s>>>(k);
-    } else {
-        plane_gemm_k<1, W, 4><<<blocks, 256, lds, s>>>(k);
-    }
+    auto launch = [&](auto kernel, unsigned threads) {
+        if (lds > 65536 - 24576) allow_dynamic_lds(reinterpret_cast<const void *>(kernel), kLdsMost);
+        kernel<<<blocks, threads, lds, s>>>(k);
+    };
+    if (gateup) launch(&plane_gemm_k<2, W, 8, true>, 512);
+    else if (nb == 2) launch(&plane_gemm_k<2, W, 8, false>, 512);
+    else launch(&plane_gemm_k<1, W, 4, false>, 256);
 }
 
 // assignments = total entries of perm (it fixes where the index behind the scales lies)
@@ -1003,16 +1015,16 @@ int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const i
     int unit_group = std::max(1, std::min(8, 16 / std::max(1, b0.cols / 256)));
     while (units % unit_group) --unit_group;
     GemmArgs k{view(b0), b1 ? view(*b1) : view(b0), xq, xs, counts, offsets, perm, plan_at(xs, tiles * 32, experts), experts, static_cast<uint16_t *>(out_f16),
-               gateup, units, unit_group, shared_expert, shared_lim};
+               units, unit_group, shared_expert, shared_lim};
     // one block per compute unit (the kernel's registers and LDS allow no second one), walking the work items
     const int cus = cu_count();
     const int64_t most = (tiles / kChunkTiles + experts + 7) / 8 * 8 * (units / unit_group);     // an upper bound of the items
     const unsigned blocks = unsigned(std::min<int64_t>((cus + 7) / 8 * 8, most));
     switch (b0.type) {
-        case TQMOE_IQ4_XS: plane_gemm_launch<WIq4xs>(nb, k, blocks, s); break;
-        case TQMOE_IQ3_S: plane_gemm_launch<WIq3s>(nb, k, blocks, s); break;
-        case TQMOE_Q4_K: plane_gemm_launch<WQ4k>(nb, k, blocks, s); break;
-        case TQMOE_NVFP4G: plane_gemm_launch<WNvfp4>(nb, k, blocks, s); break;
+        case TQMOE_IQ4_XS: plane_gemm_launch<WIq4xs>(nb, gateup != 0, k, blocks, s); break;
+        case TQMOE_IQ3_S: plane_gemm_launch<WIq3s>(nb, gateup != 0, k, blocks, s); break;
+        case TQMOE_Q4_K: plane_gemm_launch<WQ4k>(nb, gateup != 0, k, blocks, s); break;
+        case TQMOE_NVFP4G: plane_gemm_launch<WNvfp4>(nb, gateup != 0, k, blocks, s); break;
         default: return -1;
     }
     return 0;

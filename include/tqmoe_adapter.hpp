@@ -161,6 +161,24 @@ struct ExpertFormat {
         check(rc, e);
         return true;
     }
+    // the same two products on E4M3 rows for NVFP4G banks (rows of tqmoe_group_rows_fp8, scale amax / 448 as
+    // src/core/fp8_gemm.cuh:19-31); false: the format has no fp8 grouped kernel
+    static bool expert_gemm_fp8(const tqmoe_bank & m, const uint8_t * xq, const float * xs, void * y_f16, const int * counts, const int * offsets, const int * perm,
+                                int n, int topk, void * stream) {
+        tqmoe_error e = fresh();
+        const int32_t rc = tqmoe_expert_gemm_fp8(&m, xq, xs, counts, offsets, perm, n, topk, topk, 0, y_f16, stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
+    static bool expert_gemm_gateup_fp8(const tqmoe_bank & g, const tqmoe_bank & u, const uint8_t * xq, const float * xs, void * y_f16, const int * counts,
+                                       const int * offsets, const int * perm, int n, int topk, void * stream) {
+        tqmoe_error e = fresh();
+        const int32_t rc = tqmoe_expert_gemm_gateup_fp8(&g, &u, xq, xs, counts, offsets, perm, n, topk, topk, 0, y_f16, stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
     // expert_gemm (weight_format.hpp:51-53) for any bank format: half input rows [n][cols] (or one row per assignment with
     // per_expert_input), y [n * topk][rows] half. Weights are decoded to fp16 tiles on the fly; fp32 accumulation.
     static bool expert_gemm(const tqmoe_bank & m, const void * x_f16, void * y_f16, const int * counts, const int * offsets, const int * perm, int n, int topk,

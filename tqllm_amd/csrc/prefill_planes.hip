@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256) void group_rows_tile_k(const void * __restrict
     for (int ks = wave; ks < S; ks += 4) dst[ks * 64] = *reinterpret_cast<const uint4 *>(tile_rows + r * stride + ks * 32 + g * 16);
 }
 
-// The same grouped operand from rows that are already int8 (quant_rows_i8_k's output: one scale per row, the bytes of every
+// The same grouped operand from rows that are already int8 (quant_rows_k's output: one scale per row, the bytes of every
 // 32-block in operand order): a pure copy. One block per row tile; lane (g, r) of every wave moves the 16 bytes of row r,
 // half g of one k-step at a time, so each k-step's 1 KB is written by one fully coalesced store. When several
 // assignments read one input row (xdiv > 1) the row is quantised once instead of once per assignment.

@@ -7,7 +7,8 @@
 // (lane = 32 g + r holds, for row r and 32-weight sub-block j, the 16 values {8g..8g+7} and {16+8g..16+8g+7} in the byte
 // order of the bank's code bytes) is contiguous, sub-blocks in order. A wave then loads its operand with one fully
 // coalesced instruction and no shuffle. The two 8-byte halves of that operand are the operands of two
-// v_mfma_f32_32x32x16_fp8_fp8, so the fp8 path shares the layout.
+// v_mfma_f32_32x32x16_fp8_fp8, and two sub-blocks' 32 bytes the operand of one
+// v_mfma_f32_32x32x64_f8f6f4 (which is what the fp8 path issues), so the fp8 path shares the layout.
 // Integer weights stay exact. A value is d * p with an integer p per weight of up to 13 bits (IQ4_XS: (ls - 32) * kv[q];
 // IQ3_S: (1 + 2 ls) * (+-lattice magnitude); Q4_K: sc * q, with the minimum's coefficient mn as a further plane that
 // is constant over a sub-block). p is split as 64 * h + l with h, l int8, taken per sub-block from 16-entry lookup
@@ -40,7 +41,7 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kChunkTiles = 8;                // row tiles (of 32 assignments) per chunk
+constexpr int kChunkTiles = 8;                // row tiles (of 32 assignments) per chunk; formats with registers to spare take chunks of twice that
 constexpr int kPlanExperts = 1024;              // experts whose index a block keeps in LDS
 
 // four scaled values -> four operand bytes: int8 (round to nearest) or E4M3 (round to nearest even; the values are
@@ -92,35 +93,37 @@ __global__ __launch_bounds__(256) void quant_rows_k(const void * __restrict__ x,
 }
 
 // Index of the grouped rows, kept behind the row scales: tile_base[e] = row tiles of the experts before e
-// (tiles_e = ceil(count_e / 32)), chunk_base[e] = chunks of kChunkTiles row tiles before e, both with a total at [experts].
+// (tiles_e = ceil(count_e / 32)), chunk_base[e] = chunks of kChunkTiles row tiles before e, chunk_base2[e] = chunks of twice
+// as many, all with a total at [experts].
 // Behind them 16 counters the product kernel hands work out with (zero between launches).
 constexpr int kPlanCounters = 16;
-struct Plan { const int * tile_base, * chunk_base; int * counters; };
+struct Plan { const int * tile_base, * chunk_base, * chunk_base2; int * counters; };
 __host__ __device__ inline Plan plan_at(const float * scale, int64_t grouped_rows, int experts) {
     const int * p = reinterpret_cast<const int *>(scale + grouped_rows);
-    return Plan{p, p + experts + 1, const_cast<int *>(p) + 2 * (experts + 1)};
+    return Plan{p, p + experts + 1, p + 2 * (experts + 1), const_cast<int *>(p) + 3 * (experts + 1)};
 }
 
-__global__ __launch_bounds__(64) void plan_k(const int * __restrict__ counts, int experts, int * __restrict__ tile_base, int * __restrict__ chunk_base,
-                                             int * __restrict__ counters) {
+__global__ __launch_bounds__(64) void plan_k(const int * __restrict__ counts, int experts, Plan plan) {
     const int lane = threadIdx.x;
-    if (lane < kPlanCounters) counters[lane] = 0;
-    int tbase = 0, cbase = 0;
+    int * tile_base = const_cast<int *>(plan.tile_base), * chunk_base = const_cast<int *>(plan.chunk_base), * chunk_base2 = const_cast<int *>(plan.chunk_base2);
+    if (lane < kPlanCounters) plan.counters[lane] = 0;
+    int tbase = 0, cbase = 0, cbase2 = 0;
     for (int e0 = 0; e0 < experts; e0 += 64) {
         const int e = e0 + lane;
         const int tiles = e < experts ? (max(counts[e], 0) + 31) >> 5 : 0;
-        const int chunks = (tiles + kChunkTiles - 1) / kChunkTiles;
-        int ti = tiles, ci = chunks;
+        const int chunks = (tiles + kChunkTiles - 1) / kChunkTiles, chunks2 = (tiles + 2 * kChunkTiles - 1) / (2 * kChunkTiles);
+        int ti = tiles, ci = chunks, c2 = chunks2;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
-            const int a = __shfl_up(ti, d, 64), b = __shfl_up(ci, d, 64);
-            if (lane >= d) { ti += a; ci += b; }
+            const int a = __shfl_up(ti, d, 64), b = __shfl_up(ci, d, 64), c = __shfl_up(c2, d, 64);
+            if (lane >= d) { ti += a; ci += b; c2 += c; }
         }
-        if (e < experts) { tile_base[e] = tbase + ti - tiles; chunk_base[e] = cbase + ci - chunks; }
+        if (e < experts) { tile_base[e] = tbase + ti - tiles; chunk_base[e] = cbase + ci - chunks; chunk_base2[e] = cbase2 + c2 - chunks2; }
         tbase += __shfl(ti, 63, 64);
         cbase += __shfl(ci, 63, 64);
+        cbase2 += __shfl(c2, 63, 64);
     }
-    if (lane == 0) { tile_base[experts] = tbase; chunk_base[experts] = cbase; }
+    if (lane == 0) { tile_base[experts] = tbase; chunk_base[experts] = cbase; chunk_base2[experts] = cbase2; }
 }
 
 // largest e in [0, experts) with base[e] <= unit, for unit < base[experts] (experts with no unit share their successor's
@@ -332,7 +335,8 @@ __device__ const int8_t kIq4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -
 // 16 weights {8g..8g+7} and {16+8g..16+8g+7}: Src are its base pointers, Code what it loads per sub-block, Rec what
 // decoding needs of the sub-block's super-block, DRec what the fold needs of it (the lane's row, any g).
 // planes() turns a Code into kPlanes operand registers; tables() fills the lookup tables (and the lattice) in LDS.
-struct WIq4xs {   // tile-major codes (512 B per sub-block of a tile), 8-byte records (256 B per super-block of a tile)
+struct WIq4xs {
+    static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)   // tile-major codes (512 B per sub-block of a tile), 8-byte records (256 B per super-block of a tile)
     static constexpr int kPlanes = 2, kTabBytes = 64 * 32, kLattice = 1;
     static constexpr bool kFp8 = false, kMin = false, kRowMul = false;
     struct Code { uint2 c; };
@@ -359,7 +363,8 @@ struct WIq4xs {   // tile-major codes (512 B per sub-block of a tile), 8-byte re
     static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
 };
 
-struct WQ4k {   // row-major: 16 code bytes per sub-block, a 16-byte record (d | dmin << 16, twelve bytes of 6-bit scales and minimums) per super-block
+struct WQ4k {
+    static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)   // row-major: 16 code bytes per sub-block, a 16-byte record (d | dmin << 16, twelve bytes of 6-bit scales and minimums) per super-block
     static constexpr int kPlanes = 3, kTabBytes = 64 * 32, kLattice = 1;
     static constexpr bool kFp8 = false, kMin = true, kRowMul = false;
     struct Code { uint2 c; };
@@ -391,7 +396,8 @@ struct WQ4k {   // row-major: 16 code bytes per sub-block, a 16-byte record (d |
     static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
 };
 
-struct WIq3s {   // row-major: 12 code bytes per sub-block (8 lattice indices, 32 sign bits), a 16-byte record per super-block
+struct WIq3s {
+    static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)   // row-major: 12 code bytes per sub-block (8 lattice indices, 32 sign bits), a 16-byte record per super-block
     static constexpr int kPlanes = 2, kTabBytes = 16 * 32, kLattice = 512;
     static constexpr bool kFp8 = false, kMin = false, kRowMul = false;
     struct Code { uint32_t qs0, qs1, sg; };
@@ -437,7 +443,8 @@ struct WIq3s {   // row-major: 12 code bytes per sub-block (8 lattice indices, 3
     static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
 };
 
-struct WNvfp4 {   // row-major: 16 code bytes per sub-block, one E4M3 scale byte per 16 weights, one fp32 global per row
+struct WNvfp4 {
+    static constexpr bool kWideChunks = true;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)   // row-major: 16 code bytes per sub-block, one E4M3 scale byte per 16 weights, one fp32 global per row
     static constexpr int kPlanes = 1, kTabBytes = 256 * 16, kLattice = 1;
     static constexpr bool kFp8 = true, kRowMul = true;
     struct Code { uint2 c; };
@@ -495,16 +502,21 @@ template <class W> __device__ __forceinline__ void acc_clear(Acc<W> & a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) a.sum[i] = 0.f;
 }
-template <class W> __device__ __forceinline__ void acc_step(Acc<W> & a, v4i x, const v4i * w, bool first_of_sb) {
+// two consecutive sub-blocks (64 weights of the rows) of operand A and of the weight planes. int8: one
+// v_mfma_i32_32x32x32_i8 per sub-block and plane. fp8: one v_mfma_f32_32x32x64_f8f6f4 (both operands E4M3, no block
+// scales) for the pair: twice the rate of the 32x32x16 fp8 instruction on this part.
+typedef int v8i __attribute__((ext_vector_type(8)));
+template <class W> __device__ __forceinline__ void acc_step2(Acc<W> & a, v4i x0, v4i x1, const v4i * w0, const v4i * w1, bool first_of_sb) {
     if constexpr (W::kFp8) {
-        const long x0 = __builtin_bit_cast(long, v2i{x[0], x[1]}), x1 = __builtin_bit_cast(long, v2i{x[2], x[3]});
-        const long w0 = __builtin_bit_cast(long, v2i{w[0][0], w[0][1]}), w1 = __builtin_bit_cast(long, v2i{w[0][2], w[0][3]});
-        a.sum = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(x0, w0, a.sum, 0, 0, 0);
-        a.sum = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(x1, w1, a.sum, 0, 0, 0);
+        const v8i x = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        const v8i w = {w0[0][0], w0[0][1], w0[0][2], w0[0][3], w1[0][0], w1[0][1], w1[0][2], w1[0][3]};
+        a.sum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, w, a.sum, 0, 0, 0, 0, 0, 0);
     } else {
         const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-        for (int p = 0; p < W::kPlanes; ++p) a.plane[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, w[p], first_of_sb ? zero : a.plane[p], 0, 0, 0);
+        for (int p = 0; p < W::kPlanes; ++p) a.plane[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0, w0[p], first_of_sb ? zero : a.plane[p], 0, 0, 0);
+#pragma unroll
+        for (int p = 0; p < W::kPlanes; ++p) a.plane[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1, w1[p], a.plane[p], 0, 0, 0);
     }
 }
 // |64 acc_h + acc_l| <= 256 * 127 * 2^12 < 2^28: exact in int32, then one rounding into fp32
@@ -530,25 +542,30 @@ template <class W> __device__ __forceinline__ void acc_fold(Acc<W> & a, const ty
 template <int NB, class W, int WAVES, bool GATEUP>
 __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
     constexpr int THREADS = 64 * WAVES, P = W::kPlanes;
-    constexpr int TPW = 8 / WAVES;           // row tiles per wave of a shared chunk
+    constexpr int TPW = (WAVES == 8 && W::kWideChunks ? 16 : 8) / WAVES;   // row tiles per wave of a shared chunk
     constexpr int PIECES = 8 * NB / WAVES;   // (slot, sub-block) pieces a wave decodes per super-block
     constexpr int SPW = 4 * NB / WAVES;      // operand slots per wave on a lone row tile
-    static_assert(kChunkTiles == 8 && (PIECES == 2 || PIECES == 4) && (SPW == 1 || SPW == 2), "wave arrangement");
+    // row tiles per chunk: twice the usual with eight waves where the format's accumulators leave the registers for two row
+    // tiles a wave (a chunk's weights are decoded once for twice the rows, and an expert with nine to sixteen row tiles is one
+    // item per unit group instead of a full chunk and a lone tile)
+    constexpr int CT = WAVES == 8 && W::kWideChunks ? 2 * kChunkTiles : kChunkTiles;
+    static_assert((PIECES == 2 || PIECES == 4) && (SPW == 1 || SPW == 2), "wave arrangement");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     v4i * bs = reinterpret_cast<v4i *>(lds);
     __shared__ __attribute__((aligned(16))) uint8_t s_tab[W::kTabBytes];
     __shared__ uint32_t s_lat[W::kLattice];
-    __shared__ int s_asg[kChunkTiles * 32];
-    __shared__ float s_scale[kChunkTiles * 32];
+    __shared__ int s_asg[(WAVES == 8 && W::kWideChunks ? 16 : 8) * 32];
+    __shared__ float s_scale[(WAVES == 8 && W::kWideChunks ? 16 : 8) * 32];
     // the experts' index (chunk and tile prefix sums, counts, offsets), copied once: every item looks its expert up, and a
     // binary search is a chain of dependent reads
     __shared__ int s_cbase[kPlanExperts + 1], s_tbase[kPlanExperts + 1], s_cnt[kPlanExperts + 1], s_off[kPlanExperts + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 31, g = lane >> 5;
     const int mg = wave & 3, nbw = wave >> 2;     // lone row tile: weight tile of the wave within the item, operand slot (SPW == 1)
+    const int * plan_chunks = (WAVES == 8 && W::kWideChunks) ? k.plan.chunk_base2 : k.plan.chunk_base;
     const bool cached = k.experts <= kPlanExperts;
     if (cached)
         for (int i = tid; i <= k.experts; i += THREADS) {
-            s_cbase[i] = k.plan.chunk_base[i];
+            s_cbase[i] = plan_chunks[i];
             s_tbase[i] = k.plan.tile_base[i];
             s_cnt[i] = i < k.experts ? k.counts[i] : 0;
             s_off[i] = k.offsets[i];
@@ -560,7 +577,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
     // early takes more items. The next ticket is fetched under the current item's work. The last block to leave
     // clears the counters for the next launch over these rows.
     __syncthreads();
-    const int * cbase = cached ? s_cbase : k.plan.chunk_base, * tbase = cached ? s_tbase : k.plan.tile_base;
+    const int * cbase = cached ? s_cbase : plan_chunks, * tbase = cached ? s_tbase : k.plan.tile_base;
     const int * cnts = cached ? s_cnt : k.counts, * offs = cached ? s_off : k.offsets;
     const int n_chunks = cbase[k.experts];
     const int groups = k.units / k.unit_group;                  // unit groups per chunk
@@ -588,26 +605,31 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
         const int live_units = GATEUP && is_shared ? min(max(k.shared_lim / 32 - u0, 0), k.unit_group) : k.unit_group;
         const int sb_full = !GATEUP && is_shared ? k.shared_lim / 256 : NSB;   // super-blocks of a live unit's products
         const int cnt = cnts[e], tiles_e = (cnt + 31) >> 5;
-        const int first_tile = local * kChunkTiles;                         // of this expert
-        const int live_tiles = min(kChunkTiles, tiles_e - first_tile);      // of this block
+        const int first_tile = local * CT;                                  // of this expert
+        const int live_tiles = min(CT, tiles_e - first_tile);               // of this block
         // A chunk of one row tile has nothing for the waves to share: every wave then takes the tile against 32 weight
         // rows of its own (of every slot it has), four units a pass, the chunk's items taking passes in turn.
         const bool lone = live_tiles == 1 && k.units % 4 == 0;
         if (lone && ug >= k.units / 4) continue;
         // the rows' assignments and scales are only read when the results are stored: their loads are issued here and land
         // in LDS after the products, so that nothing waits for them
-        static_assert(kChunkTiles * 32 == 256 && THREADS >= 256, "one row per thread");
-        int row_asg = -1;
-        float row_scale = 0.f;
-        if (tid < kChunkTiles * 32) {
-            const int idx = first_tile * 32 + tid;
-            if (tid < live_tiles * 32 && idx < cnt) {
-                row_asg = k.perm[offs[e] + idx];
-                row_scale = k.xs[int64_t(tile_base + first_tile) * 32 + tid];
+        constexpr int RPT = (CT * 32 + THREADS - 1) / THREADS;   // rows per thread
+        int row_asg[RPT];
+        float row_scale[RPT];
+#pragma unroll
+        for (int q = 0; q < RPT; ++q) {
+            const int i = tid + q * THREADS, idx = first_tile * 32 + i;
+            row_asg[q] = -1;
+            row_scale[q] = 0.f;
+            if (i < live_tiles * 32 && idx < cnt) {
+                row_asg[q] = k.perm[offs[e] + idx];
+                row_scale[q] = k.xs[int64_t(tile_base + first_tile) * 32 + i];
             }
         }
         auto rows_to_lds = [&]() {
-            if (tid < kChunkTiles * 32) { s_asg[tid] = row_asg; s_scale[tid] = row_scale; }
+#pragma unroll
+            for (int q = 0; q < RPT; ++q)
+                if (tid + q * THREADS < CT * 32) { s_asg[tid + q * THREADS] = row_asg[q]; s_scale[tid + q * THREADS] = row_scale[q]; }
             __syncthreads();
         };
         if (lone) for (int unit = ug; unit < k.units / 4; unit += groups) {
@@ -648,12 +670,13 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                 fetch1(min(sb + 1, sbe - 1), nxt);   // past the last one the same again, from the cache: no branch, the same loads in flight on every path
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int ib = 0; ib < 8; ++ib) {
+                for (int ib = 0; ib < 8; ib += 2) {
 #pragma unroll
                     for (int q = 0; q < SPW; ++q) {
-                        v4i w[P];
-                        W::planes(cur.code[q][ib], cur.rec[q], ib, g, s_tab, s_lat, w);
-                        acc_step(acc[q], cur.a[ib], w, ib == 0);
+                        v4i w0[P], w1[P];
+                        W::planes(cur.code[q][ib], cur.rec[q], ib, g, s_tab, s_lat, w0);
+                        W::planes(cur.code[q][ib + 1], cur.rec[q], ib + 1, g, s_tab, s_lat, w1);
+                        acc_step2(acc[q], cur.a[ib], cur.a[ib + 1], w0, w1, ib == 0);
                     }
                 }
 #pragma unroll
@@ -860,16 +883,15 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                         if (jp == 3) { __builtin_amdgcn_sched_barrier(0); fetch(sb, 2); __builtin_amdgcn_sched_barrier(0); }
                         load_a((jp + kSlots - 1) % kSlots, sb * 4 + jp + kSlots - 1);
 #pragma unroll
-                        for (int h = 0; h < 2; ++h) {
-                            const int ib = 2 * jp + h;
+                        for (int b = 0; b < NB; ++b) {
+                            v4i w0[P], w1[P];
 #pragma unroll
-                            for (int b = 0; b < NB; ++b) {
-                                v4i w[P];
-#pragma unroll
-                                for (int p = 0; p < P; ++p) w[p] = bs[(((buf * NB + b) * P + p) * 8 + ib) * 64 + lane];
-#pragma unroll
-                                for (int t = 0; t < MT; ++t) acc_step(acc[t][b], a_reg[jp % kSlots][t][h], w, ib == 0);
+                            for (int p = 0; p < P; ++p) {
+                                w0[p] = bs[(((buf * NB + b) * P + p) * 8 + 2 * jp) * 64 + lane];
+                                w1[p] = bs[(((buf * NB + b) * P + p) * 8 + 2 * jp + 1) * 64 + lane];
                             }
+#pragma unroll
+                            for (int t = 0; t < MT; ++t) acc_step2(acc[t][b], a_reg[jp % kSlots][t][0], a_reg[jp % kSlots][t][1], w0, w1, jp == 0);
                         }
                     }
 #pragma unroll
@@ -908,6 +930,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
         if constexpr (TPW == 1) {
             if (my_tiles) body(std::integral_constant<int, 1>{}); else body(std::integral_constant<int, 0>{});
         } else {
+            static_assert(TPW == 2, "row tiles per wave");
             switch (my_tiles) {
                 case 0: body(std::integral_constant<int, 0>{}); break;
                 case 1: body(std::integral_constant<int, 1>{}); break;
@@ -941,7 +964,7 @@ int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int 
     return 0;
 }
 
-int64_t grouped_scale_words(int64_t assignments, int experts) { return grouped_row_tiles(assignments, experts) * 32 + 2 * (int64_t(experts) + 1) + kPlanCounters; }
+int64_t grouped_scale_words(int64_t assignments, int experts) { return grouped_row_tiles(assignments, experts) * 32 + 3 * (int64_t(experts) + 1) + kPlanCounters; }
 
 template <int XT, bool F8>
 static void group_rows_launch(const void * x, int cols, const int * counts, const int * offsets, const int * perm, int experts, int64_t tiles, int xdiv, int8_t * q,
@@ -965,7 +988,7 @@ int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const in
                               int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8) {
     const int64_t tiles = grouped_row_tiles(assignments, experts);
     const Plan plan = plan_at(scale, tiles * 32, experts);
-    plan_k<<<1, 64, 0, s>>>(counts, experts, const_cast<int *>(plan.tile_base), const_cast<int *>(plan.chunk_base), plan.counters);
+    plan_k<<<1, 64, 0, s>>>(counts, experts, plan);
 #define TQMOE_GROUP(XT) (f8 ? group_rows_launch<XT, true>(x, cols, counts, offsets, perm, experts, tiles, xdiv, q, scale, plan, s) \
                             : group_rows_launch<XT, false>(x, cols, counts, offsets, perm, experts, tiles, xdiv, q, scale, plan, s))
     switch (xtype) {
@@ -981,7 +1004,7 @@ int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, co
                                int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s) {
     const int64_t tiles = grouped_row_tiles(assignments, experts);
     const Plan plan = plan_at(scale, tiles * 32, experts);
-    plan_k<<<1, 64, 0, s>>>(counts, experts, const_cast<int *>(plan.tile_base), const_cast<int *>(plan.chunk_base), plan.counters);
+    plan_k<<<1, 64, 0, s>>>(counts, experts, plan);
     gather_rows_i8_k<<<unsigned(tiles), 256, 0, s>>>(rq, rs, cols, counts, offsets, perm, experts, xdiv, q, scale, plan);
     return 0;
 }

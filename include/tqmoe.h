@@ -233,9 +233,10 @@ int32_t tqmoe_combine_strided(const float * routed, int32_t slots, const float *
                               int32_t hidden, int32_t topk, int32_t n, void * stream, tqmoe_error * err);
 
 /* ------------------------------------------------------------------------------------------ prefill products
- * Grouped int8 x int8 -> int32 products on the matrix cores over the dispatch lists: IQ4_XS, IQ3_S and Q4_K banks, with
- * exact weights (the reference's int8 path covers its u4h formats the same way, quant_u4h.inc:783-789, 839-845, and its
- * MMQ path the IQ formats, mmq_experts.cu:193-196). Rows a multiple of 32, columns of 256.
+ * Grouped int8 x int8 -> int32 products on the matrix cores over the dispatch lists: IQ4_XS, IQ4_NL, IQ3_S, IQ3_XXS,
+ * IQ2_XXS, IQ2_XS, IQ2_S, IQ1_S and Q4_K banks, with exact weights (the reference's int8 path covers its u4h formats the same way,
+ * quant_u4h.inc:783-789, 839-845, and its MMQ path the IQ formats, mmq_experts.cu:193-196). Rows a multiple of 32,
+ * columns of 256.
  * counts / offsets / perm are tqmoe_dispatch's lists over ids [n][slots] with `experts` = the banks' experts.
  *
  * tqmoe_quant_rows_i8: per input row q = rint(x * 127 / amax), scale = amax / 127 (0 for a zero row): the per-token mode

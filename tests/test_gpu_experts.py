@@ -135,7 +135,10 @@ def check_layer(out, ids, w, want, want_ids, want_w, clear):
     assert np.array_equal(ids, want_ids)
     assert np.abs(w - want_w).max() < 3e-6
     mx, rel = synth.errors(out, want)
-    assert mx < MAX_ABS and rel < REL_RMS, (mx, rel)
+    # max-abs 1e-2 where the outputs are of order one, as the configurations' are; relative to the largest value beyond that
+    # (banks of random valid blocks can give larger outputs, and on the 8-bit grouped products one act value that rounds the
+    # other way is a step of 1 / 127 of its row's largest)
+    assert mx < MAX_ABS * max(1.0, float(np.abs(want).max())) and rel < REL_RMS, (mx, rel, float(np.abs(want).max()))
     return mx, rel
 
 

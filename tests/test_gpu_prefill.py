@@ -73,10 +73,10 @@ def grouped_setup(tq, oracle, seed, experts, ff, hidden, n, k, shared, wtype=Non
     banks = experts + (1 if shared else 0)
     raws, decs, devb = [], [], []
     for rows, cols in ((ff, hidden), (ff, hidden), (hidden, ff)):
-        w = (rng.standard_normal((banks * rows, cols)) * 0.02).astype(np.float32)
-        raw = oracle.quantize(wtype, w)
+        raw = synth.bank_blocks(wtype, banks * rows, cols, rng)     # encoded N(0, 0.02) weights, or random valid blocks of that size
         raws.append(raw)
-        dec = oracle.dequantize_nvfp4_widened(raw, w.size) if widened else oracle.dequantize(wtype, raw, w.size)
+        size = banks * rows * cols
+        dec = oracle.dequantize_nvfp4_widened(raw, size) if widened else oracle.dequantize(wtype, raw, size)
         decs.append(dec.reshape(banks, rows, cols).astype(np.float64))
         devb.append(tq.ExpertBank(wtype, raw, banks, rows, cols))
     slots = k + (1 if shared else 0)
@@ -114,7 +114,10 @@ def test_quant_rows_fp8_bit_exact(tq, oracle, kind):
         assert s[r] == np.float32(ws)
 
 
-@pytest.mark.parametrize("wtype", ["IQ4_XS", "IQ3_S", "Q4_K", "NVFP4G"])
+PLANE_FORMATS = ["IQ4_XS", "IQ3_S", "Q4_K", "NVFP4G", "IQ3_XXS", "IQ2_XXS", "IQ2_XS", "IQ2_S", "IQ1_S", "IQ4_NL"]
+
+
+@pytest.mark.parametrize("wtype", PLANE_FORMATS)
 @pytest.mark.parametrize("n,shared_ff", [(3, 0), (70, 256), (300, 512), (900, 0)])
 def test_grouped_products_against_float64(tq, oracle, n, shared_ff, wtype):
     """gate/up + SwiGLU and down products over the dispatch lists against float64 on the decoded weights and the
@@ -202,12 +205,12 @@ def test_grouped_products_refuse_the_wrong_operand_type(tq, oracle):
     counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), 2)
     x = torch.randn(4, 256, device="cuda", dtype=torch.float16)
     xq, xs = tq.group_rows_i8(x, (counts, offsets, perm), 4, 1)
-    for bank, fn in ((mk(oracle.NVFP4G), tq.expert_gemm_i8), (mk(oracle.IQ4_XS), tq.expert_gemm_fp8), (mk(oracle.IQ4_NL), tq.expert_gemm_i8)):
+    for bank, fn in ((mk(oracle.NVFP4G), tq.expert_gemm_i8), (mk(oracle.IQ4_XS), tq.expert_gemm_fp8), (mk(oracle.Q8_0), tq.expert_gemm_i8)):
         with pytest.raises(tq.TqmoeError):
             fn(bank, xq, xs, (counts, offsets, perm), 4, 1, 1)
 
 
-@pytest.mark.parametrize("wtype", ["IQ4_XS", "IQ3_S", "Q4_K", "NVFP4G"])
+@pytest.mark.parametrize("wtype", PLANE_FORMATS)
 @pytest.mark.parametrize("rows,experts", [(96, 5), (160, 5), (128, 5), (256, 5), (64, 1100)])
 def test_gemm_i8_bank_shapes(tq, oracle, rows, experts, wtype):
     """tqmoe_expert_gemm_i8 over banks whose row count changes the kernel's arrangement (one or two operand slots per block,
@@ -217,9 +220,9 @@ def test_gemm_i8_bank_shapes(tq, oracle, rows, experts, wtype):
     fp8 = wtype == "NVFP4G"
     wtype = getattr(oracle, wtype)
     rng = np.random.default_rng(rows + experts)
-    w = (rng.standard_normal((experts * rows, cols)) * 0.02).astype(np.float32)
-    raw = oracle.quantize(wtype, w)
-    dec = (oracle.dequantize_nvfp4_widened(raw, w.size) if fp8 else oracle.dequantize(wtype, raw, w.size)).reshape(experts, rows, cols).astype(np.float64)
+    raw = synth.bank_blocks(wtype, experts * rows, cols, rng)
+    size = experts * rows * cols
+    dec = (oracle.dequantize_nvfp4_widened(raw, size) if fp8 else oracle.dequantize(wtype, raw, size)).reshape(experts, rows, cols).astype(np.float64)
     bank = tq.ExpertBank(wtype, raw, experts, rows, cols)
     ids = rng.integers(0, experts, size=(n, k)).astype(np.int32)
     ids[: n // 2, 0] = 2
@@ -311,13 +314,14 @@ def test_layer_grouped_small_shapes(tq, oracle, n):
     check_layer(*run_layer(tq, oracle, cfg, n, seed=60 + n))
 
 
-@pytest.mark.parametrize("name,fmt,path,mode", [("c1", "Q4_K", "grouped_i8", 5), ("c4", "IQ3_S", "grouped_i8", 5), ("c5", "NVFP4G", "grouped_fp8", 2)])
+@pytest.mark.parametrize("name,fmt,path,mode", [("c1", "Q4_K", "grouped_i8", 5), ("c4", "IQ3_S", "grouped_i8", 5), ("c5", "NVFP4G", "grouped_fp8", 2),
+                                                ("c4", "IQ3_XXS", "grouped_i8", 5), ("c4", "IQ2_XXS", "grouped_i8", 5), ("c4", "IQ2_XS", "grouped_i8", 5),
+                                                ("c4", "IQ2_S", "grouped_i8", 5), ("c4", "IQ1_S", "grouped_i8", 5), ("c4", "IQ4_NL", "grouped_i8", 5)])
 @pytest.mark.parametrize("n", [64, 300])
 def test_layer_grouped_other_formats(tq, oracle, name, fmt, path, mode, n):
-    """Q4_K and IQ3_S banks on the int8 products, NVFP4G banks on the fp8 products, against the oracle with the same
+    """Q4_K and the lattice formats on the int8 products, NVFP4G banks on the fp8 products, against the oracle with the same
     declared operand quantisers (the distance to the fp32-activation oracle printed beside it)."""
-    base = synth.CONFIGS[name]
-    assert base["wtype"] == getattr(oracle, fmt)
+    base = dict(synth.CONFIGS[name], wtype=getattr(oracle, fmt))
     cfg = synth.small(base, 768, 512, 10, 3)
     check_layer(*run_layer(tq, oracle, cfg, n, seed=160 + n, modes=(mode, 0), path=path))
 

@@ -335,8 +335,9 @@ __device__ const int8_t kIq4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -
 // 16 weights {8g..8g+7} and {16+8g..16+8g+7}: Src are its base pointers, Code what it loads per sub-block, Rec what
 // decoding needs of the sub-block's super-block, DRec what the fold needs of it (the lane's row, any g).
 // planes() turns a Code into kPlanes operand registers; tables() fills the lookup tables (and the lattice) in LDS.
-struct WIq4xs {
-    static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)   // tile-major codes (512 B per sub-block of a tile), 8-byte records (256 B per super-block of a tile)
+struct WIq4xs {   // tile-major codes (512 B per sub-block of a tile), 8-byte records (256 B per super-block of a tile)
+    static constexpr bool kFoldSub = false;     // one scale per 32 weights: every sub-block's product is folded on its own
+    static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)
     static constexpr int kPlanes = 2, kTabBytes = 64 * 32, kLattice = 1;
     static constexpr bool kFp8 = false, kMin = false, kRowMul = false;
     struct Code { uint2 c; };
@@ -363,8 +364,9 @@ struct WIq4xs {
     static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
 };
 
-struct WQ4k {
-    static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)   // row-major: 16 code bytes per sub-block, a 16-byte record (d | dmin << 16, twelve bytes of 6-bit scales and minimums) per super-block
+struct WQ4k {   // row-major: 16 code bytes per sub-block, a 16-byte record (d | dmin << 16, twelve bytes of 6-bit scales and minimums) per super-block
+    static constexpr bool kFoldSub = false;     // one scale per 32 weights: every sub-block's product is folded on its own
+    static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)
     static constexpr int kPlanes = 3, kTabBytes = 64 * 32, kLattice = 1;
     static constexpr bool kFp8 = false, kMin = true, kRowMul = false;
     struct Code { uint2 c; };
@@ -396,8 +398,9 @@ struct WQ4k {
     static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
 };
 
-struct WIq3s {
-    static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)   // row-major: 12 code bytes per sub-block (8 lattice indices, 32 sign bits), a 16-byte record per super-block
+struct WIq3s {   // row-major: 12 code bytes per sub-block (8 lattice indices, 32 sign bits), a 16-byte record per super-block
+    static constexpr bool kFoldSub = false;     // one scale per 32 weights: every sub-block's product is folded on its own
+    static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)
     static constexpr int kPlanes = 2, kTabBytes = 16 * 32, kLattice = 512;
     static constexpr bool kFp8 = false, kMin = false, kRowMul = false;
     struct Code { uint32_t qs0, qs1, sg; };
@@ -443,8 +446,204 @@ struct WIq3s {
     static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
 };
 
-struct WNvfp4 {
-    static constexpr bool kWideChunks = true;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)   // row-major: 16 code bytes per sub-block, one E4M3 scale byte per 16 weights, one fp32 global per row
+// ---- the other lattice formats of the reference's MMQ list: magnitudes of 4 or 8 weights per lattice point (LDS copy of the
+// lattice), a sign bit per weight, a 4-bit scale s with multiplier 2 s + 1 per sub-block or per 16 weights, one fp16 d per
+// super-block (first dword of a 16-byte record). p = (2 s + 1) * (+-magnitude) through 16-entry tables per scale:
+// code = sign << 3 | level index of the magnitude (magnitude >> SH). value = d * p / 4 (IQ3_XXS) or d * p / 8 (IQ2).
+template <int SH> __device__ __forceinline__ void lattice_planes(uint32_t mag, uint32_t sign4, uint4 th, uint4 tl, v4i * p, int q) {
+    const uint32_t i3 = (mag >> SH) & 0x07070707u, sel = (spread4(sign4) << 2) | 0x03020100u;
+    p[0][q] = pick16(th, i3, sel);
+    p[1][q] = pick16(tl, i3, sel);
+}
+template <class LEVEL> __device__ __forceinline__ void lattice_tables(uint8_t * tab, int tid, int threads, LEVEL level) {
+    for (int i = tid; i < 16 * 16; i += threads) {
+        const int mag = (1 + 2 * (i >> 4)) * level(i & 7);
+        split_planes((i & 8) ? -mag : mag, tab[(i >> 4) * 32 + (i & 15)], tab[(i >> 4) * 32 + 16 + (i & 15)]);
+    }
+}
+struct WLatticeBase {   // row-major, a 16-byte record per super-block whose first 16 bits are d
+    static constexpr int kPlanes = 2, kTabBytes = 16 * 32;
+    static constexpr bool kFp8 = false, kMin = false, kRowMul = false, kWideChunks = false, kFoldSub = false;
+    typedef uint32_t Rec;    // unused by the decode (the scales sit in the code bytes)
+    typedef uint32_t DRec;
+    struct Src { const uint8_t * codes, * aux; };
+    template <int CB> static __device__ __forceinline__ Src src_of(const BankView & b, int e, int wtile, int n) {
+        const int S = b.cols / 32;
+        const int64_t row = int64_t(e) * b.rows + wtile * 32 + n;
+        return Src{b.codes + row * S * CB, b.aux + row * (S / 8) * 16};
+    }
+    static __device__ __forceinline__ Rec rec(const Src &, int) { return 0; }
+    static __device__ __forceinline__ DRec drec(const Src & s, int sb) { return *reinterpret_cast<const uint32_t *>(s.aux + int64_t(sb) * 16); }
+    static __device__ __forceinline__ float dmin(const DRec &) { return 0.f; }
+    static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
+};
+
+struct WIq3xxs : WLatticeBase {   // 12 code bytes: 8 lattice indices (4 weights each), a word of 4 x 7 sign bits + the scale
+    static constexpr int kLattice = 256;
+    struct Code { uint32_t qs0, qs1, word; };
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t * lat, int tid, int threads) {
+        lattice_tables(tab, tid, threads, [](int l) { return int(iq3xxs_level(uint32_t(l))); });
+        for (int i = tid; i < 256; i += threads) lat[i] = d_iq3xxs_grid.v[i];
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int) { return src_of<12>(b, e, wtile, n); }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) {
+        const uint32_t * c = reinterpret_cast<const uint32_t *>(s.codes + int64_t(sub) * 12);
+        return Code{c[0], c[1], c[2]};
+    }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int g, const uint8_t * tab, const uint32_t * lat, v4i * p) {
+        const uint4 * t = reinterpret_cast<const uint4 *>(tab + (c.word >> 28) * 32);
+        const uint4 th = t[0], tl = t[1];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {   // operand dword q = the group of four weights w
+            const int w = 2 * g + (q >> 1) + 4 * (q & 1);
+            const uint32_t mag = lat[((w < 4 ? c.qs0 : c.qs1) >> (8 * (w & 3))) & 0xFFu];
+            lattice_planes<3>(mag, iq3xxs_signs(c.word, w >> 1) >> (4 * (w & 1)), th, tl, p, q);
+        }
+    }
+    static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(uint16_t(r & 0xFFFFu)) * 0.25f; }
+};
+
+__device__ __forceinline__ int iq2_level(int l) { return l == 0 ? 8 : l == 1 ? 25 : l == 2 ? 43 : 0; }
+
+struct WIq2xxs : WLatticeBase {   // 8 code bytes: 4 lattice indices (8 weights each), a word of 4 x 7 sign bits + the scale
+    static constexpr int kLattice = 512;
+    struct Code { uint2 c; };
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t * lat, int tid, int threads) {
+        lattice_tables(tab, tid, threads, iq2_level);
+        for (int i = tid; i < 512; i += threads) lat[i] = d_iq2xxs_grid.v[i];
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int) { return src_of<8>(b, e, wtile, n); }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) { return Code{*reinterpret_cast<const uint2 *>(s.codes + int64_t(sub) * 8)}; }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int g, const uint8_t * tab, const uint32_t * lat, v4i * p) {
+        const uint4 * t = reinterpret_cast<const uint4 *>(tab + (c.c.y >> 28) * 32);
+        const uint4 th = t[0], tl = t[1];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int w = 2 * g + (q >> 1) + 4 * (q & 1), l = w >> 1, half = w & 1;   // group of eight weights, its half
+            const uint32_t mag = lat[2 * ((c.c.x >> (8 * l)) & 0xFFu) + half];
+            lattice_planes<4>(mag, iq3xxs_signs(c.c.y, l) >> (4 * half), th, tl, p, q);
+        }
+    }
+    static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(uint16_t(r & 0xFFFFu)) * 0.125f; }
+};
+
+struct WIq2xs : WLatticeBase {   // 12 code bytes: 4 x (9-bit lattice index | 7 sign bits << 9), a byte of two scales (a nibble per 16 weights)
+    static constexpr int kLattice = 1024;
+    struct Code { uint32_t q0, q1, sc; };
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t * lat, int tid, int threads) {
+        lattice_tables(tab, tid, threads, iq2_level);
+        for (int i = tid; i < 1024; i += threads) lat[i] = d_iq2xs_grid.v[i];
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int) { return src_of<12>(b, e, wtile, n); }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) {
+        const uint32_t * c = reinterpret_cast<const uint32_t *>(s.codes + int64_t(sub) * 12);
+        return Code{c[0], c[1], c[2]};
+    }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int g, const uint8_t * tab, const uint32_t * lat, v4i * p) {
+        const uint4 * t0 = reinterpret_cast<const uint4 *>(tab + (c.sc & 15u) * 32), * t1 = reinterpret_cast<const uint4 *>(tab + ((c.sc >> 4) & 15u) * 32);
+        const uint4 th[2] = {t0[0], t1[0]}, tl[2] = {t0[1], t1[1]};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {   // odd operand dwords hold weights 16..31: the second scale
+            const int w = 2 * g + (q >> 1) + 4 * (q & 1), l = w >> 1, half = w & 1;
+            const uint32_t qq = ((l < 2 ? c.q0 : c.q1) >> (16 * (l & 1))) & 0xFFFFu;
+            const uint32_t mag = lat[2 * (qq & 511u) + half];
+            lattice_planes<4>(mag, signs8(qq >> 9) >> (4 * half), th[q & 1], tl[q & 1], p, q);
+        }
+    }
+    static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(uint16_t(r & 0xFFFFu)) * 0.125f; }
+};
+
+struct WIq2s : WLatticeBase {   // 12 code bytes: 4 low index bytes, 4 sign bytes, a byte of high index bits, a byte of two scales
+    static constexpr int kLattice = 2048;
+    struct Code { uint32_t low, sg, hs; };
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t * lat, int tid, int threads) {
+        lattice_tables(tab, tid, threads, iq2_level);
+        for (int i = tid; i < 2048; i += threads) lat[i] = d_iq2s_grid.v[i];
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int) { return src_of<12>(b, e, wtile, n); }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) {
+        const uint32_t * c = reinterpret_cast<const uint32_t *>(s.codes + int64_t(sub) * 12);
+        return Code{c[0], c[1], c[2]};
+    }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int g, const uint8_t * tab, const uint32_t * lat, v4i * p) {
+        const uint32_t qh = c.hs & 0xFFu, sc = (c.hs >> 8) & 0xFFu;
+        const uint4 * t0 = reinterpret_cast<const uint4 *>(tab + (sc & 15u) * 32), * t1 = reinterpret_cast<const uint4 *>(tab + (sc >> 4) * 32);
+        const uint4 th[2] = {t0[0], t1[0]}, tl[2] = {t0[1], t1[1]};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int w = 2 * g + (q >> 1) + 4 * (q & 1), l = w >> 1, half = w & 1;
+            const uint32_t mag = lat[2 * iq2s_index(c.low, qh, l) + half];
+            lattice_planes<4>(mag, ((c.sg >> (8 * l)) & 0xFFu) >> (4 * half), th[q & 1], tl[q & 1], p, q);
+        }
+    }
+    static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(uint16_t(r & 0xFFFFu)) * 0.125f; }
+};
+
+struct WIq1s : WLatticeBase {   // 8 code bytes: 4 low index bytes (8 weights each), 16 bits of 4 x 3 high index bits, a 3-bit scale, the delta's sign
+    // value = d * (2 s + 1) * (g +- 1/8), g in {-1, 0, 1}: p = (2 s + 1) * (8 g +- 1), |p| <= 135, value = d * p / 8; a table per
+    // (scale, delta sign), code = the lattice byte's low two bits (0, 1, 3 for g = 0, 1, -1)
+    static constexpr int kLattice = 4096;
+    struct Code { uint2 c; };
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t * lat, int tid, int threads) {
+        for (int i = tid; i < 16 * 16; i += threads) {
+            const int t = i >> 4, c = i & 15, gval = c == 1 ? 1 : c == 3 ? -1 : 0;
+            split_planes((2 * (t & 7) + 1) * (8 * gval + ((t & 8) ? -1 : 1)), tab[t * 32 + c], tab[t * 32 + 16 + c]);
+        }
+        for (int i = tid; i < 4096; i += threads) lat[i] = d_iq1s_grid.v[i];
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int) { return src_of<8>(b, e, wtile, n); }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) { return Code{*reinterpret_cast<const uint2 *>(s.codes + int64_t(sub) * 8)}; }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int g, const uint8_t * tab, const uint32_t * lat, v4i * p) {
+        const uint4 * t = reinterpret_cast<const uint4 *>(tab + (((c.c.y >> 12) & 7u) | ((c.c.y >> 12) & 8u)) * 32);
+        const uint4 th = t[0], tl = t[1];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int w = 2 * g + (q >> 1) + 4 * (q & 1), l = w >> 1, half = w & 1;
+            const uint32_t idx = ((c.c.x >> (8 * l)) & 0xFFu) | (((c.c.y >> (3 * l)) & 7u) << 8);
+            const uint32_t i3 = lat[2 * idx + half] & 0x03030303u;
+            p[0][q] = pick16(th, i3, 0x03020100u);
+            p[1][q] = pick16(tl, i3, 0x03020100u);
+        }
+    }
+    static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(uint16_t(r & 0xFFFFu)) * 0.125f; }
+};
+
+struct WIq4nl {   // row-major: 16 code bytes per sub-block (nibbles as IQ4_XS), one fp16 scale per 32 weights (eight per 256 in the aux plane)
+    static constexpr int kPlanes = 1, kTabBytes = 16, kLattice = 1;
+    static constexpr bool kFp8 = false, kRowMul = false, kWideChunks = false;
+    static constexpr bool kFoldSub = true;
+    struct Code { uint2 c; };
+    typedef uint32_t Rec;    // unused by the decode
+    typedef uint4 DRec;      // the eight scales of the row's super-block
+    struct Src { const uint8_t * codes, * aux; };
+    static __device__ __forceinline__ void tables(uint8_t *, uint32_t *, int, int) {}
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int g) {
+        const int S = b.cols / 32;
+        const int64_t row = int64_t(e) * b.rows + wtile * 32 + n;
+        return Src{b.codes + row * S * 16 + g * 8, b.aux + row * S * 2};
+    }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) { return Code{*reinterpret_cast<const uint2 *>(s.codes + int64_t(sub) * 16)}; }
+    static __device__ __forceinline__ Rec rec(const Src &, int) { return 0; }
+    static __device__ __forceinline__ DRec drec(const Src & s, int sb) { return *reinterpret_cast<const uint4 *>(s.aux + int64_t(sb) * 16); }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int, const uint8_t *, const uint32_t *, v4i * p) {
+        uint32_t lo, hi;
+        lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(c.c.x, lo, hi);
+        p[0][0] = int(lo); p[0][1] = int(hi);
+        lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(c.c.y, lo, hi);
+        p[0][2] = int(lo); p[0][3] = int(hi);
+    }
+    static __device__ __forceinline__ float d_sub(const DRec & r, int ib) {   // scale of sub-block ib of the super-block
+        const uint32_t w = (ib >> 1) == 0 ? r.x : (ib >> 1) == 1 ? r.y : (ib >> 1) == 2 ? r.z : r.w;
+        return half_bits_to_float(uint16_t((w >> (16 * (ib & 1))) & 0xFFFFu));
+    }
+    static __device__ __forceinline__ float d(const DRec &) { return 1.f; }
+    static __device__ __forceinline__ float dmin(const DRec &) { return 0.f; }
+    static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
+};
+
+struct WNvfp4 {   // row-major: 16 code bytes per sub-block, one E4M3 scale byte per 16 weights, one fp32 global per row
+    static constexpr bool kFoldSub = false;     // one scale per 32 weights: every sub-block's product is folded on its own
+    static constexpr bool kWideChunks = true;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)
     static constexpr int kPlanes = 1, kTabBytes = 256 * 16, kLattice = 1;
     static constexpr bool kFp8 = true, kRowMul = true;
     struct Code { uint2 c; };
@@ -495,7 +694,7 @@ struct WNvfp4 {
 
 // one sub-block's products of a row tile with the planes of a weight tile
 template <class W> struct Acc {
-    v16i plane[W::kFp8 ? 1 : W::kPlanes];   // int32 sums of the current super-block (unused by the fp8 path)
+    v16i plane[W::kFp8 || W::kFoldSub ? 1 : W::kPlanes];   // int32 sums of the current super-block (unused by the fp8 path and by per-sub-block folds)
     v16f sum;                               // fp32 result so far
 };
 template <class W> __device__ __forceinline__ void acc_clear(Acc<W> & a) {
@@ -506,11 +705,19 @@ template <class W> __device__ __forceinline__ void acc_clear(Acc<W> & a) {
 // v_mfma_i32_32x32x32_i8 per sub-block and plane. fp8: one v_mfma_f32_32x32x64_f8f6f4 (both operands E4M3, no block
 // scales) for the pair: twice the rate of the 32x32x16 fp8 instruction on this part.
 typedef int v8i __attribute__((ext_vector_type(8)));
-template <class W> __device__ __forceinline__ void acc_step2(Acc<W> & a, v4i x0, v4i x1, const v4i * w0, const v4i * w1, bool first_of_sb) {
+template <class W> __device__ __forceinline__ void acc_step2(Acc<W> & a, v4i x0, v4i x1, const v4i * w0, const v4i * w1, bool first_of_sb, const typename W::DRec & r,
+                                                            int ib0) {
     if constexpr (W::kFp8) {
         const v8i x = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
         const v8i w = {w0[0][0], w0[0][1], w0[0][2], w0[0][3], w1[0][0], w1[0][1], w1[0][2], w1[0][3]};
         a.sum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, w, a.sum, 0, 0, 0, 0, 0, 0);
+    } else if constexpr (W::kFoldSub) {   // a scale per sub-block: each sub-block's integer sums (exact) go into the fp32 result at once
+        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        const v16i s0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0, w0[0], zero, 0, 0, 0);
+        const v16i s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1, w1[0], zero, 0, 0, 0);
+        const float d0 = W::d_sub(r, ib0), d1 = W::d_sub(r, ib0 + 1);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) a.sum[i] = __fmaf_rn(float(s1[i]), d1, __fmaf_rn(float(s0[i]), d0, a.sum[i]));
     } else {
         const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -521,7 +728,7 @@ template <class W> __device__ __forceinline__ void acc_step2(Acc<W> & a, v4i x0,
 }
 // |64 acc_h + acc_l| <= 256 * 127 * 2^12 < 2^28: exact in int32, then one rounding into fp32
 template <class W> __device__ __forceinline__ void acc_fold(Acc<W> & a, const typename W::DRec & r) {
-    if constexpr (!W::kFp8) {
+    if constexpr (!W::kFp8 && !W::kFoldSub) {
         const float d = W::d(r);
 #pragma unroll
         for (int i = 0; i < 16; ++i) a.sum[i] = fold_sb(a.sum[i], a.plane[0][i], a.plane[1][i], d);
@@ -676,7 +883,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                         v4i w0[P], w1[P];
                         W::planes(cur.code[q][ib], cur.rec[q], ib, g, s_tab, s_lat, w0);
                         W::planes(cur.code[q][ib + 1], cur.rec[q], ib + 1, g, s_tab, s_lat, w1);
-                        acc_step2(acc[q], cur.a[ib], cur.a[ib + 1], w0, w1, ib == 0);
+                        acc_step2(acc[q], cur.a[ib], cur.a[ib + 1], w0, w1, ib == 0, cur.drec[q], ib);
                     }
                 }
 #pragma unroll
@@ -891,7 +1098,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                                 w1[p] = bs[(((buf * NB + b) * P + p) * 8 + 2 * jp + 1) * 64 + lane];
                             }
 #pragma unroll
-                            for (int t = 0; t < MT; ++t) acc_step2(acc[t][b], a_reg[jp % kSlots][t][0], a_reg[jp % kSlots][t][1], w0, w1, jp == 0);
+                            for (int t = 0; t < MT; ++t) acc_step2(acc[t][b], a_reg[jp % kSlots][t][0], a_reg[jp % kSlots][t][1], w0, w1, jp == 0, d_rec[b], 2 * jp);
                         }
                     }
 #pragma unroll
@@ -1009,8 +1216,11 @@ int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, co
     return 0;
 }
 
-// bank formats with a plane GEMM: int8 operands (IQ4_XS, IQ3_S, Q4_K) or E4M3 operands (NVFP4G)
-bool plane_gemm_has(uint32_t type) { return type == TQMOE_IQ4_XS || type == TQMOE_IQ3_S || type == TQMOE_Q4_K || type == TQMOE_NVFP4G; }
+// bank formats with a plane GEMM: int8 operands (IQ4_XS, IQ4_NL, IQ3_S, IQ3_XXS, IQ2_XXS, IQ2_XS, IQ2_S, IQ1_S, Q4_K) or E4M3 operands (NVFP4G)
+bool plane_gemm_has(uint32_t type) {
+    return type == TQMOE_IQ4_XS || type == TQMOE_IQ3_S || type == TQMOE_Q4_K || type == TQMOE_NVFP4G || type == TQMOE_IQ3_XXS || type == TQMOE_IQ2_XXS ||
+           type == TQMOE_IQ2_XS || type == TQMOE_IQ2_S || type == TQMOE_IQ1_S || type == TQMOE_IQ4_NL;
+}
 bool plane_gemm_is_fp8(uint32_t type) { return type == TQMOE_NVFP4G; }
 
 // Two operand slots run on eight waves (a row tile each). The four-wave arrangement of the same kernel (two row tiles a wave,
@@ -1048,6 +1258,12 @@ int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const i
         case TQMOE_IQ3_S: plane_gemm_launch<WIq3s>(nb, gateup != 0, k, blocks, s); break;
         case TQMOE_Q4_K: plane_gemm_launch<WQ4k>(nb, gateup != 0, k, blocks, s); break;
         case TQMOE_NVFP4G: plane_gemm_launch<WNvfp4>(nb, gateup != 0, k, blocks, s); break;
+        case TQMOE_IQ3_XXS: plane_gemm_launch<WIq3xxs>(nb, gateup != 0, k, blocks, s); break;
+        case TQMOE_IQ2_XXS: plane_gemm_launch<WIq2xxs>(nb, gateup != 0, k, blocks, s); break;
+        case TQMOE_IQ2_XS: plane_gemm_launch<WIq2xs>(nb, gateup != 0, k, blocks, s); break;
+        case TQMOE_IQ2_S: plane_gemm_launch<WIq2s>(nb, gateup != 0, k, blocks, s); break;
+        case TQMOE_IQ1_S: plane_gemm_launch<WIq1s>(nb, gateup != 0, k, blocks, s); break;
+        case TQMOE_IQ4_NL: plane_gemm_launch<WIq4nl>(nb, gateup != 0, k, blocks, s); break;
         default: return -1;
     }
     return 0;

@@ -44,16 +44,23 @@ __global__ __launch_bounds__(256) void combine_k(const RT * __restrict__ routed,
     const int64_t t = i / h;
     const int j = int(i % h);
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s = 0; s < k; ++s) {
-        const float w = weights[t * k + s];
-        const float4 v = load4(routed + (t * slots + s) * h + j);
-        sum.x += w * v.x; sum.y += w * v.y; sum.z += w * v.z; sum.w += w * v.w;
+    // the rows and weights of up to kBatch slots are loaded before the first of them is added: one trip to memory per batch
+    // instead of one per slot (the sum keeps the slot order)
+    constexpr int kBatch = 12;
+    float sw = 0.f;
+    float4 sv = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (shared) { sw = shared_w[t]; sv = load4(shared + t * shared_ld + j); }
+    for (int s0 = 0; s0 < k; s0 += kBatch) {
+        float w[kBatch];
+        float4 v[kBatch];
+#pragma unroll
+        for (int q = 0; q < kBatch; ++q)
+            if (s0 + q < k) { w[q] = weights[t * k + s0 + q]; v[q] = load4(routed + (t * slots + s0 + q) * h + j); }
+#pragma unroll
+        for (int q = 0; q < kBatch; ++q)
+            if (s0 + q < k) { sum.x += w[q] * v[q].x; sum.y += w[q] * v[q].y; sum.z += w[q] * v[q].z; sum.w += w[q] * v[q].w; }
     }
-    if (shared) {
-        const float w = shared_w[t];
-        const float4 v = load4(shared + t * shared_ld + j);
-        sum.x += w * v.x; sum.y += w * v.y; sum.z += w * v.z; sum.w += w * v.w;
-    }
+    if (shared) { sum.x += sw * sv.x; sum.y += sw * sv.y; sum.z += sw * sv.z; sum.w += sw * sv.w; }
     if constexpr (OT == TQMOE_BF16) {
         if (residual) {
             const uint2 r = *reinterpret_cast<const uint2 *>(residual + i);
@@ -146,7 +153,8 @@ void dispatch_gateup(uint32_t type, Split sp, const GateupArgs & k, hipStream_t 
 
 // one block per expert serves every assignment of that expert when the id list is short enough to scan in the block
 constexpr int kScanIds = 2048;
-int dedup_mode(int64_t assignments) { return assignments <= kScanIds ? 1 : 0; }
+// (a single token's assignments go to different experts: nothing to share, and the scan would only stand in front of the loads)
+int dedup_mode(int64_t assignments, int slots) { return assignments > slots && assignments <= kScanIds ? 1 : 0; }
 
 int32_t matvec_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * image, void * y0, void * y1, uint32_t ytype, const int32_t * ids,
                       int64_t A, int xdiv, int slots, int topk, int shared_cols, void * stream, tqmoe_error * err, const char * what) {
@@ -162,7 +170,7 @@ int32_t matvec_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void *
     const Split sp = split_for(b0->cols / 32);
     if (sp.m == 0) return fail(err, TQMOE_E_UNSUPPORTED, "%s: cols %d is too wide for the decode kernels", what, b0->cols);
     if (int32_t rc = need_device(err, what)) return rc;
-    MatvecArgs k{view(*b0), b1 ? view(*b1) : view(*b0), static_cast<const uint8_t *>(image), y0, y1, ytype, ids, int(A), xdiv, dedup_mode(A), slots, topk, shared_cols};
+    MatvecArgs k{view(*b0), b1 ? view(*b1) : view(*b0), static_cast<const uint8_t *>(image), y0, y1, ytype, ids, int(A), xdiv, dedup_mode(A, slots), slots, topk, shared_cols};
     dispatch_matvec(b0->type, sp, b1 ? 2 : 1, k, static_cast<hipStream_t>(stream));
     return launched(err, what);
 }
@@ -260,7 +268,7 @@ extern "C" int32_t tqmoe_expert_gateup(const tqmoe_bank * gate, const tqmoe_bank
     const Split sp = split_for(gate->cols / 32);
     if (sp.m == 0) return fail(err, TQMOE_E_UNSUPPORTED, "%s: cols %d is too wide for the decode kernels", what, gate->cols);
     if (int32_t rc = need_device(err, what)) return rc;
-    GateupArgs k{view(*gate), view(*up), static_cast<const uint8_t *>(x_image), static_cast<uint8_t *>(act_image), ids, int(A), slots, topk, shared_ff, dedup_mode(A)};
+    GateupArgs k{view(*gate), view(*up), static_cast<const uint8_t *>(x_image), static_cast<uint8_t *>(act_image), ids, int(A), slots, topk, shared_ff, dedup_mode(A, slots)};
     dispatch_gateup(gate->type, sp, k, static_cast<hipStream_t>(stream));
     return launched(err, what);
 }

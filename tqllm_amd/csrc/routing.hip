@@ -227,16 +227,25 @@ template <int XT> __device__ __forceinline__ void topk_quantise_row(const TopkOu
     quantise_row_wave<XT>(o.x, token, o.cols, o.image + int64_t(token) * (o.cols / 32) * kImageSubBytes, lane);
 }
 
+// With an activation image to write the block has a second wave that does nothing else: the row's quantisation runs beside
+// the selection instead of after it.
 template <int R, int XT>
-__global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logits, TopkOut o, int e, int k, float scale) {
-    const int token = blockIdx.x, lane = threadIdx.x;
+__global__ __launch_bounds__(128) void topk_reg_k(const float * __restrict__ logits, TopkOut o, int e, int k, float scale) {
+    const int token = blockIdx.x, lane = threadIdx.x & 63;
     const float * x = logits + int64_t(token) * (e + 1);
-    // the input row's block of this lane (rows of up to 64 blocks: one per lane) is loaded now and quantised at the end, so
-    // that its latency passes under the selection
-    const int S = o.image ? o.cols / 32 : 0;
-    const bool row_in_regs = S > 0 && S <= 64;
-    float xv[32];
-    if (row_in_regs && lane < S) load_block32<XT>(o.x, int64_t(token) * o.cols + 32 * lane, xv);
+    if (threadIdx.x >= 64) {
+        const int S = o.cols / 32;
+        if (S <= 64) {   // one block of 32 values per lane
+            float xv[32];
+            if (lane < S) load_block32<XT>(o.x, int64_t(token) * o.cols + 32 * lane, xv);
+            uint8_t * image_row = o.image + int64_t(token) * S * kImageSubBytes;
+            const float amax = wave_max(lane < S ? block_amax(xv) : 0.f);
+            if (lane < S) quantise_block(xv, image_row, S, lane, amax);
+        } else {
+            topk_quantise_row<XT>(o, token, lane);
+        }
+        return;
+    }
     const float shared_logit = o.shared_weights ? x[e] : 0.f;
     int key[R];
     float m = -INFINITY, sum = 0.f;
@@ -256,6 +265,25 @@ __global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logi
     }
     float selected = 0.f, my_w = 0.f;   // lane s keeps selection s
     int my_id = 0;
+    if (k <= 64) {
+        // Every round is a chain of dependent wave reductions, so the rounds carry only what the next round needs: the
+        // winner's key stays in lane s and the probabilities are computed for all selections at once afterwards. Equal
+        // keys are rare: one ballot tells whether the winner is alone, and only a tie pays for the index reduction.
+        int my_key = kKeyZero;
+        for (int s = 0; s < k; ++s) {
+            int bk = key[0], bi = lane;
+#pragma unroll
+            for (int r = 1; r < R; ++r) if (key[r] > bk) { bk = key[r]; bi = lane + 64 * r; }   // strict: the lowest index of equal keys
+            const int topkey = wave_max_all_i(bk);
+            const unsigned long long tie = __ballot(bk == topkey);
+            const int best = __popcll(tie) == 1 ? __builtin_amdgcn_readlane(bi, __builtin_ctzll(tie)) : wave_min_all(bk == topkey ? bi : 0x7FFFFFFF);
+            if (lane == s) { my_id = best; my_key = topkey; }
+#pragma unroll
+            for (int r = 0; r < R; ++r) if (lane + 64 * r == best) key[r] = kKeyGone;
+        }
+        my_w = my_key == kKeyZero ? 0.f : expf(key_value(my_key) - m) / sum;   // the probability, as every entry's would be computed
+        for (int s = 0; s < k; ++s) selected += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_w), s));   // slot order, as the host sums them
+    } else
     for (int s = 0; s < k; ++s) {
         int bk = key[0], bi = lane;
 #pragma unroll
@@ -297,15 +325,6 @@ __global__ __launch_bounds__(64) void topk_reg_k(const float * __restrict__ logi
         __threadfence_block();
         topk_finish(o, x, token, lane, e, k, scale, selected);
     }
-    if (o.image) {
-        if (row_in_regs) {
-            uint8_t * image_row = o.image + int64_t(token) * S * kImageSubBytes;
-            const float amax = wave_max(lane < S ? block_amax(xv) : 0.f);
-            if (lane < S) quantise_block(xv, image_row, S, lane, amax);
-        } else {
-            topk_quantise_row<XT>(o, token, lane);
-        }
-    }
 }
 
 template <int XT>
@@ -339,11 +358,11 @@ __global__ __launch_bounds__(64) void topk_lds_k(const float * __restrict__ logi
 }
 
 template <int XT> void launch_topk(const float * logits, const TopkOut & o, int e, int k, int n, float scale, hipStream_t s) {
-    if (e <= 64) topk_reg_k<1, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
-    else if (e <= 128) topk_reg_k<2, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
-    else if (e <= 256) topk_reg_k<4, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
-    else if (e <= 512) topk_reg_k<8, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
-    else if (e <= 1024) topk_reg_k<16, XT><<<unsigned(n), 64, 0, s>>>(logits, o, e, k, scale);
+    if (e <= 64) topk_reg_k<1, XT><<<unsigned(n), o.image ? 128 : 64, 0, s>>>(logits, o, e, k, scale);
+    else if (e <= 128) topk_reg_k<2, XT><<<unsigned(n), o.image ? 128 : 64, 0, s>>>(logits, o, e, k, scale);
+    else if (e <= 256) topk_reg_k<4, XT><<<unsigned(n), o.image ? 128 : 64, 0, s>>>(logits, o, e, k, scale);
+    else if (e <= 512) topk_reg_k<8, XT><<<unsigned(n), o.image ? 128 : 64, 0, s>>>(logits, o, e, k, scale);
+    else if (e <= 1024) topk_reg_k<16, XT><<<unsigned(n), o.image ? 128 : 64, 0, s>>>(logits, o, e, k, scale);
     else topk_lds_k<XT><<<unsigned(n), 64, size_t(e) * sizeof(float), s>>>(logits, o, e, k, scale);
 }
 

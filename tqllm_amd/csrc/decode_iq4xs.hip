@@ -84,7 +84,6 @@ __device__ __forceinline__ v4i decode16(uint2 c, NibbleConsts nc) {
     return w;
 }
 
-
 // NB banks (gate and up, or one). gateup != 0: out0 is the activation image that receives silu(gate) * up; else out0 /
 // out1 receive the products as rows of `ytype`. wk waves share a row's super-blocks, tpw row tiles per block.
 // Dynamic LDS: the match list and the copy of the ids while the block finds its input rows, later the partial sums.
@@ -93,7 +92,7 @@ __device__ __forceinline__ v4i decode16(uint2 c, NibbleConsts nc) {
 // super-block; otherwise (rows quantised block by block, as the fused gate / up epilogue leaves them) each sub-block's
 // result is scaled in fp32.
 template <int NB, bool UNI>
-__global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * out0, void * out1, uint32_t ytype,
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void iq4xs_mfma_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * out0, void * out1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_lim, int wk,
                                                     int tpw, int gateup) {
     extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
@@ -130,7 +129,7 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
         const float * sc0 = image_scales(image_row_ptr(image, max(t0, 0) / xdiv, S), S);
         const float * sc1 = image_scales(image_row_ptr(image, max(t1, 0) / xdiv, S), S);
         const int64_t tile_g = int64_t(e) * tiles + tile;
-        const NibbleConsts pos = nibble_consts();
+        const NibbleConsts ncs = nibble_consts();
         const int sb_end = s_end / 8;   // whole super-blocks only (the launcher checks)
         // The weight bytes of a super-block: 8 bytes of codes per sub-block and the row's scale record, per lane, in
         // registers. The next super-block's are loaded before this one is multiplied, so that with several waves per SIMD
@@ -160,29 +159,47 @@ __global__ __launch_bounds__(512) void iq4xs_mfma_k(BankView b0, BankView b1, co
                 xs0[0] = p0.x; xs0[1] = p0.y; xs0[2] = p0.z; xs0[3] = p0.w; xs0[4] = p1.x; xs0[5] = p1.y; xs0[6] = p1.z; xs0[7] = p1.w;
                 xs1[0] = q0.x; xs1[1] = q0.y; xs1[2] = q0.z; xs1[3] = q0.w; xs1[4] = q1.x; xs1[5] = q1.y; xs1[6] = q1.z; xs1[7] = q1.w;
             }
+            // The products of step (bank, sub-block) + 1 are issued before the sums of this step are read: the matrix pipe's
+            // latency passes under the next step's lookups instead of in front of this step's multiply-adds.
+            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            auto issue = [&](int step) {
+                return __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[step & 7], decode16(cur.code[step >> 3][step & 7], ncs), zero, 0, 0, 0);
+            };
+            constexpr bool kAhead = UNI;   // the other kernels lose more to the registers of a second result than they gain
+            v16i acc = issue(0);
+            int si[4] = {0, 0, 0, 0};   // (hi, lo) plane sums of the two input rows, weighted by the sub-block scales
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                const uint2 rec = cur.rec[nb];
-                const float d = half_bits_to_float(iq4xs_d_bits(rec));
-                const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                int si[4] = {0, 0, 0, 0};   // (hi, lo) plane sums of the two input rows, weighted by the sub-block scales
-#pragma unroll
-                for (int ib = 0; ib < 8; ++ib) {
-                    const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[ib], decode16(cur.code[nb][ib], pos), zero, 0, 0, 0);
-                    if constexpr (UNI) {
-                        // |acc| <= 32 * 128 * 127 < 2^19 and |ls - 32| <= 32: 24-bit products, eight of them stay below 2^28
-                        const int ls = iq4xs_lsm32(rec, ib);
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) si[q] += __mul24(acc[q], ls);
-                    } else {
-                        const float ws = d * float(iq4xs_lsm32(rec, ib));
-                        accf[nb][0] += float((acc[0] << 7) + acc[1]) * (ws * xs0[ib]);
-                        accf[nb][1] += float((acc[2] << 7) + acc[3]) * (ws * xs1[ib]);
-                    }
+            for (int step = 0; step < 8 * NB; ++step) {
+                const int nb = step >> 3, ib = step & 7;
+                v16i ahead = zero;
+                if constexpr (kAhead) {
+                    if (step + 1 < 8 * NB) ahead = issue(step + 1);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
+                const uint2 rec = cur.rec[nb];
                 if constexpr (UNI) {
-                    accf[nb][0] += (float(si[0]) * 128.f + float(si[1])) * d;
-                    accf[nb][1] += (float(si[2]) * 128.f + float(si[3])) * d;
+                    // |acc| <= 32 * 128 * 127 < 2^19 and |ls - 32| <= 32: 24-bit products, eight of them stay below 2^28
+                    const int ls = iq4xs_lsm32(rec, ib);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) si[q] = (ib ? si[q] : 0) + __mul24(acc[q], ls);
+                    if (ib == 7) {
+                        const float d = half_bits_to_float(iq4xs_d_bits(rec));
+                        accf[nb][0] += (float(si[0]) * 128.f + float(si[1])) * d;
+                        accf[nb][1] += (float(si[2]) * 128.f + float(si[3])) * d;
+                    }
+                } else {
+                    const float ws = half_bits_to_float(iq4xs_d_bits(rec)) * float(iq4xs_lsm32(rec, ib));
+                    accf[nb][0] += float((acc[0] << 7) + acc[1]) * (ws * xs0[ib]);
+                    accf[nb][1] += float((acc[2] << 7) + acc[3]) * (ws * xs1[ib]);
+                }
+                // only four of the sixteen result registers are read; the others count as in use until here, or they are handed
+                // to the next lookups while the matrix pipe still writes them and every such write waits for the pipe
+                if constexpr (kAhead) {
+                    asm volatile("" : : "v"(acc));
+                    acc = ahead;
+                } else {
+                    asm volatile("" : : "v"(acc));
+                    if (step + 1 < 8 * NB) acc = issue(step + 1);
                 }
             }
             cur = nxt;

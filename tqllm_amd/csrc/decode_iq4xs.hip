@@ -91,12 +91,13 @@ __device__ __forceinline__ v4i decode16(uint2 c, NibbleConsts nc) {
 // kernel write). The 6-bit weight scales then multiply the integer results and the sums stay integers over a whole
 // super-block; otherwise (rows quantised block by block, as the fused gate / up epilogue leaves them) each sub-block's
 // result is scaled in fp32.
-template <int NB, bool UNI>
+template <int NB, bool UNI, bool STAGED>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void iq4xs_mfma_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * out0, void * out1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_lim, int wk,
-                                                    int tpw, int gateup) {
+                                                    int tpw, int gateup, int a_off) {
     extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
     __shared__ int meta[2], s_tok[kTP];
+    __shared__ float s_x0[kTP];
     __shared__ int ql[kMaxWaves * 2][32];
     const int a = blockIdx.y, e = ids[a];
     if (e < 0 || int64_t(e) * b0.rows >= b0.rows_total) return;   // skipped assignment, or an id outside the bank
@@ -104,10 +105,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
     const int n_tok = chunk_up(ids, A, a, e, mode, reinterpret_cast<int *>(stage), meta, tok);   // the lists live in the dynamic space
     if (n_tok == 0) return;
     if (threadIdx.x < kTP) s_tok[threadIdx.x] = tok[threadIdx.x];
-    __syncthreads();
 
     const int S = b0.cols / 32, NSB = S / 8, rows = b0.rows, tiles = rows / 32;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 31, g = lane >> 5;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n = lane & 31, g = lane >> 5;
     const int wk_i = wave % wk, rt_l = wave / wk, tile = blockIdx.x * tpw + rt_l;
     const bool shared_slot = (a % slots) >= topk;
     // the shared expert may have fewer rows (gate / up) or read a narrower input row (down)
@@ -115,43 +115,83 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
     const int s_end = !gateup && shared_slot ? shared_lim / 32 : S;
     const bool valid = tile < tiles && tile * 32 < row_lim;
 
+    // The weight bytes of a super-block: 8 bytes of codes per sub-block and the row's scale record, per lane, in
+    // registers. The next super-block's are loaded before this one is multiplied (into the other of two sets that swap
+    // roles, no copies), so that there are always loads in flight under the decode work. Past the wave's last
+    // super-block the same one is fetched again: a branch around the loads would make every wait a wait for all of them.
+    // The first super-block's loads go out before the input rows are staged: the two trips to memory overlap.
+    const int sb_end = s_end / 8;   // whole super-blocks only (the launcher checks)
+    const bool working = valid && wk_i < sb_end;
+    const int64_t tile_g = int64_t(e) * tiles + tile;
+    struct Cold { uint2 code[NB][8]; uint2 rec[NB]; };
+    auto fetch = [&](int sb, Cold & c) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const uint8_t * src = (nb ? b1 : b0).codes + (tile_g * S + int64_t(sb) * 8) * 512 + n * 16 + g * 8;
+#pragma unroll
+            for (int ib = 0; ib < 8; ++ib) c.code[nb][ib] = *reinterpret_cast<const uint2 *>(src + ib * 512);
+            c.rec[nb] = *reinterpret_cast<const uint2 *>((nb ? b1 : b0).aux + (tile_g * NSB + sb) * 256 + n * 8);
+        }
+    };
+    Cold c0, c1;
+    if (working) fetch(wk_i, c0);
+    // The planes and scales of the block's input rows go to LDS once: [sub-block][input row][64 bytes of planes], then
+    // [input row][sub-block] scales. The product loop then has no loads from memory but the weights', so that its waits
+    // count exactly those (a wait for an operand A load would also wait for every weight load issued before it).
+    uint8_t * a_lds = stage + a_off;
+    float * xs_lds = reinterpret_cast<float *>(a_lds + S * 256);
+    if constexpr (STAGED) {
+        const uint8_t * src_row[kTP];
+#pragma unroll
+        for (int j = 0; j < kTP; ++j) src_row[j] = image_row_ptr(image, (tok[j] >= 0 ? tok[j] : tok[0]) / xdiv, S);   // rows not served: the first row's
+        for (int i0 = threadIdx.x; i0 < S * 16; i0 += 4 * blockDim.x) {   // four pieces a thread per trip to memory
+            uint4 v[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i = min(i0 + q * int(blockDim.x), S * 16 - 1), j = (i >> 2) & 3;   // past the end: the last piece again, not stored
+                const uint8_t * row = j == 0 ? src_row[0] : j == 1 ? src_row[1] : j == 2 ? src_row[2] : src_row[3];
+                v[q] = *reinterpret_cast<const uint4 *>(row + (i >> 4) * 64 + (i & 3) * 16);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i = i0 + q * blockDim.x;
+                if (i < S * 16) *reinterpret_cast<uint4 *>(a_lds + i * 16) = v[q];
+            }
+        }
+        if constexpr (UNI) {   // the rows' one scale each
+            if (threadIdx.x < kTP) {
+                const int j = threadIdx.x;
+                s_x0[j] = image_scales(j == 0 ? src_row[0] : j == 1 ? src_row[1] : j == 2 ? src_row[2] : src_row[3], S)[0];
+            }
+        } else
+            for (int i = threadIdx.x; i < S * kTP; i += blockDim.x) {
+                const int j = i / S;
+                const uint8_t * row = j == 0 ? src_row[0] : j == 1 ? src_row[1] : j == 2 ? src_row[2] : src_row[3];
+                xs_lds[i] = image_scales(row, S)[i - j * S];
+            }
+    }
+    __syncthreads();
+
     float accf[NB][2];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) accf[nb][0] = accf[nb][1] = 0.f;
 
-    if (valid) {
-        // this lane's part of operand A: plane row n of the MFMA = plane (n & 1) of input row n >> 1. Rows past the ones
-        // served read the first row's planes: their sums land in result rows that nobody reads.
-        const int a_tok = n < 2 * kTP ? s_tok[n >> 1] : -1;
-        const uint8_t * a_row = image_row_ptr(image, max(a_tok, s_tok[0]) / xdiv, S) + (n & 1) * 32 + g * 16;
+    if (working) {
+        // this lane's part of operand A: plane row n of the MFMA = plane (n & 1) of input row n >> 1 (rows 8 and up repeat
+        // rows 0..7: their sums land in result rows that nobody reads)
+        // (not staged: straight from the image, a stride of 64 bytes per sub-block instead of the staged 256)
+        const int a_tok = max(s_tok[(n & 7) >> 1], s_tok[0]);
+        const uint8_t * a_lane = STAGED ? a_lds + ((n & 7) >> 1) * 64 + (n & 1) * 32 + g * 16 : image_row_ptr(image, a_tok / xdiv, S) + (n & 1) * 32 + g * 16;
+        constexpr int kStrideA = STAGED ? 256 : 64;
         // the two input rows whose sums land in this lane half's result registers
-        const int t0 = s_tok[2 * g], t1 = s_tok[2 * g + 1];
-        const float * sc0 = image_scales(image_row_ptr(image, max(t0, 0) / xdiv, S), S);
-        const float * sc1 = image_scales(image_row_ptr(image, max(t1, 0) / xdiv, S), S);
-        const int64_t tile_g = int64_t(e) * tiles + tile;
+        const float * sc0 = STAGED ? xs_lds + (2 * g) * S : image_scales(image_row_ptr(image, max(s_tok[2 * g], 0) / xdiv, S), S);
+        const float * sc1 = STAGED ? xs_lds + (2 * g + 1) * S : image_scales(image_row_ptr(image, max(s_tok[2 * g + 1], 0) / xdiv, S), S);
         const NibbleConsts ncs = nibble_consts();
-        const int sb_end = s_end / 8;   // whole super-blocks only (the launcher checks)
-        // The weight bytes of a super-block: 8 bytes of codes per sub-block and the row's scale record, per lane, in
-        // registers. The next super-block's are loaded before this one is multiplied, so that with several waves per SIMD
-        // there are always loads in flight under the decode work.
-        struct Cold { uint2 code[NB][8]; uint2 rec[NB]; };
-        auto fetch = [&](int sb, Cold & c) {
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                const uint8_t * src = (nb ? b1 : b0).codes + (tile_g * S + int64_t(sb) * 8) * 512 + n * 16 + g * 8;
-#pragma unroll
-                for (int ib = 0; ib < 8; ++ib) c.code[nb][ib] = *reinterpret_cast<const uint2 *>(src + ib * 512);
-                c.rec[nb] = *reinterpret_cast<const uint2 *>((nb ? b1 : b0).aux + (tile_g * NSB + sb) * 256 + n * 8);
-            }
-        };
-        Cold cur, nxt;
-        if (wk_i < sb_end) fetch(wk_i, cur);
-        for (int sb = wk_i; sb < sb_end; sb += wk) {
-            if (sb + wk < sb_end) fetch(sb + wk, nxt);
+        auto multiply = [&](int sb, const Cold & cur) {
             v4i areg[8];
 #pragma unroll
-            for (int ib = 0; ib < 8; ++ib) areg[ib] = *reinterpret_cast<const v4i *>(a_row + (sb * 8 + ib) * 64);
-            // activation scales of the 8 sub-blocks (rows not served read row 0's: nobody reads their sums)
+            for (int ib = 0; ib < 8; ++ib) areg[ib] = *reinterpret_cast<const v4i *>(a_lane + (sb * 8 + ib) * kStrideA);
+            // activation scales of the 8 sub-blocks
             float xs0[8], xs1[8];
             if constexpr (!UNI) {
                 const float4 p0 = *reinterpret_cast<const float4 *>(sc0 + sb * 8), p1 = *reinterpret_cast<const float4 *>(sc0 + sb * 8 + 4);
@@ -194,21 +234,33 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
                 }
                 // only four of the sixteen result registers are read; the others count as in use until here, or they are handed
                 // to the next lookups while the matrix pipe still writes them and every such write waits for the pipe
-                if constexpr (kAhead) {
-                    asm volatile("" : : "v"(acc));
-                    acc = ahead;
-                } else {
-                    asm volatile("" : : "v"(acc));
-                    if (step + 1 < 8 * NB) acc = issue(step + 1);
-                }
+                asm volatile("" : : "v"(acc));
+                if constexpr (kAhead) acc = ahead;
+                else if (step + 1 < 8 * NB) acc = issue(step + 1);
             }
-            cur = nxt;
+        };
+        if constexpr (STAGED) {
+            const int last = wk_i + (sb_end - 1 - wk_i) / wk * wk;   // the wave's last super-block
+            for (int sb = wk_i; sb <= last; sb += 2 * wk) {
+                fetch(min(sb + wk, last), c1);
+                multiply(sb, c0);
+                if (sb + wk > last) break;
+                fetch(min(sb + 2 * wk, last), c0);
+                multiply(sb + wk, c1);
+            }
+        } else {   // short batches: most waves have one super-block, and nothing is fetched that is not multiplied
+            for (int sb = wk_i; sb < sb_end; sb += wk) {
+                if (sb + wk < sb_end) fetch(sb + wk, c1);
+                multiply(sb, c0);
+                c0 = c1;
+            }
         }
     }
+
     if constexpr (UNI) {
         if (valid) {   // the rows' own scales, once
-            const int t0 = s_tok[2 * g], t1 = s_tok[2 * g + 1];
-            const float x0 = image_scales(image_row_ptr(image, max(t0, 0) / xdiv, S), S)[0], x1 = image_scales(image_row_ptr(image, max(t1, 0) / xdiv, S), S)[0];
+            const float x0 = STAGED ? s_x0[2 * g] : image_scales(image_row_ptr(image, max(s_tok[2 * g], 0) / xdiv, S), S)[0];
+            const float x1 = STAGED ? s_x0[2 * g + 1] : image_scales(image_row_ptr(image, max(s_tok[2 * g + 1], 0) / xdiv, S), S)[0];
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) { accf[nb][0] *= x0; accf[nb][1] *= x1; }
         }
@@ -255,12 +307,20 @@ void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0
     if (tpw > tiles) tpw = tiles;
     const dim3 grid(unsigned((tiles + tpw - 1) / tpw), unsigned(A));
     const unsigned threads = unsigned(wk * tpw * 64);
-    // dynamic LDS: the match list and the copy of the ids (2 * kMaxList ints), later the partial sums
+    // dynamic LDS: the match list and the copy of the ids (2 * kMaxList ints), later the partial sums; behind them the input
+    // rows' planes (256 bytes per sub-block) and, for rows with a scale per sub-block, the scales
     size_t lds = mode ? size_t(2) * kMaxList * sizeof(int) : 0;
     if (lds < size_t(wk * tpw) * nb * kTP * 32 * sizeof(float)) lds = size_t(wk * tpw) * nb * kTP * 32 * sizeof(float);
-    if (nb == 2 && uniform) iq4xs_mfma_k<2, true><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
-    else if (nb == 2) iq4xs_mfma_k<2, false><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
-    else iq4xs_mfma_k<1, false><<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup);
+    // the input rows go through LDS from a dozen tokens on (measured: 5 % at 16 and 32 tokens; the waves then overlap each
+    // other's waits, and what counts is that a wave's own weight loads stay in flight under its products); a short batch is
+    // one chain of dependent steps per wave, and the extra stop at a barrier costs more than the exact waits return
+    const bool staged = A >= 12 * slots;
+    const int a_off = int(lds);
+    if (staged) lds += size_t(b0.cols / 32) * (256 + (uniform ? 0 : kTP * sizeof(float)));
+    auto go = [&](auto kernel) { kernel<<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup, a_off); };
+    if (nb == 2 && uniform) staged ? go(iq4xs_mfma_k<2, true, true>) : go(iq4xs_mfma_k<2, true, false>);
+    else if (nb == 2) staged ? go(iq4xs_mfma_k<2, false, true>) : go(iq4xs_mfma_k<2, false, false>);
+    else staged ? go(iq4xs_mfma_k<1, false, true>) : go(iq4xs_mfma_k<1, false, false>);
 }
 
 }  // namespace

@@ -202,15 +202,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
             // The products of step (bank, sub-block) + 1 are issued before the sums of this step are read: the matrix pipe's
             // latency passes under the next step's lookups instead of in front of this step's multiply-adds.
             const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            // steps in the order (sub-block, bank): a sub-block's piece of operand A serves the banks one after the other
             auto issue = [&](int step) {
-                return __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[step & 7], decode16(cur.code[step >> 3][step & 7], ncs), zero, 0, 0, 0);
+                return __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[step / NB], decode16(cur.code[step % NB][step / NB], ncs), zero, 0, 0, 0);
             };
             constexpr bool kAhead = UNI;   // the other kernels lose more to the registers of a second result than they gain
             v16i acc = issue(0);
-            int si[4] = {0, 0, 0, 0};   // (hi, lo) plane sums of the two input rows, weighted by the sub-block scales
+            int si[NB][4];   // (hi, lo) plane sums of the two input rows, weighted by the sub-block scales
 #pragma unroll
             for (int step = 0; step < 8 * NB; ++step) {
-                const int nb = step >> 3, ib = step & 7;
+                const int nb = step % NB, ib = step / NB;
                 v16i ahead = zero;
                 if constexpr (kAhead) {
                     if (step + 1 < 8 * NB) ahead = issue(step + 1);
@@ -221,11 +222,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
                     // |acc| <= 32 * 128 * 127 < 2^19 and |ls - 32| <= 32: 24-bit products, eight of them stay below 2^28
                     const int ls = iq4xs_lsm32(rec, ib);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) si[q] = (ib ? si[q] : 0) + __mul24(acc[q], ls);
+                    for (int q = 0; q < 4; ++q) si[nb][q] = (ib ? si[nb][q] : 0) + __mul24(acc[q], ls);
                     if (ib == 7) {
                         const float d = half_bits_to_float(iq4xs_d_bits(rec));
-                        accf[nb][0] += (float(si[0]) * 128.f + float(si[1])) * d;
-                        accf[nb][1] += (float(si[2]) * 128.f + float(si[3])) * d;
+                        accf[nb][0] += (float(si[nb][0]) * 128.f + float(si[nb][1])) * d;
+                        accf[nb][1] += (float(si[nb][2]) * 128.f + float(si[nb][3])) * d;
                     }
                 } else {
                     const float ws = half_bits_to_float(iq4xs_d_bits(rec)) * float(iq4xs_lsm32(rec, ib));

@@ -29,13 +29,19 @@ constexpr int kMaxWaves = 8;
 // The input rows this block serves. mode 0: its own assignment only. mode 1: the assignments of ids[0..A) with this
 // block's expert, in index order, are cut into chunks of kTP; the block of each chunk's first assignment serves the
 // chunk (returns its size and the assignment indices in tok, -1 past the end) and the other blocks leave (returns 0).
-__device__ __forceinline__ int chunk_up(const int * __restrict__ ids, int A, int a, int e, int mode, int * list, int * meta, int (&tok)[kTP]) {
+// mode 1: the block's copy of the ids, and its own expert from that copy (one trip to memory for both)
+__device__ __forceinline__ int fetch_ids(const int * __restrict__ ids, int A, int a, int mode, int * list) {
+    if (mode == 0) return ids[a];
+    int * copy = list + kMaxList;
+    for (int i = threadIdx.x; i < A; i += blockDim.x) copy[i] = ids[i];
+    __syncthreads();
+    return copy[a];
+}
+__device__ __forceinline__ int chunk_up(int A, int a, int e, int mode, int * list, int * meta, int (&tok)[kTP]) {
 #pragma unroll
     for (int j = 0; j < kTP; ++j) tok[j] = -1;
     if (mode == 0) { tok[0] = a; return 1; }
-    int * copy = list + kMaxList;            // the ids, fetched by the whole block in one round trip
-    for (int i = threadIdx.x; i < A; i += blockDim.x) copy[i] = ids[i];
-    __syncthreads();
+    const int * copy = list + kMaxList;      // the ids, fetched by the whole block in one round trip (fetch_ids)
     if (threadIdx.x < 64) {   // one wave walks the ids in order: ballots keep the matches ordered
         const int lane = threadIdx.x;
         int base = 0;
@@ -99,10 +105,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
     __shared__ int meta[2], s_tok[kTP];
     __shared__ float s_x0[kTP];
     __shared__ int ql[kMaxWaves * 2][32];
-    const int a = blockIdx.y, e = ids[a];
+    const int a = blockIdx.y, e = fetch_ids(ids, A, a, mode, reinterpret_cast<int *>(stage));
     if (e < 0 || int64_t(e) * b0.rows >= b0.rows_total) return;   // skipped assignment, or an id outside the bank
     int tok[kTP];
-    const int n_tok = chunk_up(ids, A, a, e, mode, reinterpret_cast<int *>(stage), meta, tok);   // the lists live in the dynamic space
+    const int n_tok = chunk_up(A, a, e, mode, reinterpret_cast<int *>(stage), meta, tok);   // the lists live in the dynamic space
     if (n_tok == 0) return;
     if (threadIdx.x < kTP) s_tok[threadIdx.x] = tok[threadIdx.x];
 

@@ -35,7 +35,7 @@ __device__ __forceinline__ float4 load4(const uint16_t * p) {   // four fp16 val
 }
 // With a residual (bf16 rows, bf16 out) the result is bf16(bf16(sum) + residual): the reference stores the sum as bf16
 // (moe_sum) and adds the residual stream to it afterwards (add_sumsq, qwen35_forward.cpp:1248-1250), two roundings.
-template <int OT, class RT>
+template <int OT, class RT, int kBatch>
 __global__ __launch_bounds__(256) void combine_k(const RT * __restrict__ routed, int slots, const RT * __restrict__ shared, int64_t shared_ld,
                                                  const float * __restrict__ weights, const float * __restrict__ shared_w, void * __restrict__ out, int h, int k,
                                                  int64_t count, const uint16_t * __restrict__ residual) {
@@ -45,8 +45,8 @@ __global__ __launch_bounds__(256) void combine_k(const RT * __restrict__ routed,
     const int j = int(i % h);
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
     // the rows and weights of up to kBatch slots are loaded before the first of them is added: one trip to memory per batch
-    // instead of one per slot (the sum keeps the slot order)
-    constexpr int kBatch = 12;
+    // instead of one per slot (the sum keeps the slot order). A few tokens are one chain of trips per thread and take a batch
+    // of twelve; many tokens are bound by memory throughput, which the threads' number covers: a batch of one.
     float sw = 0.f;
     float4 sv = make_float4(0.f, 0.f, 0.f, 0.f);
     if (shared) { sw = shared_w[t]; sv = load4(shared + t * shared_ld + j); }
@@ -301,8 +301,14 @@ static int32_t combine_common(const RT * routed, int32_t slots, const RT * share
     const unsigned blocks = unsigned((count / 4 + 255) / 256);
     const hipStream_t s = static_cast<hipStream_t>(stream);
     if (residual && otype != TQMOE_BF16) return fail(err, TQMOE_E_UNSUPPORTED, "tqmoe_combine: a residual is added to BF16 output only");
-    if (otype == TQMOE_F32) combine_k<TQMOE_F32, RT><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count, nullptr);
-    else combine_k<TQMOE_BF16, RT><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count, residual);
+    const bool few = n <= 64;
+    if (otype == TQMOE_F32) {
+        if (few) combine_k<TQMOE_F32, RT, 12><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count, nullptr);
+        else combine_k<TQMOE_F32, RT, 1><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count, nullptr);
+    } else {
+        if (few) combine_k<TQMOE_BF16, RT, 12><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count, residual);
+        else combine_k<TQMOE_BF16, RT, 1><<<blocks, 256, 0, s>>>(routed, slots, shared, shared_ld, weights, shared_weights, out, hidden, topk, count, residual);
+    }
     return launched(err, "tqmoe_combine");
 }
 

@@ -103,25 +103,41 @@ __host__ __device__ inline Plan plan_at(const float * scale, int64_t grouped_row
     return Plan{p, p + experts + 1, p + 2 * (experts + 1), const_cast<int *>(p) + 3 * (experts + 1)};
 }
 
+// inclusive prefix sum over the wave's 64 lanes with DPP moves (rows of 16, then the rows' totals handed on)
+template <int N> __device__ __forceinline__ int dpp_row_shr(int v) { return __builtin_amdgcn_update_dpp(0, v, 0x110 + N, 0xF, 0xF, true); }
+__device__ __forceinline__ int wave_prefix_sum(int v) {
+    v += dpp_row_shr<1>(v);
+    v += dpp_row_shr<2>(v);
+    v += dpp_row_shr<4>(v);
+    v += dpp_row_shr<8>(v);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);   // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);   // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 __global__ __launch_bounds__(64) void plan_k(const int * __restrict__ counts, int experts, Plan plan) {
     const int lane = threadIdx.x;
     int * tile_base = const_cast<int *>(plan.tile_base), * chunk_base = const_cast<int *>(plan.chunk_base), * chunk_base2 = const_cast<int *>(plan.chunk_base2);
     if (lane < kPlanCounters) plan.counters[lane] = 0;
     int tbase = 0, cbase = 0, cbase2 = 0;
-    for (int e0 = 0; e0 < experts; e0 += 64) {
-        const int e = e0 + lane;
-        const int tiles = e < experts ? (max(counts[e], 0) + 31) >> 5 : 0;
-        const int chunks = (tiles + kChunkTiles - 1) / kChunkTiles, chunks2 = (tiles + 2 * kChunkTiles - 1) / (2 * kChunkTiles);
-        int ti = tiles, ci = chunks, c2 = chunks2;
+    constexpr int kAhead = 16;   // counts of 16 x 64 experts are loaded in one trip to memory, then scanned 64 at a time
+    for (int eb = 0; eb < experts; eb += 64 * kAhead) {
+        int cnt[kAhead];
 #pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const int a = __shfl_up(ti, d, 64), b = __shfl_up(ci, d, 64), c = __shfl_up(c2, d, 64);
-            if (lane >= d) { ti += a; ci += b; c2 += c; }
+        for (int i = 0; i < kAhead; ++i) cnt[i] = counts[min(eb + 64 * i + lane, experts - 1)];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+            const int e0 = eb + 64 * i;
+            if (e0 >= experts) break;
+            const int e = e0 + lane;
+            const int tiles = e < experts ? (max(cnt[i], 0) + 31) >> 5 : 0;
+            const int chunks = (tiles + kChunkTiles - 1) / kChunkTiles, chunks2 = (tiles + 2 * kChunkTiles - 1) / (2 * kChunkTiles);
+            const int ti = wave_prefix_sum(tiles), ci = wave_prefix_sum(chunks), c2 = wave_prefix_sum(chunks2);
+            if (e < experts) { tile_base[e] = tbase + ti - tiles; chunk_base[e] = cbase + ci - chunks; chunk_base2[e] = cbase2 + c2 - chunks2; }
+            tbase += __builtin_amdgcn_readlane(ti, 63);
+            cbase += __builtin_amdgcn_readlane(ci, 63);
+            cbase2 += __builtin_amdgcn_readlane(c2, 63);
         }
-        if (e < experts) { tile_base[e] = tbase + ti - tiles; chunk_base[e] = cbase + ci - chunks; chunk_base2[e] = cbase2 + c2 - chunks2; }
-        tbase += __shfl(ti, 63, 64);
-        cbase += __shfl(ci, 63, 64);
-        cbase2 += __shfl(c2, 63, 64);
     }
     if (lane == 0) { tile_base[experts] = tbase; chunk_base[experts] = cbase; chunk_base2[experts] = cbase2; }
 }

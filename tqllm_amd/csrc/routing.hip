@@ -72,82 +72,91 @@ template <int WT> int32_t launch_router_x(uint32_t xtype, const void * w, const 
 
 // Router logits of many tokens, bf16 rows on both sides: a GEMM on the matrix pipe. bf16 x bf16 products are exact in
 // fp32 and the matrix instruction accumulates in fp32, so the result differs from the scalar kernel's only by the order
-// of the sum. A block of four waves takes 128 tokens x 64 router rows; per 64 columns the block stages both operand
-// tiles in LDS with coalesced 16-byte loads (the next tiles are in registers while these are multiplied) and every wave
-// multiplies a 64 x 32 quadrant: two v_mfma_f32_32x32x16_bf16 per 16 columns.
+// of the sum. A block of four waves takes 64 tokens x 64 router rows, every wave a 32 x 32 quadrant. The kernel is a
+// chain of stages (load from memory, store to LDS, multiply), and a stage costs a trip to memory however little it
+// multiplies: so a stage is 256 columns wide (eight stages at hidden 2048), the next stage's loads are in registers while
+// this one is multiplied, and two blocks fit a compute unit. The shared expert's gate row rides along as a 65th row of the
+// last row block (one more matrix instruction per step for two of its waves), so that 512 experts are eight row blocks and
+// not nine.
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-constexpr int kRouterGemmMin = 120000;   // tokens x router rows from which a bf16 router and input take the GEMM (measured crossover: the
-                                         // GEMM's chain of 64-column stages over the hidden size sets a floor of about 30 us at hidden 2048,
-                                         // the wave-per-row kernel takes 10 us up to 16,000 and grows with tokens x rows)
-constexpr int kRgTok = 128, kRgRows = 64, kRgK = 64, kRgPad = kRgK + 8;   // halves per staged row: 16-byte reads of consecutive rows spread over the banks
+constexpr int kRouterGemmMin = 120000;   // tokens x router rows from which a bf16 router and input take the GEMM (the wave-per-row kernel
+                                         // takes 10 us up to 16,000 and grows with tokens x rows)
+constexpr int kRgTok = 64, kRgRows = 64, kRgK = 256, kRgPad = kRgK + 8;   // halves per staged row: 16-byte reads of consecutive rows spread over the banks
 
 __global__ __launch_bounds__(256) void router_gemm_bf16_k(const uint16_t * __restrict__ w, const uint16_t * __restrict__ shared, const uint16_t * __restrict__ x,
                                                             float * __restrict__ logits, int h, int e, int n) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[2][kRgTok][kRgPad];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][kRgRows][kRgPad];
+    __shared__ __attribute__((aligned(16))) uint16_t As[kRgTok][kRgPad];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[kRgRows + 1][kRgPad];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
     const int t0 = int(blockIdx.x) * kRgTok, r0 = int(blockIdx.y) * kRgRows;
-    const int mq = wave & 1, nq = wave >> 1;           // quadrant: tokens 64 mq.., router rows 32 nq..
-    // staging: thread -> (row, 16-byte piece) of the tiles; A has 128 rows x 8 pieces = 4 per thread, B 64 x 8 = 2
-    const int sp = tid & 7, sr = tid >> 3;             // piece, row (0..31)
-    const uint16_t * a_src[4], * b_src[2];
-    bool b_zero[2];
+    const bool last = blockIdx.y == gridDim.y - 1;     // this block also has row e (the shared gate, or zeros)
+    const int mq = wave & 1, nq = wave >> 1;           // quadrant: tokens 32 mq.., router rows 32 nq..
+    const bool extra = last && nq == 0;
+    // staging: thread -> 16-byte piece sp of rows sr, sr + 8, ... of both tiles (a wave's loads cover two whole rows of 512 bytes)
+    const int sp = tid & 31, sr = tid >> 5;
+    const uint16_t * a_src[8], * b_src[8];
+    bool b_zero[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a_src[i] = x + int64_t(min(t0 + sr + 32 * i, n - 1)) * h + 8 * sp;   // rows past the end repeat a valid row (not stored)
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int row = r0 + sr + 32 * i;
-        b_zero[i] = row > e || (row == e && shared == nullptr);
-        b_src[i] = (row < e ? w + int64_t(row) * h : (row == e && shared) ? shared : w) + 8 * sp;
+    for (int i = 0; i < 8; ++i) {
+        a_src[i] = x + int64_t(min(t0 + sr + 8 * i, n - 1)) * h + 8 * sp;   // rows past the end repeat a valid row (not stored)
+        const int row = r0 + sr + 8 * i;
+        b_zero[i] = row >= e;
+        b_src[i] = w + int64_t(min(row, e - 1)) * h + 8 * sp;
     }
-    uint4 a_st[4], b_st[2];
+    uint4 a_st[8], b_st[8], x_st = make_uint4(0, 0, 0, 0);
     auto fetch = [&](int k0) {
+        const bool in = k0 + 8 * sp < h;   // the last stage may be narrower
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a_st[i] = *reinterpret_cast<const uint4 *>(a_src[i] + k0);
-#pragma unroll
-        for (int i = 0; i < 2; ++i) b_st[i] = b_zero[i] ? make_uint4(0, 0, 0, 0) : *reinterpret_cast<const uint4 *>(b_src[i] + k0);
-    };
-    auto stage = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4 *>(&As[buf][sr + 32 * i][8 * sp]) = a_st[i];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4 *>(&Bs[buf][sr + 32 * i][8 * sp]) = b_st[i];
-    };
-    v16f acc[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int q = 0; q < 16; ++q) acc[i][q] = 0.f;
-    fetch(0);
-    stage(0);
-    __syncthreads();
-    const int chunks = h / kRgK;
-    for (int c = 0; c < chunks; ++c) {
-        const int buf = c & 1;
-        if (c + 1 < chunks) fetch((c + 1) * kRgK);
-#pragma unroll
-        for (int j = 0; j < kRgK / 16; ++j) {     // operand of lane (r, g): row r, columns 16 j + 8 g .. + 7
-            const v8bf b = *reinterpret_cast<const v8bf *>(&Bs[buf][nq * 32 + r][16 * j + 8 * g]);
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const v8bf a = *reinterpret_cast<const v8bf *>(&As[buf][mq * 64 + 32 * i + r][16 * j + 8 * g]);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
-            }
+        for (int i = 0; i < 8; ++i) {
+            a_st[i] = in ? *reinterpret_cast<const uint4 *>(a_src[i] + k0) : make_uint4(0, 0, 0, 0);
+            b_st[i] = in && !b_zero[i] ? *reinterpret_cast<const uint4 *>(b_src[i] + k0) : make_uint4(0, 0, 0, 0);
         }
-        if (c + 1 < chunks) stage(buf ^ 1);       // the other stage: last read before the previous barrier
+        if (last && tid < 32) x_st = in && shared ? *reinterpret_cast<const uint4 *>(shared + k0 + 8 * sp) : make_uint4(0, 0, 0, 0);
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            *reinterpret_cast<uint4 *>(&As[sr + 8 * i][8 * sp]) = a_st[i];
+            *reinterpret_cast<uint4 *>(&Bs[sr + 8 * i][8 * sp]) = b_st[i];
+        }
+        if (last && tid < 32) *reinterpret_cast<uint4 *>(&Bs[kRgRows][8 * sp]) = x_st;
+    };
+    v16f acc, accx;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc[q] = accx[q] = 0.f;
+    fetch(0);
+    for (int k0 = 0; k0 < h; k0 += kRgK) {
+        __syncthreads();          // the previous stage has been multiplied
+        stage();
         __syncthreads();
+        if (k0 + kRgK < h) fetch(k0 + kRgK);
+        const int steps = min(kRgK, h - k0) / 16;
+        auto step = [&](int j) {  // operand of lane (r, g): row r, columns 16 j + 8 g .. + 7
+            const v8bf a = *reinterpret_cast<const v8bf *>(&As[mq * 32 + r][16 * j + 8 * g]);
+            const v8bf b = *reinterpret_cast<const v8bf *>(&Bs[nq * 32 + r][16 * j + 8 * g]);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+            if (extra) {          // every column of this product is row e: lane r = 0 keeps it
+                const v8bf bx = *reinterpret_cast<const v8bf *>(&Bs[kRgRows][16 * j + 8 * g]);
+                accx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bx, accx, 0, 0, 0);
+            }
+        };
+        if (steps == kRgK / 16) {
+#pragma unroll
+            for (int j = 0; j < kRgK / 16; ++j) step(j);
+        } else {
+            for (int j = 0; j < steps; ++j) step(j);
+        }
     }
     // result register q of lane half g: token row 8 (q / 4) + 4 g + q % 4 of the 32-row tile, router row r
     const int row = r0 + nq * 32 + r;
-    if (row > e) return;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int q = 0; q < 16; ++q) {
-            const int t = t0 + mq * 64 + 32 * i + 8 * (q >> 2) + 4 * g + (q & 3);
-            if (t < n) logits[int64_t(t) * (e + 1) + row] = acc[i][q];
-        }
+    for (int q = 0; q < 16; ++q) {
+        const int t = t0 + mq * 32 + 8 * (q >> 2) + 4 * g + (q & 3);
+        if (t >= n) continue;
+        if (row < e) logits[int64_t(t) * (e + 1) + row] = acc[q];
+        if (extra && r == 0) logits[int64_t(t) * (e + 1) + e] = accx[q];
+    }
 }
 
 // ------------------------------------------------------------------------------------------------------ top-k
@@ -704,7 +713,7 @@ extern "C" int32_t tqmoe_router(const void * router, uint32_t wtype, const void 
     if (int32_t rc = need_device(err, "tqmoe_router")) return rc;
     const hipStream_t s = static_cast<hipStream_t>(stream);
     if (wtype == TQMOE_BF16 && xtype == TQMOE_BF16 && int64_t(n) * (experts + 1) >= kRouterGemmMin && hidden % 64 == 0) {
-        const dim3 grid(unsigned((n + kRgTok - 1) / kRgTok), unsigned((experts + 1 + kRgRows - 1) / kRgRows));
+        const dim3 grid(unsigned((n + kRgTok - 1) / kRgTok), unsigned((experts + kRgRows - 1) / kRgRows));
         router_gemm_bf16_k<<<grid, 256, 0, s>>>(static_cast<const uint16_t *>(router), static_cast<const uint16_t *>(shared_gate),
                                                                       static_cast<const uint16_t *>(x), logits, hidden, experts, n);
         return launched(err, "tqmoe_router");

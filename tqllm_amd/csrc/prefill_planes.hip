@@ -797,8 +797,10 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
     // Work items are (chunk of row tiles, unit of weight rows). Items that share operand A (one chunk, all units) have
     // indices that agree modulo 8, and the blocks that the round-robin of blocks over the 8 XCDs puts on one XCD take the
     // items of one residue from a counter of their own: one XCD's L2 serves a chunk's rows, and a block that finishes
-    // early takes more items. The next ticket is fetched under the current item's work. The last block to leave
-    // clears the counters for the next launch over these rows.
+    // early takes more items. The next ticket is fetched under the current item's work. A block whose own counter has
+    // run out goes on with the next XCD's, and so round all eight: the chunks of a residue differ in cost (a lone row tile
+    // against eight), so the XCDs' shares differ by a tenth and more, and only the last items of a launch lose their L2.
+    // The last block to leave clears the counters for the next launch over these rows.
     __syncthreads();
     const int * cbase = cached ? s_cbase : plan_chunks, * tbase = cached ? s_tbase : k.plan.tile_base;
     const int * cnts = cached ? s_cnt : k.counts, * offs = cached ? s_off : k.offsets;
@@ -808,7 +810,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
     const int NSB = k.b0.cols / 256, rows = k.b0.rows;
     __shared__ int s_ticket;
     int * ctr = k.plan.counters;
-    const int xcd = int(blockIdx.x) & 7;
+    int xcd = int(blockIdx.x) & 7, queues_done = 0;   // the queue this block takes from: its own XCD's first
     int ticket = 0;
     if (tid == 0) ticket = atomicAdd(&ctr[xcd], 1);
     for (;;) {
@@ -816,7 +818,12 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
         if (tid == 0) s_ticket = ticket;
         __syncthreads();
         const int item = 8 * s_ticket + xcd;
-        if (item >= items_padded) break;
+        if (item >= items_padded) {
+            if (++queues_done == 8) break;
+            xcd = (xcd + 1) & 7;
+            if (tid == 0) ticket = atomicAdd(&ctr[xcd], 1);
+            continue;
+        }
         if (tid == 0) ticket = atomicAdd(&ctr[xcd], 1);
         const int ug = (item >> 3) % groups, chunk = item / (8 * groups) * 8 + (item & 7);
         if (chunk >= n_chunks) continue;

@@ -57,6 +57,28 @@ def test_router_gemm_path(tq, oracle, n, e, h, shared):
         assert torch.equal(part, logits[5:5 + m])
 
 
+@pytest.mark.parametrize("n,e,h,shared", [(4096, 64, 2048, False), (3000, 130, 192, True), (2100, 64, 320, True), (1000, 64, 2048, False)])
+def test_router_gemm_path_f32(tq, oracle, n, e, h, shared):
+    """fp32 router rows and fp32 inputs take the matrix-pipe kernel from the same size on (the last case stays on the
+    wave-per-row kernel): fp32 products and sums, ragged shapes, with and without the shared-gate row."""
+    rng = np.random.default_rng(n + e + h)
+    w = (rng.standard_normal((e, h)) * 0.02).astype(np.float32)
+    gate = (rng.standard_normal(h) * 0.02).astype(np.float32)
+    xv = rng.standard_normal((n, h)).astype(np.float32)
+    x = dev(xv)
+    logits = tq.moe_router(dev(w), dev(gate) if shared else None, x)
+    got = logits.cpu().numpy()
+    exact = xv.astype(np.float64) @ np.vstack([w, gate if shared else np.zeros_like(gate)]).astype(np.float64).T
+    assert got.shape == (n, e + 1)
+    assert np.abs(got - exact).max() < 3e-6 * max(1.0, np.abs(exact).max() / 2)
+    if not shared:
+        assert not got[:, e].any()
+    m = -(-130000 // (e + 1))
+    if n >= m + 5:
+        part = tq.moe_router(dev(w), dev(gate) if shared else None, x[5:5 + m].contiguous())
+        assert torch.equal(part, logits[5:5 + m])
+
+
 def test_router_without_shared_gate_and_f16(tq, oracle):
     rng = np.random.default_rng(5)
     h, e, n = 512, 33, 7

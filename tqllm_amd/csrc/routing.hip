@@ -70,11 +70,11 @@ template <int WT> int32_t launch_router_x(uint32_t xtype, const void * w, const 
     return -1;
 }
 
-// Router logits of many tokens, bf16 rows on both sides: a GEMM on the matrix pipe. bf16 x bf16 products are exact in
-// fp32 and the matrix instruction accumulates in fp32, so the result differs from the scalar kernel's only by the order
-// of the sum. A block of four waves takes 64 tokens x 64 router rows, every wave a 32 x 32 quadrant. The kernel is a
+// Router logits of many tokens, bf16 rows on both sides or fp32 rows on both sides: a GEMM on the matrix pipe. bf16 x bf16
+// products are exact in fp32, the fp32 instruction multiplies and adds in fp32, and both accumulate in fp32, so the result
+// differs from the scalar kernel's only by the order of the sum. A block of four waves takes 64 tokens x 64 router rows, every wave a 32 x 32 quadrant. The kernel is a
 // chain of stages (load from memory, store to LDS, multiply), and a stage costs a trip to memory however little it
-// multiplies: so a stage is 256 columns wide (eight stages at hidden 2048), the next stage's loads are in registers while
+// multiplies: so a stage is 512 bytes of every row (256 bf16 columns: eight stages at hidden 2048; 128 fp32 columns), the next stage's loads are in registers while
 // this one is multiplied, and two blocks fit a compute unit. The shared expert's gate row rides along as a 65th row of the
 // last row block (one more matrix instruction per step for two of its waves), so that 512 experts are eight row blocks and
 // not nine.
@@ -84,8 +84,10 @@ constexpr int kRouterGemmMin = 120000;   // tokens x router rows from which a bf
                                          // takes 10 us up to 16,000 and grows with tokens x rows)
 constexpr int kRgTok = 64, kRgRows = 64, kRgK = 256, kRgPad = kRgK + 8;   // halves per staged row: 16-byte reads of consecutive rows spread over the banks
 
-__global__ __launch_bounds__(256) void router_gemm_bf16_k(const uint16_t * __restrict__ w, const uint16_t * __restrict__ shared, const uint16_t * __restrict__ x,
-                                                            float * __restrict__ logits, int h, int e, int n) {
+// F32: the rows are fp32 (h counts 2-byte units here: twice the columns); else bf16
+template <bool F32>
+__global__ __launch_bounds__(256) void router_gemm_k(const uint16_t * __restrict__ w, const uint16_t * __restrict__ shared, const uint16_t * __restrict__ x,
+                                                       float * __restrict__ logits, int h, int e, int n) {
     __shared__ __attribute__((aligned(16))) uint16_t As[kRgTok][kRgPad];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[kRgRows + 1][kRgPad];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
@@ -122,9 +124,9 @@ __global__ __launch_bounds__(256) void router_gemm_bf16_k(const uint16_t * __res
         }
         if (last && tid < 32) *reinterpret_cast<uint4 *>(&Bs[kRgRows][8 * sp]) = x_st;
     };
-    v16f acc, accx;
+    v16f acc, accx, acc1, acc2, acc3;   // the last three: fp32 rows only
 #pragma unroll
-    for (int q = 0; q < 16; ++q) acc[q] = accx[q] = 0.f;
+    for (int q = 0; q < 16; ++q) acc[q] = accx[q] = acc1[q] = acc2[q] = acc3[q] = 0.f;
     fetch(0);
     for (int k0 = 0; k0 < h; k0 += kRgK) {
         __syncthreads();          // the previous stage has been multiplied
@@ -132,13 +134,30 @@ __global__ __launch_bounds__(256) void router_gemm_bf16_k(const uint16_t * __res
         __syncthreads();
         if (k0 + kRgK < h) fetch(k0 + kRgK);
         const int steps = min(kRgK, h - k0) / 16;
-        auto step = [&](int j) {  // operand of lane (r, g): row r, columns 16 j + 8 g .. + 7
-            const v8bf a = *reinterpret_cast<const v8bf *>(&As[mq * 32 + r][16 * j + 8 * g]);
-            const v8bf b = *reinterpret_cast<const v8bf *>(&Bs[nq * 32 + r][16 * j + 8 * g]);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
-            if (extra) {          // every column of this product is row e: lane r = 0 keeps it
-                const v8bf bx = *reinterpret_cast<const v8bf *>(&Bs[kRgRows][16 * j + 8 * g]);
-                accx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bx, accx, 0, 0, 0);
+        auto step = [&](int j) {  // operand of lane (r, g): row r, the 16 bytes at halves 16 j + 8 g
+            if constexpr (F32) {  // four fp32 columns a lane: four instructions of two columns each, lane half g's s-th with the other half's s-th
+                const float4 a = *reinterpret_cast<const float4 *>(&As[mq * 32 + r][16 * j + 8 * g]);
+                const float4 b = *reinterpret_cast<const float4 *>(&Bs[nq * 32 + r][16 * j + 8 * g]);
+                // four running sums (joined at the end): a quarter of the terms each, and no instruction waits for the one before it
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc1, 0, 0, 0);
+                acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc2, 0, 0, 0);
+                acc3 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc3, 0, 0, 0);
+                if (extra) {
+                    const float4 bx = *reinterpret_cast<const float4 *>(&Bs[kRgRows][16 * j + 8 * g]);
+                    accx = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bx.x, accx, 0, 0, 0);
+                    accx = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bx.y, accx, 0, 0, 0);
+                    accx = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, bx.z, accx, 0, 0, 0);
+                    accx = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, bx.w, accx, 0, 0, 0);
+                }
+            } else {
+                const v8bf a = *reinterpret_cast<const v8bf *>(&As[mq * 32 + r][16 * j + 8 * g]);
+                const v8bf b = *reinterpret_cast<const v8bf *>(&Bs[nq * 32 + r][16 * j + 8 * g]);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+                if (extra) {      // every column of this product is row e: lane r = 0 keeps it
+                    const v8bf bx = *reinterpret_cast<const v8bf *>(&Bs[kRgRows][16 * j + 8 * g]);
+                    accx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bx, accx, 0, 0, 0);
+                }
             }
         };
         if (steps == kRgK / 16) {
@@ -147,6 +166,10 @@ __global__ __launch_bounds__(256) void router_gemm_bf16_k(const uint16_t * __res
         } else {
             for (int j = 0; j < steps; ++j) step(j);
         }
+    }
+    if constexpr (F32) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[q] = (acc[q] + acc1[q]) + (acc2[q] + acc3[q]);
     }
     // result register q of lane half g: token row 8 (q / 4) + 4 g + q % 4 of the 32-row tile, router row r
     const int row = r0 + nq * 32 + r;
@@ -712,10 +735,11 @@ extern "C" int32_t tqmoe_router(const void * router, uint32_t wtype, const void 
     if ((n + kRouterTok - 1) / kRouterTok > 65535) return fail(err, TQMOE_E_ARG, "tqmoe_router: too many tokens for one call");
     if (int32_t rc = need_device(err, "tqmoe_router")) return rc;
     const hipStream_t s = static_cast<hipStream_t>(stream);
-    if (wtype == TQMOE_BF16 && xtype == TQMOE_BF16 && int64_t(n) * (experts + 1) >= kRouterGemmMin && hidden % 64 == 0) {
+    if (wtype == xtype && (wtype == TQMOE_BF16 || wtype == TQMOE_F32) && int64_t(n) * (experts + 1) >= kRouterGemmMin && hidden % 64 == 0) {
         const dim3 grid(unsigned((n + kRgTok - 1) / kRgTok), unsigned((experts + kRgRows - 1) / kRgRows));
-        router_gemm_bf16_k<<<grid, 256, 0, s>>>(static_cast<const uint16_t *>(router), static_cast<const uint16_t *>(shared_gate),
-                                                                      static_cast<const uint16_t *>(x), logits, hidden, experts, n);
+        const uint16_t * w16 = static_cast<const uint16_t *>(router), * s16 = static_cast<const uint16_t *>(shared_gate), * x16 = static_cast<const uint16_t *>(x);
+        if (wtype == TQMOE_F32) router_gemm_k<true><<<grid, 256, 0, s>>>(w16, s16, x16, logits, 2 * hidden, experts, n);
+        else router_gemm_k<false><<<grid, 256, 0, s>>>(w16, s16, x16, logits, hidden, experts, n);
         return launched(err, "tqmoe_router");
     }
     if (wtype == TQMOE_F32) launch_router_x<TQMOE_F32>(xtype, router, shared_gate, x, logits, hidden, experts, n, s);

@@ -13,6 +13,7 @@
 // super-block ahead of the one it is multiplying, so the loads of the next super-block are in flight while this one is
 // decoded.
 #include "act_image.cuh"
+#include "decode_chunks.cuh"
 #include "decode_api.cuh"
 #include "formats.cuh"
 
@@ -22,50 +23,8 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kTP = 4;         // input rows per block
-constexpr int kMaxList = 2048; // assignments one block can scan (the launcher never passes more in mode 1)
+constexpr int kTP = kChunkRowsMax;   // input rows per block
 constexpr int kMaxWaves = 8;
-
-// The input rows this block serves. mode 0: its own assignment only. mode 1: the assignments of ids[0..A) with this
-// block's expert, in index order, are cut into chunks of kTP; the block of each chunk's first assignment serves the
-// chunk (returns its size and the assignment indices in tok, -1 past the end) and the other blocks leave (returns 0).
-// mode 1: the block's copy of the ids, and its own expert from that copy (one trip to memory for both)
-__device__ __forceinline__ int fetch_ids(const int * __restrict__ ids, int A, int a, int mode, int * list) {
-    if (mode == 0) return ids[a];
-    int * copy = list + kMaxList;
-    for (int i = threadIdx.x; i < A; i += blockDim.x) copy[i] = ids[i];
-    __syncthreads();
-    return copy[a];
-}
-__device__ __forceinline__ int chunk_up(int A, int a, int e, int mode, int * list, int * meta, int (&tok)[kTP]) {
-#pragma unroll
-    for (int j = 0; j < kTP; ++j) tok[j] = -1;
-    if (mode == 0) { tok[0] = a; return 1; }
-    const int * copy = list + kMaxList;      // the ids, fetched by the whole block in one round trip (fetch_ids)
-    if (threadIdx.x < 64) {   // one wave walks the ids in order: ballots keep the matches ordered
-        const int lane = threadIdx.x;
-        int base = 0;
-        for (int i0 = 0; i0 < A; i0 += 64) {
-            const int i = i0 + lane;
-            const bool match = i < A && copy[i] == e;
-            const unsigned long long mask = __ballot(match);
-            if (match) {
-                const int r = base + __popcll(mask & ((1ull << lane) - 1ull));
-                if (r < kMaxList) list[r] = i;
-                if (i == a) meta[1] = r;
-            }
-            base += __popcll(mask);
-        }
-        if (lane == 0) meta[0] = min(base, kMaxList);
-    }
-    __syncthreads();
-    const int cnt = meta[0], rank = meta[1];
-    if (rank % kTP) return 0;
-    const int n = min(kTP, cnt - rank);
-#pragma unroll
-    for (int j = 0; j < kTP; ++j) if (j < n) tok[j] = list[rank + j];
-    return n;
-}
 
 // 16 four-bit codes (two dwords) -> operand B of the MFMA: the lookups of lookup16(). The selector of the third pick
 // is (bit 3 of the code at bit 2) | byte position: one v_and_or_b32 when the mask and the positions sit in registers
@@ -108,7 +67,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
     const int a = blockIdx.y, e = fetch_ids(ids, A, a, mode, reinterpret_cast<int *>(stage));
     if (e < 0 || int64_t(e) * b0.rows >= b0.rows_total) return;   // skipped assignment, or an id outside the bank
     int tok[kTP];
-    const int n_tok = chunk_up(A, a, e, mode, reinterpret_cast<int *>(stage), meta, tok);   // the lists live in the dynamic space
+    const int n_tok = chunk_up(A, a, e, mode, kTP, reinterpret_cast<int *>(stage), meta, tok);   // the lists live in the dynamic space
     if (n_tok == 0) return;
     if (threadIdx.x < kTP) s_tok[threadIdx.x] = tok[threadIdx.x];
 

@@ -56,10 +56,12 @@ __device__ __forceinline__ v4i decode16(uint2 c, NibbleConsts nc) {
 // kernel write). The 6-bit weight scales then multiply the integer results and the sums stay integers over a whole
 // super-block; otherwise (rows quantised block by block, as the fused gate / up epilogue leaves them) each sub-block's
 // result is scaled in fp32.
-template <int NB, bool UNI, bool STAGED>
+// MODE 0: input rows read straight from the image; 1: staged in LDS; 2: staged, and a wave takes tl_count row tiles in turn
+template <int NB, bool UNI, int MODE>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void iq4xs_mfma_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * out0, void * out1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_lim, int wk,
-                                                    int tpw, int gateup, int a_off) {
+                                                    int tpw, int gateup, int a_off, int tl_count) {
+    constexpr bool STAGED = MODE >= 1, MULTI = MODE == 2;
     extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
     __shared__ int meta[2], s_tok[kTP];
     __shared__ float s_x0[kTP];
@@ -73,7 +75,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
 
     const int S = b0.cols / 32, NSB = S / 8, rows = b0.rows, tiles = rows / 32;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n = lane & 31, g = lane >> 5;
-    const int wk_i = wave % wk, rt_l = wave / wk, tile = blockIdx.x * tpw + rt_l;
+    const int wk_i = wave % wk, rt_l = wave / wk, tile = blockIdx.x * tl_count * tpw + rt_l;   // the wave's first (or only) row tile
     const bool shared_slot = (a % slots) >= topk;
     // the shared expert may have fewer rows (gate / up) or read a narrower input row (down)
     const int row_lim = gateup && shared_slot ? shared_lim : rows;
@@ -87,17 +89,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
     // The first super-block's loads go out before the input rows are staged: the two trips to memory overlap.
     const int sb_end = s_end / 8;   // whole super-blocks only (the launcher checks)
     const bool working = valid && wk_i < sb_end;
-    const int64_t tile_g = int64_t(e) * tiles + tile;
     struct Cold { uint2 code[NB][8]; uint2 rec[NB]; };
-    auto fetch = [&](int sb, Cold & c) {
+    // the lane's addresses in the wave's first row tile, worked out once; a fetch adds 32-bit offsets (dt row tiles further on)
+    const uint8_t * code_base[NB], * rec_base[NB];
+    {
+        const int64_t tile_g = int64_t(e) * tiles + tile;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-            const uint8_t * src = (nb ? b1 : b0).codes + (tile_g * S + int64_t(sb) * 8) * 512 + n * 16 + g * 8;
+            code_base[nb] = (nb ? b1 : b0).codes + tile_g * S * 512 + n * 16 + g * 8;
+            rec_base[nb] = (nb ? b1 : b0).aux + tile_g * NSB * 256 + n * 8;
+        }
+    }
+    auto fetch_tile = [&](int dt, int sb, Cold & c) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const uint8_t * src = code_base[nb] + uint32_t(dt * S + sb * 8) * 512u;
 #pragma unroll
             for (int ib = 0; ib < 8; ++ib) c.code[nb][ib] = *reinterpret_cast<const uint2 *>(src + ib * 512);
-            c.rec[nb] = *reinterpret_cast<const uint2 *>((nb ? b1 : b0).aux + (tile_g * NSB + sb) * 256 + n * 8);
+            c.rec[nb] = *reinterpret_cast<const uint2 *>(rec_base[nb] + uint32_t(dt * NSB + sb) * 256u);
         }
     };
+    auto fetch = [&](int sb, Cold & c) { fetch_tile(0, sb, c); };
     Cold c0, c1;
     if (working) fetch(wk_i, c0);
     // The planes and scales of the block's input rows go to LDS once: [sub-block][input row][64 bytes of planes], then
@@ -110,18 +122,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
 #pragma unroll
         for (int j = 0; j < kTP; ++j) src_row[j] = image_row_ptr(image, (tok[j] >= 0 ? tok[j] : tok[0]) / xdiv, S);   // rows not served: the first row's
         for (int i0 = threadIdx.x; i0 < S * 16; i0 += 4 * blockDim.x) {   // four pieces a thread per trip to memory
-            uint4 v[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int i = min(i0 + q * int(blockDim.x), S * 16 - 1), j = (i >> 2) & 3;   // past the end: the last piece again, not stored
+            auto piece = [&](int q) {   // past the end: the last piece again, not stored
+                const int i = min(i0 + q * int(blockDim.x), S * 16 - 1), j = (i >> 2) & 3;
                 const uint8_t * row = j == 0 ? src_row[0] : j == 1 ? src_row[1] : j == 2 ? src_row[2] : src_row[3];
-                v[q] = *reinterpret_cast<const uint4 *>(row + (i >> 4) * 64 + (i & 3) * 16);
-            }
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int i = i0 + q * blockDim.x;
-                if (i < S * 16) *reinterpret_cast<uint4 *>(a_lds + i * 16) = v[q];
-            }
+                return *reinterpret_cast<const uint4 *>(row + (i >> 4) * 64 + (i & 3) * 16);
+            };
+            auto put = [&](int q, const uint4 & v) {
+                const int i = i0 + q * int(blockDim.x);
+                if (i < S * 16) *reinterpret_cast<uint4 *>(a_lds + i * 16) = v;
+            };
+            // (four named values, not an array: an array indexed in two loops has been placed in scratch memory by the compiler,
+            // one trip to memory per piece)
+            const uint4 v0 = piece(0), v1 = piece(1), v2 = piece(2), v3 = piece(3);
+            put(0, v0); put(1, v1); put(2, v2); put(3, v3);
         }
         if constexpr (UNI) {   // the rows' one scale each
             if (threadIdx.x < kTP) {
@@ -140,6 +153,43 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
     float accf[NB][2];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) accf[nb][0] = accf[nb][1] = 0.f;
+
+    // A row tile's sums to their place. tile0: the block's first row tile of this pass.
+    auto finish = [&](int tile0, bool wave_valid) {
+        if constexpr (UNI) {
+            if (wave_valid) {   // the rows' own scales, once
+                const float x0 = STAGED ? s_x0[2 * g] : image_scales(image_row_ptr(image, max(s_tok[2 * g], 0) / xdiv, S), S)[0];
+                const float x1 = STAGED ? s_x0[2 * g + 1] : image_scales(image_row_ptr(image, max(s_tok[2 * g + 1], 0) / xdiv, S), S)[0];
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) { accf[nb][0] *= x0; accf[nb][1] *= x1; }
+            }
+        }
+        __syncthreads();                                       // the id list (or the previous pass's sums) is done with: the space now holds the partial sums
+        float (*red)[NB][kTP][32] = reinterpret_cast<float (*)[NB][kTP][32]>(stage);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) { red[wave][nb][2 * g][n] = accf[nb][0]; red[wave][nb][2 * g + 1][n] = accf[nb][1]; }
+        __syncthreads();
+
+        // the waves of a row tile hold the partial sums of its super-block shares: added here in wave order
+        const int groups = tpw * kTP, per_pass = blockDim.x >> 5;
+        for (int g0 = 0; g0 < groups; g0 += per_pass) {   // every wave runs every pass: the image quantiser exchanges lanes
+            const int grp = g0 + (threadIdx.x >> 5), i = threadIdx.x & 31;
+            const int rt = grp / kTP, j = grp % kTP, t = tile0 + rt;
+            const bool live = grp < groups && j < n_tok && t < tiles && t * 32 < row_lim;
+            float v0 = 0.f, v1 = 0.f;
+            if (live)
+                for (int w = 0; w < wk; ++w) { v0 += red[rt * wk + w][0][j][i]; if (NB == 2) v1 += red[rt * wk + w][NB - 1][j][i]; }
+            const int aj = live ? s_tok[j] : 0;
+            if (gateup) {
+                const float act = v0 / (1.f + expf(-v0)) * v1;
+                quantise_block_lanes(act, i, live, ql[threadIdx.x >> 5], static_cast<uint8_t *>(out0) + int64_t(aj) * tiles * kImageSubBytes, tiles, t);
+            } else if (live) {
+                const int64_t o = int64_t(aj) * rows + t * 32 + i;
+                if (ytype == TQMOE_F32) { static_cast<float *>(out0)[o] = v0; if (NB == 2) static_cast<float *>(out1)[o] = v1; }
+                else { static_cast<uint16_t *>(out0)[o] = float_to_bf16_bits(v0); if (NB == 2) static_cast<uint16_t *>(out1)[o] = float_to_bf16_bits(v1); }
+            }
+        }
+    };
 
     if (working) {
         // this lane's part of operand A: plane row n of the MFMA = plane (n & 1) of input row n >> 1 (rows 8 and up repeat
@@ -205,7 +255,28 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
                 else if (step + 1 < 8 * NB) acc = issue(step + 1);
             }
         };
-        if constexpr (STAGED) {
+        if constexpr (MULTI) {
+            // Several row tiles a wave, one after the other (the launcher has made sure that every wave of the block has the
+            // same steps: no ragged tiles, no shorter shared expert): the block finds its input rows and stages them once, and
+            // the weight loads run on across the tiles' ends, the next tile's first under this tile's sums.
+            const int nsteps = sb_end / wk, total = tl_count * nsteps;
+            auto fetch_step = [&](int gs, Cold & c) { fetch_tile(gs / nsteps * tpw, wk_i + gs % nsteps * wk, c); };
+            auto after = [&](int gs) {   // step gs is done: was it its tile's last?
+                if ((gs + 1) % nsteps) return;
+                finish((int(blockIdx.x) * tl_count + gs / nsteps) * tpw, true);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) accf[nb][0] = accf[nb][1] = 0.f;
+            };
+            for (int gs = 0; gs < total; gs += 2) {
+                fetch_step(min(gs + 1, total - 1), c1);
+                multiply(wk_i + gs % nsteps * wk, c0);
+                after(gs);
+                if (gs + 1 >= total) break;
+                fetch_step(min(gs + 2, total - 1), c0);
+                multiply(wk_i + (gs + 1) % nsteps * wk, c1);
+                after(gs + 1);
+            }
+        } else if constexpr (STAGED) {
             const int last = wk_i + (sb_end - 1 - wk_i) / wk * wk;   // the wave's last super-block
             for (int sb = wk_i; sb <= last; sb += 2 * wk) {
                 fetch(min(sb + wk, last), c1);
@@ -223,39 +294,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
         }
     }
 
-    if constexpr (UNI) {
-        if (valid) {   // the rows' own scales, once
-            const float x0 = STAGED ? s_x0[2 * g] : image_scales(image_row_ptr(image, max(s_tok[2 * g], 0) / xdiv, S), S)[0];
-            const float x1 = STAGED ? s_x0[2 * g + 1] : image_scales(image_row_ptr(image, max(s_tok[2 * g + 1], 0) / xdiv, S), S)[0];
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) { accf[nb][0] *= x0; accf[nb][1] *= x1; }
-        }
-    }
-    __syncthreads();                                       // the id list is done with: the space now holds the partial sums
-    float (*red)[NB][kTP][32] = reinterpret_cast<float (*)[NB][kTP][32]>(stage);
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) { red[wave][nb][2 * g][n] = accf[nb][0]; red[wave][nb][2 * g + 1][n] = accf[nb][1]; }
-    __syncthreads();
-
-    // the waves of a row tile hold the partial sums of its super-block shares: added here in wave order
-    const int groups = tpw * kTP, per_pass = blockDim.x >> 5;
-    for (int g0 = 0; g0 < groups; g0 += per_pass) {   // every wave runs every pass: the image quantiser exchanges lanes
-        const int grp = g0 + (threadIdx.x >> 5), i = threadIdx.x & 31;
-        const int rt = grp / kTP, j = grp % kTP, t = blockIdx.x * tpw + rt;
-        const bool live = grp < groups && j < n_tok && t < tiles && t * 32 < row_lim;
-        float v0 = 0.f, v1 = 0.f;
-        if (live)
-            for (int w = 0; w < wk; ++w) { v0 += red[rt * wk + w][0][j][i]; if (NB == 2) v1 += red[rt * wk + w][NB - 1][j][i]; }
-        const int aj = live ? s_tok[j] : 0;
-        if (gateup) {
-            const float act = v0 / (1.f + expf(-v0)) * v1;
-            quantise_block_lanes(act, i, live, ql[threadIdx.x >> 5], static_cast<uint8_t *>(out0) + int64_t(aj) * tiles * kImageSubBytes, tiles, t);
-        } else if (live) {
-            const int64_t o = int64_t(aj) * rows + t * 32 + i;
-            if (ytype == TQMOE_F32) { static_cast<float *>(out0)[o] = v0; if (NB == 2) static_cast<float *>(out1)[o] = v1; }
-            else { static_cast<uint16_t *>(out0)[o] = float_to_bf16_bits(v0); if (NB == 2) static_cast<uint16_t *>(out1)[o] = float_to_bf16_bits(v1); }
-        }
-    }
+    if constexpr (!MULTI) finish(blockIdx.x * tpw, valid);
 }
 
 void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0, void * out1, uint32_t ytype, const int * ids, int A, int xdiv, int mode,
@@ -271,7 +310,6 @@ void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0
     const int waves = wk == kMaxWaves ? kMaxWaves : 4;                    // per block: small blocks, a compute unit holds several and their phases interleave
     int tpw = waves / wk;                                                 // row tiles per block
     if (tpw > tiles) tpw = tiles;
-    const dim3 grid(unsigned((tiles + tpw - 1) / tpw), unsigned(A));
     const unsigned threads = unsigned(wk * tpw * 64);
     // dynamic LDS: the match list and the copy of the ids (2 * kMaxList ints), later the partial sums; behind them the input
     // rows' planes (256 bytes per sub-block) and, for rows with a scale per sub-block, the scales
@@ -281,12 +319,19 @@ void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0
     // other's waits, and what counts is that a wave's own weight loads stay in flight under its products); a short batch is
     // one chain of dependent steps per wave, and the extra stop at a barrier costs more than the exact waits return
     const bool staged = A >= 12 * slots;
+    // ... and a wave then takes up to four row tiles one after the other, as long as the grid keeps two blocks per compute
+    // unit: the block's search for its input rows and their staging are paid once for all of them
+    int tl = 1;
+    if (staged && nb == 1 && shared_lim == (gateup ? b0.rows : b0.cols))
+        while (tl < 4 && tiles % (tpw * tl * 2) == 0 && int64_t(tiles / (tpw * tl * 2)) * A >= 512) tl *= 2;
+    const dim3 grid(unsigned((tiles + tpw * tl - 1) / (tpw * tl)), unsigned(A));
     const int a_off = int(lds);
     if (staged) lds += size_t(b0.cols / 32) * (256 + (uniform ? 0 : kTP * sizeof(float)));
-    auto go = [&](auto kernel) { kernel<<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup, a_off); };
-    if (nb == 2 && uniform) staged ? go(iq4xs_mfma_k<2, true, true>) : go(iq4xs_mfma_k<2, true, false>);
-    else if (nb == 2) staged ? go(iq4xs_mfma_k<2, false, true>) : go(iq4xs_mfma_k<2, false, false>);
-    else staged ? go(iq4xs_mfma_k<1, false, true>) : go(iq4xs_mfma_k<1, false, false>);
+    auto go = [&](auto kernel) { kernel<<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup, a_off, tl); };
+    if (nb == 2 && uniform) staged ? go(iq4xs_mfma_k<2, true, 1>) : go(iq4xs_mfma_k<2, true, 0>);
+    else if (nb == 2) staged ? go(iq4xs_mfma_k<2, false, 1>) : go(iq4xs_mfma_k<2, false, 0>);
+    else if (tl > 1) go(iq4xs_mfma_k<1, false, 2>);
+    else staged ? go(iq4xs_mfma_k<1, false, 1>) : go(iq4xs_mfma_k<1, false, 0>);
 }
 
 }  // namespace

@@ -1268,7 +1268,7 @@ int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const i
     const int units = gateup ? b0.rows / 32 : b0.rows / (32 * nb);
     const int64_t tiles = grouped_row_tiles(assignments, experts);
     // units per item: about sixteen super-block steps of products behind one item's start-up, in a divisor of the units
-    int unit_group = std::max(1, std::min(8, 16 / std::max(1, b0.cols / 256)));
+    int unit_group = std::max(1, std::min(4, 16 / std::max(1, b0.cols / 256)));
     while (units % unit_group) --unit_group;
     GemmArgs k{view(b0), b1 ? view(*b1) : view(b0), xq, xs, counts, offsets, perm, plan_at(xs, tiles * 32, experts), experts, static_cast<uint16_t *>(out_f16),
                units, unit_group, shared_expert, shared_lim};

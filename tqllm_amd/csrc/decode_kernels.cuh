@@ -491,7 +491,9 @@ __device__ __forceinline__ int pair_up(const int * __restrict__ ids, int A, int 
 template <uint32_t FMT, int LPR, int M, int NB, int NT, int NJ, int NW, class Emit>
 __device__ __forceinline__ void block_rows(const Tile (&tile)[NB], int S, int rows_left, const ActBlock (&x)[NT][M], const uint32_t * grid, Emit emit) {
     using F = Sub<FMT>;
-    constexpr int RW = 64 / LPR, U = NJ >= 2 ? 2 : 1;
+    // row steps whose weight loads are in flight together: all four where a lane holds one sub-block per row (the block is
+    // then one trip to memory and one run of products), else two
+    constexpr int RW = 64 / LPR, U = (M == 1 && NJ % 4 == 0) ? 4 : NJ >= 2 ? 2 : 1;
     static_assert(NJ % U == 0, "row steps come in pairs");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rl = lane / LPR, sl = lane % LPR;

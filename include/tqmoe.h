@@ -53,6 +53,13 @@ int32_t tqmoe_router(const void * router, uint32_t wtype, const void * shared_ga
 int32_t tqmoe_topk(const float * logits, int32_t * ids, float * weights, float * shared_weights, int32_t experts,
                    int32_t topk, int32_t n, float scale, void * stream, tqmoe_error * err);
 
+/* tqmoe_topk on two routings of the same shape in one launch (this layer's and a prediction of the next layer's): the
+ * results of the two calls it stands for, bit for bit. Replaces tqllm_cuda::moe_topk2 (moe_kernels.cuh:24-25,
+ * moe.cu:261-263; called from src/models/qwen/qwen4exp/fn_layer_forward.cpp:331). experts <= 1024, as there. */
+int32_t tqmoe_topk2(const float * logits, int32_t * ids, float * weights, float * shared_weights, const float * logits2,
+                    int32_t * ids2, float * weights2, float * shared_weights2, int32_t experts, int32_t topk, int32_t n,
+                    float scale, void * stream, tqmoe_error * err);
+
 /* The reference's other routing modes, moe_route (src/experts/moe.cpp:22-113) in full:
  *   gating        TQMOE_GATE_SOFTMAX         p = softmax(logits)
  *                 TQMOE_GATE_SIGMOID         p = 1 / (1 + exp(-logit))

@@ -49,6 +49,12 @@ inline void moe_topk(const float * logits, int * ids, float * weights, float * s
     tqmoe_error e = fresh();
     check(tqmoe_topk(logits, ids, weights, shared_weights, experts, topk, n, scale, stream, &e), e);
 }
+// moe_topk2 (moe_kernels.cuh:24-25): two routings in one launch
+inline void moe_topk2(const float * logits, int * ids, float * weights, float * shared_weights, const float * logits2, int * ids2, float * weights2,
+                      float * shared_weights2, int e, int k, int n, float scale, void * stream) {
+    tqmoe_error err = fresh();
+    check(tqmoe_topk2(logits, ids, weights, shared_weights, logits2, ids2, weights2, shared_weights2, e, k, n, scale, stream, &err), err);
+}
 // moe_route (src/experts/moe.hpp:28-51) for n tokens on the device: the host function's configuration with its defaults
 // (sigmoid gating, weights not normalised, no scale); logits rows hold n_expert + 1 columns as moe_router writes them,
 // probs_bias is a device array of n_expert floats or null. Throws for a gating value outside MoeGating's.

@@ -104,6 +104,22 @@ def test_topk_matches_oracle_on_device_logits(tq, oracle, e, k, n):
     assert np.abs(sw - want_sw).max() < 3e-6
 
 
+@pytest.mark.parametrize("e,k,n", [(64, 8, 16), (512, 10, 300), (1000, 6, 9)])
+def test_topk2_equals_two_calls(tq, oracle, e, k, n):
+    """The reference's moe_topk2 (moe_kernels.cuh:24-25): two routings in one launch, the same bits as two launches; more
+    than 1024 experts are refused as there."""
+    rng = np.random.default_rng(e + k + n)
+    a, b = (dev(rng.standard_normal((n, e + 1)).astype(np.float32)) for _ in range(2))
+    first, second = tq.moe_topk2(a, b, e, k, scale=1.5)
+    for got, logits in ((first, a), (second, b)):
+        want = tq.moe_topk(logits, e, k, scale=1.5)
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
+    with pytest.raises(tq.TqmoeError):
+        big = dev(np.zeros((2, 1026), np.float32))
+        tq.moe_topk2(big, big, 1025, 2)
+
+
 def test_topk_ties_extremes_and_scale(tq, oracle):
     e, k = 96, 6
     rows = [np.full(e, 0.5, np.float32),                                   # all equal: lowest indices

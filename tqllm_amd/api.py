@@ -64,6 +64,7 @@ def lib():
         l.tqmoe_abi_version.restype = u32
         l.tqmoe_router.argtypes = [p, u32, p, p, u32, p, i32, i32, i32, p, e]
         l.tqmoe_topk.argtypes = [p, p, p, p, i32, i32, i32, f32, p, e]
+        l.tqmoe_topk2.argtypes = [p, p, p, p, p, p, p, p, i32, i32, i32, f32, p, e]
         l.tqmoe_topk_gated.argtypes = [p, p, i32, i32, p, p, p, i32, i32, i32, f32, p, e]
         l.tqmoe_dispatch_workspace_bytes.restype = sz
         l.tqmoe_dispatch_workspace_bytes.argtypes = [i32, i32, i32]
@@ -109,7 +110,7 @@ def lib():
         l.tqmoe_layer_workspace_bytes.argtypes = [C.POINTER(_Layer), i32]
         l.tqmoe_layer_forward.argtypes = [C.POINTER(_Layer), p, u32, i32, p, u32, p, p, p, p, sz, p, e]
         l.tqmoe_layer_path.argtypes = [C.POINTER(_Layer), i32]
-        for name in ("tqmoe_router", "tqmoe_topk", "tqmoe_dispatch", "tqmoe_bank_layout", "tqmoe_bank_load", "tqmoe_bank_dequant",
+        for name in ("tqmoe_router", "tqmoe_topk", "tqmoe_topk2", "tqmoe_dispatch", "tqmoe_bank_layout", "tqmoe_bank_load", "tqmoe_bank_dequant",
                      "tqmoe_quant_act", "tqmoe_expert_matvec", "tqmoe_expert_matvec2", "tqmoe_extend_ids", "tqmoe_expert_gateup", "tqmoe_expert_down", "tqmoe_combine_strided", "tqmoe_swiglu", "tqmoe_combine",
                      "tqmoe_layer_forward"):
             getattr(l, name).restype = i32
@@ -173,6 +174,21 @@ def moe_topk(logits, experts, topk, scale=1.0, gating=GATE_SOFTMAX, bias=None, n
         _check(lib().tqmoe_topk_gated(_ptr(logits), _ptr(bias), int(gating), int(bool(norm)), _ptr(ids), _ptr(weights), _ptr(shared), experts, topk,
                                       n, float(scale), _stream(logits), C.byref(err)), err)
     return ids, weights, shared
+
+
+def moe_topk2(logits, logits2, experts, topk, scale=1.0):
+    """moe_topk of two routings of one shape in one launch (moe_kernels.cuh:24-25): (ids, weights, shared) of each."""
+    n = logits.shape[0]
+    if logits2.shape != logits.shape:
+        raise ValueError("moe_topk2: the two logit arrays differ in shape")
+    out = []
+    for _ in range(2):
+        out.append((torch.empty((n, topk), dtype=torch.int32, device=logits.device), torch.empty((n, topk), dtype=torch.float32, device=logits.device),
+                    torch.empty((n,), dtype=torch.float32, device=logits.device)))
+    err = _err()
+    _check(lib().tqmoe_topk2(_ptr(logits), _ptr(out[0][0]), _ptr(out[0][1]), _ptr(out[0][2]), _ptr(logits2), _ptr(out[1][0]), _ptr(out[1][1]),
+                             _ptr(out[1][2]), experts, topk, n, float(scale), _stream(logits), C.byref(err)), err)
+    return out[0], out[1]
 
 
 def moe_dispatch(ids, experts, capacity=0):

@@ -262,7 +262,7 @@ template <int XT> __device__ __forceinline__ void topk_quantise_row(const TopkOu
 // With an activation image to write the block has a second wave that does nothing else: the row's quantisation runs beside
 // the selection instead of after it.
 template <int R, int XT>
-__global__ __launch_bounds__(128) void topk_reg_k(const float * __restrict__ logits, TopkOut o, int e, int k, float scale) {
+__device__ __forceinline__ void topk_reg_body(const float * __restrict__ logits, const TopkOut & o, int e, int k, float scale) {
     const int token = blockIdx.x, lane = threadIdx.x & 63;
     const float * x = logits + int64_t(token) * (e + 1);
     if (threadIdx.x >= 64) {
@@ -357,6 +357,18 @@ __global__ __launch_bounds__(128) void topk_reg_k(const float * __restrict__ log
         __threadfence_block();
         topk_finish(o, x, token, lane, e, k, scale, selected);
     }
+}
+
+template <int R, int XT>
+__global__ __launch_bounds__(128) void topk_reg_k(const float * __restrict__ logits, TopkOut o, int e, int k, float scale) {
+    topk_reg_body<R, XT>(logits, o, e, k, scale);
+}
+// two routings of the same shape in one launch (blockIdx.y picks): this layer's and a prediction of the next layer's
+template <int R>
+__global__ __launch_bounds__(64) void topk2_reg_k(const float * __restrict__ logits, TopkOut o, const float * __restrict__ logits2, TopkOut o2, int e, int k,
+                                                  float scale) {
+    if (blockIdx.y == 0) topk_reg_body<R, TQMOE_F32>(logits, o, e, k, scale);
+    else topk_reg_body<R, TQMOE_F32>(logits2, o2, e, k, scale);
 }
 
 template <int XT>
@@ -780,6 +792,25 @@ extern "C" int32_t tqmoe_topk(const float * logits, int32_t * ids, float * weigh
     enqueue_topk(logits, ids, weights, shared_weights, nullptr, 0, nullptr, TQMOE_F32, 0, nullptr, experts, topk, n, scale, TQMOE_GATE_SOFTMAX, nullptr, 1,
                  static_cast<hipStream_t>(stream), 0);
     return launched(err, "tqmoe_topk");
+}
+
+// The reference's moe_topk2 (src/experts/moe_kernels.cuh:24-25, src/experts/moe.cu:261-263): moe_topk on two routings in
+// one launch, at most 1024 experts.
+extern "C" int32_t tqmoe_topk2(const float * logits, int32_t * ids, float * weights, float * shared_weights, const float * logits2, int32_t * ids2,
+                               float * weights2, float * shared_weights2, int32_t experts, int32_t topk, int32_t n, float scale, void * stream,
+                               tqmoe_error * err) {
+    if (!logits || !ids || !weights || !logits2 || !ids2 || !weights2 || experts <= 0 || experts > 1024 || topk <= 0 || topk > experts || n <= 0)
+        return fail(err, TQMOE_E_ARG, "tqmoe_topk2: invalid shape or pointer (at most 1024 experts)");
+    if (int32_t rc = need_device(err, "tqmoe_topk2")) return rc;
+    const TopkOut o{ids, weights, shared_weights, nullptr, 0, nullptr, nullptr, 0, 0}, o2{ids2, weights2, shared_weights2, nullptr, 0, nullptr, nullptr, 0, 0};
+    const dim3 grid(unsigned(n), 2);
+    const hipStream_t s = static_cast<hipStream_t>(stream);
+    if (experts <= 64) topk2_reg_k<1><<<grid, 64, 0, s>>>(logits, o, logits2, o2, experts, topk, scale);
+    else if (experts <= 128) topk2_reg_k<2><<<grid, 64, 0, s>>>(logits, o, logits2, o2, experts, topk, scale);
+    else if (experts <= 256) topk2_reg_k<4><<<grid, 64, 0, s>>>(logits, o, logits2, o2, experts, topk, scale);
+    else if (experts <= 512) topk2_reg_k<8><<<grid, 64, 0, s>>>(logits, o, logits2, o2, experts, topk, scale);
+    else topk2_reg_k<16><<<grid, 64, 0, s>>>(logits, o, logits2, o2, experts, topk, scale);
+    return launched(err, "tqmoe_topk2");
 }
 
 extern "C" int32_t tqmoe_topk_gated(const float * logits, const float * probs_bias, int32_t gating, int32_t norm_weights, int32_t * ids, float * weights,

@@ -27,8 +27,25 @@ __global__ __launch_bounds__(256) void router_k(const void * __restrict__ w, con
     float acc[TOK];
 #pragma unroll
     for (int i = 0; i < TOK; ++i) acc[i] = 0.f;
-    if (has_row)
-        for (int c = lane * 8; c < h; c += 512) {
+    if (has_row) {
+        // four 512-column steps of loads at a time (one trip to memory for them instead of four), the sums in column order
+        // as before; then what is left of the row step by step
+        int c = lane * 8;
+        if constexpr (TOK == 1) {
+            for (; c + 3 * 512 < h; c += 4 * 512) {
+                float wv[4][8], xv[4][8];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    load8<WT>(wr, wbase + c + 512 * q, wv[q]);
+                    load8<XT>(x, int64_t(t0) * h + c + 512 * q, xv[q]);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[0] = fmaf(wv[q][j], xv[q][j], acc[0]);
+            }
+        }
+        for (; c < h; c += 512) {
             float wv[8];
             load8<WT>(wr, wbase + c, wv);
 #pragma unroll
@@ -41,6 +58,7 @@ __global__ __launch_bounds__(256) void router_k(const void * __restrict__ w, con
                 }
             }
         }
+    }
 #pragma unroll
     for (int i = 0; i < TOK; ++i) {
         const float s = group_sum<64>(acc[i]);

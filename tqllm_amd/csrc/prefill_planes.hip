@@ -879,7 +879,12 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                 sbe = wdead ? 0 : !GATEUP && is_shared ? k.shared_lim / 256 : NSB;
             }
             const int8_t * a_ptr = k.xq + int64_t(tile_base + first_tile) * 32 * k.b0.cols + lane * 16;
-            struct Stage { typename W::Code code[SPW][8]; typename W::Rec rec[SPW]; typename W::DRec drec[SPW]; v4i a[8]; };
+            // (the weights' codes run a super-block ahead, and so do the row tile's operands where the codes are short; with
+            // codes of 12 bytes and more the operands are read at the start of their super-block's work instead: they come
+            // from the L2, the SIMD's other wave covers the wait, and a second set of them is 32 registers that those
+            // formats spilled)
+            constexpr bool kAheadA = sizeof(typename W::Code) <= 8;
+            struct Stage { typename W::Code code[SPW][8]; typename W::Rec rec[SPW]; typename W::DRec drec[SPW]; v4i a[kAheadA ? 8 : 1]; };
             auto fetch1 = [&](int sb, Stage & st) {   // a super-block of the wave's weights and of the row tile
 #pragma unroll
                 for (int q = 0; q < SPW; ++q) {
@@ -890,13 +895,19 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                 for (int ib = 0; ib < 8; ++ib) {
 #pragma unroll
                     for (int q = 0; q < SPW; ++q) st.code[q][ib] = W::code(wsrc[q], sb * 8 + ib);
-                    st.a[ib] = *reinterpret_cast<const v4i *>(a_ptr + (int64_t(sb) * 8 + ib) * 1024);
+                    if constexpr (kAheadA) st.a[ib] = *reinterpret_cast<const v4i *>(a_ptr + (int64_t(sb) * 8 + ib) * 1024);
                 }
             };
             Acc<W> acc[SPW];
 #pragma unroll
             for (int q = 0; q < SPW; ++q) acc_clear(acc[q]);
             auto work1 = [&](int sb, Stage & cur, Stage & nxt) {
+                v4i a[8];
+#pragma unroll
+                for (int ib = 0; ib < 8; ++ib) {
+                    if constexpr (kAheadA) a[ib] = cur.a[ib];
+                    else a[ib] = *reinterpret_cast<const v4i *>(a_ptr + (int64_t(sb) * 8 + ib) * 1024);
+                }
                 fetch1(min(sb + 1, sbe - 1), nxt);   // past the last one the same again, from the cache: no branch, the same loads in flight on every path
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -906,7 +917,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                         v4i w0[P], w1[P];
                         W::planes(cur.code[q][ib], cur.rec[q], ib, g, s_tab, s_lat, w0);
                         W::planes(cur.code[q][ib + 1], cur.rec[q], ib + 1, g, s_tab, s_lat, w1);
-                        acc_step2(acc[q], cur.a[ib], cur.a[ib + 1], w0, w1, ib == 0, cur.drec[q], ib);
+                        acc_step2(acc[q], a[ib], a[ib + 1], w0, w1, ib == 0, cur.drec[q], ib);
                     }
                 }
 #pragma unroll

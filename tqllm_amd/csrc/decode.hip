@@ -167,7 +167,7 @@ int32_t matvec_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void *
     if (!image || !y0 || (b1 && !y1) || !ids || A <= 0) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
     if (A > 65535) return fail(err, TQMOE_E_ARG, "%s: more than 65535 assignments in one call", what);  // src/formats/weight/quant.cu:73
     if (ytype != TQMOE_F32 && ytype != TQMOE_BF16) return fail(err, TQMOE_E_UNSUPPORTED, "%s: output type must be F32 or BF16", what);
-    const Split sp = split_for(b0->cols / 32);
+    const Split sp = split_for(b0->cols / 32, A);
     if (sp.m == 0) return fail(err, TQMOE_E_UNSUPPORTED, "%s: cols %d is too wide for the decode kernels", what, b0->cols);
     if (int32_t rc = need_device(err, what)) return rc;
     MatvecArgs k{view(*b0), b1 ? view(*b1) : view(*b0), static_cast<const uint8_t *>(image), y0, y1, ytype, ids, int(A), xdiv, dedup_mode(A, slots), slots, topk, shared_cols};
@@ -265,7 +265,7 @@ extern "C" int32_t tqmoe_expert_gateup(const tqmoe_bank * gate, const tqmoe_bank
     if (slots > topk && (shared_ff <= 0 || shared_ff > gate->rows || shared_ff % 32)) return fail(err, TQMOE_E_ARG, "%s: invalid shared_ff", what);
     const int64_t A = int64_t(n) * slots;
     if (A > 65535) return fail(err, TQMOE_E_ARG, "%s: more than 65535 assignments in one call", what);
-    const Split sp = split_for(gate->cols / 32);
+    const Split sp = split_for(gate->cols / 32, A);
     if (sp.m == 0) return fail(err, TQMOE_E_UNSUPPORTED, "%s: cols %d is too wide for the decode kernels", what, gate->cols);
     if (int32_t rc = need_device(err, what)) return rc;
     GateupArgs k{view(*gate), view(*up), static_cast<const uint8_t *>(x_image), static_cast<uint8_t *>(act_image), ids, int(A), slots, topk, shared_ff, dedup_mode(A, slots)};

@@ -11,8 +11,13 @@ inline BankView view(const tqmoe_bank & b) {
 
 // lanes per row (8, 16, 32 or 64) and sub-blocks per lane (1..4) for S sub-blocks per row; m == 0: not supported
 struct Split { int lpr, m; };
-inline Split split_for(int S) {
+inline Split split_for(int S, int64_t assignments = 1 << 30) {
     if (S % 64 == 0) return Split{64, S / 64 <= 4 ? S / 64 : 0};
+    // 17 to 31 sub-blocks, a few assignments: a lane per sub-block with the last lanes of each 32 idle, rather than three
+    // sub-blocks per lane on 8 lanes. Three times the activation blocks in registers (190 and more) leave a SIMD two waves
+    // instead of five, and a short batch is a chain of trips to memory that only more waves shorten (one token: 15 % of the
+    // step); a long batch is bound by the vector work, and the idle lanes then cost more (64 tokens: +8 %).
+    if (S > 16 && S < 32 && assignments <= 48) return Split{32, 1};
     for (int lpr = 32; lpr >= 8; lpr >>= 1)
         if (S % lpr == 0 && S / lpr <= 4 && (S / lpr == 1 || S / lpr == 3)) return Split{lpr, S / lpr};
     return Split{64, (S + 63) / 64 <= 4 ? (S + 63) / 64 : 0};  // ragged: lanes past the row's last sub-block idle

@@ -493,7 +493,7 @@ __device__ __forceinline__ void block_rows(const Tile (&tile)[NB], int S, int ro
     using F = Sub<FMT>;
     // row steps whose weight loads are in flight together: all four where a lane holds one sub-block per row (the block is
     // then one trip to memory and one run of products), else two
-    constexpr int RW = 64 / LPR, U = (M == 1 && NJ % 4 == 0) ? 4 : NJ >= 2 ? 2 : 1;
+    constexpr int RW = 64 / LPR, U = (M == 1 && NJ % 4 == 0) ? 4 : (M >= 3) ? 1 : NJ >= 2 ? 2 : 1;
     static_assert(NJ % U == 0, "row steps come in pairs");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rl = lane / LPR, sl = lane % LPR;
@@ -545,8 +545,9 @@ __device__ __forceinline__ void load_x(const uint8_t * __restrict__ image, const
 
 // ------------------------------------------------------------------------------------------- grouped mat-vec
 // grid (row tiles, assignments), NW waves. y[a][r] for the tile's rows; NB banks (gate and up) share ids and the input.
+// (IQ3_S with three sub-blocks a lane and one bank sits three registers above what lets a SIMD hold three waves: it is held to that)
 template <uint32_t FMT, int LPR, int M, int NB, int NJ, int NW>
-__global__ __launch_bounds__(NW * 64) void matvec_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * y0, void * y1, uint32_t ytype,
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((FMT == TQMOE_IQ3_S && M == 3 && NB == 1) ? 3 : 1))) void matvec_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * y0, void * y1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_cols) {
     __shared__ __attribute__((aligned(8))) uint32_t grid_lds[lattice_dwords(FMT)];
     __shared__ int meta[2];

@@ -13,7 +13,7 @@ namespace {
 // sum by ordinary fp32 rounding only.
 constexpr int kRouterTok = 4;       // tokens per pass of a wave: the router row is read once for them
 constexpr int kRouterTokFew = 1;    // decode-sized batches: a wave per (row, token), the latency of a wave's chain is what counts
-constexpr int kRouterFew = 32;      // batches up to here take kRouterTokFew
+constexpr int kRouterFew = 7;       // batches up to here take kRouterTokFew
 template <int WT, int XT, int TOK>
 __global__ __launch_bounds__(256) void router_k(const void * __restrict__ w, const void * __restrict__ shared,
                                                 const void * __restrict__ x, float * __restrict__ logits, int h, int e, int n) {
@@ -31,6 +31,23 @@ __global__ __launch_bounds__(256) void router_k(const void * __restrict__ w, con
         // four 512-column steps of loads at a time (one trip to memory for them instead of four), the sums in column order
         // as before; then what is left of the row step by step
         int c = lane * 8;
+        if constexpr (TOK > 1) {   // two steps of loads at a time for the four tokens of a pass
+            for (; c + 512 < h; c += 2 * 512) {
+                float wv[2][8], xv[TOK][2][8];
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    load8<WT>(wr, wbase + c + 512 * q, wv[q]);
+#pragma unroll
+                    for (int i = 0; i < TOK; ++i) load8<XT>(x, int64_t(min(t0 + i, n - 1)) * h + c + 512 * q, xv[i][q]);
+                }
+#pragma unroll
+                for (int i = 0; i < TOK; ++i)
+#pragma unroll
+                    for (int q = 0; q < 2; ++q)
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) acc[i] = fmaf(wv[q][j], xv[i][q][j], acc[i]);
+            }
+        }
         if constexpr (TOK == 1) {
             for (; c + 3 * 512 < h; c += 4 * 512) {
                 float wv[4][8], xv[4][8];

@@ -1111,13 +1111,14 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
 #pragma unroll
                     for (int b = 0; b < NB; ++b) d_rec[b] = d_rec_next[b];
                     // The decode of the next step's pieces is placed between the groups of products, so that its vector
-                    // work runs while the matrix pipe works through the group just issued.
+                    // work runs while the matrix pipe works through the group just issued: in front of the step's last
+                    // group where a wave has two pieces, so that the codes (fetched behind the previous step's decode, from
+                    // memory) have had a whole step to arrive; the fetch of the step after next follows at once.
                     fetch_d(sb, 1);
 #pragma unroll
                     for (int jp = 0; jp < 4; ++jp) {
                         if constexpr (PIECES == 2) {
-                            if (jp == 1) { __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, 0); __builtin_amdgcn_sched_barrier(0); }
-                            if (jp == 2) { __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, 1); __builtin_amdgcn_sched_barrier(0); }
+                            if (jp == 3) { __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, 0); decode_one(buf ^ 1, 1); __builtin_amdgcn_sched_barrier(0); }
                         } else {
                             __builtin_amdgcn_sched_barrier(0); decode_one(buf ^ 1, jp); __builtin_amdgcn_sched_barrier(0);
                         }

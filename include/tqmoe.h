@@ -288,6 +288,37 @@ int32_t tqmoe_expert_gemm_gateup_i8(const tqmoe_bank * gate, const tqmoe_bank * 
 int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const int32_t * counts,
                              const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk,
                              int32_t shared_lim, void * y_f16, void * stream, tqmoe_error * err);
+/* The same steps with a scale per 32 values of every input row in place of one per row: the per-32-block mode of the
+ * reference's activation quantiser and of expert_gemm_i8 (k_quant_act_rows / k_expert_gemm_i8 mode 1,
+ * src/formats/weight/quant_kernels.cuh:13-19; quant_act_rows_k<false> and u4h_i8_gemm_k<.., TOKEN = false>,
+ * quant_u4h.inc:790-822, 849-935), which isolates an outlier to its block. A block's product is an exact integer sum
+ * that is scaled by the weights' scale and the row's block scale before it joins the fp32 result, as in the reference.
+ * tqmoe_quant_rows_i8_blocks: q as tqmoe_quant_rows_i8, scales fp32 [rows][cols / 32] (amax of the block / 127), qsum
+ * int16 [rows][cols / 32][2] = the sums of q over each 16 values (the reference's xsum; may be null: the products here
+ * take the weights' minimum term from a matrix product of their own and do not read it).
+ * tqmoe_group_rows_i8_blocks / tqmoe_gather_rows_i8_blocks: q / scale as above (every row scale 1) and block_scale, device
+ * fp32, tqmoe_grouped_block_scale_words(assignments, experts, cols) words ([row tile][cols / 32][32 rows]).
+ * tqmoe_expert_gemm_gateup_i8_blocks / tqmoe_expert_gemm_i8_blocks: the two products on such rows; int8 formats only. */
+int32_t tqmoe_quant_rows_i8_blocks(const void * x, uint32_t xtype, int64_t rows, int32_t cols, int8_t * q, float * scales,
+                                   int16_t * qsum, void * stream, tqmoe_error * err);
+int64_t tqmoe_grouped_block_scale_words(int64_t assignments, int32_t experts, int32_t cols);
+int32_t tqmoe_group_rows_i8_blocks(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts,
+                                   const int32_t * offsets, const int32_t * perm, int32_t experts, int64_t assignments,
+                                   int32_t xdiv, int8_t * q, float * scale, float * block_scale, void * stream,
+                                   tqmoe_error * err);
+int32_t tqmoe_gather_rows_i8_blocks(const int8_t * rows_q, const float * rows_scales, int32_t cols, const int32_t * counts,
+                                    const int32_t * offsets, const int32_t * perm, int32_t experts, int64_t assignments,
+                                    int32_t xdiv, int8_t * q, float * scale, float * block_scale, void * stream,
+                                    tqmoe_error * err);
+int32_t tqmoe_expert_gemm_gateup_i8_blocks(const tqmoe_bank * gate, const tqmoe_bank * up, const int8_t * xq,
+                                           const float * xs, const float * block_scale, const int32_t * counts,
+                                           const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots,
+                                           int32_t topk, int32_t shared_lim, void * act_f16, void * stream,
+                                           tqmoe_error * err);
+int32_t tqmoe_expert_gemm_i8_blocks(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const float * block_scale,
+                                    const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t n,
+                                    int32_t slots, int32_t topk, int32_t shared_lim, void * y_f16, void * stream,
+                                    tqmoe_error * err);
 /* The E4M3 form of the same steps for NVFP4G banks (fp8 x fp8 -> fp32 on the matrix cores): the input rows as E4M3 with
  * one scale per row, amax / 448 (the reference's fp8_quant_rows, src/core/fp8_gemm.cuh:19-31: scales applied after the
  * product); the weights widened to E4M3 bytes, e2m1 * (E4M3 scale of the 16 weights) / 8 rounded to nearest even (a

@@ -63,6 +63,8 @@ _lib.tqo_combine.argtypes = [C.c_int, _p, _p, C.c_int, _p]
 _lib.tqo_router_logits.argtypes = [_p, C.c_uint32, _p, _p, C.c_uint32, C.c_int, C.c_int, C.c_int, _p]
 _lib.tqo_quant_act_row_i8.restype = None
 _lib.tqo_quant_act_row_i8.argtypes = [_p, C.c_int, _p, _p]
+_lib.tqo_quant_act_blocks_i8.restype = None
+_lib.tqo_quant_act_blocks_i8.argtypes = [_p, C.c_int, _p, _p, _p]
 _lib.tqo_dequantize_nvfp4_widened.restype = C.c_int
 _lib.tqo_dequantize_nvfp4_widened.argtypes = [_p, _p, C.c_int64]
 _lib.tqo_quant_act_row_e4m3.restype = None
@@ -215,6 +217,16 @@ def quant_act_row_i8(x):
     s = np.empty(1, np.float32)
     _lib.tqo_quant_act_row_i8(_ptr(x), x.size, _ptr(q), _ptr(s))
     return q, float(s[0])
+
+
+def quant_act_blocks_i8(x):
+    """(q int8 [cols], scales fp32 [cols / 32], sums of q per 16 int16 [cols / 32][2])"""
+    x = _c(x, np.float32)
+    q = np.empty(x.size, np.int8)
+    s = np.empty(x.size // 32, np.float32)
+    qsum = np.empty((x.size // 32, 2), np.int16)
+    _lib.tqo_quant_act_blocks_i8(_ptr(x), x.size, _ptr(q), _ptr(s), _ptr(qsum))
+    return q, s, qsum
 
 
 def quant_act_row_e4m3(x):

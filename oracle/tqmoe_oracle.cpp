@@ -920,6 +920,20 @@ void tqo_quant_act_row_i8(const float * x, int cols, int8_t * q, float * scale) 
     for (int i = 0; i < cols; ++i) q[i] = int8_t(std::nearbyint(x[i] * mul));
 }
 
+// reference: quant_act_rows_k<false> (src/formats/weight/quant_u4h.inc:790-822): a scale per 32 values (amax / 127 of the
+// block), q = rint(x * (127 / amax)), and the sum of q over each half of 16 (the weights' "min" term of the int8 products)
+void tqo_quant_act_blocks_i8(const float * x, int cols, int8_t * q, float * scales, int16_t * qsum) {
+    for (int b = 0; b < cols / 32; ++b) {
+        tqo_quant_act_row_i8(x + 32 * b, 32, q + 32 * b, scales + b);
+        if (qsum)
+            for (int h = 0; h < 2; ++h) {
+                int sum = 0;
+                for (int i = 0; i < 16; ++i) sum += q[32 * b + 16 * h + i];
+                qsum[2 * b + h] = int16_t(sum);
+            }
+    }
+}
+
 void tqo_quant_act_row_e4m3(const float * x, int cols, uint8_t * q, float * scale) {
     float m = 0.f;
     for (int i = 0; i < cols; ++i) m = std::max(m, std::fabs(x[i]));
@@ -944,7 +958,11 @@ void requant_row_e4m3(float * x, int cols) {  // x <- dequantised per-row E4M3 i
     tqo_quant_act_row_e4m3(x, cols, q.data(), &s);
     for (int i = 0; i < cols; ++i) x[i] = tqo_e4m3_to_float(q[size_t(i)]) * s;
 }
-void requant_row(int act_mode, float * x, int cols) { if (act_mode == 2) requant_row_e4m3(x, cols); else requant_row_i8(x, cols); }
+void requant_row(int act_mode, float * x, int cols) {
+    if (act_mode == 2) requant_row_e4m3(x, cols);
+    else if (act_mode == 6) for (int b = 0; b < cols / 32; ++b) requant_row_i8(x + 32 * b, 32);   // a scale per 32 values
+    else requant_row_i8(x, cols);
+}
 // act_mode 2 reads the banks as the fp8 products do
 int decode_weights(const tqo_layer & L, uint32_t type, const void * src, float * dst, int64_t n) {
     return L.act_mode == 2 ? tqo_dequantize_nvfp4_widened(src, dst, n) : tqo_dequantize(type, src, dst, n);
@@ -986,7 +1004,7 @@ void ffn_mode(const tqo_layer & L, const float * x, const Decoded & d, int ff, f
         for (int i = 0; i < L.hidden; ++i) { g += wg[i] * x[i]; u += wu[i] * x[i]; }
         act[size_t(o)] = (g / (1.f + std::exp(-g))) * u;
     }
-    const bool f16 = L.act_mode == 5 || L.act_mode == 2;   // the grouped products keep act and y as fp16 rows
+    const bool f16 = L.act_mode == 5 || L.act_mode == 2 || L.act_mode == 6;   // the grouped products keep act and y as fp16 rows
     if (f16) for (float & v : act) v = tqo_half_to_float(tqo_float_to_half(v));
     requant_row(L.act_mode, act.data(), ff);
     for (int i = 0; i < L.hidden; ++i) {
@@ -1005,7 +1023,8 @@ int tqo_layer_forward(const tqo_layer * Lp, const float * x, const float * logit
     int elems, bytes;
     if (!tqo_block_layout(L.wtype, &elems, &bytes)) return -1;
     if (L.hidden % elems || L.ff % elems || n <= 0 || L.k <= 0 || L.k > L.n_expert) return -1;
-    if (L.act_mode != 0 && L.act_mode != 1 && L.act_mode != 2 && L.act_mode != 5) return -1;
+    if (L.act_mode != 0 && L.act_mode != 1 && L.act_mode != 2 && L.act_mode != 5 && L.act_mode != 6) return -1;
+    if (L.act_mode == 6 && (L.hidden % 32 || L.ff % 32 || (L.has_shared && L.shared_ff % 32))) return -1;
     if (L.act_mode == 2 && (L.wtype != TQO_NVFP4G || (L.wtype_down && L.wtype_down != TQO_NVFP4G))) return -1;
     if (L.has_shared && (L.shared_ff <= 0 || L.shared_ff > L.ff || L.shared_ff % elems)) return -1;
     const int E = L.n_expert, K = L.k, A = n * K, H = L.hidden;

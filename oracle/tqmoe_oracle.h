@@ -37,6 +37,8 @@
  *   tqo_layer_forward                      tests/glm_expert_bank.cu:166-184 (dequantise, route, FFN per selected
  *                                          expert, combine)
  *   tqo_quant_act_row_i8                   src/formats/weight/quant_u4h.inc:790-820 (per-token mode: scale m/127)
+ *   tqo_quant_act_blocks_i8                src/formats/weight/quant_u4h.inc:790-822 (per-32-block mode: a scale and two
+ *                                          sums of 16 per block)
  *   tqo_quant_act_row_e4m3                 src/core/fp8_gemm.cuh:19-20 (per-row scale amax/448)
  *
  * Pinned by: tests/golden/kquant_golden.bin (gguf-py values, bit for bit) for Q4_K / IQ3_S / IQ4_XS / IQ4_NL; the
@@ -113,6 +115,8 @@ int tqo_router_logits(const void * w, uint32_t wtype, const void * shared_gate, 
 /* Declared activation quantisers of the lossy operand paths. */
 void tqo_quant_act_row_i8(const float * x, int cols, int8_t * q, float * scale);     /* scale = amax/127 */
 void tqo_quant_act_row_e4m3(const float * x, int cols, uint8_t * q, float * scale);  /* scale = amax/448 */
+/* a scale per 32 values (scales[cols / 32]) and the sums of q over each 16 (qsum[cols / 32][2], may be null); cols a multiple of 32 */
+void tqo_quant_act_blocks_i8(const float * x, int cols, int8_t * q, float * scales, int16_t * qsum);
 /* NVFP4G blocks -> fp32 with e2m1 * (E4M3 scale) / 8 rounded to E4M3 before 8 * the row's global multiplies it: the
  * weights of an fp8 matrix product that keeps the global outside the operand (the 8 keeps 6 * 448 inside E4M3). n a
  * multiple of 128. */
@@ -134,7 +138,8 @@ int tqo_add_rmsnorm(uint16_t * rows, const uint16_t * residual, const float * we
  *   act_mode: 0 = fp32 activations (oracle A); 1 = the inputs of both products (the token row, the act row) passed
  *   through tqo_quant_act_row_i8 (oracle B of an int8 path that keeps fp32 intermediate rows); 5 = mode 1 with
  *   silu(gate) * up and the down product each rounded to fp16 (oracle B of the grouped int8 products, which store
- *   fp16 rows); 2 = NVFP4G banks on fp8 operands (oracle B of the grouped fp8 products): both product inputs passed
+ *   fp16 rows); 6 = mode 5 with a scale per 32 values in place of one per row (tqo_quant_act_blocks_i8: the reference's
+ *   per-32-block mode of the same products); 2 = NVFP4G banks on fp8 operands (oracle B of the grouped fp8 products): both product inputs passed
  *   through tqo_quant_act_row_e4m3, the weights through tqo_dequantize_nvfp4_widened, fp16 roundings as in mode 5.
  *   out fp32 [n][H]; ids_out [n][k], weights_out [n][k] may be null. threads: worker threads over tokens.
  *   gating (0 = softmax), raw_weights (nonzero: unnormalised), weight_scale (0 = none) and bias (or null) are

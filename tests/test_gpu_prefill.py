@@ -164,6 +164,119 @@ def test_grouped_products_against_float64(tq, oracle, n, shared_ff, wtype):
         assert np.abs(y[a] - want).max() < 2e-3 * max(1e-3, np.abs(want).max()), a
 
 
+def ungroup_block_scales(bs, counts, perm, assignments, blocks):
+    """block scales [row tile][block][32 rows] -> [assignments][blocks]"""
+    t = bs.reshape(-1, blocks, 32).transpose(0, 2, 1).reshape(-1, blocks)     # [tile * 32 + r][blocks]
+    out = np.zeros((assignments, blocks), np.float32)
+    base, at = 0, 0
+    for c in counts:
+        for i in range(c):
+            out[perm[at + i]] = t[base * 32 + i]
+        at += c
+        base += (c + 31) // 32
+    return out
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16", "f16"])
+def test_quant_rows_i8_blocks_bit_exact(tq, oracle, kind):
+    """A scale per 32 values and the sums per 16 (the reference's k_quant_act_rows mode 1) against the oracle's
+    quantiser, bit for bit; blocks whose magnitudes differ a thousandfold, a zero block and a zero row among them."""
+    rng = np.random.default_rng(8)
+    rows, cols = 37, 768
+    x = rng.standard_normal((rows, cols)).astype(np.float32) * np.repeat(rng.uniform(0.01, 30, (rows, cols // 32)), 32, axis=1).astype(np.float32)
+    x[7] = 0
+    x[9, 64:96] = 0
+    t = torch.from_numpy(x).cuda().to({"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[kind])
+    xv = t.float().cpu().numpy()
+    qd, sd, qsum = tq.quant_rows_i8_blocks(t)
+    q, s, qsum = natural_order(qd.cpu().numpy()), sd.cpu().numpy(), qsum.cpu().numpy()
+    for r in range(rows):
+        wq, ws, wsum = oracle.quant_act_blocks_i8(xv[r])
+        assert np.array_equal(q[r], wq), r
+        assert np.array_equal(s[r], ws), r
+        assert np.array_equal(qsum[r], wsum), r
+    q2, s2, none = tq.quant_rows_i8_blocks(t, sums=False)
+    assert none is None and torch.equal(q2, qd) and torch.equal(s2, sd)
+
+
+BLOCK_FORMATS = [f for f in PLANE_FORMATS if f != "NVFP4G"]
+
+
+@pytest.mark.parametrize("wtype", BLOCK_FORMATS)
+@pytest.mark.parametrize("n,shared_ff", [(3, 0), (70, 256), (300, 512)])
+def test_grouped_products_block_scales_against_float64(tq, oracle, n, shared_ff, wtype):
+    """The two products on rows with a scale per 32 values against float64 on the decoded weights and the dequantised rows
+    (the integer sum of a block is exact; fp32 scaling and accumulation over the blocks and the fp16 store separate the
+    two). The inputs have blocks of very different magnitude, where the per-row quantiser loses the small blocks: its
+    products must be measurably farther from the fp32 activations than these."""
+    experts, ff, hidden, k = 7, 512, 768, 3
+    wt = getattr(oracle, wtype)
+    decs, (gate, up, down), ids, slots, banks = grouped_setup(tq, oracle, 31 + n, experts, ff, hidden, n, k, shared_ff > 0, wt)
+    rng = np.random.default_rng(100 + n)
+    xf = rng.standard_normal((n, hidden)).astype(np.float32) * np.repeat(10.0 ** rng.uniform(-2, 1, (n, hidden // 32)), 32, axis=1).astype(np.float32)
+    xb, xv = oracle.to_bf16(xf)
+    x = torch.from_numpy(xb.view(np.int16)).cuda().view(torch.bfloat16)
+    counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), banks)
+    want_counts = np.bincount(ids.reshape(-1), minlength=banks)
+    lists = (counts, offsets, perm)
+    xq, xs, xbs = tq.group_rows_i8_blocks(x, lists, n * slots, slots)
+    # the grouped rows are the plain block quantiser's rows, gathered, and so are the gathered quantised rows
+    pq, ps, _ = tq.quant_rows_i8_blocks(x, sums=False)
+    uq, us = ungroup(xq.cpu().numpy(), xs.cpu().numpy(), want_counts, perm.cpu().numpy(), n * slots)
+    ub = ungroup_block_scales(xbs.cpu().numpy(), want_counts, perm.cpu().numpy(), n * slots, hidden // 32)
+    tok = np.arange(n * slots) // slots
+    assert np.array_equal(uq, natural_order(pq.cpu().numpy())[tok])
+    assert np.array_equal(ub, ps.cpu().numpy()[tok]) and (us == 1).all()
+    gq, gs, gbs = tq.gather_rows_i8_blocks(pq, ps, lists, n * slots, slots)
+    live = np.zeros(xq.shape[0], bool)
+    base = 0
+    for c in want_counts:
+        live[base * 32:base * 32 + c] = True
+        base += (c + 31) // 32
+    assert np.array_equal(gq.cpu().numpy()[live], xq.cpu().numpy()[live])
+    assert np.array_equal(ungroup_block_scales(gbs.cpu().numpy(), want_counts, perm.cpu().numpy(), n * slots, hidden // 32), ub)
+    act = tq.expert_gemm_gateup_i8_blocks(gate, up, xq, xs, xbs, lists, n, slots, k, shared_ff)
+    xd = natural_order(pq.cpu().numpy()).astype(np.float64) * np.repeat(ps.cpu().numpy().astype(np.float64), 32, axis=1)
+    got = act.float().cpu().numpy()
+    act_rows = tq.expert_gemm_gateup_i8(gate, up, *tq.group_rows_i8(x, lists, n * slots, slots), lists, n, slots, k, shared_ff).float().cpu().numpy()
+    err_blocks = err_rows = 0.0
+    for a in range(n * slots):
+        e = ids.reshape(-1)[a]
+        lim = shared_ff if (shared_ff and e == experts) else ff
+        g = decs[0][e][:lim] @ xd[a // slots]
+        u = decs[1][e][:lim] @ xd[a // slots]
+        want = g / (1 + np.exp(-g)) * u
+        assert np.abs(got[a, :lim] - want).max() < 2e-3 * max(1.0, np.abs(want).max()), a
+        assert not got[a, lim:].any()
+        g, u = decs[0][e][:lim] @ xv[a // slots].astype(np.float64), decs[1][e][:lim] @ xv[a // slots].astype(np.float64)
+        exact = g / (1 + np.exp(-g)) * u
+        err_blocks += np.square(got[a, :lim] - exact).sum()
+        err_rows += np.square(act_rows[a, :lim] - exact).sum()
+    assert err_blocks < 0.5 * err_rows, (err_blocks, err_rows)
+    aq, a_s, abs_ = tq.group_rows_i8_blocks(act, lists, n * slots, 1)
+    y = tq.expert_gemm_i8_blocks(down, aq, a_s, abs_, lists, n, slots, k, shared_ff).float().cpu().numpy()
+    pq, ps, _ = tq.quant_rows_i8_blocks(act, sums=False)
+    ad = natural_order(pq.cpu().numpy()).astype(np.float64) * np.repeat(ps.cpu().numpy().astype(np.float64), 32, axis=1)
+    for a in range(n * slots):
+        e = ids.reshape(-1)[a]
+        lim = shared_ff if (shared_ff and e == experts) else ff
+        want = decs[2][e][:, :lim] @ ad[a, :lim]
+        assert np.abs(y[a] - want).max() < 2e-3 * max(1e-3, np.abs(want).max()), a
+
+
+def test_block_scale_products_refuse_fp8_banks_and_missing_scales(tq, oracle):
+    decs, (gate, up, down), ids, slots, banks = grouped_setup(tq, oracle, 3, 4, 256, 256, 8, 2, False, oracle.NVFP4G)
+    counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), banks)
+    lists = (counts, offsets, perm)
+    x = torch.randn(8, 256, device="cuda", dtype=torch.bfloat16)
+    xq, xs, xbs = tq.group_rows_i8_blocks(x, lists, 8 * slots, slots)
+    with pytest.raises(Exception, match="int8"):
+        tq.expert_gemm_gateup_i8_blocks(gate, up, xq, xs, xbs, lists, 8, slots, 2, 0)
+    decs, (gate, up, down), ids, slots, banks = grouped_setup(tq, oracle, 3, 4, 256, 256, 8, 2, False, oracle.IQ4_XS)
+    with pytest.raises(Exception, match="block scales"):
+        tq.expert_gemm_i8_blocks(down, xq, xs, None, lists, 8, slots, 2, 0)
+
+
 def grouped_products_fp8(tq, oracle, decs, gate, up, down, ids, slots, banks, n, k, shared_ff, experts, ff, hidden):
     rng = np.random.default_rng(n)
     xb, xv = oracle.to_bf16(rng.standard_normal((n, hidden)).astype(np.float32))

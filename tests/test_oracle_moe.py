@@ -434,6 +434,75 @@ def test_layer_forward_lossy_operand_modes_against_float64(oracle):
         assert (np.abs(a - want) > tol).mean() > 0.5
 
 
+def _requant_blocks_i8(v):
+    """float64 restatement of the per-32-block int8 quantiser: _requant_i8 on every 32 values"""
+    v = np.asarray(v, np.float64)
+    return np.concatenate([_requant_i8(v[i:i + 32]) for i in range(0, v.size, 32)])
+
+
+def test_block_quantiser_and_layer_mode(oracle):
+    """tqo_quant_act_blocks_i8: every 32 values are the per-row quantiser's result on those 32 alone (pinned above), the
+    sums are the integer sums of each half; an input that is a multiple of its block's scale survives exactly. act_mode 6
+    of tqo_layer_forward rebuilt in float64 numpy as mode 5 with that quantiser; the rebuild with per-row scales, or with a
+    step left out, must be far from it."""
+    rng = np.random.default_rng(41)
+    x = (rng.standard_normal(256) * np.repeat(rng.uniform(0.01, 50, 8), 32)).astype(np.float32)
+    x[64:96] = 0
+    q, s, qsum = oracle.quant_act_blocks_i8(x)
+    for b in range(8):
+        wq, ws = oracle.quant_act_row_i8(x[32 * b:32 * b + 32])
+        assert np.array_equal(q[32 * b:32 * b + 32], wq) and s[b] == np.float32(ws)
+        assert qsum[b, 0] == int(wq[:16].astype(np.int32).sum()) and qsum[b, 1] == int(wq[16:].astype(np.int32).sum())
+    assert s[2] == 0 and not q[64:96].any()
+    # the extreme sums fit int16 (16 * 127), and integers times a power of two come back exactly
+    q1, s1, qs1 = oracle.quant_act_blocks_i8(np.full(32, -3.0, np.float32))
+    assert (q1 == -127).all() and qs1[0, 0] == -2032 and qs1[0, 1] == -2032
+    ints = rng.integers(-127, 128, 64).astype(np.float32)
+    ints[0], ints[32] = 127, -127
+    q2, s2, _ = oracle.quant_act_blocks_i8(ints * np.float32(0.25))
+    assert np.array_equal(q2.astype(np.float32), ints) and (s2 == np.float32(0.25)).all()
+
+    h, f, e, k, n = 256, 256, 6, 2, 6
+    for wtype, sf in ((oracle.IQ4_XS, 256), (oracle.Q4_K, 0)):
+        banks = [oracle.quantize(wtype, (rng.standard_normal(((e + 1) * r, c)) * 0.05).astype(np.float32))
+                 for r, c in ((f, h), (f, h), (h, f))]
+        dec = [oracle.dequantize(wtype, b, (e + 1) * f * h).astype(np.float64) for b in banks]
+        wg, wu, wd = dec[0].reshape(e + 1, f, h), dec[1].reshape(e + 1, f, h), dec[2].reshape(e + 1, h, f)
+        xs = (rng.standard_normal((n, h)) * np.repeat(rng.uniform(0.05, 4, (n, h // 32)), 32, axis=1)).astype(np.float32)
+        logits = rng.standard_normal((n, e + 1)).astype(np.float32)
+        got, ids, w = oracle.layer_forward(xs, logits, *banks, wtype, h, f, e, k, shared_ff=sf, act_mode=6, threads=3)
+
+        def rebuild(skip=None):
+            out = np.zeros((n, h))
+            rq = _requant_i8 if skip == "rows" else _requant_blocks_i8
+            for t in range(n):
+                xq = rq(xs[t]) if skip != "x" else xs[t].astype(np.float64)
+
+                def ffn(j, ff):
+                    g, u = wg[j, :ff] @ xq, wu[j, :ff] @ xq
+                    act = g / (1 + np.exp(-g)) * u
+                    if skip != "act16":
+                        act = _half(act)
+                    if skip != "act":
+                        act = rq(act)
+                    y = wd[j, :, :ff] @ act
+                    return _half(y) if skip != "y16" else y
+
+                out[t] = sum(float(w[t, s]) * ffn(ids[t, s], f) for s in range(k))
+                if sf:
+                    out[t] += 1 / (1 + np.exp(-float(logits[t, e]))) * ffn(e, sf)
+            return out
+
+        want = rebuild()
+        tol = 2e-5 * max(1.0, np.abs(want).max())
+        off = np.abs(got - want) > tol
+        # (eight times the quantiser's roundings per row: more values on a rounding boundary fall the other way in fp32)
+        assert off.mean() < 0.08, (wtype, off.mean())
+        assert np.abs(got - want).max() < 5e-4 * np.abs(want).max(), wtype
+        for skip in ("rows", "x", "act", "act16", "y16"):
+            assert (np.abs(got - rebuild(skip)) > tol).mean() > 0.3, (wtype, skip)
+
+
 def test_cpu_baseline_kernels_agree_with_decode(oracle, ref):
     """The CPU-baseline matvecs, row by row, with the gates of the reference's tests/test_cpu_expert_matvec.cpp:117-118, 178-195:
     fp32 variant vs decode + float64 dot rms-rel <= 1e-5; int8 variant <= 1e-2; and the AVX2 integer dots against the scalar

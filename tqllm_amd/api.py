@@ -98,6 +98,13 @@ def lib():
         l.tqmoe_gather_rows_i8.argtypes = [p, p, i32, p, p, p, i32, i64, i32, p, p, p, e]
         l.tqmoe_expert_gemm_gateup_i8.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_expert_gemm_i8.argtypes = [C.POINTER(_Bank), p, p, p, p, p, i32, i32, i32, i32, p, p, e]
+        l.tqmoe_quant_rows_i8_blocks.argtypes = [p, u32, i64, i32, p, p, p, p, e]
+        l.tqmoe_grouped_block_scale_words.restype = i64
+        l.tqmoe_grouped_block_scale_words.argtypes = [i64, i32, i32]
+        l.tqmoe_group_rows_i8_blocks.argtypes = [p, u32, i32, p, p, p, i32, i64, i32, p, p, p, p, e]
+        l.tqmoe_gather_rows_i8_blocks.argtypes = [p, p, i32, p, p, p, i32, i64, i32, p, p, p, p, e]
+        l.tqmoe_expert_gemm_gateup_i8_blocks.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, p, p, p, p, p, i32, i32, i32, i32, p, p, e]
+        l.tqmoe_expert_gemm_i8_blocks.argtypes = [C.POINTER(_Bank), p, p, p, p, p, p, i32, i32, i32, i32, p, p, e]
         l.tqmoe_quant_rows_fp8.argtypes = l.tqmoe_quant_rows_i8.argtypes
         l.tqmoe_group_rows_fp8.argtypes = l.tqmoe_group_rows_i8.argtypes
         l.tqmoe_expert_gemm_gateup_fp8.argtypes = l.tqmoe_expert_gemm_gateup_i8.argtypes
@@ -357,6 +364,52 @@ def quant_rows_fp8(x):
     return quant_rows_i8(x, fp8=True)
 
 
+def quant_rows_i8_blocks(x, sums=True):
+    """Int8 activations with a scale per 32 values (k_quant_act_rows mode 1, quant_kernels.cuh:17-19; quant_u4h.inc:790-822):
+    (q int8 [rows][cols] in the library's byte order, scales fp32 [rows][cols / 32], sums of q per 16 values int16
+    [rows][cols / 32][2] or None)."""
+    rows, cols = x.shape
+    q = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
+    scales = torch.empty((rows, cols // 32), dtype=torch.float32, device=x.device)
+    qsum = torch.empty((rows, cols // 32, 2), dtype=torch.int16, device=x.device) if sums else None
+    err = _err()
+    _check(lib().tqmoe_quant_rows_i8_blocks(_ptr(x), _ttype(x), rows, cols, _ptr(q), _ptr(scales), _ptr(qsum) if sums else None, _stream(x), C.byref(err)), err)
+    return q, scales, qsum
+
+
+def _block_scales(assignments, experts, cols, device):
+    return torch.zeros(lib().tqmoe_grouped_block_scale_words(assignments, experts, cols), dtype=torch.float32, device=device)
+
+
+def group_rows_i8_blocks(x, lists, assignments, xdiv):
+    """group_rows_i8 with a scale per row and 32 values: (q, scale, block_scale); block_scale is fp32
+    [row tiles][cols / 32][32 rows], the rows' own scales in `scale` are 1."""
+    counts, offsets, perm = lists
+    cols = x.shape[1]
+    rows = lib().tqmoe_grouped_rows(assignments, counts.numel())
+    q = torch.zeros((rows, cols), dtype=torch.int8, device=x.device)
+    scale = torch.zeros(lib().tqmoe_grouped_scale_words(assignments, counts.numel()), dtype=torch.float32, device=x.device)
+    bs = _block_scales(assignments, counts.numel(), cols, x.device)
+    err = _err()
+    _check(lib().tqmoe_group_rows_i8_blocks(_ptr(x), _ttype(x), cols, _ptr(counts), _ptr(offsets), _ptr(perm), counts.numel(), assignments, xdiv, _ptr(q),
+                                            _ptr(scale), _ptr(bs), _stream(x), C.byref(err)), err)
+    return q, scale, bs
+
+
+def gather_rows_i8_blocks(rows_q, rows_scales, lists, assignments, xdiv):
+    """The arranging step of group_rows_i8_blocks alone, from rows quant_rows_i8_blocks has quantised."""
+    counts, offsets, perm = lists
+    cols = rows_q.shape[1]
+    rows = lib().tqmoe_grouped_rows(assignments, counts.numel())
+    q = torch.zeros((rows, cols), dtype=torch.int8, device=rows_q.device)
+    scale = torch.zeros(lib().tqmoe_grouped_scale_words(assignments, counts.numel()), dtype=torch.float32, device=rows_q.device)
+    bs = _block_scales(assignments, counts.numel(), cols, rows_q.device)
+    err = _err()
+    _check(lib().tqmoe_gather_rows_i8_blocks(_ptr(rows_q), _ptr(rows_scales), cols, _ptr(counts), _ptr(offsets), _ptr(perm), counts.numel(), assignments, xdiv,
+                                             _ptr(q), _ptr(scale), _ptr(bs), _stream(rows_q), C.byref(err)), err)
+    return q, scale, bs
+
+
 def group_rows_i8(x, lists, assignments, xdiv, fp8=False):
     """Per-row int8 quantisation of the input row (a // xdiv) of every listed assignment a, gathered expert by expert into
     the operand-major row tiles the grouped products read (mmq_quantize_act_rows, mmq_experts.cu:79-95, in role):
@@ -447,6 +500,28 @@ def expert_gemm_i8(bank, xq, xs, lists, n, slots, topk, shared_ff=0, fp8=False):
 
 def expert_gemm_fp8(bank, xq, xs, lists, n, slots, topk, shared_ff=0):
     return expert_gemm_i8(bank, xq, xs, lists, n, slots, topk, shared_ff, fp8=True)
+
+
+def expert_gemm_gateup_i8_blocks(gate, up, xq, xs, block_scale, lists, n, slots, topk, shared_ff=0):
+    """expert_gemm_gateup_i8 on rows with a scale per 32 values (expert_gemm_i8's mode 1, quant_kernels.cuh:13-16)."""
+    counts, offsets, perm = lists
+    act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=xq.device)
+    err = _err()
+    g, u = gate.view(), up.view()
+    _check(lib().tqmoe_expert_gemm_gateup_i8_blocks(C.byref(g), C.byref(u), _ptr(xq), _ptr(xs), _ptr(block_scale), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots,
+                                                    topk, shared_ff, _ptr(act), _stream(xq), C.byref(err)), err)
+    return act
+
+
+def expert_gemm_i8_blocks(bank, xq, xs, block_scale, lists, n, slots, topk, shared_ff=0):
+    """WeightFormat::expert_gemm_i8 (weight_format.hpp:54-56) with a scale per 32 values of the input rows (mode 1)."""
+    counts, offsets, perm = lists
+    y = torch.zeros((n * slots, bank.rows), dtype=torch.float16, device=xq.device)
+    err = _err()
+    b = bank.view()
+    _check(lib().tqmoe_expert_gemm_i8_blocks(C.byref(b), _ptr(xq), _ptr(xs), _ptr(block_scale), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff,
+                                             _ptr(y), _stream(xq), C.byref(err)), err)
+    return y
 
 
 def moe_swiglu(gate, up):

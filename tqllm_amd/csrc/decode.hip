@@ -10,14 +10,16 @@ int32_t enqueue_gemm_f16(const tqmoe_bank & b0, const tqmoe_bank * b1, const voi
                          int experts, int64_t assignments, int xdiv, void * out, uint32_t out_type, int gateup, int shared_expert, int shared_lim, hipStream_t s);
 int64_t grouped_row_tiles(int64_t assignments, int experts);
 int64_t grouped_scale_words(int64_t assignments, int experts);
+int32_t enqueue_quant_rows_i8_blocks(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, int16_t * qsum, hipStream_t s);
 int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, const int * counts, const int * offsets, const int * perm, int experts,
-                               int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s);
+                               int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, float * block_scale);
 int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
-                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8);
+                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8, float * block_scale);
 bool plane_gemm_has(uint32_t type);
 bool plane_gemm_is_fp8(uint32_t type);
 int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
-                           const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s);
+                           const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s,
+                           const float * xbs);
 
 namespace {
 
@@ -360,6 +362,20 @@ extern "C" int32_t tqmoe_quant_rows_fp8(const void * x, uint32_t xtype, int64_t 
     return quant_rows_common(x, xtype, rows, cols, q, scale, stream, err, true, "tqmoe_quant_rows_fp8");
 }
 
+extern "C" int32_t tqmoe_quant_rows_i8_blocks(const void * x, uint32_t xtype, int64_t rows, int32_t cols, int8_t * q, float * scales, int16_t * qsum, void * stream,
+                                              tqmoe_error * err) {
+    const char * what = "tqmoe_quant_rows_i8_blocks";
+    if (!x || !q || !scales || rows <= 0 || cols <= 0 || cols % 32 || (rows + 3) / 4 > 0x7FFFFFFF) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported element type", what);
+    if (int32_t rc = need_device(err, what)) return rc;
+    enqueue_quant_rows_i8_blocks(x, xtype, rows, cols, q, scales, qsum, static_cast<hipStream_t>(stream));
+    return launched(err, what);
+}
+
+extern "C" int64_t tqmoe_grouped_block_scale_words(int64_t assignments, int32_t experts, int32_t cols) {
+    return assignments > 0 && experts > 0 && cols > 0 && cols % 32 == 0 ? grouped_row_tiles(assignments, experts) * 32 * (cols / 32) : 0;
+}
+
 extern "C" int64_t tqmoe_grouped_rows(int64_t assignments, int32_t experts) {
     return assignments > 0 && experts > 0 ? grouped_row_tiles(assignments, experts) * 32 : 0;
 }
@@ -369,14 +385,23 @@ extern "C" int64_t tqmoe_grouped_scale_words(int64_t assignments, int32_t expert
 }
 
 static int32_t group_rows_common(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t experts,
-                                 int64_t assignments, int32_t xdiv, void * q, float * scale, void * stream, tqmoe_error * err, bool f8, const char * what) {
+                                 int64_t assignments, int32_t xdiv, void * q, float * scale, void * stream, tqmoe_error * err, bool f8, const char * what,
+                                 float * block_scale = nullptr, bool blocks = false) {
+    if (blocks && !block_scale) return fail(err, TQMOE_E_ARG, "%s: block scales missing", what);
     if (!x || !counts || !offsets || !perm || !q || !scale || cols <= 0 || cols % 32 || experts <= 0 || experts > 4096 || assignments <= 0 || xdiv <= 0 ||
         grouped_row_tiles(assignments, experts) > 0x7FFFFFFF)
         return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
     if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported element type", what);
     if (int32_t rc = need_device(err, what)) return rc;
-    enqueue_group_rows_i8(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, static_cast<int8_t *>(q), scale, static_cast<hipStream_t>(stream), f8);
+    enqueue_group_rows_i8(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, static_cast<int8_t *>(q), scale, static_cast<hipStream_t>(stream), f8,
+                          block_scale);
     return launched(err, what);
+}
+
+extern "C" int32_t tqmoe_group_rows_i8_blocks(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm,
+                                              int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q, float * scale, float * block_scale, void * stream,
+                                              tqmoe_error * err) {
+    return group_rows_common(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, stream, err, false, "tqmoe_group_rows_i8_blocks", block_scale, true);
 }
 
 extern "C" int32_t tqmoe_group_rows_i8(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm,
@@ -389,20 +414,34 @@ extern "C" int32_t tqmoe_group_rows_fp8(const void * x, uint32_t xtype, int32_t 
     return group_rows_common(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, stream, err, true, "tqmoe_group_rows_fp8");
 }
 
+static int32_t gather_rows_common(const int8_t * rows_q, const float * rows_scale, int32_t cols, const int32_t * counts, const int32_t * offsets,
+                                  const int32_t * perm, int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q, float * scale, float * block_scale,
+                                  bool blocks, void * stream, tqmoe_error * err, const char * what) {
+    if (!rows_q || !rows_scale || !counts || !offsets || !perm || !q || !scale || (blocks && !block_scale) || cols <= 0 || cols % 32 || experts <= 0 ||
+        experts > 4096 || assignments <= 0 || xdiv <= 0 || grouped_row_tiles(assignments, experts) > 0x7FFFFFFF)
+        return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    if (int32_t rc = need_device(err, what)) return rc;
+    enqueue_gather_rows_i8(rows_q, rows_scale, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, static_cast<hipStream_t>(stream), block_scale);
+    return launched(err, what);
+}
+
 extern "C" int32_t tqmoe_gather_rows_i8(const int8_t * rows_q, const float * rows_scale, int32_t cols, const int32_t * counts, const int32_t * offsets,
                                         const int32_t * perm, int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q, float * scale, void * stream,
                                         tqmoe_error * err) {
-    if (!rows_q || !rows_scale || !counts || !offsets || !perm || !q || !scale || cols <= 0 || cols % 32 || experts <= 0 || experts > 4096 || assignments <= 0 ||
-        xdiv <= 0 || grouped_row_tiles(assignments, experts) > 0x7FFFFFFF)
-        return fail(err, TQMOE_E_ARG, "tqmoe_gather_rows_i8: invalid shape or pointer");
-    if (int32_t rc = need_device(err, "tqmoe_gather_rows_i8")) return rc;
-    enqueue_gather_rows_i8(rows_q, rows_scale, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, static_cast<hipStream_t>(stream));
-    return launched(err, "tqmoe_gather_rows_i8");
+    return gather_rows_common(rows_q, rows_scale, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, nullptr, false, stream, err, "tqmoe_gather_rows_i8");
+}
+
+extern "C" int32_t tqmoe_gather_rows_i8_blocks(const int8_t * rows_q, const float * rows_scales, int32_t cols, const int32_t * counts, const int32_t * offsets,
+                                               const int32_t * perm, int32_t experts, int64_t assignments, int32_t xdiv, int8_t * q, float * scale,
+                                               float * block_scale, void * stream, tqmoe_error * err) {
+    return gather_rows_common(rows_q, rows_scales, cols, counts, offsets, perm, experts, assignments, xdiv, q, scale, block_scale, true, stream, err,
+                              "tqmoe_gather_rows_i8_blocks");
 }
 
 static int32_t gemm_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                            const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
-                           tqmoe_error * err, const char * what, bool fp8) {
+                           tqmoe_error * err, const char * what, bool fp8, const float * block_scale = nullptr, bool blocks = false) {
+    if (blocks && !block_scale) return fail(err, TQMOE_E_ARG, "%s: block scales missing", what);
     if (int32_t rc = check_bank(b0, what, err)) return rc;
     if (b1) {
         if (int32_t rc = check_bank(b1, what, err)) return rc;
@@ -420,7 +459,7 @@ static int32_t gemm_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const i
     if (int32_t rc = need_device(err, what)) return rc;
     const int shared_expert = slots > topk ? b0->experts - 1 : -1;
     if (enqueue_plane_gemm(*b0, b1, xq, xs, counts, offsets, perm, b0->experts, int64_t(n) * slots, out, gateup, shared_expert, shared_lim,
-                           static_cast<hipStream_t>(stream)))
+                           static_cast<hipStream_t>(stream), block_scale))
         return fail(err, TQMOE_E_ARG, "%s: too many assignments for one call", what);
     return launched(err, what);
 }
@@ -436,6 +475,21 @@ extern "C" int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * 
                                         const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * y_f16, void * stream,
                                         tqmoe_error * err) {
     return gemm_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8", false);
+}
+
+extern "C" int32_t tqmoe_expert_gemm_gateup_i8_blocks(const tqmoe_bank * gate, const tqmoe_bank * up, const int8_t * xq, const float * xs, const float * block_scale,
+                                                      const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk,
+                                                      int32_t shared_lim, void * act_f16, void * stream, tqmoe_error * err) {
+    if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_gemm_gateup_i8_blocks: second bank missing");
+    return gemm_common(gate, up, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err, "tqmoe_expert_gemm_gateup_i8_blocks", false,
+                       block_scale, true);
+}
+
+extern "C" int32_t tqmoe_expert_gemm_i8_blocks(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const float * block_scale, const int32_t * counts,
+                                               const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim,
+                                               void * y_f16, void * stream, tqmoe_error * err) {
+    return gemm_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8_blocks", false, block_scale,
+                       true);
 }
 
 extern "C" int32_t tqmoe_expert_gemm_gateup_fp8(const tqmoe_bank * gate, const tqmoe_bank * up, const uint8_t * xq, const float * xs, const int32_t * counts,

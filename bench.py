@@ -98,7 +98,7 @@ def build_banks(torch, tq, cfg, banks, seed):
     return out, gen
 
 
-def build_point(torch, tq, cfg, trios, gen, tokens):
+def build_point(torch, tq, cfg, trios, gen, tokens, act_blocks=False):
     """One layer and one input batch per bank for a point of `tokens` tokens."""
     h = cfg["hidden"]
     skew = cfg["zipf_from"] is not None and tokens >= cfg["zipf_from"]
@@ -117,7 +117,7 @@ def build_point(torch, tq, cfg, trios, gen, tokens):
             router[:, -1] = torch.log(p).float()
             x[:, -1] = 1.0
         sgate = (torch.randn((h,), device="cuda", generator=gen) * 0.02).to(rdt) if cfg["shared_ff"] else None
-        layers.append(tq.MoeLayer(router.to(rdt), sgate, *trio, cfg["topk"], shared_ff=cfg["shared_ff"]))
+        layers.append(tq.MoeLayer(router.to(rdt), sgate, *trio, cfg["topk"], shared_ff=cfg["shared_ff"], act_blocks=act_blocks))
         xs.append(x.to(xdt))
     torch.cuda.synchronize()
     return layers, xs, skew
@@ -138,7 +138,7 @@ def time_calls(torch, fn, calls, warmup):
 
 def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
     R = len(trios)
-    layers, xs, skew = build_point(torch, tq, cfg, trios, gen, T)
+    layers, xs, skew = build_point(torch, tq, cfg, trios, gen, T, act_blocks=args.act_blocks)
     h, f, k = cfg["hidden"], cfg["ff"], cfg["topk"]
     slots = k + (1 if cfg["shared_ff"] else 0)
     outs = [torch.empty((T, h), dtype=torch.float32, device="cuda") for _ in range(R)]
@@ -203,7 +203,12 @@ def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
         else:
             counts, offsets, perm, _ = tq.moe_dispatch(ext, cfg["experts"] + shared)
             lists = (counts, offsets, perm)
-            if path in ("grouped_i8", "grouped_fp8"):
+            if path == "grouped_i8" and args.act_blocks:   # a scale per 32 activations: the block scales ride along
+                xq, xsc, xbs = tq.group_rows_i8_blocks(x, lists, T * slots, slots)
+                act = tq.expert_gemm_gateup_i8_blocks(l.gate, l.up, xq, xsc, xbs, lists, T, slots, k, cfg["shared_ff"])
+                aq, asc, abs_ = tq.group_rows_i8_blocks(act, lists, T * slots, 1)
+                prep.append((l, lists, xq, (xsc, xbs), aq, (asc, abs_)))
+            elif path in ("grouped_i8", "grouped_fp8"):
                 xq, xsc = tq.group_rows_i8(x, lists, T * slots, slots, fp8=fp8)
                 act = tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, k, cfg["shared_ff"], fp8=fp8)
                 aq, asc = tq.group_rows_i8(act, lists, T * slots, 1, fp8=fp8)
@@ -219,7 +224,10 @@ def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
                 tq.expert_gateup(l.gate, l.up, img, ext, k, shared_ff=cfg["shared_ff"], act_image=act)
             elif path in ("grouped_i8", "grouped_fp8"):
                 l, lists, xq, xsc, aq, asc = item
-                tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, k, cfg["shared_ff"], fp8=fp8)
+                if isinstance(xsc, tuple):
+                    tq.expert_gemm_gateup_i8_blocks(l.gate, l.up, xq, xsc[0], xsc[1], lists, T, slots, k, cfg["shared_ff"])
+                else:
+                    tq.expert_gemm_gateup_i8(l.gate, l.up, xq, xsc, lists, T, slots, k, cfg["shared_ff"], fp8=fp8)
             else:
                 l, lists, x, act = item
                 tq.expert_gemm_gateup(l.gate, l.up, x, lists, T, slots, k, cfg["shared_ff"])
@@ -231,7 +239,10 @@ def measure_point(torch, tq, cfg, key, trios, gen, T, args, traffic):
                 tq.expert_down(l.down, act, ext, k, shared_ff=cfg["shared_ff"], y=y)
             elif path in ("grouped_i8", "grouped_fp8"):
                 l, lists, xq, xsc, aq, asc = item
-                tq.expert_gemm_i8(l.down, aq, asc, lists, T, slots, k, cfg["shared_ff"], fp8=fp8)
+                if isinstance(asc, tuple):
+                    tq.expert_gemm_i8_blocks(l.down, aq, asc[0], asc[1], lists, T, slots, k, cfg["shared_ff"])
+                else:
+                    tq.expert_gemm_i8(l.down, aq, asc, lists, T, slots, k, cfg["shared_ff"], fp8=fp8)
             else:
                 l, lists, x, act = item
                 tq.expert_gemm(l.down, act, lists, T, slots, k, cfg["shared_ff"], per_expert_input=True, out_type=tq.F32)
@@ -303,6 +314,8 @@ def main():
     ap.add_argument("--banks", type=int, default=8, help="independent expert banks the steps rotate over")
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--act-blocks", action="store_true", help="int8 grouped products with a scale per 32 activations in place of one per token "
+                    "(the reference's TQFN_PREFILL_INT8=1); the headline numbers are measured without it")
     ap.add_argument("--copy-mb", type=int, default=0, help="also run one plain device copy of this many MiB (a kernel of known "
                     "traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this command)")
     args = ap.parse_args()
@@ -338,7 +351,8 @@ def main():
         "data": "synthetic: random valid %s blocks (weights of about 0.02), N(0,1) activations; %d rotating banks" % (cfg["fmt"], args.banks),
         "config": {"workload": "%s; T=%d, %s" % (cfg["label"], head["tokens"], head["routing"]), "tokens": head["tokens"], "launch": head["launch"],
                    "path": head["path"], "distinct_experts_per_step": head["distinct_experts_per_step"],
-                   "points": "tokens " + ", ".join(str(p["tokens"]) for p in points)},
+                   "points": "tokens " + ", ".join(str(p["tokens"]) for p in points),
+                   "activation_scales": "per 32 values" if args.act_blocks else "per token"},
         "roofline": head["roofline"], "layer": head["layer"], "points": points,
     }
     if not args.no_cpu:

@@ -407,6 +407,10 @@ typedef struct tqmoe_layer {
     int32_t gating;                   /* 0: softmax, else a TQMOE_GATE_ value */
     int32_t raw_weights;              /* nonzero: the selected weights are not normalised */
     const float * probs_bias;         /* device [n_expert] fp32 selection bias, or NULL */
+    /* Activation scales of the int8 grouped products, the reference's TQFN_PREFILL_INT8 (fn_prefill.cpp:100): zero (or a
+     * descriptor that ends before this field) = one scale per token (its value 2), nonzero = one per 32 values (its
+     * value 1). The fp8 and fp16 grouped products and the decode kernels ignore it. */
+    int32_t act_blocks;
 } tqmoe_layer;
 
 size_t  tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t n);

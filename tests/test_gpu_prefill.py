@@ -387,12 +387,12 @@ def test_gather_of_quantised_rows_equals_group_rows(tq, dtype):
     assert torch.equal(s1[rows:].view(torch.int32), s2[rows:].view(torch.int32))      # the tile index behind the scales
 
 
-def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0), path="grouped_i8"):
+def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0), path="grouped_i8", act_blocks=False):
     raws = synth.make_banks(cfg, seed=seed, distinct=distinct)
     gate, up, down = banks_on_device(cfg, raws)
     inp = synth.make_inputs(cfg, n, seed=seed + 1, zipf=zipf)
     layer = tq.MoeLayer(dev(inp["router"]), dev(inp["shared_gate"]) if cfg["shared_ff"] else None, gate, up, down, cfg["topk"],
-                        shared_ff=cfg["shared_ff"])
+                        shared_ff=cfg["shared_ff"], act_blocks=act_blocks)
     assert layer.path(n) == path
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
     wants = {}
@@ -404,8 +404,8 @@ def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0), 
 
 
 def check_layer(out, ids, w, wants, clear):
-    fp8 = 5 not in wants
-    want, want_ids, want_w = wants[2] if fp8 else wants[5]
+    fp8 = 2 in wants
+    want, want_ids, want_w = wants[2] if fp8 else wants[5] if 5 in wants else wants[6]
     assert np.array_equal(ids[clear], want_ids[clear])
     assert np.abs(w[clear] - want_w[clear]).max() < 3e-6
     mx, rel = synth.errors(out[clear], want[clear])
@@ -437,6 +437,41 @@ def test_layer_grouped_other_formats(tq, oracle, name, fmt, path, mode, n):
     base = dict(synth.CONFIGS[name], wtype=getattr(oracle, fmt))
     cfg = synth.small(base, 768, 512, 10, 3)
     check_layer(*run_layer(tq, oracle, cfg, n, seed=160 + n, modes=(mode, 0), path=path))
+
+
+@pytest.mark.parametrize("fmt,n", [("IQ4_XS", 64), ("IQ4_XS", 300), ("Q4_K", 300), ("IQ3_S", 300), ("IQ4_NL", 300), ("IQ2_S", 64)])
+def test_layer_block_scales(tq, oracle, fmt, n):
+    """The layer with act_blocks set (a scale per 32 activations on both products' inputs, the reference's
+    TQFN_PREFILL_INT8=1) against the oracle's mode of the same quantiser; the per-token oracle must be farther away."""
+    base = dict(synth.CONFIGS["c2" if fmt == "IQ4_XS" else "c4"], wtype=getattr(oracle, fmt))
+    cfg = synth.small(base, 768, 512, 10, 3)
+    out, ids, w, wants, clear = run_layer(tq, oracle, cfg, n, seed=260 + n, modes=(6, 0, 5), act_blocks=True)
+    wants6 = {6: wants[6], 0: wants[0]}
+    mx, rel = check_layer(out, ids, w, wants6, clear)
+    mx5, rel5 = synth.errors(out[clear], wants[5][0][clear])
+    assert rel5 > 3 * rel, (rel, rel5)
+
+
+def test_layer_descriptor_without_the_block_field(tq, oracle):
+    """A descriptor that ends before act_blocks (an older caller) runs with a scale per token."""
+    import ctypes as C
+    cfg = synth.small(synth.CONFIGS["c2"], 512, 256, 6, 2)
+    raws = synth.make_banks(cfg, seed=5)
+    gate, up, down = banks_on_device(cfg, raws)
+    inp = synth.make_inputs(cfg, 96, seed=6)
+    outs = []
+    for blocks, size in ((False, None), (True, tq.api._Layer.act_blocks.offset), (True, None)):
+        layer = tq.MoeLayer(dev(inp["router"]), dev(inp["shared_gate"]), gate, up, down, cfg["topk"], shared_ff=cfg["shared_ff"], act_blocks=blocks)
+        if size is not None:
+            full = layer.desc
+
+            def short(full=full, size=size):
+                d = full()
+                d.struct_size = size
+                return d
+            layer.desc = short
+        outs.append(layer.forward(dev(inp["x"])).float().cpu())
+    assert torch.equal(outs[0], outs[1]) and not torch.equal(outs[0], outs[2])
 
 
 def test_layer_grouped_small_skewed(tq, oracle):

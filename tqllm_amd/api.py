@@ -46,7 +46,7 @@ class _Layer(C.Structure):
                 ("topk", C.c_int32), ("has_shared", C.c_int32), ("shared_ff", C.c_int32), ("weight_scale", C.c_float),
                 ("router", C.c_void_p), ("shared_gate", C.c_void_p), ("router_type", C.c_uint32),
                 ("gate", _Bank), ("up", _Bank), ("down", _Bank),
-                ("gating", C.c_int32), ("raw_weights", C.c_int32), ("probs_bias", C.c_void_p)]
+                ("gating", C.c_int32), ("raw_weights", C.c_int32), ("probs_bias", C.c_void_p), ("act_blocks", C.c_int32)]
 
 
 _lib = None
@@ -568,8 +568,9 @@ class MoeLayer:
     """hidden states + router weights + expert banks in, combined hidden states out, in one library call."""
 
     def __init__(self, router, shared_gate, gate, up, down, topk, shared_ff=0, weight_scale=1.0, gating=GATE_SOFTMAX, probs_bias=None,
-                 norm_weights=True):
+                 norm_weights=True, act_blocks=False):
         self.router, self.shared_gate, self.gate, self.up, self.down = router, shared_gate, gate, up, down
+        self.act_blocks = act_blocks   # int8 grouped products: a scale per 32 activations in place of one per token
         self.n_expert, self.hidden = router.shape
         self.ff, self.topk, self.shared_ff, self.weight_scale = gate.rows, topk, shared_ff, weight_scale
         self.gating, self.probs_bias, self.norm_weights = gating, probs_bias, norm_weights
@@ -579,7 +580,7 @@ class MoeLayer:
         return _Layer(C.sizeof(_Layer), self.hidden, self.ff, self.n_expert, self.topk, int(self.shared_ff > 0), self.shared_ff,
                       float(self.weight_scale), self.router.data_ptr(), self.shared_gate.data_ptr() if self.shared_gate is not None else None,
                       _ttype(self.router), self.gate.view(), self.up.view(), self.down.view(), int(self.gating), int(not self.norm_weights),
-                      self.probs_bias.data_ptr() if self.probs_bias is not None else None)
+                      self.probs_bias.data_ptr() if self.probs_bias is not None else None, int(self.act_blocks))
 
     def path(self, n):
         """'decode', 'grouped_i8', 'grouped_f16' or 'grouped_fp8': the expert products a batch of n tokens takes"""

@@ -162,6 +162,17 @@ __device__ __forceinline__ void q4k_scale_min(const uint32_t (&q)[3], int j, int
     else { sc = (byte(j + 4) & 15) | ((byte(j - 4) >> 6) << 4); mn = (byte(j + 4) >> 4) | ((byte(j) >> 6) << 4); }
 }
 
+// the same without a branch or an indexed read, for a sub-block number that is only known at run time: bytes j % 4 of the
+// three dwords are all that either case reads (a branch here splits the caller's loop body into blocks, and work that
+// the compiler then moves across them stays in registers for the whole body)
+__device__ __forceinline__ void q4k_scale_min_flat(uint32_t q0, uint32_t q1, uint32_t q2, int j, int & sc, int & mn) {
+    const int sh = 8 * (j & 3);
+    const uint32_t a = (q0 >> sh) & 0xFFu, b = (q1 >> sh) & 0xFFu, c = (q2 >> sh) & 0xFFu;
+    const bool low = j < 4;
+    sc = int(low ? a & 63u : (c & 15u) | ((a >> 6) << 4));
+    mn = int(low ? b & 63u : (c >> 4) | ((b >> 6) << 4));
+}
+
 // IQ4_XS: the 8-byte record of a 256-weight super-block as the device holds it. GGUF's (d, scales_h, scales_l[4]) is the
 // same 64 bits arranged for extraction in one instruction each: the eight 6-bit scales are stored minus 32 as signed
 // fields (what the decoder multiplies by), five in x at bits 6 ib, three in y at bits 14 + 6 (ib - 5); the fp16 d sits in

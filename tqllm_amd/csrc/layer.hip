@@ -26,6 +26,8 @@ struct Plan {  // byte offsets into the workspace
     size_t logits, ids, weights, shared_w, ids_ext, total;
     size_t ximage, aimage, y;                                                // decode path
     size_t xq, xs, counts, offsets, perm, dispatch_ws, act16, aq, as, y16, rq, rs;   // grouped path
+    bool blocks;            // int8 products with a scale per 32 activations
+    size_t xbs, abks;        // their block scales
 };
 
 // the 8-bit grouped products: both banks' formats have one with the same operand type (int8, or E4M3 for NVFP4G)
@@ -33,6 +35,11 @@ bool int8_ok(const tqmoe_layer & L) {
     return plane_gemm_has(L.gate.type) && plane_gemm_has(L.down.type) && plane_gemm_is_fp8(L.gate.type) == plane_gemm_is_fp8(L.down.type) &&
            L.hidden % 256 == 0 && L.ff % 256 == 0 && (!L.has_shared || L.shared_ff % 256 == 0);
 }
+
+// The descriptor grew twice: one that ends before the routing fields means softmax, normalised, no bias; one that ends
+// before act_blocks means a scale per token.
+constexpr size_t kLayerBaseSize = offsetof(tqmoe_layer, gating), kLayerRoutingSize = offsetof(tqmoe_layer, act_blocks);
+bool act_blocks_of(const tqmoe_layer & L) { return L.struct_size >= sizeof(tqmoe_layer) && L.act_blocks != 0; }
 
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
@@ -72,8 +79,13 @@ Plan plan_for(const tqmoe_layer & L, int n) {
         p.xs = take(gwords * 4);
         p.aq = take(grows * L.ff);
         p.as = take(gwords * 4);
+        p.blocks = act_blocks_of(L) && !plane_gemm_is_fp8(L.gate.type);
         p.rq = take(c * L.hidden);        // the chunk's input rows as int8, quantised once, then gathered per assignment
-        p.rs = take(c * 4);
+        p.rs = take(c * 4 * (p.blocks ? size_t(L.hidden / 32) : 1));
+        if (p.blocks) {
+            p.xbs = take(size_t(tqmoe_grouped_block_scale_words(int64_t(a), banks, L.hidden)) * 4);
+            p.abks = take(size_t(tqmoe_grouped_block_scale_words(int64_t(a), banks, L.ff)) * 4);
+        }
     } else if (!p.grouped) {
         p.ximage = take(tqmoe_act_image_bytes(n, L.hidden));
         p.aimage = take(tqmoe_act_image_bytes(int32_t(a), L.ff));
@@ -83,11 +95,9 @@ Plan plan_for(const tqmoe_layer & L, int n) {
     return p;
 }
 
-// The routing fields were appended to the descriptor: one that ends before them means softmax, normalised, no bias.
-constexpr size_t kLayerBaseSize = offsetof(tqmoe_layer, gating);
 struct Routing { int32_t gating; int32_t norm; const float * bias; };
 Routing routing_of(const tqmoe_layer & L) {
-    if (L.struct_size < sizeof(tqmoe_layer)) return Routing{TQMOE_GATE_SOFTMAX, 1, nullptr};
+    if (L.struct_size < kLayerRoutingSize) return Routing{TQMOE_GATE_SOFTMAX, 1, nullptr};
     return Routing{L.gating ? L.gating : int32_t(TQMOE_GATE_SOFTMAX), L.raw_weights ? 0 : 1, L.probs_bias};
 }
 
@@ -196,6 +206,13 @@ static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t
                 if (int32_t rc = tqmoe_expert_gemm_gateup_fp8(&L.gate, &L.up, xq8, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
                 if (int32_t rc = tqmoe_group_rows_fp8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq8, as, stream, err)) return rc;
                 if (int32_t rc = tqmoe_expert_gemm_fp8(&L.down, aq8, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
+            } else if (p.blocks) {
+            float * xbs = reinterpret_cast<float *>(ws + p.xbs), * abks = reinterpret_cast<float *>(ws + p.abks);
+            if (int32_t rc = tqmoe_quant_rows_i8_blocks(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, rq, rs, nullptr, stream, err)) return rc;
+            if (int32_t rc = tqmoe_gather_rows_i8_blocks(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, xbs, stream, err)) return rc;
+            if (int32_t rc = tqmoe_expert_gemm_gateup_i8_blocks(&L.gate, &L.up, xq, xs, xbs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
+            if (int32_t rc = tqmoe_group_rows_i8_blocks(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, abks, stream, err)) return rc;
+            if (int32_t rc = tqmoe_expert_gemm_i8_blocks(&L.down, aq, as, abks, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
             } else {
             if (int32_t rc = tqmoe_quant_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, rq, rs, stream, err)) return rc;
             if (int32_t rc = tqmoe_gather_rows_i8(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, stream, err)) return rc;

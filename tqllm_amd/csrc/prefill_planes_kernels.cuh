@@ -467,9 +467,8 @@ struct WQ4k {   // row-major: 16 code bytes per sub-block, a 16-byte record (d |
     static __device__ __forceinline__ Rec rec(const Src & s, int sb) { return *reinterpret_cast<const uint4 *>(s.aux + int64_t(sb) * 16); }
     static __device__ __forceinline__ DRec drec(const Src & s, int sb) { return *reinterpret_cast<const uint32_t *>(s.aux + int64_t(sb) * 16); }
     static __device__ __forceinline__ void planes(const Code & c, const Rec & r, int ib, int, const uint8_t * tab, const uint32_t *, v4i * p) {
-        const uint32_t sc12[3] = {r.y, r.z, r.w};
         int sc, mn;
-        q4k_scale_min(sc12, ib, sc, mn);
+        q4k_scale_min_flat(r.y, r.z, r.w, ib, sc, mn);
         const uint4 * t = reinterpret_cast<const uint4 *>(tab + sc * 32);
         decode_planes(c.c, t[0], t[1], p[0], p[1]);
         const int m = mn * 0x01010101;   // the minimum's coefficient, the same for the sub-block's 32 weights
@@ -835,21 +834,17 @@ template <class W> __device__ __forceinline__ void acc_block_fold(Acc<W> & a, co
         a.sum[4 * c + 3] = __fmaf_rn(t[4 * c + 3], sc[c].w, a.sum[4 * c + 3]);
     }
 }
-// two consecutive sub-blocks with a row scale each (sc0, sc1)
-template <class W> __device__ __forceinline__ void acc_step2_blocks(Acc<W> & a, v4i x0, v4i x1, const v4i * w0, const v4i * w1, const typename W::DRec & r, int ib0,
-                                                                   const float4 * sc0, const float4 * sc1) {
+// one sub-block of a row tile against one slot's weights, the row scales of that sub-block in sc
+template <class W> __device__ __forceinline__ void acc_step_block(Acc<W> & a, v4i x, const v4i * w, const typename W::DRec & r, int ib, const float4 * sc) {
     static_assert(!W::kFp8, "a scale per sub-block: int8 operands only");
     const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    // (one sub-block at a time, fenced: issued together, the sums of several sub-blocks and slots are more than the registers hold)
-    v16i s0[W::kPlanes], s1[W::kPlanes];
+    v16i s[W::kPlanes];
 #pragma unroll
-    for (int p = 0; p < W::kPlanes; ++p) s0[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0, w0[p], zero, 0, 0, 0);
-    acc_block_fold(a, s0, r, ib0, sc0);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int p = 0; p < W::kPlanes; ++p) s1[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1, w1[p], zero, 0, 0, 0);
-    acc_block_fold(a, s1, r, ib0 + 1, sc1);
-    __builtin_amdgcn_sched_barrier(0);
+    for (int p = 0; p < W::kPlanes; ++p) s[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, w[p], zero, 0, 0, 0);
+    acc_block_fold(a, s, r, ib, sc);
+    // (the result is pinned here: where the loop body is several basic blocks the compiler otherwise moves the scaling of
+    // every sub-block behind the last of them and keeps all their integer sums until then, far more than the registers hold)
+    asm volatile("" : "+v"(a.sum));
 }
 // |64 acc_h + acc_l| <= 256 * 127 * 2^12 < 2^28: exact in int32, then one rounding into fp32
 template <class W> __device__ __forceinline__ void acc_fold(Acc<W> & a, const typename W::DRec & r) {
@@ -1238,17 +1233,29 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                         }
                         if (jp == 3) { __builtin_amdgcn_sched_barrier(0); fetch(sb, 2); __builtin_amdgcn_sched_barrier(0); }
                         load_a((jp + kSlots - 1) % kSlots, sb * 4 + jp + kSlots - 1);
-                        [[maybe_unused]] float4 sc[MTA][2][4];
-                        if constexpr (BLK) {   // (fenced: the scheduler would otherwise start every group's scales at the top and run out of registers)
-                            __builtin_amdgcn_sched_barrier(0);
+                        if constexpr (BLK) {
+                            // one sub-block at a time, fenced: its row scales, then each slot's weights and products (started
+                            // all at once, the scales and integer sums of a whole group are more than the registers hold)
 #pragma unroll
-                            for (int t = 0; t < MT; ++t)
+                            for (int h = 0; h < 2; ++h) {
+                                __builtin_amdgcn_sched_barrier(0);
+                                float4 sc[MTA][4];
 #pragma unroll
-                                for (int h = 0; h < 2; ++h)
+                                for (int t = 0; t < MT; ++t)
 #pragma unroll
                                     for (int c = 0; c < 4; ++c)
-                                        sc[t][h][c] = *reinterpret_cast<const float4 *>(sc_base + t * sc_tile + (int64_t(sb) * 8 + 2 * jp + h) * 32 + 8 * c);
-                        }
+                                        sc[t][c] = *reinterpret_cast<const float4 *>(sc_base + t * sc_tile + (int64_t(sb) * 8 + 2 * jp + h) * 32 + 8 * c);
+#pragma unroll
+                                for (int b = 0; b < NB; ++b) {
+                                    v4i w[P];
+#pragma unroll
+                                    for (int p = 0; p < P; ++p) w[p] = bs[(((buf * NB + b) * P + p) * 8 + 2 * jp + h) * 64 + lane];
+#pragma unroll
+                                    for (int t = 0; t < MT; ++t) acc_step_block(acc[t][b], a_reg[jp % kSlots][t][h], w, d_rec[b], 2 * jp + h, sc[t]);
+                                    __builtin_amdgcn_sched_barrier(0);
+                                }
+                            }
+                        } else
 #pragma unroll
                         for (int b = 0; b < NB; ++b) {
                             v4i w0[P], w1[P];
@@ -1258,13 +1265,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                                 w1[p] = bs[(((buf * NB + b) * P + p) * 8 + 2 * jp + 1) * 64 + lane];
                             }
 #pragma unroll
-                            for (int t = 0; t < MT; ++t) {
-                                if constexpr (BLK) {
-                                    acc_step2_blocks(acc[t][b], a_reg[jp % kSlots][t][0], a_reg[jp % kSlots][t][1], w0, w1, d_rec[b], 2 * jp, sc[t][0], sc[t][1]);
-                                } else {
-                                    acc_step2(acc[t][b], a_reg[jp % kSlots][t][0], a_reg[jp % kSlots][t][1], w0, w1, jp == 0, d_rec[b], 2 * jp);
-                                }
-                            }
+                            for (int t = 0; t < MT; ++t) acc_step2(acc[t][b], a_reg[jp % kSlots][t][0], a_reg[jp % kSlots][t][1], w0, w1, jp == 0, d_rec[b], 2 * jp);
                         }
                     }
                     if constexpr (!BLK) {

@@ -846,6 +846,22 @@ template <class W> __device__ __forceinline__ void acc_step_block(Acc<W> & a, v4
     // every sub-block behind the last of them and keeps all their integer sums until then, far more than the registers hold)
     asm volatile("" : "+v"(a.sum));
 }
+// two consecutive sub-blocks: both sets of products are issued before the first is scaled, so that the matrix pipe works
+// through the second while the vector pipe scales the first
+template <class W> __device__ __forceinline__ void acc_step2_blocks(Acc<W> & a, v4i x0, v4i x1, const v4i * w0, const v4i * w1, const typename W::DRec & r, int ib0,
+                                                                   const float4 * sc0, const float4 * sc1) {
+    static_assert(!W::kFp8, "a scale per sub-block: int8 operands only");
+    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    v16i s0[W::kPlanes], s1[W::kPlanes];
+#pragma unroll
+    for (int p = 0; p < W::kPlanes; ++p) s0[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0, w0[p], zero, 0, 0, 0);
+#pragma unroll
+    for (int p = 0; p < W::kPlanes; ++p) s1[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1, w1[p], zero, 0, 0, 0);
+    acc_block_fold(a, s0, r, ib0, sc0);
+    asm volatile("" : "+v"(a.sum));     // (pinned, as in acc_step_block)
+    acc_block_fold(a, s1, r, ib0 + 1, sc1);
+    asm volatile("" : "+v"(a.sum));
+}
 // |64 acc_h + acc_l| <= 256 * 127 * 2^12 < 2^28: exact in int32, then one rounding into fp32
 template <class W> __device__ __forceinline__ void acc_fold(Acc<W> & a, const typename W::DRec & r) {
     if constexpr (!W::kFp8 && !W::kFoldSub) {
@@ -1189,7 +1205,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                 for (int p = 0; p < P; ++p) bs[(((buf * NB + my_slot) * P + p) * 8 + ib) * 64 + lane] = w[p];
             };
             // operand A (the same rows for every unit), two k-steps (sub-blocks) per slot
-            constexpr int kSlots = BLK ? 2 : 4;   // (the per-sub-block scales and sums need the registers of two slots)
+            constexpr int kSlots = 4;
             v4i a_reg[kSlots][MTA][2];
             auto load_a = [&](int slot, int pair) {   // pair counted from the current unit's first
                 const int at = pair < pairs_u ? pair : last ? pairs_u - 1 : pair - pairs_u;
@@ -1234,26 +1250,29 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                         if (jp == 3) { __builtin_amdgcn_sched_barrier(0); fetch(sb, 2); __builtin_amdgcn_sched_barrier(0); }
                         load_a((jp + kSlots - 1) % kSlots, sb * 4 + jp + kSlots - 1);
                         if constexpr (BLK) {
-                            // one sub-block at a time, fenced: its row scales, then each slot's weights and products (started
-                            // all at once, the scales and integer sums of a whole group are more than the registers hold)
+                            // a group at a time, fenced: its row scales, then each slot's weights and products (started all at
+                            // once, the scales and integer sums of a whole step are more than the registers hold)
+                            __builtin_amdgcn_sched_barrier(0);
+                            float4 sc[MTA][2][4];
 #pragma unroll
-                            for (int h = 0; h < 2; ++h) {
-                                __builtin_amdgcn_sched_barrier(0);
-                                float4 sc[MTA][4];
+                            for (int t = 0; t < MT; ++t)
 #pragma unroll
-                                for (int t = 0; t < MT; ++t)
+                                for (int h = 0; h < 2; ++h)
 #pragma unroll
                                     for (int c = 0; c < 4; ++c)
-                                        sc[t][c] = *reinterpret_cast<const float4 *>(sc_base + t * sc_tile + (int64_t(sb) * 8 + 2 * jp + h) * 32 + 8 * c);
+                                        sc[t][h][c] = *reinterpret_cast<const float4 *>(sc_base + t * sc_tile + (int64_t(sb) * 8 + 2 * jp + h) * 32 + 8 * c);
 #pragma unroll
-                                for (int b = 0; b < NB; ++b) {
-                                    v4i w[P];
+                            for (int b = 0; b < NB; ++b) {
+                                v4i w0[P], w1[P];
 #pragma unroll
-                                    for (int p = 0; p < P; ++p) w[p] = bs[(((buf * NB + b) * P + p) * 8 + 2 * jp + h) * 64 + lane];
-#pragma unroll
-                                    for (int t = 0; t < MT; ++t) acc_step_block(acc[t][b], a_reg[jp % kSlots][t][h], w, d_rec[b], 2 * jp + h, sc[t]);
-                                    __builtin_amdgcn_sched_barrier(0);
+                                for (int p = 0; p < P; ++p) {
+                                    w0[p] = bs[(((buf * NB + b) * P + p) * 8 + 2 * jp) * 64 + lane];
+                                    w1[p] = bs[(((buf * NB + b) * P + p) * 8 + 2 * jp + 1) * 64 + lane];
                                 }
+#pragma unroll
+                                for (int t = 0; t < MT; ++t)
+                                    acc_step2_blocks(acc[t][b], a_reg[jp % kSlots][t][0], a_reg[jp % kSlots][t][1], w0, w1, d_rec[b], 2 * jp, sc[t][0], sc[t][1]);
+                                __builtin_amdgcn_sched_barrier(0);
                             }
                         } else
 #pragma unroll

@@ -167,6 +167,24 @@ struct ExpertFormat {
         check(rc, e);
         return true;
     }
+    // the two int8 products in mode 1 (a scale per 32 values of every row, quant_kernels.cuh:13-16): block_scale is
+    // tqmoe_group_rows_i8_blocks' third output for the same lists
+    static bool expert_gemm_i8_blocks(const tqmoe_bank & m, const int8_t * xq, const float * xs, const float * block_scale, void * y_f16, const int * counts,
+                                      const int * offsets, const int * perm, int n, int topk, void * stream) {
+        tqmoe_error e = fresh();
+        const int32_t rc = tqmoe_expert_gemm_i8_blocks(&m, xq, xs, block_scale, counts, offsets, perm, n, topk, topk, 0, y_f16, stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
+    static bool expert_gemm_gateup_i8_blocks(const tqmoe_bank & g, const tqmoe_bank & u, const int8_t * xq, const float * xs, const float * block_scale, void * y_f16,
+                                             const int * counts, const int * offsets, const int * perm, int n, int topk, void * stream) {
+        tqmoe_error e = fresh();
+        const int32_t rc = tqmoe_expert_gemm_gateup_i8_blocks(&g, &u, xq, xs, block_scale, counts, offsets, perm, n, topk, topk, 0, y_f16, stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
     // the same two products on E4M3 rows for NVFP4G banks (rows of tqmoe_group_rows_fp8, scale amax / 448 as
     // src/core/fp8_gemm.cuh:19-31); false: the format has no fp8 grouped kernel
     static bool expert_gemm_fp8(const tqmoe_bank & m, const uint8_t * xq, const float * xs, void * y_f16, const int * counts, const int * offsets, const int * perm,

@@ -960,9 +960,7 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
         const int live_tiles = min(CT, tiles_e - first_tile);               // of this block
         // A chunk of one row tile has nothing for the waves to share: every wave then takes the tile against 32 weight
         // rows of its own (of every slot it has), four units a pass, the chunk's items taking passes in turn.
-        // (with a scale per sub-block the lone arrangement's stages and the per-sub-block sums do not fit the registers: such
-        // chunks go the shared way, one wave multiplying)
-        const bool lone = !BLK && live_tiles == 1 && k.units % 4 == 0;
+        const bool lone = live_tiles == 1 && k.units % 4 == 0;
         if (lone && ug >= k.units / 4) continue;
         // the rows' assignments and scales are only read when the results are stored: their loads are issued here and land
         // in LDS after the products, so that nothing waits for them
@@ -1002,11 +1000,13 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                 sbe = wdead ? 0 : !GATEUP && is_shared ? k.shared_lim / 256 : NSB;
             }
             const int8_t * a_ptr = k.xq + int64_t(tile_base + first_tile) * 32 * k.b0.cols + lane * 16;
+            // (row scales per sub-block: the four float4 of the lane's 16 result rows, 8 c + 4 g + 0..3)
+            [[maybe_unused]] const float * sc_ptr = BLK ? k.xbs + int64_t(tile_base + first_tile) * (k.b0.cols / 32) * 32 + 4 * g : nullptr;
             // (the weights' codes run a super-block ahead, and so do the row tile's operands where the codes are short; with
             // codes of 12 bytes and more the operands are read at the start of their super-block's work instead: they come
             // from the L2, the SIMD's other wave covers the wait, and a second set of them is 32 registers that those
             // formats spilled)
-            constexpr bool kAheadA = sizeof(typename W::Code) <= 8;
+            constexpr bool kAheadA = sizeof(typename W::Code) <= 8 && !BLK;   // (with a scale per sub-block the second set does not fit beside the sums and scales)
             struct Stage { typename W::Code code[SPW][8]; typename W::Rec rec[SPW]; typename W::DRec drec[SPW]; v4i a[kAheadA ? 8 : 1]; };
             auto fetch1 = [&](int sb, Stage & st) {   // a super-block of the wave's weights and of the row tile
 #pragma unroll
@@ -1035,16 +1035,27 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ib = 0; ib < 8; ib += 2) {
+                    [[maybe_unused]] float4 sc[2][4];
+                    if constexpr (BLK) {   // (fenced: started all at the top, the scales of a super-block are more than the registers hold)
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) sc[h][c] = *reinterpret_cast<const float4 *>(sc_ptr + (int64_t(sb) * 8 + ib + h) * 32 + 8 * c);
+                    }
 #pragma unroll
                     for (int q = 0; q < SPW; ++q) {
                         v4i w0[P], w1[P];
                         W::planes(cur.code[q][ib], cur.rec[q], ib, g, s_tab, s_lat, w0);
                         W::planes(cur.code[q][ib + 1], cur.rec[q], ib + 1, g, s_tab, s_lat, w1);
-                        acc_step2(acc[q], a[ib], a[ib + 1], w0, w1, ib == 0, cur.drec[q], ib);
+                        if constexpr (BLK) acc_step2_blocks(acc[q], a[ib], a[ib + 1], w0, w1, cur.drec[q], ib, sc[0], sc[1]);
+                        else acc_step2(acc[q], a[ib], a[ib + 1], w0, w1, ib == 0, cur.drec[q], ib);
                     }
                 }
+                if constexpr (!BLK) {
 #pragma unroll
-                for (int q = 0; q < SPW; ++q) acc_fold(acc[q], cur.drec[q]);
+                    for (int q = 0; q < SPW; ++q) acc_fold(acc[q], cur.drec[q]);
+                }
             };
             if (sbe > 0) {
                 Stage s0, s1;

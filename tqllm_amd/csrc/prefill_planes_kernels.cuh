@@ -15,6 +15,9 @@
 // tables in LDS (one pair per scale value) and applied with v_perm_b32. The planes go through one MFMA each that
 // accumulate over the whole 256-weight super-block, so the scales cost no vector instruction per product; per
 // super-block the results fold as acc += d * (64 * acc_h + acc_l) - dmin * acc_m in fp32.
+// With a scale per row and 32-value sub-block in place of one per row (the reference's other int8 mode) the integer sums
+// cannot ride through the super-block: every sub-block's MFMAs start from zero and its sums are scaled by the weights'
+// scale and the row's scale of that sub-block as they join the fp32 result (the BLK instances of the kernel).
 // NVFP4G weights are e2m1 * E4M3 scale (per 16 weights) * fp32 global (per row): the product of the first two is rounded
 // to E4M3 (a declared lossy operand: six significant bits into four), again through a 16-entry table per scale byte; the
 // fp8 MFMA accumulates in fp32 over the whole row and the global multiplies the result.
@@ -834,18 +837,6 @@ template <class W> __device__ __forceinline__ void acc_block_fold(Acc<W> & a, co
         a.sum[4 * c + 3] = __fmaf_rn(t[4 * c + 3], sc[c].w, a.sum[4 * c + 3]);
     }
 }
-// one sub-block of a row tile against one slot's weights, the row scales of that sub-block in sc
-template <class W> __device__ __forceinline__ void acc_step_block(Acc<W> & a, v4i x, const v4i * w, const typename W::DRec & r, int ib, const float4 * sc) {
-    static_assert(!W::kFp8, "a scale per sub-block: int8 operands only");
-    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    v16i s[W::kPlanes];
-#pragma unroll
-    for (int p = 0; p < W::kPlanes; ++p) s[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, w[p], zero, 0, 0, 0);
-    acc_block_fold(a, s, r, ib, sc);
-    // (the result is pinned here: where the loop body is several basic blocks the compiler otherwise moves the scaling of
-    // every sub-block behind the last of them and keeps all their integer sums until then, far more than the registers hold)
-    asm volatile("" : "+v"(a.sum));
-}
 // two consecutive sub-blocks: both sets of products are issued before the first is scaled, so that the matrix pipe works
 // through the second while the vector pipe scales the first
 template <class W> __device__ __forceinline__ void acc_step2_blocks(Acc<W> & a, v4i x0, v4i x1, const v4i * w0, const v4i * w1, const typename W::DRec & r, int ib0,
@@ -857,8 +848,11 @@ template <class W> __device__ __forceinline__ void acc_step2_blocks(Acc<W> & a, 
     for (int p = 0; p < W::kPlanes; ++p) s0[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x0, w0[p], zero, 0, 0, 0);
 #pragma unroll
     for (int p = 0; p < W::kPlanes; ++p) s1[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x1, w1[p], zero, 0, 0, 0);
+    // The result is pinned after each scaling: where the loop body is several basic blocks (a format whose decode
+    // branches) the compiler otherwise moves the scaling of every sub-block behind the last of them and keeps all their
+    // integer sums until then, far more than the registers hold.
     acc_block_fold(a, s0, r, ib0, sc0);
-    asm volatile("" : "+v"(a.sum));     // (pinned, as in acc_step_block)
+    asm volatile("" : "+v"(a.sum));
     acc_block_fold(a, s1, r, ib0 + 1, sc1);
     asm volatile("" : "+v"(a.sum));
 }

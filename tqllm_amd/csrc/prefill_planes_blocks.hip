@@ -7,9 +7,9 @@ namespace tqmoe {
 
 int32_t plane_gemm_blocks(uint32_t type, int nb, bool gateup, const GemmArgs & k, unsigned blocks, hipStream_t s) {
     switch (type) {
-        case TQMOE_IQ4_XS: plane_gemm_launch<WIq4xs, true>(nb, gateup, k, blocks, s); break;
+        case TQMOE_IQ4_XS: plane_gemm_launch<WIq4xsSub, true>(nb, gateup, k, blocks, s); break;
         case TQMOE_IQ3_S: plane_gemm_launch<WIq3s, true>(nb, gateup, k, blocks, s); break;
-        case TQMOE_Q4_K: plane_gemm_launch<WQ4k, true>(nb, gateup, k, blocks, s); break;
+        case TQMOE_Q4_K: plane_gemm_launch<WQ4kSub, true>(nb, gateup, k, blocks, s); break;
         case TQMOE_IQ3_XXS: plane_gemm_launch<WIq3xxs, true>(nb, gateup, k, blocks, s); break;
         case TQMOE_IQ2_XXS: plane_gemm_launch<WIq2xxs, true>(nb, gateup, k, blocks, s); break;
         case TQMOE_IQ2_XS: plane_gemm_launch<WIq2xs, true>(nb, gateup, k, blocks, s); break;

@@ -449,6 +449,25 @@ struct WIq4xs {   // tile-major codes (512 B per sub-block of a tile), 8-byte re
     static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
 };
 
+// IQ4_XS for rows with a scale per sub-block: the sub-block scale no longer needs to ride inside the operand (every
+// sub-block's sums are scaled on their own anyway), so one plane of the 16 table values and d * (ls - 32) as the
+// sub-block's fp32 scale: half the MFMAs, LDS traffic and lookups of the two-plane form.
+struct WIq4xsSub : WIq4xs {
+    static constexpr bool kFoldSub = true;
+    static constexpr int kPlanes = 1, kTabBytes = 16;
+    static __device__ __forceinline__ void tables(uint8_t *, uint32_t *, int, int) {}
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int, const uint8_t *, const uint32_t *, v4i * p) {
+        uint32_t lo, hi;
+        lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(c.c.x, lo, hi);
+        p[0][0] = int(lo); p[0][1] = int(hi);
+        lookup16<kIq4T0, kIq4T1, kIq4T2, kIq4T3>(c.c.y, lo, hi);
+        p[0][2] = int(lo); p[0][3] = int(hi);
+    }
+    static __device__ __forceinline__ float d_sub(const DRec & r, int ib) {   // exact: an 11-bit significand times a 6-bit integer
+        return __fmul_rn(half_bits_to_float(iq4xs_d_bits(r)), float(iq4xs_lsm32(r, ib)));
+    }
+};
+
 struct WQ4k {   // row-major: 16 code bytes per sub-block, a 16-byte record (d | dmin << 16, twelve bytes of 6-bit scales and minimums) per super-block
     static constexpr bool kFoldSub = false;     // one scale per 32 weights: every sub-block's product is folded on its own
     static constexpr bool kWideChunks = false;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)
@@ -480,6 +499,30 @@ struct WQ4k {   // row-major: 16 code bytes per sub-block, a 16-byte record (d |
     static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(uint16_t(r & 0xFFFFu)); }
     static __device__ __forceinline__ float dmin(const DRec & r) { return half_bits_to_float(uint16_t(r >> 16)); }
     static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
+};
+
+// Q4_K for rows with a scale per sub-block, likewise: the 4-bit codes themselves as one plane (no lookup), a plane of ones
+// whose product is the sum of the row's values, and d * sc, dmin * mn as the sub-block's fp32 scales.
+struct WQ4kSub : WQ4k {
+    static constexpr bool kFoldSub = true;
+    static constexpr int kPlanes = 2, kTabBytes = 16;
+    typedef uint4 DRec;      // the whole record: the fold needs the sub-block's scale and minimum
+    static __device__ __forceinline__ void tables(uint8_t *, uint32_t *, int, int) {}
+    static __device__ __forceinline__ DRec drec(const Src & s, int sb) { return rec(s, sb); }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int, const uint8_t *, const uint32_t *, v4i * p) {
+        p[0] = v4i{int(c.c.x & 0x0F0F0F0Fu), int((c.c.x >> 4) & 0x0F0F0F0Fu), int(c.c.y & 0x0F0F0F0Fu), int((c.c.y >> 4) & 0x0F0F0F0Fu)};
+        p[1] = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    }
+    static __device__ __forceinline__ float d_sub(const DRec & r, int ib) {      // exact: 11 bits times 6 bits
+        int sc, mn;
+        q4k_scale_min_flat(r.y, r.z, r.w, ib, sc, mn);
+        return __fmul_rn(half_bits_to_float(uint16_t(r.x & 0xFFFFu)), float(sc));
+    }
+    static __device__ __forceinline__ float dmin_sub(const DRec & r, int ib) {
+        int sc, mn;
+        q4k_scale_min_flat(r.y, r.z, r.w, ib, sc, mn);
+        return __fmul_rn(half_bits_to_float(uint16_t(r.x >> 16)), float(mn));
+    }
 };
 
 struct WIq3s {   // row-major: 12 code bytes per sub-block (8 lattice indices, 32 sign bits), a 16-byte record per super-block
@@ -819,6 +862,11 @@ template <class W> __device__ __forceinline__ void acc_block_fold(Acc<W> & a, co
         const float d = W::d_sub(r, ib);
 #pragma unroll
         for (int i = 0; i < 16; ++i) t[i] = __fmul_rn(float(s[0][i]), d);
+        if constexpr (W::kMin) {   // the second plane is the sum of the row's values
+            const float m = -W::dmin_sub(r, ib);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) t[i] = __fmaf_rn(float(s[1][i]), m, t[i]);
+        }
     } else {
         const float d = W::d(r);
 #pragma unroll

@@ -93,111 +93,6 @@ template <bool F8> __device__ __forceinline__ uint32_t pack4_q(float a, float b,
 }
 template <bool F8> constexpr float kOperandMax = F8 ? 448.f : 127.f;
 
-// the largest magnitude over the four lanes that hold a 32-value block (eight values each)
-__device__ __forceinline__ float quad_max(float v) {
-    v = fmaxf(v, dpp_f<kDppXor1>(v));
-    return fmaxf(v, dpp_f<kDppXor2>(v));
-}
-__device__ __forceinline__ int byte_sum_i8(uint32_t w) { return int(int8_t(w)) + int(int8_t(w >> 8)) + int(int8_t(w >> 16)) + int(int8_t(w >> 24)); }
-
-// rows of 8-bit activations: q = rint(x * 127 / amax) per row, scale = amax / 127 (E4M3: 448 in place of 127); one wave per row.
-// BLK: amax and scale per block of 32 values (scale [rows][cols / 32]) and, when asked for, the sums of q over each 16
-// values (qsum [rows][cols / 32][2]).
-template <int XT, bool F8, bool BLK = false>
-__global__ __launch_bounds__(256) void quant_rows_k(const void * __restrict__ x, int64_t rows, int cols, int8_t * __restrict__ q, float * __restrict__ scale,
-                                                    int16_t * __restrict__ qsum = nullptr) {
-    const int lane = threadIdx.x & 63;
-    const int64_t row = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const int groups = cols / 8;   // 8 consecutive values = natural dwords 2j, 2j + 1 of a 32-block
-    if constexpr (BLK) {           // (a block's four lanes enter or leave the loop together: cols is a multiple of 32)
-        uint32_t * out = reinterpret_cast<uint32_t *>(q + row * cols);
-        for (int gi = lane; gi < groups; gi += 64) {
-            float v[8];
-            load8<XT>(x, row * cols + gi * 8, v);
-            float amax = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-            amax = quad_max(amax);
-            const float mul = amax > 0.f ? 127.f / amax : 0.f;
-            const uint32_t w[2] = {pack4_q<false>(v[0] * mul, v[1] * mul, v[2] * mul, v[3] * mul), pack4_q<false>(v[4] * mul, v[5] * mul, v[6] * mul, v[7] * mul)};
-            const int blk = gi >> 2, d0 = 2 * (gi & 3);
-            out[blk * 8 + plane_pos(d0)] = w[0];
-            out[blk * 8 + plane_pos(d0 + 1)] = w[1];
-            if ((gi & 3) == 0) scale[row * (cols / 32) + blk] = amax / 127.f;
-            if (qsum) {
-                int sum = byte_sum_i8(w[0]) + byte_sum_i8(w[1]);
-                sum += dpp_i<kDppXor1>(sum);
-                if ((gi & 1) == 0) qsum[(row * (cols / 32) + blk) * 2 + ((gi & 3) >> 1)] = int16_t(sum);
-            }
-        }
-        return;
-    }
-    float amax = 0.f;
-    for (int gi = lane; gi < groups; gi += 64) {
-        float v[8];
-        load8<XT>(x, row * cols + gi * 8, v);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-    }
-    amax = fmaxf(amax, dpp_f<kDppXor1>(amax));
-    amax = fmaxf(amax, dpp_f<kDppXor2>(amax));
-    amax = fmaxf(amax, dpp_f<kDppHalfMirror>(amax));
-    amax = fmaxf(amax, dpp_f<kDppMirror>(amax));
-    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-    const float mul = amax > 0.f ? kOperandMax<F8> / amax : 0.f;
-    if (lane == 0) scale[row] = amax / kOperandMax<F8>;
-    uint32_t * out = reinterpret_cast<uint32_t *>(q + row * cols);
-    for (int gi = lane; gi < groups; gi += 64) {
-        float v[8];
-        load8<XT>(x, row * cols + gi * 8, v);
-        const uint32_t w[2] = {pack4_q<F8>(v[0] * mul, v[1] * mul, v[2] * mul, v[3] * mul), pack4_q<F8>(v[4] * mul, v[5] * mul, v[6] * mul, v[7] * mul)};
-        const int blk = gi >> 2, d0 = 2 * (gi & 3);
-        out[blk * 8 + plane_pos(d0)] = w[0];
-        out[blk * 8 + plane_pos(d0 + 1)] = w[1];
-    }
-}
-
-// inclusive prefix sum over the wave's 64 lanes with DPP moves (rows of 16, then the rows' totals handed on)
-template <int N> __device__ __forceinline__ int dpp_row_shr(int v) { return __builtin_amdgcn_update_dpp(0, v, 0x110 + N, 0xF, 0xF, true); }
-__device__ __forceinline__ int wave_prefix_sum(int v) {
-    v += dpp_row_shr<1>(v);
-    v += dpp_row_shr<2>(v);
-    v += dpp_row_shr<4>(v);
-    v += dpp_row_shr<8>(v);
-    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);   // row_bcast:15 into rows 1 and 3
-    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);   // row_bcast:31 into rows 2 and 3
-    return v;
-}
-
-__global__ __launch_bounds__(64) void plan_k(const int * __restrict__ counts, int experts, Plan plan) {
-    const int lane = threadIdx.x;
-    int * tile_base = const_cast<int *>(plan.tile_base), * chunk_base = const_cast<int *>(plan.chunk_base), * chunk_base2 = const_cast<int *>(plan.chunk_base2);
-    if (lane < kPlanCounters) plan.counters[lane] = 0;
-    int tbase = 0, cbase = 0, cbase2 = 0;
-    constexpr int kAhead = 16;   // counts of 16 x 64 experts are loaded in one trip to memory, then scanned 64 at a time
-    for (int eb = 0; eb < experts; eb += 64 * kAhead) {
-        int cnt[kAhead];
-#pragma unroll
-        for (int i = 0; i < kAhead; ++i) cnt[i] = counts[min(eb + 64 * i + lane, experts - 1)];
-#pragma unroll
-        for (int i = 0; i < kAhead; ++i) {
-            const int e0 = eb + 64 * i;
-            if (e0 >= experts) break;
-            const int e = e0 + lane;
-            const int tiles = e < experts ? (max(cnt[i], 0) + 31) >> 5 : 0;
-            const int chunks = (tiles + kChunkTiles - 1) / kChunkTiles, chunks2 = (tiles + 2 * kChunkTiles - 1) / (2 * kChunkTiles);
-            const int ti = wave_prefix_sum(tiles), ci = wave_prefix_sum(chunks), c2 = wave_prefix_sum(chunks2);
-            if (e < experts) { tile_base[e] = tbase + ti - tiles; chunk_base[e] = cbase + ci - chunks; chunk_base2[e] = cbase2 + c2 - chunks2; }
-            tbase += __builtin_amdgcn_readlane(ti, 63);
-            cbase += __builtin_amdgcn_readlane(ci, 63);
-            cbase2 += __builtin_amdgcn_readlane(c2, 63);
-        }
-    }
-    if (lane == 0) { tile_base[experts] = tbase; chunk_base[experts] = cbase; chunk_base2[experts] = cbase2; }
-}
-
 // largest e in [0, experts) with base[e] <= unit, for unit < base[experts] (experts with no unit share their successor's
 // base and are skipped by taking the last of equal entries)
 __device__ __forceinline__ int owner_of(const int * __restrict__ base, int experts, int unit) {
@@ -207,162 +102,6 @@ __device__ __forceinline__ int owner_of(const int * __restrict__ base, int exper
         if (base[mid] <= unit) lo = mid; else hi = mid;
     }
     return lo;
-}
-
-// Rows of the grouped operand: block b takes rows [8 (b % 4), +8) of row tile b / 4, one wave per two rows. Row i of
-// expert e's tiles is assignment perm[offsets[e] + i], its source row a / xdiv. Rows past the expert's count are left as
-// they are (their products are never stored).
-template <int XT, bool F8, bool BLK = false>
-__global__ __launch_bounds__(256) void group_rows_k(const void * __restrict__ x, int cols, const int * __restrict__ counts, const int * __restrict__ offsets,
-                                                         const int * __restrict__ perm, int experts, int xdiv, int8_t * __restrict__ q, float * __restrict__ scale,
-                                                         Plan plan, float * __restrict__ block_scale = nullptr) {
-    const int tile_index = int(blockIdx.x >> 2);
-    if (tile_index >= plan.tile_base[experts]) return;
-    const int e = owner_of(plan.tile_base, experts, tile_index);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int cnt = counts[e], groups = cols / 8, lt = tile_index - plan.tile_base[e];
-    uint32_t * tile = reinterpret_cast<uint32_t *>(q + int64_t(tile_index) * 32 * cols);
-#pragma unroll
-    for (int rr = 0; rr < 2; ++rr) {
-        const int r = int(blockIdx.x & 3) * 8 + wave * 2 + rr;
-        const int i = lt * 32 + r;
-        if (i >= cnt) break;
-        const int64_t row = perm[offsets[e] + i] / xdiv;
-        float amax = 0.f;
-        if constexpr (!BLK) {
-            for (int gi = lane; gi < groups; gi += 64) {
-                float v[8];
-                load8<XT>(x, row * cols + gi * 8, v);
-#pragma unroll
-                for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-            }
-            amax = wave_max(amax);
-        }
-        float mul = amax > 0.f ? kOperandMax<F8> / amax : 0.f;
-        if (lane == 0) scale[int64_t(tile_index) * 32 + r] = BLK ? 1.f : amax / kOperandMax<F8>;
-        for (int gi = lane; gi < groups; gi += 64) {
-            float v[8];
-            load8<XT>(x, row * cols + gi * 8, v);
-            if constexpr (BLK) {   // the block's own scale (its four lanes run together: cols is a multiple of 32)
-                amax = 0.f;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-                amax = quad_max(amax);
-                mul = amax > 0.f ? kOperandMax<F8> / amax : 0.f;
-                if ((gi & 3) == 0) block_scale[(int64_t(tile_index) * (cols / 32) + (gi >> 2)) * 32 + r] = amax / kOperandMax<F8>;
-            }
-            const uint32_t wd[2] = {pack4_q<F8>(v[0] * mul, v[1] * mul, v[2] * mul, v[3] * mul), pack4_q<F8>(v[4] * mul, v[5] * mul, v[6] * mul, v[7] * mul)};
-            const int sub = gi >> 2, d0 = 2 * (gi & 3);
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int p = plane_pos(d0 + h);          // dword of the 32-byte block; its half p / 4 is the lane group g
-                tile[sub * 256 + ((p >> 2) * 32 + r) * 4 + (p & 3)] = wd[h];
-            }
-        }
-    }
-}
-
-// The same for row lengths that are a multiple of 256 up to 2048: one block per row tile. A wave quantises eight rows out of registers
-// (one read of the input) into an LDS copy of the tile, every 32-byte block already in operand order; then lane (g, r)
-// of every wave moves the 16 bytes of row r, half g of one k-step at a time, so each k-step's 1 KB leaves as one fully
-// coalesced store instead of 256 scattered dwords.
-template <int XT, int GPL, bool F8, bool BLK = false>   // groups of 8 values per lane: 512 (GPL - 1) < cols <= 512 GPL
-__global__ __launch_bounds__(256) void group_rows_tile_k(const void * __restrict__ x, int cols, const int * __restrict__ counts, const int * __restrict__ offsets,
-                                                              const int * __restrict__ perm, int experts, int xdiv, int8_t * __restrict__ q, float * __restrict__ scale,
-                                                              Plan plan, float * __restrict__ block_scale = nullptr) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t tile_rows[];   // [32][cols + 16]
-    const int tile_index = int(blockIdx.x);
-    if (tile_index >= plan.tile_base[experts]) return;
-    const int e = owner_of(plan.tile_base, experts, tile_index);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, stride = cols + 16;
-    const int cnt = counts[e], first = (tile_index - plan.tile_base[e]) * 32, off = offsets[e];
-    constexpr int kBatch = GPL == 3 ? 2 : 8 / GPL;   // rows whose loads are in flight together: about 64 values per lane
-    const int groups = cols / 8;
-    for (int r0 = wave * 8; r0 < wave * 8 + 8; r0 += kBatch) {
-        if (first + r0 >= cnt) break;
-        float v[kBatch][GPL][8];
-#pragma unroll
-        for (int b = 0; b < kBatch; ++b) {
-            const int i = min(first + r0 + b, cnt - 1);          // past the count: a valid row again, not stored
-            const int64_t row = perm[off + i] / xdiv;
-#pragma unroll
-            for (int gq = 0; gq < GPL; ++gq) {
-                if (lane + 64 * gq < groups) load8<XT>(x, row * cols + (lane + 64 * gq) * 8, v[b][gq]);
-                else
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) v[b][gq][j] = 0.f;
-            }
-        }
-#pragma unroll
-        for (int b = 0; b < kBatch; ++b) {
-            const int r = r0 + b;
-            float amax = 0.f;
-#pragma unroll
-            for (int gq = 0; gq < GPL; ++gq)
-#pragma unroll
-                for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[b][gq][j]));
-            if constexpr (!BLK) amax = wave_max(amax);
-            float mul = amax > 0.f ? kOperandMax<F8> / amax : 0.f;
-            // (a scale per block: the four lanes of a block hold its values in the same gq, and take every branch below together)
-            float bmax[GPL];
-            if constexpr (BLK) {
-#pragma unroll
-                for (int gq = 0; gq < GPL; ++gq) {
-                    float m = 0.f;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[b][gq][j]));
-                    bmax[gq] = quad_max(m);
-                }
-            }
-            if (first + r < cnt) {
-                if (lane == 0) scale[int64_t(tile_index) * 32 + r] = BLK ? 1.f : amax / kOperandMax<F8>;
-#pragma unroll
-                for (int gq = 0; gq < GPL; ++gq) {
-                    const int gi = lane + 64 * gq, sub = gi >> 2, d0 = 2 * (gi & 3);
-                    if (gi >= groups) break;
-                    if constexpr (BLK) {
-                        mul = bmax[gq] > 0.f ? kOperandMax<F8> / bmax[gq] : 0.f;
-                        if ((gi & 3) == 0) block_scale[(int64_t(tile_index) * (cols / 32) + sub) * 32 + r] = bmax[gq] / kOperandMax<F8>;
-                    }
-                    const float * vv = v[b][gq];
-                    const uint32_t wd[2] = {pack4_q<F8>(vv[0] * mul, vv[1] * mul, vv[2] * mul, vv[3] * mul), pack4_q<F8>(vv[4] * mul, vv[5] * mul, vv[6] * mul, vv[7] * mul)};
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) *reinterpret_cast<uint32_t *>(tile_rows + r * stride + sub * 32 + plane_pos(d0 + h) * 4) = wd[h];
-                }
-            }
-        }
-    }
-    __syncthreads();
-    const int r = lane & 31, g = lane >> 5;
-    if (first + r >= cnt) return;                     // rows past the expert's count are left as they are
-    uint4 * dst = reinterpret_cast<uint4 *>(q + int64_t(tile_index) * 32 * cols) + lane;
-    const int S = cols / 32;
-    for (int ks = wave; ks < S; ks += 4) dst[ks * 64] = *reinterpret_cast<const uint4 *>(tile_rows + r * stride + ks * 32 + g * 16);
-}
-
-// The same grouped operand from rows that are already int8 (quant_rows_k's output: one scale per row, the bytes of every
-// 32-block in operand order): a pure copy. One block per row tile; lane (g, r) of every wave moves the 16 bytes of row r,
-// half g of one k-step at a time, so each k-step's 1 KB is written by one fully coalesced store. When several
-// assignments read one input row (xdiv > 1) the row is quantised once instead of once per assignment.
-// block_scale: rs holds a scale per row and 32-value block ([rows][cols / 32]); they go to block_scale
-// [row tile][block][32 rows] and the rows' own scales are 1.
-__global__ __launch_bounds__(256) void gather_rows_i8_k(const int8_t * __restrict__ rq, const float * __restrict__ rs, int cols, const int * __restrict__ counts,
-                                                          const int * __restrict__ offsets, const int * __restrict__ perm, int experts, int xdiv,
-                                                          int8_t * __restrict__ q, float * __restrict__ scale, Plan plan, float * __restrict__ block_scale = nullptr) {
-    const int tile_index = int(blockIdx.x);
-    if (tile_index >= plan.tile_base[experts]) return;
-    const int e = owner_of(plan.tile_base, experts, tile_index);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, g = lane >> 5;
-    const int i = (tile_index - plan.tile_base[e]) * 32 + r;
-    if (i >= counts[e]) return;                       // rows past the expert's count are left as they are
-    const int64_t row = perm[offsets[e] + i] / xdiv;
-    const int S = cols / 32;
-    if (wave == 0 && g == 0) scale[int64_t(tile_index) * 32 + r] = block_scale ? 1.f : rs[row];
-    const uint4 * src = reinterpret_cast<const uint4 *>(rq + row * cols) + g;
-    uint4 * dst = reinterpret_cast<uint4 *>(q + int64_t(tile_index) * 32 * cols) + lane;
-    for (int ks = wave; ks < S; ks += 4) dst[ks * 64] = src[ks * 2];
-    if (block_scale && g == 0)
-        for (int ks = wave; ks < S; ks += 4) block_scale[(int64_t(tile_index) * S + ks) * 32 + r] = rs[row * S + ks];
 }
 
 typedef float v16f __attribute__((ext_vector_type(16)));

@@ -584,6 +584,7 @@ template <class W> __device__ __forceinline__ void acc_step2(Acc<W> & a, v4i x0,
         const float d0 = W::d_sub(r, ib0), d1 = W::d_sub(r, ib0 + 1);
 #pragma unroll
         for (int i = 0; i < 16; ++i) a.sum[i] = __fmaf_rn(float(s1[i]), d1, __fmaf_rn(float(s0[i]), d0, a.sum[i]));
+        asm volatile("" : "+v"(a.sum));   // (pinned: see acc_step2_blocks)
     } else {
         const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll

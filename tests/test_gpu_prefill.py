@@ -264,6 +264,30 @@ def test_grouped_products_block_scales_against_float64(tq, oracle, n, shared_ff,
         assert np.abs(y[a] - want).max() < 2e-3 * max(1e-3, np.abs(want).max()), a
 
 
+@pytest.mark.parametrize("cols", [2304, 4096])
+def test_group_rows_blocks_long_rows(tq, cols):
+    """Rows longer than 2048 values take the grouping kernel that works row by row: the same bytes and block scales as the
+    plain block quantiser's rows, gathered."""
+    rng = np.random.default_rng(cols)
+    n, experts, k = 45, 5, 2
+    ids = np.stack([rng.permutation(experts)[:k] for _ in range(n)]).astype(np.int32)
+    x = torch.from_numpy(rng.standard_normal((n, cols)).astype(np.float32) * np.repeat(10.0 ** rng.uniform(-2, 1, (n, cols // 32)), 32, axis=1).astype(np.float32))
+    x = x.cuda().to(torch.float16)
+    counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), experts)
+    lists = (counts, offsets, perm)
+    want_counts = np.bincount(ids.reshape(-1), minlength=experts)
+    xq, xs, xbs = tq.group_rows_i8_blocks(x, lists, n * k, k)
+    pq, ps, _ = tq.quant_rows_i8_blocks(x, sums=False)
+    uq, us = ungroup(xq.cpu().numpy(), xs.cpu().numpy(), want_counts, perm.cpu().numpy(), n * k)
+    ub = ungroup_block_scales(xbs.cpu().numpy(), want_counts, perm.cpu().numpy(), n * k, cols // 32)
+    tok = np.arange(n * k) // k
+    assert np.array_equal(uq, natural_order(pq.cpu().numpy())[tok])
+    assert np.array_equal(ub, ps.cpu().numpy()[tok]) and (us == 1).all()
+    gq, gs, gbs = tq.gather_rows_i8_blocks(pq, ps, lists, n * k, k)
+    assert np.array_equal(ungroup(gq.cpu().numpy(), gs.cpu().numpy(), want_counts, perm.cpu().numpy(), n * k)[0], uq)
+    assert np.array_equal(ungroup_block_scales(gbs.cpu().numpy(), want_counts, perm.cpu().numpy(), n * k, cols // 32), ub)
+
+
 def test_block_scale_products_refuse_fp8_banks_and_missing_scales(tq, oracle):
     decs, (gate, up, down), ids, slots, banks = grouped_setup(tq, oracle, 3, 4, 256, 256, 8, 2, False, oracle.NVFP4G)
     counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), banks)

@@ -33,7 +33,8 @@ def test_router_logits(tq, oracle, name, n):
 
 
 @pytest.mark.parametrize("n,e,h,shared", [(32, 512, 2048, True), (100, 33, 512, False), (4096, 512, 2048, True), (77, 64, 192, True),
-                                          (250, 600, 512, False), (1000, 130, 192, True), (9000, 1100, 256, True)])
+                                          (250, 600, 512, False), (1000, 130, 192, True), (9000, 1100, 256, True),
+                                          (2100, 64, 320, True), (4096, 100, 2048, False)])   # few router rows: eight waves a block
 def test_router_gemm_path(tq, oracle, n, e, h, shared):
     """bf16 router rows and bf16 inputs take the matrix-pipe kernel from about 120,000 tokens x rows (64-token blocks, 128-token
     blocks for the largest grids), the wave-per-row kernel below: same logits to the same bar, ragged token and row counts,

@@ -119,33 +119,38 @@ constexpr int kRouterGemmMin = 120000;   // tokens x router rows from which a bf
                                          // takes 10 us up to 16,000 and grows with tokens x rows)
 constexpr int kRgTok = 64, kRgRows = 64, kRgK = 256, kRgPad = kRgK + 8;   // halves per staged row: 16-byte reads of consecutive rows spread over the banks
 
-// F32: the rows are fp32 (h counts 2-byte units here: twice the columns); else bf16
-template <bool F32>
-__global__ __launch_bounds__(256) void router_gemm_k(const uint16_t * __restrict__ w, const uint16_t * __restrict__ shared, const uint16_t * __restrict__ x,
+// F32: the rows are fp32 (h counts 2-byte units here: twice the columns); else bf16.
+// KS = 2: eight waves, the second four take the second half of every stage's steps and hand their sums to the first four
+// through LDS at the end (first half + second half, a fixed order): for grids that leave most compute units without a
+// block, where a block's own chain of stages is the whole time.
+template <bool F32, int KS = 1>
+__global__ __launch_bounds__(256 * KS) void router_gemm_k(const uint16_t * __restrict__ w, const uint16_t * __restrict__ shared, const uint16_t * __restrict__ x,
                                                        float * __restrict__ logits, int h, int e, int n) {
     __shared__ __attribute__((aligned(16))) uint16_t As[kRgTok][kRgPad];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[kRgRows + 1][kRgPad];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
     const int t0 = int(blockIdx.x) * kRgTok, r0 = int(blockIdx.y) * kRgRows;
     const bool last = blockIdx.y == gridDim.y - 1;     // this block also has row e (the shared gate, or zeros)
-    const int mq = wave & 1, nq = wave >> 1;           // quadrant: tokens 32 mq.., router rows 32 nq..
+    const int mq = wave & 1, nq = (wave >> 1) & 1;     // quadrant: tokens 32 mq.., router rows 32 nq..
+    const int kh = wave >> 2;                          // which part of every stage's steps (0 when KS == 1)
     const bool extra = last && nq == 0;
-    // staging: thread -> 16-byte piece sp of rows sr, sr + 8, ... of both tiles (a wave's loads cover two whole rows of 512 bytes)
+    // staging: thread -> 16-byte piece sp of rows sr, sr + 8 KS, ... of both tiles (a wave's loads cover two whole rows of 512 bytes)
+    constexpr int SR = 8 / KS;                         // rows of each tile a thread stages
     const int sp = tid & 31, sr = tid >> 5;
-    const uint16_t * a_src[8], * b_src[8];
-    bool b_zero[8];
+    const uint16_t * a_src[SR], * b_src[SR];
+    bool b_zero[SR];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        a_src[i] = x + int64_t(min(t0 + sr + 8 * i, n - 1)) * h + 8 * sp;   // rows past the end repeat a valid row (not stored)
-        const int row = r0 + sr + 8 * i;
+    for (int i = 0; i < SR; ++i) {
+        a_src[i] = x + int64_t(min(t0 + sr + 8 * KS * i, n - 1)) * h + 8 * sp;   // rows past the end repeat a valid row (not stored)
+        const int row = r0 + sr + 8 * KS * i;
         b_zero[i] = row >= e;
         b_src[i] = w + int64_t(min(row, e - 1)) * h + 8 * sp;
     }
-    uint4 a_st[8], b_st[8], x_st = make_uint4(0, 0, 0, 0);
+    uint4 a_st[SR], b_st[SR], x_st = make_uint4(0, 0, 0, 0);
     auto fetch = [&](int k0) {
         const bool in = k0 + 8 * sp < h;   // the last stage may be narrower
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < SR; ++i) {
             a_st[i] = in ? *reinterpret_cast<const uint4 *>(a_src[i] + k0) : make_uint4(0, 0, 0, 0);
             b_st[i] = in && !b_zero[i] ? *reinterpret_cast<const uint4 *>(b_src[i] + k0) : make_uint4(0, 0, 0, 0);
         }
@@ -153,9 +158,9 @@ __global__ __launch_bounds__(256) void router_gemm_k(const uint16_t * __restrict
     };
     auto stage = [&]() {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            *reinterpret_cast<uint4 *>(&As[sr + 8 * i][8 * sp]) = a_st[i];
-            *reinterpret_cast<uint4 *>(&Bs[sr + 8 * i][8 * sp]) = b_st[i];
+        for (int i = 0; i < SR; ++i) {
+            *reinterpret_cast<uint4 *>(&As[sr + 8 * KS * i][8 * sp]) = a_st[i];
+            *reinterpret_cast<uint4 *>(&Bs[sr + 8 * KS * i][8 * sp]) = b_st[i];
         }
         if (last && tid < 32) *reinterpret_cast<uint4 *>(&Bs[kRgRows][8 * sp]) = x_st;
     };
@@ -197,14 +202,36 @@ __global__ __launch_bounds__(256) void router_gemm_k(const uint16_t * __restrict
         };
         if (steps == kRgK / 16) {
 #pragma unroll
-            for (int j = 0; j < kRgK / 16; ++j) step(j);
+            for (int j = 0; j < kRgK / 16 / KS; ++j) step(kh * (kRgK / 16 / KS) + j);
         } else {
-            for (int j = 0; j < steps; ++j) step(j);
+            const int per = (steps + KS - 1) / KS;
+            for (int j = kh * per; j < min(steps, (kh + 1) * per); ++j) step(j);
         }
     }
     if constexpr (F32) {
 #pragma unroll
         for (int q = 0; q < 16; ++q) acc[q] = (acc[q] + acc1[q]) + (acc2[q] + acc3[q]);
+    }
+    if constexpr (KS == 2) {   // the second part's sums to the first part's waves, through the space of the row tiles
+        __syncthreads();       // the last stage has been multiplied
+        float * ex = reinterpret_cast<float *>(&As[0][0]);   // [quadrant][17 registers][64 lanes] floats: 17.4 KB of As's 33.8 KB
+        static_assert(sizeof(As) >= 4 * 17 * 64 * sizeof(float), "exchange space");
+        if (kh == 1) {
+#pragma unroll
+            for (int q = 0; q < 16; ++q) ex[((wave & 3) * 17 + q) * 64 + lane] = acc[q];
+            if (extra) {
+#pragma unroll
+                for (int q = 0; q < 16; ++q) if (r == 0) ex[((wave & 3) * 17 + 16) * 64 + 16 * g + q] = accx[q];
+            }
+        }
+        __syncthreads();
+        if (kh == 1) return;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[q] += ex[((wave & 3) * 17 + q) * 64 + lane];
+        if (extra && r == 0) {
+#pragma unroll
+            for (int q = 0; q < 16; ++q) accx[q] += ex[((wave & 3) * 17 + 16) * 64 + 16 * g + q];
+        }
     }
     // result register q of lane half g: token row 8 (q / 4) + 4 g + q % 4 of the 32-row tile, router row r
     const int row = r0 + nq * 32 + r;
@@ -785,8 +812,16 @@ extern "C" int32_t tqmoe_router(const void * router, uint32_t wtype, const void 
     if (wtype == xtype && (wtype == TQMOE_BF16 || wtype == TQMOE_F32) && int64_t(n) * (experts + 1) >= kRouterGemmMin && hidden % 64 == 0) {
         const dim3 grid(unsigned((n + kRgTok - 1) / kRgTok), unsigned((experts + kRgRows - 1) / kRgRows));
         const uint16_t * w16 = static_cast<const uint16_t *>(router), * s16 = static_cast<const uint16_t *>(shared_gate), * x16 = static_cast<const uint16_t *>(x);
-        if (wtype == TQMOE_F32) router_gemm_k<true><<<grid, 256, 0, s>>>(w16, s16, x16, logits, 2 * hidden, experts, n);
-        else router_gemm_k<false><<<grid, 256, 0, s>>>(w16, s16, x16, logits, hidden, experts, n);
+        // a layer of few experts has few blocks: eight waves a block then, the steps of every stage split between two sets
+        // of four (decided by the router rows alone, so that a token's logits do not depend on the batch around it)
+        const bool split = grid.y <= 2;
+        if (wtype == TQMOE_F32) {
+            if (split) router_gemm_k<true, 2><<<grid, 512, 0, s>>>(w16, s16, x16, logits, 2 * hidden, experts, n);
+            else router_gemm_k<true><<<grid, 256, 0, s>>>(w16, s16, x16, logits, 2 * hidden, experts, n);
+        } else {
+            if (split) router_gemm_k<false, 2><<<grid, 512, 0, s>>>(w16, s16, x16, logits, hidden, experts, n);
+            else router_gemm_k<false><<<grid, 256, 0, s>>>(w16, s16, x16, logits, hidden, experts, n);
+        }
         return launched(err, "tqmoe_router");
     }
     if (wtype == TQMOE_F32) launch_router_x<TQMOE_F32>(xtype, router, shared_gate, x, logits, hidden, experts, n, s);

@@ -95,9 +95,28 @@ int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets,
  * ends), whose address is looked up on the first call on a device. Limit: ceil(n * topk / 1024) * experts <= 1,048,576
  * (for 512 experts about two million assignments), beyond it TQMOE_E_WORKSPACE. Calls on one GPU share that array:
  * two calls that overlap in time on the same GPU (different streams) race; calls on one stream are ordered. Nothing
- * in the array needs clearing between calls (every entry a call reads, it has written first). */
+ * in the array needs clearing between calls (every entry a call reads, it has written first).
+ * offsets and perm may be NULL when groups is given: counts + groups alone are what tqllm_cuda::moe_group
+ * (moe_kernels.cuh:29) produces, and with capacity = n this call is that function with ascending lists.
+ * The array's address is looked up on the first call on a device (a module load may happen then): a caller that will
+ * capture the call into a HIP graph calls tqmoe_static_scratch_init() once per device beforehand. */
 int32_t tqmoe_dispatch_static(const int32_t * ids, int32_t * counts, int32_t * offsets, int32_t * perm, int32_t * groups,
                               int32_t capacity, int32_t experts, int32_t n, int32_t topk, void * stream, tqmoe_error * err);
+int32_t tqmoe_static_scratch_init(tqmoe_error * err);
+
+/* counts[ids[i]] += 1 for i < count, 64-bit counters that run on over many calls (ids < 0 skipped): the routing histogram
+ * tqllm_cuda::moe_count (moe_kernels.cuh, moe.cu:183-186). */
+int32_t tqmoe_count(const int32_t * ids, uint64_t * counts, int32_t count, void * stream, tqmoe_error * err);
+
+/* Slot and de-duplication maps of one routed decode call, tqllm_cuda::moe_dedup_maps (moe_kernels.cuh:34-39, moe.cu:453-493)
+ * with the map layout of src/formats/weight/quant_kernels.cuh:26-27 (kDedupCols = 8, kDedupStride = 18):
+ *   slots[a] = slot_of[ids[a]] (-1 for ids[a] < 0), a < count <= 1024; slots may be NULL;
+ *   gu / dn: `groups` entries of 18 ints each (groups >= count; either may be NULL). The assignments of a slot, in ascending a,
+ *   are cut into runs of up to 8; every run is one entry {slot, columns, input row x 8, output row x 8}; entries are numbered
+ *   in the order of their first assignment; input row = a / topk in gu and a in dn, output row = a; unused columns and the
+ *   entries behind the last run hold -1. The result is deterministic. */
+int32_t tqmoe_dedup_maps(const int32_t * ids, const int32_t * slot_of, int32_t count, int32_t topk, int32_t * slots, int32_t * gu,
+                         int32_t * dn, int32_t groups, void * stream, tqmoe_error * err);
 
 /* -------------------------------------------------------------------------------------------------- banks
  * A bank is one projection of every expert: `experts` matrices of rows x cols stacked row-wise, expert e at row
@@ -225,6 +244,11 @@ int32_t tqmoe_expert_down(const tqmoe_bank * down, const void * act_image, float
 /* act[i] = silu(gate[i]) * up[i], fp32 in and out (the reference's moe_swiglu, moe_kernels.cuh:71-72, rounds its
  * bf16 inputs' product through bf16 to fp16; here nothing is rounded below fp32). */
 int32_t tqmoe_swiglu(const float * gate, const float * up, float * act, int64_t count, void * stream, tqmoe_error * err);
+/* the same with the reference's optional clamp (MoeConfig::swiglu_clamp, src/experts/moe.hpp:34-36; moe_expert_ffn,
+ * src/experts/moe.cpp:128-143): swiglu_clamp <= 1e-6: none; else up goes to [-swiglu_clamp, swiglu_clamp] and either the gate
+ * to at most swiglu_clamp before the activation (clamp_gate nonzero) or silu(gate) to at most swiglu_clamp after it. */
+int32_t tqmoe_swiglu_clamped(const float * gate, const float * up, float * act, int64_t count, float swiglu_clamp, int32_t clamp_gate,
+                             void * stream, tqmoe_error * err);
 
 /* out[t][j] = sum_s weights[t][s] * routed[t * topk + s][j] (s ascending) + shared_weights[t] * shared[t][j];
  * routed / shared fp32, shared and shared_weights may be NULL together; out of otype (F32 or BF16).
@@ -358,6 +382,28 @@ int32_t tqmoe_expert_gemm(const tqmoe_bank * bank, const void * x, uint32_t xtyp
  * The order inside an expert is kept; the products do not depend on it. */
 int32_t tqmoe_lists_from_groups(const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts,
                                 int32_t * offsets, int32_t * perm, void * stream, tqmoe_error * err);
+/* The same, and counts_out [experts] = min(counts, capacity): the counts the grouped products must be given with these lists
+ * (with the caller's own counts an expert whose count exceeds the capacity would run past its span of perm). */
+int32_t tqmoe_lists_from_groups_clamped(const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts,
+                                        int32_t * counts_out, int32_t * offsets, int32_t * perm, void * stream, tqmoe_error * err);
+
+/* WeightFormat::expert_gemm_i8 with the reference's own operands (weight_format.hpp:54-56; called from
+ * src/models/qwen/qwen4exp/fn_prefill.cpp:192-194 on the rows k_quant_act_rows leaves, quant_kernels.cuh:13-19):
+ *   xq    device int8 [input rows][cols], natural order;
+ *   xs    device fp32 [input rows][cols / 32]: mode 1 the blocks' scales, mode 2 the token's scale in every entry ([row][0] is read);
+ *   xsum  the reference's int16 sums per 16 values: not read (may be NULL);
+ *   counts [experts], groups [experts][capacity]: the reference's lists of assignment indices a; input row a / topk, or a with
+ *   per_expert_input; experts must be the bank's;
+ *   y     device [assignments][bank rows] of ytype (BF16 as the reference, or F16); rows of unlisted assignments stay untouched.
+ * One call enqueues the list conversion, the arranging of the rows into the operand tiles and the product.
+ * max_assignments bounds the listed assignments (n * topk of the pass); scratch: device memory of
+ * tqmoe_expert_gemm_i8_ref_scratch_bytes(experts, max_assignments, cols, mode), dead after the call.
+ * TQMOE_E_UNSUPPORTED (the base class's `false`): no int8 grouped product for the bank's format. */
+size_t  tqmoe_expert_gemm_i8_ref_scratch_bytes(int32_t experts, int64_t max_assignments, int32_t cols, int32_t mode);
+int32_t tqmoe_expert_gemm_i8_ref(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const int16_t * xsum, void * y, uint32_t ytype,
+                                 const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts, int32_t topk,
+                                 int32_t per_expert_input, int32_t mode, int64_t max_assignments, void * scratch, size_t scratch_bytes,
+                                 void * stream, tqmoe_error * err);
 
 /* tqmoe_combine_strided with fp16 rows (the prefill products' output) */
 int32_t tqmoe_combine_strided_f16(const void * routed, int32_t slots, const void * shared, int64_t shared_ld,
@@ -391,8 +437,8 @@ int32_t tqmoe_add_rmsnorm(void * rows, const void * residual, const float * weig
  * The shared expert, when has_shared, is expert index n_expert of the three banks (so banks hold n_expert + 1
  * matrices), uses the first shared_ff rows of gate / up and the first shared_ff columns of down, and is weighted by
  * sigmoid(router logit column n_expert), or by 1 when shared_gate is NULL (an always-on shared expert without a gate row).
- * MoeConfig::swiglu_clamp (src/experts/moe.hpp) is not carried: the fused SwiGLU is unclamped, a model that clamps runs
- * the modular entry points with its own activation step. */
+ * MoeConfig::swiglu_clamp (src/experts/moe.hpp:34-36) and the clamp_gate switch of moe_expert_ffn (src/experts/moe.cpp:115-143)
+ * are the descriptor's last two fields. */
 typedef struct tqmoe_layer {
     uint32_t struct_size;
     int32_t hidden, ff, n_expert, topk;
@@ -411,6 +457,12 @@ typedef struct tqmoe_layer {
      * descriptor that ends before this field) = one scale per token (its value 2), nonzero = one per 32 values (its
      * value 1). The fp8 and fp16 grouped products and the decode kernels ignore it. */
     int32_t act_blocks;
+    /* Clamp of the SwiGLU inputs, applied in the fused gate / up epilogues of every path (routed and shared experts alike).
+     * swiglu_clamp <= 1e-6 (or a descriptor that ends before this field): none. Else up is clamped to
+     * [-swiglu_clamp, swiglu_clamp] and either the gate to at most swiglu_clamp before the activation (clamp_gate nonzero:
+     * the GLM branch) or silu(gate) to at most swiglu_clamp after it (clamp_gate zero), as moe_expert_ffn does. */
+    float swiglu_clamp;
+    int32_t clamp_gate;
 } tqmoe_layer;
 
 size_t  tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t n);

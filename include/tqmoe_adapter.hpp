@@ -83,25 +83,30 @@ inline void moe_sum_add(const float * routed, const float * shared, const float 
     tqmoe_error e = fresh();
     check(tqmoe_combine_residual(routed, TQMOE_F32, topk, shared, hidden, weights, shared_weights, m_bf16, x_bf16, hidden, topk, n, stream, &e), e);
 }
-// moe_group (moe_kernels.cuh:29): groups [experts][n], counts [experts]. The lists are ascending inside each expert
-// (the reference's device version is atomic-ordered). `scratch` holds the offsets, the permutation and the workspace:
-// moe_group_scratch_bytes() device bytes.
-inline size_t moe_group_scratch_bytes(int experts, int n, int topk) {
-    return size_t(experts + 1) * 4 + size_t(n) * topk * 4 + 512 + tqmoe_dispatch_workspace_bytes(experts, n, topk);
-}
-inline void moe_group(const int * ids, int * counts, int * groups, int experts, int n, int topk, void * scratch, void * stream) {
+// moe_group (moe_kernels.cuh:29), the reference's signature: groups [experts][n], counts [experts]; negative ids are skipped.
+// The lists are ascending inside each expert (the reference's device version is atomic-ordered). No workspace: the chunk
+// counts live in the library's own device image (tqmoe_dispatch_static), so calls that overlap in time on one GPU must not
+// be issued from two streams.
+inline void moe_group(const int * ids, int * counts, int * groups, int experts, int n, int topk, void * stream) {
     tqmoe_error e = fresh();
-    char * p = static_cast<char *>(scratch);
-    int32_t * offsets = reinterpret_cast<int32_t *>(p);
-    size_t at = (size_t(experts + 1) * 4 + 255) / 256 * 256;
-    int32_t * perm = reinterpret_cast<int32_t *>(p + at);
-    at = (at + size_t(n) * topk * 4 + 255) / 256 * 256;
-    check(tqmoe_dispatch(ids, counts, offsets, perm, groups, n, experts, n, topk, p + at, tqmoe_dispatch_workspace_bytes(experts, n, topk), stream, &e), e);
+    check(tqmoe_dispatch_static(ids, counts, nullptr, nullptr, groups, n, experts, n, topk, stream, &e), e);
 }
-// moe_swiglu (moe_kernels.cuh:71-72), fp32 in and out here
-inline void moe_swiglu(const float * gate, const float * up, float * act, int count, void * stream) {
+// moe_count (moe_kernels.cuh, moe.cu:183-186): counts[ids[i]] += 1, 64-bit counters
+inline void moe_count(const int * ids, unsigned long long * counts, int count, void * stream) {
     tqmoe_error e = fresh();
-    check(tqmoe_swiglu(gate, up, act, count, stream, &e), e);
+    check(tqmoe_count(ids, reinterpret_cast<uint64_t *>(counts), count, stream, &e), e);
+}
+// moe_dedup_maps (moe_kernels.cuh:34-39) with the map layout of quant_kernels.cuh:26-27
+constexpr int kDedupCols = 8, kDedupStride = 2 + 2 * kDedupCols;
+inline void moe_dedup_maps(const int * ids, const int * slot_of, int count, int topk, int * slots, int * gu, int * dn, int groups, void * stream) {
+    tqmoe_error e = fresh();
+    check(tqmoe_dedup_maps(ids, slot_of, count, topk, slots, gu, dn, groups, stream, &e), e);
+}
+// moe_swiglu (moe_kernels.cuh:71-72), fp32 in and out here; swiglu_clamp / clamp_gate: MoeConfig::swiglu_clamp and the switch
+// of moe_expert_ffn (src/experts/moe.hpp:34-36, moe.cpp:128-143), off by default
+inline void moe_swiglu(const float * gate, const float * up, float * act, int count, void * stream, float swiglu_clamp = 0.f, bool clamp_gate = false) {
+    tqmoe_error e = fresh();
+    check(tqmoe_swiglu_clamped(gate, up, act, count, swiglu_clamp, clamp_gate ? 1 : 0, stream, &e), e);
 }
 // moe_sum (moe_kernels.cuh:73-74): routed / shared fp32 here, out bf16 as there
 inline void moe_sum(const float * routed, const float * shared, const float * weights, const float * shared_weights, void * out_bf16, int hidden, int topk, int n,
@@ -243,10 +248,12 @@ struct ExpertFormat {
 // grouped call (n * topk of the pass; 0 = experts * capacity, always safe, costs idle blocks). Return values and
 // exceptions are the base's: false = "no such kernel for this format, fall back", std::invalid_argument on bad shapes,
 // std::runtime_error on device errors.
-inline size_t expert_scratch_bytes(int cols, int input_rows, int max_assignments, int experts) {
+// int8_mode: 0 = no expert_gemm_i8 calls, else the largest mode they will pass (1 needs room for the block scales too)
+inline size_t expert_scratch_bytes(int cols, int input_rows, int max_assignments, int experts, int int8_mode = 0) {
     const size_t image = tqmoe_act_image_bytes(input_rows, cols);
-    const size_t lists = (size_t(experts) + 1 + size_t(max_assignments)) * 4 + 512;
-    return image > lists ? image : lists;
+    const size_t lists = (2 * size_t(experts) + 1 + size_t(max_assignments)) * 4 + 1024;
+    const size_t i8 = int8_mode ? tqmoe_expert_gemm_i8_ref_scratch_bytes(experts, max_assignments, cols, int8_mode == 1 ? 1 : 2) : 0;
+    return image > lists ? (image > i8 ? image : i8) : (lists > i8 ? lists : i8);
 }
 
 template <class Base, class MatT, class HalfT, class Bf16T, class StreamT>
@@ -275,39 +282,59 @@ struct ExpertOverrides : Base {
         const tqmoe_bank bg = bank_of(g, rows), bu = bank_of(u, rows);
         check(tqmoe_expert_matvec2_rows(&bg, &bu, x, TQMOE_F16, yg, yu, TQMOE_BF16, ids, n, topk, scratch, scratch_bytes, (void *)stream, &e), e);
     }
-    // the lists in this library's form, in the scratch: offsets [experts + 1], then perm
-    bool lists(const int * counts, const int * groups, int capacity, int experts, int32_t *& offsets, int32_t *& perm, int64_t & bound, StreamT stream) const {
-        bound = max_assignments > 0 ? max_assignments : int64_t(experts) * capacity;
-        const size_t at = (size_t(experts + 1) * 4 + 255) / 256 * 256;
-        if (!scratch || scratch_bytes < at + size_t(bound) * 4) throw std::invalid_argument("tqmoe adapter: scratch too small for the dispatch lists");
-        offsets = static_cast<int32_t *>(scratch);
-        perm = reinterpret_cast<int32_t *>(static_cast<char *>(scratch) + at);
+    // the lists in this library's form, in the scratch: the counts clamped to the capacity [experts], offsets [experts + 1],
+    // then perm. The products are given the clamped counts: a count above the capacity names entries the lists do not hold.
+    struct Lists { int32_t * counts, * offsets, * perm; int64_t bound; };
+    Lists lists(const MatT & m, int rows, const int * counts, const int * groups, int capacity, int experts, StreamT stream) const {
+        if (rows <= 0 || m.rows != int64_t(experts) * rows) throw std::invalid_argument("tqmoe adapter: the lists' expert count differs from the bank's");
+        Lists l{};
+        l.bound = max_assignments > 0 ? max_assignments : int64_t(experts) * capacity;
+        const size_t at0 = (size_t(experts) * 4 + 255) / 256 * 256, at1 = at0 + (size_t(experts + 1) * 4 + 255) / 256 * 256;
+        if (!scratch || scratch_bytes < at1 + size_t(l.bound) * 4) throw std::invalid_argument("tqmoe adapter: scratch too small for the dispatch lists");
+        char * p = static_cast<char *>(scratch);
+        l.counts = reinterpret_cast<int32_t *>(p);
+        l.offsets = reinterpret_cast<int32_t *>(p + at0);
+        l.perm = reinterpret_cast<int32_t *>(p + at1);
         tqmoe_error e = fresh();
-        check(tqmoe_lists_from_groups(counts, groups, capacity, experts, offsets, perm, (void *)stream, &e), e);
-        return true;
+        check(tqmoe_lists_from_groups_clamped(counts, groups, capacity, experts, l.counts, l.offsets, l.perm, (void *)stream, &e), e);
+        return l;
     }
     bool expert_gemm(const MatT & m, const HalfT * x, Bf16T * y, int rows, const int * counts, const int * groups, int capacity, int experts, int topk,
                      bool per_expert_input, StreamT stream) const override {
-        int32_t * offsets, * perm;
-        int64_t bound;
-        lists(counts, groups, capacity, experts, offsets, perm, bound, stream);
+        const Lists l = lists(m, rows, counts, groups, capacity, experts, stream);
         tqmoe_error e = fresh();
         const tqmoe_bank b = bank_of(m, rows);
-        const int32_t n = int32_t((bound + topk - 1) / topk);
-        const int32_t rc = tqmoe_expert_gemm(&b, x, TQMOE_F16, counts, offsets, perm, n, topk, topk, 0, per_expert_input ? 1 : 0, y, TQMOE_BF16, (void *)stream, &e);
+        const int32_t n = int32_t((l.bound + topk - 1) / topk);
+        const int32_t rc = tqmoe_expert_gemm(&b, x, TQMOE_F16, l.counts, l.offsets, l.perm, n, topk, topk, 0, per_expert_input ? 1 : 0, y, TQMOE_BF16, (void *)stream, &e);
         if (rc == TQMOE_E_UNSUPPORTED) return false;
         check(rc, e);
         return true;
     }
     bool expert_gemm_gateup(const MatT & g, const MatT & u, const HalfT * x, HalfT * y, int rows, const int * counts, const int * groups, int capacity,
                             int experts, int topk, StreamT stream) const override {
-        int32_t * offsets, * perm;
-        int64_t bound;
-        lists(counts, groups, capacity, experts, offsets, perm, bound, stream);
+        const Lists l = lists(g, rows, counts, groups, capacity, experts, stream);
         tqmoe_error e = fresh();
         const tqmoe_bank bg = bank_of(g, rows), bu = bank_of(u, rows);
-        const int32_t n = int32_t((bound + topk - 1) / topk);
-        const int32_t rc = tqmoe_expert_gemm_gateup(&bg, &bu, x, TQMOE_F16, counts, offsets, perm, n, topk, topk, 0, y, (void *)stream, &e);
+        const int32_t n = int32_t((l.bound + topk - 1) / topk);
+        const int32_t rc = tqmoe_expert_gemm_gateup(&bg, &bu, x, TQMOE_F16, l.counts, l.offsets, l.perm, n, topk, topk, 0, y, (void *)stream, &e);
+        if (rc == TQMOE_E_UNSUPPORTED) return false;
+        check(rc, e);
+        return true;
+    }
+    // expert_gemm_i8 (weight_format.hpp:54-56) on the reference's own operands: xq int8 [rows_in][cols] in natural order, xs fp32
+    // [rows_in][cols / 32] (mode 1 a scale per 32 values, mode 2 the token's scale in every entry), xsum the int16 sums per 16
+    // values (not read: the minimum term of the formats that have one comes from an operand plane of its own), bf16 rows out.
+    // The scratch holds the lists, the rows arranged into operand tiles and their scales (expert_scratch_bytes with int8_mode).
+    // false: the format has no int8 grouped product (the caller falls back to expert_gemm), or a mode other than 1 and 2.
+    bool expert_gemm_i8(const MatT & m, const int8_t * xq, const float * xs, const int16_t * xsum, Bf16T * y, int rows, const int * counts, const int * groups,
+                        int capacity, int experts, int topk, bool per_expert_input, StreamT stream, int mode) const override {
+        if (rows <= 0 || m.rows != int64_t(experts) * rows) throw std::invalid_argument("tqmoe adapter: the lists' expert count differs from the bank's");
+        if (mode != 1 && mode != 2) return false;
+        tqmoe_error e = fresh();
+        const tqmoe_bank b = bank_of(m, rows);
+        const int64_t bound = max_assignments > 0 ? max_assignments : int64_t(experts) * capacity;
+        const int32_t rc = tqmoe_expert_gemm_i8_ref(&b, xq, xs, xsum, y, TQMOE_BF16, counts, groups, capacity, experts, topk, per_expert_input ? 1 : 0, mode, bound,
+                                                    scratch, scratch_bytes, (void *)stream, &e);
         if (rc == TQMOE_E_UNSUPPORTED) return false;
         check(rc, e);
         return true;

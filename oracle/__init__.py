@@ -49,8 +49,6 @@ _lib.tqo_float_to_e4m3.argtypes = [C.c_float]
 _lib.tqo_dequantize.argtypes = [C.c_uint32, _p, _p, C.c_int64]
 _lib.tqo_quantize.argtypes = [C.c_uint32, _p, _p, C.c_int64, C.c_int64]
 _lib.tqo_route.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _p, _p, _p, _p]
-_lib.tqo_route_min_gap_ulps.restype = C.c_double
-_lib.tqo_route_min_gap_ulps.argtypes = [C.c_int, C.c_int, _p]
 _lib.tqo_route_softmax_collision.argtypes = [C.c_int, C.c_int, _p]
 _lib.tqo_shared_weight.restype = C.c_float
 _lib.tqo_shared_weight.argtypes = [C.c_float]
@@ -81,7 +79,7 @@ class _Layer(C.Structure):
     _fields_ = [("hidden", C.c_int), ("ff", C.c_int), ("n_expert", C.c_int), ("k", C.c_int), ("has_shared", C.c_int),
                 ("shared_ff", C.c_int), ("wtype", C.c_uint32), ("gate", _p), ("up", _p), ("down", _p),
                 ("act_mode", C.c_int), ("threads", C.c_int), ("gating", C.c_int), ("raw_weights", C.c_int),
-                ("weight_scale", C.c_float), ("bias", _p), ("wtype_down", C.c_uint32)]
+                ("weight_scale", C.c_float), ("bias", _p), ("wtype_down", C.c_uint32), ("swiglu_clamp", C.c_float), ("clamp_gate", C.c_int), ("act_out", _p)]
 
 
 _lib.tqo_layer_forward.argtypes = [C.POINTER(_Layer), _p, _p, C.c_int, _p, _p, _p]
@@ -161,11 +159,6 @@ def route(logits, k, gating=GATE_SOFTMAX, norm=True, scale=1.0, bias=None):
         if _lib.tqo_route(gating, e, k, int(norm), float(scale), _ptr(lg[t]), _ptr(b), _ptr(ids[t]), _ptr(w[t])):
             raise ValueError("tqo_route: bad shape")
     return ids, w
-
-
-def route_min_gap_ulps(logits, k):
-    lg = np.atleast_2d(_c(logits, np.float32))
-    return np.array([_lib.tqo_route_min_gap_ulps(lg.shape[1], k, _ptr(lg[t])) for t in range(lg.shape[0])])
 
 
 def route_softmax_collision(logits, k):
@@ -250,20 +243,27 @@ def add_rmsnorm(rows_bits, residual_bits, weight, eps):
 
 
 def layer_forward(x, logits, gate, up, down, wtype, hidden, ff, n_expert, k, shared_ff=0, act_mode=0, threads=8, gating=GATE_SOFTMAX,
-                  norm=True, scale=1.0, bias=None, wtype_down=0):
-    """Whole layer on the host; returns (out [n][H] fp32, ids [n][k], weights [n][k])."""
+                  norm=True, scale=1.0, bias=None, wtype_down=0, swiglu_clamp=0.0, clamp_gate=False, return_act=False):
+    """Whole layer on the host; returns (out [n][H] fp32, ids [n][k], weights [n][k]); with return_act (act modes other than 0)
+    also the rows silu(gate) * up that the down product's quantiser receives, [n][slots][ff] (zero beyond a shared row's shared_ff)."""
     bias = _c(bias, np.float32) if bias is not None else None
     x, logits = _c(x, np.float32), _c(logits, np.float32)
     gate, up, down = (_c(a, np.uint8) for a in (gate, up, down))
     n = x.shape[0]
     L = _Layer(hidden, ff, n_expert, k, int(shared_ff > 0), shared_ff, wtype, _ptr(gate), _ptr(up), _ptr(down), act_mode, threads,
-               int(gating), int(not norm), float(scale), _ptr(bias), int(wtype_down))
+               int(gating), int(not norm), float(scale), _ptr(bias), int(wtype_down), float(swiglu_clamp), int(bool(clamp_gate)), None)
+    act = None
+    if return_act:
+        if act_mode == 0:
+            raise ValueError("tqo_layer_forward: act rows are returned by the act modes other than 0")
+        act = np.zeros((n, k + int(shared_ff > 0), ff), np.float32)
+        L.act_out = _ptr(act)
     out = np.empty((n, hidden), np.float32)
     ids = np.empty((n, k), np.int32)
     w = np.empty((n, k), np.float32)
     if _lib.tqo_layer_forward(C.byref(L), _ptr(x), _ptr(logits), n, _ptr(out), _ptr(ids), _ptr(w)):
         raise ValueError("tqo_layer_forward: bad configuration")
-    return out, ids, w
+    return (out, ids, w, act) if return_act else (out, ids, w)
 
 
 def cpu_expert_bench(wtype, gate, up, down, hidden, ff, n_expert, threads, int8_act, reps=3):

@@ -752,20 +752,6 @@ int tqo_route(int gating, int n_expert, int k, int norm_weights, float weight_sc
     return 0;
 }
 
-double tqo_route_min_gap_ulps(int n_expert, int k, const float * logits) {
-    std::vector<float> probs;
-    gate_probs(TQO_GATE_SOFTMAX, n_expert, logits, probs);
-    std::sort(probs.begin(), probs.end(), [](float a, float b) { return a > b; });
-    double best = INFINITY;
-    for (int s = 0; s < k && s + 1 < n_expert; ++s) {
-        const float hi = probs[size_t(s)], lo = probs[size_t(s) + 1];
-        if (hi == lo) continue;
-        const float ulp = std::nextafter(hi, INFINITY) - hi;
-        best = std::min(best, double(hi - lo) / double(ulp));
-    }
-    return best;
-}
-
 int tqo_route_softmax_collision(int n_expert, int k, const float * logits) {
     std::vector<float> probs;
     gate_probs(TQO_GATE_SOFTMAX, n_expert, logits, probs);
@@ -995,17 +981,26 @@ int decode_expert(const tqo_layer & L, int e, int ff, Decoded & d) {
 }
 
 // FFN with the declared activation quantiser applied to both matvec inputs
-void ffn_mode(const tqo_layer & L, const float * x, const Decoded & d, int ff, float * out) {
-    if (L.act_mode == 0) { tqo_expert_ffn(x, L.hidden, d.gate.data(), d.up.data(), d.down.data(), ff, 0.f, 0, out); return; }
+void ffn_mode(const tqo_layer & L, const float * x, const Decoded & d, int ff, float * out, float * act_out = nullptr) {
+    if (L.act_mode == 0) { tqo_expert_ffn(x, L.hidden, d.gate.data(), d.up.data(), d.down.data(), ff, L.swiglu_clamp, L.clamp_gate, out); return; }
     std::vector<float> act(static_cast<size_t>(ff));
+    const float limit = L.swiglu_clamp;
+    const bool clamp = limit > 1e-6f;   // src/experts/moe.cpp:128-143, as tqo_expert_ffn
     for (int o = 0; o < ff; ++o) {
         float g = 0.f, u = 0.f;
         const float * wg = d.gate.data() + size_t(o) * L.hidden, * wu = d.up.data() + size_t(o) * L.hidden;
         for (int i = 0; i < L.hidden; ++i) { g += wg[i] * x[i]; u += wu[i] * x[i]; }
-        act[size_t(o)] = (g / (1.f + std::exp(-g))) * u;
+        if (clamp) {
+            u = std::min(std::max(u, -limit), limit);
+            if (L.clamp_gate) g = std::min(g, limit);
+        }
+        float s = g / (1.f + std::exp(-g));
+        if (clamp && !L.clamp_gate) s = std::min(s, limit);
+        act[size_t(o)] = s * u;
     }
     const bool f16 = L.act_mode == 5 || L.act_mode == 2 || L.act_mode == 6;   // the grouped products keep act and y as fp16 rows
     if (f16) for (float & v : act) v = tqo_half_to_float(tqo_float_to_half(v));
+    if (act_out) std::copy(act.begin(), act.end(), act_out);
     requant_row(L.act_mode, act.data(), ff);
     for (int i = 0; i < L.hidden; ++i) {
         float s = 0.f;
@@ -1053,11 +1048,14 @@ int tqo_layer_forward(const tqo_layer * Lp, const float * x, const float * logit
                 if (decode_expert(L, e, L.ff, d)) { failed = 1; continue; }
                 for (int i = offsets[size_t(e)]; i < offsets[size_t(e) + 1]; ++i) {
                     const int a = perm[size_t(i)];
-                    ffn_mode(L, xin.data() + size_t(a / K) * H, d, L.ff, routed.data() + size_t(a) * H);
+                    const size_t arow = size_t(a / K) * size_t(K + (L.has_shared ? 1 : 0)) + size_t(a % K);
+                    ffn_mode(L, xin.data() + size_t(a / K) * H, d, L.ff, routed.data() + size_t(a) * H, L.act_out ? L.act_out + arow * L.ff : nullptr);
                 }
             } else {
                 if (decode_expert(L, E, L.shared_ff, d)) { failed = 1; continue; }
-                for (int t = 0; t < n; ++t) ffn_mode(L, xin.data() + size_t(t) * H, d, L.shared_ff, shared.data() + size_t(t) * H);
+                for (int t = 0; t < n; ++t)
+                    ffn_mode(L, xin.data() + size_t(t) * H, d, L.shared_ff, shared.data() + size_t(t) * H,
+                             L.act_out ? L.act_out + (size_t(t) * size_t(K + 1) + size_t(K)) * L.ff : nullptr);
             }
         }
     };

@@ -86,10 +86,6 @@ int tqo_quantize(uint32_t type, const float * src, void * dst, int64_t n, int64_
  * the lower index) and weights[k] */
 int tqo_route(int gating, int n_expert, int k, int norm_weights, float weight_scale, const float * logits,
               const float * bias, int32_t * ids, float * weights);
-/* smallest gap, in units of the larger value's ulp, between neighbouring selection values among the k + 1 largest
- * (softmax probabilities as tqo_route computes them); a token with a gap of a few ulp is a near tie, where an
- * exp() that rounds differently may order the pair differently. Equal values (true ties) are skipped. */
-double tqo_route_min_gap_ulps(int n_expert, int k, const float * logits);
 /* 1 when, among the k + 1 largest softmax probabilities as tqo_route computes them (ties to the lower index), two
  * neighbours have the same nonzero fp32 probability although their logits differ, or one of them is a subnormal number:
  * the tokens on which a selection by logit (what a kernel with another exp() can reproduce exactly) and the reference's
@@ -155,6 +151,11 @@ typedef struct tqo_layer {
     float weight_scale;
     const float * bias;
     uint32_t wtype_down;   /* format of the down bank when it differs from gate / up (0: the same) */
+    float swiglu_clamp;    /* MoeConfig::swiglu_clamp of every expert FFN (src/experts/moe.cpp:128-143); <= 1e-6: none */
+    int clamp_gate;        /* its clamp_gate switch */
+    float * act_out;       /* optional (act modes other than 0): [n * slots][ff] the rows silu(gate) * up as the down product's quantiser
+                              receives them (after the fp16 rounding of the modes that have one), row t * slots + s, slots = k + has_shared;
+                              a shared row has shared_ff values */
 } tqo_layer;
 int tqo_layer_forward(const tqo_layer * L, const float * x, const float * logits, int n, float * out,
                       int32_t * ids_out, float * weights_out);

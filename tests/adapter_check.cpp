@@ -2,12 +2,16 @@
 // of tqllm::WeightFormat, called by base pointer. The base below restates those virtuals' signatures
 // (src/formats/weight/weight_format.hpp:22-28, 51-73) with stand-in element types, so that the `override`s of
 // tqmoe_hip::ExpertOverrides only compile if they match; then one decode product pair, one decode product with a row per
-// assignment, and the two grouped products over counts / groups / capacity run on the GPU and their results are written
-// out for tests/test_gpu_adapter.py, which compares them with the oracle.
+// assignment, the two grouped products over counts / groups / capacity, the int8 grouped product on the reference's own
+// operands (both activation modes) and moe_group with the reference's seven arguments run on the GPU, and their results are
+// written out for tests/test_gpu_adapter.py, which compares them with the oracle.
 //
 // usage: adapter_check <dir>   reads <dir>/meta.txt (type experts rows cols n topk capacity) and the arrays
-// gate.bin, up.bin (GGUF blocks), x.bin (fp16 [n][cols]), ids.bin (int32 [n][topk]), counts.bin, groups.bin; writes
-// yg.bin, yu.bin, y1.bin (bf16 [n * topk][rows]), act.bin (fp16), yd.bin (bf16)
+// gate.bin, up.bin (GGUF blocks), x.bin (fp16 [n][cols]), ids.bin (int32 [n][topk]), counts.bin, groups.bin, and for the int8
+// product xq1.bin / xq2.bin (int8 [n][cols], natural order: quantised per block / per token), xs1.bin / xs2.bin (fp32
+// [n][cols / 32]: a scale per block / the token's scale repeated), xsum.bin (int16 [n][cols / 32][2]); writes yg.bin, yu.bin, y1.bin (bf16 [n * topk][rows]), act.bin (fp16), yd.bin
+// (bf16), yi1.bin / yi2.bin (bf16: the int8 product in modes 1 and 2; absent when the format has none), ycap.bin (bf16: expert_gemm
+// with a capacity below the largest count), mg_counts.bin / mg_groups.bin (int32: moe_group)
 #include <hip/hip_runtime_api.h>
 
 #include <cstdint>
@@ -34,6 +38,8 @@ struct Mat {
 struct WeightFormat {
     virtual ~WeightFormat() = default;
     virtual bool expert_gemm(const Mat &, const __half *, __nv_bfloat16 *, int, const int *, const int *, int, int, int, bool, cudaStream_t) const { return false; }
+    virtual bool expert_gemm_i8(const Mat &, const int8_t *, const float *, const int16_t *, __nv_bfloat16 *, int, const int *, const int *, int, int, int, bool,
+                                cudaStream_t, int) const { return false; }
     virtual bool expert_gemm_gateup(const Mat &, const Mat &, const __half *, __half *, int, const int *, const int *, int, int, int, cudaStream_t) const { return false; }
     virtual bool has_expert_matvec() const { return false; }
     virtual void expert_matvec(const Mat &, const __half *, __nv_bfloat16 *, int, const int *, int, int, bool, cudaStream_t) const {}
@@ -99,7 +105,7 @@ int main(int argc, char ** argv) {
         const int * ids = static_cast<const int *>(to_device(slurp(dir + "/ids.bin")));
         const int * counts = static_cast<const int *>(to_device(slurp(dir + "/counts.bin")));
         const int * groups = static_cast<const int *>(to_device(slurp(dir + "/groups.bin")));
-        const size_t sb = tqmoe_hip::expert_scratch_bytes(cols, A, A, experts);
+        const size_t sb = tqmoe_hip::expert_scratch_bytes(cols, A, A, experts, 1);
         fmt.set_scratch(device_zeros(sb), sb);
         fmt.max_assignments = A;
 
@@ -112,6 +118,45 @@ int main(int argc, char ** argv) {
         base->expert_matvec(mats[0], x, y1, rows, ids, n, topk, false, nullptr);
         if (!base->expert_gemm_gateup(mats[0], mats[1], x, act, rows, counts, groups, capacity, experts, topk, nullptr)) return 4;
         if (!base->expert_gemm(mats[1], x, yd, rows, counts, groups, capacity, experts, topk, false, nullptr)) return 5;
+        // the int8 grouped product on the rows the reference's activation quantiser leaves, both modes; `false` = no such kernel
+        {
+            const int8_t * xq = static_cast<const int8_t *>(to_device(slurp(dir + "/xq1.bin"))), * xq2 = static_cast<const int8_t *>(to_device(slurp(dir + "/xq2.bin")));
+            const float * xs1 = static_cast<const float *>(to_device(slurp(dir + "/xs1.bin"))), * xs2 = static_cast<const float *>(to_device(slurp(dir + "/xs2.bin")));
+            const int16_t * xsum = static_cast<const int16_t *>(to_device(slurp(dir + "/xsum.bin")));
+            __nv_bfloat16 * yi = static_cast<__nv_bfloat16 *>(device_zeros(ybytes));
+            if (base->expert_gemm_i8(mats[1], xq, xs1, xsum, yi, rows, counts, groups, capacity, experts, topk, false, nullptr, 1)) {
+                hip(hipDeviceSynchronize(), "synchronize");
+                dump(dir + "/yi1.bin", yi, ybytes);
+                hip(hipMemset(yi, 0, ybytes), "hipMemset");
+                if (!base->expert_gemm_i8(mats[1], xq2, xs2, xsum, yi, rows, counts, groups, capacity, experts, topk, false, nullptr, 2)) return 7;
+                hip(hipDeviceSynchronize(), "synchronize");
+                dump(dir + "/yi2.bin", yi, ybytes);
+            }
+            if (base->expert_gemm_i8(mats[1], xq, xs2, xsum, yi, rows, counts, groups, capacity, experts, topk, false, nullptr, 3)) return 8;   // the v3 modes: not here
+        }
+        // a capacity below the largest count: the lists are cut at the capacity, and so must the products be (no row of another
+        // expert's list, no row twice)
+        {
+            __nv_bfloat16 * ycap = static_cast<__nv_bfloat16 *>(device_zeros(ybytes));
+            std::vector<char> gh = slurp(dir + "/groups.bin");
+            const int cap2 = 3;
+            std::vector<int> cut(size_t(experts) * cap2);
+            for (int e = 0; e < experts; ++e) for (int j = 0; j < cap2; ++j) cut[size_t(e) * cap2 + j] = reinterpret_cast<const int *>(gh.data())[size_t(e) * capacity + j];
+            const int * groups2 = static_cast<const int *>(to_device(std::vector<char>(reinterpret_cast<const char *>(cut.data()), reinterpret_cast<const char *>(cut.data() + cut.size()))));
+            if (!base->expert_gemm(mats[1], x, ycap, rows, counts, groups2, cap2, experts, topk, false, nullptr)) return 9;
+            hip(hipDeviceSynchronize(), "synchronize");
+            dump(dir + "/ycap.bin", ycap, ybytes);
+        }
+        // moe_group with the reference's seven arguments (moe_kernels.cuh:29): counts [experts], groups [experts][n]
+        {
+            int * mc = static_cast<int *>(device_zeros(size_t(experts) * 4));
+            std::vector<char> fill(size_t(experts) * n * 4, char(0xFF));
+            int * mg = static_cast<int *>(to_device(fill));
+            tqmoe_hip::moe_group(ids, mc, mg, experts, n, topk, nullptr);
+            hip(hipDeviceSynchronize(), "synchronize");
+            dump(dir + "/mg_counts.bin", mc, size_t(experts) * 4);
+            dump(dir + "/mg_groups.bin", mg, size_t(experts) * n * 4);
+        }
         hip(hipDeviceSynchronize(), "synchronize");
         dump(dir + "/yg.bin", yg, ybytes);
         dump(dir + "/yu.bin", yu, ybytes);
@@ -122,6 +167,10 @@ int main(int argc, char ** argv) {
         bool threw = false;
         try { base->expert_matvec(mats[0], x, y1, rows, ids, 0, topk, false, nullptr); } catch (const std::invalid_argument &) { threw = true; }
         if (!threw) return 6;
+        // lists for another number of experts than the bank holds: refused, not read past the arrays
+        threw = false;
+        try { base->expert_gemm(mats[1], x, yd, rows, counts, groups, capacity, experts - 1, topk, false, nullptr); } catch (const std::invalid_argument &) { threw = true; }
+        if (!threw) return 10;
     } catch (const std::exception & ex) {
         std::fprintf(stderr, "adapter_check: %s\n", ex.what());
         return 1;

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import synth
-from gpu_util import banks_on_device, clear_tokens, dev, oracle_mode
+from gpu_util import banks_on_device, clear_tokens, clear_tokens_gated, dev, oracle_mode
 
 pytestmark = pytest.mark.gpu
 
@@ -138,7 +138,9 @@ def check_layer(out, ids, w, want, want_ids, want_w, clear):
     # max-abs 1e-2 where the outputs are of order one, as the configurations' are; relative to the largest value beyond that
     # (banks of random valid blocks can give larger outputs, and on the 8-bit grouped products one act value that rounds the
     # other way is a step of 1 / 127 of its row's largest)
-    assert mx < MAX_ABS * max(1.0, float(np.abs(want).max())) and rel < REL_RMS, (mx, rel, float(np.abs(want).max()))
+    top = float(np.abs(want).max())
+    print("layer, %d tokens: max-abs %.3g (largest value %.3g, bar %.3g) rel-rms %.3g" % (len(out), mx, top, MAX_ABS * max(1.0, top), rel))
+    assert mx < MAX_ABS * max(1.0, top) and rel < REL_RMS, (mx, rel, top)
     return mx, rel
 
 
@@ -217,8 +219,10 @@ def test_layer_other_routing_modes(tq, oracle, gating, norm, biased, scale, n):
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
     want, want_ids, want_w = oracle.layer_forward(inp["x"][1], logits, *raws, cfg["wtype"], cfg["hidden"], cfg["ff"], e, k, shared_ff=cfg["shared_ff"],
                                                   act_mode=oracle_mode(layer, n), threads=16, gating=gating, norm=norm, scale=scale, bias=bias)
-    same = (ids == want_ids).all(axis=1)          # near-tied tokens may swap neighbours; the routing test bounds how many
-    assert same.mean() > 0.97
+    # ids bit-exact on every token whose selection values are not within fp32 rounding of each other (counted and printed)
+    clear = clear_tokens_gated(logits, e, k, gating, bias, ids, want_ids, "%d tokens" % n)
+    assert np.array_equal(ids[clear], want_ids[clear])
+    same = (ids == want_ids).all(axis=1)
     assert np.abs(w[same] - want_w[same]).max() < 4e-6 * max(1.0, float(np.abs(want_w).max()))
     mx, rel = synth.errors(out[same], want[same])
     assert mx < MAX_ABS * max(1.0, float(np.abs(want_w).sum(axis=1).max())) and rel < REL_RMS, (mx, rel)

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import synth
-from gpu_util import clear_tokens, dev, oracle_type
+from gpu_util import clear_tokens, clear_tokens_gated, dev, oracle_type
 
 pytestmark = pytest.mark.gpu
 
@@ -137,22 +137,6 @@ def test_topk_ties_extremes_and_scale(tq, oracle):
     assert ids[0].tolist() == list(range(k)) and ids[3][0] == 10
 
 
-def selection_values(logits, gating, bias):
-    """float64 selection values of moe_route (src/experts/moe.cpp:33-65): a token is a clear case when its k + 1 largest
-    are further apart than the fp32 rounding of the gating function."""
-    lg = logits.astype(np.float64)
-    if gating == 1:
-        p = np.exp(lg - lg.max(axis=1, keepdims=True))
-        p /= p.sum(axis=1, keepdims=True)
-    elif gating == 2:
-        p = 1 / (1 + np.exp(-lg))
-    elif gating == 3:
-        p = lg
-    else:
-        p = np.sqrt(np.logaddexp(0, lg))
-    return p + bias.astype(np.float64) if bias is not None else p
-
-
 @pytest.mark.parametrize("gating", [1, 2, 3, 4])
 @pytest.mark.parametrize("e,k,n", [(256, 8, 64), (512, 10, 16), (64, 6, 33), (1500, 4, 20), (160, 70, 24), (5, 5, 12)])
 def test_topk_gated_matches_oracle(tq, oracle, gating, e, k, n):
@@ -167,12 +151,10 @@ def test_topk_gated_matches_oracle(tq, oracle, gating, e, k, n):
                 ids, w, sw = (t.cpu().numpy() for t in tq.moe_topk(dev(logits), e, k, scale, gating=gating, bias=dev(bias) if biased else None,
                                                                    norm=norm))
                 want_ids, want_w = oracle.route(logits[:, :e], k, gating, norm, scale, bias)
-                v = -np.sort(-selection_values(logits[:, :e], gating, bias), axis=1)[:, :k + 1]
-                room = 2e-6 * (np.abs(v[:, :-1]) + (float(np.abs(bias).max()) if biased else 0.0))   # fp32 rounding of value and sum
-                clear = (v[:, :-1] - v[:, 1:] > room).all(axis=1)
-                assert clear.mean() > 0.9
-                assert np.array_equal(ids[clear], want_ids[clear])
+                # exempt: at most one token per case (18 of the 5070 tokens of all the cases here); no other token may differ
+                clear = clear_tokens_gated(logits, e, k, gating, bias, ids, want_ids, "%d experts top-%d, bias %s norm %s" % (e, k, biased, norm), most=1)
                 same = (ids == want_ids).all(axis=1)
+                assert np.array_equal(ids[clear], want_ids[clear])
                 assert np.abs(w[same] - want_w[same]).max() < 4e-6 * max(1.0, float(np.abs(want_w).max()))
                 want_sw = np.array([oracle.shared_weight(x) for x in logits[:, e]], np.float32)
                 assert np.abs(sw - want_sw).max() < 3e-6

@@ -134,11 +134,51 @@ def test_route_matches_reference_objects(oracle, ref):
             assert np.array_equal(w[0].view(np.uint32), rw.view(np.uint32))   # same libm, same order: bit for bit
 
 
-def test_min_gap_flags_near_ties(oracle):
-    lg = np.zeros(16, np.float32)
-    lg[:4] = [3.0, 2.0, np.nextafter(np.float32(2.0), np.float32(0)), 1.0]
-    assert oracle.route_min_gap_ulps(lg, 3)[0] < 4
-    assert oracle.route_min_gap_ulps(np.arange(16, dtype=np.float32), 3)[0] > 1e5
+def softmax_probs_f32(lg):
+    """the reference's fp32 softmax, step by step (src/experts/moe.cpp:36-47): exp(l - max), a sequential sum, a division"""
+    e = np.exp((lg - lg.max()).astype(np.float32)).astype(np.float32)
+    s = np.float32(0)
+    for v in e:
+        s = np.float32(s + v)
+    return (e / s).astype(np.float32)
+
+
+def test_softmax_collision_flags_exactly_the_unreproducible_rows(oracle):
+    """tqo_route_softmax_collision decides which tokens the GPU routing checks may exempt: rows where two *different* logits
+    have one fp32 probability at the selection boundary (a selection by logit and the reference's by rounded probability
+    can then differ), or where a boundary probability is subnormal. Everything else must not be flagged."""
+    lg = np.full(12, -9.0, np.float32)
+    near = np.float32(-1e-4)                                  # a ulp of this logit moves exp() by 7e-12, far below a ulp of the result
+    lg[:3] = [0.0, near, np.nextafter(near, np.float32(-1))]
+    p = softmax_probs_f32(lg)
+    assert lg[1] != lg[2] and p[1] == p[2] and p[1] > 0       # the pair really collides in probability
+    assert oracle.route_softmax_collision(lg, 2)[0]           # boundary between slots 1 and 2: flagged
+    assert oracle.route_softmax_collision(lg, 3)[0]           # the pair inside the selection decides the order of the ids: flagged
+    assert not oracle.route_softmax_collision(lg, 1)[0]       # boundary between 0.0 and the pair: clear
+    moved = lg.copy()
+    moved[[1, 2]] = moved[[2, 1]]                             # the same pair in the other index order: still a collision
+    assert oracle.route_softmax_collision(moved, 2)[0]
+    # the reference's own choice on that row is by probability, ties to the lower index: id 1 before id 2 both ways
+    assert oracle.route(lg, 2)[0][0].tolist() == [0, 1] and oracle.route(moved, 2)[0][0].tolist() == [0, 1]
+    # exact ties of equal logits are ordered by index on both sides: not flagged
+    tie = lg.copy()
+    tie[2] = tie[1]
+    assert not oracle.route_softmax_collision(tie, 2)[0]
+    # wide gaps: not flagged, whatever k
+    wide = np.arange(12, dtype=np.float32) * 0.75
+    assert not oracle.route_softmax_collision(wide, 1)[0] and not oracle.route_softmax_collision(wide, 8)[0]
+    # a subnormal probability at the boundary (exp(-90) ~ 8e-40): flagged; the same row cut before it: clear
+    sub = np.array([0.0, -1.0, -90.0, -200.0, -300.0], np.float32)
+    ps = softmax_probs_f32(sub)
+    assert 0 < ps[2] < np.finfo(np.float32).tiny and ps[3] == 0
+    assert oracle.route_softmax_collision(sub, 2)[0] and oracle.route_softmax_collision(sub, 3)[0]
+    assert not oracle.route_softmax_collision(sub, 1)[0]
+    # probabilities that underflowed to exact zero are ordered by index: no collision although the logits differ
+    zeros = np.array([0.0, -1.0, -200.0, -300.0, -250.0], np.float32)
+    assert not oracle.route_softmax_collision(zeros, 4)[0]
+    # random rows: collisions are rare (the tests allow one exempt token in 500)
+    rng = np.random.default_rng(3)
+    assert oracle.route_softmax_collision(rng.standard_normal((2000, 512)).astype(np.float32), 10).sum() <= 4
 
 
 def test_dispatch_brute_force(oracle):
@@ -375,6 +415,20 @@ def test_layer_forward_fp8_mode_against_float64(oracle):
     assert np.abs(got - want).max() < 2e-3 * np.abs(want).max()
     for skip in ("w", "x", "act", "act16", "y16"):
         assert (np.abs(got - rebuild(skip)) > tol).mean() > 0.3, skip
+    # the act rows the layer can hand back: row (t, s) = fp16(silu(g) * u) of the slot's expert on the quantised token row, the
+    # shared expert in the last slot with its first shared_ff values; same output as without them
+    got2, ids2, w2, act = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=sf, act_mode=2, threads=2, return_act=True)
+    assert np.array_equal(got2, got) and act.shape == (n, k + 1, f)
+    wg, wu = wide[0].reshape(e + 1, f, h), wide[1].reshape(e + 1, f, h)
+    for t in range(n):
+        xq = _requant_e4m3(oracle, x[t])
+        for s in range(k + 1):
+            j, ff = (ids[t, s], f) if s < k else (e, sf)
+            g, u = wg[j, :ff] @ xq, wu[j, :ff] @ xq
+            want_act = _half(g / (1 + np.exp(-g)) * u)
+            step = np.maximum(np.abs(want_act) * 2.0 ** -10, 2.0 ** -24)        # one fp16 step: fp32 sums against float64 here
+            assert (np.abs(act[t, s, :ff] - want_act) <= step).all() and (act[t, s, :ff] != want_act).mean() < 0.02
+            assert not act[t, s, ff:].any()
     # banks of another format have no such mode
     with pytest.raises(Exception):
         oracle.layer_forward(x, logits, *banks, oracle.IQ4_XS, h, f, e, k, act_mode=2)
@@ -432,6 +486,61 @@ def test_layer_forward_lossy_operand_modes_against_float64(oracle):
         # the fp32 oracle is none of them either
         a, _, _ = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=sf, act_mode=0, threads=1)
         assert (np.abs(a - want) > tol).mean() > 0.5
+
+
+def test_layer_forward_swiglu_clamp_against_float64(oracle):
+    """The swiglu_clamp / clamp_gate fields of tqo_layer_forward (MoeConfig::swiglu_clamp, moe_expert_ffn's switch:
+    src/experts/moe.cpp:128-143) in the fp32 mode and in the int8 mode the grouped products are gated by, rebuilt in float64:
+    up clamped to [-c, c]; clamp_gate: gate clamped to at most c before the activation; else silu(gate) clamped to at most c
+    after it. The limit is set where it really bites; without the clamp, or with the other branch, the rebuild is far off."""
+    rng = np.random.default_rng(29)
+    h, f, e, k, n, sf = 256, 256, 5, 2, 5, 256
+    wtype = oracle.IQ4_XS
+    banks = [oracle.quantize(wtype, (rng.standard_normal(((e + 1) * r, c)) * 0.08).astype(np.float32)) for r, c in ((f, h), (f, h), (h, f))]
+    dec = [oracle.dequantize(wtype, b, (e + 1) * f * h).astype(np.float64) for b in banks]
+    wg, wu, wd = dec[0].reshape(e + 1, f, h), dec[1].reshape(e + 1, f, h), dec[2].reshape(e + 1, h, f)
+    x = rng.standard_normal((n, h)).astype(np.float32)
+    logits = rng.standard_normal((n, e + 1)).astype(np.float32)
+    limit = 0.6
+    g_all = np.abs(wg[0] @ x[0].astype(np.float64))
+    assert (g_all > limit).mean() > 0.2                       # the limit cuts a fair share of the values
+
+    def rebuild(ids, w, mode, clamp, gate_first):
+        out = np.zeros((n, h))
+        for t in range(n):
+            xq = _requant_i8(x[t]) if mode == 5 else x[t].astype(np.float64)
+
+            def ffn(j, ff):
+                g, u = wg[j, :ff] @ xq, wu[j, :ff] @ xq
+                if clamp:
+                    u = np.clip(u, -limit, limit)
+                    if gate_first:
+                        g = np.minimum(g, limit)
+                sl = g / (1 + np.exp(-g))
+                if clamp and not gate_first:
+                    sl = np.minimum(sl, limit)
+                act = sl * u
+                if mode == 5:
+                    act = _requant_i8(_half(act))
+                y = wd[j, :, :ff] @ act
+                return _half(y) if mode == 5 else y
+
+            out[t] = sum(float(w[t, s]) * ffn(ids[t, s], f) for s in range(k)) + 1 / (1 + np.exp(-float(logits[t, e]))) * ffn(e, sf)
+        return out
+
+    for mode in (0, 5):
+        for gate_first in (False, True):
+            got, ids, w = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=sf, act_mode=mode, threads=2, swiglu_clamp=limit,
+                                               clamp_gate=gate_first)
+            want = rebuild(ids, w, mode, True, gate_first)
+            tol = (2e-5 if mode == 0 else 5e-4) * max(1.0, np.abs(want).max())
+            assert (np.abs(got - want) > tol).mean() < 0.01, (mode, gate_first)
+            for other in (rebuild(ids, w, mode, False, gate_first), rebuild(ids, w, mode, True, not gate_first)):
+                assert (np.abs(got - other) > tol).mean() > 0.3, (mode, gate_first)
+    # a limit at or below 1e-6 is no clamp (the reference's `limit > eps` test)
+    a, _, _ = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=sf, threads=2, swiglu_clamp=1e-6, clamp_gate=True)
+    b, _, _ = oracle.layer_forward(x, logits, *banks, wtype, h, f, e, k, shared_ff=sf, threads=2)
+    assert np.array_equal(a, b)
 
 
 def _requant_blocks_i8(v):

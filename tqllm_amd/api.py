@@ -46,7 +46,8 @@ class _Layer(C.Structure):
                 ("topk", C.c_int32), ("has_shared", C.c_int32), ("shared_ff", C.c_int32), ("weight_scale", C.c_float),
                 ("router", C.c_void_p), ("shared_gate", C.c_void_p), ("router_type", C.c_uint32),
                 ("gate", _Bank), ("up", _Bank), ("down", _Bank),
-                ("gating", C.c_int32), ("raw_weights", C.c_int32), ("probs_bias", C.c_void_p), ("act_blocks", C.c_int32)]
+                ("gating", C.c_int32), ("raw_weights", C.c_int32), ("probs_bias", C.c_void_p), ("act_blocks", C.c_int32),
+                ("swiglu_clamp", C.c_float), ("clamp_gate", C.c_int32)]
 
 
 _lib = None
@@ -70,6 +71,14 @@ def lib():
         l.tqmoe_dispatch_workspace_bytes.argtypes = [i32, i32, i32]
         l.tqmoe_dispatch.argtypes = [p, p, p, p, p, i32, i32, i32, i32, p, sz, p, e]
         l.tqmoe_dispatch_static.argtypes = [p, p, p, p, p, i32, i32, i32, i32, p, e]
+        l.tqmoe_static_scratch_init.argtypes = [e]
+        l.tqmoe_count.argtypes = [p, p, i32, p, e]
+        l.tqmoe_dedup_maps.argtypes = [p, p, i32, i32, p, p, p, i32, p, e]
+        l.tqmoe_lists_from_groups_clamped.argtypes = [p, p, i32, i32, p, p, p, p, e]
+        l.tqmoe_expert_gemm_i8_ref_scratch_bytes.restype = sz
+        l.tqmoe_expert_gemm_i8_ref_scratch_bytes.argtypes = [i32, i64, i32, i32]
+        l.tqmoe_expert_gemm_i8_ref.argtypes = [C.POINTER(_Bank), p, p, p, p, u32, p, p, i32, i32, i32, i32, i32, i64, p, sz, p, e]
+        l.tqmoe_swiglu_clamped.argtypes = [p, p, p, i64, f32, i32, p, e]
         l.tqmoe_bank_layout.argtypes = [u32, i64, i32, C.POINTER(sz), C.POINTER(sz), e]
         l.tqmoe_bank_load.argtypes = [u32, p, i64, i32, p, p, p, p, e]
         l.tqmoe_bank_dequant.argtypes = [C.POINTER(_Bank), i64, i64, p, p, e]
@@ -215,8 +224,71 @@ def moe_dispatch(ids, experts, capacity=0):
     return counts, offsets, perm, groups
 
 
+def moe_group(ids, experts):
+    """tqllm_cuda::moe_group (moe_kernels.cuh:29): (counts [E], groups [E][n]) of ids [n][topk], ascending inside each expert;
+    entries of groups past an expert's count are -1 here (the library leaves them untouched)."""
+    n, topk = ids.shape
+    counts = torch.empty(experts, dtype=torch.int32, device=ids.device)
+    groups = torch.full((experts, n), -1, dtype=torch.int32, device=ids.device)
+    moe_dispatch_into(ids, experts, counts, None, None, groups, n)
+    return counts, groups
+
+
+def moe_count(ids, counts):
+    """counts[ids[i]] += 1 into the caller's uint64-sized counters (int64 tensor), tqllm_cuda::moe_count (moe.cu:183-186)."""
+    err = _err()
+    _check(lib().tqmoe_count(_ptr(ids), _ptr(counts), ids.numel(), _stream(ids), C.byref(err)), err)
+    return counts
+
+
+DEDUP_COLS, DEDUP_STRIDE = 8, 18     # kDedupCols, kDedupStride (src/formats/weight/quant_kernels.cuh:26-27)
+
+
+def moe_dedup_maps(ids, slot_of, topk, groups=None):
+    """tqllm_cuda::moe_dedup_maps (moe_kernels.cuh:34-39): (slots [count], gu [groups][18], dn [groups][18]) of the flat ids."""
+    count = ids.numel()
+    groups = count if groups is None else groups
+    dev = ids.device
+    slots = torch.empty(count, dtype=torch.int32, device=dev)
+    gu = torch.empty((groups, DEDUP_STRIDE), dtype=torch.int32, device=dev)
+    dn = torch.empty((groups, DEDUP_STRIDE), dtype=torch.int32, device=dev)
+    err = _err()
+    _check(lib().tqmoe_dedup_maps(_ptr(ids), _ptr(slot_of), count, topk, _ptr(slots), _ptr(gu), _ptr(dn), groups, _stream(ids), C.byref(err)), err)
+    return slots, gu, dn
+
+
+def lists_from_groups(counts, groups, bound=None):
+    """The reference's counts / groups [E][capacity] as (counts clamped to the capacity, offsets, perm) for the grouped products."""
+    experts, capacity = groups.shape
+    dev = groups.device
+    cc = torch.empty(experts, dtype=torch.int32, device=dev)
+    offsets = torch.empty(experts + 1, dtype=torch.int32, device=dev)
+    perm = torch.full((bound or experts * capacity,), -1, dtype=torch.int32, device=dev)
+    err = _err()
+    _check(lib().tqmoe_lists_from_groups_clamped(_ptr(counts), _ptr(groups), capacity, experts, _ptr(cc), _ptr(offsets), _ptr(perm), _stream(groups),
+                                                 C.byref(err)), err)
+    return cc, offsets, perm
+
+
+def expert_gemm_i8_ref(bank, xq, xs, counts, groups, topk, assignments, per_expert_input=False, mode=2, out_dtype=torch.bfloat16, y=None):
+    """WeightFormat::expert_gemm_i8 with the reference's own operands (weight_format.hpp:54-56): xq int8 [rows][cols] in natural
+    order, xs fp32 [rows][cols / 32] (mode 1: per block; mode 2: the token's scale, [row][0] read), counts [E],
+    groups [E][capacity]; y [assignments][bank rows], bf16 as the reference (or fp16)."""
+    experts, capacity = groups.shape
+    if y is None:
+        y = torch.zeros((assignments, bank.rows), dtype=out_dtype, device=xq.device)
+    need = lib().tqmoe_expert_gemm_i8_ref_scratch_bytes(experts, assignments, bank.cols, mode)
+    scratch = torch.zeros(max(need, 16), dtype=torch.uint8, device=xq.device)
+    err = _err()
+    b = bank.view()
+    _check(lib().tqmoe_expert_gemm_i8_ref(C.byref(b), _ptr(xq), _ptr(xs), None, _ptr(y), _ttype(y), _ptr(counts), _ptr(groups), capacity, experts, topk,
+                                          int(per_expert_input), mode, assignments, _ptr(scratch), scratch.numel(), _stream(xq), C.byref(err)), err)
+    return y
+
+
 def moe_dispatch_into(ids, experts, counts, offsets, perm, groups=None, capacity=0):
-    """tqmoe_dispatch_static into tensors the caller already holds: the library's built-in scratch, nothing allocated."""
+    """tqmoe_dispatch_static into tensors the caller already holds: the library's built-in scratch, nothing allocated.
+    offsets and perm may be None when groups is given (counts + groups: moe_group)."""
     n, topk = ids.shape
     err = _err()
     _check(lib().tqmoe_dispatch_static(_ptr(ids), _ptr(counts), _ptr(offsets), _ptr(perm), _ptr(groups), capacity, experts, n, topk,
@@ -524,10 +596,12 @@ def expert_gemm_i8_blocks(bank, xq, xs, block_scale, lists, n, slots, topk, shar
     return y
 
 
-def moe_swiglu(gate, up):
+def moe_swiglu(gate, up, swiglu_clamp=0.0, clamp_gate=False):
+    """silu(gate) * up in fp32 (moe_kernels.cuh:71-72) with the optional clamp of moe_expert_ffn (src/experts/moe.cpp:128-143)."""
     act = torch.empty_like(gate)
     err = _err()
-    _check(lib().tqmoe_swiglu(_ptr(gate), _ptr(up), _ptr(act), gate.numel(), _stream(gate), C.byref(err)), err)
+    _check(lib().tqmoe_swiglu_clamped(_ptr(gate), _ptr(up), _ptr(act), gate.numel(), float(swiglu_clamp), int(bool(clamp_gate)), _stream(gate),
+                                      C.byref(err)), err)
     return act
 
 
@@ -568,7 +642,8 @@ class MoeLayer:
     """hidden states + router weights + expert banks in, combined hidden states out, in one library call."""
 
     def __init__(self, router, shared_gate, gate, up, down, topk, shared_ff=0, weight_scale=1.0, gating=GATE_SOFTMAX, probs_bias=None,
-                 norm_weights=True, act_blocks=False):
+                 norm_weights=True, act_blocks=False, swiglu_clamp=0.0, clamp_gate=False):
+        self.swiglu_clamp, self.clamp_gate = swiglu_clamp, clamp_gate   # MoeConfig::swiglu_clamp, moe_expert_ffn's clamp_gate
         self.router, self.shared_gate, self.gate, self.up, self.down = router, shared_gate, gate, up, down
         self.act_blocks = act_blocks   # int8 grouped products: a scale per 32 activations in place of one per token
         self.n_expert, self.hidden = router.shape
@@ -580,7 +655,8 @@ class MoeLayer:
         return _Layer(C.sizeof(_Layer), self.hidden, self.ff, self.n_expert, self.topk, int(self.shared_ff > 0), self.shared_ff,
                       float(self.weight_scale), self.router.data_ptr(), self.shared_gate.data_ptr() if self.shared_gate is not None else None,
                       _ttype(self.router), self.gate.view(), self.up.view(), self.down.view(), int(self.gating), int(not self.norm_weights),
-                      self.probs_bias.data_ptr() if self.probs_bias is not None else None, int(self.act_blocks))
+                      self.probs_bias.data_ptr() if self.probs_bias is not None else None, int(self.act_blocks), float(self.swiglu_clamp),
+                      int(bool(self.clamp_gate)))
 
     def path(self, n):
         """'decode', 'grouped_i8', 'grouped_f16' or 'grouped_fp8': the expert products a batch of n tokens takes"""

@@ -87,6 +87,18 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // ----------------------------------------------------------------------------------------------- device side
 constexpr int kWave = 64;
 
+// The optional clamp of the SwiGLU inputs (MoeConfig::swiglu_clamp, src/experts/moe.hpp:34-36; moe_expert_ffn,
+// src/experts/moe.cpp:128-143): limit <= 1e-6 is no clamp; else up goes to [-limit, limit] and either the gate to
+// (-inf, limit] before the activation (gate_first, the GLM branch) or silu(gate) to (-inf, limit] after it.
+struct Glu { float limit; int gate_first; };
+__device__ __forceinline__ void glu_clamp_inputs(const Glu c, float & g, float & u) {
+    if (c.limit > 1e-6f) {
+        u = fminf(fmaxf(u, -c.limit), c.limit);
+        if (c.gate_first) g = fminf(g, c.limit);
+    }
+}
+__device__ __forceinline__ float glu_clamp_silu(const Glu c, float s) { return c.limit > 1e-6f && !c.gate_first ? fminf(s, c.limit) : s; }
+
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t h) { return __uint_as_float(uint32_t(h) << 16); }
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {  // round to nearest even
     const uint32_t x = __float_as_uint(f);

@@ -7,7 +7,7 @@ int32_t check_bank(const tqmoe_bank * b, const char * what, tqmoe_error * err); 
 // prefill_planes.hip (f8: E4M3 operand bytes in place of int8)
 int32_t enqueue_quant_rows_i8(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, hipStream_t s, bool f8);
 int32_t enqueue_gemm_f16(const tqmoe_bank & b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int * counts, const int * offsets, const int * perm,
-                         int experts, int64_t assignments, int xdiv, void * out, uint32_t out_type, int gateup, int shared_expert, int shared_lim, hipStream_t s);
+                         int experts, int64_t assignments, int xdiv, void * out, uint32_t out_type, int gateup, int shared_expert, int shared_lim, hipStream_t s, Glu glu);
 int64_t grouped_row_tiles(int64_t assignments, int experts);
 int64_t grouped_scale_words(int64_t assignments, int experts);
 int32_t enqueue_quant_rows_i8_blocks(const void * x, uint32_t xtype, int64_t rows, int cols, int8_t * q, float * scale, int16_t * qsum, hipStream_t s);
@@ -15,17 +15,33 @@ int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, co
                                int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, float * block_scale);
 int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
                               int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8, float * block_scale);
+int32_t enqueue_gather_rows_natural(const int8_t * rq, const float * rs, int cols, const int * counts, const int * offsets, const int * perm, int experts,
+                                    int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, float * block_scale);
 bool plane_gemm_has(uint32_t type);
 bool plane_gemm_is_fp8(uint32_t type);
 int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
                            const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s,
-                           const float * xbs);
+                           const float * xbs, Glu glu, int out_bf16);
+
+int32_t expert_gateup_glu(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x_image, void * act_image, const int32_t * ids, int32_t n,
+                          int32_t slots, int32_t topk, int32_t shared_ff, Glu glu, void * stream, tqmoe_error * err);
+int32_t gemm_8bit_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
+                         const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
+                         tqmoe_error * err, const char * what, bool fp8, const float * block_scale = nullptr, bool blocks = false, Glu glu = Glu{0.f, 0},
+                         int out_bf16 = 0);
+int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int32_t * counts, const int32_t * offsets,
+                        const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, int32_t xdiv, void * out, uint32_t otype, int gateup,
+                        void * stream, tqmoe_error * err, const char * what, Glu glu = Glu{0.f, 0});
 
 namespace {
 
-__global__ __launch_bounds__(256) void swiglu_k(const float * __restrict__ g, const float * __restrict__ u, float * __restrict__ act, int64_t count) {
+__global__ __launch_bounds__(256) void swiglu_k(const float * __restrict__ g, const float * __restrict__ u, float * __restrict__ act, int64_t count, Glu glu) {
     const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
-    if (i < count) { const float a = g[i]; act[i] = a / (1.f + expf(-a)) * u[i]; }
+    if (i < count) {
+        float a = g[i], b = u[i];
+        glu_clamp_inputs(glu, a, b);
+        act[i] = glu_clamp_silu(glu, a / (1.f + expf(-a))) * b;
+    }
 }
 
 // out[t][j] = sum_s weights[t][s] * routed[t][s][j] (s < topk ascending, rows `slots` per token) + shared_w[t] * shared[t][j]
@@ -85,8 +101,10 @@ __global__ __launch_bounds__(256) void extend_ids_k(const int * __restrict__ ids
 // The reference's dispatch lists (counts [E], groups [E][capacity]) as the lists this library's grouped products read:
 // offsets = exclusive scan of the counts, perm = the experts' lists one behind the other. One block; the order inside an
 // expert is kept as it is (the reference's device lists are in no particular order, its host lists ascending).
+// counts_out (may be null): the counts the lists really hold, min(counts, capacity): what the products must be given, or
+// an expert whose count exceeds the capacity would run past its span of perm.
 __global__ __launch_bounds__(1024) void lists_from_groups_k(const int * __restrict__ counts, const int * __restrict__ groups, int capacity, int E,
-                                                            int * __restrict__ offsets, int * __restrict__ perm) {
+                                                            int * __restrict__ offsets, int * __restrict__ perm, int * __restrict__ counts_out) {
     __shared__ int part[1024];
     extern __shared__ int start[];   // E + 1
     const int tid = threadIdx.x, per = (E + 1023) / 1024, lo = min(tid * per, E), hi = min(lo + per, E);
@@ -105,6 +123,7 @@ __global__ __launch_bounds__(1024) void lists_from_groups_k(const int * __restri
     if (tid == 1023) start[E] = part[1023];
     __syncthreads();
     for (int e = tid; e <= E; e += 1024) offsets[e] = start[e];
+    if (counts_out) for (int e = tid; e < E; e += 1024) counts_out[e] = start[e + 1] - start[e];
     const int lane = tid & 63, wave = tid >> 6;
     for (int e = wave; e < E; e += 16) {   // a wave per expert: coalesced reads of its list
         const int c = start[e + 1] - start[e];
@@ -239,13 +258,18 @@ extern "C" int32_t tqmoe_expert_matvec2_rows(const tqmoe_bank * gate, const tqmo
     return matvec_rows_common(gate, up, x, xtype, y_gate, y_up, ytype, ids, n, topk, 0, scratch, scratch_bytes, stream, err, "tqmoe_expert_matvec2_rows");
 }
 
-extern "C" int32_t tqmoe_lists_from_groups(const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts, int32_t * offsets, int32_t * perm,
-                                           void * stream, tqmoe_error * err) {
+extern "C" int32_t tqmoe_lists_from_groups_clamped(const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts, int32_t * counts_out,
+                                                   int32_t * offsets, int32_t * perm, void * stream, tqmoe_error * err) {
     if (!counts || !groups || !offsets || !perm || capacity <= 0 || experts <= 0 || experts > 4096)
         return fail(err, TQMOE_E_ARG, "tqmoe_lists_from_groups: invalid shape or pointer");
     if (int32_t rc = need_device(err, "tqmoe_lists_from_groups")) return rc;
-    lists_from_groups_k<<<1, 1024, size_t(experts + 1) * sizeof(int), static_cast<hipStream_t>(stream)>>>(counts, groups, capacity, experts, offsets, perm);
+    lists_from_groups_k<<<1, 1024, size_t(experts + 1) * sizeof(int), static_cast<hipStream_t>(stream)>>>(counts, groups, capacity, experts, offsets, perm, counts_out);
     return launched(err, "tqmoe_lists_from_groups");
+}
+
+extern "C" int32_t tqmoe_lists_from_groups(const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts, int32_t * offsets, int32_t * perm,
+                                           void * stream, tqmoe_error * err) {
+    return tqmoe_lists_from_groups_clamped(counts, groups, capacity, experts, nullptr, offsets, perm, stream, err);
 }
 
 extern "C" int32_t tqmoe_extend_ids(const int32_t * ids, int32_t * out, int32_t topk, int32_t n, int32_t extra, void * stream, tqmoe_error * err) {
@@ -256,8 +280,10 @@ extern "C" int32_t tqmoe_extend_ids(const int32_t * ids, int32_t * out, int32_t 
     return launched(err, "tqmoe_extend_ids");
 }
 
-extern "C" int32_t tqmoe_expert_gateup(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x_image, void * act_image, const int32_t * ids,
-                                       int32_t n, int32_t slots, int32_t topk, int32_t shared_ff, void * stream, tqmoe_error * err) {
+// The gate / up products of the three paths with the optional clamp of the SwiGLU inputs (the layer's swiglu_clamp); the
+// C entry points are these without a clamp.
+int32_t tqmoe::expert_gateup_glu(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x_image, void * act_image, const int32_t * ids, int32_t n,
+                                 int32_t slots, int32_t topk, int32_t shared_ff, Glu glu, void * stream, tqmoe_error * err) {
     const char * what = "tqmoe_expert_gateup";
     if (int32_t rc = check_bank(gate, what, err)) return rc;
     if (int32_t rc = check_bank(up, what, err)) return rc;
@@ -270,9 +296,14 @@ extern "C" int32_t tqmoe_expert_gateup(const tqmoe_bank * gate, const tqmoe_bank
     const Split sp = split_for(gate->cols / 32, A);
     if (sp.m == 0) return fail(err, TQMOE_E_UNSUPPORTED, "%s: cols %d is too wide for the decode kernels", what, gate->cols);
     if (int32_t rc = need_device(err, what)) return rc;
-    GateupArgs k{view(*gate), view(*up), static_cast<const uint8_t *>(x_image), static_cast<uint8_t *>(act_image), ids, int(A), slots, topk, shared_ff, dedup_mode(A, slots)};
+    GateupArgs k{view(*gate), view(*up), static_cast<const uint8_t *>(x_image), static_cast<uint8_t *>(act_image), ids, int(A), slots, topk, shared_ff, dedup_mode(A, slots), glu};
     dispatch_gateup(gate->type, sp, k, static_cast<hipStream_t>(stream));
     return launched(err, what);
+}
+
+extern "C" int32_t tqmoe_expert_gateup(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x_image, void * act_image, const int32_t * ids,
+                                       int32_t n, int32_t slots, int32_t topk, int32_t shared_ff, void * stream, tqmoe_error * err) {
+    return expert_gateup_glu(gate, up, x_image, act_image, ids, n, slots, topk, shared_ff, Glu{0.f, 0}, stream, err);
 }
 
 extern "C" int32_t tqmoe_expert_down(const tqmoe_bank * down, const void * act_image, float * y, const int32_t * ids, int32_t n, int32_t slots,
@@ -284,11 +315,16 @@ extern "C" int32_t tqmoe_expert_down(const tqmoe_bank * down, const void * act_i
     return matvec_common(down, nullptr, act_image, y, nullptr, TQMOE_F32, ids, int64_t(n) * slots, 1, slots, topk, shared_ff, stream, err, what);
 }
 
-extern "C" int32_t tqmoe_swiglu(const float * gate, const float * up, float * act, int64_t count, void * stream, tqmoe_error * err) {
+extern "C" int32_t tqmoe_swiglu_clamped(const float * gate, const float * up, float * act, int64_t count, float swiglu_clamp, int32_t clamp_gate, void * stream,
+                                        tqmoe_error * err) {
     if (!gate || !up || !act || count <= 0 || (count + 255) / 256 > 0x7FFFFFFF) return fail(err, TQMOE_E_ARG, "tqmoe_swiglu: invalid size or pointer");
     if (int32_t rc = need_device(err, "tqmoe_swiglu")) return rc;
-    swiglu_k<<<unsigned((count + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(gate, up, act, count);
+    swiglu_k<<<unsigned((count + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(gate, up, act, count, Glu{swiglu_clamp, clamp_gate ? 1 : 0});
     return launched(err, "tqmoe_swiglu");
+}
+
+extern "C" int32_t tqmoe_swiglu(const float * gate, const float * up, float * act, int64_t count, void * stream, tqmoe_error * err) {
+    return tqmoe_swiglu_clamped(gate, up, act, count, 0.f, 0, stream, err);
 }
 
 template <class RT>
@@ -438,9 +474,9 @@ extern "C" int32_t tqmoe_gather_rows_i8_blocks(const int8_t * rows_q, const floa
                               "tqmoe_gather_rows_i8_blocks");
 }
 
-static int32_t gemm_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
+int32_t tqmoe::gemm_8bit_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                            const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
-                           tqmoe_error * err, const char * what, bool fp8, const float * block_scale = nullptr, bool blocks = false) {
+                           tqmoe_error * err, const char * what, bool fp8, const float * block_scale, bool blocks, Glu glu, int out_bf16) {
     if (blocks && !block_scale) return fail(err, TQMOE_E_ARG, "%s: block scales missing", what);
     if (int32_t rc = check_bank(b0, what, err)) return rc;
     if (b1) {
@@ -459,7 +495,7 @@ static int32_t gemm_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const i
     if (int32_t rc = need_device(err, what)) return rc;
     const int shared_expert = slots > topk ? b0->experts - 1 : -1;
     if (enqueue_plane_gemm(*b0, b1, xq, xs, counts, offsets, perm, b0->experts, int64_t(n) * slots, out, gateup, shared_expert, shared_lim,
-                           static_cast<hipStream_t>(stream), block_scale))
+                           static_cast<hipStream_t>(stream), block_scale, glu, out_bf16))
         return fail(err, TQMOE_E_ARG, "%s: too many assignments for one call", what);
     return launched(err, what);
 }
@@ -468,27 +504,80 @@ extern "C" int32_t tqmoe_expert_gemm_gateup_i8(const tqmoe_bank * gate, const tq
                                                const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim,
                                                void * act_f16, void * stream, tqmoe_error * err) {
     if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_gemm_gateup_i8: second bank missing");
-    return gemm_common(gate, up, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err, "tqmoe_expert_gemm_gateup_i8", false);
+    return gemm_8bit_common(gate, up, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err, "tqmoe_expert_gemm_gateup_i8", false);
 }
 
 extern "C" int32_t tqmoe_expert_gemm_i8(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                                         const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * y_f16, void * stream,
                                         tqmoe_error * err) {
-    return gemm_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8", false);
+    return gemm_8bit_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8", false);
+}
+
+// scratch of tqmoe_expert_gemm_i8_ref: clamped counts | offsets | perm | grouped rows | their scales and index | block scales
+namespace {
+struct RefScratch { size_t counts, offsets, perm, q, scale, block_scale, total; };
+RefScratch ref_scratch(int experts, int64_t bound, int cols, int mode) {
+    RefScratch r{};
+    size_t o = 0;
+    auto take = [&](size_t bytes) { const size_t at = o; o = align_up(o + bytes, 256); return at; };
+    r.counts = take(size_t(experts) * 4);
+    r.offsets = take(size_t(experts + 1) * 4);
+    r.perm = take(size_t(bound) * 4);
+    r.q = take(size_t(tqmoe_grouped_rows(bound, experts)) * size_t(cols));
+    r.scale = take(size_t(tqmoe_grouped_scale_words(bound, experts)) * 4);
+    r.block_scale = take(mode == 1 ? size_t(tqmoe_grouped_block_scale_words(bound, experts, cols)) * 4 : 0);
+    r.total = o;
+    return r;
+}
+}  // namespace
+
+extern "C" size_t tqmoe_expert_gemm_i8_ref_scratch_bytes(int32_t experts, int64_t max_assignments, int32_t cols, int32_t mode) {
+    if (experts <= 0 || experts > 4096 || max_assignments <= 0 || cols <= 0 || cols % 32 || (mode != 1 && mode != 2)) return 0;
+    return ref_scratch(experts, max_assignments, cols, mode).total;
+}
+
+extern "C" int32_t tqmoe_expert_gemm_i8_ref(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const int16_t * xsum, void * y, uint32_t ytype,
+                                            const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts, int32_t topk,
+                                            int32_t per_expert_input, int32_t mode, int64_t max_assignments, void * scratch, size_t scratch_bytes,
+                                            void * stream, tqmoe_error * err) {
+    const char * what = "tqmoe_expert_gemm_i8_ref";
+    (void)xsum;   // the sums of q per 16 values feed the reference's minimum term; the products here take that term from a plane of their own
+    if (int32_t rc = check_bank(bank, what, err)) return rc;
+    if (mode != 1 && mode != 2) return fail(err, TQMOE_E_UNSUPPORTED, "%s: mode %d (1: a scale per 32 values, 2: per token)", what, mode);
+    if (ytype != TQMOE_BF16 && ytype != TQMOE_F16) return fail(err, TQMOE_E_UNSUPPORTED, "%s: output rows are BF16 or F16", what);
+    if (!xq || !xs || !y || !counts || !groups || capacity <= 0 || experts <= 0 || topk <= 0 || max_assignments <= 0)
+        return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    if (experts != bank->experts) return fail(err, TQMOE_E_ARG, "%s: %d lists for a bank of %d experts", what, experts, bank->experts);
+    if (max_assignments > int64_t(experts) * capacity) max_assignments = int64_t(experts) * capacity;
+    const RefScratch r = ref_scratch(experts, max_assignments, bank->cols, mode);
+    if (!scratch || scratch_bytes < r.total) return fail(err, TQMOE_E_WORKSPACE, "%s: scratch of %zu bytes needed", what, r.total);
+    if (!plane_gemm_has(bank->type) || plane_gemm_is_fp8(bank->type))
+        return fail(err, TQMOE_E_UNSUPPORTED, "%s: no int8 grouped product for bank type %u (false in the reference's terms)", what, bank->type);
+    uint8_t * ws = static_cast<uint8_t *>(scratch);
+    int32_t * cc = reinterpret_cast<int32_t *>(ws + r.counts), * offsets = reinterpret_cast<int32_t *>(ws + r.offsets), * perm = reinterpret_cast<int32_t *>(ws + r.perm);
+    int8_t * q = reinterpret_cast<int8_t *>(ws + r.q);
+    float * scale = reinterpret_cast<float *>(ws + r.scale), * bscale = mode == 1 ? reinterpret_cast<float *>(ws + r.block_scale) : nullptr;
+    if (int32_t rc = tqmoe_lists_from_groups_clamped(counts, groups, capacity, experts, cc, offsets, perm, stream, err)) return rc;
+    enqueue_gather_rows_natural(xq, xs, bank->cols, cc, offsets, perm, experts, max_assignments, per_expert_input ? 1 : topk, q, scale,
+                                static_cast<hipStream_t>(stream), bscale);
+    if (int32_t rc = launched(err, what)) return rc;
+    // (n x slots only bounds the listed assignments: it fixes where the index behind the scales lies)
+    return gemm_8bit_common(bank, nullptr, q, scale, cc, offsets, perm, 1, int32_t(max_assignments), int32_t(max_assignments), 0, y, 0, stream, err, what, false,
+                            bscale, mode == 1, Glu{0.f, 0}, ytype == TQMOE_BF16);
 }
 
 extern "C" int32_t tqmoe_expert_gemm_gateup_i8_blocks(const tqmoe_bank * gate, const tqmoe_bank * up, const int8_t * xq, const float * xs, const float * block_scale,
                                                       const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk,
                                                       int32_t shared_lim, void * act_f16, void * stream, tqmoe_error * err) {
     if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_gemm_gateup_i8_blocks: second bank missing");
-    return gemm_common(gate, up, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err, "tqmoe_expert_gemm_gateup_i8_blocks", false,
+    return gemm_8bit_common(gate, up, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err, "tqmoe_expert_gemm_gateup_i8_blocks", false,
                        block_scale, true);
 }
 
 extern "C" int32_t tqmoe_expert_gemm_i8_blocks(const tqmoe_bank * bank, const int8_t * xq, const float * xs, const float * block_scale, const int32_t * counts,
                                                const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim,
                                                void * y_f16, void * stream, tqmoe_error * err) {
-    return gemm_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8_blocks", false, block_scale,
+    return gemm_8bit_common(bank, nullptr, xq, xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err, "tqmoe_expert_gemm_i8_blocks", false, block_scale,
                        true);
 }
 
@@ -496,20 +585,20 @@ extern "C" int32_t tqmoe_expert_gemm_gateup_fp8(const tqmoe_bank * gate, const t
                                                 const int32_t * offsets, const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim,
                                                 void * act_f16, void * stream, tqmoe_error * err) {
     if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_gemm_gateup_fp8: second bank missing");
-    return gemm_common(gate, up, reinterpret_cast<const int8_t *>(xq), xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err,
+    return gemm_8bit_common(gate, up, reinterpret_cast<const int8_t *>(xq), xs, counts, offsets, perm, n, slots, topk, shared_lim, act_f16, 1, stream, err,
                        "tqmoe_expert_gemm_gateup_fp8", true);
 }
 
 extern "C" int32_t tqmoe_expert_gemm_fp8(const tqmoe_bank * bank, const uint8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                                          const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * y_f16, void * stream,
                                          tqmoe_error * err) {
-    return gemm_common(bank, nullptr, reinterpret_cast<const int8_t *>(xq), xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err,
+    return gemm_8bit_common(bank, nullptr, reinterpret_cast<const int8_t *>(xq), xs, counts, offsets, perm, n, slots, topk, shared_lim, y_f16, 0, stream, err,
                        "tqmoe_expert_gemm_fp8", true);
 }
 
-static int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int32_t * counts, const int32_t * offsets,
+int32_t tqmoe::gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int32_t * counts, const int32_t * offsets,
                                const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, int32_t xdiv, void * out, uint32_t otype, int gateup,
-                               void * stream, tqmoe_error * err, const char * what) {
+                               void * stream, tqmoe_error * err, const char * what, Glu glu) {
     if (int32_t rc = check_bank(b0, what, err)) return rc;
     if (b1) {
         if (int32_t rc = check_bank(b1, what, err)) return rc;
@@ -524,7 +613,7 @@ static int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, con
     if (int32_t rc = need_device(err, what)) return rc;
     const int shared_expert = slots > topk ? b0->experts - 1 : -1;
     if (enqueue_gemm_f16(*b0, b1, x, xtype, counts, offsets, perm, b0->experts, int64_t(n) * slots, xdiv, out, otype, gateup, shared_expert,
-                         shared_lim, static_cast<hipStream_t>(stream)))
+                         shared_lim, static_cast<hipStream_t>(stream), glu))
         return fail(err, TQMOE_E_ARG, "%s: too many assignments for one call", what);
     return launched(err, what);
 }

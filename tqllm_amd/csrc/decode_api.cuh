@@ -37,6 +37,7 @@ struct GateupArgs {
     uint8_t * aimage;
     const int * ids;
     int A, slots, topk, shared_ff, mode;
+    Glu glu;                  // the optional clamp of the SwiGLU inputs
 };
 
 // arguments of the grouped fp16 products (prefill_f16_kernels.cuh)
@@ -54,6 +55,7 @@ struct F16Args {
     int gateup;
     int shared_expert;        // the expert whose rows (gate / up) or columns (down) stop at shared_lim, or -1
     int shared_lim;
+    Glu glu;                  // gateup: the optional clamp of the SwiGLU inputs
 };
 // the grouped fp16 product of one bank format; wide: 128 input rows per block (grid.y counts such units), else 64
 template <uint32_t FMT> struct F16Launch {

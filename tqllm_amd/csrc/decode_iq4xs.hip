@@ -60,7 +60,7 @@ __device__ __forceinline__ v4i decode16(uint2 c, NibbleConsts nc) {
 template <int NB, bool UNI, int MODE>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void iq4xs_mfma_k(BankView b0, BankView b1, const uint8_t * __restrict__ image, void * out0, void * out1, uint32_t ytype,
                                                     const int * __restrict__ ids, int A, int xdiv, int mode, int slots, int topk, int shared_lim, int wk,
-                                                    int tpw, int gateup, int a_off, int tl_count) {
+                                                    int tpw, int gateup, int a_off, int tl_count, Glu glu) {
     constexpr bool STAGED = MODE >= 1, MULTI = MODE == 2;
     extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
     __shared__ int meta[2], s_tok[kTP];
@@ -181,7 +181,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
                 for (int w = 0; w < wk; ++w) { v0 += red[rt * wk + w][0][j][i]; if (NB == 2) v1 += red[rt * wk + w][NB - 1][j][i]; }
             const int aj = live ? s_tok[j] : 0;
             if (gateup) {
-                const float act = v0 / (1.f + expf(-v0)) * v1;
+                glu_clamp_inputs(glu, v0, v1);
+                const float act = glu_clamp_silu(glu, v0 / (1.f + expf(-v0))) * v1;
                 quantise_block_lanes(act, i, live, ql[threadIdx.x >> 5], static_cast<uint8_t *>(out0) + int64_t(aj) * tiles * kImageSubBytes, tiles, t);
             } else if (live) {
                 const int64_t o = int64_t(aj) * rows + t * 32 + i;
@@ -298,7 +299,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3))) void i
 }
 
 void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0, void * out1, uint32_t ytype, const int * ids, int A, int xdiv, int mode,
-            int slots, int topk, int shared_lim, int gateup, bool uniform, hipStream_t s) {
+            int slots, int topk, int shared_lim, int gateup, bool uniform, Glu glu, hipStream_t s) {
     const int NSB = b0.cols / 256, tiles = b0.rows / 32;
     // Waves that share a row's super-blocks: as many as it takes to put a few thousand waves in flight (a short batch
     // is bound by the latency of one wave's chain), fewer when the batch has the waves anyway (a longer chain per
@@ -327,7 +328,7 @@ void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0
     const dim3 grid(unsigned((tiles + tpw * tl - 1) / (tpw * tl)), unsigned(A));
     const int a_off = int(lds);
     if (staged) lds += size_t(b0.cols / 32) * (256 + (uniform ? 0 : kTP * sizeof(float)));
-    auto go = [&](auto kernel) { kernel<<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup, a_off, tl); };
+    auto go = [&](auto kernel) { kernel<<<grid, threads, lds, s>>>(b0, b1, image, out0, out1, ytype, ids, A, xdiv, mode, slots, topk, shared_lim, wk, tpw, gateup, a_off, tl, glu); };
     if (nb == 2 && uniform) staged ? go(iq4xs_mfma_k<2, true, 1>) : go(iq4xs_mfma_k<2, true, 0>);
     else if (nb == 2) staged ? go(iq4xs_mfma_k<2, false, 1>) : go(iq4xs_mfma_k<2, false, 0>);
     else if (tl > 1) go(iq4xs_mfma_k<1, false, 2>);
@@ -337,10 +338,10 @@ void launch(int nb, BankView b0, BankView b1, const uint8_t * image, void * out0
 }  // namespace
 
 template <> void DecodeLaunch<TQMOE_IQ4_XS>::matvec(Split, int nb, const MatvecArgs & k, hipStream_t s) {
-    launch(nb, k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols, 0, false, s);
+    launch(nb, k.b0, k.b1, k.image, k.y0, k.y1, k.ytype, k.ids, k.A, k.xdiv, k.mode, k.slots, k.topk, k.shared_cols, 0, false, Glu{0.f, 0}, s);
 }
 template <> void DecodeLaunch<TQMOE_IQ4_XS>::gateup(Split, const GateupArgs & k, hipStream_t s) {
-    launch(2, k.bg, k.bu, k.ximage, k.aimage, nullptr, TQMOE_F32, k.ids, k.A, k.slots, k.mode, k.slots, k.topk, k.shared_ff, 1, true, s);
+    launch(2, k.bg, k.bu, k.ximage, k.aimage, nullptr, TQMOE_F32, k.ids, k.A, k.slots, k.mode, k.slots, k.topk, k.shared_ff, 1, true, k.glu, s);
 }
 
 }  // namespace tqmoe

@@ -588,7 +588,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((FMT ==
 // [n][slots] expert of every (token, slot); slots past topk hold the shared expert, which only has shared_ff rows.
 template <uint32_t FMT, int LPR, int M, int NW>
 __global__ __launch_bounds__(NW * 64) void gateup_k(BankView bg, BankView bu, const uint8_t * __restrict__ ximage, uint8_t * __restrict__ aimage,
-                                                    const int * __restrict__ ids, int A, int slots, int topk, int shared_ff, int mode) {
+                                                    const int * __restrict__ ids, int A, int slots, int topk, int shared_ff, int mode, Glu glu) {
     constexpr int RW = 64 / LPR, NJ = 32 / (NW * RW);
     static_assert(NJ >= 1 && NJ * NW * RW == 32, "a block makes exactly 32 rows");
     __shared__ __attribute__((aligned(8))) uint32_t grid_lds[lattice_dwords(FMT)];
@@ -619,8 +619,9 @@ __global__ __launch_bounds__(NW * 64) void gateup_k(BankView bg, BankView bu, co
     const int tid = threadIdx.x, which = tid >> 5, i = tid & 31;
     if (tid < 64) {                                                 // the whole wave: the lane exchanges need every lane
         const bool live = which < cnt;
-        const float g = live ? gl[which][i] : 0.f, u = live ? ul[which][i] : 0.f;
-        quantise_block_lanes(g / (1.f + expf(-g)) * u, i, live, ql[which], aimage + int64_t(which ? a1 : a) * SA * kImageSubBytes, SA, blockIdx.x);
+        float g = live ? gl[which][i] : 0.f, u = live ? ul[which][i] : 0.f;
+        glu_clamp_inputs(glu, g, u);
+        quantise_block_lanes(glu_clamp_silu(glu, g / (1.f + expf(-g))) * u, i, live, ql[which], aimage + int64_t(which ? a1 : a) * SA * kImageSubBytes, SA, blockIdx.x);
     }
 }
 
@@ -638,7 +639,7 @@ template <uint32_t FMT, int LPR, int M> void launch_one_gateup(const GateupArgs 
     const dim3 grid(unsigned(k.bg.rows / 32), unsigned(k.A));
     // as many waves as divide the block's 32 rows: 8 for 8 lanes or more per row
     constexpr int NW = 32 / (64 / LPR) >= kGateupNW ? kGateupNW : 32 / (64 / LPR);
-    gateup_k<FMT, LPR, M, NW><<<grid, NW * 64, 0, s>>>(k.bg, k.bu, k.ximage, k.aimage, k.ids, k.A, k.slots, k.topk, k.shared_ff, k.mode);
+    gateup_k<FMT, LPR, M, NW><<<grid, NW * 64, 0, s>>>(k.bg, k.bu, k.ximage, k.aimage, k.ids, k.A, k.slots, k.topk, k.shared_ff, k.mode, k.glu);
 }
 
 // the (lanes per row, sub-blocks per lane) pairs split_for() can return

@@ -10,6 +10,15 @@ int32_t enqueue_topk(const float * logits, int32_t * ids, float * weights, float
                      const float * bias, int32_t norm, hipStream_t s, int32_t shared_ungated);
 bool plane_gemm_has(uint32_t type);
 bool plane_gemm_is_fp8(uint32_t type);
+// decode.hip: the gate / up products with the clamp of the SwiGLU inputs
+int32_t expert_gateup_glu(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x_image, void * act_image, const int32_t * ids, int32_t n,
+                          int32_t slots, int32_t topk, int32_t shared_ff, Glu glu, void * stream, tqmoe_error * err);
+int32_t gemm_8bit_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
+                         const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
+                         tqmoe_error * err, const char * what, bool fp8, const float * block_scale, bool blocks, Glu glu, int out_bf16);
+int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int32_t * counts, const int32_t * offsets,
+                        const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, int32_t xdiv, void * out, uint32_t otype, int gateup,
+                        void * stream, tqmoe_error * err, const char * what, Glu glu);
 
 namespace {
 
@@ -36,10 +45,13 @@ bool int8_ok(const tqmoe_layer & L) {
            L.hidden % 256 == 0 && L.ff % 256 == 0 && (!L.has_shared || L.shared_ff % 256 == 0);
 }
 
-// The descriptor grew twice: one that ends before the routing fields means softmax, normalised, no bias; one that ends
-// before act_blocks means a scale per token.
+// The descriptor grew three times: one that ends before the routing fields means softmax, normalised, no bias; one that
+// ends before act_blocks means a scale per token; one that ends before swiglu_clamp means no clamp.
 constexpr size_t kLayerBaseSize = offsetof(tqmoe_layer, gating), kLayerRoutingSize = offsetof(tqmoe_layer, act_blocks);
-bool act_blocks_of(const tqmoe_layer & L) { return L.struct_size >= sizeof(tqmoe_layer) && L.act_blocks != 0; }
+constexpr size_t kLayerBlocksSize = offsetof(tqmoe_layer, swiglu_clamp);
+bool act_blocks_of(const tqmoe_layer & L) { return L.struct_size >= kLayerBlocksSize && L.act_blocks != 0; }
+// a descriptor that ends before swiglu_clamp does not clamp
+Glu glu_of(const tqmoe_layer & L) { return L.struct_size >= sizeof(tqmoe_layer) ? Glu{L.swiglu_clamp, L.clamp_gate ? 1 : 0} : Glu{0.f, 0}; }
 
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
@@ -161,6 +173,7 @@ static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t
     // one launch: top-k, the ids extended by the shared expert, and (decode path) the input rows' activation image
     int32_t * ext = L.has_shared ? reinterpret_cast<int32_t *>(ws + p.ids_ext) : nullptr;
     const Routing rt = routing_of(L);
+    const Glu glu = glu_of(L);
     enqueue_topk(logits, ids, weights, shared_w, ext, L.n_expert, x, xtype, L.hidden, p.grouped ? nullptr : ws + p.ximage, L.n_expert, L.topk, n,
                  L.weight_scale, rt.gating, rt.bias, rt.norm, static_cast<hipStream_t>(stream), L.has_shared && !L.shared_gate);
     if (int32_t rc = launched(err, "tqmoe_layer_forward (top-k)")) return rc;
@@ -190,8 +203,8 @@ static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t
             if (int32_t rc = tqmoe_dispatch(cid, counts, offsets, perm, nullptr, 0, banks, c, slots, ws + p.dispatch_ws,
                                             tqmoe_dispatch_workspace_bytes(banks, c, slots), stream, err)) return rc;
             if (!p.int8) {
-                if (int32_t rc = tqmoe_expert_gemm_gateup(&L.gate, &L.up, xb + size_t(t0) * L.hidden * xbytes, xtype, counts, offsets, perm, c, slots, L.topk, L.shared_ff,
-                                                          act16, stream, err)) return rc;
+                if (int32_t rc = gemm_f16_common(&L.gate, &L.up, xb + size_t(t0) * L.hidden * xbytes, xtype, counts, offsets, perm, c, slots, L.topk, L.shared_ff, slots,
+                                                 act16, TQMOE_F16, 1, stream, err, "tqmoe_layer_forward (gate / up)", glu)) return rc;
                 float * y32 = reinterpret_cast<float *>(y16);
                 if (int32_t rc = tqmoe_expert_gemm(&L.down, act16, TQMOE_F16, counts, offsets, perm, c, slots, L.topk, L.shared_ff, 1, y32, TQMOE_F32, stream, err)) return rc;
                 if (int32_t rc = combine(y32, TQMOE_F32, L.has_shared ? y32 + size_t(L.topk) * L.hidden : nullptr)) return rc;
@@ -200,23 +213,26 @@ static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t
             int8_t * rq = reinterpret_cast<int8_t *>(ws + p.rq);
             float * rs = reinterpret_cast<float *>(ws + p.rs);
             if (plane_gemm_is_fp8(L.gate.type)) {
-                uint8_t * xq8 = reinterpret_cast<uint8_t *>(xq), * aq8 = reinterpret_cast<uint8_t *>(aq);
+                uint8_t * aq8 = reinterpret_cast<uint8_t *>(aq);
                 if (int32_t rc = tqmoe_quant_rows_fp8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, reinterpret_cast<uint8_t *>(rq), rs, stream, err)) return rc;
                 if (int32_t rc = tqmoe_gather_rows_i8(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, stream, err)) return rc;
-                if (int32_t rc = tqmoe_expert_gemm_gateup_fp8(&L.gate, &L.up, xq8, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
+                if (int32_t rc = gemm_8bit_common(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, 1, stream, err,
+                                                  "tqmoe_layer_forward (gate / up)", true, nullptr, false, glu, 0)) return rc;
                 if (int32_t rc = tqmoe_group_rows_fp8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq8, as, stream, err)) return rc;
                 if (int32_t rc = tqmoe_expert_gemm_fp8(&L.down, aq8, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
             } else if (p.blocks) {
             float * xbs = reinterpret_cast<float *>(ws + p.xbs), * abks = reinterpret_cast<float *>(ws + p.abks);
             if (int32_t rc = tqmoe_quant_rows_i8_blocks(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, rq, rs, nullptr, stream, err)) return rc;
             if (int32_t rc = tqmoe_gather_rows_i8_blocks(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, xbs, stream, err)) return rc;
-            if (int32_t rc = tqmoe_expert_gemm_gateup_i8_blocks(&L.gate, &L.up, xq, xs, xbs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
+            if (int32_t rc = gemm_8bit_common(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, 1, stream, err,
+                                              "tqmoe_layer_forward (gate / up)", false, xbs, true, glu, 0)) return rc;
             if (int32_t rc = tqmoe_group_rows_i8_blocks(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, abks, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_i8_blocks(&L.down, aq, as, abks, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
             } else {
             if (int32_t rc = tqmoe_quant_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, rq, rs, stream, err)) return rc;
             if (int32_t rc = tqmoe_gather_rows_i8(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, stream, err)) return rc;
-            if (int32_t rc = tqmoe_expert_gemm_gateup_i8(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, stream, err)) return rc;
+            if (int32_t rc = gemm_8bit_common(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, 1, stream, err,
+                                              "tqmoe_layer_forward (gate / up)", false, nullptr, false, glu, 0)) return rc;
             if (int32_t rc = tqmoe_group_rows_i8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_gemm_i8(&L.down, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
             }
@@ -225,7 +241,7 @@ static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t
         } else {
             const uint8_t * ximage = ws + p.ximage + tqmoe_act_image_bytes(1, L.hidden) * size_t(t0);
             float * y = reinterpret_cast<float *>(ws + p.y);
-            if (int32_t rc = tqmoe_expert_gateup(&L.gate, &L.up, ximage, ws + p.aimage, cid, c, slots, L.topk, L.shared_ff, stream, err)) return rc;
+            if (int32_t rc = expert_gateup_glu(&L.gate, &L.up, ximage, ws + p.aimage, cid, c, slots, L.topk, L.shared_ff, glu, stream, err)) return rc;
             if (int32_t rc = tqmoe_expert_down(&L.down, ws + p.aimage, y, cid, c, slots, L.topk, L.shared_ff, stream, err)) return rc;
             if (int32_t rc = combine(y, TQMOE_F32, L.has_shared ? y + size_t(L.topk) * L.hidden : nullptr)) return rc;
         }

@@ -25,8 +25,8 @@ void dispatch_f16(uint32_t type, const F16Args & k, bool two, bool wide, dim3 gr
 
 // assignments = total entries of perm; the grid covers the most row blocks the lists can need
 int32_t enqueue_gemm_f16(const tqmoe_bank & b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int * counts, const int * offsets, const int * perm,
-                         int experts, int64_t assignments, int xdiv, void * out, uint32_t out_type, int gateup, int shared_expert, int shared_lim, hipStream_t s) {
-    const F16Args k{view(b0), b1 ? view(*b1) : view(b0), x, xtype, counts, offsets, perm, experts, xdiv, out, out_type, gateup, shared_expert, shared_lim};
+                         int experts, int64_t assignments, int xdiv, void * out, uint32_t out_type, int gateup, int shared_expert, int shared_lim, hipStream_t s, Glu glu) {
+    const F16Args k{view(b0), b1 ? view(*b1) : view(b0), x, xtype, counts, offsets, perm, experts, xdiv, out, out_type, gateup, shared_expert, shared_lim, glu};
     const bool wide = assignments >= int64_t(experts) * kWideFrom;   // half a wide tile filled on average
     const int tile = wide ? 128 : 64;                                // input rows of a block
     const int64_t units = assignments / tile + experts;              // sum of ceil(count / tile) never exceeds this

@@ -265,7 +265,11 @@ __global__ __launch_bounds__(256, 2) void expert_gemm_f16_k(F16Args k) {
             const int a = s_asg[mi * 32 + 8 * (i >> 2) + 4 * g + (i & 3)];
             if (a < 0) continue;
             float v = acc[0][mi][i];
-            if (k.gateup) v = v * __builtin_amdgcn_rcpf(1.f + __expf(-v)) * acc[NB - 1][mi][i];
+            if (k.gateup) {
+                float u = acc[NB - 1][mi][i];
+                glu_clamp_inputs(k.glu, v, u);
+                v = glu_clamp_silu(k.glu, v * __builtin_amdgcn_rcpf(1.f + __expf(-v))) * u;
+            }
             v = col < row_lim ? v : 0.f;
             if (k.out_type == TQMOE_F32) static_cast<float *>(k.out)[int64_t(a) * rows + col] = v;
             else if (k.out_type == TQMOE_BF16) static_cast<uint16_t *>(k.out)[int64_t(a) * rows + col] = float_to_bf16_bits(v);

@@ -265,6 +265,32 @@ __global__ __launch_bounds__(256) void gather_rows_i8_k(const int8_t * __restric
         for (int ks = wave; ks < S; ks += 4) block_scale[(int64_t(tile_index) * S + ks) * 32 + r] = rs[row * S + ks];
 }
 
+// The grouped operand from int8 rows in natural order with scales laid out [rows][cols / 32] (what the reference's activation
+// quantiser leaves: quant_act_rows_k, src/formats/weight/quant_u4h.inc:790-822): lane (g, r) reads the two 8-byte halves of
+// its 16 operand bytes (values 8 g .. 8 g + 7 and 16 + 8 g .. 16 + 8 g + 7 of the block) and interleaves their dwords.
+// per_block: every block's own scale goes to block_scale and the rows' scales are 1; else the row's scale is its first entry.
+__global__ __launch_bounds__(256) void gather_rows_natural_k(const int8_t * __restrict__ rq, const float * __restrict__ rs, int cols, const int * __restrict__ counts,
+                                                             const int * __restrict__ offsets, const int * __restrict__ perm, int experts, int xdiv,
+                                                             int8_t * __restrict__ q, float * __restrict__ scale, Plan plan, float * __restrict__ block_scale) {
+    const int tile_index = int(blockIdx.x);
+    if (tile_index >= plan.tile_base[experts]) return;
+    const int e = owner_of(plan.tile_base, experts, tile_index);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, g = lane >> 5;
+    const int i = (tile_index - plan.tile_base[e]) * 32 + r;
+    if (i >= counts[e]) return;                       // rows past the expert's count are left as they are
+    const int64_t row = perm[offsets[e] + i] / xdiv;
+    const int S = cols / 32;
+    if (wave == 0 && g == 0) scale[int64_t(tile_index) * 32 + r] = block_scale ? 1.f : rs[row * S];
+    const uint2 * src = reinterpret_cast<const uint2 *>(rq + row * cols) + g;
+    uint4 * dst = reinterpret_cast<uint4 *>(q + int64_t(tile_index) * 32 * cols) + lane;
+    for (int ks = wave; ks < S; ks += 4) {
+        const uint2 lo = src[ks * 4], hi = src[ks * 4 + 2];
+        dst[ks * 64] = make_uint4(lo.x, hi.x, lo.y, hi.y);
+    }
+    if (block_scale && g == 0)
+        for (int ks = wave; ks < S; ks += 4) block_scale[(int64_t(tile_index) * S + ks) * 32 + r] = rs[row * S + ks];
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------- entry helpers
@@ -341,6 +367,15 @@ int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, co
     return 0;
 }
 
+int32_t enqueue_gather_rows_natural(const int8_t * rq, const float * rs, int cols, const int * counts, const int * offsets, const int * perm, int experts,
+                                    int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, float * block_scale) {
+    const int64_t tiles = grouped_row_tiles(assignments, experts);
+    const Plan plan = plan_at(scale, tiles * 32, experts);
+    plan_k<<<1, 64, 0, s>>>(counts, experts, plan);
+    gather_rows_natural_k<<<unsigned(tiles), 256, 0, s>>>(rq, rs, cols, counts, offsets, perm, experts, xdiv, q, scale, plan, block_scale);
+    return 0;
+}
+
 // bank formats with a plane GEMM: int8 operands (IQ4_XS, IQ4_NL, IQ3_S, IQ3_XXS, IQ2_XXS, IQ2_XS, IQ2_S, IQ1_S, Q4_K) or E4M3 operands (NVFP4G)
 bool plane_gemm_has(uint32_t type) {
     return type == TQMOE_IQ4_XS || type == TQMOE_IQ3_S || type == TQMOE_Q4_K || type == TQMOE_NVFP4G || type == TQMOE_IQ3_XXS || type == TQMOE_IQ2_XXS ||
@@ -353,7 +388,7 @@ bool plane_gemm_is_fp8(uint32_t type) { return type == TQMOE_NVFP4G; }
 int32_t plane_gemm_blocks(uint32_t type, int nb, bool gateup, const GemmArgs & k, unsigned blocks, hipStream_t s);
 int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
                            const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s,
-                           const float * xbs) {
+                           const float * xbs, Glu glu, int out_bf16) {
     const int nb = gateup || b0.rows % 64 == 0 ? 2 : 1;
     const int units = gateup ? b0.rows / 32 : b0.rows / (32 * nb);
     const int64_t tiles = grouped_row_tiles(assignments, experts);
@@ -361,7 +396,7 @@ int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const i
     int unit_group = std::max(1, std::min(4, 16 / std::max(1, b0.cols / 256)));
     while (units % unit_group) --unit_group;
     GemmArgs k{view(b0), b1 ? view(*b1) : view(b0), xq, xs, counts, offsets, perm, plan_at(xs, tiles * 32, experts), experts, static_cast<uint16_t *>(out_f16),
-               units, unit_group, shared_expert, shared_lim, xbs};
+               units, unit_group, shared_expert, shared_lim, xbs, glu, out_bf16};
     // one block per compute unit (the kernel's registers and LDS allow no second one), walking the work items
     const int cus = cu_count();
     const int64_t most = (tiles / kChunkTiles + experts + 7) / 8 * 8 * (units / unit_group);     // an upper bound of the items

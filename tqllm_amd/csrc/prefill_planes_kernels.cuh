@@ -68,6 +68,8 @@ struct GemmArgs {
     int shared_expert;        // index of the expert whose rows (gate / up) or columns (down) stop at shared_lim, or -1
     int shared_lim;
     const float * xbs;        // a scale per row and 32-value sub-block, [row tile][sub-block][32 rows] (the rows' own scales are then 1), or null
+    Glu glu;                  // gate / up: the optional clamp of the SwiGLU inputs
+    int out_bf16;             // the results as bf16 rows in place of fp16
 };
 
 namespace {
@@ -145,12 +147,16 @@ __device__ __forceinline__ uint16_t to_half_bits(float v) {
     asm volatile("" : "+v"(v));
     return __half_as_ushort(__float2half_rn(v));
 }
-__device__ __forceinline__ uint16_t swiglu_half(float g_acc, float u_acc, float sc) {
-    const float gv = __fmul_rn(g_acc, sc), uv = __fmul_rn(u_acc, sc);
+__device__ __forceinline__ uint16_t swiglu_half(float g_acc, float u_acc, float sc, const Glu glu) {
+    float gv = __fmul_rn(g_acc, sc), uv = __fmul_rn(u_acc, sc);
+    glu_clamp_inputs(glu, gv, uv);
     const float den = __fadd_rn(1.f, __expf(-gv));
-    return to_half_bits(__fmul_rn(__fdiv_rn(gv, den), uv));
+    return to_half_bits(__fmul_rn(glu_clamp_silu(glu, __fdiv_rn(gv, den)), uv));
 }
-__device__ __forceinline__ uint16_t scaled_half(float acc, float sc) { return to_half_bits(__fmul_rn(acc, sc)); }
+__device__ __forceinline__ uint16_t scaled_half(float acc, float sc, int bf16) {
+    const float v = __fmul_rn(acc, sc);
+    return bf16 ? float_to_bf16_bits(v) : to_half_bits(v);
+}
 
 __device__ const int8_t kIq4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
@@ -880,10 +886,10 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                     uint16_t * o = k.out + int64_t(asg[i]) * rows;
                     if (GATEUP) {
                         const float up = kExchange ? ex[(mg * 16 + i) * 64 + lane] : acc[SPW - 1].sum[i];
-                        o[wt[0] * 32 + n] = swiglu_half(acc[0].sum[i], up, scl[i]);
+                        o[wt[0] * 32 + n] = swiglu_half(acc[0].sum[i], up, scl[i], k.glu);
                     } else {
 #pragma unroll
-                        for (int q = 0; q < SPW; ++q) o[wt[q] * 32 + n] = scaled_half(acc[q].sum[i], scl[i]);
+                        for (int q = 0; q < SPW; ++q) o[wt[q] * 32 + n] = scaled_half(acc[q].sum[i], scl[i], k.out_bf16);
                     }
                 }
             }
@@ -946,10 +952,10 @@ __global__ __launch_bounds__(64 * WAVES) void plane_gemm_k(GemmArgs k) {
                         if (asg[i] < 0) continue;
                         uint16_t * o = k.out + int64_t(asg[i]) * rows;
                         if (GATEUP) {
-                            o[u * 32 + n] = zero ? uint16_t(0) : swiglu_half(acc[t][0].sum[i], acc[t][NB - 1].sum[i], scl[i]);
+                            o[u * 32 + n] = zero ? uint16_t(0) : swiglu_half(acc[t][0].sum[i], acc[t][NB - 1].sum[i], scl[i], k.glu);
                         } else {
 #pragma unroll
-                            for (int b = 0; b < NB; ++b) o[(NB * u + b) * 32 + n] = zero ? uint16_t(0) : scaled_half(acc[t][b].sum[i], scl[i]);
+                            for (int b = 0; b < NB; ++b) o[(NB * u + b) * 32 + n] = zero ? uint16_t(0) : scaled_half(acc[t][b].sum[i], scl[i], k.out_bf16);
                         }
                     }
                 }

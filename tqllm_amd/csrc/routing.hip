@@ -1,4 +1,5 @@
 // Router logits, softmax + top-k, and the stable token-to-expert dispatch.
+#include <atomic>
 #include <mutex>
 
 #include "act_image.cuh"
@@ -694,7 +695,7 @@ __device__ void place_chunk(const int * __restrict__ ids, const int * __restrict
         for (int w = 0; w < waves; ++w) {  // waves take their turn in index order
             if (wave == w && e >= 0) {
                 const int slot = (prefix ? prefix[e] : 0) + run[e] + rank;
-                perm[offsets[e] + slot] = a;
+                if (perm) perm[offsets[e] + slot] = a;
                 if (groups && slot < capacity) groups[int64_t(e) * capacity + slot] = a;
             }
             __syncthreads();
@@ -767,12 +768,12 @@ __global__ __launch_bounds__(1024) void dispatch_place_wide_k(const int * __rest
     if (e >= 0) {
         int slot = before_e + rank;
         for (int w = 0; w < wave; ++w) slot += hist[w * E + e];
-        perm[start[e] + slot] = a;
+        if (perm) perm[start[e] + slot] = a;
         if (groups && slot < capacity) groups[int64_t(e) * capacity + slot] = a;
     }
     if (chunk == 0) {
-        for (int j = tid; j < E; j += 1024) { counts[j] = total[j]; offsets[j] = start[j]; }
-        if (tid == 0) offsets[E] = start[E];
+        for (int j = tid; j < E; j += 1024) { counts[j] = total[j]; if (offsets) offsets[j] = start[j]; }
+        if (tid == 0 && offsets) offsets[E] = start[E];
     }
 }
 
@@ -786,8 +787,8 @@ __global__ __launch_bounds__(256) void dispatch_small_k(const int * __restrict__
     for (int a = threadIdx.x; a < A; a += 256) { const int e = ids[a]; if (e >= 0 && e < E) atomicAdd(&hist[e], 1); }
     __syncthreads();
     block_exclusive_scan(hist, offs, E, scratch);
-    for (int j = threadIdx.x; j < E; j += 256) { counts[j] = hist[j]; offsets[j] = offs[j]; }
-    if (threadIdx.x == 0) offsets[E] = offs[E];
+    for (int j = threadIdx.x; j < E; j += 256) { counts[j] = hist[j]; if (offsets) offsets[j] = offs[j]; }
+    if (threadIdx.x == 0 && offsets) offsets[E] = offs[E];
     __syncthreads();
     zero_lds(hist, E);
     __syncthreads();
@@ -900,17 +901,20 @@ extern "C" size_t tqmoe_dispatch_workspace_bytes(int32_t experts, int32_t n, int
     return chunks <= 1 ? 16 : size_t(chunks) * size_t(experts) * sizeof(int);
 }
 
-// Scratch of tqmoe_dispatch_static: the per-chunk counts, in the library's own device image (every GPU the library runs
-// on holds its copy until the process ends). In host code the array's name is not a device address: the address on the
-// current device comes from hipGetSymbolAddress, once per device, and only that pointer is handed to the kernels.
+// Scratch of tqmoe_dispatch_static: the per-chunk counts (and, for a caller that passes no offsets array, the offsets the
+// placement of more than 1024 experts reads), in the library's own device image (every GPU the library runs on holds its
+// copy until the process ends). In host code the array's name is not a device address: the address on the current device
+// comes from hipGetSymbolAddress, once per device, and only that pointer is handed to the kernels.
 constexpr int kStaticInts = 1 << 20;                 // 4 MiB: chunks x experts may not exceed it
-static __device__ __align__(256) int scratch[kStaticInts];
+constexpr int kStaticOffsets = 4352;                 // behind them: room for the offsets of up to 4096 experts
+static __device__ __align__(256) int scratch[kStaticInts + kStaticOffsets];
 
 namespace tqmoe {
 namespace {
-// the launches of tqmoe_dispatch; cc: chunks x experts ints of scratch for more than one chunk
+// the launches of tqmoe_dispatch; cc: chunks x experts ints of scratch for more than one chunk. offsets and perm may be
+// null where the caller only wants counts and groups (spare_offsets: experts + 1 ints the scan may use instead).
 int32_t enqueue_dispatch(const int32_t * ids, int32_t * counts, int32_t * offsets, int32_t * perm, int32_t * groups, int32_t capacity, int32_t experts,
-                         int A, int chunks, int * cc, hipStream_t s, tqmoe_error * err, const char * what) {
+                         int A, int chunks, int * cc, int * spare_offsets, hipStream_t s, tqmoe_error * err, const char * what) {
     if (chunks == 1) {
         dispatch_small_k<<<1, 256, size_t(2 * experts + 1 + 256) * sizeof(int), s>>>(ids, counts, offsets, perm, groups, capacity, A, experts);
         return launched(err, what);
@@ -922,27 +926,85 @@ int32_t enqueue_dispatch(const int32_t * ids, int32_t * counts, int32_t * offset
         dispatch_place_wide_k<<<unsigned(chunks), 1024, lds, s>>>(ids, cc, counts, offsets, perm, groups, capacity, A, experts, chunks);
         return launched(err, what);
     }
-    dispatch_scan_k<<<1, 1024, size_t(experts + 1024) * sizeof(int), s>>>(cc, counts, offsets, chunks, experts);
-    dispatch_place_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, offsets, cc, perm, groups, capacity, A, experts);
+    int32_t * offs = offsets ? offsets : spare_offsets;
+    dispatch_scan_k<<<1, 1024, size_t(experts + 1024) * sizeof(int), s>>>(cc, counts, offs, chunks, experts);
+    dispatch_place_k<<<unsigned(chunks), 256, size_t(experts) * sizeof(int), s>>>(ids, offs, cc, perm, groups, capacity, A, experts);
     return launched(err, what);
 }
 
+// Address of ::scratch on each device: looked up once (under the mutex), read without a lock afterwards.
 constexpr int kMaxDevices = 64;
-int * g_scratch_ptr[kMaxDevices];                    // address of ::scratch on each device, looked up on first use
+std::atomic<int *> g_scratch_ptr[kMaxDevices];
 std::mutex g_scratch_mutex;
 
 int32_t static_scratch(int ** out, tqmoe_error * err) {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(err, TQMOE_E_DEVICE, "tqmoe_dispatch_static: no usable current device");
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (!g_scratch_ptr[dev]) {
-        void * p = nullptr;
-        const hipError_t rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-        if (rc != hipSuccess || !p) return fail(err, TQMOE_E_DEVICE, "tqmoe_dispatch_static: hipGetSymbolAddress: %s", hipGetErrorString(rc));
-        g_scratch_ptr[dev] = static_cast<int *>(p);
+    int * p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            void * sym = nullptr;
+            const hipError_t rc = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+            if (rc != hipSuccess || !sym) return fail(err, TQMOE_E_DEVICE, "tqmoe_dispatch_static: hipGetSymbolAddress: %s", hipGetErrorString(rc));
+            p = static_cast<int *>(sym);
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
     }
-    *out = g_scratch_ptr[dev];
+    *out = p;
     return 0;
+}
+
+// counts[ids[i]] += 1 as 64-bit counters (a routing profile that runs on over many calls)
+__global__ __launch_bounds__(256) void count_k(const int * __restrict__ ids, unsigned long long * __restrict__ counts, int count) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < count) { const int e = ids[i]; if (e >= 0) atomicAdd(counts + e, 1ull); }
+}
+
+// The decode grouping maps of one routed call, one block. Assignment a has slot s = slot_of[ids[a]] (-1 for a skipped id).
+// The assignments of a slot, in ascending a, are cut into runs of kDedupCols; the run is a group, groups are numbered by
+// their first assignment. Every thread walks the slots of the assignments before it (LDS broadcast reads), which gives its
+// rank in its slot and the assignment that opened its run; a block-wide prefix over the opening flags numbers the groups.
+constexpr int kDedupCols = 8, kDedupStride = 2 + 2 * kDedupCols;
+__global__ __launch_bounds__(1024) void dedup_maps_k(const int * __restrict__ ids, const int * __restrict__ slot_of, int count, int topk,
+                                                     int * __restrict__ slots, int * __restrict__ gu, int * __restrict__ dn, int groups) {
+    __shared__ int s_slot[1024], s_group[1024], s_wave[16];
+    const int a = threadIdx.x, lane = a & 63, wave = a >> 6;
+    for (int i = a; i < groups * kDedupStride; i += 1024) { if (gu) gu[i] = -1; if (dn) dn[i] = -1; }
+    int s = -1;
+    if (a < count) { const int e = ids[a]; s = e >= 0 ? slot_of[e] : -1; if (slots) slots[a] = s; }
+    s_slot[a] = a < count ? s : -1;
+    __syncthreads();
+    int rank = 0, total = 0, opener = a;
+    if (s >= 0) {
+        for (int b = 0; b < count; ++b) {
+            if (s_slot[b] != s) continue;
+            if (b < a) { if ((rank & (kDedupCols - 1)) == 0) opener = b; ++rank; }
+            ++total;
+        }
+        if ((rank & (kDedupCols - 1)) == 0) opener = a;
+    }
+    const bool opens = s >= 0 && (rank & (kDedupCols - 1)) == 0;
+    const unsigned long long m = __ballot(opens);
+    if (lane == 0) s_wave[wave] = __popcll(m);
+    __syncthreads();
+    int g = __popcll(m & ((1ull << lane) - 1ull));
+    for (int w = 0; w < wave; ++w) g += s_wave[w];
+    s_group[a] = g;                 // meaningful where the thread opens a group
+    __syncthreads();
+    if (s < 0) return;
+    const int col = rank & (kDedupCols - 1), first = rank - col;
+    int * maps[2] = {gu, dn};
+#pragma unroll
+    for (int part = 0; part < 2; ++part) {
+        int * e = maps[part];
+        if (!e) continue;
+        e += int64_t(s_group[opener]) * kDedupStride;
+        if (col == 0) { e[0] = s; e[1] = min(kDedupCols, total - first); }
+        e[2 + col] = part ? a : a / topk;
+        e[2 + kDedupCols + col] = a;
+    }
 }
 }  // namespace
 }  // namespace tqmoe
@@ -959,19 +1021,41 @@ extern "C" int32_t tqmoe_dispatch(const int32_t * ids, int32_t * counts, int32_t
     const hipStream_t s = static_cast<hipStream_t>(stream);
     if (chunks > 1 && (!workspace || workspace_bytes < tqmoe_dispatch_workspace_bytes(experts, n, topk)))
         return fail(err, TQMOE_E_WORKSPACE, "tqmoe_dispatch: workspace of %zu bytes needed", tqmoe_dispatch_workspace_bytes(experts, n, topk));
-    return enqueue_dispatch(ids, counts, offsets, perm, groups, capacity, experts, A, chunks, static_cast<int *>(workspace), s, err, "tqmoe_dispatch");
+    return enqueue_dispatch(ids, counts, offsets, perm, groups, capacity, experts, A, chunks, static_cast<int *>(workspace), nullptr, s, err, "tqmoe_dispatch");
 }
 
 extern "C" int32_t tqmoe_dispatch_static(const int32_t * ids, int32_t * counts, int32_t * offsets, int32_t * perm, int32_t * groups,
                                          int32_t capacity, int32_t experts, int32_t n, int32_t topk, void * stream, tqmoe_error * err) {
-    if (!ids || !counts || !offsets || !perm || experts <= 0 || experts > 4096 || n <= 0 || topk <= 0 || (groups && capacity <= 0))
+    if (!ids || !counts || experts <= 0 || experts > 4096 || n <= 0 || topk <= 0 || (groups && capacity <= 0) || (!groups && !perm))
         return fail(err, TQMOE_E_ARG, "tqmoe_dispatch_static: invalid shape or pointer");
     const int64_t A64 = int64_t(n) * topk, chunks64 = (A64 + kChunk - 1) / kChunk;
+    if (A64 > (1 << 30)) return fail(err, TQMOE_E_ARG, "tqmoe_dispatch_static: too many assignments");
     if (chunks64 > 1 && chunks64 * experts > kStaticInts)
         return fail(err, TQMOE_E_WORKSPACE, "tqmoe_dispatch_static: %lld assignments x %d experts need %lld scratch ints, the built-in scratch holds %d "
                     "(use tqmoe_dispatch with a workspace)", (long long)A64, experts, (long long)(chunks64 * experts), kStaticInts);
     int * cc = nullptr;
     if (int32_t rc = static_scratch(&cc, err)) return rc;
-    return enqueue_dispatch(ids, counts, offsets, perm, groups, capacity, experts, int(A64), int(chunks64), cc, static_cast<hipStream_t>(stream), err,
-                            "tqmoe_dispatch_static");
+    return enqueue_dispatch(ids, counts, offsets, perm, groups, capacity, experts, int(A64), int(chunks64), cc, cc + kStaticInts,
+                            static_cast<hipStream_t>(stream), err, "tqmoe_dispatch_static");
+}
+
+extern "C" int32_t tqmoe_static_scratch_init(tqmoe_error * err) {
+    int * p = nullptr;
+    if (int32_t rc = need_device(err, "tqmoe_static_scratch_init")) return rc;
+    return static_scratch(&p, err) ? TQMOE_E_DEVICE : ok(err);
+}
+
+extern "C" int32_t tqmoe_count(const int32_t * ids, uint64_t * counts, int32_t count, void * stream, tqmoe_error * err) {
+    if (!ids || !counts || count <= 0) return fail(err, TQMOE_E_ARG, "tqmoe_count: invalid size or pointer");
+    if (int32_t rc = need_device(err, "tqmoe_count")) return rc;
+    count_k<<<unsigned((count + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(ids, reinterpret_cast<unsigned long long *>(counts), count);
+    return launched(err, "tqmoe_count");
+}
+
+extern "C" int32_t tqmoe_dedup_maps(const int32_t * ids, const int32_t * slot_of, int32_t count, int32_t topk, int32_t * slots, int32_t * gu, int32_t * dn,
+                                    int32_t groups, void * stream, tqmoe_error * err) {
+    if (!ids || !slot_of || count <= 0 || count > 1024 || topk <= 0 || groups < count) return fail(err, TQMOE_E_ARG, "tqmoe_dedup_maps: invalid shape");
+    if (int32_t rc = need_device(err, "tqmoe_dedup_maps")) return rc;
+    dedup_maps_k<<<1, 1024, 0, static_cast<hipStream_t>(stream)>>>(ids, slot_of, count, topk, slots, gu, dn, groups);
+    return launched(err, "tqmoe_dedup_maps");
 }

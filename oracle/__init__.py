@@ -357,6 +357,47 @@ def cpu_baseline_sweep(wtype, hidden, ff, experts_per_token, cores, budget_s=12.
             "sweep": sweep, "row_split_ms_per_expert": latency}
 
 
+def cpu_reference_shape(cores, sample_experts=24):
+    """The shape the reference's own program runs (tests/bench_cpu_expert_mt.cpp:26-61: 24 experts of IQ4_NL gate / up 640 x 2560
+    and down 2560 x 640, one token), on one thread and on all cores, fp32 and int8 activations: ms per expert and GB/s of
+    packed weights, for continuity with the figures that program prints."""
+    rng = np.random.default_rng(8)
+    hidden, ff = 2560, 640
+    banks = [random_blocks(IQ4_NL, sample_experts * rows, cols, rng) for rows, cols in ((ff, hidden), (ff, hidden), (hidden, ff))]
+    expert_bytes = sum(b.size for b in banks) / sample_experts
+    rows = []
+    for nt in sorted({1, cores}):
+        for int8 in (False, True):
+            t_pass, _ = cpu_expert_bench(IQ4_NL, *banks, hidden, ff, sample_experts, nt, int8, reps=2)
+            rows.append({"threads": nt, "variant": "int8" if int8 else "fp32", "ms_per_expert": round(t_pass / sample_experts * 1e3, 4),
+                         "gb_per_s": round(expert_bytes * sample_experts / t_pass / 1e9, 2)})
+    return {"shape": "IQ4_NL, %d experts, gate/up %dx%d, down %dx%d (tests/bench_cpu_expert_mt.cpp)" % (sample_experts, ff, hidden, hidden, ff), "rows": rows}
+
+
+def cpu_config1_layer(cores, tokens=(1, 16)):
+    """Configuration 1 whole on the host ("CPU reference, one MoE layer": hidden 2048, 64 Q4_K experts, softmax top-8
+    renormalised, ff 768, fp32 router and activations): router logits, routing, the selected experts' FFN from the decoded
+    weights in fp32, combine, on all cores. This is the correctness path timed as it is (it decodes every selected expert to
+    fp32 first), not a tuned kernel: tokens/s per batch size."""
+    import time
+    rng = np.random.default_rng(9)
+    h, f, e, k = 2048, 768, 64, 8
+    banks = [random_blocks(Q4_K, e * rows, cols, rng) for rows, cols in ((f, h), (f, h), (h, f))]
+    router = (rng.standard_normal((e, h)) * 0.02).astype(np.float32)
+    out = []
+    for n in tokens:
+        x = rng.standard_normal((n, h)).astype(np.float32)
+        best = None
+        for _ in range(2):
+            t0 = time.time()
+            logits = router_logits(router, F32, None, x, F32, h, e, n)
+            layer_forward(x, logits, *banks, Q4_K, h, f, e, k, threads=cores)
+            dt = time.time() - t0
+            best = dt if best is None else min(best, dt)
+        out.append({"tokens": n, "ms": round(best * 1e3, 2), "tokens_per_s": round(n / best, 1), "threads": cores})
+    return out
+
+
 def ref_lib():
     """The reference's own host objects, or None where they were not built (no reference tree)."""
     if not os.path.exists(REF_PATH):

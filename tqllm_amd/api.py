@@ -517,11 +517,12 @@ def gather_rows_i8(rows_q, rows_scale, lists, assignments, xdiv):
     return q, scale
 
 
-def expert_gemm_gateup(gate, up, x, lists, n, slots, topk, shared_ff=0):
+def expert_gemm_gateup(gate, up, x, lists, n, slots, topk, shared_ff=0, act=None):
     """WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59), any bank format, fp16 operands: fp16 act [n * slots][ff];
     rows of assignments that are in no list are zero here (the library leaves them untouched)."""
     counts, offsets, perm = lists
-    act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=x.device)
+    if act is None:
+        act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=x.device)
     err = _err()
     g, u = gate.view(), up.view()
     _check(lib().tqmoe_expert_gemm_gateup(C.byref(g), C.byref(u), _ptr(x), _ttype(x), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff,
@@ -529,10 +530,11 @@ def expert_gemm_gateup(gate, up, x, lists, n, slots, topk, shared_ff=0):
     return act
 
 
-def expert_gemm(bank, x, lists, n, slots, topk, shared_ff=0, per_expert_input=False, out_type=F16):
+def expert_gemm(bank, x, lists, n, slots, topk, shared_ff=0, per_expert_input=False, out_type=F16, y=None):
     """WeightFormat::expert_gemm (weight_format.hpp:51-53), any bank format, fp16 operands: y [n * slots][rows], fp16 or fp32."""
     counts, offsets, perm = lists
-    y = torch.zeros((n * slots, bank.rows), dtype=torch.float16 if out_type == F16 else torch.float32, device=x.device)
+    if y is None:
+        y = torch.zeros((n * slots, bank.rows), dtype=torch.float16 if out_type == F16 else torch.float32, device=x.device)
     err = _err()
     b = bank.view()
     _check(lib().tqmoe_expert_gemm(C.byref(b), _ptr(x), _ttype(x), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff, int(per_expert_input),
@@ -540,11 +542,12 @@ def expert_gemm(bank, x, lists, n, slots, topk, shared_ff=0, per_expert_input=Fa
     return y
 
 
-def expert_gemm_gateup_i8(gate, up, xq, xs, lists, n, slots, topk, shared_ff=0, fp8=False):
+def expert_gemm_gateup_i8(gate, up, xq, xs, lists, n, slots, topk, shared_ff=0, fp8=False, act=None):
     """WeightFormat::expert_gemm_gateup (weight_format.hpp:57-59) on int8 rows: fp16 act [n * slots][ff]; rows of
     assignments that are in no list are zero here (the library leaves them untouched)."""
     counts, offsets, perm = lists
-    act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=xq.device)
+    if act is None:
+        act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=xq.device)
     err = _err()
     g, u = gate.view(), up.view()
     fn = lib().tqmoe_expert_gemm_gateup_fp8 if fp8 else lib().tqmoe_expert_gemm_gateup_i8
@@ -558,11 +561,12 @@ def expert_gemm_gateup_fp8(gate, up, xq, xs, lists, n, slots, topk, shared_ff=0)
     return expert_gemm_gateup_i8(gate, up, xq, xs, lists, n, slots, topk, shared_ff, fp8=True)
 
 
-def expert_gemm_i8(bank, xq, xs, lists, n, slots, topk, shared_ff=0, fp8=False):
+def expert_gemm_i8(bank, xq, xs, lists, n, slots, topk, shared_ff=0, fp8=False, y=None):
     """WeightFormat::expert_gemm_i8 (weight_format.hpp:54-56), per-token scales, one input row per assignment: fp16
     y [n * slots][rows]."""
     counts, offsets, perm = lists
-    y = torch.zeros((n * slots, bank.rows), dtype=torch.float16, device=xq.device)
+    if y is None:
+        y = torch.zeros((n * slots, bank.rows), dtype=torch.float16, device=xq.device)
     err = _err()
     b = bank.view()
     fn = lib().tqmoe_expert_gemm_fp8 if fp8 else lib().tqmoe_expert_gemm_i8
@@ -574,10 +578,11 @@ def expert_gemm_fp8(bank, xq, xs, lists, n, slots, topk, shared_ff=0):
     return expert_gemm_i8(bank, xq, xs, lists, n, slots, topk, shared_ff, fp8=True)
 
 
-def expert_gemm_gateup_i8_blocks(gate, up, xq, xs, block_scale, lists, n, slots, topk, shared_ff=0):
+def expert_gemm_gateup_i8_blocks(gate, up, xq, xs, block_scale, lists, n, slots, topk, shared_ff=0, act=None):
     """expert_gemm_gateup_i8 on rows with a scale per 32 values (expert_gemm_i8's mode 1, quant_kernels.cuh:13-16)."""
     counts, offsets, perm = lists
-    act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=xq.device)
+    if act is None:
+        act = torch.zeros((n * slots, gate.rows), dtype=torch.float16, device=xq.device)
     err = _err()
     g, u = gate.view(), up.view()
     _check(lib().tqmoe_expert_gemm_gateup_i8_blocks(C.byref(g), C.byref(u), _ptr(xq), _ptr(xs), _ptr(block_scale), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots,
@@ -585,10 +590,11 @@ def expert_gemm_gateup_i8_blocks(gate, up, xq, xs, block_scale, lists, n, slots,
     return act
 
 
-def expert_gemm_i8_blocks(bank, xq, xs, block_scale, lists, n, slots, topk, shared_ff=0):
+def expert_gemm_i8_blocks(bank, xq, xs, block_scale, lists, n, slots, topk, shared_ff=0, y=None):
     """WeightFormat::expert_gemm_i8 (weight_format.hpp:54-56) with a scale per 32 values of the input rows (mode 1)."""
     counts, offsets, perm = lists
-    y = torch.zeros((n * slots, bank.rows), dtype=torch.float16, device=xq.device)
+    if y is None:
+        y = torch.zeros((n * slots, bank.rows), dtype=torch.float16, device=xq.device)
     err = _err()
     b = bank.view()
     _check(lib().tqmoe_expert_gemm_i8_blocks(C.byref(b), _ptr(xq), _ptr(xs), _ptr(block_scale), _ptr(counts), _ptr(offsets), _ptr(perm), n, slots, topk, shared_ff,

@@ -14,21 +14,24 @@ int32_t enqueue_quant_rows_i8_blocks(const void * x, uint32_t xtype, int64_t row
 int32_t enqueue_gather_rows_i8(const int8_t * rq, const float * rs, int cols, const int * counts, const int * offsets, const int * perm, int experts,
                                int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, float * block_scale);
 int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
-                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8, float * block_scale);
+                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8, float * block_scale, const float * plan_from);
 int32_t enqueue_gather_rows_natural(const int8_t * rq, const float * rs, int cols, const int * counts, const int * offsets, const int * perm, int experts,
                                     int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, float * block_scale);
 bool plane_gemm_has(uint32_t type);
 bool plane_gemm_is_fp8(uint32_t type);
 int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
                            const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s,
-                           const float * xbs, Glu glu, int out_bf16);
+                           const float * xbs, Glu glu, int out_bf16, const float * plan_from);
+int32_t group_rows_common(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t experts,
+                          int64_t assignments, int32_t xdiv, void * q, float * scale, void * stream, tqmoe_error * err, bool f8, const char * what,
+                          float * block_scale = nullptr, bool blocks = false, const float * plan_from = nullptr);
 
 int32_t expert_gateup_glu(const tqmoe_bank * gate, const tqmoe_bank * up, const void * x_image, void * act_image, const int32_t * ids, int32_t n,
                           int32_t slots, int32_t topk, int32_t shared_ff, Glu glu, void * stream, tqmoe_error * err);
 int32_t gemm_8bit_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                          const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
                          tqmoe_error * err, const char * what, bool fp8, const float * block_scale = nullptr, bool blocks = false, Glu glu = Glu{0.f, 0},
-                         int out_bf16 = 0);
+                         int out_bf16 = 0, const float * plan_from = nullptr);
 int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int32_t * counts, const int32_t * offsets,
                         const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, int32_t xdiv, void * out, uint32_t otype, int gateup,
                         void * stream, tqmoe_error * err, const char * what, Glu glu = Glu{0.f, 0});
@@ -420,9 +423,9 @@ extern "C" int64_t tqmoe_grouped_scale_words(int64_t assignments, int32_t expert
     return assignments > 0 && experts > 0 ? grouped_scale_words(assignments, experts) : 0;
 }
 
-static int32_t group_rows_common(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t experts,
+int32_t tqmoe::group_rows_common(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t experts,
                                  int64_t assignments, int32_t xdiv, void * q, float * scale, void * stream, tqmoe_error * err, bool f8, const char * what,
-                                 float * block_scale = nullptr, bool blocks = false) {
+                                 float * block_scale, bool blocks, const float * plan_from) {
     if (blocks && !block_scale) return fail(err, TQMOE_E_ARG, "%s: block scales missing", what);
     if (!x || !counts || !offsets || !perm || !q || !scale || cols <= 0 || cols % 32 || experts <= 0 || experts > 4096 || assignments <= 0 || xdiv <= 0 ||
         grouped_row_tiles(assignments, experts) > 0x7FFFFFFF)
@@ -430,7 +433,7 @@ static int32_t group_rows_common(const void * x, uint32_t xtype, int32_t cols, c
     if (!is_act_type(xtype)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported element type", what);
     if (int32_t rc = need_device(err, what)) return rc;
     enqueue_group_rows_i8(x, xtype, cols, counts, offsets, perm, experts, assignments, xdiv, static_cast<int8_t *>(q), scale, static_cast<hipStream_t>(stream), f8,
-                          block_scale);
+                          block_scale, plan_from);
     return launched(err, what);
 }
 
@@ -476,7 +479,7 @@ extern "C" int32_t tqmoe_gather_rows_i8_blocks(const int8_t * rows_q, const floa
 
 int32_t tqmoe::gemm_8bit_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                            const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
-                           tqmoe_error * err, const char * what, bool fp8, const float * block_scale, bool blocks, Glu glu, int out_bf16) {
+                           tqmoe_error * err, const char * what, bool fp8, const float * block_scale, bool blocks, Glu glu, int out_bf16, const float * plan_from) {
     if (blocks && !block_scale) return fail(err, TQMOE_E_ARG, "%s: block scales missing", what);
     if (int32_t rc = check_bank(b0, what, err)) return rc;
     if (b1) {
@@ -495,7 +498,7 @@ int32_t tqmoe::gemm_8bit_common(const tqmoe_bank * b0, const tqmoe_bank * b1, co
     if (int32_t rc = need_device(err, what)) return rc;
     const int shared_expert = slots > topk ? b0->experts - 1 : -1;
     if (enqueue_plane_gemm(*b0, b1, xq, xs, counts, offsets, perm, b0->experts, int64_t(n) * slots, out, gateup, shared_expert, shared_lim,
-                           static_cast<hipStream_t>(stream), block_scale, glu, out_bf16))
+                           static_cast<hipStream_t>(stream), block_scale, glu, out_bf16, plan_from))
         return fail(err, TQMOE_E_ARG, "%s: too many assignments for one call", what);
     return launched(err, what);
 }

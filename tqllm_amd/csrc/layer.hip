@@ -15,7 +15,11 @@ int32_t expert_gateup_glu(const tqmoe_bank * gate, const tqmoe_bank * up, const 
                           int32_t slots, int32_t topk, int32_t shared_ff, Glu glu, void * stream, tqmoe_error * err);
 int32_t gemm_8bit_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int32_t * counts, const int32_t * offsets,
                          const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, void * out, int gateup, void * stream,
-                         tqmoe_error * err, const char * what, bool fp8, const float * block_scale, bool blocks, Glu glu, int out_bf16);
+                         tqmoe_error * err, const char * what, bool fp8, const float * block_scale, bool blocks, Glu glu, int out_bf16, const float * plan_from);
+// the act rows' grouping and the down product read the index that the input rows' grouping built (the same lists)
+int32_t group_rows_common(const void * x, uint32_t xtype, int32_t cols, const int32_t * counts, const int32_t * offsets, const int32_t * perm, int32_t experts,
+                          int64_t assignments, int32_t xdiv, void * q, float * scale, void * stream, tqmoe_error * err, bool f8, const char * what,
+                          float * block_scale, bool blocks, const float * plan_from);
 int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void * x, uint32_t xtype, const int32_t * counts, const int32_t * offsets,
                         const int32_t * perm, int32_t n, int32_t slots, int32_t topk, int32_t shared_lim, int32_t xdiv, void * out, uint32_t otype, int gateup,
                         void * stream, tqmoe_error * err, const char * what, Glu glu);
@@ -213,28 +217,33 @@ static int32_t layer_forward(const tqmoe_layer * layer, const void * x, uint32_t
             int8_t * rq = reinterpret_cast<int8_t *>(ws + p.rq);
             float * rs = reinterpret_cast<float *>(ws + p.rs);
             if (plane_gemm_is_fp8(L.gate.type)) {
-                uint8_t * aq8 = reinterpret_cast<uint8_t *>(aq);
                 if (int32_t rc = tqmoe_quant_rows_fp8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, reinterpret_cast<uint8_t *>(rq), rs, stream, err)) return rc;
                 if (int32_t rc = tqmoe_gather_rows_i8(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, stream, err)) return rc;
                 if (int32_t rc = gemm_8bit_common(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, 1, stream, err,
-                                                  "tqmoe_layer_forward (gate / up)", true, nullptr, false, glu, 0)) return rc;
-                if (int32_t rc = tqmoe_group_rows_fp8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq8, as, stream, err)) return rc;
-                if (int32_t rc = tqmoe_expert_gemm_fp8(&L.down, aq8, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
+                                                  "tqmoe_layer_forward (gate / up)", true, nullptr, false, glu, 0, nullptr)) return rc;
+                if (int32_t rc = group_rows_common(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err, true,
+                                                   "tqmoe_layer_forward (act rows)", nullptr, false, xs)) return rc;
+                if (int32_t rc = gemm_8bit_common(&L.down, nullptr, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, 0, stream, err,
+                                                  "tqmoe_layer_forward (down)", true, nullptr, false, Glu{0.f, 0}, 0, xs)) return rc;
             } else if (p.blocks) {
             float * xbs = reinterpret_cast<float *>(ws + p.xbs), * abks = reinterpret_cast<float *>(ws + p.abks);
             if (int32_t rc = tqmoe_quant_rows_i8_blocks(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, rq, rs, nullptr, stream, err)) return rc;
             if (int32_t rc = tqmoe_gather_rows_i8_blocks(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, xbs, stream, err)) return rc;
             if (int32_t rc = gemm_8bit_common(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, 1, stream, err,
-                                              "tqmoe_layer_forward (gate / up)", false, xbs, true, glu, 0)) return rc;
-            if (int32_t rc = tqmoe_group_rows_i8_blocks(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, abks, stream, err)) return rc;
-            if (int32_t rc = tqmoe_expert_gemm_i8_blocks(&L.down, aq, as, abks, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
+                                              "tqmoe_layer_forward (gate / up)", false, xbs, true, glu, 0, nullptr)) return rc;
+            if (int32_t rc = group_rows_common(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err, false,
+                                               "tqmoe_layer_forward (act rows)", abks, true, xs)) return rc;
+            if (int32_t rc = gemm_8bit_common(&L.down, nullptr, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, 0, stream, err,
+                                              "tqmoe_layer_forward (down)", false, abks, true, Glu{0.f, 0}, 0, xs)) return rc;
             } else {
             if (int32_t rc = tqmoe_quant_rows_i8(xb + size_t(t0) * L.hidden * xbytes, xtype, c, L.hidden, rq, rs, stream, err)) return rc;
             if (int32_t rc = tqmoe_gather_rows_i8(rq, rs, L.hidden, counts, offsets, perm, banks, int64_t(c) * slots, slots, xq, xs, stream, err)) return rc;
             if (int32_t rc = gemm_8bit_common(&L.gate, &L.up, xq, xs, counts, offsets, perm, c, slots, L.topk, L.shared_ff, act16, 1, stream, err,
-                                              "tqmoe_layer_forward (gate / up)", false, nullptr, false, glu, 0)) return rc;
-            if (int32_t rc = tqmoe_group_rows_i8(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err)) return rc;
-            if (int32_t rc = tqmoe_expert_gemm_i8(&L.down, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, stream, err)) return rc;
+                                              "tqmoe_layer_forward (gate / up)", false, nullptr, false, glu, 0, nullptr)) return rc;
+            if (int32_t rc = group_rows_common(act16, TQMOE_F16, L.ff, counts, offsets, perm, banks, int64_t(c) * slots, 1, aq, as, stream, err, false,
+                                               "tqmoe_layer_forward (act rows)", nullptr, false, xs)) return rc;
+            if (int32_t rc = gemm_8bit_common(&L.down, nullptr, aq, as, counts, offsets, perm, c, slots, L.topk, L.shared_ff, y16, 0, stream, err,
+                                              "tqmoe_layer_forward (down)", false, nullptr, false, Glu{0.f, 0}, 0, xs)) return rc;
             }
             }
             if (int32_t rc = combine(y16, TQMOE_F16, L.has_shared ? y16 + size_t(L.topk) * L.hidden : nullptr)) return rc;

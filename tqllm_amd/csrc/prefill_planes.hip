@@ -341,11 +341,13 @@ static void group_rows_launch(const void * x, int cols, const int * counts, cons
 }
 
 // block_scale (int8 only): a scale per row and 32-value block, [row tile][block][32 rows]; the rows' own scales are then 1
+// plan_from: the scales of another grouping of the same lists (same counts, same experts, same bound of assignments) whose
+// index is read in place of building this one's again; the products on these rows must then be given it as well
 int32_t enqueue_group_rows_i8(const void * x, uint32_t xtype, int cols, const int * counts, const int * offsets, const int * perm, int experts,
-                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8, float * block_scale) {
+                              int64_t assignments, int xdiv, int8_t * q, float * scale, hipStream_t s, bool f8, float * block_scale, const float * plan_from) {
     const int64_t tiles = grouped_row_tiles(assignments, experts);
-    const Plan plan = plan_at(scale, tiles * 32, experts);
-    plan_k<<<1, 64, 0, s>>>(counts, experts, plan);
+    const Plan plan = plan_at(plan_from ? plan_from : scale, tiles * 32, experts);
+    if (!plan_from) plan_k<<<1, 64, 0, s>>>(counts, experts, plan);
 #define TQMOE_GROUP(XT) (f8 ? group_rows_launch<XT, true, false>(x, cols, counts, offsets, perm, experts, tiles, xdiv, q, scale, plan, s, nullptr) \
                          : block_scale ? group_rows_launch<XT, false, true>(x, cols, counts, offsets, perm, experts, tiles, xdiv, q, scale, plan, s, block_scale) \
                                        : group_rows_launch<XT, false, false>(x, cols, counts, offsets, perm, experts, tiles, xdiv, q, scale, plan, s, nullptr))
@@ -388,14 +390,14 @@ bool plane_gemm_is_fp8(uint32_t type) { return type == TQMOE_NVFP4G; }
 int32_t plane_gemm_blocks(uint32_t type, int nb, bool gateup, const GemmArgs & k, unsigned blocks, hipStream_t s);
 int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
                            const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s,
-                           const float * xbs, Glu glu, int out_bf16) {
+                           const float * xbs, Glu glu, int out_bf16, const float * plan_from) {
     const int nb = gateup || b0.rows % 64 == 0 ? 2 : 1;
     const int units = gateup ? b0.rows / 32 : b0.rows / (32 * nb);
     const int64_t tiles = grouped_row_tiles(assignments, experts);
     // units per item: about sixteen super-block steps of products behind one item's start-up, in a divisor of the units
     int unit_group = std::max(1, std::min(4, 16 / std::max(1, b0.cols / 256)));
     while (units % unit_group) --unit_group;
-    GemmArgs k{view(b0), b1 ? view(*b1) : view(b0), xq, xs, counts, offsets, perm, plan_at(xs, tiles * 32, experts), experts, static_cast<uint16_t *>(out_f16),
+    GemmArgs k{view(b0), b1 ? view(*b1) : view(b0), xq, xs, counts, offsets, perm, plan_at(plan_from ? plan_from : xs, tiles * 32, experts), experts, static_cast<uint16_t *>(out_f16),
                units, unit_group, shared_expert, shared_lim, xbs, glu, out_bf16};
     // one block per compute unit (the kernel's registers and LDS allow no second one), walking the work items
     const int cus = cu_count();

@@ -220,6 +220,19 @@ int32_t tqmoe_expert_matvec2_rows(const tqmoe_bank * gate, const tqmoe_bank * up
                                   void * y_gate, void * y_up, uint32_t ytype, const int32_t * ids, int32_t n, int32_t topk,
                                   void * scratch, size_t scratch_bytes, void * stream, tqmoe_error * err);
 
+/* The same products over the decode grouping maps of tqmoe_dedup_maps (kDedupStride = 18 ints a group: slot, columns, input
+ * row x 8, output row x 8): y[output row][r] = sum_c W[slot * rows + r][c] * x[input row][c] for every column of every group
+ * whose slot is not negative. WeightFormat::expert_matvec_dedup / expert_matvec_dedup2 (weight_format.hpp:66-69; kernels
+ * src/formats/weight/quant.cu:113-129, 196-205, quant_u4h.inc:437-447, 488-491). bank2 / y2: a second bank of the same format
+ * and shape over the same maps (gate and up), or NULL. x: device rows of xtype; y: device rows of bank rows elements of ytype
+ * (F32 or BF16); rows no column names stay untouched. The map's columns run as assignments of the decode kernels (which read an
+ * expert's weights once for all of them); scratch: device memory of tqmoe_expert_matvec_dedup_scratch_bytes(), dead after
+ * the call. groups * 8 <= 65535. */
+size_t  tqmoe_expert_matvec_dedup_scratch_bytes(int32_t groups, int32_t rows, int32_t cols, uint32_t ytype, int32_t two_banks);
+int32_t tqmoe_expert_matvec_dedup(const tqmoe_bank * bank, const tqmoe_bank * bank2, const void * x, uint32_t xtype, void * y,
+                                  void * y2, uint32_t ytype, const int32_t * dmap, int32_t groups, void * scratch,
+                                  size_t scratch_bytes, void * stream, tqmoe_error * err);
+
 /* Decode stages of the layer (tqmoe_layer_forward is router, top-k, tqmoe_extend_ids, tqmoe_quant_act, these two and
  * tqmoe_combine_strided). `ids` holds the expert of every (token, slot), [n][slots]: the routed ids and, when
  * slots == topk + 1, the shared expert's bank index in the last slot (tqmoe_extend_ids makes it). One block serves every

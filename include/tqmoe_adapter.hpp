@@ -282,6 +282,22 @@ struct ExpertOverrides : Base {
         const tqmoe_bank bg = bank_of(g, rows), bu = bank_of(u, rows);
         check(tqmoe_expert_matvec2_rows(&bg, &bu, x, TQMOE_F16, yg, yu, TQMOE_BF16, ids, n, topk, scratch, scratch_bytes, (void *)stream, &e), e);
     }
+    // expert_matvec_dedup / expert_matvec_dedup2 (weight_format.hpp:66-69) over the maps of moe_dedup_maps; the scratch must hold
+    // tqmoe_expert_matvec_dedup_scratch_bytes(groups, rows, cols, TQMOE_BF16, two banks). The base's has_expert_dedup() follows its
+    // u4h_id(), which stays -1 here (the id selects kernels of the reference's own u4h family): an engine that asks
+    // has_expert_dedup() finds these, one that asks u4h_id() takes expert_matvec, which serves an expert's rows together as well.
+    bool has_expert_dedup() const override { return true; }
+    void expert_matvec_dedup(const MatT & m, const HalfT * x, Bf16T * y, int rows, const int * dmap, int groups, StreamT stream) const override {
+        tqmoe_error e = fresh();
+        const tqmoe_bank b = bank_of(m, rows);
+        check(tqmoe_expert_matvec_dedup(&b, nullptr, x, TQMOE_F16, y, nullptr, TQMOE_BF16, dmap, groups, scratch, scratch_bytes, (void *)stream, &e), e);
+    }
+    void expert_matvec_dedup2(const MatT & g, const MatT & u, const HalfT * x, Bf16T * yg, Bf16T * yu, int rows, const int * dmap, int groups,
+                              StreamT stream) const override {
+        tqmoe_error e = fresh();
+        const tqmoe_bank bg = bank_of(g, rows), bu = bank_of(u, rows);
+        check(tqmoe_expert_matvec_dedup(&bg, &bu, x, TQMOE_F16, yg, yu, TQMOE_BF16, dmap, groups, scratch, scratch_bytes, (void *)stream, &e), e);
+    }
     // the lists in this library's form, in the scratch: the counts clamped to the capacity [experts], offsets [experts + 1],
     // then perm. The products are given the clamped counts: a count above the capacity names entries the lists do not hold.
     struct Lists { int32_t * counts, * offsets, * perm; int64_t bound; };

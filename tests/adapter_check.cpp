@@ -10,10 +10,11 @@
 // gate.bin, up.bin (GGUF blocks), x.bin (fp16 [n][cols]), ids.bin (int32 [n][topk]), counts.bin, groups.bin, and for the int8
 // product xq1.bin / xq2.bin (int8 [n][cols], natural order: quantised per block / per token), xs1.bin / xs2.bin (fp32
 // [n][cols / 32]: a scale per block / the token's scale repeated), xsum.bin (int16 [n][cols / 32][2]); writes yg.bin, yu.bin, y1.bin (bf16 [n * topk][rows]), act.bin (fp16), yd.bin
-// (bf16), yi1.bin / yi2.bin (bf16: the int8 product in modes 1 and 2; absent when the format has none), ycap.bin (bf16: expert_gemm
+// (bf16), dg.bin / du.bin / dg1.bin (bf16: expert_matvec_dedup2 and expert_matvec_dedup over maps built by moe_dedup_maps), yi1.bin / yi2.bin (bf16: the int8 product in modes 1 and 2; absent when the format has none), ycap.bin (bf16: expert_gemm
 // with a capacity below the largest count), mg_counts.bin / mg_groups.bin (int32: moe_group)
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cstdint>
 #include <cstdio>
 #include <fstream>
@@ -44,6 +45,10 @@ struct WeightFormat {
     virtual bool has_expert_matvec() const { return false; }
     virtual void expert_matvec(const Mat &, const __half *, __nv_bfloat16 *, int, const int *, int, int, bool, cudaStream_t) const {}
     virtual void expert_matvec2(const Mat &, const Mat &, const __half *, __nv_bfloat16 *, __nv_bfloat16 *, int, const int *, int, int, cudaStream_t) const {}
+    virtual int u4h_id() const { return -1; }
+    virtual bool has_expert_dedup() const { return u4h_id() >= 0; }
+    virtual void expert_matvec_dedup(const Mat &, const __half *, __nv_bfloat16 *, int, const int *, int, cudaStream_t) const {}
+    virtual void expert_matvec_dedup2(const Mat &, const Mat &, const __half *, __nv_bfloat16 *, __nv_bfloat16 *, int, const int *, int, cudaStream_t) const {}
 };
 }  // namespace tqllm
 
@@ -105,7 +110,8 @@ int main(int argc, char ** argv) {
         const int * ids = static_cast<const int *>(to_device(slurp(dir + "/ids.bin")));
         const int * counts = static_cast<const int *>(to_device(slurp(dir + "/counts.bin")));
         const int * groups = static_cast<const int *>(to_device(slurp(dir + "/groups.bin")));
-        const size_t sb = tqmoe_hip::expert_scratch_bytes(cols, A, A, experts, 1);
+        size_t sb = tqmoe_hip::expert_scratch_bytes(cols, A, A, experts, 1);
+        sb = std::max(sb, tqmoe_expert_matvec_dedup_scratch_bytes(A, rows, cols, TQMOE_BF16, 1));
         fmt.set_scratch(device_zeros(sb), sb);
         fmt.max_assignments = A;
 
@@ -146,6 +152,25 @@ int main(int argc, char ** argv) {
             if (!base->expert_gemm(mats[1], x, ycap, rows, counts, groups2, cap2, experts, topk, false, nullptr)) return 9;
             hip(hipDeviceSynchronize(), "synchronize");
             dump(dir + "/ycap.bin", ycap, ybytes);
+        }
+        // the decode grouping maps built on the device (moe_dedup_maps, every expert in its own bank slot) and the pair of products
+        // over them: the rows must be those of expert_matvec2 over the ids
+        if (A <= 1024) {
+            if (!base->has_expert_dedup()) return 11;
+            std::vector<int> ident(experts);
+            for (int e = 0; e < experts; ++e) ident[e] = e;
+            const int * slot_of = static_cast<const int *>(to_device(std::vector<char>(reinterpret_cast<const char *>(ident.data()), reinterpret_cast<const char *>(ident.data() + experts))));
+            int * gu = static_cast<int *>(device_zeros(size_t(A) * tqmoe_hip::kDedupStride * 4)), * dn = static_cast<int *>(device_zeros(size_t(A) * tqmoe_hip::kDedupStride * 4));
+            tqmoe_hip::moe_dedup_maps(ids, slot_of, A, topk, nullptr, gu, dn, A, nullptr);
+            __nv_bfloat16 * dg = static_cast<__nv_bfloat16 *>(device_zeros(ybytes)), * du = static_cast<__nv_bfloat16 *>(device_zeros(ybytes));
+            base->expert_matvec_dedup2(mats[0], mats[1], x, dg, du, rows, gu, A, nullptr);
+            hip(hipDeviceSynchronize(), "synchronize");
+            dump(dir + "/dg.bin", dg, ybytes);
+            dump(dir + "/du.bin", du, ybytes);
+            hip(hipMemset(dg, 0, ybytes), "hipMemset");
+            base->expert_matvec_dedup(mats[0], x, dg, rows, gu, A, nullptr);
+            hip(hipDeviceSynchronize(), "synchronize");
+            dump(dir + "/dg1.bin", dg, ybytes);
         }
         // moe_group with the reference's seven arguments (moe_kernels.cuh:29): counts [experts], groups [experts][n]
         {

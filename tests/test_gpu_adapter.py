@@ -84,6 +84,11 @@ def test_adapter_through_reference_signatures(oracle, tmp_path, wtype_name):
     want_act = g / (1 + np.exp(-g)) * u
     err = np.abs(act - want_act)[listed]
     assert err.max() < 1e-2 * max(1.0, np.abs(want_act).max()) and np.sqrt(np.mean(err ** 2) / np.mean(want_act[listed] ** 2)) < 5e-3
+    # the products over the decode grouping maps give the rows of the products over the ids (the same kernels; the waves may
+    # split a row's sum differently for another number of assignments, so to fp32 rounding: at most one bf16 step)
+    dg, du, dg1 = (bf16_to_f64(read(name, np.uint16)) for name in ("dg", "du", "dg1"))
+    for got, ref in ((dg, yg), (du, yu), (dg1, yg)):
+        assert np.abs(got - ref).max() <= 2.0 ** -7 * np.abs(ref).max() and (got != ref).mean() < 0.01 and not got[~listed].any()
     # moe_group with the reference's seven arguments: counts and ascending lists [experts][n]
     mc = np.fromfile(os.path.join(d, "mg_counts.bin"), np.int32)
     mg = np.fromfile(os.path.join(d, "mg_groups.bin"), np.int32).reshape(experts, n)

@@ -65,6 +65,32 @@ def test_dedup_maps_bit_exact(tq, experts, n, topk, skew):
         tq.moe_dedup_maps(dev(ids), dev(slot_of), topk, len(ids) - 1)
 
 
+@pytest.mark.parametrize("wtype_name", ["IQ4_XS", "IQ3_S"])
+def test_matvec_over_dedup_maps(tq, oracle, wtype_name):
+    """The products over the maps of moe_dedup_maps (gate / up from the token rows, down from a row per assignment) equal the
+    products over the ids (to fp32 rounding: the waves may split a row's sum differently for another number of assignments),
+    with bank slots that are not the experts' numbers and skipped assignments."""
+    wtype = getattr(oracle, wtype_name)
+    rng = np.random.default_rng(5)
+    experts, rows, cols, n, topk = 12, 128, 512, 9, 4
+    slot_of = rng.permutation(experts).astype(np.int32)
+    ids = np.stack([rng.permutation(experts)[:topk] for _ in range(n)]).astype(np.int32)
+    ids[2, 1] = -1
+    banks = [tq.ExpertBank(wtype, synth.bank_blocks(wtype, experts * rows, cols, rng), experts, rows, cols) for _ in range(2)]
+    x = torch.randn(n, cols, device="cuda", dtype=torch.float16)
+    slots, gu, dn = tq.moe_dedup_maps(dev(ids.reshape(-1)), dev(slot_of), topk)
+    slot_ids = slots.view(n, topk)
+    img = tq.quant_act(x)
+    want_g, want_u = tq.expert_matvec2(banks[0], banks[1], img, slot_ids)
+    got_g, got_u = tq.expert_matvec_dedup(banks[0], x, gu, n * topk, bank2=banks[1])
+    for got, want in ((got_g, want_g), (got_u, want_u)):
+        assert (got - want).abs().max().item() <= 2e-6 * want.abs().max().item()
+    xa = torch.randn(n * topk, cols, device="cuda", dtype=torch.float16)          # a row per assignment: the down product's input
+    want_d = tq.expert_matvec(banks[0], tq.quant_act(xa), slot_ids, per_expert_input=True, out_type=tq.BF16)
+    got_d = tq.expert_matvec_dedup(banks[0], xa, dn, n * topk, out_type=tq.BF16)
+    assert (got_d.float() - want_d.float()).abs().max().item() <= 2.0 ** -7 * want_d.float().abs().max().item() and not got_d[2 * topk + 1].any()
+
+
 def test_count_and_group(tq, oracle):
     rng = np.random.default_rng(4)
     experts, n, topk = 96, 700, 6

@@ -79,6 +79,9 @@ def lib():
         l.tqmoe_expert_gemm_i8_ref_scratch_bytes.argtypes = [i32, i64, i32, i32]
         l.tqmoe_expert_gemm_i8_ref.argtypes = [C.POINTER(_Bank), p, p, p, p, u32, p, p, i32, i32, i32, i32, i32, i64, p, sz, p, e]
         l.tqmoe_swiglu_clamped.argtypes = [p, p, p, i64, f32, i32, p, e]
+        l.tqmoe_expert_matvec_dedup_scratch_bytes.restype = sz
+        l.tqmoe_expert_matvec_dedup_scratch_bytes.argtypes = [i32, i32, i32, u32, i32]
+        l.tqmoe_expert_matvec_dedup.argtypes = [C.POINTER(_Bank), C.POINTER(_Bank), p, u32, p, p, u32, p, i32, p, sz, p, e]
         l.tqmoe_bank_layout.argtypes = [u32, i64, i32, C.POINTER(sz), C.POINTER(sz), e]
         l.tqmoe_bank_load.argtypes = [u32, p, i64, i32, p, p, p, p, e]
         l.tqmoe_bank_dequant.argtypes = [C.POINTER(_Bank), i64, i64, p, p, e]
@@ -255,6 +258,22 @@ def moe_dedup_maps(ids, slot_of, topk, groups=None):
     err = _err()
     _check(lib().tqmoe_dedup_maps(_ptr(ids), _ptr(slot_of), count, topk, _ptr(slots), _ptr(gu), _ptr(dn), groups, _stream(ids), C.byref(err)), err)
     return slots, gu, dn
+
+
+def expert_matvec_dedup(bank, x, dmap, out_rows, bank2=None, out_type=F32):
+    """WeightFormat::expert_matvec_dedup / _dedup2 (weight_format.hpp:66-69) over a map of moe_dedup_maps: y [out_rows][rows]
+    (and a second one for bank2); rows no column names stay zero here."""
+    groups = dmap.shape[0]
+    y = torch.zeros((out_rows, bank.rows), dtype=_OUT_TYPE[out_type], device=x.device)
+    y2 = torch.zeros_like(y) if bank2 is not None else None
+    need = lib().tqmoe_expert_matvec_dedup_scratch_bytes(groups, bank.rows, bank.cols, out_type, int(bank2 is not None))
+    scratch = torch.empty(max(need, 16), dtype=torch.uint8, device=x.device)
+    err = _err()
+    b = bank.view()
+    b2 = bank2.view() if bank2 is not None else None
+    _check(lib().tqmoe_expert_matvec_dedup(C.byref(b), C.byref(b2) if b2 is not None else None, _ptr(x), _ttype(x), _ptr(y), _ptr(y2), out_type, _ptr(dmap), groups,
+                                           _ptr(scratch), scratch.numel(), _stream(x), C.byref(err)), err)
+    return (y, y2) if bank2 is not None else y
 
 
 def lists_from_groups(counts, groups, bound=None):

@@ -139,11 +139,14 @@ template <int XT> __device__ __forceinline__ void quantise_row_wave(const void *
         quantise_block(v, image_row, S, s, amax);
     }
 }
+// row_map (may be null): image row i is made of input row row_map[i]; a negative entry leaves the image row as it is
 template <int XT>
-__global__ __launch_bounds__(256) void quant_act_k(const void * __restrict__ x, int n, int cols, uint8_t * __restrict__ image) {
+__global__ __launch_bounds__(256) void quant_act_k(const void * __restrict__ x, int n, int cols, uint8_t * __restrict__ image, const int * __restrict__ row_map = nullptr) {
     const int64_t row = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (row >= n) return;
-    quantise_row_wave<XT>(x, row, cols, image + row * int64_t(cols / 32) * kImageSubBytes, threadIdx.x & 63);
+    const int64_t src = row_map ? row_map[row] : row;
+    if (src < 0) return;
+    quantise_row_wave<XT>(x, src, cols, image + row * int64_t(cols / 32) * kImageSubBytes, threadIdx.x & 63);
 }
 
 }  // namespace

@@ -134,6 +134,31 @@ __global__ __launch_bounds__(1024) void lists_from_groups_k(const int * __restri
     }
 }
 
+// The decode grouping maps (kDedupStride ints per group: slot, columns, input row x 8, output row x 8; src/formats/weight/
+// quant_kernels.cuh:26-27) as one virtual assignment per map column: its expert (-1 for a column the map does not use, or a
+// group whose slot is negative), its input row and its output row.
+constexpr int kDedupCols = 8, kDedupStride = 2 + 2 * kDedupCols;
+__global__ __launch_bounds__(256) void dedup_expand_k(const int * __restrict__ dmap, int groups, int * __restrict__ ids, int * __restrict__ in_row, int * __restrict__ out_row) {
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= groups * kDedupCols) return;
+    const int * e = dmap + int64_t(j / kDedupCols) * kDedupStride;
+    const int c = j % kDedupCols;
+    const bool live = e[0] >= 0 && c < e[1];
+    ids[j] = live ? e[0] : -1;
+    in_row[j] = live ? e[2 + c] : -1;
+    out_row[j] = live ? e[2 + kDedupCols + c] : -1;
+}
+// y[out_row[j]] = tmp[j] for the live columns; rows of 2-byte elements (bf16) or 4-byte ones (fp32), `words` dwords a row
+__global__ __launch_bounds__(256) void dedup_scatter_k(const uint32_t * __restrict__ tmp0, const uint32_t * __restrict__ tmp1, uint32_t * __restrict__ y0,
+                                                       uint32_t * __restrict__ y1, const int * __restrict__ out_row, int words) {
+    const int o = out_row[blockIdx.x];
+    if (o < 0) return;
+    for (int i = threadIdx.x; i < words; i += 256) {
+        y0[int64_t(o) * words + i] = tmp0[int64_t(blockIdx.x) * words + i];
+        if (tmp1) y1[int64_t(o) * words + i] = tmp1[int64_t(blockIdx.x) * words + i];
+    }
+}
+
 void dispatch_matvec(uint32_t type, Split sp, int nb, const MatvecArgs & k, hipStream_t s) {
     switch (type) {
         case TQMOE_IQ4_XS: DecodeLaunch<TQMOE_IQ4_XS>::matvec(sp, nb, k, s); break;
@@ -259,6 +284,58 @@ extern "C" int32_t tqmoe_expert_matvec2_rows(const tqmoe_bank * gate, const tqmo
                                              tqmoe_error * err) {
     if (!up) return fail(err, TQMOE_E_ARG, "tqmoe_expert_matvec2_rows: second bank missing");
     return matvec_rows_common(gate, up, x, xtype, y_gate, y_up, ytype, ids, n, topk, 0, scratch, scratch_bytes, stream, err, "tqmoe_expert_matvec2_rows");
+}
+
+// scratch of tqmoe_expert_matvec_dedup: ids | input rows | output rows | activation image of the columns | result rows (x2)
+namespace {
+struct DedupScratch { size_t ids, in_row, out_row, image, y0, y1, total; };
+DedupScratch dedup_scratch(int groups, int rows, int cols, uint32_t ytype, bool two) {
+    DedupScratch r{};
+    size_t o = 0;
+    auto take = [&](size_t bytes) { const size_t at = o; o = align_up(o + bytes, 256); return at; };
+    const size_t n = size_t(groups) * kDedupCols;
+    r.ids = take(n * 4); r.in_row = take(n * 4); r.out_row = take(n * 4);
+    r.image = take(tqmoe_act_image_bytes(int32_t(n), cols));
+    r.y0 = take(n * rows * elem_bytes(ytype));
+    r.y1 = take(two ? n * rows * elem_bytes(ytype) : 0);
+    r.total = o;
+    return r;
+}
+}  // namespace
+
+extern "C" size_t tqmoe_expert_matvec_dedup_scratch_bytes(int32_t groups, int32_t rows, int32_t cols, uint32_t ytype, int32_t two_banks) {
+    if (groups <= 0 || rows <= 0 || cols <= 0 || cols % 32 || (ytype != TQMOE_F32 && ytype != TQMOE_BF16)) return 0;
+    return dedup_scratch(groups, rows, cols, ytype, two_banks != 0).total;
+}
+
+extern "C" int32_t tqmoe_expert_matvec_dedup(const tqmoe_bank * bank, const tqmoe_bank * bank2, const void * x, uint32_t xtype, void * y, void * y2, uint32_t ytype,
+                                             const int32_t * dmap, int32_t groups, void * scratch, size_t scratch_bytes, void * stream, tqmoe_error * err) {
+    const char * what = "tqmoe_expert_matvec_dedup";
+    if (int32_t rc = check_bank(bank, what, err)) return rc;
+    if (!x || !y || (bank2 && !y2) || !dmap || groups <= 0 || int64_t(groups) * kDedupCols > 65535) return fail(err, TQMOE_E_ARG, "%s: invalid shape or pointer", what);
+    if (!is_act_type(xtype) || (ytype != TQMOE_F32 && ytype != TQMOE_BF16)) return fail(err, TQMOE_E_UNSUPPORTED, "%s: unsupported element type", what);
+    const DedupScratch r = dedup_scratch(groups, bank->rows, bank->cols, ytype, bank2 != nullptr);
+    if (!scratch || scratch_bytes < r.total) return fail(err, TQMOE_E_WORKSPACE, "%s: scratch of %zu bytes needed", what, r.total);
+    if (int32_t rc = need_device(err, what)) return rc;
+    uint8_t * ws = static_cast<uint8_t *>(scratch);
+    int32_t * ids = reinterpret_cast<int32_t *>(ws + r.ids), * in_row = reinterpret_cast<int32_t *>(ws + r.in_row), * out_row = reinterpret_cast<int32_t *>(ws + r.out_row);
+    const int n = groups * kDedupCols;
+    const hipStream_t s = static_cast<hipStream_t>(stream);
+    dedup_expand_k<<<unsigned((n + 255) / 256), 256, 0, s>>>(dmap, groups, ids, in_row, out_row);
+    const unsigned qblocks = unsigned((n + 3) / 4);
+    switch (xtype) {
+        case TQMOE_F32: quant_act_k<TQMOE_F32><<<qblocks, 256, 0, s>>>(x, n, bank->cols, ws + r.image, in_row); break;
+        case TQMOE_F16: quant_act_k<TQMOE_F16><<<qblocks, 256, 0, s>>>(x, n, bank->cols, ws + r.image, in_row); break;
+        default: quant_act_k<TQMOE_BF16><<<qblocks, 256, 0, s>>>(x, n, bank->cols, ws + r.image, in_row); break;
+    }
+    if (int32_t rc = launched(err, what)) return rc;
+    // a virtual assignment per map column, one input row each; the kernels serve an expert's columns together as they do for ids
+    if (int32_t rc = matvec_common(bank, bank2, ws + r.image, ws + r.y0, bank2 ? ws + r.y1 : nullptr, ytype, ids, n, 1, 1, 1, 0, stream, err, what)) return rc;
+    const int words = int(size_t(bank->rows) * elem_bytes(ytype) / 4);
+    if (size_t(bank->rows) * elem_bytes(ytype) % 4) return fail(err, TQMOE_E_ARG, "%s: rows must make whole dwords", what);
+    dedup_scatter_k<<<unsigned(n), 256, 0, s>>>(reinterpret_cast<const uint32_t *>(ws + r.y0), bank2 ? reinterpret_cast<const uint32_t *>(ws + r.y1) : nullptr,
+                                                static_cast<uint32_t *>(y), static_cast<uint32_t *>(y2), out_row, words);
+    return launched(err, what);
 }
 
 extern "C" int32_t tqmoe_lists_from_groups_clamped(const int32_t * counts, const int32_t * groups, int32_t capacity, int32_t experts, int32_t * counts_out,

@@ -159,8 +159,11 @@ int32_t tqmoe_dedup_maps(const int32_t * ids, const int32_t * slot_of, int32_t c
  *   IQ4_NL  codes 16 B, GGUF's own nibble order; aux 2 B per sub-block: its d (f16).
  *   Q4_0    as IQ4_NL (the weight is the nibble minus 8).
  *   Q8_0    codes 32 B: the int8 values; aux 2 B per sub-block: its d (f16).
- * cols must be a multiple of 256 (128 for NVFP4G). The grouped int8 products take IQ4_XS only; every format has the
- * decode products and the fp16 grouped products (tqmoe_expert_gemm, tqmoe_expert_gemm_gateup). */
+ * cols must be a multiple of 256 (128 for NVFP4G). Every format has the decode products and the fp16 grouped products
+ * (tqmoe_expert_gemm, tqmoe_expert_gemm_gateup). The grouped int8 products take the formats with one scale per 32 weights
+ * (IQ4_XS, IQ4_NL, IQ3_S, IQ3_XXS, IQ2_XXS, IQ2_XS, IQ2_S, IQ1_S, Q4_K, Q5_K, Q4_0, Q8_0), the grouped fp8 products NVFP4G;
+ * Q6_K, Q3_K and Q2_K (a scale per 16 weights, half the depth of the int8 matrix instruction) have the fp16 grouped
+ * products only. */
 typedef struct tqmoe_bank {
     uint32_t struct_size;
     uint32_t type;            /* one of the bank formats of the enum above */

@@ -114,7 +114,7 @@ def test_quant_rows_fp8_bit_exact(tq, oracle, kind):
         assert s[r] == np.float32(ws)
 
 
-PLANE_FORMATS = ["IQ4_XS", "IQ3_S", "Q4_K", "NVFP4G", "IQ3_XXS", "IQ2_XXS", "IQ2_XS", "IQ2_S", "IQ1_S", "IQ4_NL"]
+PLANE_FORMATS = ["IQ4_XS", "IQ3_S", "Q4_K", "NVFP4G", "IQ3_XXS", "IQ2_XXS", "IQ2_XS", "IQ2_S", "IQ1_S", "IQ4_NL", "Q5_K", "Q4_0", "Q8_0"]
 
 
 @pytest.mark.parametrize("wtype", PLANE_FORMATS)
@@ -342,7 +342,7 @@ def test_grouped_products_refuse_the_wrong_operand_type(tq, oracle):
     counts, offsets, perm, _ = tq.moe_dispatch(dev(ids), 2)
     x = torch.randn(4, 256, device="cuda", dtype=torch.float16)
     xq, xs = tq.group_rows_i8(x, (counts, offsets, perm), 4, 1)
-    for bank, fn in ((mk(oracle.NVFP4G), tq.expert_gemm_i8), (mk(oracle.IQ4_XS), tq.expert_gemm_fp8), (mk(oracle.Q8_0), tq.expert_gemm_i8)):
+    for bank, fn in ((mk(oracle.NVFP4G), tq.expert_gemm_i8), (mk(oracle.IQ4_XS), tq.expert_gemm_fp8), (mk(oracle.Q6_K), tq.expert_gemm_i8)):
         with pytest.raises(tq.TqmoeError):
             fn(bank, xq, xs, (counts, offsets, perm), 4, 1, 1)
 
@@ -455,7 +455,8 @@ def test_layer_grouped_small_shapes(tq, oracle, n):
 
 @pytest.mark.parametrize("name,fmt,path,mode", [("c1", "Q4_K", "grouped_i8", 5), ("c4", "IQ3_S", "grouped_i8", 5), ("c5", "NVFP4G", "grouped_fp8", 2),
                                                 ("c4", "IQ3_XXS", "grouped_i8", 5), ("c4", "IQ2_XXS", "grouped_i8", 5), ("c4", "IQ2_XS", "grouped_i8", 5),
-                                                ("c4", "IQ2_S", "grouped_i8", 5), ("c4", "IQ1_S", "grouped_i8", 5), ("c4", "IQ4_NL", "grouped_i8", 5)])
+                                                ("c4", "IQ2_S", "grouped_i8", 5), ("c4", "IQ1_S", "grouped_i8", 5), ("c4", "IQ4_NL", "grouped_i8", 5),
+                                                ("c4", "Q5_K", "grouped_i8", 5), ("c4", "Q4_0", "grouped_i8", 5), ("c4", "Q8_0", "grouped_i8", 5)])
 @pytest.mark.parametrize("n", [64, 300])
 def test_layer_grouped_other_formats(tq, oracle, name, fmt, path, mode, n):
     """Q4_K and the lattice formats on the int8 products, NVFP4G banks on the fp8 products, against the oracle with the same
@@ -465,7 +466,7 @@ def test_layer_grouped_other_formats(tq, oracle, name, fmt, path, mode, n):
     check_layer(*run_layer(tq, oracle, cfg, n, seed=160 + n, modes=(mode, 0), path=path))
 
 
-@pytest.mark.parametrize("fmt,n", [("IQ4_XS", 64), ("IQ4_XS", 300), ("Q4_K", 300), ("IQ3_S", 300), ("IQ4_NL", 300), ("IQ2_S", 64)])
+@pytest.mark.parametrize("fmt,n", [("IQ4_XS", 64), ("IQ4_XS", 300), ("Q4_K", 300), ("IQ3_S", 300), ("IQ4_NL", 300), ("IQ2_S", 64), ("Q5_K", 300), ("Q4_0", 64), ("Q8_0", 300)])
 def test_layer_block_scales(tq, oracle, fmt, n):
     """The layer with act_blocks set (a scale per 32 activations on both products' inputs, the reference's
     TQFN_PREFILL_INT8=1) against the oracle's mode of the same quantiser; the per-token oracle must be farther away."""

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtqmoe.so")
-SOURCES = ["routing.hip", "bank.hip", "decode.hip", "decode_iq4xs.hip", "decode_q4k.hip", "decode_iq3s.hip", "decode_nvfp4.hip", "decode_iq4nl.hip", "decode_q8_0.hip", "decode_q5k.hip", "decode_q6k.hip", "decode_iq3xxs.hip", "decode_iq2s.hip", "decode_q2k.hip", "decode_iq1s.hip", "decode_q4_0.hip", "decode_q3k.hip", "decode_iq2xxs.hip", "decode_iq2xs.hip", "prefill_planes.hip", "prefill_planes_blocks.hip", "prefill_f16.hip", "norm.hip", "layer.hip"]
+SOURCES = ["routing.hip", "bank.hip", "decode.hip", "decode_iq4xs.hip", "decode_q4k.hip", "decode_iq3s.hip", "decode_nvfp4.hip", "decode_iq4nl.hip", "decode_q8_0.hip", "decode_q5k.hip", "decode_q6k.hip", "decode_iq3xxs.hip", "decode_iq2s.hip", "decode_q2k.hip", "decode_iq1s.hip", "decode_q4_0.hip", "decode_q3k.hip", "decode_iq2xxs.hip", "decode_iq2xs.hip", "prefill_planes.hip", "prefill_planes_blocks.hip", "prefill_planes_legacy.hip", "prefill_f16.hip", "norm.hip", "layer.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",
          # packed FP32 VALU forms are kept out of every kernel
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -378,16 +378,19 @@ int32_t enqueue_gather_rows_natural(const int8_t * rq, const float * rs, int col
     return 0;
 }
 
-// bank formats with a plane GEMM: int8 operands (IQ4_XS, IQ4_NL, IQ3_S, IQ3_XXS, IQ2_XXS, IQ2_XS, IQ2_S, IQ1_S, Q4_K) or E4M3 operands (NVFP4G)
+// bank formats with a plane GEMM: int8 operands (IQ4_XS, IQ4_NL, IQ3_S, IQ3_XXS, IQ2_XXS, IQ2_XS, IQ2_S, IQ1_S, Q4_K, Q5_K, Q4_0, Q8_0) or E4M3
+// operands (NVFP4G). Q6_K, Q3_K and Q2_K carry a scale per 16 weights, half the depth of the matrix instruction: their
+// grouped products go through the fp16 kernels.
 bool plane_gemm_has(uint32_t type) {
     return type == TQMOE_IQ4_XS || type == TQMOE_IQ3_S || type == TQMOE_Q4_K || type == TQMOE_NVFP4G || type == TQMOE_IQ3_XXS || type == TQMOE_IQ2_XXS ||
-           type == TQMOE_IQ2_XS || type == TQMOE_IQ2_S || type == TQMOE_IQ1_S || type == TQMOE_IQ4_NL;
+           type == TQMOE_IQ2_XS || type == TQMOE_IQ2_S || type == TQMOE_IQ1_S || type == TQMOE_IQ4_NL || type == TQMOE_Q5_K || type == TQMOE_Q4_0 || type == TQMOE_Q8_0;
 }
 bool plane_gemm_is_fp8(uint32_t type) { return type == TQMOE_NVFP4G; }
 
 // assignments = total entries of perm (it fixes where the index behind the scales lies)
 // xbs: a scale per row and 32-value sub-block (int8 operands only), or null
 int32_t plane_gemm_blocks(uint32_t type, int nb, bool gateup, const GemmArgs & k, unsigned blocks, hipStream_t s);
+int32_t plane_gemm_legacy(uint32_t type, int nb, bool gateup, bool blk, const GemmArgs & k, unsigned blocks, hipStream_t s);
 int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const int8_t * xq, const float * xs, const int * counts, const int * offsets,
                            const int * perm, int experts, int64_t assignments, void * out_f16, int gateup, int shared_expert, int shared_lim, hipStream_t s,
                            const float * xbs, Glu glu, int out_bf16, const float * plan_from) {
@@ -403,6 +406,7 @@ int32_t enqueue_plane_gemm(const tqmoe_bank & b0, const tqmoe_bank * b1, const i
     const int cus = cu_count();
     const int64_t most = (tiles / kChunkTiles + experts + 7) / 8 * 8 * (units / unit_group);     // an upper bound of the items
     const unsigned blocks = unsigned(std::min<int64_t>((cus + 7) / 8 * 8, most));
+    if (b0.type == TQMOE_Q5_K || b0.type == TQMOE_Q4_0 || b0.type == TQMOE_Q8_0) return plane_gemm_legacy(b0.type, nb, gateup != 0, xbs != nullptr, k, blocks, s);
     if (xbs) return plane_gemm_blocks(b0.type, nb, gateup != 0, k, blocks, s);
     switch (b0.type) {
         case TQMOE_IQ4_XS: plane_gemm_launch<WIq4xs>(nb, gateup != 0, k, blocks, s); break;

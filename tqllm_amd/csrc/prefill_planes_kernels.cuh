@@ -513,6 +513,109 @@ struct WIq4nl {   // row-major: 16 code bytes per sub-block (nibbles as IQ4_XS),
     static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
 };
 
+// Q4_0: IQ4_NL's layout; the weight is the nibble minus 8 (no lookup)
+struct WQ4_0 : WIq4nl {
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int, const uint8_t *, const uint32_t *, v4i * p) {
+        p[0] = v4i{int(minus_k<8>(c.c.x & 0x0F0F0F0Fu)), int(minus_k<8>((c.c.x >> 4) & 0x0F0F0F0Fu)),
+                   int(minus_k<8>(c.c.y & 0x0F0F0F0Fu)), int(minus_k<8>((c.c.y >> 4) & 0x0F0F0F0Fu))};
+    }
+};
+
+// Q8_0: 32 int8 values per sub-block, the operand itself: lane (n, g) reads values 8g.. and 16 + 8g.. (two 8-byte loads)
+struct WQ8_0 : WIq4nl {
+    struct Code { uint2 lo, hi; };
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int g) {
+        const int S = b.cols / 32;
+        const int64_t row = int64_t(e) * b.rows + wtile * 32 + n;
+        return Src{b.codes + row * S * 32 + g * 8, b.aux + row * S * 2};
+    }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) {
+        const uint8_t * c = s.codes + int64_t(sub) * 32;
+        return Code{*reinterpret_cast<const uint2 *>(c), *reinterpret_cast<const uint2 *>(c + 16)};
+    }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int, const uint8_t *, const uint32_t *, v4i * p) {
+        p[0] = v4i{int(c.lo.x), int(c.hi.x), int(c.lo.y), int(c.hi.y)};
+    }
+};
+
+// Q5_K: Q4_K's layout and header, and a word per sub-block with the fifth bit of its 32 codes (after the header in the
+// 48-byte record). The products sc * q of a 5-bit code q are looked up as for Q4_K, from two pairs of 16-entry tables per
+// scale (q below 16, q from 16 on), and the fifth bit chooses between the two results bit by bit.
+struct WQ5k {
+    static constexpr bool kFoldSub = false, kWideChunks = false;
+    static constexpr int kPlanes = 3, kTabBytes = 64 * 64, kLattice = 1;
+    static constexpr bool kFp8 = false, kMin = true, kRowMul = false;
+    struct Code { uint2 c; uint32_t hb; };
+    typedef uint4 Rec;
+    typedef uint32_t DRec;
+    struct Src { const uint8_t * codes, * aux; };
+    static __device__ __forceinline__ void tables(uint8_t * tab, uint32_t *, int tid, int threads) {   // per 6-bit scale sc: sc * q, q = 0..15 (h, l), q = 16..31 (h, l)
+        for (int i = tid; i < 64 * 32; i += threads) {
+            const int sc = i >> 5, q = i & 31;
+            split_planes(q * sc, tab[sc * 64 + (q >> 4) * 32 + (q & 15)], tab[sc * 64 + (q >> 4) * 32 + 16 + (q & 15)]);
+        }
+    }
+    static __device__ __forceinline__ Src src(const BankView & b, int e, int wtile, int n, int g) {
+        const int S = b.cols / 32;
+        const int64_t row = int64_t(e) * b.rows + wtile * 32 + n;
+        return Src{b.codes + row * S * 16 + g * 8, b.aux + row * (S / 8) * 48};
+    }
+    static __device__ __forceinline__ Code code(const Src & s, int sub) {
+        return Code{*reinterpret_cast<const uint2 *>(s.codes + int64_t(sub) * 16), *reinterpret_cast<const uint32_t *>(s.aux + int64_t(sub >> 3) * 48 + 16 + 4 * (sub & 7))};
+    }
+    static __device__ __forceinline__ Rec rec(const Src & s, int sb) { return *reinterpret_cast<const uint4 *>(s.aux + int64_t(sb) * 48); }
+    static __device__ __forceinline__ DRec drec(const Src & s, int sb) { return *reinterpret_cast<const uint32_t *>(s.aux + int64_t(sb) * 48); }
+    static __device__ __forceinline__ int choose(uint32_t mask, int on, int off) { return int((uint32_t(on) & mask) | (uint32_t(off) & ~mask)); }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec & r, int ib, int g, const uint8_t * tab, const uint32_t *, v4i * p) {
+        int sc, mn;
+        q4k_scale_min_flat(r.y, r.z, r.w, ib, sc, mn);
+        const uint4 * t = reinterpret_cast<const uint4 *>(tab + sc * 64);
+        const uint4 h0 = t[0], l0 = t[1], h1 = t[2], l1 = t[3];
+        const uint32_t cw[2] = {c.c.x, c.c.y};
+        const uint32_t hb = c.hb >> (8 * g);   // the fifth bits of the lane's values: bits 0..7 (values 8g..), 16..23 (values 16 + 8g..)
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+            const NibbleKeys k = nibble_keys(cw[w]);
+            const uint32_t m_lo = spread4(hb >> (4 * w)) * 0xFFu, m_hi = spread4(hb >> (16 + 4 * w)) * 0xFFu;
+            p[0][2 * w] = choose(m_lo, pick16(h1, k.i_lo, k.s_lo), pick16(h0, k.i_lo, k.s_lo));
+            p[0][2 * w + 1] = choose(m_hi, pick16(h1, k.i_hi, k.s_hi), pick16(h0, k.i_hi, k.s_hi));
+            p[1][2 * w] = choose(m_lo, pick16(l1, k.i_lo, k.s_lo), pick16(l0, k.i_lo, k.s_lo));
+            p[1][2 * w + 1] = choose(m_hi, pick16(l1, k.i_hi, k.s_hi), pick16(l0, k.i_hi, k.s_hi));
+        }
+        const int m = mn * 0x01010101;
+        p[2] = v4i{m, m, m, m};
+    }
+    static __device__ __forceinline__ float d(const DRec & r) { return half_bits_to_float(uint16_t(r & 0xFFFFu)); }
+    static __device__ __forceinline__ float dmin(const DRec & r) { return half_bits_to_float(uint16_t(r >> 16)); }
+    static __device__ __forceinline__ float rowmul(const BankView &, int, int, int) { return 1.f; }
+};
+
+// Q5_K for rows with a scale per sub-block: the 5-bit codes themselves as one plane, a plane of ones, d * sc and dmin * mn
+// as the sub-block's fp32 scales (as WQ4kSub)
+struct WQ5kSub : WQ5k {
+    static constexpr bool kFoldSub = true;
+    static constexpr int kPlanes = 2, kTabBytes = 16;
+    typedef uint4 DRec;
+    static __device__ __forceinline__ void tables(uint8_t *, uint32_t *, int, int) {}
+    static __device__ __forceinline__ DRec drec(const Src & s, int sb) { return rec(s, sb); }
+    static __device__ __forceinline__ void planes(const Code & c, const Rec &, int, int g, const uint8_t *, const uint32_t *, v4i * p) {
+        const uint32_t hb = c.hb >> (8 * g);
+        p[0] = v4i{int((c.c.x & 0x0F0F0F0Fu) | (spread4(hb) << 4)), int(((c.c.x >> 4) & 0x0F0F0F0Fu) | (spread4(hb >> 16) << 4)),
+                   int((c.c.y & 0x0F0F0F0Fu) | (spread4(hb >> 4) << 4)), int(((c.c.y >> 4) & 0x0F0F0F0Fu) | (spread4(hb >> 20) << 4))};
+        p[1] = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    }
+    static __device__ __forceinline__ float d_sub(const DRec & r, int ib) {      // exact: 11 bits times 6 bits
+        int sc, mn;
+        q4k_scale_min_flat(r.y, r.z, r.w, ib, sc, mn);
+        return __fmul_rn(half_bits_to_float(uint16_t(r.x & 0xFFFFu)), float(sc));
+    }
+    static __device__ __forceinline__ float dmin_sub(const DRec & r, int ib) {
+        int sc, mn;
+        q4k_scale_min_flat(r.y, r.z, r.w, ib, sc, mn);
+        return __fmul_rn(half_bits_to_float(uint16_t(r.x >> 16)), float(mn));
+    }
+};
+
 struct WNvfp4 {   // row-major: 16 code bytes per sub-block, one E4M3 scale byte per 16 weights, one fp32 global per row
     static constexpr bool kFoldSub = false;     // one scale per 32 weights: every sub-block's product is folded on its own
     static constexpr bool kWideChunks = true;   // chunks of sixteen row tiles on eight waves (two row tiles a wave)

@@ -469,9 +469,11 @@ typedef struct tqmoe_layer {
     int32_t gating;                   /* 0: softmax, else a TQMOE_GATE_ value */
     int32_t raw_weights;              /* nonzero: the selected weights are not normalised */
     const float * probs_bias;         /* device [n_expert] fp32 selection bias, or NULL */
-    /* Activation scales of the int8 grouped products, the reference's TQFN_PREFILL_INT8 (fn_prefill.cpp:100): zero (or a
-     * descriptor that ends before this field) = one scale per token (its value 2), nonzero = one per 32 values (its
-     * value 1). The fp8 and fp16 grouped products and the decode kernels ignore it. */
+    /* The reference's TQFN_PREFILL_INT8 (fn_prefill.cpp:100). 0 (or a descriptor that ends before this field): the library
+     * picks the grouped products of a prefill-sized batch, the 8-bit ones (a scale per token) where they are the faster ones
+     * for the banks' formats and the batch, else the fp16 ones. 1: the int8 grouped products with one scale per 32
+     * activations (its value 1). 2: the int8 grouped products with one scale per token (its value 2). 1 and 2 apply where
+     * both banks' formats have int8 grouped products; NVFP4G banks (fp8 products) and the decode kernels ignore the field. */
     int32_t act_blocks;
     /* Clamp of the SwiGLU inputs, applied in the fused gate / up epilogues of every path (routed and shared experts alike).
      * swiglu_clamp <= 1e-6 (or a descriptor that ends before this field): none. Else up is clamped to
@@ -485,7 +487,9 @@ size_t  tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t n);
 /* Which expert products tqmoe_layer_forward runs for n tokens of this layer (the choice depends on the batch and the
  * bank formats only, never on the data, so that a token's result does not depend on what else is routed; the reference
  * makes its switch slot-independent for the same reason, src/models/qwen/qwen4exp/fn_layer_forward.cpp:408-414):
- * the decode kernels (one read of every distinct expert), the grouped int8 products, or the grouped fp16 products.
+ * the decode kernels (one read of every distinct expert), the grouped 8-bit products, or the grouped fp16 products.
+ * With act_blocks zero the grouped products are the ones measured faster for the formats: int8 for IQ4_XS from 1024
+ * tokens and for the two- and three-bit lattice formats, fp8 for NVFP4G, fp16 otherwise.
  * Negative: the descriptor is invalid. */
 enum { TQMOE_PATH_DECODE = 0, TQMOE_PATH_GROUPED_I8 = 1, TQMOE_PATH_GROUPED_F16 = 2, TQMOE_PATH_GROUPED_FP8 = 3 };
 int32_t tqmoe_layer_path(const tqmoe_layer * layer, int32_t n);

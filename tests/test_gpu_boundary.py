@@ -144,7 +144,7 @@ def test_layer_swiglu_clamp(tq, oracle, name, n, path, clamp_gate):
     inp = synth.make_inputs(cfg, n, seed=701)
     limit = 0.5
     mk = lambda c: tq.MoeLayer(dev(inp["router"]), dev(inp["shared_gate"]) if cfg["shared_ff"] else None, gate, up, down, cfg["topk"], shared_ff=cfg["shared_ff"],
-                               swiglu_clamp=c, clamp_gate=clamp_gate)
+                               swiglu_clamp=c, clamp_gate=clamp_gate, act_blocks=2 if path == "grouped_i8" else 0)
     layer = mk(limit)
     assert layer.path(n) == path
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))

@@ -411,12 +411,13 @@ def test_gather_of_quantised_rows_equals_group_rows(tq, dtype):
     assert torch.equal(s1[rows:].view(torch.int32), s2[rows:].view(torch.int32))      # the tile index behind the scales
 
 
-def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0), path="grouped_i8", act_blocks=False):
+def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0), path="grouped_i8", act_blocks=False, request=True):
     raws = synth.make_banks(cfg, seed=seed, distinct=distinct)
     gate, up, down = banks_on_device(cfg, raws)
     inp = synth.make_inputs(cfg, n, seed=seed + 1, zipf=zipf)
+    # the int8 products are asked for (a scale per token unless act_blocks): left alone the library picks the faster products
     layer = tq.MoeLayer(dev(inp["router"]), dev(inp["shared_gate"]) if cfg["shared_ff"] else None, gate, up, down, cfg["topk"],
-                        shared_ff=cfg["shared_ff"], act_blocks=act_blocks)
+                        shared_ff=cfg["shared_ff"], act_blocks=1 if act_blocks else 2 if path == "grouped_i8" and request else 0)
     assert layer.path(n) == path
     out, ids, w, logits = (t.cpu().numpy() for t in layer.forward(dev(inp["x"]), return_routing=True))
     wants = {}
@@ -429,7 +430,7 @@ def run_layer(tq, oracle, cfg, n, seed, distinct=None, zipf=None, modes=(5, 0), 
 
 def check_layer(out, ids, w, wants, clear):
     fp8 = 2 in wants
-    want, want_ids, want_w = wants[2] if fp8 else wants[5] if 5 in wants else wants[6]
+    want, want_ids, want_w = wants[2] if fp8 else wants[5] if 5 in wants else wants[6] if 6 in wants else wants[0]
     assert np.array_equal(ids[clear], want_ids[clear])
     assert np.abs(w[clear] - want_w[clear]).max() < 3e-6
     mx, rel = synth.errors(out[clear], want[clear])
@@ -464,6 +465,20 @@ def test_layer_grouped_other_formats(tq, oracle, name, fmt, path, mode, n):
     base = dict(synth.CONFIGS[name], wtype=getattr(oracle, fmt))
     cfg = synth.small(base, 768, 512, 10, 3)
     check_layer(*run_layer(tq, oracle, cfg, n, seed=160 + n, modes=(mode, 0), path=path))
+
+
+@pytest.mark.parametrize("fmt,name,n,path", [("IQ4_XS", "c2", 8, "decode"), ("IQ4_XS", "c2", 300, "grouped_f16"), ("IQ4_XS", "c2", 1024, "grouped_i8"),
+                                             ("Q4_K", "c1", 1024, "grouped_f16"), ("IQ3_S", "c4", 300, "grouped_f16"), ("Q8_0", "c4", 300, "grouped_f16"),
+                                             ("IQ2_S", "c4", 300, "grouped_i8"), ("IQ1_S", "c4", 300, "grouped_i8"), ("NVFP4G", "c5", 300, "grouped_fp8"),
+                                             ("Q6_K", "c4", 300, "grouped_f16")])
+def test_layer_products_left_to_the_library(tq, oracle, fmt, name, n, path):
+    """With nothing asked for (act_blocks 0) the layer takes the products measured faster for the formats and the batch: the
+    decode kernels for few tokens, then the fp16 grouped products, the int8 ones for IQ4_XS from 1024 tokens and for the
+    lattice formats, the fp8 ones for NVFP4G; each against the oracle of its operand format."""
+    base = dict(synth.CONFIGS[name], wtype=getattr(oracle, fmt))
+    cfg = synth.small(base, 768, 512, 10, 3)
+    mode = {"decode": 0, "grouped_f16": 0, "grouped_i8": 5, "grouped_fp8": 2}[path]
+    check_layer(*run_layer(tq, oracle, cfg, n, seed=860 + n, modes=(mode,), path=path, request=False))
 
 
 @pytest.mark.parametrize("fmt,n", [("IQ4_XS", 64), ("IQ4_XS", 300), ("Q4_K", 300), ("IQ3_S", 300), ("IQ4_NL", 300), ("IQ2_S", 64), ("Q5_K", 300), ("Q4_0", 64), ("Q8_0", 300)])
@@ -538,8 +553,9 @@ def test_layer_config3_full_size_properties(tq, oracle):
     assert np.array_equal(counts.cpu().numpy(), np.bincount(flat, minlength=cfg["experts"]))
     assert np.array_equal(perm.cpu().numpy(), np.argsort(flat, kind="stable"))
     assert counts.max().item() > 128 * 3                      # the crowded experts span several chunks
-    # a sub-batch taken in another order gives bit-identical rows
-    pick = torch.from_numpy(np.random.default_rng(1).permutation(n)[:700].copy()).cuda()
+    # a sub-batch taken in another order gives bit-identical rows (1100 tokens: on the same products as the full batch)
+    assert layer.path(n) == layer.path(1100) == "grouped_i8"
+    pick = torch.from_numpy(np.random.default_rng(1).permutation(n)[:1100].copy()).cuda()
     sub = layer.forward(x[pick].contiguous())
     assert torch.equal(sub, out[pick])
     # and 128 of them against the oracle: the first 96 tokens and 32 spread over the rows of the most crowded expert

@@ -670,7 +670,7 @@ class MoeLayer:
                  norm_weights=True, act_blocks=False, swiglu_clamp=0.0, clamp_gate=False):
         self.swiglu_clamp, self.clamp_gate = swiglu_clamp, clamp_gate   # MoeConfig::swiglu_clamp, moe_expert_ffn's clamp_gate
         self.router, self.shared_gate, self.gate, self.up, self.down = router, shared_gate, gate, up, down
-        self.act_blocks = act_blocks   # int8 grouped products: a scale per 32 activations in place of one per token
+        self.act_blocks = act_blocks   # 0 / False: the library picks the grouped products; 1 / True: int8 with a scale per 32 activations; 2: int8 with a scale per token
         self.n_expert, self.hidden = router.shape
         self.ff, self.topk, self.shared_ff, self.weight_scale = gate.rows, topk, shared_ff, weight_scale
         self.gating, self.probs_bias, self.norm_weights = gating, probs_bias, norm_weights

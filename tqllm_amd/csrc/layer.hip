@@ -26,8 +26,12 @@ int32_t gemm_f16_common(const tqmoe_bank * b0, const tqmoe_bank * b1, const void
 
 namespace {
 
-// Token counts from kGroupedMin up take the grouped int8 products (IQ4_XS banks), fewer the decode kernels.
+// Where the descriptor asks for the int8 grouped products (act_blocks nonzero), IQ4_XS banks take them from kGroupedMin tokens.
 constexpr int kGroupedMin = 64;
+// Left to the library (act_blocks zero), IQ4_XS banks take them from kInt8Tokens tokens: measured at 512 experts, top-10, on
+// uniform and on Zipf routing, the fp16 grouped products are level or up to a fifth faster below (most experts then hold a
+// row tile or two, which the fp16 kernel's one-expert blocks serve better), the int8 products a seventh faster at 4096.
+constexpr int kInt8Tokens = 1024;
 constexpr int kDecodeAssignments = 65535;   // per decode launch
 constexpr int kDecodeDedup = 2048;          // assignments up to which the decode kernels serve an expert's rows together
 constexpr int kGroupedPerBank = 3;          // assignments per expert from which the fp16 grouped products are the faster path
@@ -53,20 +57,35 @@ bool int8_ok(const tqmoe_layer & L) {
 // ends before act_blocks means a scale per token; one that ends before swiglu_clamp means no clamp.
 constexpr size_t kLayerBaseSize = offsetof(tqmoe_layer, gating), kLayerRoutingSize = offsetof(tqmoe_layer, act_blocks);
 constexpr size_t kLayerBlocksSize = offsetof(tqmoe_layer, swiglu_clamp);
-bool act_blocks_of(const tqmoe_layer & L) { return L.struct_size >= kLayerBlocksSize && L.act_blocks != 0; }
+// the descriptor's request for the int8 grouped products: 0 none (the library chooses), 1 a scale per 32 activations, 2 a scale per token
+int int8_mode_of(const tqmoe_layer & L) { return L.struct_size >= kLayerBlocksSize ? (L.act_blocks == 1 ? 1 : L.act_blocks == 2 ? 2 : 0) : 0; }
+bool act_blocks_of(const tqmoe_layer & L) { return int8_mode_of(L) == 1; }
+// Formats whose 8-bit grouped products are the faster ones at n tokens (measured against the fp16 grouped products at 256
+// experts top-8 and at 64 experts top-8, 512 and 4096 tokens): the lattice formats of two and three bits (a tenth faster),
+// NVFP4G on its fp8 products, IQ4_XS from kInt8Tokens tokens. IQ3_S, Q4_K, Q5_K, IQ4_NL, Q4_0 and Q8_0 run 5 to 25 % faster
+// on the fp16 products (their row-major codes reach the int8 kernel's lanes in 8-byte pieces of 32 different rows).
+bool int8_faster(uint32_t type, int n) {
+    switch (type) {
+        case TQMOE_IQ4_XS: return n >= kInt8Tokens;
+        case TQMOE_NVFP4G: case TQMOE_IQ3_XXS: case TQMOE_IQ2_XXS: case TQMOE_IQ2_XS: case TQMOE_IQ2_S: case TQMOE_IQ1_S: return true;
+        default: return false;
+    }
+}
 // a descriptor that ends before swiglu_clamp does not clamp
 Glu glu_of(const tqmoe_layer & L) { return L.struct_size >= sizeof(tqmoe_layer) ? Glu{L.swiglu_clamp, L.clamp_gate ? 1 : 0} : Glu{0.f, 0}; }
 
 Plan plan_for(const tqmoe_layer & L, int n) {
     Plan p{};
     const int slots = L.topk + (L.has_shared ? 1 : 0), banks = L.n_expert + (L.has_shared ? 1 : 0);
-    // IQ4_XS banks (tile-major): the int8 grouped products from kGroupedMin tokens. Every other format, on the 8-bit or the
-    // fp16 grouped products: from kGroupedPerBank assignments per bank matrix on average (measured: the decode kernels' time
-    // grows with the assignments, the grouped products' with the experts they decode, and the two cross at about three
-    // assignments per expert), and in any case once the decode kernels no longer read every expert's weights once (they
-    // group an expert's rows up to kDecodeDedup assignments a launch)
+    // Few tokens: the decode kernels. From kGroupedPerBank assignments per bank matrix on average the grouped products
+    // (measured: the decode kernels' time grows with the assignments, the grouped products' with the experts they decode, and
+    // the two cross at about three assignments per expert), and in any case once the decode kernels no longer read every
+    // expert's weights once (they group an expert's rows up to kDecodeDedup assignments a launch).
+    // Which grouped products: the descriptor's request (act_blocks), else the faster ones for the formats (int8_faster).
     const bool many = int64_t(n) * slots > std::min<int64_t>(kDecodeDedup, int64_t(kGroupedPerBank) * banks);
-    p.int8 = int8_ok(L) && (L.gate.type == TQMOE_IQ4_XS && L.down.type == TQMOE_IQ4_XS ? n >= kGroupedMin : many);
+    const bool iq4xs = L.gate.type == TQMOE_IQ4_XS && L.down.type == TQMOE_IQ4_XS;
+    if (int8_mode_of(L) != 0) p.int8 = int8_ok(L) && (iq4xs ? n >= kGroupedMin : many);
+    else p.int8 = int8_ok(L) && many && int8_faster(L.gate.type, n) && int8_faster(L.down.type, n);
     p.grouped = p.int8 || many;
     // the grouped products take 2^24 assignments a pass (32-bit block and byte counts stay far from their limits), the
     // decode kernels 65535

@@ -489,7 +489,7 @@ size_t  tqmoe_layer_workspace_bytes(const tqmoe_layer * layer, int32_t n);
  * makes its switch slot-independent for the same reason, src/models/qwen/qwen4exp/fn_layer_forward.cpp:408-414):
  * the decode kernels (one read of every distinct expert), the grouped 8-bit products, or the grouped fp16 products.
  * With act_blocks zero the grouped products are the ones measured faster for the formats: int8 for IQ4_XS from 1024
- * tokens and for the two- and three-bit lattice formats, fp8 for NVFP4G, fp16 otherwise.
+ * tokens, for Q4_K from 2048 and for the two- and three-bit lattice formats, fp8 for NVFP4G, fp16 otherwise.
  * Negative: the descriptor is invalid. */
 enum { TQMOE_PATH_DECODE = 0, TQMOE_PATH_GROUPED_I8 = 1, TQMOE_PATH_GROUPED_F16 = 2, TQMOE_PATH_GROUPED_FP8 = 3 };
 int32_t tqmoe_layer_path(const tqmoe_layer * layer, int32_t n);

@@ -181,6 +181,48 @@ def dispatch(ids, n_expert):
     return counts, offsets, perm
 
 
+DEDUP_COLS, DEDUP_STRIDE = 8, 18    # kDedupCols, kDedupStride (src/experts/moe_kernels.cuh:33-38)
+
+
+def dedup_maps(ids, slot_of, topk, groups):
+    """The decode grouping maps of moe_dedup_maps, one assignment at a time as the reference's kernel computes them
+    (src/experts/moe.cu:452-483): slots[a] = slot_of[ids[a]] (-1 for a skipped assignment); an assignment's rank among the
+    assignments of its slot gives its chunk (rank / 8) and column (rank % 8); its group is the number of groups opened by
+    earlier assignments than its chunk's opener; a group's record is [slot, columns, 8 inputs, 8 outputs] with the token
+    (gu) or the assignment (dn) as input and the assignment as output, unused entries -1. Pure Python: small inputs only.
+    Returns (slots [count], gu [groups][18], dn [groups][18])."""
+    ids = np.asarray(ids, np.int32).reshape(-1)
+    count = ids.size
+    slot = np.array([slot_of[e] if e >= 0 else -1 for e in ids], np.int32)
+    gu = np.full((groups, DEDUP_STRIDE), -1, np.int32)
+    dn = np.full((groups, DEDUP_STRIDE), -1, np.int32)
+    rank = np.array([int((slot[:a] == slot[a]).sum()) for a in range(count)])
+    total = np.array([int((slot == slot[a]).sum()) for a in range(count)])
+    opens = (slot >= 0) & (rank % DEDUP_COLS == 0)
+    for a in range(count):
+        if slot[a] < 0:
+            continue
+        chunk, col = divmod(int(rank[a]), DEDUP_COLS)
+        same = np.flatnonzero(slot[:a + 1] == slot[a])
+        opener = int(same[chunk * DEDUP_COLS])
+        g = int(opens[:opener].sum())
+        cols = min(DEDUP_COLS, int(total[a]) - chunk * DEDUP_COLS)
+        for part, e in ((0, gu), (1, dn)):
+            if col == 0:
+                e[g, 0], e[g, 1] = slot[a], cols
+            e[g, 2 + col] = a if part else a // topk
+            e[g, 2 + DEDUP_COLS + col] = a
+    return slot, gu, dn
+
+
+def count(ids, counts):
+    """moe_count (src/experts/moe.cu:183-186, 279-282): counts[ids[i]] += 1 on 64-bit running counters; negative ids are
+    skipped here as everywhere in this library (the reference's callers never pass them to this function)."""
+    ids = np.asarray(ids).reshape(-1)
+    np.add.at(counts, ids[ids >= 0], 1)
+    return counts
+
+
 def expert_ffn(x, w_gate, w_up, w_down, clamp=0.0, clamp_gate=False):
     x, w_gate, w_up, w_down = (_c(a, np.float32) for a in (x, w_gate, w_up, w_down))
     ff, hidden = w_gate.shape

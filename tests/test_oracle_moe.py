@@ -666,3 +666,53 @@ def test_cpu_baseline_kernels_agree_with_decode(oracle, ref):
     assert np.sqrt(np.mean((y - want) ** 2) / np.mean(want ** 2)) < 1e-5
     ref.ref_iq4nl_matvec(2, p(raw), rows, cols, p(x), 1, p(y))
     assert np.sqrt(np.mean((y - want) ** 2) / np.mean(want ** 2)) < 1e-2
+
+
+def sequential_dedup_maps(ids, slot_of, topk, groups):
+    """An independent build of the decode grouping maps: walk the assignments in order and keep, per bank slot, the group that
+    is open and how many columns it has; a full group (8 columns) is closed and the next assignment of that slot opens a new
+    one with the next free group number."""
+    gu = np.full((groups, 18), -1, np.int32)
+    dn = np.full((groups, 18), -1, np.int32)
+    slots = np.array([slot_of[e] if e >= 0 else -1 for e in ids], np.int32)
+    open_group, ng = {}, 0
+    for a, s in enumerate(slots):
+        if s < 0:
+            continue
+        g, used = open_group.get(int(s), (-1, 8))
+        if used == 8:
+            g, used = ng, 0
+            ng += 1
+            gu[g, 0] = dn[g, 0] = s
+        gu[g, 1] = dn[g, 1] = used + 1
+        gu[g, 2 + used], gu[g, 10 + used] = a // topk, a
+        dn[g, 2 + used], dn[g, 10 + used] = a, a
+        open_group[int(s)] = (g, used + 1)
+    return slots, gu, dn
+
+
+def test_dedup_maps_against_a_sequential_build_and_by_hand(oracle):
+    """oracle.dedup_maps follows the reference's kernel (every assignment finds its group by itself); it must equal the
+    sequential walk on random inputs (skipped assignments, crowded slots that fill several groups, slots that are not the
+    expert numbers), and a case worked by hand."""
+    # by hand: topk 2, tokens 0..4; expert 7 appears 9 times (a full group and a second one), expert 2 twice, one skipped
+    ids = np.array([7, 2, 7, -1, 7, 7, 7, 2, 7, 7, 7, 7], np.int32)
+    slot_of = np.arange(10, dtype=np.int32) + 100
+    slots, gu, dn = oracle.dedup_maps(ids, slot_of, 2, len(ids))
+    assert slots.tolist() == [107, 102, 107, -1, 107, 107, 107, 102, 107, 107, 107, 107]
+    # groups in order of opening: slot 107 (assignments 0 2 4 5 6 8 9 10), slot 102 (1 7), slot 107 again (11)
+    assert gu[0].tolist() == [107, 8, 0, 1, 2, 2, 3, 4, 4, 5, 0, 2, 4, 5, 6, 8, 9, 10]
+    assert gu[1].tolist() == [102, 2, 0, 3, -1, -1, -1, -1, -1, -1, 1, 7, -1, -1, -1, -1, -1, -1]
+    assert gu[2].tolist() == [107, 1, 5] + [-1] * 7 + [11] + [-1] * 7
+    assert dn[0].tolist() == [107, 8, 0, 2, 4, 5, 6, 8, 9, 10, 0, 2, 4, 5, 6, 8, 9, 10]
+    assert (gu[3:] == -1).all() and (dn[3:] == -1).all()
+    rng = np.random.default_rng(3)
+    for experts, n, topk in ((6, 40, 3), (64, 30, 8), (3, 100, 2), (500, 16, 10)):
+        ids = rng.integers(-1, experts, n * topk).astype(np.int32)
+        slot_of = rng.permutation(experts * 2)[:experts].astype(np.int32)
+        got = oracle.dedup_maps(ids, slot_of, topk, len(ids) + 3)
+        want = sequential_dedup_maps(ids, slot_of, topk, len(ids) + 3)
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w)
+    counts = np.array([5, 0, 1 << 40], np.int64)
+    assert oracle.count(np.array([[0, 2, -1], [2, 2, 0]]), counts).tolist() == [7, 0, (1 << 40) + 3]

@@ -61,12 +61,15 @@ constexpr size_t kLayerBlocksSize = offsetof(tqmoe_layer, swiglu_clamp);
 int int8_mode_of(const tqmoe_layer & L) { return L.struct_size >= kLayerBlocksSize ? (L.act_blocks == 1 ? 1 : L.act_blocks == 2 ? 2 : 0) : 0; }
 bool act_blocks_of(const tqmoe_layer & L) { return int8_mode_of(L) == 1; }
 // Formats whose 8-bit grouped products are the faster ones at n tokens (measured against the fp16 grouped products at 256
-// experts top-8 and at 64 experts top-8, 512 and 4096 tokens): the lattice formats of two and three bits (a tenth faster),
-// NVFP4G on its fp8 products, IQ4_XS from kInt8Tokens tokens. IQ3_S, Q4_K, Q5_K, IQ4_NL, Q4_0 and Q8_0 run 5 to 25 % faster
-// on the fp16 products (their row-major codes reach the int8 kernel's lanes in 8-byte pieces of 32 different rows).
+// experts top-8 and at 64 experts top-8, 256 to 4096 tokens, uniform and Zipf routing): the lattice formats of two and three
+// bits (a tenth faster), NVFP4G on its fp8 products, IQ4_XS from kInt8Tokens tokens, Q4_K from 2048 tokens (with fp32 input
+// rows, which the fp16 kernel converts block by block, int8 is a tenth faster there; with 16-bit rows the two are level).
+// IQ3_S, Q5_K, IQ4_NL, Q4_0 and Q8_0 run 5 to 25 % faster on the fp16 products (their row-major codes reach the int8 kernel's
+// lanes in 8-byte pieces of 32 different rows, and two int8 planes cost the matrix pipe what one fp16 operand does).
 bool int8_faster(uint32_t type, int n) {
     switch (type) {
         case TQMOE_IQ4_XS: return n >= kInt8Tokens;
+        case TQMOE_Q4_K: return n >= 2 * kInt8Tokens;
         case TQMOE_NVFP4G: case TQMOE_IQ3_XXS: case TQMOE_IQ2_XXS: case TQMOE_IQ2_XS: case TQMOE_IQ2_S: case TQMOE_IQ1_S: return true;
         default: return false;
     }
